@@ -1,0 +1,188 @@
+/*
+ * tokenselect.h - C ABI of libtokenselect_hip.so: TokenSelect's decode-time
+ * token-level KV selection and sparse attention for AMD MI355X (gfx950).
+ *
+ * Every entry point takes plain pointers and sizes.  All data pointers are
+ * device pointers unless a parameter says "host".  bf16 tensors are passed as
+ * `const void*` (16-bit brain floats, row-major, innermost dimension
+ * contiguous).  Launches are asynchronous on the given HIP stream; the library
+ * never synchronises, never allocates device memory and keeps no mutable
+ * global state, so calls are re-entrant across streams.
+ *
+ * Return value: TS_OK or a negative TS_E* code; ts_last_error() then holds a
+ * thread-local message.  Arguments are validated on the host before anything
+ * touches the GPU, so a bad call fails without a device.
+ *
+ * Citations "tr.py:N" are into the reference's patcher/token_retrieval.py.
+ */
+#ifndef TOKENSELECT_H_
+#define TOKENSELECT_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TS_VERSION 100
+
+#define TS_OK 0
+#define TS_EINVAL (-1)     /* null pointer or scalar out of range            */
+#define TS_ESHAPE (-2)     /* head_dim / head-group shape not supported      */
+#define TS_EWORKSPACE (-3) /* workspace or an output stride is too small     */
+#define TS_EHIP (-4)       /* the HIP runtime reported a launch error        */
+
+#define TS_ROPE_NONE 0
+#define TS_ROPE_LLAMA 1 /* FlashInfer pos_encoding_mode="ROPE_LLAMA", tr.py:822 */
+
+#define TS_HEADMAP_MOD 0 /* kv head = h % Hkv: the reference's scoring, tr.py:202 */
+#define TS_HEADMAP_DIV 1 /* kv head = h / (H/Hkv): conventional GQA             */
+
+#define TS_DTYPE_F32 0
+#define TS_DTYPE_BF16 1
+
+typedef void* ts_stream_t; /* a hipStream_t; NULL is the default stream */
+
+/* Static per-layer configuration: the module globals that patch() sets
+ * (tr.py:29-39, 885-918) plus the attention scalars RadixAttention carries
+ * (tr.py:816-822). */
+typedef struct ts_config {
+  int32_t num_heads;    /* H: query heads on this rank                        */
+  int32_t num_kv_heads; /* Hkv: KV heads on this rank; H % Hkv == 0           */
+  int32_t head_dim;     /* D: 128                                             */
+  int32_t page_size;    /* tokens per KV page; 1 = the reference's per-token  */
+                        /* table token_indices, tr.py:293-297                 */
+  int32_t n_init;       /* sink tokens always kept (N_INIT)                   */
+  int32_t n_local;      /* local-window tokens always kept (N_Local)          */
+  int32_t top_k;        /* TOP_K; upper bound of the per-request k            */
+  int32_t pool_kernel;  /* KERNEL_SIZE for vote max-pooling, <= 0 = off       */
+  int32_t head_map;     /* TS_HEADMAP_* used by the scoring pass              */
+  int32_t rope_mode;    /* TS_ROPE_* applied inside the attention kernel      */
+  float rope_theta;     /* ROPE_BASE                                          */
+  float rope_scale;     /* ROPE_SCALE                                         */
+  float sm_scale;       /* RadixAttention.scaling                             */
+  float logit_cap;      /* RadixAttention.logit_cap; <= 0 = off               */
+} ts_config;
+
+/* The running requests of one decode step.  The reference handles one request
+ * (tr.py:130); a batch applies the same semantics to each request on its own. */
+typedef struct ts_batch {
+  int32_t batch;            /* B                                               */
+  int32_t max_seq_len;      /* host: upper bound of seq_lens[], sizes grids    */
+  const int32_t* seq_lens;  /* [B] tokens held per request, the new one included
+                               (num_tokens[layer], tr.py:376)                  */
+  const int32_t* table;     /* logical page -> physical page; request b's row
+                               starts at table + b*table_stride.  Physical slot
+                               of logical token t: table[t/ps]*ps + t%ps       */
+  int64_t table_stride;     /* elements between rows                           */
+  const int32_t* k_per_req; /* [B] per-request k (<= top_k), or NULL = top_k   */
+} ts_batch;
+
+/* Optional selection-cache state for one layer (tr.py:301-322, 394-421).
+ * All arrays are device memory owned by the caller and persist across steps. */
+typedef struct ts_selcache {
+  void* q_cache;        /* [B, H*D] bf16: fingerprint of the last miss          */
+  int32_t* topk_cache;  /* [B, top_k] cached logical positions (+n_init)        */
+  int32_t* cache_len;   /* [B] entries cached; 0 = no query seen (is_first_query) */
+  int64_t* counters;    /* [B, 2] skip_count, retrieval_count (tr.py:420-421)   */
+  float threshold;      /* similarity_threshold, bf16(0.9)=0.8984375 (tr.py:313) */
+} ts_selcache;
+
+int ts_version(void);
+const char* ts_last_error(void);
+
+/* RotaryEmbedding.apply_rotary_pos_emb (tr.py:98-107):
+ * out = bf16(float(x)*cos[pos] + float(rotate_half(x))*sin[pos]), products and
+ * sum rounded separately as torch does.  x, out: [rows, heads, dim] bf16;
+ * cos_table, sin_table: [table_rows, dim] fp32; position_ids: [rows] int64. */
+int ts_rope_apply(const void* x, void* out, const float* cos_table, const float* sin_table,
+                  const int64_t* position_ids, int64_t table_rows, int64_t rows,
+                  int32_t heads, int32_t dim, ts_stream_t stream);
+
+/* paged_matmul (tr.py:234-261): scores[h,t] = sum_d query[h,d] *
+ * token[indices[t], h % Hkv, d], fp32 accumulation, no scaling.
+ * query [H,D] bf16; token [pool_rows,Hkv,D] bf16; indices [n] int32;
+ * scores [H,n] of scores_dtype (the reference allocates bf16, tr.py:345-347). */
+int ts_paged_matmul(const void* query, const void* token, int64_t pool_rows,
+                    const int32_t* indices, void* scores, int32_t scores_dtype, int64_t n,
+                    int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
+                    ts_stream_t stream);
+
+/* Scoring pass of get_topk_tokens over a ragged batch (tr.py:350-359): for every
+ * request that is not dense (n_init+k+n_local >= L, tr.py:377) and whose
+ * skip[b] is 0, scores[(b*H+h)*score_stride + t] for candidates t in
+ * [0, L-n_init-n_local) and the per-head softmax statistics
+ * stats[(b*H+h)*2 + {0,1}] = {max_t s, sum_t exp(s - max)}.
+ * qf [B,H,D] bf16 is the rotated fingerprint (tr.py:380-392). */
+size_t ts_score_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+             int64_t pool_rows, const int32_t* skip, float* scores, int64_t score_stride,
+             float* stats, void* workspace, size_t workspace_bytes, ts_stream_t stream);
+
+/* Soft vote (tr.py:361): votes[b*vote_stride + t] = sum_h exp(s[h,t]-max_h)/Z_h,
+ * then the optional max-pool of tr.py:366-369 when cfg->pool_kernel > 0
+ * (pooled is then the output and votes the scratch; both [B, vote_stride]). */
+int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
+            int64_t score_stride, const float* stats, const int32_t* skip, float* votes,
+            float* pooled, int64_t vote_stride, ts_stream_t stream);
+
+/* Ragged top-k + sort + index assembly (tr.py:371-373, 433-449).  Per request:
+ * the k_b largest votes (ties: lowest position first), ascending, offset by
+ * n_init, between the n_init sink positions and the n_local newest positions;
+ * sel_pos holds those logical positions, sel the physical slots through the
+ * table, sel_len[b] = n_init+k_b+n_local.  A dense request (tr.py:377-378)
+ * gets all L positions.  With hit != NULL and hit[b] != 0 the middle segment is
+ * taken from cache->topk_cache instead (tr.py:419); on a miss the new positions
+ * are stored there when cache != NULL (tr.py:415).
+ * sel, sel_pos: [B, sel_stride] int32, sel_stride >= n_init+top_k+n_local. */
+size_t ts_topk_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
+                   int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
+                   int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
+                   void* workspace, size_t workspace_bytes, ts_stream_t stream);
+
+/* Selection-cache decision (tr.py:394-401, 416-421) for one layer, no host
+ * sync: hit[b] = cache_len[b] > 0 && cos(q_cache[b], qf[b]) >= threshold; on a
+ * miss q_cache[b] = qf[b].  Dense requests (tr.py:377) are left untouched with
+ * hit[b] = 0.  Counters advance as the reference's do. */
+int ts_selcache_step(const ts_config* cfg, const ts_batch* bt, const void* qf,
+                     const ts_selcache* cache, int32_t* hit, ts_stream_t stream);
+
+/* Decode attention over the selected slots: FlashInfer
+ * BatchDecodeWithPagedKVCacheWrapper.forward with page_size 1 as called at
+ * tr.py:815-823.  Head h reads KV head h/(H/Hkv); with TS_ROPE_LLAMA the query
+ * is rotated to position S-1 and selected key j to position j inside the kernel.
+ * q, out: [B,H,D] bf16; k_pool, v_pool: [pool_rows,Hkv,D] bf16;
+ * sel [B, sel_stride] int32 with sel_len[b] valid entries (<= max_sel_len). */
+size_t ts_attn_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_sel_len);
+int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_pool,
+                          const void* v_pool, int64_t pool_rows, const int32_t* sel,
+                          int64_t sel_stride, const int32_t* sel_len, int32_t batch,
+                          int32_t max_sel_len, void* out, void* workspace,
+                          size_t workspace_bytes, ts_stream_t stream);
+
+/* KV store + table append (patched_radix_attention_store_kv_cache tr.py:844-854,
+ * add_k_cache tr.py:332-336) for page_size 1: k_pool[loc[b]] = k[b],
+ * v_pool[loc[b]] = v[b], table[b][seq_lens[b]] = loc[b], seq_lens[b] += 1. */
+int ts_kv_store(const ts_config* cfg, const void* k, const void* v, const int32_t* out_cache_loc,
+                void* k_pool, void* v_pool, int64_t pool_rows, int32_t* table,
+                int64_t table_stride, int32_t* seq_lens, int32_t batch, int32_t max_tokens,
+                ts_stream_t stream);
+
+/* One layer of patched_radix_attention_decode_forward_flashinfer after the KV
+ * store (tr.py:791-825): fingerprint (q rotated with q_cos/q_sin, the [D] table
+ * rows of position n_local, tr.py:380-388) -> [selection cache] -> score ->
+ * vote -> top-k -> assembly -> sparse attention.  q, out: [B,H*D] bf16.
+ * cache may be NULL (QUERY_CACHE=False as released, tr.py:918). */
+size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, const float* q_cos,
+                    const float* q_sin, const void* k_pool, const void* v_pool,
+                    int64_t pool_rows, const ts_selcache* cache, void* out, int32_t* sel,
+                    int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
+                    size_t workspace_bytes, ts_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TOKENSELECT_H_ */

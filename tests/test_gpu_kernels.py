@@ -1,0 +1,229 @@
+"""GPU parity of each kernel against the CPU oracle on seeded inputs, through
+the C ABI.  Tolerances: fp32 scores 1e-3 relative (to the score RMS); selected
+positions identical up to ties at the k-th vote; bf16 attention output 2e-2
+absolute."""
+
+import pytest
+import torch
+
+import oracle
+from tokenselect_amd import ops, workloads
+from helpers import assert_index_sets_match, assert_scores_close, cpu_tabs, oracle_layer, say
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    dict(num_heads=32, num_kv_heads=8, rope_theta=5e5),   # Llama-3-8B
+    dict(num_heads=28, num_kv_heads=4, rope_theta=1e6),   # Qwen2-7B
+    dict(num_heads=8, num_kv_heads=1, rope_theta=1e4),    # TP shard of a 64/8 model
+    dict(num_heads=4, num_kv_heads=2, rope_theta=1e4),
+    dict(num_heads=8, num_kv_heads=8, rope_theta=1e4),    # MHA
+    dict(num_heads=16, num_kv_heads=4, rope_theta=1e4),
+]
+
+
+def small(dev, shape, seed, lens=(3000,), ks=(64,), page=1, n_init=8, n_local=16, **kw):
+    return workloads.build("small", shape, list(lens), list(ks), page, dev, seed,
+                           n_init=n_init, n_local=n_local, **kw)
+
+
+def fingerprint(wl, dev):
+    c = wl.cfg
+    cos, sin = ops.scoring_cos_sin(c.head_dim, c.rope_theta, c.rope_scale, c.n_local, dev)
+    return ops.rope_apply(wl.q.view(len(wl.seq_lens), c.num_heads, c.head_dim), cos, sin, None)
+
+
+def test_rope_apply_bit_exact(dev):
+    say("rope_apply rows=5 heads=6 dim=128")
+    torch.manual_seed(0)
+    x = torch.randn(5, 6, 128).bfloat16()
+    pos = torch.tensor([0, 3, 511, 512, 77])
+    cos, sin = oracle.rope.cos_sin_tables(513, 128, 5e5, 1.0)
+    ref = oracle.rope.apply(x, pos, 5e5, 1.0)
+    got = ops.rope_apply(x.to(dev), cos.squeeze(1).contiguous().to(dev),
+                         sin.squeeze(1).contiguous().to(dev), pos.to(dev))
+    assert torch.equal(got.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_paged_matmul(dev, shape, out_dtype):
+    H, Hkv = shape["num_heads"], shape["num_kv_heads"]
+    say(f"paged_matmul H={H} Hkv={Hkv} n=2500 out={out_dtype}")
+    g = torch.Generator().manual_seed(H * 100 + Hkv)
+    P, n = 4096, 2500
+    token = torch.randn(P, Hkv, 128, generator=g).bfloat16()
+    query = torch.randn(H, 128, generator=g).bfloat16()
+    idx = torch.randperm(P, generator=g)[:n].int()
+    scores = torch.empty((H, n), dtype=out_dtype, device=dev)
+    ops.paged_matmul(query.to(dev), token.to(dev), idx.to(dev), scores, n, H, Hkv, 128)
+    ref = oracle.select.score(query, token, idx)
+    if out_dtype == torch.float32:
+        assert_scores_close(scores.cpu(), ref, "paged_matmul fp32")
+    else:  # one bf16 rounding of the fp32 score: within one bf16 ulp (2^-8 relative)
+        got = scores.float().cpu()
+        assert bool(((got - ref).abs() <= ref.abs() * 2.0 ** -8 + 1e-6).all())
+        assert (got != ref.bfloat16().float()).float().mean().item() < 1e-3
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("page", [1, 16])
+def test_score_vote_topk(dev, shape, page):
+    lens, ks = [3000, 777, 40, 1531], [64, 100, 64, 1]
+    say(f"score/vote/topk H={shape['num_heads']} Hkv={shape['num_kv_heads']} page={page} lens={lens}")
+    wl = small(dev, shape, seed=page + shape["num_heads"], lens=lens, ks=ks, page=page, top_k=100)
+    c = wl.cfg
+    qf = fingerprint(wl, dev)
+    scores, stats = ops.score(c, wl.batch, qf, wl.k_pool)
+    votes = ops.vote(c, wl.batch, scores, stats)
+    sel, sel_pos, sel_len = ops.topk_ragged(c, wl.batch, votes)
+    torch.cuda.synchronize()
+    details = []
+    ref_sel, _ = oracle_layer(wl, details)
+    tabs = cpu_tabs(wl)
+    for b, (L, k) in enumerate(zip(wl.seq_lens, wl.k_list)):
+        S = int(sel_len[b])
+        if oracle.select.is_dense(L, c.n_init, c.n_local, k):
+            assert S == L
+            assert torch.equal(sel[b, :L].cpu(), tabs[b][:L])
+            assert torch.equal(sel_pos[b, :L].cpu(), torch.arange(L, dtype=torch.int32))
+            continue
+        d = details[b]
+        n = L - c.n_init - c.n_local
+        assert torch.equal(qf[b].reshape(-1).cpu().view(torch.int16), d["qf"].view(torch.int16))
+        assert_scores_close(scores[b, :, :n].cpu(), d["scores"], f"scores b={b}")
+        ref_stats_m = d["scores"].max(dim=1).values
+        assert torch.allclose(stats[b, :, 0].cpu(), ref_stats_m, rtol=1e-5, atol=1e-5)
+        assert torch.allclose(votes[b, :n].cpu(), d["votes"], rtol=2e-4, atol=1e-9)
+        assert S == c.n_init + k + c.n_local
+        pos = sel_pos[b, :S].cpu()
+        assert torch.equal(pos[:c.n_init], torch.arange(c.n_init, dtype=torch.int32))
+        assert torch.equal(pos[c.n_init + k:], torch.arange(L - c.n_local, L, dtype=torch.int32))
+        mid = pos[c.n_init:c.n_init + k]
+        assert bool((mid[1:] > mid[:-1]).all()) if k > 1 else True
+        assert_index_sets_match(mid, d["top_pos"], d["votes"], c.n_init, f"top-k b={b}")
+        assert torch.equal(sel[b, :S].cpu(), tabs[b][pos.long()])
+
+
+def test_topk_ties_and_extremes(dev):
+    say("topk ties / k=1 / k=n-1")
+    shape = SHAPES[0]
+    for n_extra, k in [(50, 1), (50, 49), (3000, 17)]:
+        L = 8 + 16 + n_extra
+        wl = small(dev, shape, seed=5, lens=[L], ks=[k], top_k=k)
+        n = L - 24
+        # all-equal votes -> the k lowest positions
+        votes = torch.full((1, ops.score_stride_for(L)), 0.25, dtype=torch.float32, device=dev)
+        sel, pos, slen = ops.topk_ragged(wl.cfg, wl.batch, votes)
+        assert torch.equal(pos[0, 8:8 + k].cpu(), torch.arange(8, 8 + k, dtype=torch.int32))
+        # tie-free random votes -> argsort
+        g = torch.Generator().manual_seed(n)
+        v = torch.rand(n, generator=g)
+        votes[0, :n] = v.to(dev)
+        sel, pos, slen = ops.topk_ragged(wl.cfg, wl.batch, votes)
+        ref = torch.sort(torch.argsort(v, descending=True)[:k]).values + 8
+        assert torch.equal(pos[0, 8:8 + k].cpu().long(), ref)
+        # negative and mixed-sign values keep their order
+        v2 = torch.randn(n, generator=g)
+        votes[0, :n] = v2.to(dev)
+        sel, pos, slen = ops.topk_ragged(wl.cfg, wl.batch, votes)
+        ref = torch.sort(torch.argsort(v2, descending=True)[:k]).values + 8
+        assert torch.equal(pos[0, 8:8 + k].cpu().long(), ref)
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("rope_mode", ["ROPE_LLAMA", "NONE"])
+def test_sparse_attention(dev, shape, rope_mode):
+    say(f"attention H={shape['num_heads']} Hkv={shape['num_kv_heads']} rope={rope_mode}")
+    wl = small(dev, shape, seed=11, lens=[2000, 300], ks=[64, 64])
+    c = wl.cfg
+    c.rope_mode = rope_mode
+    g = torch.Generator().manual_seed(3)
+    lens = [700, 37]
+    sel = torch.zeros((2, 700), dtype=torch.int32)
+    for b, S in enumerate(lens):
+        sel[b, :S] = torch.randperm(wl.k_pool.shape[0], generator=g)[:S].int()
+    sel_len = torch.tensor(lens, dtype=torch.int32)
+    out = ops.sparse_decode_attention(c, wl.q, wl.k_pool, wl.v_pool, sel.to(dev), sel_len.to(dev))
+    kc, vc, qc = wl.k_pool.cpu(), wl.v_pool.cpu(), wl.q.cpu()
+    for b, S in enumerate(lens):
+        ref = oracle.attend.sparse_decode_attention(
+            qc[b].view(c.num_heads, 128), kc, vc, sel[b, :S], 128 ** -0.5, c.rope_theta, 1.0, 0.0,
+            rope_mode)
+        err = (out[b].cpu().float() - ref.reshape(-1).float()).abs().max().item()
+        assert err <= 2e-2, f"attention b={b}: max abs err {err}"
+
+
+def test_attention_soft_cap(dev):
+    say("attention logit_cap=30")
+    wl = small(dev, SHAPES[0], seed=12, lens=[500], ks=[64])
+    c = wl.cfg
+    c.logit_cap = 30.0
+    c.sm_scale = 1.0  # large logits so the cap bites
+    S = 256
+    sel = torch.arange(S, dtype=torch.int32).view(1, S)
+    out = ops.sparse_decode_attention(c, wl.q, wl.k_pool, wl.v_pool, sel.to(dev),
+                                      torch.tensor([S], dtype=torch.int32, device=dev))
+    ref = oracle.attend.sparse_decode_attention(wl.q.cpu()[0].view(c.num_heads, 128), wl.k_pool.cpu(),
+                                                wl.v_pool.cpu(), sel[0], 1.0, c.rope_theta, 1.0, 30.0)
+    assert (out[0].cpu().float() - ref.reshape(-1).float()).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("shape", SHAPES[:2], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("page", [1, 16])
+def test_decode_layer(dev, shape, page):
+    lens, ks = [5000, 100, 2048, 901], [256, 256, 200, 256]
+    say(f"decode_layer H={shape['num_heads']} page={page} lens={lens}")
+    wl = small(dev, shape, seed=21 + page, lens=lens, ks=ks, page=page, top_k=256, n_init=16,
+               n_local=32)
+    layer = ops.DecodeLayer(wl.cfg, len(lens), max(lens), dev)
+    out, sel, sel_pos, sel_len = layer(wl.q, wl.k_pool, wl.v_pool, wl.batch)
+    torch.cuda.synchronize()
+    details = []
+    ref_sel, ref_out = oracle_layer(wl, details)
+    for b in range(len(lens)):
+        S = int(sel_len[b])
+        assert S == ref_sel[b].shape[0]
+        if details[b]:
+            c = wl.cfg
+            assert_index_sets_match(sel_pos[b, c.n_init:S - c.n_local].cpu(), details[b]["top_pos"],
+                                    details[b]["votes"], c.n_init, f"layer top-k b={b}")
+        if torch.equal(sel[b, :S].cpu(), ref_sel[b]):
+            err = (out[b].cpu().float() - ref_out[b].float()).abs().max().item()
+            assert err <= 2e-2, f"decode_layer out b={b}: {err}"
+
+
+def test_max_pool_votes(dev):
+    for kernel in (5, 6, 32):
+        say(f"max-pool kernel={kernel}")
+        wl = small(dev, SHAPES[0], seed=31, lens=[2500, 900], ks=[64, 64], pool_kernel=kernel)
+        c = wl.cfg
+        qf = fingerprint(wl, dev)
+        scores, stats = ops.score(c, wl.batch, qf, wl.k_pool)
+        votes = ops.vote(c, wl.batch, scores, stats)
+        sel, sel_pos, sel_len = ops.topk_ragged(c, wl.batch, votes)
+        details = []
+        oracle_layer(wl, details)
+        for b, L in enumerate(wl.seq_lens):
+            n_out = details[b]["votes"].shape[0]
+            assert torch.allclose(votes[b, :n_out].cpu(), details[b]["votes"], rtol=2e-4, atol=1e-9)
+            S = int(sel_len[b])
+            assert_index_sets_match(sel_pos[b, c.n_init:S - c.n_local].cpu(), details[b]["top_pos"],
+                                    details[b]["votes"], c.n_init, f"pooled top-k b={b}", rtol=3e-4)
+
+
+def test_kv_store(dev):
+    say("kv_store")
+    wl = small(dev, SHAPES[0], seed=41, lens=[100, 50], ks=[16, 16], extra_pages=8)
+    c = wl.cfg
+    table = torch.zeros((2, 128), dtype=torch.int32, device=dev)
+    table[:, :wl.table.shape[1]] = wl.table
+    seq = wl.seq_lens_dev.clone()
+    loc = torch.tensor([wl.k_pool.shape[0] - 1, wl.k_pool.shape[0] - 2], dtype=torch.int32, device=dev)
+    k = torch.randn(2, c.num_kv_heads * 128, device=dev).bfloat16()
+    v = torch.randn(2, c.num_kv_heads * 128, device=dev).bfloat16()
+    ops.kv_store(c, k, v, loc, wl.k_pool, wl.v_pool, table, seq)
+    assert seq.tolist() == [101, 51]
+    assert table[0, 100].item() == loc[0].item() and table[1, 50].item() == loc[1].item()
+    assert torch.equal(wl.k_pool[loc[0].item()].reshape(-1), k[0])
+    assert torch.equal(wl.v_pool[loc[1].item()].reshape(-1), v[1])

@@ -1,0 +1,170 @@
+// Host-side plumbing of the C ABI: error state, argument validation and the
+// per-layer driver that chains the kernels of one decode step.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "ts_common.h"
+
+namespace ts {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TS_EHIP, "%s: %s", what, hipGetErrorString(e));
+  return TS_OK;
+}
+
+bool group_supported(int num_kv_heads, int group) {
+  bool kv_ok = num_kv_heads == 1 || num_kv_heads == 2 || num_kv_heads == 4 || num_kv_heads == 8;
+  bool g_ok = group == 1 || group == 2 || group == 4 || group == 7 || group == 8;
+  return kv_ok && g_ok;
+}
+
+int validate_config(const ts_config* cfg) {
+  TS_REQUIRE(cfg != nullptr, TS_EINVAL, "config is NULL");
+  TS_REQUIRE(cfg->head_dim == kHeadDim, TS_ESHAPE, "head_dim %d not supported (only 128)",
+             cfg->head_dim);
+  TS_REQUIRE(cfg->num_heads > 0 && cfg->num_kv_heads > 0, TS_EINVAL,
+             "num_heads=%d num_kv_heads=%d must be positive", cfg->num_heads, cfg->num_kv_heads);
+  TS_REQUIRE(cfg->num_heads % cfg->num_kv_heads == 0, TS_ESHAPE,
+             "num_heads %d not a multiple of num_kv_heads %d", cfg->num_heads, cfg->num_kv_heads);
+  TS_REQUIRE(group_supported(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads), TS_ESHAPE,
+             "unsupported head shape: num_kv_heads=%d (1,2,4,8) group=%d (1,2,4,7,8)",
+             cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
+  TS_REQUIRE(page_shift_of(cfg->page_size) >= 0, TS_EINVAL, "page_size %d is not a power of two",
+             cfg->page_size);
+  TS_REQUIRE(cfg->n_init >= 0 && cfg->n_local >= 0 && cfg->top_k >= 1, TS_EINVAL,
+             "n_init=%d n_local=%d top_k=%d out of range", cfg->n_init, cfg->n_local, cfg->top_k);
+  TS_REQUIRE(cfg->head_map == TS_HEADMAP_MOD || cfg->head_map == TS_HEADMAP_DIV, TS_EINVAL,
+             "head_map %d unknown", cfg->head_map);
+  TS_REQUIRE(cfg->rope_mode == TS_ROPE_NONE || cfg->rope_mode == TS_ROPE_LLAMA, TS_EINVAL,
+             "rope_mode %d unknown", cfg->rope_mode);
+  if (cfg->rope_mode == TS_ROPE_LLAMA)
+    TS_REQUIRE(cfg->rope_theta > 0.f && cfg->rope_scale > 0.f, TS_EINVAL,
+               "rope_theta=%g rope_scale=%g must be positive", cfg->rope_theta, cfg->rope_scale);
+  return TS_OK;
+}
+
+int validate_batch(const ts_config* cfg, const ts_batch* bt) {
+  (void)cfg;
+  TS_REQUIRE(bt != nullptr, TS_EINVAL, "batch is NULL");
+  TS_REQUIRE(bt->batch >= 1, TS_EINVAL, "batch %d < 1", bt->batch);
+  TS_REQUIRE(bt->max_seq_len >= 1, TS_EINVAL, "max_seq_len %d < 1", bt->max_seq_len);
+  TS_REQUIRE(bt->seq_lens != nullptr, TS_EINVAL, "seq_lens is NULL");
+  TS_REQUIRE(bt->table != nullptr, TS_EINVAL, "table is NULL");
+  TS_REQUIRE(bt->batch == 1 || bt->table_stride * (int64_t)cfg->page_size >= bt->max_seq_len,
+             TS_EINVAL, "table_stride %lld too small for max_seq_len %d at page_size %d",
+             (long long)bt->table_stride, bt->max_seq_len, cfg->page_size);
+  return TS_OK;
+}
+
+int score_tokens_per_block(int64_t total_candidates) {
+  // Aim for about four resident workgroups per CU on 256 CUs; 64-row granularity
+  // keeps every wave on whole 16-row tiles.
+  int64_t per = ceil_div(total_candidates, 1024);
+  per = ceil_div(per, 64) * 64;
+  if (per < 64) per = 64;
+  if (per > 512) per = 512;
+  return (int)per;
+}
+
+}  // namespace ts
+
+using namespace ts;
+
+extern "C" {
+
+int ts_version(void) { return TS_VERSION; }
+
+const char* ts_last_error(void) { return ts::g_error; }
+
+// Workspace of ts_decode_layer, carved in this order (256-byte aligned pieces).
+struct LayerWorkspace {
+  size_t qf, hit, scores, stats, votes, pooled, score_ws, topk_ws, attn_ws, total;
+  int64_t score_stride;
+  int32_t max_sel;
+};
+
+static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+  LayerWorkspace w;
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    size_t at = off;
+    off += align_up(bytes, 256);
+    return at;
+  };
+  const size_t B = (size_t)batch, H = (size_t)cfg->num_heads;
+  w.score_stride = (int64_t)align_up((size_t)max_seq_len, 64);
+  w.max_sel = cfg->n_init + cfg->top_k + cfg->n_local;
+  w.qf = take(B * H * kHeadDim * 2);
+  w.hit = take(B * 4);
+  w.scores = take(B * H * (size_t)w.score_stride * 4);
+  w.stats = take(B * H * 2 * 4);
+  w.votes = take(B * (size_t)w.score_stride * 4);
+  w.pooled = take(cfg->pool_kernel > 0 ? B * (size_t)w.score_stride * 4 : 0);
+  w.score_ws = take(ts_score_workspace_bytes(cfg, batch, max_seq_len));
+  w.topk_ws = take(ts_topk_workspace_bytes(cfg, batch, max_seq_len));
+  w.attn_ws = take(ts_attn_workspace_bytes(cfg, batch, w.max_sel));
+  w.total = off;
+  return w;
+}
+
+size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+  if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
+  return layer_workspace(cfg, batch, max_seq_len).total;
+}
+
+int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, const float* q_cos,
+                    const float* q_sin, const void* k_pool, const void* v_pool,
+                    int64_t pool_rows, const ts_selcache* cache, void* out, int32_t* sel,
+                    int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
+                    size_t workspace_bytes, ts_stream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_TRY(validate_batch(cfg, bt));
+  TS_REQUIRE(q && q_cos && q_sin && k_pool && v_pool && out && sel && sel_pos && sel_len, TS_EINVAL,
+             "ts_decode_layer: NULL tensor argument");
+  TS_REQUIRE(pool_rows >= 1, TS_EINVAL, "pool_rows %lld < 1", (long long)pool_rows);
+  LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);
+  TS_REQUIRE(sel_stride >= w.max_sel, TS_EWORKSPACE, "sel_stride %lld < n_init+top_k+n_local = %d",
+             (long long)sel_stride, w.max_sel);
+  TS_REQUIRE(workspace != nullptr && workspace_bytes >= w.total, TS_EWORKSPACE,
+             "workspace %zu bytes < required %zu", workspace_bytes, w.total);
+  if (cache)
+    TS_REQUIRE(cache->q_cache && cache->topk_cache && cache->cache_len && cache->counters, TS_EINVAL,
+               "selection cache has a NULL array");
+
+  char* ws = (char*)workspace;
+  void* qf = ws + w.qf;
+  int32_t* hit = cache ? (int32_t*)(ws + w.hit) : nullptr;
+  float* scores = (float*)(ws + w.scores);
+  float* stats = (float*)(ws + w.stats);
+  float* votes = (float*)(ws + w.votes);
+  float* pooled = cfg->pool_kernel > 0 ? (float*)(ws + w.pooled) : nullptr;
+
+  // Fingerprint: every request's single decode row is rotated to n_local
+  // (tr.py:381-388); the mean over one row is the row itself (tr.py:392).
+  TS_TRY(ts_rope_apply(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
+                       stream));
+  if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
+  TS_TRY(ts_score(cfg, bt, qf, k_pool, pool_rows, hit, scores, w.score_stride, stats,
+                  ws + w.score_ws, w.topk_ws - w.score_ws, stream));
+  TS_TRY(ts_vote(cfg, bt, scores, w.score_stride, stats, hit, votes, pooled, w.score_stride,
+                 stream));
+  TS_TRY(ts_topk_ragged(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache, sel, sel_pos,
+                        sel_stride, sel_len, ws + w.topk_ws, w.attn_ws - w.topk_ws, stream));
+  TS_TRY(ts_sparse_decode_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len,
+                               bt->batch, w.max_sel, out, ws + w.attn_ws, w.total - w.attn_ws,
+                               stream));
+  return TS_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,121 @@
+// Shared host/device helpers for libtokenselect_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/tokenselect.h"
+
+namespace ts {
+
+// ---------------------------------------------------------------- host side
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+int validate_config(const ts_config* cfg);
+int validate_batch(const ts_config* cfg, const ts_batch* bt);
+bool group_supported(int num_kv_heads, int group);
+
+#define TS_REQUIRE(cond, code, ...)                     \
+  do {                                                  \
+    if (!(cond)) return ::ts::fail((code), __VA_ARGS__); \
+  } while (0)
+
+#define TS_TRY(expr)            \
+  do {                          \
+    int _rc = (expr);           \
+    if (_rc != TS_OK) return _rc; \
+  } while (0)
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Candidate rows per workgroup of the scoring pass, shared by the launcher,
+// the statistics merge and the workspace query.
+int score_tokens_per_block(int64_t total_candidates);
+
+constexpr int kHeadDim = 128;
+constexpr float kNegBig = -3.0e38f;  // finite stand-in for -inf in running maxima
+
+// -------------------------------------------------------------- device side
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+
+// Round-to-nearest-even, NaN kept quiet: the rounding torch applies on .to(bfloat16).
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)0x7fc0;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
+constexpr int kRowRor1 = 0x121, kRowRor2 = 0x122, kRowRor4 = 0x124, kRowRor8 = 0x128;
+
+// Sum over the 16 lanes of a DPP row; every lane of the row gets the total.
+__device__ __forceinline__ float row16_sum(float x) {
+  x += dpp_move<kRowRor8>(x);
+  x += dpp_move<kRowRor4>(x);
+  x += dpp_move<kRowRor2>(x);
+  x += dpp_move<kRowRor1>(x);
+  return x;
+}
+
+// Merge two (max, sum-of-exp) softmax partials.
+__device__ __forceinline__ void softmax_merge(float& m, float& l, float m2, float l2) {
+  float mm = fmaxf(m, m2);
+  l = l * __expf(m - mm) + l2 * __expf(m2 - mm);
+  m = mm;
+}
+
+__device__ __forceinline__ void row16_softmax_merge(float& m, float& l) {
+  softmax_merge(m, l, dpp_move<kRowRor8>(m), dpp_move<kRowRor8>(l));
+  softmax_merge(m, l, dpp_move<kRowRor4>(m), dpp_move<kRowRor4>(l));
+  softmax_merge(m, l, dpp_move<kRowRor2>(m), dpp_move<kRowRor2>(l));
+  softmax_merge(m, l, dpp_move<kRowRor1>(m), dpp_move<kRowRor1>(l));
+}
+
+// Per-request geometry of the selection, evaluated on the device so that no
+// host synchronisation is needed (tr.py:376-378, 424-426).
+struct ReqGeom {
+  int seq_len;  // L
+  int k;        // per-request top-k
+  int n;        // candidates = L - n_init - n_local (0 when dense)
+  bool dense;   // n_init + k + n_local >= L
+};
+
+// seq_lens[b] is clamped to the host's max_seq_len, the bound every buffer and
+// grid was sized for.
+__device__ __forceinline__ ReqGeom request_geometry(const int32_t* seq_lens, const int32_t* k_per_req,
+                                                    int b, int n_init, int n_local, int top_k,
+                                                    int max_seq_len) {
+  ReqGeom g;
+  g.seq_len = min(max(seq_lens[b], 0), max_seq_len);
+  int k = k_per_req ? k_per_req[b] : top_k;
+  g.k = k < 0 ? 0 : (k > top_k ? top_k : k);
+  g.dense = (n_init + g.k + n_local >= g.seq_len);
+  g.n = g.dense ? 0 : g.seq_len - n_init - n_local;
+  return g;
+}
+
+// Logical position -> physical KV slot through the (paged) table; page sizes are
+// powers of two.  The slot is clamped to the pool so that a corrupt table cannot
+// fault the GPU.
+__device__ __forceinline__ uint32_t lookup_slot(const int32_t* tab, int pos, int page_size,
+                                                int page_shift, uint32_t pool_rows) {
+  const uint32_t slot =
+      ((uint32_t)tab[pos >> page_shift] << page_shift) + (uint32_t)(pos & (page_size - 1));
+  return slot < pool_rows ? slot : pool_rows - 1;
+}
+
+static inline int page_shift_of(int page_size) {
+  if (page_size <= 0 || (page_size & (page_size - 1))) return -1;
+  int s = 0;
+  while ((1 << s) < page_size) ++s;
+  return s;
+}
+
+}  // namespace ts

@@ -1,0 +1,135 @@
+// Soft vote: per-head softmax over the candidates summed over heads (tr.py:361),
+// and the optional max-pool smoothing of the votes (tr.py:366-369).
+#include "ts_common.h"
+
+namespace ts {
+
+constexpr int kMaxHeads = 128;
+
+struct VoteArgs {
+  const float* scores;
+  int64_t score_stride;
+  const float* stats;
+  const int32_t* seq_lens;
+  const int32_t* k_per_req;
+  const int32_t* skip;
+  int n_init, n_local, top_k, num_heads, max_seq_len;
+  float* votes;
+  int64_t vote_stride;
+};
+
+// One thread per candidate, heads visited in ascending order (fp32 sum).
+__global__ __launch_bounds__(256) void vote_kernel(VoteArgs a) {
+  const int b = blockIdx.y;
+  if (a.skip && a.skip[b]) return;
+  const ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  const int t0 = blockIdx.x * 1024;
+  if (t0 >= geo.n) return;
+
+  __shared__ float s_max[kMaxHeads];
+  __shared__ float s_rz[kMaxHeads];
+  const int H = a.num_heads;
+  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    s_max[h] = a.stats[((size_t)b * H + h) * 2];
+    s_rz[h] = 1.0f / a.stats[((size_t)b * H + h) * 2 + 1];
+  }
+  __syncthreads();
+
+  const float* base = a.scores + (size_t)b * H * (size_t)a.score_stride;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int t = t0 + r * 256 + threadIdx.x;
+    if (t >= geo.n) break;
+    float c = 0.f;
+    for (int h = 0; h < H; ++h) {
+      const float s = base[(size_t)h * a.score_stride + t];
+      c += __expf(s - s_max[h]) * s_rz[h];
+    }
+    a.votes[(size_t)b * a.vote_stride + t] = c;
+  }
+}
+
+struct PoolArgs {
+  const float* votes;
+  float* pooled;
+  int64_t vote_stride;
+  const int32_t* seq_lens;
+  const int32_t* k_per_req;
+  const int32_t* skip;
+  int n_init, n_local, top_k, kernel, max_seq_len;
+};
+
+// max_pool1d(kernel, stride 1, padding (kernel-1)/2) over the n votes: output t
+// covers inputs [t - pad, t - pad + kernel) clipped to [0, n); an even kernel
+// yields n-1 outputs (tr.py:366-369).
+__global__ __launch_bounds__(256) void pool_kernel(PoolArgs a) {
+  const int b = blockIdx.y;
+  if (a.skip && a.skip[b]) return;
+  const ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  const int pad = (a.kernel - 1) / 2;
+  const int n_out = geo.n + 2 * pad - a.kernel + 1;
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= n_out) return;
+  const float* v = a.votes + (size_t)b * a.vote_stride;
+  const int lo = max(t - pad, 0), hi = min(t - pad + a.kernel, geo.n);
+  float m = v[lo];
+  for (int i = lo + 1; i < hi; ++i) m = fmaxf(m, v[i]);
+  a.pooled[(size_t)b * a.vote_stride + t] = m;
+}
+
+}  // namespace ts
+
+using namespace ts;
+
+extern "C" int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
+                       int64_t score_stride, const float* stats, const int32_t* skip, float* votes,
+                       float* pooled, int64_t vote_stride, ts_stream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_TRY(validate_batch(cfg, bt));
+  TS_REQUIRE(scores && stats && votes, TS_EINVAL, "ts_vote: NULL tensor argument");
+  TS_REQUIRE(cfg->num_heads <= kMaxHeads, TS_ESHAPE, "num_heads %d > %d", cfg->num_heads, kMaxHeads);
+  TS_REQUIRE(cfg->pool_kernel <= 0 || pooled != nullptr, TS_EINVAL,
+             "ts_vote: pool_kernel %d needs a pooled buffer", cfg->pool_kernel);
+  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
+  TS_REQUIRE(score_stride >= max_n && vote_stride >= max_n, TS_EWORKSPACE,
+             "ts_vote: stride (%lld, %lld) < max candidates %d", (long long)score_stride,
+             (long long)vote_stride, max_n);
+  if (max_n <= 0) return TS_OK;
+
+  VoteArgs a;
+  a.scores = scores;
+  a.score_stride = score_stride;
+  a.stats = stats;
+  a.seq_lens = bt->seq_lens;
+  a.k_per_req = bt->k_per_req;
+  a.skip = skip;
+  a.n_init = cfg->n_init;
+  a.n_local = cfg->n_local;
+  a.top_k = cfg->top_k;
+  a.max_seq_len = bt->max_seq_len;
+  a.num_heads = cfg->num_heads;
+  a.votes = votes;
+  a.vote_stride = vote_stride;
+  hipLaunchKernelGGL(vote_kernel, dim3((unsigned)ceil_div(max_n, 1024), (unsigned)bt->batch),
+                     dim3(256), 0, (hipStream_t)stream, a);
+  TS_TRY(check_launch("vote_kernel"));
+
+  if (cfg->pool_kernel > 0) {
+    PoolArgs p;
+    p.votes = votes;
+    p.pooled = pooled;
+    p.vote_stride = vote_stride;
+    p.seq_lens = bt->seq_lens;
+    p.k_per_req = bt->k_per_req;
+    p.skip = skip;
+    p.n_init = cfg->n_init;
+    p.n_local = cfg->n_local;
+    p.top_k = cfg->top_k;
+    p.max_seq_len = bt->max_seq_len;
+    p.kernel = cfg->pool_kernel;
+    hipLaunchKernelGGL(pool_kernel, dim3((unsigned)ceil_div(max_n, 256), (unsigned)bt->batch),
+                       dim3(256), 0, (hipStream_t)stream, p);
+    TS_TRY(check_launch("pool_kernel"));
+  }
+  return TS_OK;
+}

@@ -1,0 +1,378 @@
+"""Tensor-level entry points over the C ABI of ``libtokenselect_hip.so``.
+
+PyTorch is plumbing here: it owns device memory and the HIP stream.  Every
+function checks dtype / device / contiguity / shapes on the host, then passes raw
+pointers and the current stream to the library.  Nothing is computed in Python
+and there is no fallback path.
+"""
+
+import ctypes
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import TsBatch, TsConfig, TsSelCache
+
+HEAD_DIM = 128
+
+
+@dataclass
+class LayerConfig:
+    """The reference's module globals (tr.py:29-39) plus the attention scalars a
+    ``RadixAttention`` carries (tr.py:816-822), for one layer shape."""
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int = HEAD_DIM
+    page_size: int = 1
+    n_init: int = 1
+    n_local: int = 16
+    top_k: int = 16
+    pool_kernel: int = -1
+    head_map: str = "mod"          # scoring: kv = h % Hkv (tr.py:202)
+    rope_mode: str = "ROPE_LLAMA"  # attention: in-kernel RoPE (tr.py:822)
+    rope_theta: float = 1e6
+    rope_scale: float = 1.0
+    sm_scale: Optional[float] = None
+    logit_cap: float = 0.0
+
+    def to_c(self) -> TsConfig:
+        sm = self.sm_scale if self.sm_scale is not None else self.head_dim ** -0.5
+        return TsConfig(
+            self.num_heads, self.num_kv_heads, self.head_dim, self.page_size, self.n_init,
+            self.n_local, self.top_k, self.pool_kernel,
+            _lib.TS_HEADMAP_MOD if self.head_map == "mod" else _lib.TS_HEADMAP_DIV,
+            _lib.TS_ROPE_LLAMA if self.rope_mode == "ROPE_LLAMA" else _lib.TS_ROPE_NONE,
+            float(self.rope_theta), float(self.rope_scale), float(sm), float(self.logit_cap))
+
+    @property
+    def max_sel(self) -> int:
+        return self.n_init + self.top_k + self.n_local
+
+
+@dataclass
+class Batch:
+    """Running requests of a decode step.  ``table`` is ``[B, pages]`` int32
+    (logical page -> physical page; with ``page_size`` 1 it is the reference's
+    ``token_indices`` row, tr.py:293-297); ``seq_lens`` is ``[B]`` int32 on the
+    device; ``max_seq_len`` is the host's upper bound of it."""
+    seq_lens: torch.Tensor
+    table: torch.Tensor
+    max_seq_len: int
+    k_per_req: Optional[torch.Tensor] = None
+
+    @property
+    def batch(self) -> int:
+        return int(self.seq_lens.shape[0])
+
+
+@dataclass
+class SelectionCache:
+    """Selection-cache state of one layer (tr.py:301-322)."""
+    q_cache: torch.Tensor      # [B, H*D] bf16
+    topk_cache: torch.Tensor   # [B, top_k] int32
+    cache_len: torch.Tensor    # [B] int32
+    counters: torch.Tensor     # [B, 2] int64: skip_count, retrieval_count
+    threshold: float
+
+    @classmethod
+    def allocate(cls, cfg: LayerConfig, batch: int, device, threshold: Optional[float] = None):
+        if threshold is None:  # 0.9 stored in bf16 (tr.py:313-315)
+            threshold = float(torch.tensor(0.9, dtype=torch.bfloat16))
+        return cls(
+            torch.zeros((batch, cfg.num_heads * cfg.head_dim), dtype=torch.bfloat16, device=device),
+            torch.zeros((batch, cfg.top_k), dtype=torch.int32, device=device),
+            torch.zeros((batch,), dtype=torch.int32, device=device),
+            torch.zeros((batch, 2), dtype=torch.int64, device=device), threshold)
+
+
+# ------------------------------------------------------------------ helpers
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(t: torch.Tensor, name: str, dtype, ndim: Optional[int] = None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if ndim is not None and t.dim() != ndim:
+        raise ValueError(f"{name} must have {ndim} dims, got shape {tuple(t.shape)}")
+
+
+def _check_pool(cfg: LayerConfig, pool: torch.Tensor, name: str):
+    _need(pool, name, torch.bfloat16, 3)
+    if pool.shape[1] != cfg.num_kv_heads or pool.shape[2] != cfg.head_dim:
+        raise ValueError(f"{name} must be [rows, {cfg.num_kv_heads}, {cfg.head_dim}], "
+                         f"got {tuple(pool.shape)}")
+
+
+def _c_batch(cfg: LayerConfig, bt: Batch) -> TsBatch:
+    _need(bt.seq_lens, "seq_lens", torch.int32, 1)
+    _need(bt.table, "table", torch.int32, 2)
+    if bt.table.shape[0] != bt.batch:
+        raise ValueError("table must have one row per request")
+    if bt.table.shape[1] * cfg.page_size < bt.max_seq_len:
+        raise ValueError(f"table row of {bt.table.shape[1]} pages (page_size {cfg.page_size}) "
+                         f"cannot address max_seq_len {bt.max_seq_len}")
+    if bt.k_per_req is not None:
+        _need(bt.k_per_req, "k_per_req", torch.int32, 1)
+        if bt.k_per_req.shape[0] != bt.batch:
+            raise ValueError("k_per_req must have one entry per request")
+    return TsBatch(bt.batch, int(bt.max_seq_len), _p(bt.seq_lens), _p(bt.table),
+                   int(bt.table.stride(0)), _p(bt.k_per_req))
+
+
+def _c_cache(cache: Optional[SelectionCache], cfg: LayerConfig, batch: int):
+    if cache is None:
+        return None
+    _need(cache.q_cache, "q_cache", torch.bfloat16, 2)
+    _need(cache.topk_cache, "topk_cache", torch.int32, 2)
+    _need(cache.cache_len, "cache_len", torch.int32, 1)
+    _need(cache.counters, "counters", torch.int64, 2)
+    if (tuple(cache.q_cache.shape) != (batch, cfg.num_heads * cfg.head_dim)
+            or tuple(cache.topk_cache.shape) != (batch, cfg.top_k)
+            or cache.cache_len.shape[0] != batch or tuple(cache.counters.shape) != (batch, 2)):
+        raise ValueError("selection cache arrays do not match batch / config")
+    return ctypes.byref(TsSelCache(_p(cache.q_cache), _p(cache.topk_cache), _p(cache.cache_len),
+                                   _p(cache.counters), float(cache.threshold)))
+
+
+def score_stride_for(max_seq_len: int) -> int:
+    return (max_seq_len + 63) // 64 * 64
+
+
+# ------------------------------------------------------------- entry points
+def rope_apply(x: torch.Tensor, cos_table: torch.Tensor, sin_table: torch.Tensor,
+               position_ids: Optional[torch.Tensor]) -> torch.Tensor:
+    """``RotaryEmbedding.apply_rotary_pos_emb`` (tr.py:98-107).  ``x`` is
+    ``[rows, heads, dim]`` bf16; tables ``[T, dim]`` fp32; ``position_ids`` int64
+    ``[rows]`` (``None``: every row uses table row 0)."""
+    _need(x, "x", torch.bfloat16, 3)
+    _need(cos_table, "cos_table", torch.float32, 2)
+    _need(sin_table, "sin_table", torch.float32, 2)
+    rows, heads, dim = x.shape
+    if cos_table.shape != sin_table.shape or cos_table.shape[1] != dim:
+        raise ValueError("cos/sin tables must both be [T, dim]")
+    if position_ids is not None:
+        _need(position_ids, "position_ids", torch.int64, 1)
+        if position_ids.shape[0] != rows:
+            raise ValueError("position_ids must have one entry per row")
+    out = torch.empty_like(x)
+    _lib.check(_lib.load().ts_rope_apply(_p(x), _p(out), _p(cos_table), _p(sin_table),
+                                         _p(position_ids), cos_table.shape[0], rows, heads, dim,
+                                         _stream()))
+    return out
+
+
+def paged_matmul(query: torch.Tensor, token: torch.Tensor, indices: torch.Tensor,
+                 scores: torch.Tensor, num_relevant_tokens: int, num_heads: int,
+                 num_kv_heads: int, head_dim: int) -> None:
+    """tr.py:234-261: fills ``scores[h, t]`` (bf16 or fp32) in place."""
+    _need(query, "query", torch.bfloat16)
+    _need(token, "token", torch.bfloat16, 3)
+    _need(indices, "indices", torch.int32, 1)
+    if scores.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError("scores must be float32 or bfloat16")
+    _need(scores, "scores", scores.dtype, 2)
+    if query.numel() != num_heads * head_dim:
+        raise ValueError("query must hold num_heads*head_dim elements")
+    if token.shape[1] != num_kv_heads or token.shape[2] != head_dim:
+        raise ValueError("token must be [rows, num_kv_heads, head_dim]")
+    if indices.shape[0] < num_relevant_tokens or tuple(scores.shape) != (num_heads, num_relevant_tokens):
+        raise ValueError("indices / scores do not match num_relevant_tokens")
+    dt = _lib.TS_DTYPE_F32 if scores.dtype == torch.float32 else _lib.TS_DTYPE_BF16
+    _lib.check(_lib.load().ts_paged_matmul(_p(query), _p(token), token.shape[0], _p(indices),
+                                           _p(scores), dt, num_relevant_tokens, num_heads,
+                                           num_kv_heads, head_dim, _stream()))
+
+
+def score(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
+          skip: Optional[torch.Tensor] = None, out: Optional[Tuple] = None):
+    """Scoring pass (tr.py:350-359) + per-head softmax statistics.  Returns
+    ``(scores [B,H,stride] fp32, stats [B,H,2] fp32)``; only the first
+    ``L_b - n_init - n_local`` columns of a non-dense request are written."""
+    c, cb = cfg.to_c(), _c_batch(cfg, bt)
+    _need(qf, "qf", torch.bfloat16)
+    _check_pool(cfg, k_pool, "k_pool")
+    B, H = bt.batch, cfg.num_heads
+    if qf.numel() != B * H * cfg.head_dim:
+        raise ValueError("qf must hold B*H*D elements")
+    if skip is not None:
+        _need(skip, "skip", torch.int32, 1)
+    lib = _lib.load()
+    if out is None:
+        stride = score_stride_for(bt.max_seq_len)
+        scores = torch.empty((B, H, stride), dtype=torch.float32, device=qf.device)
+        stats = torch.empty((B, H, 2), dtype=torch.float32, device=qf.device)
+        ws_bytes = lib.ts_score_workspace_bytes(ctypes.byref(c), B, bt.max_seq_len)
+        ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=qf.device)
+    else:
+        scores, stats, ws = out
+    _lib.check(lib.ts_score(ctypes.byref(c), ctypes.byref(cb), _p(qf), _p(k_pool), k_pool.shape[0],
+                            _p(skip), _p(scores), scores.shape[2], _p(stats), _p(ws), ws.numel(),
+                            _stream()))
+    return scores, stats
+
+
+def vote(cfg: LayerConfig, bt: Batch, scores: torch.Tensor, stats: torch.Tensor,
+         skip: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Soft vote (tr.py:361) and optional max-pool (tr.py:366-369): ``[B, stride]`` fp32."""
+    c, cb = cfg.to_c(), _c_batch(cfg, bt)
+    _need(scores, "scores", torch.float32, 3)
+    _need(stats, "stats", torch.float32, 3)
+    B, H = bt.batch, cfg.num_heads
+    if scores.shape[0] != B or scores.shape[1] != H or tuple(stats.shape) != (B, H, 2):
+        raise ValueError("scores / stats do not match batch / heads")
+    stride = scores.shape[2]
+    votes = torch.empty((B, stride), dtype=torch.float32, device=scores.device)
+    pooled = torch.empty_like(votes) if cfg.pool_kernel > 0 else None
+    _lib.check(_lib.load().ts_vote(ctypes.byref(c), ctypes.byref(cb), _p(scores), stride, _p(stats),
+                                   _p(skip), _p(votes), _p(pooled), stride, _stream()))
+    return pooled if pooled is not None else votes
+
+
+def topk_ragged(cfg: LayerConfig, bt: Batch, votes: torch.Tensor,
+                hit: Optional[torch.Tensor] = None, cache: Optional[SelectionCache] = None):
+    """Top-k + sort + assembly (tr.py:371-373, 433-449).  Returns
+    ``(sel [B,max_sel] int32 physical slots, sel_pos [B,max_sel] int32 logical
+    positions, sel_len [B] int32)``."""
+    c, cb = cfg.to_c(), _c_batch(cfg, bt)
+    _need(votes, "votes", torch.float32, 2)
+    B = bt.batch
+    if votes.shape[0] != B:
+        raise ValueError("votes must have one row per request")
+    if hit is not None:
+        _need(hit, "hit", torch.int32, 1)
+    sel = torch.empty((B, cfg.max_sel), dtype=torch.int32, device=votes.device)
+    sel_pos = torch.empty_like(sel)
+    sel_len = torch.empty((B,), dtype=torch.int32, device=votes.device)
+    ws = torch.empty((256,), dtype=torch.uint8, device=votes.device)
+    _lib.check(_lib.load().ts_topk_ragged(ctypes.byref(c), ctypes.byref(cb), _p(votes),
+                                          votes.shape[1], _p(hit), _c_cache(cache, cfg, B), _p(sel),
+                                          _p(sel_pos), cfg.max_sel, _p(sel_len), _p(ws), ws.numel(),
+                                          _stream()))
+    return sel, sel_pos, sel_len
+
+
+def selcache_step(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, cache: SelectionCache) -> torch.Tensor:
+    """Selection-cache decision (tr.py:394-401, 416-421): ``hit [B]`` int32."""
+    c, cb = cfg.to_c(), _c_batch(cfg, bt)
+    _need(qf, "qf", torch.bfloat16)
+    if qf.numel() != bt.batch * cfg.num_heads * cfg.head_dim:
+        raise ValueError("qf must hold B*H*D elements")
+    hit = torch.empty((bt.batch,), dtype=torch.int32, device=qf.device)
+    _lib.check(_lib.load().ts_selcache_step(ctypes.byref(c), ctypes.byref(cb), _p(qf),
+                                            _c_cache(cache, cfg, bt.batch), _p(hit), _stream()))
+    return hit
+
+
+def sparse_decode_attention(cfg: LayerConfig, q: torch.Tensor, k_pool: torch.Tensor,
+                            v_pool: torch.Tensor, sel: torch.Tensor, sel_len: torch.Tensor,
+                            max_sel_len: Optional[int] = None) -> torch.Tensor:
+    """Decode attention over the selected slots (tr.py:815-823): ``[B, H*D]`` bf16."""
+    c = cfg.to_c()
+    _need(q, "q", torch.bfloat16)
+    _check_pool(cfg, k_pool, "k_pool")
+    _check_pool(cfg, v_pool, "v_pool")
+    _need(sel, "sel", torch.int32, 2)
+    _need(sel_len, "sel_len", torch.int32, 1)
+    B = sel.shape[0]
+    if k_pool.shape != v_pool.shape:
+        raise ValueError("k_pool and v_pool must have the same shape")
+    if q.numel() != B * cfg.num_heads * cfg.head_dim or sel_len.shape[0] != B:
+        raise ValueError("q / sel_len do not match the batch of sel")
+    max_sel_len = sel.shape[1] if max_sel_len is None else int(max_sel_len)
+    if max_sel_len > sel.shape[1]:
+        raise ValueError("max_sel_len exceeds the width of sel")
+    lib = _lib.load()
+    out = torch.empty((B, cfg.num_heads * cfg.head_dim), dtype=torch.bfloat16, device=q.device)
+    ws_bytes = lib.ts_attn_workspace_bytes(ctypes.byref(c), B, max_sel_len)
+    ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=q.device)
+    _lib.check(lib.ts_sparse_decode_attn(ctypes.byref(c), _p(q), _p(k_pool), _p(v_pool),
+                                         k_pool.shape[0], _p(sel), sel.stride(0), _p(sel_len), B,
+                                         max_sel_len, _p(out), _p(ws), ws.numel(), _stream()))
+    return out
+
+
+def kv_store(cfg: LayerConfig, k: torch.Tensor, v: torch.Tensor, out_cache_loc: torch.Tensor,
+             k_pool: torch.Tensor, v_pool: torch.Tensor, table: torch.Tensor,
+             seq_lens: torch.Tensor) -> None:
+    """KV store + table append of a decode step (tr.py:844-854, 332-336)."""
+    c = cfg.to_c()
+    _need(k, "k", torch.bfloat16)
+    _need(v, "v", torch.bfloat16)
+    _need(out_cache_loc, "out_cache_loc", torch.int32, 1)
+    _check_pool(cfg, k_pool, "k_pool")
+    _check_pool(cfg, v_pool, "v_pool")
+    _need(table, "table", torch.int32, 2)
+    _need(seq_lens, "seq_lens", torch.int32, 1)
+    B = out_cache_loc.shape[0]
+    row = cfg.num_kv_heads * cfg.head_dim
+    if k.numel() != B * row or v.numel() != B * row or table.shape[0] != B or seq_lens.shape[0] != B:
+        raise ValueError("k / v / table / seq_lens do not match the batch")
+    _lib.check(_lib.load().ts_kv_store(ctypes.byref(c), _p(k), _p(v), _p(out_cache_loc), _p(k_pool),
+                                       _p(v_pool), k_pool.shape[0], _p(table), table.stride(0),
+                                       _p(seq_lens), B, table.shape[1], _stream()))
+
+
+def scoring_cos_sin(head_dim: int, rope_base: float, rope_scale, n_local: int, device):
+    """Row ``n_local`` of the reference's cos/sin tables (tr.py:75-96), built with
+    the same fp32 torch expressions on the host: ``(cos [1,D], sin [1,D])``."""
+    inv_freq = 1.0 / (rope_base ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    t = torch.arange(n_local + 1)
+    freqs = torch.outer(t * rope_scale, inv_freq)[n_local:n_local + 1]
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.cos().to(device).contiguous(), emb.sin().to(device).contiguous()
+
+
+class DecodeLayer:
+    """One layer of the patched decode forward after the KV store
+    (tr.py:791-825) as a single library call; buffers are allocated once."""
+
+    def __init__(self, cfg: LayerConfig, batch: int, max_seq_len: int, device):
+        self.cfg, self.batch, self.max_seq_len = cfg, batch, max_seq_len
+        self._c = cfg.to_c()
+        lib = _lib.load()
+        nbytes = lib.ts_decode_layer_workspace_bytes(ctypes.byref(self._c), batch, max_seq_len)
+        if nbytes == 0:
+            _lib.check(lib.ts_score(ctypes.byref(self._c), None, None, None, 0, None, None, 0, None,
+                                    None, 0, None))  # surfaces the config error
+        self.workspace = torch.empty((nbytes,), dtype=torch.uint8, device=device)
+        self.q_cos, self.q_sin = scoring_cos_sin(cfg.head_dim, cfg.rope_theta, cfg.rope_scale,
+                                                 cfg.n_local, device)
+        self.out = torch.empty((batch, cfg.num_heads * cfg.head_dim), dtype=torch.bfloat16,
+                               device=device)
+        self.sel = torch.empty((batch, cfg.max_sel), dtype=torch.int32, device=device)
+        self.sel_pos = torch.empty_like(self.sel)
+        self.sel_len = torch.empty((batch,), dtype=torch.int32, device=device)
+
+    def __call__(self, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch,
+                 cache: Optional[SelectionCache] = None):
+        cfg = self.cfg
+        cb = _c_batch(cfg, bt)
+        if bt.batch != self.batch or bt.max_seq_len > self.max_seq_len:
+            raise ValueError("batch / max_seq_len exceed what this DecodeLayer was sized for")
+        _need(q, "q", torch.bfloat16)
+        if q.numel() != self.batch * cfg.num_heads * cfg.head_dim:
+            raise ValueError("q must hold B*H*D elements")
+        _check_pool(cfg, k_pool, "k_pool")
+        _check_pool(cfg, v_pool, "v_pool")
+        if k_pool.shape != v_pool.shape:
+            raise ValueError("k_pool and v_pool must have the same shape")
+        cb.max_seq_len = self.max_seq_len  # keeps the workspace layout fixed across steps
+        _lib.check(_lib.load().ts_decode_layer(
+            ctypes.byref(self._c), ctypes.byref(cb), _p(q), _p(self.q_cos), _p(self.q_sin),
+            _p(k_pool), _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, self.batch), _p(self.out),
+            _p(self.sel), _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
+            self.workspace.numel(), _stream()))
+        return self.out, self.sel, self.sel_pos, self.sel_len
