@@ -92,10 +92,15 @@ typedef struct ts_selcache {
 int ts_version(void);
 const char* ts_last_error(void);
 
+/* TS_OK when the library supports this configuration (head_dim 128; Hkv in
+ * {1,2,4,8}; H/Hkv in {1,2,4,7,8}; power-of-two page size), else the error. */
+int ts_check_config(const ts_config* cfg);
+
 /* RotaryEmbedding.apply_rotary_pos_emb (tr.py:98-107):
  * out = bf16(float(x)*cos[pos] + float(rotate_half(x))*sin[pos]), products and
  * sum rounded separately as torch does.  x, out: [rows, heads, dim] bf16;
- * cos_table, sin_table: [table_rows, dim] fp32; position_ids: [rows] int64. */
+ * cos_table, sin_table: [table_rows, dim] fp32; position_ids: [rows] int64, or
+ * NULL when every row uses table row 0. */
 int ts_rope_apply(const void* x, void* out, const float* cos_table, const float* sin_table,
                   const int64_t* position_ids, int64_t table_rows, int64_t rows,
                   int32_t heads, int32_t dim, ts_stream_t stream);
@@ -109,23 +114,26 @@ int ts_paged_matmul(const void* query, const void* token, int64_t pool_rows,
                     int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
                     ts_stream_t stream);
 
-/* Scoring pass of get_topk_tokens over a ragged batch (tr.py:350-359): for every
- * request that is not dense (n_init+k+n_local >= L, tr.py:377) and whose
- * skip[b] is 0, scores[(b*H+h)*score_stride + t] for candidates t in
- * [0, L-n_init-n_local) and the per-head softmax statistics
- * stats[(b*H+h)*2 + {0,1}] = {max_t s, sum_t exp(s - max)}.
- * qf [B,H,D] bf16 is the rotated fingerprint (tr.py:380-392). */
-size_t ts_score_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+/* Scoring pass of get_topk_tokens over a ragged batch (tr.py:350-359), one
+ * kernel launch: for every request that is not dense (n_init+k+n_local >= L,
+ * tr.py:377) and whose skip[b] is 0, scores[(b*H+h)*score_stride + t] for
+ * candidates t in [0, L-n_init-n_local), and per-workgroup softmax partials
+ * (max, sum exp) that ts_vote merges.  partials holds at least
+ * ts_score_partials_bytes() bytes.  qf [B,H,D] bf16 is the rotated fingerprint
+ * (tr.py:380-392). */
+size_t ts_score_partials_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
 int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
              int64_t pool_rows, const int32_t* skip, float* scores, int64_t score_stride,
-             float* stats, void* workspace, size_t workspace_bytes, ts_stream_t stream);
+             float* partials, size_t partials_bytes, ts_stream_t stream);
 
-/* Soft vote (tr.py:361): votes[b*vote_stride + t] = sum_h exp(s[h,t]-max_h)/Z_h,
- * then the optional max-pool of tr.py:366-369 when cfg->pool_kernel > 0
- * (pooled is then the output and votes the scratch; both [B, vote_stride]). */
+/* Soft vote (tr.py:361): merges the partials into stats[(b*H+h)*2 + {0,1}] =
+ * {max_t s, sum_t exp(s - max)}, then votes[b*vote_stride + t] =
+ * sum_h exp(s[h,t]-max_h)/Z_h, then the optional max-pool of tr.py:366-369 when
+ * cfg->pool_kernel > 0 (pooled is then the result and votes the scratch; both
+ * [B, vote_stride]). */
 int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
-            int64_t score_stride, const float* stats, const int32_t* skip, float* votes,
-            float* pooled, int64_t vote_stride, ts_stream_t stream);
+            int64_t score_stride, const float* partials, const int32_t* skip, float* stats,
+            float* votes, float* pooled, int64_t vote_stride, ts_stream_t stream);
 
 /* Ragged top-k + sort + index assembly (tr.py:371-373, 433-449).  Per request:
  * the k_b largest votes (ties: lowest position first), ascending, offset by

@@ -74,8 +74,8 @@ def test_score_vote_topk(dev, shape, page):
     wl = small(dev, shape, seed=page + shape["num_heads"], lens=lens, ks=ks, page=page, top_k=100)
     c = wl.cfg
     qf = fingerprint(wl, dev)
-    scores, stats = ops.score(c, wl.batch, qf, wl.k_pool)
-    votes = ops.vote(c, wl.batch, scores, stats)
+    scores, partials = ops.score(c, wl.batch, qf, wl.k_pool)
+    votes, stats = ops.vote(c, wl.batch, scores, partials)
     sel, sel_pos, sel_len = ops.topk_ragged(c, wl.batch, votes)
     torch.cuda.synchronize()
     details = []
@@ -199,8 +199,8 @@ def test_max_pool_votes(dev):
         wl = small(dev, SHAPES[0], seed=31, lens=[2500, 900], ks=[64, 64], pool_kernel=kernel)
         c = wl.cfg
         qf = fingerprint(wl, dev)
-        scores, stats = ops.score(c, wl.batch, qf, wl.k_pool)
-        votes = ops.vote(c, wl.batch, scores, stats)
+        scores, partials = ops.score(c, wl.batch, qf, wl.k_pool)
+        votes, stats = ops.vote(c, wl.batch, scores, partials)
         sel, sel_pos, sel_len = ops.topk_ragged(c, wl.batch, votes)
         details = []
         oracle_layer(wl, details)

@@ -87,9 +87,12 @@ int ts_version(void) { return TS_VERSION; }
 
 const char* ts_last_error(void) { return ts::g_error; }
 
+int ts_check_config(const ts_config* cfg) { return validate_config(cfg); }
+
 // Workspace of ts_decode_layer, carved in this order (256-byte aligned pieces).
 struct LayerWorkspace {
-  size_t qf, hit, scores, stats, votes, pooled, score_ws, topk_ws, attn_ws, total;
+  size_t qf, hit, scores, stats, votes, pooled, partials, topk_ws, attn_ws, total;
+  size_t partials_bytes;
   int64_t score_stride;
   int32_t max_sel;
 };
@@ -111,7 +114,8 @@ static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32
   w.stats = take(B * H * 2 * 4);
   w.votes = take(B * (size_t)w.score_stride * 4);
   w.pooled = take(cfg->pool_kernel > 0 ? B * (size_t)w.score_stride * 4 : 0);
-  w.score_ws = take(ts_score_workspace_bytes(cfg, batch, max_seq_len));
+  w.partials_bytes = ts_score_partials_bytes(cfg, batch, max_seq_len);
+  w.partials = take(w.partials_bytes);
   w.topk_ws = take(ts_topk_workspace_bytes(cfg, batch, max_seq_len));
   w.attn_ws = take(ts_attn_workspace_bytes(cfg, batch, w.max_sel));
   w.total = off;
@@ -155,10 +159,11 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
   TS_TRY(ts_rope_apply(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
                        stream));
   if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
-  TS_TRY(ts_score(cfg, bt, qf, k_pool, pool_rows, hit, scores, w.score_stride, stats,
-                  ws + w.score_ws, w.topk_ws - w.score_ws, stream));
-  TS_TRY(ts_vote(cfg, bt, scores, w.score_stride, stats, hit, votes, pooled, w.score_stride,
-                 stream));
+  float* partials = (float*)(ws + w.partials);
+  TS_TRY(ts_score(cfg, bt, qf, k_pool, pool_rows, hit, scores, w.score_stride, partials,
+                  w.partials_bytes, stream));
+  TS_TRY(ts_vote(cfg, bt, scores, w.score_stride, partials, hit, stats, votes, pooled,
+                 w.score_stride, stream));
   TS_TRY(ts_topk_ragged(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache, sel, sel_pos,
                         sel_stride, sel_len, ws + w.topk_ws, w.attn_ws - w.topk_ws, stream));
   TS_TRY(ts_sparse_decode_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len,

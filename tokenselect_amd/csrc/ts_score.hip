@@ -285,25 +285,6 @@ __global__ __launch_bounds__(256, ((HKV >= 4 ? HKV / 4 : 1) * G > 8 ? 2 : TS_SCO
   }
 }
 
-// Merge the per-workgroup softmax partials of one (request, head).
-__global__ __launch_bounds__(64) void score_stats_kernel(ScoreArgs a, float* __restrict__ stats) {
-  const int h = blockIdx.x, b = blockIdx.y;
-  if (a.skip && a.skip[b]) return;
-  ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
-  if (geo.n <= 0) return;
-  const int chunks = (geo.n + a.tokens_per_block - 1) / a.tokens_per_block;
-  const float* p = a.partials + ((size_t)b * a.num_heads + h) * a.nchunks * 2;
-  float m = kNegBig, l = 0.f;
-  for (int c = threadIdx.x; c < chunks; c += 64) softmax_merge(m, l, p[2 * c], p[2 * c + 1]);
-  row16_softmax_merge(m, l);
-  softmax_merge(m, l, __shfl_xor(m, 16), __shfl_xor(l, 16));
-  softmax_merge(m, l, __shfl_xor(m, 32), __shfl_xor(l, 32));
-  if (threadIdx.x == 0) {
-    stats[((size_t)b * a.num_heads + h) * 2] = m;
-    stats[((size_t)b * a.num_heads + h) * 2 + 1] = l;
-  }
-}
-
 template <bool OUT_BF16>
 static int launch_score(int hkv, int group, const ScoreArgs& a, dim3 grid, hipStream_t stream) {
 #define TS_SCORE_CASE(HKV_, G_)                                                              \
@@ -328,7 +309,7 @@ using namespace ts;
 
 extern "C" {
 
-size_t ts_score_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+size_t ts_score_partials_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
   const int tpb = score_tokens_per_block((int64_t)batch * max_seq_len);
   const size_t nchunks = (size_t)ceil_div(max_seq_len, tpb);
@@ -337,18 +318,18 @@ size_t ts_score_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max
 
 int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
              int64_t pool_rows, const int32_t* skip, float* scores, int64_t score_stride,
-             float* stats, void* workspace, size_t workspace_bytes, ts_stream_t stream) {
+             float* partials, size_t partials_bytes, ts_stream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
-  TS_REQUIRE(qf && k_pool && scores && stats, TS_EINVAL, "ts_score: NULL tensor argument");
+  TS_REQUIRE(qf && k_pool && scores && partials, TS_EINVAL, "ts_score: NULL tensor argument");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
   TS_REQUIRE(score_stride >= max_n && score_stride >= 1, TS_EWORKSPACE,
              "score_stride %lld < max candidates %d", (long long)score_stride, max_n);
-  const size_t need = ts_score_workspace_bytes(cfg, bt->batch, bt->max_seq_len);
-  TS_REQUIRE(workspace != nullptr && workspace_bytes >= need, TS_EWORKSPACE,
-             "ts_score: workspace %zu bytes < required %zu", workspace_bytes, need);
+  const size_t need = ts_score_partials_bytes(cfg, bt->batch, bt->max_seq_len);
+  TS_REQUIRE(partials_bytes >= need, TS_EWORKSPACE, "ts_score: partials %zu bytes < required %zu",
+             partials_bytes, need);
   if (max_n <= 0) return TS_OK;  // every request is dense
 
   ScoreArgs a;
@@ -369,17 +350,14 @@ int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const voi
   a.direct_n = -1;
   a.scores = scores;
   a.score_stride = score_stride;
-  a.partials = (float*)workspace;
+  a.partials = partials;
   a.tokens_per_block = score_tokens_per_block((int64_t)bt->batch * bt->max_seq_len);
   a.nchunks = (int)ceil_div(bt->max_seq_len, a.tokens_per_block);
   a.num_heads = cfg->num_heads;
   a.head_map = cfg->head_map;
   const dim3 grid((unsigned)ceil_div(max_n, a.tokens_per_block), (unsigned)bt->batch);
-  TS_TRY(launch_score<false>(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, a, grid,
-                             (hipStream_t)stream));
-  hipLaunchKernelGGL(score_stats_kernel, dim3((unsigned)cfg->num_heads, (unsigned)bt->batch), dim3(64),
-                     0, (hipStream_t)stream, a, stats);
-  return check_launch("score_stats_kernel");
+  return launch_score<false>(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, a, grid,
+                             (hipStream_t)stream);
 }
 
 int ts_paged_matmul(const void* query, const void* token, int64_t pool_rows,

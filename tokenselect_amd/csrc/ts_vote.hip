@@ -9,7 +9,9 @@ constexpr int kMaxHeads = 128;
 struct VoteArgs {
   const float* scores;
   int64_t score_stride;
-  const float* stats;
+  const float* partials;  // [B,H,nchunks,2] from the scoring pass
+  int nchunks, tokens_per_block;
+  float* stats;           // [B,H,2] merged (max, sum exp)
   const int32_t* seq_lens;
   const int32_t* k_per_req;
   const int32_t* skip;
@@ -17,6 +19,25 @@ struct VoteArgs {
   float* votes;
   int64_t vote_stride;
 };
+
+// Merge the per-workgroup softmax partials of one (request, head).
+__global__ __launch_bounds__(64) void stats_merge_kernel(VoteArgs a) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  if (a.skip && a.skip[b]) return;
+  const ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  if (geo.n <= 0) return;
+  const int chunks = (geo.n + a.tokens_per_block - 1) / a.tokens_per_block;
+  const float* p = a.partials + ((size_t)b * a.num_heads + h) * a.nchunks * 2;
+  float m = kNegBig, l = 0.f;
+  for (int c = threadIdx.x; c < chunks; c += 64) softmax_merge(m, l, p[2 * c], p[2 * c + 1]);
+  row16_softmax_merge(m, l);
+  softmax_merge(m, l, __shfl_xor(m, 16), __shfl_xor(l, 16));
+  softmax_merge(m, l, __shfl_xor(m, 32), __shfl_xor(l, 32));
+  if (threadIdx.x == 0) {
+    a.stats[((size_t)b * a.num_heads + h) * 2] = m;
+    a.stats[((size_t)b * a.num_heads + h) * 2 + 1] = l;
+  }
+}
 
 // One thread per candidate, heads visited in ascending order (fp32 sum).
 __global__ __launch_bounds__(256) void vote_kernel(VoteArgs a) {
@@ -82,11 +103,12 @@ __global__ __launch_bounds__(256) void pool_kernel(PoolArgs a) {
 using namespace ts;
 
 extern "C" int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
-                       int64_t score_stride, const float* stats, const int32_t* skip, float* votes,
-                       float* pooled, int64_t vote_stride, ts_stream_t stream) {
+                       int64_t score_stride, const float* partials, const int32_t* skip,
+                       float* stats, float* votes, float* pooled, int64_t vote_stride,
+                       ts_stream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
-  TS_REQUIRE(scores && stats && votes, TS_EINVAL, "ts_vote: NULL tensor argument");
+  TS_REQUIRE(scores && partials && stats && votes, TS_EINVAL, "ts_vote: NULL tensor argument");
   TS_REQUIRE(cfg->num_heads <= kMaxHeads, TS_ESHAPE, "num_heads %d > %d", cfg->num_heads, kMaxHeads);
   TS_REQUIRE(cfg->pool_kernel <= 0 || pooled != nullptr, TS_EINVAL,
              "ts_vote: pool_kernel %d needs a pooled buffer", cfg->pool_kernel);
@@ -99,6 +121,9 @@ extern "C" int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* sc
   VoteArgs a;
   a.scores = scores;
   a.score_stride = score_stride;
+  a.partials = partials;
+  a.tokens_per_block = score_tokens_per_block((int64_t)bt->batch * bt->max_seq_len);
+  a.nchunks = (int)ceil_div(bt->max_seq_len, a.tokens_per_block);
   a.stats = stats;
   a.seq_lens = bt->seq_lens;
   a.k_per_req = bt->k_per_req;
@@ -110,6 +135,9 @@ extern "C" int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* sc
   a.num_heads = cfg->num_heads;
   a.votes = votes;
   a.vote_stride = vote_stride;
+  hipLaunchKernelGGL(stats_merge_kernel, dim3((unsigned)cfg->num_heads, (unsigned)bt->batch), dim3(64),
+                     0, (hipStream_t)stream, a);
+  TS_TRY(check_launch("stats_merge_kernel"));
   hipLaunchKernelGGL(vote_kernel, dim3((unsigned)ceil_div(max_n, 1024), (unsigned)bt->batch),
                      dim3(256), 0, (hipStream_t)stream, a);
   TS_TRY(check_launch("vote_kernel"));

@@ -198,9 +198,10 @@ def paged_matmul(query: torch.Tensor, token: torch.Tensor, indices: torch.Tensor
 
 def score(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
           skip: Optional[torch.Tensor] = None, out: Optional[Tuple] = None):
-    """Scoring pass (tr.py:350-359) + per-head softmax statistics.  Returns
-    ``(scores [B,H,stride] fp32, stats [B,H,2] fp32)``; only the first
-    ``L_b - n_init - n_local`` columns of a non-dense request are written."""
+    """Scoring pass (tr.py:350-359), one kernel launch.  Returns ``(scores
+    [B,H,stride] fp32, partials)``; only the first ``L_b - n_init - n_local``
+    columns of a non-dense request are written.  ``partials`` are the
+    per-workgroup softmax statistics that :func:`vote` merges."""
     c, cb = cfg.to_c(), _c_batch(cfg, bt)
     _need(qf, "qf", torch.bfloat16)
     _check_pool(cfg, k_pool, "k_pool")
@@ -213,32 +214,38 @@ def score(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
     if out is None:
         stride = score_stride_for(bt.max_seq_len)
         scores = torch.empty((B, H, stride), dtype=torch.float32, device=qf.device)
-        stats = torch.empty((B, H, 2), dtype=torch.float32, device=qf.device)
-        ws_bytes = lib.ts_score_workspace_bytes(ctypes.byref(c), B, bt.max_seq_len)
-        ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=qf.device)
+        nbytes = lib.ts_score_partials_bytes(ctypes.byref(c), B, bt.max_seq_len)
+        partials = torch.empty((max(nbytes, 256) // 4,), dtype=torch.float32, device=qf.device)
     else:
-        scores, stats, ws = out
+        scores, partials = out
+        _need(scores, "scores", torch.float32, 3)
+        _need(partials, "partials", torch.float32, 1)
     _lib.check(lib.ts_score(ctypes.byref(c), ctypes.byref(cb), _p(qf), _p(k_pool), k_pool.shape[0],
-                            _p(skip), _p(scores), scores.shape[2], _p(stats), _p(ws), ws.numel(),
-                            _stream()))
-    return scores, stats
+                            _p(skip), _p(scores), scores.shape[2], _p(partials),
+                            partials.numel() * 4, _stream()))
+    return scores, partials
 
 
-def vote(cfg: LayerConfig, bt: Batch, scores: torch.Tensor, stats: torch.Tensor,
-         skip: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Soft vote (tr.py:361) and optional max-pool (tr.py:366-369): ``[B, stride]`` fp32."""
+def vote(cfg: LayerConfig, bt: Batch, scores: torch.Tensor, partials: torch.Tensor,
+         skip: Optional[torch.Tensor] = None):
+    """Soft vote (tr.py:361) and optional max-pool (tr.py:366-369).  Returns
+    ``(votes [B, stride] fp32, stats [B,H,2] fp32 = per-head (max, sum exp))``."""
     c, cb = cfg.to_c(), _c_batch(cfg, bt)
     _need(scores, "scores", torch.float32, 3)
-    _need(stats, "stats", torch.float32, 3)
+    _need(partials, "partials", torch.float32, 1)
     B, H = bt.batch, cfg.num_heads
-    if scores.shape[0] != B or scores.shape[1] != H or tuple(stats.shape) != (B, H, 2):
-        raise ValueError("scores / stats do not match batch / heads")
+    if scores.shape[0] != B or scores.shape[1] != H:
+        raise ValueError("scores do not match batch / heads")
+    lib = _lib.load()
+    if partials.numel() * 4 < lib.ts_score_partials_bytes(ctypes.byref(c), B, bt.max_seq_len):
+        raise ValueError("partials buffer is smaller than ts_score_partials_bytes()")
     stride = scores.shape[2]
+    stats = torch.empty((B, H, 2), dtype=torch.float32, device=scores.device)
     votes = torch.empty((B, stride), dtype=torch.float32, device=scores.device)
     pooled = torch.empty_like(votes) if cfg.pool_kernel > 0 else None
-    _lib.check(_lib.load().ts_vote(ctypes.byref(c), ctypes.byref(cb), _p(scores), stride, _p(stats),
-                                   _p(skip), _p(votes), _p(pooled), stride, _stream()))
-    return pooled if pooled is not None else votes
+    _lib.check(lib.ts_vote(ctypes.byref(c), ctypes.byref(cb), _p(scores), stride, _p(partials),
+                           _p(skip), _p(stats), _p(votes), _p(pooled), stride, _stream()))
+    return (pooled if pooled is not None else votes), stats
 
 
 def topk_ragged(cfg: LayerConfig, bt: Batch, votes: torch.Tensor,
@@ -343,10 +350,8 @@ class DecodeLayer:
         self.cfg, self.batch, self.max_seq_len = cfg, batch, max_seq_len
         self._c = cfg.to_c()
         lib = _lib.load()
+        _lib.check(lib.ts_check_config(ctypes.byref(self._c)))
         nbytes = lib.ts_decode_layer_workspace_bytes(ctypes.byref(self._c), batch, max_seq_len)
-        if nbytes == 0:
-            _lib.check(lib.ts_score(ctypes.byref(self._c), None, None, None, 0, None, None, 0, None,
-                                    None, 0, None))  # surfaces the config error
         self.workspace = torch.empty((nbytes,), dtype=torch.uint8, device=device)
         self.q_cos, self.q_sin = scoring_cos_sin(cfg.head_dim, cfg.rope_theta, cfg.rope_scale,
                                                  cfg.n_local, device)
@@ -369,6 +374,8 @@ class DecodeLayer:
         _check_pool(cfg, v_pool, "v_pool")
         if k_pool.shape != v_pool.shape:
             raise ValueError("k_pool and v_pool must have the same shape")
+        if bt.table.shape[1] * cfg.page_size < self.max_seq_len:
+            raise ValueError("table rows must address the max_seq_len this DecodeLayer was sized for")
         cb.max_seq_len = self.max_seq_len  # keeps the workspace layout fixed across steps
         _lib.check(_lib.load().ts_decode_layer(
             ctypes.byref(self._c), ctypes.byref(cb), _p(q), _p(self.q_cos), _p(self.q_sin),
