@@ -1,0 +1,134 @@
+"""CPU-side checks of the C ABI: the built library loads without a GPU, exports
+every symbol ``include/tokenselect.h`` declares, and rejects bad arguments on the
+host (before any HIP call) with the documented error codes."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from tokenselect_amd import _lib, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_lib.LIB_PATH):
+        from tokenselect_amd import build
+        build.build(verbose=False)
+    return _lib.load()
+
+
+def cfg(**kw):
+    base = dict(num_heads=32, num_kv_heads=8, head_dim=128, page_size=1, n_init=128, n_local=512,
+                top_k=2048, pool_kernel=-1, head_map=0, rope_mode=1, rope_theta=5e5, rope_scale=1.0,
+                sm_scale=0.088, logit_cap=0.0)
+    base.update(kw)
+    return _lib.TsConfig(*[base[name] for name, _ in _lib.TsConfig._fields_])
+
+
+def err(lib):
+    return lib.ts_last_error().decode()
+
+
+def test_header_symbols_are_exported_and_bound(lib):
+    header = open(os.path.join(ROOT, "include", "tokenselect.h")).read()
+    declared = set(re.findall(r"\b(ts_[a-z_]+)\s*\(", header))
+    assert declared, "no declarations found in the header"
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+    assert declared == set(_lib.SIGNATURES), "ctypes signatures and header disagree"
+    assert lib.ts_version() == int(re.search(r"#define TS_VERSION (\d+)", header).group(1))
+
+
+def test_struct_layouts_match_the_header():
+    assert ctypes.sizeof(_lib.TsConfig) == 14 * 4
+    assert ctypes.sizeof(_lib.TsBatch) == 8 + 8 + 8 + 8 + 8
+    assert _lib.TsBatch.seq_lens.offset == 8 and _lib.TsBatch.table_stride.offset == 24
+    assert ctypes.sizeof(_lib.TsSelCache) == 4 * 8 + 8
+
+
+def test_config_validation(lib):
+    assert lib.ts_check_config(ctypes.byref(cfg())) == _lib.TS_OK
+    assert lib.ts_check_config(None) == _lib.TS_EINVAL
+    assert lib.ts_check_config(ctypes.byref(cfg(head_dim=64))) == _lib.TS_ESHAPE
+    assert "head_dim 64" in err(lib)
+    assert lib.ts_check_config(ctypes.byref(cfg(num_heads=30))) == _lib.TS_ESHAPE
+    assert lib.ts_check_config(ctypes.byref(cfg(num_heads=24, num_kv_heads=8))) == _lib.TS_ESHAPE
+    assert lib.ts_check_config(ctypes.byref(cfg(page_size=12))) == _lib.TS_EINVAL
+    assert lib.ts_check_config(ctypes.byref(cfg(top_k=0))) == _lib.TS_EINVAL
+    assert lib.ts_check_config(ctypes.byref(cfg(rope_mode=7))) == _lib.TS_EINVAL
+    assert lib.ts_check_config(ctypes.byref(cfg(rope_theta=0.0))) == _lib.TS_EINVAL
+    for hkv, g in [(1, 8), (2, 2), (4, 7), (8, 4), (8, 8), (4, 1)]:
+        assert lib.ts_check_config(ctypes.byref(cfg(num_heads=hkv * g, num_kv_heads=hkv))) == 0
+
+
+def test_workspace_queries(lib):
+    c = cfg()
+    assert lib.ts_decode_layer_workspace_bytes(ctypes.byref(c), 1, 131072) > 32 * 131072 * 4
+    assert lib.ts_decode_layer_workspace_bytes(ctypes.byref(cfg(head_dim=64)), 1, 1024) == 0
+    assert lib.ts_score_partials_bytes(ctypes.byref(c), 1, 131072) % 256 == 0
+    assert lib.ts_attn_workspace_bytes(ctypes.byref(c), 4, 2688) > 0
+
+
+def test_null_and_range_errors_need_no_gpu(lib):
+    c = cfg()
+    one = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
+    bt = _lib.TsBatch(1, 4096, one, one, 4096, None)
+    assert lib.ts_score(ctypes.byref(c), None, one, one, 10, None, one, 4096, one, 1 << 20,
+                        None) == _lib.TS_EINVAL
+    assert lib.ts_score(ctypes.byref(c), ctypes.byref(bt), None, one, 10, None, one, 4096, one,
+                        1 << 20, None) == _lib.TS_EINVAL
+    assert "NULL" in err(lib)
+    # score stride smaller than the candidate count
+    assert lib.ts_score(ctypes.byref(c), ctypes.byref(bt), one, one, 10, None, one, 100, one,
+                        1 << 20, None) == _lib.TS_EWORKSPACE
+    # partials buffer too small
+    assert lib.ts_score(ctypes.byref(c), ctypes.byref(bt), one, one, 10, None, one, 4096, one, 16,
+                        None) == _lib.TS_EWORKSPACE
+    bad = _lib.TsBatch(0, 4096, one, one, 4096, None)
+    assert lib.ts_vote(ctypes.byref(c), ctypes.byref(bad), one, 4096, one, None, one, one, None,
+                       4096, None) == _lib.TS_EINVAL
+    # table rows too short for a batch of 2
+    short = _lib.TsBatch(2, 4096, one, one, 100, None)
+    assert lib.ts_topk_ragged(ctypes.byref(c), ctypes.byref(short), one, 4096, None, None, one, one,
+                              4096, one, one, 256, None) == _lib.TS_EINVAL
+    # sel_stride below n_init + top_k + n_local
+    assert lib.ts_topk_ragged(ctypes.byref(c), ctypes.byref(bt), one, 4096, None, None, one, one,
+                              100, one, one, 256, None) == _lib.TS_EWORKSPACE
+    # hit flags without a cache
+    assert lib.ts_topk_ragged(ctypes.byref(c), ctypes.byref(bt), one, 4096, one, None, one, one,
+                              4096, one, one, 256, None) == _lib.TS_EINVAL
+    assert lib.ts_sparse_decode_attn(ctypes.byref(c), one, one, one, 10, one, 4096, one, 1, 2688,
+                                     one, one, 16, None) == _lib.TS_EWORKSPACE
+    assert lib.ts_paged_matmul(one, one, 10, one, one, 5, 10, 32, 8, 128, None) == _lib.TS_EINVAL
+    assert lib.ts_paged_matmul(one, one, 10, one, one, 0, 10, 32, 8, 64, None) == _lib.TS_ESHAPE
+    assert lib.ts_rope_apply(one, one, one, one, None, 1, 1, 4, 127, None) == _lib.TS_ESHAPE
+    assert lib.ts_kv_store(ctypes.byref(cfg(page_size=16)), one, one, one, one, one, 10, one, 100,
+                           one, 1, 100, None) == _lib.TS_EINVAL
+    assert lib.ts_decode_layer(ctypes.byref(c), ctypes.byref(bt), one, one, one, one, one, 10, None,
+                               one, one, one, 4096, one, one, 64, None) == _lib.TS_EWORKSPACE
+    assert "workspace" in err(lib)
+
+
+def test_python_layer_refuses_cpu_tensors(lib):
+    c = ops.LayerConfig(num_heads=4, num_kv_heads=2, n_init=1, n_local=2, top_k=4)
+    x = torch.zeros(1, 4, 128, dtype=torch.bfloat16)
+    t = torch.zeros(4, 128)
+    with pytest.raises(ValueError, match="no CPU path"):
+        ops.rope_apply(x, t, t, None)
+    bt = ops.Batch(torch.zeros(1, dtype=torch.int32), torch.zeros(1, 64, dtype=torch.int32), 64)
+    with pytest.raises(ValueError, match="no CPU path"):
+        ops.score(c, bt, x, torch.zeros(64, 2, 128, dtype=torch.bfloat16))
+    with pytest.raises(TypeError):
+        ops.rope_apply(x.float(), t, t, None)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libtokenselect_hip.so"))
+    with pytest.raises(ImportError, match="no CPU fallback"):
+        _lib.load()

@@ -1,0 +1,348 @@
+"""Pins the CPU oracle.  The reference has no tests, golden vectors or fixtures
+for this path, and its module cannot be imported here (SGLang / vLLM /
+FlashInfer / CUDA), so every oracle function is checked against something the
+mathematics fixes: an independent formulation, a library routine, a closed
+form, an invariant, or brute force on tiny inputs.  None of the checks retypes
+the oracle's own expression."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from oracle import attend, rope, selcache, select
+
+
+def rnd(*shape, seed=0, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g).to(dtype)
+
+
+# ------------------------------------------------------------------- RoPE
+def complex_rope(x, pos, base, scale=1.0):
+    """Independent formulation: pair (i, i+D/2) is a complex number multiplied by
+    exp(i * pos * scale * base^(-2i/D)), evaluated in float64."""
+    d = x.shape[-1]
+    half = d // 2
+    xc = torch.complex(x[..., :half].double(), x[..., half:].double())
+    freq = torch.tensor([base ** (-2.0 * i / d) for i in range(half)], dtype=torch.float64)
+    ang = pos.double().view(-1, 1, 1) * scale * freq
+    rot = xc * torch.polar(torch.ones_like(ang), ang)
+    return torch.cat((rot.real, rot.imag), dim=-1)
+
+
+@pytest.mark.parametrize("base", [1e4, 5e5, 1e6])
+def test_rope_matches_complex_multiplication(base):
+    x = rnd(7, 3, 128, seed=1, dtype=torch.float32)
+    pos = torch.tensor([0, 1, 2, 17, 512, 513, 4000])
+    got = rope.apply(x, pos, base)
+    ref = complex_rope(x, pos, base)
+    # fp32 tables: angle error ~ pos * 2^-24, so compare at 1e-3 absolute for pos <= 4000
+    assert (got.double() - ref).abs().max() < 2e-3
+    assert (got[:5].double() - ref[:5]).abs().max() < 2e-4
+
+
+def test_rope_position_zero_is_identity_and_norm_is_kept():
+    x = rnd(4, 2, 128, seed=2)
+    assert torch.equal(rope.apply(x, torch.zeros(4, dtype=torch.long), 5e5), x)
+    xf = x.float()
+    y = rope.apply(xf, torch.tensor([5, 77, 512, 1023]), 5e5)
+    pair_norm = lambda t: t[..., :64] ** 2 + t[..., 64:] ** 2
+    assert torch.allclose(pair_norm(y), pair_norm(xf), rtol=1e-5, atol=1e-5)
+
+
+def test_rope_relative_position_property():
+    q, k = rnd(1, 4, 128, seed=3, dtype=torch.float32), rnd(1, 4, 128, seed=4, dtype=torch.float32)
+    for a, b in [(512, 100), (30, 29), (700, 0)]:
+        lhs = (rope.apply(q, torch.tensor([a]), 1e4) * rope.apply(k, torch.tensor([b]), 1e4)).sum(-1)
+        rhs = (rope.apply(q, torch.tensor([a - b]), 1e4) * k).sum(-1)
+        assert torch.allclose(lhs, rhs, rtol=1e-4, atol=1e-3)
+
+
+def test_rope_distance_scale_multiplies_the_position():
+    x = rnd(1, 2, 128, seed=5, dtype=torch.float32)
+    assert torch.allclose(rope.apply(x, torch.tensor([6]), 1e4, distance_scale=2),
+                          rope.apply(x, torch.tensor([12]), 1e4), atol=1e-5)
+
+
+def test_scoring_query_rotates_to_n_local_and_rounds_to_bf16():
+    q = rnd(1, 4 * 128, seed=6)
+    qf = rope.scoring_query(q, 4, 128, 512, 5e5)
+    assert qf.dtype == torch.bfloat16 and qf.shape == (512,)
+    ref = complex_rope(q.view(1, 4, 128).float(), torch.tensor([512]), 5e5).view(-1)
+    assert (qf.double() - ref).abs().max() < 0.02  # one bf16 rounding of values ~N(0,1)
+    # two rows: positions n_local and n_local+1, then the mean over rows
+    q2 = rnd(2, 4 * 128, seed=7)
+    qf2 = rope.scoring_query(q2, 4, 128, 16, 1e4)
+    ref2 = complex_rope(q2.view(2, 4, 128).float(), torch.tensor([16, 17]), 1e4).view(2, -1).mean(0)
+    assert (qf2.double() - ref2).abs().max() < 0.03
+
+
+# ------------------------------------------------------------------ score
+def brute_score(qf, k_pool, cand, mapping):
+    H, D = qf.shape
+    out = torch.zeros(H, len(cand), dtype=torch.float64)
+    for h in range(H):
+        for t, slot in enumerate(cand.tolist()):
+            acc = 0.0
+            for d in range(D):
+                acc += float(qf[h, d]) * float(k_pool[slot, mapping(h), d])
+            out[h, t] = acc
+    return out
+
+
+def test_score_brute_force_and_head_map_discriminator():
+    H, Hkv, D, P = 4, 2, 16, 12
+    qf, k_pool = rnd(H, D, seed=8), rnd(P, Hkv, D, seed=9)
+    cand = torch.tensor([5, 0, 11, 3, 7], dtype=torch.int32)
+    got = select.score(qf, k_pool, cand)
+    mod = brute_score(qf, k_pool, cand, lambda h: h % Hkv)
+    div = brute_score(qf, k_pool, cand, lambda h: h // (H // Hkv))
+    assert (got.double() - mod).abs().max() < 1e-5           # the reference's h % Hkv
+    assert (got.double() - div).abs().max() > 0.5            # and NOT the conventional h // G
+    assert (select.score(qf, k_pool, cand, head_map="div").double() - div).abs().max() < 1e-5
+
+
+def test_score_one_hot_known_answers_and_no_scaling():
+    H, Hkv, D, P = 4, 2, 128, 6
+    k_pool = torch.zeros(P, Hkv, D, dtype=torch.bfloat16)
+    k_pool[3, 1, 10] = 2.0
+    k_pool[4, 0, 127] = -3.0
+    qf = torch.zeros(H, D, dtype=torch.bfloat16)
+    qf[1, 10] = 1.5      # head 1 -> kv head 1
+    qf[2, 127] = 4.0     # head 2 -> kv head 0
+    s = select.score(qf, k_pool, torch.arange(P, dtype=torch.int32))
+    expect = torch.zeros(H, P)
+    expect[1, 3] = 3.0   # raw dot product: no 1/sqrt(D)
+    expect[2, 4] = -12.0
+    expect[3, 3] = 0.0
+    assert torch.equal(s, expect)
+
+
+def test_score_follows_the_table_not_the_pool_order():
+    qf, k_pool = rnd(8, 128, seed=10), rnd(64, 2, 128, seed=11)
+    perm = torch.randperm(64, generator=torch.Generator().manual_seed(1))
+    cand = torch.arange(40, dtype=torch.int32)
+    base = select.score(qf, k_pool, cand)
+    shuffled_pool = torch.empty_like(k_pool)
+    shuffled_pool[perm] = k_pool                      # row r moves to slot perm[r]
+    assert torch.equal(select.score(qf, shuffled_pool, perm[:40].int()), base)
+
+
+def test_ref_rounding_mode_is_bf16_and_close():
+    qf, k_pool = rnd(4, 128, seed=12), rnd(50, 2, 128, seed=13)
+    cand = torch.arange(50, dtype=torch.int32)
+    s32 = select.score(qf, k_pool, cand)
+    s16 = select.score(qf, k_pool, cand, mode="ref_rounding")
+    assert s16.dtype == torch.bfloat16
+    assert (s16.float() - s32).abs().max() < 0.02 * s32.abs().max()
+    assert select.vote(s16).dtype == torch.bfloat16
+
+
+# ------------------------------------------------------------- vote / pool
+def test_vote_mass_shift_invariance_and_single_head():
+    s = rnd(6, 300, seed=14, dtype=torch.float32) * 5
+    c = select.vote(s)
+    assert abs(c.sum().item() - 6.0) < 1e-4                   # each head contributes mass 1
+    shifted = s + torch.tensor([3.0, -7.0, 0.0, 100.0, -50.0, 1.0]).view(6, 1)
+    assert torch.allclose(select.vote(shifted), c, rtol=1e-4, atol=1e-7)
+    one = s[:1]
+    e = torch.exp(one[0].double() - one[0].double().max())
+    assert torch.allclose(select.vote(one).double(), e / e.sum(), rtol=1e-5, atol=1e-9)
+
+
+@pytest.mark.parametrize("kernel", [1, 2, 5, 6, 32])
+def test_max_pool_matches_naive_window(kernel):
+    v = torch.rand(97, generator=torch.Generator().manual_seed(kernel))
+    got = select.max_pool(v, kernel)
+    pad = (kernel - 1) // 2
+    n_out = 97 + 2 * pad - kernel + 1
+    assert got.shape[0] == n_out == (97 if kernel % 2 else 96)   # even kernels lose one element
+    for t in (0, 1, n_out // 2, n_out - 1):
+        lo, hi = max(t - pad, 0), min(t - pad + kernel, 97)
+        assert got[t].item() == v[lo:hi].max().item()
+    assert select.max_pool(v, -1) is v and select.max_pool(v, 0) is v
+
+
+# ------------------------------------------------------------------- top-k
+def test_topk_sorted_against_argsort_and_extremes():
+    v = torch.rand(500, generator=torch.Generator().manual_seed(15))
+    for k in (1, 7, 499):
+        ref = sorted(sorted(range(500), key=lambda i: -v[i].item())[:k])
+        got = select.topk_sorted(v, k)
+        assert got.tolist() == ref
+        assert got.dtype == torch.int64
+    planted = torch.zeros(100)
+    planted[[3, 50, 99]] = torch.tensor([5.0, 7.0, 6.0])
+    assert select.topk_sorted(planted, 3).tolist() == [3, 50, 99]
+
+
+# ---------------------------------------------------------------- assembly
+def test_assemble_structure_and_dense_rule():
+    L, n_init, n_local, k = 100, 4, 8, 5
+    tab = (torch.arange(L, dtype=torch.int32) * 3 + 1)
+    top = torch.tensor([10, 20, 21, 50, 91])
+    out = select.assemble(tab, L, n_init, n_local, top)
+    assert out.shape[0] == n_init + k + n_local and out.dtype == torch.int32
+    assert out[:n_init].tolist() == [1, 4, 7, 10]
+    assert out[-n_local:].tolist() == [(L - n_local + i) * 3 + 1 for i in range(n_local)]
+    assert out[n_init:n_init + k].tolist() == [t * 3 + 1 for t in top.tolist()]
+    ident = torch.arange(L, dtype=torch.int32)
+    assert select.assemble(ident, L, n_init, n_local, top)[n_init:n_init + k].tolist() == top.tolist()
+    assert select.is_dense(17, 4, 8, 5) and not select.is_dense(18, 4, 8, 5)
+
+
+def test_retrieval_indices_end_to_end_small():
+    H, Hkv, D, P, L = 4, 2, 128, 300, 200
+    n_init, n_local, k = 4, 8, 16
+    k_pool = rnd(P, Hkv, D, seed=16)
+    q = rnd(1, H * D, seed=17)
+    tab = torch.randperm(P, generator=torch.Generator().manual_seed(2))[:L].int()
+    assert select.retrieval_indices(q, k_pool, tab, n_init + k + n_local, H, D, n_init, n_local, k,
+                                    1e4) is None
+    d = {}
+    out = select.retrieval_indices(q, k_pool, tab, L, H, D, n_init, n_local, k, 1e4, detail=d)
+    assert out.shape[0] == n_init + k + n_local
+    assert out[:n_init].tolist() == tab[:n_init].tolist()
+    assert out[-n_local:].tolist() == tab[L - n_local:L].tolist()
+    top = d["top_pos"]
+    assert top.min() >= n_init and top.max() < L - n_local
+    assert bool((top[1:] > top[:-1]).all())
+    # independent recomputation: float64 softmax votes over the candidate rows
+    qf = complex_rope(q.view(1, H, D).float(), torch.tensor([n_local]), 1e4)[0].to(torch.bfloat16)
+    cand = tab[n_init:L - n_local].long()
+    s = torch.stack([k_pool[cand, h % Hkv].double() @ qf[h].double() for h in range(H)])
+    votes = torch.softmax(s, -1).sum(0)
+    ref = torch.sort(torch.topk(votes, k).indices).values + n_init
+    assert top.tolist() == ref.tolist()
+
+
+def test_planted_tokens_dominate_the_selection():
+    """Known answer: candidates shifted far along every query's direction must all be selected."""
+    H, Hkv, D, P, L = 8, 2, 128, 600, 600
+    n_init, n_local, k = 8, 16, 32
+    g = torch.Generator().manual_seed(18)
+    k_pool = torch.randn(P, Hkv, D, generator=g).bfloat16()
+    q = torch.randn(1, H * D, generator=g).bfloat16()
+    tab = torch.arange(L, dtype=torch.int32)
+    qf = rope.scoring_query(q, H, D, n_local, 1e4).view(H, D).float()
+    planted = torch.randperm(L - n_init - n_local, generator=g)[:k] + n_init
+    for kvh in range(Hkv):
+        direction = qf[kvh::Hkv].mean(0)
+        k_pool[planted, kvh] = (k_pool[planted, kvh].float()
+                                + 12.0 * direction / direction.norm()).bfloat16()
+    d = {}
+    select.retrieval_indices(q, k_pool, tab, L, H, D, n_init, n_local, k, 1e4, detail=d)
+    assert sorted(d["top_pos"].tolist()) == sorted(planted.tolist())
+
+
+def test_expand_page_table():
+    pt = torch.tensor([7, 2, 9], dtype=torch.int32)
+    assert select.expand_page_table(pt, 10, 4).tolist() == [28, 29, 30, 31, 8, 9, 10, 11, 36, 37]
+    assert select.expand_page_table(pt, 3, 1).tolist() == [7, 2, 9]
+
+
+# --------------------------------------------------------------- attention
+def sdpa_reference(q, k_pool, v_pool, slots, scale):
+    H, Hkv = q.shape[0], k_pool.shape[1]
+    k = k_pool[slots.long()].float().permute(1, 0, 2).repeat_interleave(H // Hkv, dim=0)
+    v = v_pool[slots.long()].float().permute(1, 0, 2).repeat_interleave(H // Hkv, dim=0)
+    return F.scaled_dot_product_attention(q.float().unsqueeze(1), k, v, scale=scale).squeeze(1)
+
+
+def test_attention_without_rope_is_textbook_sdpa_with_standard_gqa():
+    H, Hkv, D, P = 8, 2, 128, 90
+    q, k_pool, v_pool = rnd(H, D, seed=19), rnd(P, Hkv, D, seed=20), rnd(P, Hkv, D, seed=21)
+    slots = torch.randperm(P, generator=torch.Generator().manual_seed(3))[:40].int()
+    got = attend.sparse_decode_attention(q, k_pool, v_pool, slots, D ** -0.5, 1e4, rope_mode="NONE")
+    ref = sdpa_reference(q, k_pool, v_pool, slots, D ** -0.5)
+    assert got.dtype == torch.bfloat16
+    assert (got.float() - ref).abs().max() < 1e-2
+    full = attend.sparse_decode_attention(q, k_pool, v_pool, torch.arange(P, dtype=torch.int32),
+                                          D ** -0.5, 1e4, rope_mode="NONE")
+    assert (full.float() - sdpa_reference(q, k_pool, v_pool, torch.arange(P), D ** -0.5)).abs().max() < 1e-2
+
+
+def test_attention_rope_positions_are_list_indices():
+    """Rotating q to S-1 and key j to j equals SDPA on tensors rotated by the
+    independent complex formulation; a common position offset changes nothing."""
+    H, Hkv, D, P, S = 4, 2, 128, 70, 33
+    q, k_pool, v_pool = rnd(H, D, seed=22), rnd(P, Hkv, D, seed=23), rnd(P, Hkv, D, seed=24)
+    slots = torch.randperm(P, generator=torch.Generator().manual_seed(4))[:S].int()
+    got = attend.sparse_decode_attention(q, k_pool, v_pool, slots, D ** -0.5, 5e5, rope_scale=1.0)
+    for offset in (0, 1000):
+        qr = complex_rope(q.float().unsqueeze(0), torch.tensor([S - 1 + offset]), 5e5)[0]
+        kr = complex_rope(k_pool[slots.long()].float(), torch.arange(S) + offset, 5e5)
+        logits = torch.einsum("hd,shd->hs", qr, kr[:, torch.arange(H) // (H // Hkv)]) * D ** -0.5
+        ref = torch.einsum("hs,shd->hd", torch.softmax(logits, -1),
+                           v_pool[slots.long()].double()[:, torch.arange(H) // (H // Hkv)])
+        assert (got.double() - ref).abs().max() < 1e-2
+    scaled = attend.sparse_decode_attention(q, k_pool, v_pool, slots, D ** -0.5, 5e5, rope_scale=4.0)
+    assert (scaled.float() - got.float()).abs().max() > 1e-3   # rope_scale divides the angle
+
+
+def test_attention_soft_cap():
+    H, Hkv, D, P = 4, 2, 128, 40
+    q, k_pool, v_pool = rnd(H, D, seed=25), rnd(P, Hkv, D, seed=26), rnd(P, Hkv, D, seed=27)
+    slots = torch.arange(P, dtype=torch.int32)
+    plain = attend.sparse_decode_attention(q, k_pool, v_pool, slots, 1.0, 1e4, rope_mode="NONE")
+    huge = attend.sparse_decode_attention(q, k_pool, v_pool, slots, 1.0, 1e4, 1.0, 1e6, "NONE")
+    assert (plain.float() - huge.float()).abs().max() < 2e-2   # cap >> logits: no effect
+    tight = attend.sparse_decode_attention(q, k_pool, v_pool, slots, 1.0, 1e4, 1.0, 1.0, "NONE")
+    k = k_pool.float()[:, torch.arange(H) // 2]
+    logits = torch.tanh(torch.einsum("hd,shd->hs", q.float(), k))
+    ref = torch.einsum("hs,shd->hd", torch.softmax(logits, -1), v_pool.float()[:, torch.arange(H) // 2])
+    assert (tight.float() - ref).abs().max() < 1e-2
+
+
+# --------------------------------------------------------- selection cache
+def test_selection_cache_state_machine():
+    assert selcache.THRESHOLD == 0.8984375
+    q = rnd(512, seed=28)
+    calls = []
+    sel = lambda: (calls.append(1), torch.tensor([len(calls)]))[1]
+    c = selcache.SelectionCache()
+    top, hit = c.step(q, sel)
+    assert not hit and top.tolist() == [1]                     # first query always selects
+    top, hit = c.step(q, sel)
+    assert hit and top.tolist() == [1] and c.skip_count == 1   # cos(q, q) = 1
+    top, hit = c.step(-q, sel)
+    assert not hit and top.tolist() == [2]                     # cos = -1
+    ortho = rnd(512, seed=29)
+    ortho = (ortho.float() - (ortho.float() @ (-q).float()) / (q.float() @ q.float()) * (-q).float())
+    top, hit = c.step(ortho.bfloat16(), sel)
+    assert not hit                                             # cos ~ 0
+    assert c.retrieval_count == 4 and c.skip_count == 1
+
+
+def test_anchor_is_the_last_miss_not_the_previous_query():
+    """AR(1) drift: cos to the anchor decays 0.95, 0.9025, 0.857 ... so the
+    reference's last-miss anchor re-selects at the third step, while a
+    previous-query anchor would keep hitting."""
+    g = torch.Generator().manual_seed(30)
+    dim, rho = 4096, 0.95
+    qs = [torch.randn(dim, generator=g)]
+    for _ in range(12):
+        qs.append(rho * qs[-1] + math.sqrt(1 - rho * rho) * torch.randn(dim, generator=g))
+    ref, alt = selcache.SelectionCache(), selcache.SelectionCache(anchor="previous")
+    sel = lambda: torch.tensor([0])
+    hits_ref = [ref.step(q.bfloat16(), sel)[1] for q in qs]
+    hits_alt = [alt.step(q.bfloat16(), sel)[1] for q in qs]
+    assert hits_ref[:4] == [False, True, True, False]
+    assert all(hits_alt[1:])
+    assert ref.skip_count < alt.skip_count
+
+
+def test_batched_layer_applies_single_request_semantics():
+    H, Hkv, D, P = 4, 2, 128, 400
+    k_pool, v_pool = rnd(P, Hkv, D, seed=31), rnd(P, Hkv, D, seed=32)
+    q = rnd(2, H * D, seed=33)
+    tabs = [torch.arange(0, 250, dtype=torch.int32), torch.arange(250, 278, dtype=torch.int32)]
+    sels, out = oracle.layer.decode_layer(q, k_pool, v_pool, tabs, [250, 28], H, D, 4, 8, [16, 16],
+                                          1e4, 1.0, D ** -0.5)
+    assert sels[0].shape[0] == 28 and sels[1].tolist() == tabs[1].tolist()   # second one is dense
+    alone = oracle.layer.decode_layer(q[1:], k_pool, v_pool, tabs[1:], [28], H, D, 4, 8, [16],
+                                      1e4, 1.0, D ** -0.5)[1]
+    assert torch.equal(out[1], alone[0])

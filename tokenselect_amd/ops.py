@@ -362,7 +362,7 @@ class DecodeLayer:
         self.sel_len = torch.empty((batch,), dtype=torch.int32, device=device)
 
     def __call__(self, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch,
-                 cache: Optional[SelectionCache] = None):
+                 cache: Optional[SelectionCache] = None, out: Optional[torch.Tensor] = None):
         cfg = self.cfg
         cb = _c_batch(cfg, bt)
         if bt.batch != self.batch or bt.max_seq_len > self.max_seq_len:
@@ -374,12 +374,15 @@ class DecodeLayer:
         _check_pool(cfg, v_pool, "v_pool")
         if k_pool.shape != v_pool.shape:
             raise ValueError("k_pool and v_pool must have the same shape")
-        if bt.table.shape[1] * cfg.page_size < self.max_seq_len:
-            raise ValueError("table rows must address the max_seq_len this DecodeLayer was sized for")
-        cb.max_seq_len = self.max_seq_len  # keeps the workspace layout fixed across steps
+        if out is None:
+            out = self.out
+        else:
+            _need(out, "out", torch.bfloat16)
+            if out.numel() != self.out.numel():
+                raise ValueError("out must hold B*H*D elements")
         _lib.check(_lib.load().ts_decode_layer(
             ctypes.byref(self._c), ctypes.byref(cb), _p(q), _p(self.q_cos), _p(self.q_sin),
-            _p(k_pool), _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, self.batch), _p(self.out),
+            _p(k_pool), _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, self.batch), _p(out),
             _p(self.sel), _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
             self.workspace.numel(), _stream()))
-        return self.out, self.sel, self.sel_pos, self.sel_len
+        return out, self.sel, self.sel_pos, self.sel_len
