@@ -1,0 +1,61 @@
+"""The committed golden fixture (tests/golden/decode_layer_small.npz, written by
+tests/golden/make_fixtures.py from this repository's oracle): the oracle must
+still reproduce it (CPU), and the HIP path must match it (GPU)."""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+FIXTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "decode_layer_small.npz")
+
+
+def load():
+    z = np.load(FIXTURE, allow_pickle=False)
+    H, HKV, D, n_init, n_local, top_k, page = [int(x) for x in z["meta"]]
+    bf = lambda name: torch.from_numpy(z[name].copy()).view(torch.bfloat16)
+    return dict(z=z, H=H, HKV=HKV, D=D, n_init=n_init, n_local=n_local, top_k=top_k, page=page,
+                rope_base=float(z["rope_base"][0]), seq_lens=[int(x) for x in z["seq_lens"]],
+                table=torch.from_numpy(z["table"].copy()), k_pool=bf("k_pool"), v_pool=bf("v_pool"),
+                q=bf("q"), out=bf("out"))
+
+
+def test_oracle_reproduces_the_fixture():
+    f = load()
+    tabs = [oracle.select.expand_page_table(f["table"][b], L, f["page"])
+            for b, L in enumerate(f["seq_lens"])]
+    details = []
+    sels, out = oracle.layer.decode_layer(
+        f["q"], f["k_pool"], f["v_pool"], tabs, f["seq_lens"], f["H"], f["D"], f["n_init"],
+        f["n_local"], [f["top_k"]] * len(tabs), f["rope_base"], 1.0, f["D"] ** -0.5, details=details)
+    for b, sel in enumerate(sels):
+        assert sel.tolist() == f["z"][f"sel_{b}"].tolist()
+        if details[b]:
+            assert np.allclose(details[b]["scores"].numpy(), f["z"][f"scores_{b}"], rtol=1e-5, atol=1e-4)
+            assert details[b]["top_pos"].tolist() == f["z"][f"top_pos_{b}"].tolist()
+    assert (out.float() - f["out"].float()).abs().max().item() <= 1e-2
+    assert "sel_1" in f["z"] and "top_pos_1" not in f["z"]      # request 1 is the dense case
+    assert f["z"]["sel_1"].shape[0] == f["seq_lens"][1]
+
+
+@pytest.mark.gpu
+def test_hip_path_matches_the_fixture(dev):
+    from tokenselect_amd import ops
+    f = load()
+    B = len(f["seq_lens"])
+    cfg = ops.LayerConfig(num_heads=f["H"], num_kv_heads=f["HKV"], page_size=f["page"],
+                          n_init=f["n_init"], n_local=f["n_local"], top_k=f["top_k"],
+                          rope_theta=f["rope_base"])
+    bt = ops.Batch(torch.tensor(f["seq_lens"], dtype=torch.int32, device=dev),
+                   f["table"].to(dev).contiguous(), max(f["seq_lens"]))
+    layer = ops.DecodeLayer(cfg, B, max(f["seq_lens"]), dev)
+    out, sel, sel_pos, sel_len = layer(f["q"].to(dev), f["k_pool"].to(dev), f["v_pool"].to(dev), bt)
+    torch.cuda.synchronize()
+    for b in range(B):
+        want = f["z"][f"sel_{b}"]
+        assert int(sel_len[b]) == want.shape[0]
+        assert sel[b, :want.shape[0]].cpu().tolist() == want.tolist()
+    assert (out.cpu().float() - f["out"].float()).abs().max().item() <= 2e-2
