@@ -122,6 +122,9 @@ int ts_paged_matmul(const void* query, const void* token, int64_t pool_rows,
  * ts_score_partials_bytes() bytes.  qf [B,H,D] bf16 is the rotated fingerprint
  * (tr.py:380-392). */
 size_t ts_score_partials_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+/* Recommended score_stride / vote_stride (elements) for max_seq_len: a multiple
+ * of 64 that is not a power-of-two distance between head rows. */
+int64_t ts_score_stride(int32_t max_seq_len);
 int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
              int64_t pool_rows, const int32_t* skip, float* scores, int64_t score_stride,
              float* partials, size_t partials_bytes, ts_stream_t stream);

@@ -56,6 +56,7 @@ SIGNATURES = {
     "ts_rope_apply": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _ptr]),
     "ts_paged_matmul": (_i32, [_ptr, _ptr, _i64, _ptr, _ptr, _i32, _i64, _i32, _i32, _i32, _ptr]),
     "ts_score_partials_bytes": (_size, [_CFG, _i32, _i32]),
+    "ts_score_stride": (_i64, [_i32]),
     "ts_score": (_i32, [_CFG, _BT, _ptr, _ptr, _i64, _ptr, _ptr, _i64, _ptr, _size, _ptr]),
     "ts_vote": (_i32, [_CFG, _BT, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
     "ts_topk_workspace_bytes": (_size, [_CFG, _i32, _i32]),

@@ -2,6 +2,7 @@
 // per-layer driver that chains the kernels of one decode step.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include "ts_common.h"
 
@@ -68,12 +69,19 @@ int validate_batch(const ts_config* cfg, const ts_batch* bt) {
 }
 
 int score_tokens_per_block(int64_t total_candidates) {
-  // Aim for about four resident workgroups per CU on 256 CUs; 64-row granularity
-  // keeps every wave on whole 16-row tiles.
-  int64_t per = ceil_div(total_candidates, 1024);
+  // The scoring kernel keeps one workgroup per CU resident (its operand and
+  // staging registers fill the register file), so aim for one workgroup per CU on
+  // 256 CUs; 64-row granularity keeps every wave on whole 16-row tiles.
+  static const int forced = [] {
+    const char* e = getenv("TS_SCORE_TOKENS_PER_BLOCK");  // tuning override, multiple of 64
+    const int v = e ? atoi(e) : 0;
+    return (v >= 64 && v <= 8192) ? v / 64 * 64 : 0;
+  }();
+  if (forced) return forced;
+  int64_t per = ceil_div(total_candidates, 256);
   per = ceil_div(per, 64) * 64;
   if (per < 64) per = 64;
-  if (per > 512) per = 512;
+  if (per > 1024) per = 1024;
   return (int)per;
 }
 
@@ -88,6 +96,15 @@ int ts_version(void) { return TS_VERSION; }
 const char* ts_last_error(void) { return ts::g_error; }
 
 int ts_check_config(const ts_config* cfg) { return validate_config(cfg); }
+
+int64_t ts_score_stride(int32_t max_seq_len) {
+  // An odd number of 256-byte units between head rows: the H rows that a tile of
+  // tokens touches then spread over the memory channels instead of piling onto
+  // one (a power-of-two stride such as 131072 floats does exactly that).
+  int64_t units = ceil_div(max_seq_len > 0 ? max_seq_len : 1, 64);
+  if ((units & 1) == 0) units += 1;
+  return units * 64;
+}
 
 // Workspace of ts_decode_layer, carved in this order (256-byte aligned pieces).
 struct LayerWorkspace {
@@ -106,7 +123,7 @@ static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32
     return at;
   };
   const size_t B = (size_t)batch, H = (size_t)cfg->num_heads;
-  w.score_stride = (int64_t)align_up((size_t)max_seq_len, 64);
+  w.score_stride = ts_score_stride(max_seq_len);
   w.max_sel = cfg->n_init + cfg->top_k + cfg->n_local;
   w.qf = take(B * H * kHeadDim * 2);
   w.hit = take(B * 4);

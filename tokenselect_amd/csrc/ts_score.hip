@@ -2,25 +2,30 @@
 // paged KV cache (the reference's paged_matmul_kernel, tr.py:166-231), plus the
 // per-head softmax statistics the soft vote needs (tr.py:361).
 //
-// Data movement: a wavefront reads one token row (Hkv*256 bytes, contiguous in
-// the pool) with 128-bit loads, 16 lanes per KV head, so every row is fetched
-// from HBM exactly once for all H query heads.  The G = H/Hkv queries that share
-// a KV head live in registers as packed bf16 pairs; products are exact and
-// accumulated in fp32 (v_dot2_f32_bf16), then reduced over the 16 lanes of the
-// DPP row.  Results of 16 consecutive rows are transposed into lanes so that the
-// score store is one contiguous 64-byte segment per head.
+// The pass is bound by HBM: every candidate row (Hkv*256 bytes) is read exactly
+// once for all H query heads.  The dot products go through the matrix cores, not
+// because the shape is a dense GEMM (it is 4 to 8 query rows per KV head) but
+// because one v_mfma_f32_16x16x32_bf16 replaces 64 dot/reduce/select vector
+// instructions and leaves the wavefront free to keep loads in flight:
+//
+//   B operand = keys:    lane l holds token (l%16) of a 16-token tile, 8 dims
+//                        [32c + 8(l/16), +8) of one KV head - a 128-bit load
+//                        straight from HBM into the operand registers;
+//   A operand = queries: row 4*(g%4) + g/4 holds query g of the KV head, so
+//   D result:            lane l, register r = score of query (l/16) + 4r for
+//                        token l%16 - already one token per lane, 16
+//                        consecutive tokens per 16-lane row: a 64-byte store
+//                        per head, no cross-lane traffic at all.
+//
+// Products of bf16 pairs are exact in fp32 and the accumulation is fp32.
+// Loads are double-buffered in half iterations (16 x 128-bit loads per lane
+// each) and the table entry of the next tile is fetched one iteration ahead.
 #include "ts_common.h"
-
-#ifndef TS_SCORE_SUBBATCH
-#define TS_SCORE_SUBBATCH 4  // wave steps per load sub-batch: 4 or 8
-#endif
-#ifndef TS_SCORE_WAVES_PER_EU
-#define TS_SCORE_WAVES_PER_EU 3
-#endif
 
 namespace ts {
 
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 struct ScoreArgs {
   const uint16_t* qf;      // [B,H,128] bf16 rotated fingerprints
@@ -42,33 +47,22 @@ struct ScoreArgs {
   int head_map;
 };
 
-__device__ __forceinline__ float dot8(const uint4& k, const uint32_t (&q)[4]) {
-  float acc = 0.f;
-  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, k.x),
-                                        __builtin_bit_cast(bf16x2_t, q[0]), acc, false);
-  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, k.y),
-                                        __builtin_bit_cast(bf16x2_t, q[1]), acc, false);
-  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, k.z),
-                                        __builtin_bit_cast(bf16x2_t, q[2]), acc, false);
-  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, k.w),
-                                        __builtin_bit_cast(bf16x2_t, q[3]), acc, false);
-  return acc;
-}
-
 template <int HKV, int G>
 __device__ __forceinline__ int head_of(int kvh, int g, int head_map) {
   return head_map == TS_HEADMAP_MOD ? kvh + HKV * g : kvh * G + g;
 }
 
-// Lane layout.  HKV >= 4: a wave step covers one token; 16-lane group `lg` reads
-// KV heads lg, lg+4, ... (KVS 1-KB loads per row).  HKV < 4: a row is shorter
-// than 1 KB, so a step covers TPW = 4/HKV tokens and group lg reads KV head
-// lg % HKV of token lg / HKV.
+// One iteration of a wave covers TG tiles of 16 tokens and all HKV heads: always
+// 8 (tile, KV head) units = 32 loads of 1 KB.  Units 0-3 and 4-7 alternate
+// between two register buffers.
 template <int HKV, int G, bool OUT_BF16>
-__global__ __launch_bounds__(256, ((HKV >= 4 ? HKV / 4 : 1) * G > 8 ? 2 : TS_SCORE_WAVES_PER_EU)) void score_kernel(ScoreArgs a) {
-  constexpr int KVS = HKV >= 4 ? HKV / 4 : 1;
-  constexpr int TPW = HKV >= 4 ? 1 : 4 / HKV;
-  constexpr int TILE = 16 * TPW;
+__global__ __launch_bounds__(256, 1) void score_kernel(ScoreArgs a) {
+  constexpr int TG = 8 / HKV;
+  constexpr int UNITS = 8;
+  constexpr int HALF = UNITS / 2;
+  constexpr int NR = (G + 3) / 4;  // result registers in use per unit
+  constexpr int ITER = 16 * TG;    // tokens per iteration
+  constexpr uint32_t ROW_BYTES = HKV * kHeadDim * 2;
 
   const int b = blockIdx.y;
   int n, first_pos;
@@ -77,7 +71,8 @@ __global__ __launch_bounds__(256, ((HKV >= 4 ? HKV / 4 : 1) * G > 8 ? 2 : TS_SCO
     first_pos = 0;
   } else {
     if (a.skip && a.skip[b]) return;
-    ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+    ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
+                                   a.max_seq_len);
     n = geo.n;
     first_pos = a.n_init;
   }
@@ -86,166 +81,141 @@ __global__ __launch_bounds__(256, ((HKV >= 4 ? HKV / 4 : 1) * G > 8 ? 2 : TS_SCO
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int lg = lane >> 4, l16 = lane & 15;
-  const int tok_sub = HKV >= 4 ? 0 : lg / HKV;
+  const int rg = lane >> 4;   // k-group of the operands, row group of the result
+  const int col = lane & 15;  // token inside a tile
   const int H = a.num_heads;
   const int32_t* tab = a.table + (int64_t)b * a.table_stride;
 
-  uint32_t qreg[KVS][G][4];
-  uint32_t kv_off[KVS];  // byte offset of this lane's 16 bytes inside a token row
+  // A operands: query (col/4 + 4*(col%4)) of each KV head, dims [32c + 8rg, +8).
+  bf16x8_t qa[HKV][4];
+  {
+    const int g = (col >> 2) + 4 * (col & 3);
 #pragma unroll
-  for (int s = 0; s < KVS; ++s) {
-    const int kvh = HKV >= 4 ? lg + 4 * s : lg % HKV;
-    kv_off[s] = (uint32_t)(kvh * kHeadDim + l16 * 8) * 2u;
+    for (int kvh = 0; kvh < HKV; ++kvh) {
+      const int h = head_of<HKV, G>(kvh, g < G ? g : 0, a.head_map);
+      const uint16_t* qrow = a.qf + ((size_t)b * H + h) * kHeadDim + rg * 8;
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const int h = head_of<HKV, G>(kvh, g, a.head_map);
-      const uint4 v = *(const uint4*)(a.qf + ((size_t)b * H + h) * kHeadDim + l16 * 8);
-      qreg[s][g][0] = v.x;
-      qreg[s][g][1] = v.y;
-      qreg[s][g][2] = v.z;
-      qreg[s][g][3] = v.w;
+      for (int c = 0; c < 4; ++c) {
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (g < G) v = *(const uint4*)(qrow + c * 32);
+        qa[kvh][c] = __builtin_bit_cast(bf16x8_t, v);
+      }
     }
   }
 
-  float run_m[KVS][G], run_l[KVS][G];
+  float run_m[HKV][NR], run_l[HKV][NR];
 #pragma unroll
-  for (int s = 0; s < KVS; ++s)
+  for (int kvh = 0; kvh < HKV; ++kvh)
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      run_m[s][g] = kNegBig;
-      run_l[s][g] = 0.f;
+    for (int r = 0; r < NR; ++r) {
+      run_m[kvh][r] = kNegBig;
+      run_l[kvh][r] = 0.f;
     }
 
   const int per_wave = a.tokens_per_block >> 2;
   const int wave_lo = block_lo + wave * per_wave;
   const int wave_hi = min(wave_lo + per_wave, n);
 
-  // A tile is 16 wave steps (16*TPW tokens) whose results are transposed into
-  // the 16 lanes of a row.  It is loaded in sub-batches of SB steps that
-  // alternate between two register buffers, so that the loads of the next
-  // sub-batch are in flight while the current one is reduced.
-  constexpr int SB = TS_SCORE_SUBBATCH;
-  constexpr int NSB = 16 / SB;  // sub-batches per tile (even)
-  uint4 buf0[SB][KVS], buf1[SB][KVS];
-
-  // Lane i resolves the slot of token tile+i.  The table load and the slot
-  // arithmetic are split so that the load of the next tile's entries is issued a
-  // whole tile before its value is needed.  Out-of-range lanes and tiles are
-  // clamped to the wave's last token: every load stays in bounds and no branch
+  // Lane (rg, col) addresses token `tile + col` of every tile.  The table load and
+  // the slot arithmetic are split so that the entry of the next iteration is
+  // requested a whole iteration before it is needed.  Positions past the wave's
+  // range are clamped to its last token: every load stays in bounds and no branch
   // splits the load pipeline.
   const int last_pos = first_pos + max(wave_hi - 1, 0);
   const int page_mask = a.page_size - 1;
   auto table_entry = [&](int tile) -> int32_t {
-    const int pos = min(first_pos + tile + lane, last_pos);
+    const int pos = min(first_pos + tile + col, last_pos);
     return tab[pos >> a.page_shift];
   };
-  auto slot_from = [&](int32_t entry, int tile) -> uint32_t {
-    const int pos = min(first_pos + tile + lane, last_pos);
-    const uint32_t slot = ((uint32_t)entry << a.page_shift) + (uint32_t)(pos & page_mask);
-    return slot < a.pool_rows ? slot : a.pool_rows - 1;
+  auto row_ptr = [&](int32_t entry, int tile) -> const char* {
+    const int pos = min(first_pos + tile + col, last_pos);
+    uint32_t slot = ((uint32_t)entry << a.page_shift) + (uint32_t)(pos & page_mask);
+    slot = slot < a.pool_rows ? slot : a.pool_rows - 1;
+    return (const char*)a.k_pool + (size_t)slot * ROW_BYTES + rg * 16;
   };
 
-  auto issue = [&](uint4 (&buf)[SB][KVS], uint32_t slots, int first_step) {
+  uint4 buf0[HALF][4], buf1[HALF][4];
+  auto issue = [&](uint4 (&buf)[HALF][4], auto& rows, int first_unit) {
 #pragma unroll
-    for (int i = 0; i < SB; ++i) {
-      const int step = first_step + i;
-      uint32_t slot;
-      if (TPW == 1) {
-        slot = __builtin_amdgcn_readlane(slots, step);
-      } else if (TPW == 2) {
-        const uint32_t s0 = __builtin_amdgcn_readlane(slots, 2 * step);
-        const uint32_t s1 = __builtin_amdgcn_readlane(slots, 2 * step + 1);
-        slot = tok_sub ? s1 : s0;
-      } else {
-        const uint32_t s0 = __builtin_amdgcn_readlane(slots, 4 * step);
-        const uint32_t s1 = __builtin_amdgcn_readlane(slots, 4 * step + 1);
-        const uint32_t s2 = __builtin_amdgcn_readlane(slots, 4 * step + 2);
-        const uint32_t s3 = __builtin_amdgcn_readlane(slots, 4 * step + 3);
-        slot = tok_sub == 0 ? s0 : (tok_sub == 1 ? s1 : (tok_sub == 2 ? s2 : s3));
-      }
-      const char* row = (const char*)a.k_pool + (size_t)slot * (size_t)(HKV * kHeadDim * 2);
+    for (int i = 0; i < HALF; ++i) {
+      const int u = first_unit + i;
+      const char* p = rows[u / HKV] + (u % HKV) * (kHeadDim * 2);
 #pragma unroll
-      for (int s = 0; s < KVS; ++s) {
-        uint32_t off = kv_off[s];
-        asm volatile("" : "+v"(off));  // keep the 32-bit lane offset next to its use
-        buf[i][s] = *(const uint4*)(row + off);
-      }
+      for (int c = 0; c < 4; ++c) buf[i][c] = *(const uint4*)(p + c * 64);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto multiply = [&](const uint4 (&buf)[HALF][4], f32x4_t (&acc)[UNITS], int first_unit) {
+#pragma unroll
+    for (int i = 0; i < HALF; ++i) {
+      const int u = first_unit + i;
+      f32x4_t d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[u % HKV][c],
+                                                    __builtin_bit_cast(bf16x8_t, buf[i][c]), d, 0, 0, 0);
+      acc[u] = d;
     }
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  auto reduce = [&](const uint4 (&buf)[SB][KVS], float (&res)[KVS][G], int first_step) {
-#pragma unroll
-    for (int i = 0; i < SB; ++i) {
-#pragma unroll
-      for (int s = 0; s < KVS; ++s)
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-          const float p = row16_sum(dot8(buf[i][s], qreg[s][g]));
-          res[s][g] = (l16 == first_step + i) ? p : res[s][g];
-          // Pin the select here; otherwise the compiler sinks the whole chain
-          // into the store block and keeps every partial sum alive until then.
-          asm volatile("" : "+v"(res[s][g]));
-        }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  uint32_t slots_cur = 0;
+  const char* rows_cur[TG];
+  const char* rows_next[TG];
   if (wave_lo < wave_hi) {
-    slots_cur = slot_from(table_entry(wave_lo), wave_lo);
-    issue(buf0, slots_cur, 0);
+#pragma unroll
+    for (int t = 0; t < TG; ++t) rows_cur[t] = row_ptr(table_entry(wave_lo + 16 * t), wave_lo + 16 * t);
+    issue(buf0, rows_cur, 0);
   }
 
-  for (int tile = wave_lo; tile < wave_hi; tile += TILE) {
-    float res[KVS][G];
+  for (int base = wave_lo; base < wave_hi; base += ITER) {
+    int32_t entry_next[TG];
 #pragma unroll
-    for (int s = 0; s < KVS; ++s)
-#pragma unroll
-      for (int g = 0; g < G; ++g) res[s][g] = 0.f;
-
-    const int32_t entry_next = table_entry(tile + TILE);
-    uint32_t slots_next = 0;
+    for (int t = 0; t < TG; ++t) entry_next[t] = table_entry(base + ITER + 16 * t);
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int sb = 0; sb < NSB; sb += 2) {
-      // buf0 holds sub-batch sb; fetch sb+1 into buf1, then sb+2 into buf0.
-      issue(buf1, slots_cur, (sb + 1) * SB);
-      reduce(buf0, res, sb * SB);
-      if (sb + 2 < NSB) {
-        issue(buf0, slots_cur, (sb + 2) * SB);
-      } else {
-        slots_next = slot_from(entry_next, tile + TILE);
-        issue(buf0, slots_next, 0);
-      }
-      reduce(buf1, res, (sb + 1) * SB);
-    }
-    slots_cur = slots_next;
 
-    // Lane l16 of each group now holds token tile + l16*TPW + tok_sub.
-    const int mytok = tile + l16 * TPW + tok_sub;
-    if (mytok < wave_hi) {
+    f32x4_t acc[UNITS];
+    issue(buf1, rows_cur, HALF);
+    multiply(buf0, acc, 0);
 #pragma unroll
-      for (int s = 0; s < KVS; ++s) {
-        const int kvh = HKV >= 4 ? lg + 4 * s : lg % HKV;
+    for (int t = 0; t < TG; ++t) rows_next[t] = row_ptr(entry_next[t], base + ITER + 16 * t);
+    issue(buf0, rows_next, 0);
+    multiply(buf1, acc, HALF);
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
+    for (int t = 0; t < TG; ++t) rows_cur[t] = rows_next[t];
+
+    // Lane (rg, col), register r of unit (tile t, head kvh): query rg + 4r, token
+    // base + 16t + col.
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+      const int t = u / HKV, kvh = u % HKV;
+      const int tok = base + 16 * t + col;
+#pragma unroll
+      for (int r = 0; r < NR; ++r) {
+        const int g = rg + 4 * r;
+        if (g < G && tok < wave_hi) {
           const int h = head_of<HKV, G>(kvh, g, a.head_map);
-          const float x = res[s][g];
-          const size_t at = ((size_t)b * H + h) * (size_t)a.score_stride + (size_t)mytok;
+          const float x = acc[u][r];
+          const size_t at = ((size_t)b * H + h) * (size_t)a.score_stride + (size_t)tok;
+#ifndef TS_DBG_NOSTORE
           if (OUT_BF16)
             ((uint16_t*)a.scores)[at] = f32_to_bf16(x);
           else
             ((float*)a.scores)[at] = x;
+#else
+          if (x == 1234.5678f) ((float*)a.scores)[at] = x;
+#endif
+#ifdef TS_DBG_NOSTATS
+          run_l[kvh][r] += x;
+          continue;
+#endif
           // Online (max, sum exp) with a single exponential per element.
-          const float d = x - run_m[s][g];
+          const float d = x - run_m[kvh][r];
           const float e = __expf(-fabsf(d));
           if (d > 0.f) {
-            run_l[s][g] = run_l[s][g] * e + 1.f;
-            run_m[s][g] = x;
+            run_l[kvh][r] = run_l[kvh][r] * e + 1.f;
+            run_m[kvh][r] = x;
           } else {
-            run_l[s][g] += e;
+            run_l[kvh][r] += e;
           }
         }
       }
@@ -254,17 +224,17 @@ __global__ __launch_bounds__(256, ((HKV >= 4 ? HKV / 4 : 1) * G > 8 ? 2 : TS_SCO
 
   if (a.partials == nullptr) return;
 
-  __shared__ float sm_m[4][4][KVS][G];
-  __shared__ float sm_l[4][4][KVS][G];
+  __shared__ float sm_m[4][4][HKV][NR];
+  __shared__ float sm_l[4][4][HKV][NR];
 #pragma unroll
-  for (int s = 0; s < KVS; ++s)
+  for (int kvh = 0; kvh < HKV; ++kvh)
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float m = run_m[s][g], l = run_l[s][g];
+    for (int r = 0; r < NR; ++r) {
+      float m = run_m[kvh][r], l = run_l[kvh][r];
       row16_softmax_merge(m, l);
-      if (l16 == 0) {
-        sm_m[wave][lg][s][g] = m;
-        sm_l[wave][lg][s][g] = l;
+      if (col == 0) {
+        sm_m[wave][rg][kvh][r] = m;
+        sm_l[wave][rg][kvh][r] = l;
       }
     }
   __syncthreads();
@@ -272,13 +242,13 @@ __global__ __launch_bounds__(256, ((HKV >= 4 ? HKV / 4 : 1) * G > 8 ? 2 : TS_SCO
     const int h = threadIdx.x;
     float m = kNegBig, l = 0.f;
     for (int w = 0; w < 4; ++w)
-      for (int gi = 0; gi < 4; ++gi)
-        for (int s = 0; s < KVS; ++s) {
-          const int kvh = HKV >= 4 ? gi + 4 * s : gi % HKV;
-          for (int g = 0; g < G; ++g)
-            if (head_of<HKV, G>(kvh, g, a.head_map) == h)
-              softmax_merge(m, l, sm_m[w][gi][s][g], sm_l[w][gi][s][g]);
-        }
+      for (int g4 = 0; g4 < 4; ++g4)
+        for (int kvh = 0; kvh < HKV; ++kvh)
+          for (int r = 0; r < NR; ++r) {
+            const int g = g4 + 4 * r;
+            if (g < G && head_of<HKV, G>(kvh, g, a.head_map) == h)
+              softmax_merge(m, l, sm_m[w][g4][kvh][r], sm_l[w][g4][kvh][r]);
+          }
     float* p = a.partials + (((size_t)b * H + h) * a.nchunks + blockIdx.x) * 2;
     p[0] = m;
     p[1] = l;

@@ -1,49 +1,172 @@
 // Ragged top-k, ascending sort and index assembly (tr.py:371-373, 433-449).
 //
-// One workgroup per request runs an exact radix select over order-preserving
-// 32-bit keys of the fp32 votes (four 8-bit passes with an LDS histogram),
-// which yields the k-th largest key T and how many elements equal to T are
-// needed.  A single ordered compaction pass then emits, in ascending position,
-// every element above T plus the lowest-positioned ties at T: the output is
-// sorted without a sort and is bit-stable across runs.  The same kernel writes
-// the sink and local-window segments and translates logical positions to
-// physical slots through the table.
-#include "ts_common.h"
+// Exact radix select on order-preserving 32-bit keys of the fp32 votes, split
+// 11 + 11 + 10 bits, spread over many workgroups:
+//
+//   hist   (grid over candidates)  histogram of the top 11 key bits per request
+//   mark   (grid over candidates)  finds the threshold bin t0; every candidate in
+//                                  a higher bin is selected for sure and gets its
+//                                  bit in a position bitmap (one plain 64-bit
+//                                  store per wavefront); candidates inside bin t0
+//                                  are appended to a short list and histogrammed
+//                                  on their next 11 bits
+//   final  (one workgroup/request) resolves the remaining 21 bits on the short
+//                                  list (ties at the k-th key: lowest position
+//                                  first), sets their bits, then walks the bitmap
+//                                  with a popcount prefix scan and emits the
+//                                  selected positions in ascending order, together
+//                                  with the sink and local-window segments and
+//                                  the logical -> physical translation.
+//
+// The output is sorted without a sort and bit-stable across runs (no result
+// depends on the order in which atomics land).
+#include "ts_topk.h"
 
 namespace ts {
 
-constexpr int kTopkThreads = 1024;
-constexpr int kTopkWaves = kTopkThreads / 64;
-
-struct TopkArgs {
-  const float* votes;
-  int64_t vote_stride;
-  const int32_t* seq_lens;
-  const int32_t* table;
-  int64_t table_stride;
-  const int32_t* k_per_req;
-  const int32_t* hit;
-  int32_t* topk_cache;  // [B, top_k] or NULL
-  int32_t* cache_len;   // [B] or NULL
-  int n_init, n_local, top_k, page_size, page_shift, pool_kernel, max_seq_len;
-  uint32_t pool_rows;
-  int32_t* sel;
-  int32_t* sel_pos;
-  int64_t sel_stride;
-  int32_t* sel_len;
-};
-
-// Monotone map fp32 -> uint32: larger float <=> larger key.
-__device__ __forceinline__ uint32_t vote_key(float v) {
-  const uint32_t u = __float_as_uint(v);
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+__device__ __forceinline__ int pooled_count(int n, int pool_kernel) {
+  return (pool_kernel > 0 && (pool_kernel & 1) == 0) ? n - 1 : n;  // even kernel: one fewer
 }
 
-__global__ __launch_bounds__(kTopkThreads) void topk_kernel(TopkArgs a) {
+// Block-wide search of a descending histogram: finds the bin t such that
+// count(bins > t) < need <= count(bins >= t).  `hist` has NB entries (global or
+// LDS), NB a multiple of blockDim.x.  Returns t and count(bins > t) to every
+// thread.  `scratch` is LDS of blockDim.x/64 + 2 words.
+template <int NB>
+__device__ __forceinline__ void find_threshold_bin(const uint32_t* hist, uint32_t need,
+                                                   uint32_t* scratch, uint32_t& t_out,
+                                                   uint32_t& above_out) {
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int per = NB / nthreads;  // bins per thread, thread 0 owns the highest bins
+  const int lane = tid & 63, wave = tid >> 6, nwaves = nthreads >> 6;
+  const int hi_bin = NB - 1 - tid * per;
+  uint32_t local[8];
+  uint32_t mine = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    local[i] = 0;
+    if (i < per) {
+      local[i] = hist[hi_bin - i];
+      mine += local[i];
+    }
+  }
+  // exclusive prefix of `mine` over threads (descending bins)
+  uint32_t incl = mine;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63) scratch[wave] = incl;
+  if (tid == 0) {
+    scratch[nwaves] = 0;
+    scratch[nwaves + 1] = 0;
+  }
+  __syncthreads();
+  uint32_t wave_base = 0;
+  for (int w = 0; w < wave; ++w) wave_base += scratch[w];
+  const uint32_t before = wave_base + incl - mine;  // count in bins above this thread's range
+  if (before < need && need <= before + mine) {      // the crossing lies in this thread's bins
+    uint32_t run = before;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (i < per) {
+        if (run < need && need <= run + local[i]) {
+          scratch[nwaves] = (uint32_t)(hi_bin - i);
+          scratch[nwaves + 1] = run;
+        }
+        run += local[i];
+      }
+  }
+  __syncthreads();
+  t_out = scratch[nwaves];
+  above_out = scratch[nwaves + 1];
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(256) void topk_zero_kernel(uint32_t* __restrict__ ws,
+                                                        size_t stride_words) {
+  uint32_t* p = ws + (size_t)blockIdx.x * stride_words;
+  for (int i = threadIdx.x; i < kTopkCounterWords; i += 256) p[i] = 0u;
+}
+
+__global__ __launch_bounds__(256) void topk_hist_kernel(TopkArgs a) {
+  const int b = blockIdx.y;
+  if (a.hit && a.hit[b]) return;
+  const ReqGeom geo =
+      request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  const int n = pooled_count(geo.n, a.pool_kernel);
+  const int lo = blockIdx.x * kTopkSlice;
+  if (lo >= n) return;
+  __shared__ uint32_t lh[kTopkBins];
+  for (int i = threadIdx.x; i < kTopkBins; i += 256) lh[i] = 0u;
+  __syncthreads();
+  const float* votes = a.votes + (int64_t)b * a.vote_stride;
+  for (int i = lo + threadIdx.x; i < min(lo + kTopkSlice, n); i += 256)
+    atomicAdd(&lh[key_bin0(vote_key(votes[i]))], 1u);
+  __syncthreads();
+  uint32_t* hist0 = topk_ws(a.ws, a.ws_stride, b) + kTopkHist0;
+  for (int i = threadIdx.x; i < kTopkBins; i += 256)
+    if (lh[i]) atomicAdd(&hist0[i], lh[i]);
+}
+
+__global__ __launch_bounds__(256) void topk_mark_kernel(TopkArgs a) {
+  const int b = blockIdx.y;
+  if (a.hit && a.hit[b]) return;
+  const ReqGeom geo =
+      request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  const int n = pooled_count(geo.n, a.pool_kernel);
+  const int lo = blockIdx.x * kTopkSlice;
+  if (lo >= n) return;
+
+  __shared__ uint32_t scratch[8];
+  __shared__ uint32_t lh[kTopkBins];
+  uint32_t* ws = topk_ws(a.ws, a.ws_stride, b);
+  uint32_t t0, above0;
+  find_threshold_bin<kTopkBins>(ws + kTopkHist0, (uint32_t)geo.k, scratch, t0, above0);
+  for (int i = threadIdx.x; i < kTopkBins; i += 256) lh[i] = 0u;
+  __syncthreads();
+
+  const float* votes = a.votes + (int64_t)b * a.vote_stride;
+  uint64_t* bitmap = (uint64_t*)(ws + kTopkCounterWords);
+  uint2* cand = (uint2*)(ws + kTopkCounterWords + a.bitmap_words);
+  const int lane = threadIdx.x & 63;
+  // Whole 64-position groups per wave iteration so that a bitmap word has one writer.
+  for (int base = lo + (threadIdx.x & ~63); base < min(lo + kTopkSlice, n); base += 256) {
+    const int i = base + lane;
+    uint32_t key = 0;
+    bool gt = false, eq = false;
+    if (i < n) {
+      key = vote_key(votes[i]);
+      const uint32_t bin = key_bin0(key);
+      gt = bin > t0;
+      eq = bin == t0;
+    }
+    const uint64_t gt_mask = __ballot(gt), eq_mask = __ballot(eq);
+    if (lane == 0) bitmap[base >> 6] = gt_mask;
+    if (eq_mask) {
+      uint32_t slot = 0;
+      if (lane == 0) slot = atomicAdd(&ws[kTopkCandCount], (uint32_t)__popcll(eq_mask));
+      slot = __shfl(slot, 0);
+      if (eq) {
+        const uint32_t at = slot + __popcll(eq_mask & ((1ull << lane) - 1ull));
+        if (at < a.cand_cap) cand[at] = make_uint2(key, (uint32_t)i);  // cap: counters not cleared
+        atomicAdd(&lh[key_bin1(key)], 1u);
+      }
+    }
+  }
+  __syncthreads();
+  uint32_t* hist1 = ws + kTopkHist1;
+  for (int i = threadIdx.x; i < kTopkBins; i += 256)
+    if (lh[i]) atomicAdd(&hist1[i], lh[i]);
+}
+
+__global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs a) {
   const int b = blockIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  const ReqGeom geo =
+      request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
   const int32_t* tab = a.table + (int64_t)b * a.table_stride;
   int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
   int32_t* sel_pos = a.sel_pos + (int64_t)b * a.sel_stride;
@@ -55,145 +178,148 @@ __global__ __launch_bounds__(kTopkThreads) void topk_kernel(TopkArgs a) {
   };
 
   if (geo.dense) {  // tr.py:377-378, 741-744: attend over every token
-    for (int i = tid; i < L; i += kTopkThreads) emit(i, i);
+    for (int i = tid; i < L; i += kTopkFinalThreads) emit(i, i);
     if (tid == 0) a.sel_len[b] = L;
     return;
   }
-
   const bool is_hit = a.hit && a.hit[b];
   const int k = is_hit ? min(a.cache_len[b], a.top_k) : geo.k;
   if (tid == 0) a.sel_len[b] = a.n_init + k + a.n_local;
-  for (int i = tid; i < a.n_init; i += kTopkThreads) emit(i, i);
-  for (int i = tid; i < a.n_local; i += kTopkThreads) emit(a.n_init + k + i, L - a.n_local + i);
-
+  for (int i = tid; i < a.n_init; i += kTopkFinalThreads) emit(i, i);
+  for (int i = tid; i < a.n_local; i += kTopkFinalThreads) emit(a.n_init + k + i, L - a.n_local + i);
   if (is_hit) {  // tr.py:419: reuse the cached positions
     const int32_t* cached = a.topk_cache + (int64_t)b * a.top_k;
-    for (int i = tid; i < k; i += kTopkThreads) emit(a.n_init + i, cached[i]);
+    for (int i = tid; i < k; i += kTopkFinalThreads) emit(a.n_init + i, cached[i]);
     return;
   }
 
-  int n = geo.n;
-  if (a.pool_kernel > 0 && (a.pool_kernel & 1) == 0) n -= 1;  // even kernel: one output fewer
-  const float* votes = a.votes + (int64_t)b * a.vote_stride;
+  const int n = pooled_count(geo.n, a.pool_kernel);
+  uint32_t* ws = topk_ws(a.ws, a.ws_stride, b);
+  uint32_t* bitmap32 = ws + kTopkCounterWords;
+  const uint2* cand = (const uint2*)(ws + kTopkCounterWords + a.bitmap_words);
+  const int ncand = (int)min(ws[kTopkCandCount], (uint32_t)n);
 
-  __shared__ uint32_t hist[256];
-  __shared__ uint32_t suffix[256];
-  __shared__ uint32_t s_prefix, s_need;
-  __shared__ uint32_t wave_gt[kTopkWaves], wave_eq[kTopkWaves];
+  __shared__ uint32_t scratch[kTopkFinalThreads / 64 + 2];
+  __shared__ uint32_t lh[1024];
+  auto mark = [&](uint32_t pos) { atomicOr(&bitmap32[pos >> 5], 1u << (pos & 31u)); };
 
-  uint32_t prefix = 0, mask = 0, need = (uint32_t)k;
-  for (int pass = 0; pass < 4; ++pass) {
-    const int shift = 24 - 8 * pass;
-    if (tid < 256) hist[tid] = 0;
-    __syncthreads();
-    for (int i = tid; i < n; i += kTopkThreads) {
-      const uint32_t key = vote_key(votes[i]);
-      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
-    }
-    __syncthreads();
-    // Inclusive suffix sums: suffix[d] = number of matching keys with digit >= d.
-    if (tid < 256) suffix[tid] = hist[tid];
-    __syncthreads();
-    for (int off = 1; off < 256; off <<= 1) {
-      uint32_t add = 0;
-      if (tid < 256 && tid + off < 256) add = suffix[tid + off];
-      __syncthreads();
-      if (tid < 256) suffix[tid] += add;
-      __syncthreads();
-    }
-    if (tid < 256) {
-      const uint32_t above = tid < 255 ? suffix[tid + 1] : 0u;
-      if (suffix[tid] >= need && above < need) {  // exactly one digit satisfies this
-        s_prefix = prefix | ((uint32_t)tid << shift);
-        s_need = need - above;
-      }
-    }
-    __syncthreads();
-    prefix = s_prefix;
-    need = s_need;
-    mask |= 255u << shift;
-    __syncthreads();
+  uint32_t t0, above0, t1, above1, t2, above2;
+  find_threshold_bin<kTopkBins>(ws + kTopkHist0, (uint32_t)k, scratch, t0, above0);
+  const uint32_t need1 = (uint32_t)k - above0;  // still to take inside bin t0
+  find_threshold_bin<kTopkBins>(ws + kTopkHist1, need1, scratch, t1, above1);
+  const uint32_t need2 = need1 - above1;  // still to take inside (t0, t1)
+
+  for (int i = tid; i < 1024; i += kTopkFinalThreads) lh[i] = 0u;
+  __syncthreads();
+  for (int i = tid; i < ncand; i += kTopkFinalThreads) {
+    const uint2 c = cand[i];
+    const uint32_t b1 = key_bin1(c.x);
+    if (b1 > t1)
+      mark(c.y);
+    else if (b1 == t1)
+      atomicAdd(&lh[key_bin2(c.x)], 1u);
   }
-  const uint32_t kth = prefix;     // key of the k-th largest vote
-  const uint32_t need_eq = need;   // ties at kth to take, lowest position first
+  __syncthreads();
+  find_threshold_bin<1024>(lh, need2, scratch, t2, above2);
+  const uint32_t need_eq = need2 - above2;  // ties at the k-th key still to take
+  const uint32_t count_eq = lh[t2];
+  __syncthreads();
 
-  int32_t* cache_out = a.topk_cache ? a.topk_cache + (int64_t)b * a.top_k : nullptr;
-  uint32_t run_gt = 0, run_eq = 0;
-  for (int base = 0; base < n; base += kTopkThreads) {
-    const int i = base + tid;
-    uint32_t key = 0;
-    const bool in = i < n;
-    if (in) key = vote_key(votes[i]);
-    const bool gt = in && key > kth;
-    const bool eq = in && key == kth;
-    const uint64_t gt_mask = __ballot(gt), eq_mask = __ballot(eq);
-    if (lane == 0) {
-      wave_gt[wave] = __popcll(gt_mask);
-      wave_eq[wave] = __popcll(eq_mask);
+  if (count_eq == need_eq) {  // the usual case: every tie is selected
+    for (int i = tid; i < ncand; i += kTopkFinalThreads) {
+      const uint2 c = cand[i];
+      if (key_bin1(c.x) == t1 && key_bin2(c.x) >= t2) mark(c.y);
+    }
+  } else {
+    // More ties than places: keep the need_eq lowest positions.  Positions are
+    // unique, so a two-digit radix select on the position finds the largest one kept.
+    uint32_t p_hi, p_lo, skip_hi, skip_lo;
+    for (int i = tid; i < 1024; i += kTopkFinalThreads) lh[i] = 0u;
+    __syncthreads();
+    auto is_tie = [&](const uint2& c) { return key_bin1(c.x) == t1 && key_bin2(c.x) == t2; };
+    for (int i = tid; i < ncand; i += kTopkFinalThreads) {
+      const uint2 c = cand[i];
+      if (is_tie(c)) atomicAdd(&lh[1023u - (c.y >> 10)], 1u);  // descending bin = ascending position
     }
     __syncthreads();
-    uint32_t gt_before = 0, eq_before = 0, gt_total = 0, eq_total = 0;
+    find_threshold_bin<1024>(lh, need_eq, scratch, p_hi, skip_hi);
+    const uint32_t pos_hi = 1023u - p_hi;
+    for (int i = tid; i < 1024; i += kTopkFinalThreads) lh[i] = 0u;
+    __syncthreads();
+    for (int i = tid; i < ncand; i += kTopkFinalThreads) {
+      const uint2 c = cand[i];
+      if (is_tie(c) && (c.y >> 10) == pos_hi) atomicAdd(&lh[1023u - (c.y & 1023u)], 1u);
+    }
+    __syncthreads();
+    find_threshold_bin<1024>(lh, need_eq - skip_hi, scratch, p_lo, skip_lo);
+    const uint32_t last_pos = (pos_hi << 10) | (1023u - p_lo);
+    for (int i = tid; i < ncand; i += kTopkFinalThreads) {
+      const uint2 c = cand[i];
+      if (key_bin1(c.x) == t1 && (key_bin2(c.x) > t2 || (key_bin2(c.x) == t2 && c.y <= last_pos)))
+        mark(c.y);
+    }
+  }
+  __threadfence();
+  __syncthreads();
+
+  // Ordered emission: popcount prefix scan over the bitmap, one word per thread per round.
+  int32_t* cache_out = a.topk_cache ? a.topk_cache + (int64_t)b * a.top_k : nullptr;
+  const int words = (n + 31) >> 5;
+  uint32_t running = 0;
+  for (int base = 0; base < words; base += kTopkFinalThreads) {
+    const int w = base + tid;
+    uint32_t bits = 0;
+    if (w < words) {
+      bits = __hip_atomic_load(&bitmap32[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int rem = n - (w << 5);
+      if (rem < 32) bits &= (1u << rem) - 1u;  // positions past n hold stale bits
+    }
+    const uint32_t cnt = __popc(bits);
+    uint32_t incl = cnt;
 #pragma unroll
-    for (int w = 0; w < kTopkWaves; ++w) {
-      const uint32_t g = wave_gt[w], e = wave_eq[w];
-      if (w < wave) {
-        gt_before += g;
-        eq_before += e;
+    for (int off = 1; off < 64; off <<= 1) {
+      const uint32_t up = __shfl_up(incl, off);
+      if (lane >= off) incl += up;
+    }
+    if (lane == 63) scratch[wave] = incl;
+    __syncthreads();
+    uint32_t wave_base = 0, total = 0;
+#pragma unroll
+    for (int x = 0; x < kTopkFinalThreads / 64; ++x) {
+      const uint32_t s = scratch[x];
+      if (x < wave) wave_base += s;
+      total += s;
+    }
+    uint32_t out = running + wave_base + incl - cnt;
+    while (bits) {
+      const int bit = __ffs(bits) - 1;
+      bits &= bits - 1u;
+      if (out < (uint32_t)k) {
+        const int pos = a.n_init + (w << 5) + bit;
+        emit(a.n_init + (int)out, pos);
+        if (cache_out) cache_out[out] = pos;
       }
-      gt_total += g;
-      eq_total += e;
+      ++out;
     }
-    const uint64_t below = (1ull << lane) - 1ull;
-    gt_before += __popcll(gt_mask & below);
-    eq_before += __popcll(eq_mask & below);
-    const uint32_t eq_rank = run_eq + eq_before;
-    if (gt || (eq && eq_rank < need_eq)) {
-      const uint32_t out = run_gt + gt_before + min(eq_rank, need_eq);
-      const int pos = a.n_init + i;
-      emit(a.n_init + (int)out, pos);
-      if (cache_out) cache_out[out] = pos;
-    }
-    run_gt += gt_total;
-    run_eq += eq_total;
+    running += total;
     __syncthreads();
   }
   if (tid == 0 && a.cache_len) a.cache_len[b] = k;
 }
 
-}  // namespace ts
-
-using namespace ts;
-
-extern "C" {
-
-size_t ts_topk_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
-  (void)cfg;
-  (void)batch;
-  (void)max_seq_len;
-  return 256;
+static size_t bitmap_words_for(int max_n) {
+  return align_up((size_t)ceil_div(max_n > 0 ? max_n : 1, 64) * 2, 64);
 }
 
-int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
-                   int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
-                   int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
-                   void* workspace, size_t workspace_bytes, ts_stream_t stream) {
-  (void)workspace;
-  (void)workspace_bytes;
-  TS_TRY(validate_config(cfg));
-  TS_TRY(validate_batch(cfg, bt));
-  TS_REQUIRE(votes && sel && sel_pos && sel_len, TS_EINVAL, "ts_topk_ragged: NULL tensor argument");
-  const int max_sel = cfg->n_init + cfg->top_k + cfg->n_local;
-  TS_REQUIRE(sel_stride >= max_sel, TS_EWORKSPACE, "sel_stride %lld < n_init+top_k+n_local = %d",
-             (long long)sel_stride, max_sel);
-  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
-  TS_REQUIRE(vote_stride >= max_n, TS_EWORKSPACE, "vote_stride %lld < max candidates %d",
-             (long long)vote_stride, max_n);
-  TS_REQUIRE(hit == nullptr || cache != nullptr, TS_EINVAL,
-             "ts_topk_ragged: hit flags need the selection cache");
-  if (cache)
-    TS_REQUIRE(cache->topk_cache && cache->cache_len, TS_EINVAL,
-               "ts_topk_ragged: selection cache has a NULL array");
+size_t topk_ws_stride_words(int max_n) {
+  return align_up(kTopkCounterWords + bitmap_words_for(max_n) + (size_t)(max_n > 0 ? max_n : 1) * 2,
+                  64);
+}
 
+TopkArgs make_topk_args(const ts_config* cfg, const ts_batch* bt, const float* votes,
+                        int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
+                        int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
+                        uint32_t* workspace) {
   TopkArgs a;
   a.votes = votes;
   a.vote_stride = vote_stride;
@@ -216,9 +342,69 @@ int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
   a.sel_pos = sel_pos;
   a.sel_stride = sel_stride;
   a.sel_len = sel_len;
-  hipLaunchKernelGGL(topk_kernel, dim3((unsigned)bt->batch), dim3(kTopkThreads), 0,
-                     (hipStream_t)stream, a);
-  return check_launch("topk_kernel");
+  a.ws = workspace;
+  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
+  a.bitmap_words = (int)bitmap_words_for(max_n);
+  a.cand_cap = (uint32_t)(max_n > 0 ? max_n : 1);
+  a.ws_stride = topk_ws_stride_words(max_n);
+  return a;
+}
+
+int launch_topk(const TopkArgs& a, int batch, int max_n, bool zero, bool hist, hipStream_t stream) {
+  if (max_n > 0) {
+    const dim3 grid((unsigned)ceil_div(max_n, kTopkSlice), (unsigned)batch);
+    if (zero) {
+      hipLaunchKernelGGL(topk_zero_kernel, dim3((unsigned)batch), dim3(256), 0, stream, a.ws,
+                         a.ws_stride);
+      TS_TRY(check_launch("topk_zero_kernel"));
+    }
+    if (hist) {
+      hipLaunchKernelGGL(topk_hist_kernel, grid, dim3(256), 0, stream, a);
+      TS_TRY(check_launch("topk_hist_kernel"));
+    }
+    hipLaunchKernelGGL(topk_mark_kernel, grid, dim3(256), 0, stream, a);
+    TS_TRY(check_launch("topk_mark_kernel"));
+  }
+  hipLaunchKernelGGL(topk_final_kernel, dim3((unsigned)batch), dim3(kTopkFinalThreads), 0, stream, a);
+  return check_launch("topk_final_kernel");
+}
+
+}  // namespace ts
+
+using namespace ts;
+
+extern "C" {
+
+size_t ts_topk_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+  if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
+  const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
+  return align_up(topk_ws_stride_words(max_n) * 4 * (size_t)batch, 256);
+}
+
+int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
+                   int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
+                   int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
+                   void* workspace, size_t workspace_bytes, ts_stream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_TRY(validate_batch(cfg, bt));
+  TS_REQUIRE(votes && sel && sel_pos && sel_len, TS_EINVAL, "ts_topk_ragged: NULL tensor argument");
+  const int max_sel = cfg->n_init + cfg->top_k + cfg->n_local;
+  TS_REQUIRE(sel_stride >= max_sel, TS_EWORKSPACE, "sel_stride %lld < n_init+top_k+n_local = %d",
+             (long long)sel_stride, max_sel);
+  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
+  TS_REQUIRE(vote_stride >= max_n, TS_EWORKSPACE, "vote_stride %lld < max candidates %d",
+             (long long)vote_stride, max_n);
+  TS_REQUIRE(hit == nullptr || cache != nullptr, TS_EINVAL,
+             "ts_topk_ragged: hit flags need the selection cache");
+  if (cache)
+    TS_REQUIRE(cache->topk_cache && cache->cache_len, TS_EINVAL,
+               "ts_topk_ragged: selection cache has a NULL array");
+  const size_t need = ts_topk_workspace_bytes(cfg, bt->batch, bt->max_seq_len);
+  TS_REQUIRE(workspace != nullptr && workspace_bytes >= need, TS_EWORKSPACE,
+             "ts_topk_ragged: workspace %zu bytes < required %zu", workspace_bytes, need);
+  const TopkArgs a = make_topk_args(cfg, bt, votes, vote_stride, hit, cache, sel, sel_pos,
+                                    sel_stride, sel_len, (uint32_t*)workspace);
+  return launch_topk(a, bt->batch, max_n, /*zero=*/true, /*hist=*/true, (hipStream_t)stream);
 }
 
 }  // extern "C"

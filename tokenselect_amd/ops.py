@@ -148,7 +148,9 @@ def _c_cache(cache: Optional[SelectionCache], cfg: LayerConfig, batch: int):
 
 
 def score_stride_for(max_seq_len: int) -> int:
-    return (max_seq_len + 63) // 64 * 64
+    """Row stride of the score / vote buffers: ``ts_score_stride`` (a multiple of 64
+    elements that keeps head rows off a power-of-two distance)."""
+    return int(_lib.load().ts_score_stride(int(max_seq_len)))
 
 
 # ------------------------------------------------------------- entry points
@@ -263,8 +265,10 @@ def topk_ragged(cfg: LayerConfig, bt: Batch, votes: torch.Tensor,
     sel = torch.empty((B, cfg.max_sel), dtype=torch.int32, device=votes.device)
     sel_pos = torch.empty_like(sel)
     sel_len = torch.empty((B,), dtype=torch.int32, device=votes.device)
-    ws = torch.empty((256,), dtype=torch.uint8, device=votes.device)
-    _lib.check(_lib.load().ts_topk_ragged(ctypes.byref(c), ctypes.byref(cb), _p(votes),
+    lib = _lib.load()
+    nbytes = lib.ts_topk_workspace_bytes(ctypes.byref(c), B, bt.max_seq_len)
+    ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=votes.device)
+    _lib.check(lib.ts_topk_ragged(ctypes.byref(c), ctypes.byref(cb), _p(votes),
                                           votes.shape[1], _p(hit), _c_cache(cache, cfg, B), _p(sel),
                                           _p(sel_pos), cfg.max_sel, _p(sel_len), _p(ws), ws.numel(),
                                           _stream()))
