@@ -116,24 +116,28 @@ int ts_paged_matmul(const void* query, const void* token, int64_t pool_rows,
 
 /* Scoring pass of get_topk_tokens over a ragged batch (tr.py:350-359), one
  * kernel launch: for every request that is not dense (n_init+k+n_local >= L,
- * tr.py:377) and whose skip[b] is 0, scores[(b*H+h)*score_stride + t] for
- * candidates t in [0, L-n_init-n_local), and per-workgroup softmax partials
- * (max, sum exp) that ts_vote merges.  partials holds at least
- * ts_score_partials_bytes() bytes.  qf [B,H,D] bf16 is the rotated fingerprint
- * (tr.py:380-392). */
+ * tr.py:377) and whose skip[b] is 0, the fp32 score of every candidate t in
+ * [0, L-n_init-n_local) and query head, and per-workgroup softmax partials
+ * (max, sum exp) that ts_vote merges.
+ * scores is tile-major so that it can be written in long bursts:
+ *   scores[((b*score_stride/16 + t/16)*H + slot)*16 + t%16],
+ * 16 candidates per tile, head slot = kvh*G + g for query g of KV head kvh
+ * (head kvh + Hkv*g under TS_HEADMAP_MOD, head kvh*G + g under TS_HEADMAP_DIV);
+ * score_stride is the number of candidate slots per request, a multiple of 16.
+ * partials holds at least ts_score_partials_bytes() bytes.  qf [B,H,D] bf16 is
+ * the rotated fingerprint (tr.py:380-392). */
 size_t ts_score_partials_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
-/* Recommended score_stride / vote_stride (elements) for max_seq_len: a multiple
- * of 64 that is not a power-of-two distance between head rows. */
+/* Recommended score_stride / vote_stride for max_seq_len (a multiple of 64). */
 int64_t ts_score_stride(int32_t max_seq_len);
 int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
              int64_t pool_rows, const int32_t* skip, float* scores, int64_t score_stride,
              float* partials, size_t partials_bytes, ts_stream_t stream);
 
 /* Soft vote (tr.py:361): merges the partials into stats[(b*H+h)*2 + {0,1}] =
- * {max_t s, sum_t exp(s - max)}, then votes[b*vote_stride + t] =
- * sum_h exp(s[h,t]-max_h)/Z_h, then the optional max-pool of tr.py:366-369 when
- * cfg->pool_kernel > 0 (pooled is then the result and votes the scratch; both
- * [B, vote_stride]). */
+ * {max_t s, sum_t exp(s - max)} (by head h), then votes[b*vote_stride + t] =
+ * sum_h exp(s[h,t]-max_h)/Z_h from the tile-major scores, then the optional
+ * max-pool of tr.py:366-369 when cfg->pool_kernel > 0 (pooled is then the result
+ * and votes the scratch; both [B, vote_stride]). */
 int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
             int64_t score_stride, const float* partials, const int32_t* skip, float* stats,
             float* votes, float* pooled, int64_t vote_stride, ts_stream_t stream);

@@ -91,7 +91,8 @@ def test_score_vote_topk(dev, shape, page):
         d = details[b]
         n = L - c.n_init - c.n_local
         assert torch.equal(qf[b].reshape(-1).cpu().view(torch.int16), d["qf"].view(torch.int16))
-        assert_scores_close(scores[b, :, :n].cpu(), d["scores"], f"scores b={b}")
+        assert_scores_close(ops.scores_head_major(c, scores)[b, :, :n].cpu(), d["scores"],
+                            f"scores b={b}")
         ref_stats_m = d["scores"].max(dim=1).values
         assert torch.allclose(stats[b, :, 0].cpu(), ref_stats_m, rtol=1e-5, atol=1e-5)
         assert torch.allclose(votes[b, :n].cpu(), d["votes"], rtol=2e-4, atol=1e-9)

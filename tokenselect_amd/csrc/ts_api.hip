@@ -68,20 +68,20 @@ int validate_batch(const ts_config* cfg, const ts_batch* bt) {
   return TS_OK;
 }
 
-int score_tokens_per_block(int64_t total_candidates) {
-  // The scoring kernel keeps one workgroup per CU resident (its operand and
-  // staging registers fill the register file), so aim for one workgroup per CU on
-  // 256 CUs; 64-row granularity keeps every wave on whole 16-row tiles.
+int score_tokens_per_block(int64_t total_candidates, int num_heads) {
+  // Two workgroups per CU are resident (register budget), so aim for 512
+  // workgroups on 256 CUs, in 64-row steps (every wave on whole 16-row tiles).  A
+  // workgroup stages its fp32 scores in LDS, tokens * heads * 4 bytes <= 64 KB.
   static const int forced = [] {
     const char* e = getenv("TS_SCORE_TOKENS_PER_BLOCK");  // tuning override, multiple of 64
     const int v = e ? atoi(e) : 0;
     return (v >= 64 && v <= 8192) ? v / 64 * 64 : 0;
   }();
-  if (forced) return forced;
-  int64_t per = ceil_div(total_candidates, 256);
-  per = ceil_div(per, 64) * 64;
+  int64_t cap = (16384 / (num_heads > 0 ? num_heads : 1)) / 64 * 64;
+  if (cap < 64) cap = 64;
+  int64_t per = forced ? forced : ceil_div(ceil_div(total_candidates, 512), 64) * 64;
   if (per < 64) per = 64;
-  if (per > 1024) per = 1024;
+  if (per > cap) per = cap;
   return (int)per;
 }
 
@@ -98,12 +98,7 @@ const char* ts_last_error(void) { return ts::g_error; }
 int ts_check_config(const ts_config* cfg) { return validate_config(cfg); }
 
 int64_t ts_score_stride(int32_t max_seq_len) {
-  // An odd number of 256-byte units between head rows: the H rows that a tile of
-  // tokens touches then spread over the memory channels instead of piling onto
-  // one (a power-of-two stride such as 131072 floats does exactly that).
-  int64_t units = ceil_div(max_seq_len > 0 ? max_seq_len : 1, 64);
-  if ((units & 1) == 0) units += 1;
-  return units * 64;
+  return ceil_div(max_seq_len > 0 ? max_seq_len : 1, 64) * 64;
 }
 
 // Workspace of ts_decode_layer, carved in this order (256-byte aligned pieces).

@@ -31,7 +31,7 @@ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Candidate rows per workgroup of the scoring pass, shared by the launcher,
 // the statistics merge and the workspace query.
-int score_tokens_per_block(int64_t total_candidates);
+int score_tokens_per_block(int64_t total_candidates, int num_heads);
 
 constexpr int kHeadDim = 128;
 constexpr float kNegBig = -3.0e38f;  // finite stand-in for -inf in running maxima

@@ -4,22 +4,30 @@
 //
 // The pass is bound by HBM: every candidate row (Hkv*256 bytes) is read exactly
 // once for all H query heads.  The dot products go through the matrix cores, not
-// because the shape is a dense GEMM (it is 4 to 8 query rows per KV head) but
-// because one v_mfma_f32_16x16x32_bf16 replaces 64 dot/reduce/select vector
-// instructions and leaves the wavefront free to keep loads in flight:
+// because the shape is a dense GEMM (it is 1 to 8 query rows per KV head) but
+// because one v_mfma_f32_16x16x32_bf16 replaces some 64 dot / reduce / select
+// vector instructions, which is what lets a wavefront keep 32 KB of loads in
+// flight instead of computing.
 //
-//   B operand = keys:    lane l holds token (l%16) of a 16-token tile, 8 dims
-//                        [32c + 8(l/16), +8) of one KV head - a 128-bit load
-//                        straight from HBM into the operand registers;
-//   A operand = queries: row 4*(g%4) + g/4 holds query g of the KV head, so
-//   D result:            lane l, register r = score of query (l/16) + 4r for
-//                        token l%16 - already one token per lane, 16
-//                        consecutive tokens per 16-lane row: a 64-byte store
-//                        per head, no cross-lane traffic at all.
+// Operand layout (lane l: rg = l/16, t4 = (l%16)/4, p = l%4).  One load
+// instruction covers four tokens of a tile and one KV head: lane l reads the 16
+// bytes at offset 64*rg + 16*p of token 4m + t4, so each token's 256-byte head
+// row is fetched as one contiguous piece and every 128-byte line is consumed by
+// a single instruction.  Seen as the B operand (column l%16, k-group rg), column
+// (t4, p) holds the dims {8(4rg + p) + e} of token t4: a quarter of the head
+// dimension per column.  The A operand uses the same mapping with the query head
+// in place of the token, so that D[(g, p'), (t4, p)] is the partial dot product
+// of query g and token t4 over quarter p when p' == p.  Each lane keeps the
+// diagonal element (register p of its 4 results) and the four quarters are added
+// across the 4 lanes of a quad with two DPP quad_perm adds.  After the four
+// instructions of a tile (m = 0..3) lane (rg, t4, p) keeps the result of m == p:
+// the score of query rg for token 4p + t4, one token per lane, 16 tokens per
+// 16-lane row, stored as one 64-byte segment per head.
 //
 // Products of bf16 pairs are exact in fp32 and the accumulation is fp32.
 // Loads are double-buffered in half iterations (16 x 128-bit loads per lane
-// each) and the table entry of the next tile is fetched one iteration ahead.
+// each) and the table entries of the next iteration are fetched one iteration
+// ahead.
 #include "ts_common.h"
 
 namespace ts {
@@ -52,15 +60,35 @@ __device__ __forceinline__ int head_of(int kvh, int g, int head_map) {
   return head_map == TS_HEADMAP_MOD ? kvh + HKV * g : kvh * G + g;
 }
 
+// 128-bit load with the non-temporal hint: the keys are read once, and keeping
+// them out of the caches' replacement order is worth about 10 % of streaming
+// bandwidth on this part.
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+__device__ __forceinline__ uint4 load_streaming(const char* p) {
+  const u32x4_t v = __builtin_nontemporal_load((const u32x4_t*)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+constexpr int kQuadSwap1 = 0xB1;  // quad_perm [1,0,3,2]
+constexpr int kQuadSwap2 = 0x4E;  // quad_perm [2,3,0,1]
+
 // One iteration of a wave covers TG tiles of 16 tokens and all HKV heads: always
 // 8 (tile, KV head) units = 32 loads of 1 KB.  Units 0-3 and 4-7 alternate
 // between two register buffers.
-template <int HKV, int G, bool OUT_BF16>
-__global__ __launch_bounds__(256, 1) void score_kernel(ScoreArgs a) {
+//
+// TILED (the selection path): fp32 scores leave the kernel tile-major,
+// scores[b][tile][head slot][16 tokens] with head slot = kvh*G + g.  They are
+// staged in LDS and written once per workgroup as one contiguous burst: trickling
+// 64-byte pieces into 32 separate head rows while the keys stream in costs a
+// quarter of the read bandwidth (DRAM read/write turnarounds).  Not TILED
+// (paged_matmul): scores[h][t] row-major in the caller's dtype, stored directly.
+template <int HKV, int G, bool OUT_BF16, bool TILED>
+__global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a) {
+  extern __shared__ float stage[];  // TILED: [tiles of the workgroup][H][16]
   constexpr int TG = 8 / HKV;
   constexpr int UNITS = 8;
   constexpr int HALF = UNITS / 2;
-  constexpr int NR = (G + 3) / 4;  // result registers in use per unit
+  constexpr int NA = (G + 3) / 4;  // A operands (4 query heads each) per KV head
   constexpr int ITER = 16 * TG;    // tokens per iteration
   constexpr uint32_t ROW_BYTES = HKV * kHeadDim * 2;
 
@@ -81,186 +109,225 @@ __global__ __launch_bounds__(256, 1) void score_kernel(ScoreArgs a) {
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int rg = lane >> 4;   // k-group of the operands, row group of the result
-  const int col = lane & 15;  // token inside a tile
+  const int rg = lane >> 4;        // k-group of the operands, row group of the result
+  const int t4 = (lane & 15) >> 2;  // token of a 4-token group / query of a 4-query group
+  const int p = lane & 3;           // quarter of the head dimension
+  const uint32_t lane_off = (uint32_t)(rg * 64 + p * 16);
   const int H = a.num_heads;
   const int32_t* tab = a.table + (int64_t)b * a.table_stride;
 
-  // A operands: query (col/4 + 4*(col%4)) of each KV head, dims [32c + 8rg, +8).
-  bf16x8_t qa[HKV][4];
-  {
-    const int g = (col >> 2) + 4 * (col & 3);
-#pragma unroll
-    for (int kvh = 0; kvh < HKV; ++kvh) {
-      const int h = head_of<HKV, G>(kvh, g < G ? g : 0, a.head_map);
-      const uint16_t* qrow = a.qf + ((size_t)b * H + h) * kHeadDim + rg * 8;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (g < G) v = *(const uint4*)(qrow + c * 32);
-        qa[kvh][c] = __builtin_bit_cast(bf16x8_t, v);
-      }
-    }
-  }
-
-  float run_m[HKV][NR], run_l[HKV][NR];
+  // A operands: query 4*na + t4 of each KV head, same byte offsets as the keys.
+  bf16x8_t qa[HKV][NA];
 #pragma unroll
   for (int kvh = 0; kvh < HKV; ++kvh)
 #pragma unroll
-    for (int r = 0; r < NR; ++r) {
-      run_m[kvh][r] = kNegBig;
-      run_l[kvh][r] = 0.f;
+    for (int na = 0; na < NA; ++na) {
+      const int g = 4 * na + t4;
+      const int h = head_of<HKV, G>(kvh, g < G ? g : 0, a.head_map);
+      uint4 v = *(const uint4*)((const char*)(a.qf + ((size_t)b * H + h) * kHeadDim) + lane_off);
+      if (g >= G) v = make_uint4(0u, 0u, 0u, 0u);
+      qa[kvh][na] = __builtin_bit_cast(bf16x8_t, v);
+    }
+
+  float run_m[HKV][NA], run_l[HKV][NA];
+#pragma unroll
+  for (int kvh = 0; kvh < HKV; ++kvh)
+#pragma unroll
+    for (int na = 0; na < NA; ++na) {
+      run_m[kvh][na] = kNegBig;
+      run_l[kvh][na] = 0.f;
     }
 
   const int per_wave = a.tokens_per_block >> 2;
   const int wave_lo = block_lo + wave * per_wave;
   const int wave_hi = min(wave_lo + per_wave, n);
 
-  // Lane (rg, col) addresses token `tile + col` of every tile.  The table load and
-  // the slot arithmetic are split so that the entry of the next iteration is
-  // requested a whole iteration before it is needed.  Positions past the wave's
-  // range are clamped to its last token: every load stays in bounds and no branch
-  // splits the load pipeline.
+  // Lane (rg, t4, p) addresses tokens tile + 4m + t4, m = 0..3, of every tile.
+  // The table loads and the slot arithmetic are split so that the entries of the
+  // next iteration are requested a whole iteration before they are needed.
+  // Positions past the wave's range are clamped to its last token: every load
+  // stays in bounds and no branch splits the load pipeline.
   const int last_pos = first_pos + max(wave_hi - 1, 0);
   const int page_mask = a.page_size - 1;
-  auto table_entry = [&](int tile) -> int32_t {
-    const int pos = min(first_pos + tile + col, last_pos);
+  auto table_entry = [&](int tok) -> int32_t {
+    const int pos = min(first_pos + tok, last_pos);
     return tab[pos >> a.page_shift];
   };
-  auto row_ptr = [&](int32_t entry, int tile) -> const char* {
-    const int pos = min(first_pos + tile + col, last_pos);
+  // Byte offset of this lane's 16 bytes inside the pool.  Offsets, not pointers,
+  // are carried across iterations: a pointer rebuilt from the kernel argument at
+  // the load is known to be global memory, whereas a loop-carried pointer decays
+  // to a flat access, whose completion the wave must wait for in full.
+  auto row_off = [&](int32_t entry, int tok) -> size_t {
+    const int pos = min(first_pos + tok, last_pos);
     uint32_t slot = ((uint32_t)entry << a.page_shift) + (uint32_t)(pos & page_mask);
     slot = slot < a.pool_rows ? slot : a.pool_rows - 1;
-    return (const char*)a.k_pool + (size_t)slot * ROW_BYTES + rg * 16;
+    return (size_t)slot * ROW_BYTES + lane_off;
   };
+  const char* const pool = (const char*)a.k_pool;
+
+  // Lane-constant bit masks: all ones where p == i.  Selecting with and/or keeps
+  // the loop free of branches (a ternary chain on p is lowered to a switch).
+  uint32_t pmask[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    pmask[i] = p == i ? 0xffffffffu : 0u;
+    asm volatile("" : "+v"(pmask[i]));
+  }
 
   uint4 buf0[HALF][4], buf1[HALF][4];
   auto issue = [&](uint4 (&buf)[HALF][4], auto& rows, int first_unit) {
 #pragma unroll
     for (int i = 0; i < HALF; ++i) {
       const int u = first_unit + i;
-      const char* p = rows[u / HKV] + (u % HKV) * (kHeadDim * 2);
 #pragma unroll
-      for (int c = 0; c < 4; ++c) buf[i][c] = *(const uint4*)(p + c * 64);
+      for (int m = 0; m < 4; ++m)
+        buf[i][m] = load_streaming(pool + rows[u / HKV][m] + (u % HKV) * (kHeadDim * 2));
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  auto multiply = [&](const uint4 (&buf)[HALF][4], f32x4_t (&acc)[UNITS], int first_unit) {
+  // res[u][na]: score of query 4*na + rg (of the unit's KV head) for token
+  // tile + 4p + t4.
+  auto multiply = [&](const uint4 (&buf)[HALF][4], float (&res)[UNITS][NA], int first_unit) {
 #pragma unroll
     for (int i = 0; i < HALF; ++i) {
       const int u = first_unit + i;
-      f32x4_t d = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[u % HKV][c],
-                                                    __builtin_bit_cast(bf16x8_t, buf[i][c]), d, 0, 0, 0);
-      acc[u] = d;
+      for (int na = 0; na < NA; ++na) {
+        uint32_t keep = 0u;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+          const f32x4_t d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              qa[u % HKV][na], __builtin_bit_cast(bf16x8_t, buf[i][m]), zero, 0, 0, 0);
+          float v = __uint_as_float((__float_as_uint(d[0]) & pmask[0]) | (__float_as_uint(d[1]) & pmask[1]) |
+                                    (__float_as_uint(d[2]) & pmask[2]) | (__float_as_uint(d[3]) & pmask[3]));
+          v += dpp_move<kQuadSwap1>(v);
+          v += dpp_move<kQuadSwap2>(v);
+          keep |= __float_as_uint(v) & pmask[m];
+        }
+        res[u][na] = __uint_as_float(keep);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  const char* rows_cur[TG];
-  const char* rows_next[TG];
+  size_t rows_cur[TG][4];
+  size_t rows_next[TG][4];
   if (wave_lo < wave_hi) {
 #pragma unroll
-    for (int t = 0; t < TG; ++t) rows_cur[t] = row_ptr(table_entry(wave_lo + 16 * t), wave_lo + 16 * t);
+    for (int t = 0; t < TG; ++t)
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int tok = wave_lo + 16 * t + 4 * m + t4;
+        rows_cur[t][m] = row_off(table_entry(tok), tok);
+      }
     issue(buf0, rows_cur, 0);
   }
 
   for (int base = wave_lo; base < wave_hi; base += ITER) {
-    int32_t entry_next[TG];
+    int32_t entry_next[TG][4];
 #pragma unroll
-    for (int t = 0; t < TG; ++t) entry_next[t] = table_entry(base + ITER + 16 * t);
+    for (int t = 0; t < TG; ++t)
+#pragma unroll
+      for (int m = 0; m < 4; ++m) entry_next[t][m] = table_entry(base + ITER + 16 * t + 4 * m + t4);
     __builtin_amdgcn_sched_barrier(0);
 
-    f32x4_t acc[UNITS];
+    float res[UNITS][NA];
     issue(buf1, rows_cur, HALF);
-    multiply(buf0, acc, 0);
+    multiply(buf0, res, 0);
 #pragma unroll
-    for (int t = 0; t < TG; ++t) rows_next[t] = row_ptr(entry_next[t], base + ITER + 16 * t);
+    for (int t = 0; t < TG; ++t)
+#pragma unroll
+      for (int m = 0; m < 4; ++m)
+        rows_next[t][m] = row_off(entry_next[t][m], base + ITER + 16 * t + 4 * m + t4);
     issue(buf0, rows_next, 0);
-    multiply(buf1, acc, HALF);
+    multiply(buf1, res, HALF);
 #pragma unroll
-    for (int t = 0; t < TG; ++t) rows_cur[t] = rows_next[t];
+    for (int t = 0; t < TG; ++t)
+#pragma unroll
+      for (int m = 0; m < 4; ++m) rows_cur[t][m] = rows_next[t][m];
 
-    // Lane (rg, col), register r of unit (tile t, head kvh): query rg + 4r, token
-    // base + 16t + col.
 #pragma unroll
     for (int u = 0; u < UNITS; ++u) {
       const int t = u / HKV, kvh = u % HKV;
-      const int tok = base + 16 * t + col;
+      const int tok = base + 16 * t + 4 * p + t4;
 #pragma unroll
-      for (int r = 0; r < NR; ++r) {
-        const int g = rg + 4 * r;
+      for (int na = 0; na < NA; ++na) {
+        const int g = 4 * na + rg;
         if (g < G && tok < wave_hi) {
           const int h = head_of<HKV, G>(kvh, g, a.head_map);
-          const float x = acc[u][r];
-          const size_t at = ((size_t)b * H + h) * (size_t)a.score_stride + (size_t)tok;
-#ifndef TS_DBG_NOSTORE
-          if (OUT_BF16)
-            ((uint16_t*)a.scores)[at] = f32_to_bf16(x);
-          else
-            ((float*)a.scores)[at] = x;
-#else
-          if (x == 1234.5678f) ((float*)a.scores)[at] = x;
-#endif
-#ifdef TS_DBG_NOSTATS
-          run_l[kvh][r] += x;
-          continue;
-#endif
+          const float x = res[u][na];
+          if (TILED) {
+            stage[(((tok - block_lo) >> 4) * H + kvh * G + g) * 16 + (tok & 15)] = x;
+          } else {
+            const size_t at = ((size_t)b * H + h) * (size_t)a.score_stride + (size_t)tok;
+            if (OUT_BF16)
+              ((uint16_t*)a.scores)[at] = f32_to_bf16(x);
+            else
+              ((float*)a.scores)[at] = x;
+          }
           // Online (max, sum exp) with a single exponential per element.
-          const float d = x - run_m[kvh][r];
+          const float d = x - run_m[kvh][na];
           const float e = __expf(-fabsf(d));
           if (d > 0.f) {
-            run_l[kvh][r] = run_l[kvh][r] * e + 1.f;
-            run_m[kvh][r] = x;
+            run_l[kvh][na] = run_l[kvh][na] * e + 1.f;
+            run_m[kvh][na] = x;
           } else {
-            run_l[kvh][r] += e;
+            run_l[kvh][na] += e;
           }
         }
       }
     }
   }
 
+  if (TILED) {  // one contiguous burst per workgroup
+    __syncthreads();
+    const int tiles = (min(a.tokens_per_block, n - block_lo) + 15) >> 4;
+    float4* dst = (float4*)((float*)a.scores + ((size_t)b * a.score_stride + block_lo) * H);
+    const float4* src = (const float4*)stage;
+    for (int i = threadIdx.x; i < tiles * H * 4; i += 256) dst[i] = src[i];
+  }
   if (a.partials == nullptr) return;
 
-  __shared__ float sm_m[4][4][HKV][NR];
-  __shared__ float sm_l[4][4][HKV][NR];
+  // Per-workgroup (max, sum exp) of every head: 16 lanes of a row, then 4 waves.
+  __shared__ float sm_m[4][4][HKV][NA];
+  __shared__ float sm_l[4][4][HKV][NA];
 #pragma unroll
   for (int kvh = 0; kvh < HKV; ++kvh)
 #pragma unroll
-    for (int r = 0; r < NR; ++r) {
-      float m = run_m[kvh][r], l = run_l[kvh][r];
+    for (int na = 0; na < NA; ++na) {
+      float m = run_m[kvh][na], l = run_l[kvh][na];
       row16_softmax_merge(m, l);
-      if (col == 0) {
-        sm_m[wave][rg][kvh][r] = m;
-        sm_l[wave][rg][kvh][r] = l;
+      if ((lane & 15) == 0) {
+        sm_m[wave][rg][kvh][na] = m;
+        sm_l[wave][rg][kvh][na] = l;
       }
     }
   __syncthreads();
-  if ((int)threadIdx.x < H) {
-    const int h = threadIdx.x;
-    float m = kNegBig, l = 0.f;
-    for (int w = 0; w < 4; ++w)
-      for (int g4 = 0; g4 < 4; ++g4)
-        for (int kvh = 0; kvh < HKV; ++kvh)
-          for (int r = 0; r < NR; ++r) {
-            const int g = g4 + 4 * r;
-            if (g < G && head_of<HKV, G>(kvh, g, a.head_map) == h)
-              softmax_merge(m, l, sm_m[w][g4][kvh][r], sm_l[w][g4][kvh][r]);
-          }
-    float* p = a.partials + (((size_t)b * H + h) * a.nchunks + blockIdx.x) * 2;
-    p[0] = m;
-    p[1] = l;
+  if ((int)threadIdx.x < 4 * HKV * NA) {
+    const int na = threadIdx.x % NA;
+    const int kvh = (threadIdx.x / NA) % HKV;
+    const int g4 = threadIdx.x / (NA * HKV);
+    const int g = 4 * na + g4;
+    if (g < G) {
+      float m = sm_m[0][g4][kvh][na], l = sm_l[0][g4][kvh][na];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) softmax_merge(m, l, sm_m[w][g4][kvh][na], sm_l[w][g4][kvh][na]);
+      const int h = head_of<HKV, G>(kvh, g, a.head_map);
+      float* out = a.partials + (((size_t)b * H + h) * a.nchunks + blockIdx.x) * 2;
+      out[0] = m;
+      out[1] = l;
+    }
   }
 }
 
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool TILED>
 static int launch_score(int hkv, int group, const ScoreArgs& a, dim3 grid, hipStream_t stream) {
-#define TS_SCORE_CASE(HKV_, G_)                                                              \
-  if (hkv == HKV_ && group == G_) {                                                          \
-    hipLaunchKernelGGL((score_kernel<HKV_, G_, OUT_BF16>), grid, dim3(256), 0, stream, a);   \
-    return check_launch("score_kernel");                                                     \
+  const size_t lds = TILED ? (size_t)a.tokens_per_block * a.num_heads * sizeof(float) : 0;
+#define TS_SCORE_CASE(HKV_, G_)                                                                  \
+  if (hkv == HKV_ && group == G_) {                                                              \
+    hipLaunchKernelGGL((score_kernel<HKV_, G_, OUT_BF16, TILED>), grid, dim3(256), lds, stream, a); \
+    return check_launch("score_kernel");                                                         \
   }
 #define TS_SCORE_ROW(HKV_) \
   TS_SCORE_CASE(HKV_, 1) TS_SCORE_CASE(HKV_, 2) TS_SCORE_CASE(HKV_, 4) TS_SCORE_CASE(HKV_, 7) TS_SCORE_CASE(HKV_, 8)
@@ -281,7 +348,7 @@ extern "C" {
 
 size_t ts_score_partials_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
-  const int tpb = score_tokens_per_block((int64_t)batch * max_seq_len);
+  const int tpb = score_tokens_per_block((int64_t)batch * max_seq_len, cfg->num_heads);
   const size_t nchunks = (size_t)ceil_div(max_seq_len, tpb);
   return align_up((size_t)batch * cfg->num_heads * nchunks * 2 * sizeof(float), 256);
 }
@@ -295,8 +362,9 @@ int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const voi
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
-  TS_REQUIRE(score_stride >= max_n && score_stride >= 1, TS_EWORKSPACE,
-             "score_stride %lld < max candidates %d", (long long)score_stride, max_n);
+  TS_REQUIRE(score_stride >= max_n && score_stride >= 16 && score_stride % 16 == 0, TS_EWORKSPACE,
+             "score_stride %lld must be a multiple of 16 and >= max candidates %d",
+             (long long)score_stride, max_n);
   const size_t need = ts_score_partials_bytes(cfg, bt->batch, bt->max_seq_len);
   TS_REQUIRE(partials_bytes >= need, TS_EWORKSPACE, "ts_score: partials %zu bytes < required %zu",
              partials_bytes, need);
@@ -321,13 +389,13 @@ int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const voi
   a.scores = scores;
   a.score_stride = score_stride;
   a.partials = partials;
-  a.tokens_per_block = score_tokens_per_block((int64_t)bt->batch * bt->max_seq_len);
+  a.tokens_per_block = score_tokens_per_block((int64_t)bt->batch * bt->max_seq_len, cfg->num_heads);
   a.nchunks = (int)ceil_div(bt->max_seq_len, a.tokens_per_block);
   a.num_heads = cfg->num_heads;
   a.head_map = cfg->head_map;
   const dim3 grid((unsigned)ceil_div(max_n, a.tokens_per_block), (unsigned)bt->batch);
-  return launch_score<false>(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, a, grid,
-                             (hipStream_t)stream);
+  return launch_score<false, true>(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, a, grid,
+                                   (hipStream_t)stream);
 }
 
 int ts_paged_matmul(const void* query, const void* token, int64_t pool_rows,
@@ -366,14 +434,16 @@ int ts_paged_matmul(const void* query, const void* token, int64_t pool_rows,
   a.scores = scores;
   a.score_stride = n;
   a.partials = nullptr;
-  a.tokens_per_block = score_tokens_per_block(n);
+  a.tokens_per_block = score_tokens_per_block(n, num_heads);
   a.nchunks = (int)ceil_div(n, a.tokens_per_block);
   a.num_heads = num_heads;
   a.head_map = TS_HEADMAP_MOD;
   const dim3 grid((unsigned)a.nchunks, 1);
   if (scores_dtype == TS_DTYPE_BF16)
-    return launch_score<true>(num_kv_heads, num_heads / num_kv_heads, a, grid, (hipStream_t)stream);
-  return launch_score<false>(num_kv_heads, num_heads / num_kv_heads, a, grid, (hipStream_t)stream);
+    return launch_score<true, false>(num_kv_heads, num_heads / num_kv_heads, a, grid,
+                                     (hipStream_t)stream);
+  return launch_score<false, false>(num_kv_heads, num_heads / num_kv_heads, a, grid,
+                                    (hipStream_t)stream);
 }
 
 }  // extern "C"

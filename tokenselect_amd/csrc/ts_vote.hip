@@ -1,5 +1,9 @@
 // Soft vote: per-head softmax over the candidates summed over heads (tr.py:361),
 // and the optional max-pool smoothing of the votes (tr.py:366-369).
+//
+// Scores arrive tile-major from the scoring pass: scores[b][tile][slot][16] with
+// head slot = kvh*G + g (see ts_score.hip); a thread owns one candidate and walks
+// the H slots of its tile, so a wavefront reads four contiguous 16*H*4-byte tiles.
 #include "ts_common.h"
 
 namespace ts {
@@ -8,14 +12,14 @@ constexpr int kMaxHeads = 128;
 
 struct VoteArgs {
   const float* scores;
-  int64_t score_stride;
-  const float* partials;  // [B,H,nchunks,2] from the scoring pass
+  int64_t score_stride;   // token slots per request (multiple of 16)
+  const float* partials;  // [B,H,nchunks,2] from the scoring pass, by head
   int nchunks, tokens_per_block;
-  float* stats;           // [B,H,2] merged (max, sum exp)
+  float* stats;           // [B,H,2] merged (max, sum exp), by head
   const int32_t* seq_lens;
   const int32_t* k_per_req;
   const int32_t* skip;
-  int n_init, n_local, top_k, num_heads, max_seq_len;
+  int n_init, n_local, top_k, num_heads, num_kv_heads, head_map, max_seq_len;
   float* votes;
   int64_t vote_stride;
 };
@@ -24,7 +28,8 @@ struct VoteArgs {
 __global__ __launch_bounds__(64) void stats_merge_kernel(VoteArgs a) {
   const int h = blockIdx.x, b = blockIdx.y;
   if (a.skip && a.skip[b]) return;
-  const ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  const ReqGeom geo =
+      request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
   if (geo.n <= 0) return;
   const int chunks = (geo.n + a.tokens_per_block - 1) / a.tokens_per_block;
   const float* p = a.partials + ((size_t)b * a.num_heads + h) * a.nchunks * 2;
@@ -39,35 +44,40 @@ __global__ __launch_bounds__(64) void stats_merge_kernel(VoteArgs a) {
   }
 }
 
-// One thread per candidate, heads visited in ascending order (fp32 sum).
+// One thread per candidate; fp32 sum over the head slots in slot order.
 __global__ __launch_bounds__(256) void vote_kernel(VoteArgs a) {
   const int b = blockIdx.y;
   if (a.skip && a.skip[b]) return;
-  const ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
-  const int t0 = blockIdx.x * 1024;
-  if (t0 >= geo.n) return;
+  const ReqGeom geo =
+      request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (blockIdx.x * 256 >= geo.n) return;
 
   __shared__ float s_max[kMaxHeads];
   __shared__ float s_rz[kMaxHeads];
   const int H = a.num_heads;
-  for (int h = threadIdx.x; h < H; h += blockDim.x) {
-    s_max[h] = a.stats[((size_t)b * H + h) * 2];
-    s_rz[h] = 1.0f / a.stats[((size_t)b * H + h) * 2 + 1];
+  const int group = H / a.num_kv_heads;
+  for (int slot = threadIdx.x; slot < H; slot += 256) {
+    const int kvh = slot / group, g = slot % group;
+    const int h = a.head_map == TS_HEADMAP_MOD ? kvh + a.num_kv_heads * g : slot;
+    s_max[slot] = a.stats[((size_t)b * H + h) * 2];
+    s_rz[slot] = 1.0f / a.stats[((size_t)b * H + h) * 2 + 1];
   }
   __syncthreads();
+  if (t >= geo.n) return;
 
-  const float* base = a.scores + (size_t)b * H * (size_t)a.score_stride;
+  const float* p = a.scores + ((size_t)b * a.score_stride + (size_t)(t & ~15)) * H + (t & 15);
+  float c = 0.f;
+  int slot = 0;
+  for (; slot + 8 <= H; slot += 8) {
+    float s[8];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int t = t0 + r * 256 + threadIdx.x;
-    if (t >= geo.n) break;
-    float c = 0.f;
-    for (int h = 0; h < H; ++h) {
-      const float s = base[(size_t)h * a.score_stride + t];
-      c += __expf(s - s_max[h]) * s_rz[h];
-    }
-    a.votes[(size_t)b * a.vote_stride + t] = c;
+    for (int i = 0; i < 8; ++i) s[i] = p[(slot + i) * 16];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) c += __expf(s[i] - s_max[slot + i]) * s_rz[slot + i];
   }
+  for (; slot < H; ++slot) c += __expf(p[slot * 16] - s_max[slot]) * s_rz[slot];
+  a.votes[(size_t)b * a.vote_stride + t] = c;
 }
 
 struct PoolArgs {
@@ -86,7 +96,8 @@ struct PoolArgs {
 __global__ __launch_bounds__(256) void pool_kernel(PoolArgs a) {
   const int b = blockIdx.y;
   if (a.skip && a.skip[b]) return;
-  const ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  const ReqGeom geo =
+      request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
   const int pad = (a.kernel - 1) / 2;
   const int n_out = geo.n + 2 * pad - a.kernel + 1;
   const int t = blockIdx.x * 256 + threadIdx.x;
@@ -113,16 +124,16 @@ extern "C" int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* sc
   TS_REQUIRE(cfg->pool_kernel <= 0 || pooled != nullptr, TS_EINVAL,
              "ts_vote: pool_kernel %d needs a pooled buffer", cfg->pool_kernel);
   const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
-  TS_REQUIRE(score_stride >= max_n && vote_stride >= max_n, TS_EWORKSPACE,
-             "ts_vote: stride (%lld, %lld) < max candidates %d", (long long)score_stride,
-             (long long)vote_stride, max_n);
+  TS_REQUIRE(score_stride >= max_n && score_stride % 16 == 0 && vote_stride >= max_n, TS_EWORKSPACE,
+             "ts_vote: stride (%lld, %lld) < max candidates %d or score_stride not a multiple of 16",
+             (long long)score_stride, (long long)vote_stride, max_n);
   if (max_n <= 0) return TS_OK;
 
   VoteArgs a;
   a.scores = scores;
   a.score_stride = score_stride;
   a.partials = partials;
-  a.tokens_per_block = score_tokens_per_block((int64_t)bt->batch * bt->max_seq_len);
+  a.tokens_per_block = score_tokens_per_block((int64_t)bt->batch * bt->max_seq_len, cfg->num_heads);
   a.nchunks = (int)ceil_div(bt->max_seq_len, a.tokens_per_block);
   a.stats = stats;
   a.seq_lens = bt->seq_lens;
@@ -133,13 +144,15 @@ extern "C" int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* sc
   a.top_k = cfg->top_k;
   a.max_seq_len = bt->max_seq_len;
   a.num_heads = cfg->num_heads;
+  a.num_kv_heads = cfg->num_kv_heads;
+  a.head_map = cfg->head_map;
   a.votes = votes;
   a.vote_stride = vote_stride;
   hipLaunchKernelGGL(stats_merge_kernel, dim3((unsigned)cfg->num_heads, (unsigned)bt->batch), dim3(64),
                      0, (hipStream_t)stream, a);
   TS_TRY(check_launch("stats_merge_kernel"));
-  hipLaunchKernelGGL(vote_kernel, dim3((unsigned)ceil_div(max_n, 1024), (unsigned)bt->batch),
-                     dim3(256), 0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(vote_kernel, dim3((unsigned)ceil_div(max_n, 256), (unsigned)bt->batch), dim3(256),
+                     0, (hipStream_t)stream, a);
   TS_TRY(check_launch("vote_kernel"));
 
   if (cfg->pool_kernel > 0) {

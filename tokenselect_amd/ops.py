@@ -200,9 +200,11 @@ def paged_matmul(query: torch.Tensor, token: torch.Tensor, indices: torch.Tensor
 
 def score(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
           skip: Optional[torch.Tensor] = None, out: Optional[Tuple] = None):
-    """Scoring pass (tr.py:350-359), one kernel launch.  Returns ``(scores
-    [B,H,stride] fp32, partials)``; only the first ``L_b - n_init - n_local``
-    columns of a non-dense request are written.  ``partials`` are the
+    """Scoring pass (tr.py:350-359), one kernel launch.  Returns ``(scores,
+    partials)``.  ``scores`` is fp32 ``[B, stride/16, H, 16]``: tile-major, 16
+    candidates per tile, head slots ``kvh*G + g`` inside a tile (see
+    :func:`scores_head_major`); only the first ``L_b - n_init - n_local``
+    candidates of a non-dense request are written.  ``partials`` are the
     per-workgroup softmax statistics that :func:`vote` merges."""
     c, cb = cfg.to_c(), _c_batch(cfg, bt)
     _need(qf, "qf", torch.bfloat16)
@@ -215,17 +217,32 @@ def score(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
     lib = _lib.load()
     if out is None:
         stride = score_stride_for(bt.max_seq_len)
-        scores = torch.empty((B, H, stride), dtype=torch.float32, device=qf.device)
+        scores = torch.empty((B, stride // 16, H, 16), dtype=torch.float32, device=qf.device)
         nbytes = lib.ts_score_partials_bytes(ctypes.byref(c), B, bt.max_seq_len)
         partials = torch.empty((max(nbytes, 256) // 4,), dtype=torch.float32, device=qf.device)
     else:
         scores, partials = out
-        _need(scores, "scores", torch.float32, 3)
+        _need(scores, "scores", torch.float32, 4)
         _need(partials, "partials", torch.float32, 1)
+    if scores.shape[0] != B or scores.shape[2] != H or scores.shape[3] != 16:
+        raise ValueError("scores must be [B, stride/16, H, 16]")
     _lib.check(lib.ts_score(ctypes.byref(c), ctypes.byref(cb), _p(qf), _p(k_pool), k_pool.shape[0],
-                            _p(skip), _p(scores), scores.shape[2], _p(partials),
+                            _p(skip), _p(scores), scores.shape[1] * 16, _p(partials),
                             partials.numel() * 4, _stream()))
     return scores, partials
+
+
+def scores_head_major(cfg: LayerConfig, scores: torch.Tensor) -> torch.Tensor:
+    """``[B, H, stride]`` view-copy of the tile-major scores, rows in true head
+    order (slot ``kvh*G + g`` is head ``kvh + Hkv*g`` under the reference's ``%``
+    map, head ``kvh*G + g`` under the conventional one)."""
+    B, tiles, H, _ = scores.shape
+    group = H // cfg.num_kv_heads
+    slots = torch.arange(H, device=scores.device)
+    heads = (slots // group) + cfg.num_kv_heads * (slots % group) if cfg.head_map == "mod" else slots
+    out = torch.empty((B, H, tiles * 16), dtype=scores.dtype, device=scores.device)
+    out[:, heads] = scores.permute(0, 2, 1, 3).reshape(B, H, tiles * 16)
+    return out
 
 
 def vote(cfg: LayerConfig, bt: Batch, scores: torch.Tensor, partials: torch.Tensor,
@@ -233,15 +250,15 @@ def vote(cfg: LayerConfig, bt: Batch, scores: torch.Tensor, partials: torch.Tens
     """Soft vote (tr.py:361) and optional max-pool (tr.py:366-369).  Returns
     ``(votes [B, stride] fp32, stats [B,H,2] fp32 = per-head (max, sum exp))``."""
     c, cb = cfg.to_c(), _c_batch(cfg, bt)
-    _need(scores, "scores", torch.float32, 3)
+    _need(scores, "scores", torch.float32, 4)
     _need(partials, "partials", torch.float32, 1)
     B, H = bt.batch, cfg.num_heads
-    if scores.shape[0] != B or scores.shape[1] != H:
-        raise ValueError("scores do not match batch / heads")
+    if scores.shape[0] != B or scores.shape[2] != H or scores.shape[3] != 16:
+        raise ValueError("scores must be [B, stride/16, H, 16]")
     lib = _lib.load()
     if partials.numel() * 4 < lib.ts_score_partials_bytes(ctypes.byref(c), B, bt.max_seq_len):
         raise ValueError("partials buffer is smaller than ts_score_partials_bytes()")
-    stride = scores.shape[2]
+    stride = scores.shape[1] * 16
     stats = torch.empty((B, H, 2), dtype=torch.float32, device=scores.device)
     votes = torch.empty((B, stride), dtype=torch.float32, device=scores.device)
     pooled = torch.empty_like(votes) if cfg.pool_kernel > 0 else None
