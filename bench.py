@@ -7,9 +7,14 @@ attention) over one synthetic batch resident in HBM, issued as a single
 ``ts_decode_layer`` call.  The default workload is the Llama-3-8B layer at
 128K context in a page-16 KV pool (``--workload c2``).
 
+Every step reads a different copy of the K/V pool (``--pools``, default 4, as
+consecutive layers of a model do): the copies together exceed the 256 MB
+last-level cache, so the keys really stream from HBM in every timed pass.
+
 Prints one JSON line: the per-layer latency, the roofline figures of the
-scoring kernel (algorithmic bytes / HIP-event time of ``ts_score``, which is
-exactly one kernel launch) and the CPU oracle timed on the host cores.
+scoring kernel (algorithmic bytes / HIP-event time of the one kernel launch that
+streams the keys: the cooperative score + vote kernel when the batch fits it,
+else ``ts_score``) and the CPU oracle timed on the host cores.
 """
 
 import argparse
@@ -26,17 +31,22 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 
-def event_time_us(fn, launches: int, warmup: int):
-    """Average duration of `fn`'s work on the current stream, HIP events around
-    every launch (torch.cuda.Event records on the stream the library launches on)."""
-    for _ in range(warmup):
-        fn()
+def event_time_us(fn, launches: int, warmup: int, before=None):
+    """Average duration of `fn(i)`'s work on the current stream, HIP events around
+    every launch (torch.cuda.Event records on the stream the library launches on).
+    `before()` runs ahead of each start event, outside the timed span."""
+    for i in range(warmup):
+        if before:
+            before()
+        fn(i)
     torch.cuda.synchronize()
     pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
              for _ in range(launches)]
-    for start, end in pairs:
+    for i, (start, end) in enumerate(pairs):
+        if before:
+            before()
         start.record()
-        fn()
+        fn(i)
         end.record()
     torch.cuda.synchronize()
     times = [s.elapsed_time(e) * 1e3 for s, e in pairs]
@@ -79,6 +89,8 @@ def main():
     ap.add_argument("--cpu-reps", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layers", type=int, default=32, help="layers for the tokens/s figure")
+    ap.add_argument("--pools", type=int, default=4,
+                    help="copies of the K/V pool cycled through, one per step")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the one-GPU hot path only; run with --gpus 1 "
@@ -92,29 +104,45 @@ def main():
     wl = {"c1": workloads.config1, "c2": workloads.config2, "c3": workloads.config3}[args.workload](dev)
     c, bt, B = wl.cfg, wl.batch, len(wl.seq_lens)
     layer = ops.DecodeLayer(c, B, bt.max_seq_len, dev)
+    n_pools = max(1, args.pools)
+    k_pools = [wl.k_pool] + [wl.k_pool.clone() for _ in range(n_pools - 1)]
+    v_pools = [wl.v_pool] + [wl.v_pool.clone() for _ in range(n_pools - 1)]
 
-    def step():
-        layer(wl.q, wl.k_pool, wl.v_pool, bt)
+    def step(i):
+        layer(wl.q, k_pools[i % n_pools], v_pools[i % n_pools], bt)
 
-    for _ in range(args.warmup):
-        step()
+    for i in range(args.warmup):
+        step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    for i in range(args.steps):
+        step(i)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     us_per_layer = elapsed / args.steps * 1e6
 
-    # Kernel-level roofline figures: the scoring kernel and the gather attention.
+    # Kernel-level roofline figures: the kernel that streams the keys, and the
+    # gather attention.
     cos, sin = ops.scoring_cos_sin(c.head_dim, c.rope_theta, c.rope_scale, c.n_local, dev)
     qf = ops.rope_apply(wl.q.view(B, c.num_heads, c.head_dim), cos, sin, None)
-    bufs = ops.score(c, bt, qf, wl.k_pool)
-    score_us, score_min = event_time_us(lambda: ops.score(c, bt, qf, wl.k_pool, out=bufs),
-                                        args.steps, args.warmup)
+    fused = ops.score_vote_supported(c, B, bt.max_seq_len)
+    if fused:
+        space = ops.SelectionWorkspace(c, B, bt.max_seq_len, dev)
+        score_us, score_min = event_time_us(
+            lambda i: ops.score_vote(c, bt, qf, k_pools[i % n_pools], space),
+            args.steps, args.warmup, before=space.reset)
+        if space.fault():
+            sys.exit("bench.py: the grid-wide wait of the score+vote kernel gave up")
+        score_kernel = "ts::score_kernel<Hkv,G,false,2> (cooperative score + vote)"
+    else:
+        bufs = ops.score(c, bt, qf, wl.k_pool)
+        score_us, score_min = event_time_us(
+            lambda i: ops.score(c, bt, qf, k_pools[i % n_pools], out=bufs), args.steps, args.warmup)
+        score_kernel = "ts::score_kernel<Hkv,G,false,1> (ts_score)"
     sel, sel_len = layer.sel, layer.sel_len
     attn_us, _ = event_time_us(
-        lambda: ops.sparse_decode_attention(c, wl.q, wl.k_pool, wl.v_pool, sel, sel_len),
+        lambda i: ops.sparse_decode_attention(c, wl.q, k_pools[i % n_pools], v_pools[i % n_pools],
+                                              sel, sel_len),
         args.steps, args.warmup)
     score_bytes, attn_bytes = wl.score_bytes(), wl.attn_bytes()
     score_gbs = score_bytes / score_us / 1e3
@@ -135,10 +163,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": wl.name, "batch": B, "seq_lens_max": max(wl.seq_lens),
                    "page_size": c.page_size, "top_k": c.top_k, "n_init": c.n_init,
-                   "n_local": c.n_local},
+                   "n_local": c.n_local, "kv_pool_copies": n_pools},
         "tokens_per_s": round(B / (us_per_layer * 1e-6 * args.layers), 1),
         "tokens_per_s_note": f"selection+attention only, {args.layers} layers per token",
-        "roofline": {"bound": "hbm", "kernel": "ts::score_kernel", "achieved": round(score_gbs, 1),
+        "roofline": {"bound": "hbm", "kernel": score_kernel, "achieved": round(score_gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(score_gbs / HBM_PEAK_GBS, 4),
                      "traffic": None, "bytes_per_launch": score_bytes,
                      "us_per_launch": round(score_us, 2), "us_min": round(score_min, 2)},

@@ -106,6 +106,54 @@ def test_score_vote_topk(dev, shape, page):
         assert torch.equal(sel[b, :S].cpu(), tabs[b][pos.long()])
 
 
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("page", [1, 16])
+def test_fused_score_vote(dev, shape, page):
+    """The cooperative score + vote kernel against the oracle's votes and against the
+    separate kernels' selection, twice in a row on one workspace (counters are
+    accumulated into, so a missed reset shows up on the second pass)."""
+    lens, ks = [3000, 777, 40, 1531], [64, 100, 64, 1]
+    say(f"fused score+vote H={shape['num_heads']} Hkv={shape['num_kv_heads']} page={page} lens={lens}")
+    wl = small(dev, shape, seed=page + shape["num_heads"], lens=lens, ks=ks, page=page, top_k=100)
+    c = wl.cfg
+    assert ops.score_vote_supported(c, len(lens), max(lens))
+    qf = fingerprint(wl, dev)
+    space = ops.SelectionWorkspace(c, len(lens), max(lens), dev)
+    details = []
+    oracle_layer(wl, details)
+    votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool))
+    sel_sep, pos_sep, len_sep = ops.topk_ragged(c, wl.batch, votes_sep)
+    for attempt in range(2):
+        space.reset()
+        votes = ops.score_vote(c, wl.batch, qf, wl.k_pool, space)
+        sel, sel_pos, sel_len = ops.topk_ragged(c, wl.batch, votes, counted=space)
+        torch.cuda.synchronize()
+        assert not space.fault()
+        assert torch.equal(sel_len, len_sep)
+        for b, (L, k) in enumerate(zip(wl.seq_lens, wl.k_list)):
+            S = int(sel_len[b])
+            if not details[b]:
+                assert torch.equal(sel[b, :S], sel_sep[b, :S])
+                continue
+            n = L - c.n_init - c.n_local
+            assert torch.allclose(votes[b, :n].cpu(), details[b]["votes"], rtol=2e-4, atol=1e-9), \
+                f"votes b={b} attempt={attempt}"
+            assert_index_sets_match(sel_pos[b, c.n_init:c.n_init + k].cpu(), details[b]["top_pos"],
+                                    details[b]["votes"], c.n_init, f"fused top-k b={b}")
+            assert torch.equal(sel_pos[b, :c.n_init], pos_sep[b, :c.n_init])
+            assert torch.equal(sel_pos[b, c.n_init + k:S], pos_sep[b, c.n_init + k:S])
+
+
+def test_fused_score_vote_rejects_unsupported(dev):
+    say("fused score+vote: pool_kernel on -> TS_ESHAPE")
+    wl = small(dev, SHAPES[0], seed=3, lens=[2000], ks=[64], pool_kernel=5)
+    assert not ops.score_vote_supported(wl.cfg, 1, 2000)
+    space = ops.SelectionWorkspace(wl.cfg, 1, 2000, dev)
+    space.reset()
+    with pytest.raises(RuntimeError, match="ts_score_vote"):
+        ops.score_vote(wl.cfg, wl.batch, fingerprint(wl, dev), wl.k_pool, space)
+
+
 def test_topk_ties_and_extremes(dev):
     say("topk ties / k=1 / k=n-1")
     shape = SHAPES[0]
@@ -170,13 +218,17 @@ def test_attention_soft_cap(dev):
     assert (out[0].cpu().float() - ref.reshape(-1).float()).abs().max().item() <= 2e-2
 
 
-@pytest.mark.parametrize("shape", SHAPES[:2], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
-@pytest.mark.parametrize("page", [1, 16])
-def test_decode_layer(dev, shape, page):
-    lens, ks = [5000, 100, 2048, 901], [256, 256, 200, 256]
-    say(f"decode_layer H={shape['num_heads']} page={page} lens={lens}")
-    wl = small(dev, shape, seed=21 + page, lens=lens, ks=ks, page=page, top_k=256, n_init=16,
-               n_local=32)
+@pytest.fixture
+def fused_vote(request):
+    """Runs the layer with the cooperative score + vote kernel (True) or with the
+    separate kernels (False); restores the library default afterwards."""
+    previous = ops.set_fused_vote(request.param)
+    yield request.param
+    ops.set_fused_vote(previous)
+
+
+def check_layer(wl, dev, tag):
+    lens = wl.seq_lens
     layer = ops.DecodeLayer(wl.cfg, len(lens), max(lens), dev)
     out, sel, sel_pos, sel_len = layer(wl.q, wl.k_pool, wl.v_pool, wl.batch)
     torch.cuda.synchronize()
@@ -188,10 +240,54 @@ def test_decode_layer(dev, shape, page):
         if details[b]:
             c = wl.cfg
             assert_index_sets_match(sel_pos[b, c.n_init:S - c.n_local].cpu(), details[b]["top_pos"],
-                                    details[b]["votes"], c.n_init, f"layer top-k b={b}")
+                                    details[b]["votes"], c.n_init, f"{tag} top-k b={b}")
         if torch.equal(sel[b, :S].cpu(), ref_sel[b]):
             err = (out[b].cpu().float() - ref_out[b].float()).abs().max().item()
-            assert err <= 2e-2, f"decode_layer out b={b}: {err}"
+            assert err <= 2e-2, f"{tag} out b={b}: {err}"
+    return sel_pos, sel_len
+
+
+@pytest.mark.parametrize("shape", SHAPES[:2], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("page", [1, 16])
+@pytest.mark.parametrize("fused_vote", [True, False], indirect=True, ids=["fused", "separate"])
+def test_decode_layer(dev, shape, page, fused_vote):
+    lens, ks = [5000, 100, 2048, 901], [256, 256, 200, 256]
+    say(f"decode_layer H={shape['num_heads']} page={page} lens={lens} fused={fused_vote}")
+    wl = small(dev, shape, seed=21 + page, lens=lens, ks=ks, page=page, top_k=256, n_init=16,
+               n_local=32)
+    check_layer(wl, dev, "decode_layer")
+
+
+@pytest.mark.parametrize("shape", SHAPES[2:], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("fused_vote", [True], indirect=True, ids=["fused"])
+def test_decode_layer_fused_shapes(dev, shape, fused_vote):
+    lens, ks = [3001, 40, 1500], [128, 128, 100]
+    say(f"decode_layer fused H={shape['num_heads']}kv{shape['num_kv_heads']} lens={lens}")
+    wl = small(dev, shape, seed=77, lens=lens, ks=ks, page=16, top_k=128)
+    check_layer(wl, dev, "decode_layer fused")
+
+
+@pytest.mark.parametrize("fused_vote", [True, False], indirect=True, ids=["fused", "separate"])
+def test_decode_layer_many_chunks(dev, fused_vote):
+    """Long ragged batch: hundreds of workgroups per request meet at the grid-wide
+    rendezvous and the statistics merge walks more than 64 chunks per head."""
+    lens, ks = [70000, 9000, 33000], [1024, 512, 1024]
+    say(f"decode_layer long lens={lens} fused={fused_vote}")
+    wl = small(dev, SHAPES[0], seed=5, lens=lens, ks=ks, page=16, top_k=1024, n_init=128,
+               n_local=512)
+    check_layer(wl, dev, "decode_layer long")
+
+
+@pytest.mark.parametrize("fused_vote", [True], indirect=True, ids=["fused"])
+def test_decode_layer_fused_full_lds(dev, fused_vote):
+    """Four 64K requests: the largest batch whose scores still fit the LDS of the
+    device (512 candidates per workgroup, more than 64 KB of LDS each)."""
+    lens, ks = [65536, 65536, 60000, 65536], [2048, 2048, 2048, 1000]
+    say(f"decode_layer fused, LDS-filling batch lens={lens}")
+    wl = small(dev, SHAPES[0], seed=9, lens=lens, ks=ks, page=1, top_k=2048, n_init=128,
+               n_local=512)
+    assert ops.score_vote_supported(wl.cfg, len(lens), max(lens))
+    check_layer(wl, dev, "decode_layer full LDS")
 
 
 def test_max_pool_votes(dev):

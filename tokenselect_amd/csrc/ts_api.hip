@@ -4,7 +4,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 
-#include "ts_common.h"
+#include "ts_score.h"
+#include "ts_topk.h"
 
 namespace ts {
 
@@ -148,7 +149,8 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
   TS_TRY(validate_batch(cfg, bt));
   TS_REQUIRE(q && q_cos && q_sin && k_pool && v_pool && out && sel && sel_pos && sel_len, TS_EINVAL,
              "ts_decode_layer: NULL tensor argument");
-  TS_REQUIRE(pool_rows >= 1, TS_EINVAL, "pool_rows %lld < 1", (long long)pool_rows);
+  TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
+             (long long)pool_rows);
   LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);
   TS_REQUIRE(sel_stride >= w.max_sel, TS_EWORKSPACE, "sel_stride %lld < n_init+top_k+n_local = %d",
              (long long)sel_stride, w.max_sel);
@@ -166,18 +168,42 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
   float* votes = (float*)(ws + w.votes);
   float* pooled = cfg->pool_kernel > 0 ? (float*)(ws + w.pooled) : nullptr;
 
+  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
+  const int fused_tpb = fused_tokens_per_block(cfg, bt->batch, bt->max_seq_len);
+  uint32_t* topk_words = (uint32_t*)(ws + w.topk_ws);
+  const TopkArgs topk = make_topk_args(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache,
+                                       sel, sel_pos, sel_stride, sel_len, topk_words);
+
   // Fingerprint: every request's single decode row is rotated to n_local
-  // (tr.py:381-388); the mean over one row is the row itself (tr.py:392).
-  TS_TRY(ts_rope_apply(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
-                       stream));
+  // (tr.py:381-388); the mean over one row is the row itself (tr.py:392).  The same
+  // launch clears the selection counters when the fused kernel is going to fill them.
+  ZeroRegion zero, zero_sync;
+  if (fused_tpb > 0) {
+    zero.base = topk_words;
+    zero.stride = (int64_t)topk.ws_stride;
+    zero.words = kTopkCounterWords;
+    zero.count = bt->batch;
+    zero_sync.base = topk_sync_area(topk_words, bt->batch, max_n);
+    zero_sync.stride = kSyncSlotWords;
+    zero_sync.words = 2;
+    zero_sync.count = kSyncSlots + 1;
+  }
+  TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim, zero,
+                     zero_sync, (hipStream_t)stream));
   if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
   float* partials = (float*)(ws + w.partials);
-  TS_TRY(ts_score(cfg, bt, qf, k_pool, pool_rows, hit, scores, w.score_stride, partials,
-                  w.partials_bytes, stream));
-  TS_TRY(ts_vote(cfg, bt, scores, w.score_stride, partials, hit, stats, votes, pooled,
-                 w.score_stride, stream));
-  TS_TRY(ts_topk_ragged(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache, sel, sel_pos,
-                        sel_stride, sel_len, ws + w.topk_ws, w.attn_ws - w.topk_ws, stream));
+  if (fused_tpb > 0) {
+    const size_t topk_bytes = w.attn_ws - w.topk_ws;
+    TS_TRY(ts_score_vote(cfg, bt, qf, k_pool, pool_rows, hit, votes, w.score_stride, partials,
+                         w.partials_bytes, topk_words, topk_bytes, stream));
+    TS_TRY(launch_topk(topk, bt->batch, max_n, /*zero=*/false, /*hist=*/false, (hipStream_t)stream));
+  } else {
+    TS_TRY(ts_score(cfg, bt, qf, k_pool, pool_rows, hit, scores, w.score_stride, partials,
+                    w.partials_bytes, stream));
+    TS_TRY(ts_vote(cfg, bt, scores, w.score_stride, partials, hit, stats, votes, pooled,
+                   w.score_stride, stream));
+    TS_TRY(launch_topk(topk, bt->batch, max_n, /*zero=*/true, /*hist=*/true, (hipStream_t)stream));
+  }
   TS_TRY(ts_sparse_decode_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len,
                                bt->batch, w.max_sel, out, ws + w.attn_ws, w.total - w.attn_ws,
                                stream));

@@ -33,6 +33,19 @@ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // the statistics merge and the workspace query.
 int score_tokens_per_block(int64_t total_candidates, int num_heads);
 
+// Words the rotation kernel clears on the side (two such regions per launch):
+// `count` pieces of `words` 32-bit words, `stride` words apart (all zero: nothing
+// to clear).
+struct ZeroRegion {
+  uint32_t* base = nullptr;
+  int64_t stride = 0;
+  int words = 0;
+  int count = 0;
+};
+int launch_rope(const void* x, void* out, const float* cos_table, const float* sin_table,
+                const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
+                const ZeroRegion& zero, const ZeroRegion& zero2, hipStream_t stream);
+
 constexpr int kHeadDim = 128;
 constexpr float kNegBig = -3.0e38f;  // finite stand-in for -inf in running maxima
 

@@ -13,11 +13,19 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(const uint16_t* __restr
                                                          const float* __restrict__ sin_table,
                                                          const int64_t* __restrict__ position_ids,
                                                          int64_t table_rows, int64_t rows, int heads,
-                                                         int dim) {
+                                                         int dim, ZeroRegion zero, ZeroRegion zero2) {
 #pragma clang fp contract(off)
   const int half = dim >> 1;
   const int64_t pairs = rows * heads * half;
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  // Counters the later kernels of a decode step accumulate into: `count` pieces
+  // of `words` words, `stride` words apart.
+  const int64_t zero_total = (int64_t)zero.count * zero.words;
+  for (int64_t w = gid; w < zero_total; w += (int64_t)gridDim.x * blockDim.x)
+    zero.base[(w / zero.words) * zero.stride + w % zero.words] = 0u;
+  const int64_t zero2_total = (int64_t)zero2.count * zero2.words;
+  for (int64_t w = gid; w < zero2_total; w += (int64_t)gridDim.x * blockDim.x)
+    zero2.base[(w / zero2.words) * zero2.stride + w % zero2.words] = 0u;
   if (gid >= pairs) return;
   const int i = (int)(gid % half);
   const int64_t rh = gid / half;
@@ -36,6 +44,18 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(const uint16_t* __restr
   out[base + i + half] = f32_to_bf16(hi);
 }
 
+int launch_rope(const void* x, void* out, const float* cos_table, const float* sin_table,
+                const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
+                const ZeroRegion& zero, const ZeroRegion& zero2, hipStream_t stream) {
+  const int64_t pairs = rows * heads * (dim / 2);
+  const int64_t blocks = ceil_div(pairs, 256);
+  TS_REQUIRE(blocks <= 0x7fffffff, TS_EINVAL, "ts_rope_apply: too many rows");
+  hipLaunchKernelGGL(rope_apply_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                     (const uint16_t*)x, (uint16_t*)out, cos_table, sin_table, position_ids,
+                     table_rows, rows, heads, dim, zero, zero2);
+  return check_launch("rope_apply_kernel");
+}
+
 }  // namespace ts
 
 using namespace ts;
@@ -50,11 +70,6 @@ extern "C" int ts_rope_apply(const void* x, void* out, const float* cos_table,
              (long long)table_rows);
   TS_REQUIRE(dim >= 2 && dim % 2 == 0, TS_ESHAPE, "ts_rope_apply: dim %d must be even", dim);
   if (rows == 0) return TS_OK;
-  const int64_t pairs = rows * heads * (dim / 2);
-  const int64_t blocks = ceil_div(pairs, 256);
-  TS_REQUIRE(blocks <= 0x7fffffff, TS_EINVAL, "ts_rope_apply: too many rows");
-  hipLaunchKernelGGL(rope_apply_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                     (const uint16_t*)x, (uint16_t*)out, cos_table, sin_table, position_ids,
-                     table_rows, rows, heads, dim);
-  return check_launch("rope_apply_kernel");
+  return launch_rope(x, out, cos_table, sin_table, position_ids, table_rows, rows, heads, dim,
+                     ZeroRegion{}, ZeroRegion{}, (hipStream_t)stream);
 }
