@@ -171,8 +171,10 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
   const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
   const int fused_tpb = fused_tokens_per_block(cfg, bt->batch, bt->max_seq_len);
   uint32_t* topk_words = (uint32_t*)(ws + w.topk_ws);
-  const TopkArgs topk = make_topk_args(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache,
-                                       sel, sel_pos, sel_stride, sel_len, topk_words);
+  TopkArgs topk = make_topk_args(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache, sel,
+                                 sel_pos, sel_stride, sel_len, topk_words);
+  topk.clear = attn_tickets(cfg, bt->batch, w.max_sel, ws + w.attn_ws);
+  topk.clear_per_req = cfg->num_kv_heads;
 
   // Fingerprint: every request's single decode row is rotated to n_local
   // (tr.py:381-388); the mean over one row is the row itself (tr.py:392).  The same
@@ -204,9 +206,8 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
                    w.score_stride, stream));
     TS_TRY(launch_topk(topk, bt->batch, max_n, /*zero=*/true, /*hist=*/true, (hipStream_t)stream));
   }
-  TS_TRY(ts_sparse_decode_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len,
-                               bt->batch, w.max_sel, out, ws + w.attn_ws, w.total - w.attn_ws,
-                               stream));
+  TS_TRY(launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, bt->batch,
+                     w.max_sel, out, ws + w.attn_ws, /*tickets_clear=*/true, (hipStream_t)stream));
   return TS_OK;
 }
 

@@ -1,14 +1,19 @@
 // Decode attention over the selected KV slots: the FlashInfer paged decode the
 // reference calls at tr.py:815-823 (page size 1, in-kernel Llama RoPE).
 //
-// Split-K: grid (splits, Hkv, B).  A workgroup owns a contiguous range of the
-// request's selected list for one KV head and keeps the G = H/Hkv query heads
-// that read it in registers.  Sixteen lanes gather one K row and one V row
-// (256 bytes each, 128-bit loads); sixteen such lane groups per workgroup walk
-// the range with stride 16.  Keys are rotated to their index in the selected
-// list, the query to S-1; softmax is online in fp32.  Partial (max, sum, acc)
-// triples are merged first across the lane groups, then across splits by a
-// second small kernel.
+// Split-K in one launch: grid (splits, Hkv, B).  A workgroup owns a contiguous
+// range of the request's selected list for one KV head and keeps the G = H/Hkv
+// query heads that read it in registers.  Sixteen lanes gather one K row and one
+// V row (256 bytes each, 128-bit loads); the sixteen lane groups of a workgroup
+// walk the range with stride 16, eight tokens per lane group in flight (the slots,
+// then all sixteen rows, are requested before the first is used: the pass is
+// bound by memory latency, not bandwidth).  Keys are rotated to their index in
+// the selected list, the query to S-1; softmax is online in fp32.  Partial
+// (max, sum, acc) triples are merged across the lane groups and waves, written
+// with device-coherent stores, and the workgroup that draws the last ticket of
+// its (request, KV head) merges the splits and writes the bf16 output.
+#include <math.h>
+
 #include "ts_common.h"
 
 namespace ts {
@@ -23,11 +28,12 @@ struct AttnArgs {
   const int32_t* sel_len;
   int num_heads, num_kv_heads;
   int rope_mode;
-  float rope_theta, rope_rcp_scale, sm_scale, logit_cap;
+  float log2_theta, rope_rcp_scale, sm_scale, logit_cap;
   int nsplit, max_sel_len;
-  float* part_acc;  // [B,H,nsplit,128]
-  float* part_ml;   // [B,H,nsplit,2]
-  uint16_t* out;    // [B,H,128] bf16
+  float* part_acc;    // [B,H,nsplit,128]
+  float* part_ml;     // [B,H,nsplit,2]
+  uint32_t* tickets;  // [B,Hkv], zero at launch and again when the kernel ends
+  uint16_t* out;      // [B,H,128] bf16
 };
 
 __device__ __forceinline__ void unpack8(const uint4& w, float (&f)[8]) {
@@ -41,8 +47,31 @@ __device__ __forceinline__ void unpack8(const uint4& w, float (&f)[8]) {
   f[7] = bf16_hi(w.w);
 }
 
+// sin and cos of an angle of up to some 1e5 radians: two-constant reduction by
+// 2 pi (hi + lo parts, each product exact inside the FMA), then the hardware
+// functions on [-pi, pi].
+__device__ __forceinline__ void sincos_reduced(float x, float& sn, float& cs) {
+  const float k = rintf(x * 0.15915494309189535f);
+  float r = fmaf(-k, 6.2831854820251465f, x);
+  r = fmaf(-k, -1.7484555e-07f, r);
+  sn = __sinf(r);
+  cs = __cosf(r);
+}
+
+__device__ __forceinline__ float2 load_coherent2(const float* p) {
+  const uint64_t v =
+      __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return make_float2(__uint_as_float((uint32_t)v), __uint_as_float((uint32_t)(v >> 32)));
+}
+__device__ __forceinline__ void store_coherent2(float* p, float x, float y) {
+  const uint64_t v = (uint64_t)__float_as_uint(x) | ((uint64_t)__float_as_uint(y) << 32);
+  __hip_atomic_store((uint64_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+constexpr int kAttnInFlight = 8;  // tokens per lane group requested together
+
 template <int G>
-__global__ __launch_bounds__(256) void attn_split_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int S = min(max(a.sel_len[b], 0), a.max_sel_len);
   const int chunk = (S + a.nsplit - 1) / a.nsplit;
@@ -55,32 +84,48 @@ __global__ __launch_bounds__(256) void attn_split_kernel(AttnArgs a) {
   const bool upper = l16 >= 8;  // second half of the head dimension
   const int H = a.num_heads;
   const bool rope = a.rope_mode == TS_ROPE_LLAMA;
+  const int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
+  const size_t row_elems = (size_t)a.num_kv_heads * kHeadDim;
 
-  // Frequencies of this lane's 8 rotation pairs (pair index = dim mod 64).
+  // First batch of slots: requested before the rotation set-up below.
+  uint32_t slot[kAttnInFlight];
+  auto load_slots = [&](int j0) {
+#pragma unroll
+    for (int u = 0; u < kAttnInFlight; ++u) {
+      const int j = min(j0 + 16 * u, max(hi - 1, 0));
+      slot[u] = hi > lo ? (uint32_t)sel[j] : 0u;
+    }
+  };
+  load_slots(lo + lg);
+
+  // Frequencies of this lane's 8 rotation pairs (pair index = dim mod 64):
+  // theta^(-2 pair / 128) / scale.
   float freq[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const int pair = (l16 & 7) * 8 + e;
-    freq[e] = a.rope_rcp_scale * powf(a.rope_theta, -2.0f * (float)pair / (float)kHeadDim);
+    freq[e] = a.rope_rcp_scale * exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
   }
 
   // Query rows of the G heads, rotated to position S-1.
   float qv[G][8];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const uint16_t* qrow = a.q + ((size_t)b * H + (size_t)kvh * G + g) * kHeadDim;
-    float mine[8], other[8];
-    unpack8(*(const uint4*)(qrow + l16 * 8), mine);
-    unpack8(*(const uint4*)(qrow + (l16 ^ 8) * 8), other);
+  {
+    float qc[8], qs[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      if (rope) {
-        float sn, cs;
-        sincosf((float)(S - 1) * freq[e], &sn, &cs);
-        qv[g][e] = upper ? mine[e] * cs + other[e] * sn : mine[e] * cs - other[e] * sn;
-      } else {
-        qv[g][e] = mine[e];
-      }
+      qc[e] = 1.f;
+      qs[e] = 0.f;
+      if (rope) sincos_reduced((float)(S - 1) * freq[e], qs[e], qc[e]);
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const uint16_t* qrow = a.q + ((size_t)b * H + (size_t)kvh * G + g) * kHeadDim;
+      float mine[8], other[8];
+      unpack8(*(const uint4*)(qrow + l16 * 8), mine);
+      unpack8(*(const uint4*)(qrow + (l16 ^ 8) * 8), other);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        qv[g][e] = upper ? mine[e] * qc[e] + other[e] * qs[e] : mine[e] * qc[e] - other[e] * qs[e];
     }
   }
 
@@ -88,14 +133,13 @@ __global__ __launch_bounds__(256) void attn_split_kernel(AttnArgs a) {
   float kc[8], ks[8], dc[8], ds[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
+    kc[e] = 1.f;
+    ks[e] = 0.f;
+    dc[e] = 1.f;
+    ds[e] = 0.f;
     if (rope) {
-      sincosf((float)(lo + lg) * freq[e], &ks[e], &kc[e]);
-      sincosf(16.0f * freq[e], &ds[e], &dc[e]);
-    } else {
-      kc[e] = 1.f;
-      ks[e] = 0.f;
-      dc[e] = 1.f;
-      ds[e] = 0.f;
+      sincos_reduced((float)(lo + lg) * freq[e], ks[e], kc[e]);
+      sincos_reduced(16.0f * freq[e], ds[e], dc[e]);
     }
   }
 
@@ -108,47 +152,56 @@ __global__ __launch_bounds__(256) void attn_split_kernel(AttnArgs a) {
     for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
   }
 
-  const int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
-  const size_t row_elems = (size_t)a.num_kv_heads * kHeadDim;
-  for (int j = lo + lg; j < hi; j += 16) {
-    uint32_t slot = (uint32_t)sel[j];
-    slot = slot < a.pool_rows ? slot : a.pool_rows - 1;
-    const size_t at = (size_t)slot * row_elems + (size_t)kvh * kHeadDim + l16 * 8;
-    const uint4 kraw = *(const uint4*)(a.k_pool + at);
-    const uint4 vraw = *(const uint4*)(a.v_pool + at);
-    float kf[8], vf[8];
-    unpack8(kraw, kf);
-    unpack8(vraw, vf);
-    if (rope) {
+  for (int j0 = lo + lg; j0 < hi; j0 += 16 * kAttnInFlight) {
+    uint4 kraw[kAttnInFlight], vraw[kAttnInFlight];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float partner = dpp_move<kRowRor8>(kf[e]);  // dim +-64 of the same token
-        kf[e] = upper ? kf[e] * kc[e] + partner * ks[e] : kf[e] * kc[e] - partner * ks[e];
-        const float c2 = kc[e] * dc[e] - ks[e] * ds[e];
-        ks[e] = ks[e] * dc[e] + kc[e] * ds[e];
-        kc[e] = c2;
-      }
+    for (int u = 0; u < kAttnInFlight; ++u) {
+      const uint32_t sl = slot[u] < a.pool_rows ? slot[u] : a.pool_rows - 1;
+      const size_t at = (size_t)sl * row_elems + (size_t)kvh * kHeadDim + l16 * 8;
+      kraw[u] = *(const uint4*)(a.k_pool + at);
+      vraw[u] = *(const uint4*)(a.v_pool + at);
     }
+    if (j0 + 16 * kAttnInFlight < hi) load_slots(j0 + 16 * kAttnInFlight);
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float p = 0.f;
+    for (int u = 0; u < kAttnInFlight; ++u) {
+      const bool valid = j0 + 16 * u < hi;  // uniform over the 16 lanes of a group
+      float kf[8], vf[8];
+      unpack8(kraw[u], kf);
+      unpack8(vraw[u], vf);
+      if (rope) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) p += qv[g][e] * kf[e];
-      p = row16_sum(p) * a.sm_scale;
-      if (a.logit_cap > 0.f) p = a.logit_cap * tanhf(p / a.logit_cap);
-      const float mn = fmaxf(m[g], p);
-      const float alpha = __expf(m[g] - mn);
-      const float w = __expf(p - mn);
-      l[g] = l[g] * alpha + w;
+        for (int e = 0; e < 8; ++e) {
+          const float partner = dpp_move<kRowRor8>(kf[e]);  // dim +-64 of the same token
+          kf[e] = upper ? kf[e] * kc[e] + partner * ks[e] : kf[e] * kc[e] - partner * ks[e];
+          const float c2 = kc[e] * dc[e] - ks[e] * ds[e];
+          ks[e] = ks[e] * dc[e] + kc[e] * ds[e];
+          kc[e] = c2;
+        }
+      }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * alpha + w * vf[e];
-      m[g] = mn;
+      for (int g = 0; g < G; ++g) {
+        float p = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) p += qv[g][e] * kf[e];
+        p = row16_sum(p) * a.sm_scale;
+        if (a.logit_cap > 0.f) p = a.logit_cap * tanhf(p / a.logit_cap);
+        if (valid) {
+          const float mn = fmaxf(m[g], p);
+          const float alpha = __expf(m[g] - mn);
+          const float w = __expf(p - mn);
+          l[g] = l[g] * alpha + w;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * alpha + w * vf[e];
+          m[g] = mn;
+        }
+      }
     }
   }
 
   // Merge the four lane groups of a wave (rows of 16 lanes), then the four waves.
   __shared__ float sm_acc[4][G][kHeadDim];
   __shared__ float sm_m[4][G], sm_l[4][G];
+  __shared__ uint32_t s_last;
 #pragma unroll
   for (int g = 0; g < G; ++g) {
 #pragma unroll
@@ -171,50 +224,146 @@ __global__ __launch_bounds__(256) void attn_split_kernel(AttnArgs a) {
     }
   }
   __syncthreads();
-  for (int idx = tid; idx < G * kHeadDim; idx += 256) {
-    const int g = idx / kHeadDim, d = idx % kHeadDim;
+  // A thread owns two adjacent dims of one head: one 64-bit coherent store.
+  for (int idx = tid; idx < G * (kHeadDim / 2); idx += 256) {
+    const int g = idx / (kHeadDim / 2), d = (idx % (kHeadDim / 2)) * 2;
     float mm = kNegBig;
 #pragma unroll
     for (int w = 0; w < 4; ++w) mm = fmaxf(mm, sm_m[w][g]);
-    float o = 0.f, ll = 0.f;
+    float o0 = 0.f, o1 = 0.f, ll = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       const float sc = __expf(sm_m[w][g] - mm);
-      o += sm_acc[w][g][d] * sc;
+      o0 += sm_acc[w][g][d] * sc;
+      o1 += sm_acc[w][g][d + 1] * sc;
       ll += sm_l[w][g] * sc;
     }
     const size_t ph = ((size_t)b * H + (size_t)kvh * G + g) * a.nsplit + split;
-    a.part_acc[ph * kHeadDim + d] = o;
-    if (d == 0) {
-      a.part_ml[ph * 2] = mm;
-      a.part_ml[ph * 2 + 1] = ll;
-    }
+    store_coherent2(a.part_acc + ph * kHeadDim + d, o0, o1);
+    if (d == 0) store_coherent2(a.part_ml + ph * 2, mm, ll);
   }
+
+  // Ticket: the stores above are acknowledged before the workgroup is counted.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  uint32_t* ticket = a.tickets + (size_t)b * a.num_kv_heads + kvh;
+  if (tid == 0) {
+    const uint32_t before =
+        __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = before + 1 == (uint32_t)a.nsplit ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!s_last) return;
+
+  // out[b,h,:] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s, rounded to
+  // bf16; splits in index order, 16 of them in flight.
+  for (int idx = tid; idx < G * (kHeadDim / 2); idx += 256) {
+    const int g = idx / (kHeadDim / 2), d = (idx % (kHeadDim / 2)) * 2;
+    const size_t ph = ((size_t)b * H + (size_t)kvh * G + g) * a.nsplit;
+    float mm = kNegBig, ll = 0.f, o0 = 0.f, o1 = 0.f;
+    for (int s0 = 0; s0 < a.nsplit; s0 += 16) {
+      float2 ml[16], ac[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int sp = min(s0 + i, a.nsplit - 1);
+        ml[i] = load_coherent2(a.part_ml + (ph + sp) * 2);
+        ac[i] = load_coherent2(a.part_acc + (ph + sp) * kHeadDim + d);
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        if (s0 + i < a.nsplit) {
+          const float mn = fmaxf(mm, ml[i].x);
+          const float a1 = __expf(mm - mn), a2 = __expf(ml[i].x - mn);
+          ll = ll * a1 + ml[i].y * a2;
+          o0 = o0 * a1 + ac[i].x * a2;
+          o1 = o1 * a1 + ac[i].y * a2;
+          mm = mn;
+        }
+      }
+    }
+    const uint32_t packed = (uint32_t)f32_to_bf16(ll > 0.f ? o0 / ll : 0.f) |
+                            ((uint32_t)f32_to_bf16(ll > 0.f ? o1 / ll : 0.f) << 16);
+    *(uint32_t*)(a.out + ((size_t)b * H + (size_t)kvh * G + g) * kHeadDim + d) = packed;
+  }
+  if (tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// out[b,h,:] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s, rounded to bf16.
-__global__ __launch_bounds__(kHeadDim) void attn_merge_kernel(AttnArgs a) {
-  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
-  const size_t ph = ((size_t)b * a.num_heads + h) * a.nsplit;
-  float mm = kNegBig;
-  for (int s = 0; s < a.nsplit; ++s) mm = fmaxf(mm, a.part_ml[(ph + s) * 2]);
-  float o = 0.f, ll = 0.f;
-  for (int s = 0; s < a.nsplit; ++s) {
-    const float sc = __expf(a.part_ml[(ph + s) * 2] - mm);
-    o += a.part_acc[(ph + s) * kHeadDim + d] * sc;
-    ll += a.part_ml[(ph + s) * 2 + 1] * sc;
-  }
-  a.out[((size_t)b * a.num_heads + h) * kHeadDim + d] = f32_to_bf16(ll > 0.f ? o / ll : 0.f);
+__global__ __launch_bounds__(256) void attn_zero_kernel(uint32_t* tickets, int count) {
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < count; i += gridDim.x * 256) tickets[i] = 0u;
 }
 
 static int attn_splits(int batch, int num_kv_heads, int max_sel_len) {
-  // About two workgroups per CU in total; at least 16 tokens per split.
-  int64_t want = ceil_div(512, (int64_t)batch * num_kv_heads);
-  int64_t cap = ceil_div(max_sel_len, 16);
+  // One batch of loads per lane group (16 groups x 8 tokens = 128 tokens per
+  // workgroup) as long as that keeps the grid near a thousand workgroups.
+  int64_t want = ceil_div(max_sel_len, 16 * kAttnInFlight);
+  const int64_t cap = ceil_div(1024, (int64_t)batch * num_kv_heads);
   if (want > cap) want = cap;
   if (want < 1) want = 1;
-  if (want > 256) want = 256;
   return (int)want;
+}
+
+struct AttnWorkspace {
+  size_t acc, ml, tickets, total;
+};
+static AttnWorkspace attn_workspace(const ts_config* cfg, int batch, int max_sel_len) {
+  const size_t ns = (size_t)attn_splits(batch, cfg->num_kv_heads, max_sel_len);
+  const size_t heads = (size_t)batch * cfg->num_heads;
+  AttnWorkspace w;
+  w.acc = 0;
+  w.ml = w.acc + align_up(heads * ns * kHeadDim * 4, 256);
+  w.tickets = w.ml + align_up(heads * ns * 2 * 4, 256);
+  w.total = w.tickets + align_up((size_t)batch * cfg->num_kv_heads * 4, 256);
+  return w;
+}
+
+uint32_t* attn_tickets(const ts_config* cfg, int batch, int max_sel_len, void* workspace) {
+  return (uint32_t*)((char*)workspace + attn_workspace(cfg, batch, max_sel_len).tickets);
+}
+
+int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const void* v_pool,
+                int64_t pool_rows, const int32_t* sel, int64_t sel_stride, const int32_t* sel_len,
+                int batch, int max_sel_len, void* out, void* workspace, bool tickets_clear,
+                hipStream_t st) {
+  const AttnWorkspace w = attn_workspace(cfg, batch, max_sel_len);
+  AttnArgs a;
+  a.q = (const uint16_t*)q;
+  a.k_pool = (const uint16_t*)k_pool;
+  a.v_pool = (const uint16_t*)v_pool;
+  a.pool_rows = (uint32_t)pool_rows;
+  a.sel = sel;
+  a.sel_stride = sel_stride;
+  a.sel_len = sel_len;
+  a.num_heads = cfg->num_heads;
+  a.num_kv_heads = cfg->num_kv_heads;
+  a.rope_mode = cfg->rope_mode;
+  a.log2_theta = cfg->rope_mode == TS_ROPE_LLAMA ? (float)log2((double)cfg->rope_theta) : 0.f;
+  a.rope_rcp_scale = cfg->rope_mode == TS_ROPE_LLAMA ? 1.0f / cfg->rope_scale : 1.0f;
+  a.sm_scale = cfg->sm_scale;
+  a.logit_cap = cfg->logit_cap;
+  a.nsplit = attn_splits(batch, cfg->num_kv_heads, max_sel_len);
+  a.max_sel_len = max_sel_len;
+  a.part_acc = (float*)((char*)workspace + w.acc);
+  a.part_ml = (float*)((char*)workspace + w.ml);
+  a.tickets = (uint32_t*)((char*)workspace + w.tickets);
+  a.out = (uint16_t*)out;
+
+  if (!tickets_clear) {
+    const int count = batch * cfg->num_kv_heads;
+    hipLaunchKernelGGL(attn_zero_kernel, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, st,
+                       a.tickets, count);
+    TS_TRY(check_launch("attn_zero_kernel"));
+  }
+  const dim3 grid((unsigned)a.nsplit, (unsigned)cfg->num_kv_heads, (unsigned)batch);
+  const int group = cfg->num_heads / cfg->num_kv_heads;
+  switch (group) {
+    case 1: hipLaunchKernelGGL(attn_kernel<1>, grid, dim3(256), 0, st, a); break;
+    case 2: hipLaunchKernelGGL(attn_kernel<2>, grid, dim3(256), 0, st, a); break;
+    case 4: hipLaunchKernelGGL(attn_kernel<4>, grid, dim3(256), 0, st, a); break;
+    case 7: hipLaunchKernelGGL(attn_kernel<7>, grid, dim3(256), 0, st, a); break;
+    case 8: hipLaunchKernelGGL(attn_kernel<8>, grid, dim3(256), 0, st, a); break;
+    default: return fail(TS_ESHAPE, "unsupported head group %d", group);
+  }
+  return check_launch("attn_kernel");
 }
 
 }  // namespace ts
@@ -225,9 +374,7 @@ extern "C" {
 
 size_t ts_attn_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_sel_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_sel_len < 1) return 0;
-  const size_t ns = (size_t)attn_splits(batch, cfg->num_kv_heads, max_sel_len);
-  const size_t heads = (size_t)batch * cfg->num_heads;
-  return align_up(heads * ns * kHeadDim * 4, 256) + align_up(heads * ns * 2 * 4, 256);
+  return attn_workspace(cfg, batch, max_sel_len).total;
 }
 
 int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_pool,
@@ -247,44 +394,8 @@ int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_poo
   const size_t need = ts_attn_workspace_bytes(cfg, batch, max_sel_len);
   TS_REQUIRE(workspace != nullptr && workspace_bytes >= need, TS_EWORKSPACE,
              "ts_sparse_decode_attn: workspace %zu bytes < required %zu", workspace_bytes, need);
-
-  AttnArgs a;
-  a.q = (const uint16_t*)q;
-  a.k_pool = (const uint16_t*)k_pool;
-  a.v_pool = (const uint16_t*)v_pool;
-  a.pool_rows = (uint32_t)pool_rows;
-  a.sel = sel;
-  a.sel_stride = sel_stride;
-  a.sel_len = sel_len;
-  a.num_heads = cfg->num_heads;
-  a.num_kv_heads = cfg->num_kv_heads;
-  a.rope_mode = cfg->rope_mode;
-  a.rope_theta = cfg->rope_theta;
-  a.rope_rcp_scale = cfg->rope_mode == TS_ROPE_LLAMA ? 1.0f / cfg->rope_scale : 1.0f;
-  a.sm_scale = cfg->sm_scale;
-  a.logit_cap = cfg->logit_cap;
-  a.nsplit = attn_splits(batch, cfg->num_kv_heads, max_sel_len);
-  a.max_sel_len = max_sel_len;
-  const size_t heads = (size_t)batch * cfg->num_heads;
-  a.part_acc = (float*)workspace;
-  a.part_ml = (float*)((char*)workspace + align_up(heads * a.nsplit * kHeadDim * 4, 256));
-  a.out = (uint16_t*)out;
-
-  const dim3 grid((unsigned)a.nsplit, (unsigned)cfg->num_kv_heads, (unsigned)batch);
-  const int group = cfg->num_heads / cfg->num_kv_heads;
-  hipStream_t st = (hipStream_t)stream;
-  switch (group) {
-    case 1: hipLaunchKernelGGL(attn_split_kernel<1>, grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL(attn_split_kernel<2>, grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL(attn_split_kernel<4>, grid, dim3(256), 0, st, a); break;
-    case 7: hipLaunchKernelGGL(attn_split_kernel<7>, grid, dim3(256), 0, st, a); break;
-    case 8: hipLaunchKernelGGL(attn_split_kernel<8>, grid, dim3(256), 0, st, a); break;
-    default: return fail(TS_ESHAPE, "unsupported head group %d", group);
-  }
-  TS_TRY(check_launch("attn_split_kernel"));
-  hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)cfg->num_heads, (unsigned)batch),
-                     dim3(kHeadDim), 0, st, a);
-  return check_launch("attn_merge_kernel");
+  return launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, batch, max_sel_len,
+                     out, workspace, /*tickets_clear=*/false, (hipStream_t)stream);
 }
 
 }  // extern "C"

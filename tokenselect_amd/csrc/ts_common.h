@@ -46,6 +46,16 @@ int launch_rope(const void* x, void* out, const float* cos_table, const float* s
                 const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
                 const ZeroRegion& zero, const ZeroRegion& zero2, hipStream_t stream);
 
+// Sparse decode attention (ts_attn.hip).  The kernel counts its workgroups in per
+// (request, KV head) tickets inside the workspace, which must be zero at launch:
+// tickets_clear = false makes the launcher clear them first, true says an earlier
+// kernel of the stream already did (attn_tickets() tells it where they are).
+uint32_t* attn_tickets(const ts_config* cfg, int batch, int max_sel_len, void* workspace);
+int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const void* v_pool,
+                int64_t pool_rows, const int32_t* sel, int64_t sel_stride, const int32_t* sel_len,
+                int batch, int max_sel_len, void* out, void* workspace, bool tickets_clear,
+                hipStream_t stream);
+
 constexpr int kHeadDim = 128;
 constexpr float kNegBig = -3.0e38f;  // finite stand-in for -inf in running maxima
 

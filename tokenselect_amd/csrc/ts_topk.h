@@ -51,6 +51,10 @@ struct TopkArgs {
   size_t ws_stride;   // words per request
   int bitmap_words;   // 32-bit words of the bitmap region
   uint32_t cand_cap;  // entries of the candidate list
+  // Words the last kernel clears for whoever runs next on the stream (the
+  // attention's tickets): clear_per_req words per request, or NULL.
+  uint32_t* clear;
+  int clear_per_req;
 };
 
 __device__ __host__ __forceinline__ uint32_t* topk_ws(uint32_t* ws, size_t stride, int b) {

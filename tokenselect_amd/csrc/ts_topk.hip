@@ -181,6 +181,9 @@ __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs 
   int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
   int32_t* sel_pos = a.sel_pos + (int64_t)b * a.sel_stride;
   const int L = geo.seq_len;
+  if (a.clear)
+    for (int i = tid; i < a.clear_per_req; i += kTopkFinalThreads)
+      a.clear[(size_t)b * a.clear_per_req + i] = 0u;
 
   auto emit = [&](int out_idx, int pos) {
     sel_pos[out_idx] = pos;
@@ -357,6 +360,8 @@ TopkArgs make_topk_args(const ts_config* cfg, const ts_batch* bt, const float* v
   a.bitmap_words = (int)bitmap_words_for(max_n);
   a.cand_cap = (uint32_t)(max_n > 0 ? max_n : 1);
   a.ws_stride = topk_ws_stride_words(max_n);
+  a.clear = nullptr;
+  a.clear_per_req = 0;
   return a;
 }
 
