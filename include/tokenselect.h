@@ -157,35 +157,31 @@ int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
                    int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
                    void* workspace, size_t workspace_bytes, ts_stream_t stream);
 
-/* Score and soft vote in one launch (tr.py:360-361 without the [H, n] score
- * tensor in between): the scores stay in LDS, every workgroup publishes its
- * softmax partials, the grid meets, the statistics are merged, the grid meets
- * again, and each workgroup turns its own scores into votes[b, t] and into the
- * first histogram of the selection inside topk_workspace.  The launch is an
- * ordinary one sized so that all its workgroups are resident together; that
- * holds while nothing else runs on the device beside the caller's stream (a
- * cooperative launch would enforce it, at about 25 us per call).  Same votes as ts_score + ts_vote up to fp32 rounding
- * of the statistics merge.  Usable when ts_score_vote_supported() returns 1:
- * pool_kernel off and batch x candidates small enough (some 260K candidates for
- * 32 heads) for the scores to fit the LDS of the device (TS_ESHAPE otherwise).  topk_workspace must have been
- * cleared by ts_topk_reset() since its last use, and the selection then
- * continues with ts_topk_ragged_counted(), which is ts_topk_ragged() without
- * the clearing and counting passes.  The grid-wide wait is bounded (2 s); if
- * it ever gives up, the fault word of topk_workspace (the second 32-bit word of
- * its last 65 * 4096 bytes) is set to 1 and the votes of that launch are not
- * valid.  No counterpart in the reference, which
- * materialises the scores. */
-int ts_score_vote_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
-int ts_topk_reset(const ts_config* cfg, int32_t batch, int32_t max_seq_len, void* topk_workspace,
-                  size_t topk_workspace_bytes, ts_stream_t stream);
-int ts_score_vote(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
-                  int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
-                  float* partials, size_t partials_bytes, void* topk_workspace,
-                  size_t topk_workspace_bytes, ts_stream_t stream);
-int ts_topk_ragged_counted(const ts_config* cfg, const ts_batch* bt, const float* votes,
-                           int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
-                           int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
-                           void* workspace, size_t workspace_bytes, ts_stream_t stream);
+/* The whole selection in one launch (tr.py:350-373, 424-449 without the [H, n]
+ * score tensor, the [n] vote vector or the sort in between): score, per-head
+ * softmax, vote, exact k-th largest vote, ascending positions, index assembly.
+ * The scores stay in LDS.  The workgroups of the launch meet six times: softmax
+ * partials, merged statistics, three histogram rounds over the 11 + 11 + 10
+ * bits of the vote keys, and the per-workgroup counts that place each
+ * workgroup's selected positions in the output.  Outputs and the hit / cache
+ * arguments are those of ts_topk_ragged (same tie rule: lowest position first);
+ * votes, when not NULL, also receives the [B, vote_stride] fp32 votes.
+ * Usable when ts_select_supported() returns 1: pool_kernel off and batch x
+ * candidates small enough (some 260K candidates for 32 heads) for the scores to
+ * fit the LDS of the device; TS_ESHAPE otherwise, and the caller runs
+ * ts_score + ts_vote + ts_topk_ragged.  The launch is an ordinary one sized so
+ * that all its workgroups are resident together; that holds while nothing else
+ * runs on the device beside the caller's stream (a cooperative launch would
+ * enforce it, at about 25 us per call).  Every grid-wide wait is bounded (2 s);
+ * if one ever gives up, the first 32-bit word of the last 65 * 4096 bytes of
+ * the workspace is set to 1 and the outputs of that launch are not valid.
+ * No counterpart in the reference, which materialises every intermediate. */
+int ts_select_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+size_t ts_select_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+int ts_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+              int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
+              int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
+              int64_t vote_stride, void* workspace, size_t workspace_bytes, ts_stream_t stream);
 
 /* Selection-cache decision (tr.py:394-401, 416-421) for one layer, no host
  * sync: hit[b] = cache_len[b] > 0 && cos(q_cache[b], qf[b]) >= threshold; on a
@@ -221,14 +217,13 @@ int ts_kv_store(const ts_config* cfg, const void* k, const void* v, const int32_
  * vote -> top-k -> assembly -> sparse attention.  q, out: [B,H*D] bf16.
  * cache may be NULL (QUERY_CACHE=False as released, tr.py:918).
  *
- * When the whole batch fits one co-resident grid and pool_kernel is off, score
- * and vote run as one kernel (ts_score_vote) that keeps the scores in LDS and
- * never writes them to memory; otherwise ts_score, ts_vote and ts_topk_ragged run as
- * they do on their own.  Both forms give the same selection.
- * ts_set_fused_vote(0) forces the separate kernels for the calling process
+ * When ts_select_supported() holds, the selection runs as the single ts_select
+ * kernel; otherwise ts_score, ts_vote and ts_topk_ragged run as they do on
+ * their own.  Both forms give the same selection.
+ * ts_set_fused_select(0) forces the separate kernels for the calling process
  * (1 restores the default); it returns the previous setting and has no
  * counterpart in the reference. */
-int ts_set_fused_vote(int enable);
+int ts_set_fused_select(int enable);
 size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
 int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, const float* q_cos,
                     const float* q_sin, const void* k_pool, const void* v_pool,

@@ -108,50 +108,78 @@ def test_score_vote_topk(dev, shape, page):
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
 @pytest.mark.parametrize("page", [1, 16])
-def test_fused_score_vote(dev, shape, page):
-    """The cooperative score + vote kernel against the oracle's votes and against the
-    separate kernels' selection, twice in a row on one workspace (counters are
-    accumulated into, so a missed reset shows up on the second pass)."""
+def test_fused_select(dev, shape, page):
+    """The single-launch selection against the oracle's votes and selection and against
+    the separate kernels, twice in a row on one workspace (its counters are
+    accumulated into, so a missed clearing shows up on the second pass)."""
     lens, ks = [3000, 777, 40, 1531], [64, 100, 64, 1]
-    say(f"fused score+vote H={shape['num_heads']} Hkv={shape['num_kv_heads']} page={page} lens={lens}")
+    say(f"fused select H={shape['num_heads']} Hkv={shape['num_kv_heads']} page={page} lens={lens}")
     wl = small(dev, shape, seed=page + shape["num_heads"], lens=lens, ks=ks, page=page, top_k=100)
     c = wl.cfg
-    assert ops.score_vote_supported(c, len(lens), max(lens))
+    assert ops.select_supported(c, len(lens), max(lens))
     qf = fingerprint(wl, dev)
-    space = ops.SelectionWorkspace(c, len(lens), max(lens), dev)
     details = []
     oracle_layer(wl, details)
     votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool))
     sel_sep, pos_sep, len_sep = ops.topk_ragged(c, wl.batch, votes_sep)
+    space = None
     for attempt in range(2):
-        space.reset()
-        votes = ops.score_vote(c, wl.batch, qf, wl.k_pool, space)
-        sel, sel_pos, sel_len = ops.topk_ragged(c, wl.batch, votes, counted=space)
+        sel, sel_pos, sel_len, votes, space = ops.select(c, wl.batch, qf, wl.k_pool,
+                                                         want_votes=True, workspace=space)
         torch.cuda.synchronize()
-        assert not space.fault()
+        assert not ops.select_fault(c, wl.batch, space)
         assert torch.equal(sel_len, len_sep)
+        tabs = cpu_tabs(wl)
         for b, (L, k) in enumerate(zip(wl.seq_lens, wl.k_list)):
             S = int(sel_len[b])
-            if not details[b]:
+            if not details[b]:  # dense
                 assert torch.equal(sel[b, :S], sel_sep[b, :S])
+                assert torch.equal(sel_pos[b, :S], pos_sep[b, :S])
                 continue
             n = L - c.n_init - c.n_local
             assert torch.allclose(votes[b, :n].cpu(), details[b]["votes"], rtol=2e-4, atol=1e-9), \
                 f"votes b={b} attempt={attempt}"
-            assert_index_sets_match(sel_pos[b, c.n_init:c.n_init + k].cpu(), details[b]["top_pos"],
-                                    details[b]["votes"], c.n_init, f"fused top-k b={b}")
-            assert torch.equal(sel_pos[b, :c.n_init], pos_sep[b, :c.n_init])
-            assert torch.equal(sel_pos[b, c.n_init + k:S], pos_sep[b, c.n_init + k:S])
+            pos = sel_pos[b, :S].cpu()
+            mid = pos[c.n_init:c.n_init + k]
+            assert bool((mid[1:] > mid[:-1]).all()) if k > 1 else True
+            assert_index_sets_match(mid, details[b]["top_pos"], details[b]["votes"], c.n_init,
+                                    f"fused top-k b={b} attempt={attempt}")
+            assert torch.equal(pos[:c.n_init], pos_sep[b, :c.n_init].cpu())
+            assert torch.equal(pos[c.n_init + k:], pos_sep[b, c.n_init + k:S].cpu())
+            assert torch.equal(sel[b, :S].cpu(), tabs[b][pos.long()])
 
 
-def test_fused_score_vote_rejects_unsupported(dev):
-    say("fused score+vote: pool_kernel on -> TS_ESHAPE")
+def test_fused_select_ties(dev):
+    """Duplicated key rows give exactly equal votes: the k-th vote is shared by many
+    candidates and the ones at the lowest positions must win, as in the separate
+    top-k; the cut falls in the middle of a workgroup and between workgroups."""
+    say("fused select: exact ties at the k-th vote")
+    for seed, (L, k) in enumerate([(4000, 300), (4000, 64), (1500, 700)]):
+        wl = small(dev, SHAPES[0], seed=50 + seed, lens=[L], ks=[k], page=1, top_k=k)
+        c = wl.cfg
+        # Every candidate row becomes a copy of one of 7 rows: 7 distinct votes.
+        tab = wl.table[0, :L].long()
+        src = tab[c.n_init + (torch.arange(L, device=dev) % 7)]
+        wl.k_pool[tab] = wl.k_pool[src]
+        qf = fingerprint(wl, dev)
+        votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool))
+        _, pos_sep, len_sep = ops.topk_ragged(c, wl.batch, votes_sep)
+        _, sel_pos, sel_len, votes, space = ops.select(c, wl.batch, qf, wl.k_pool, want_votes=True)
+        torch.cuda.synchronize()
+        assert not ops.select_fault(c, wl.batch, space)
+        n = L - c.n_init - c.n_local
+        assert torch.unique(votes[0, :n]).numel() <= 7
+        assert torch.allclose(votes[0, :n], votes_sep[0, :n], rtol=1e-5, atol=0)
+        assert torch.equal(sel_len, len_sep)
+        assert torch.equal(sel_pos[0, :int(sel_len[0])], pos_sep[0, :int(sel_len[0])])
+
+
+def test_fused_select_rejects_unsupported(dev):
+    say("fused select: pool_kernel on -> TS_ESHAPE")
     wl = small(dev, SHAPES[0], seed=3, lens=[2000], ks=[64], pool_kernel=5)
-    assert not ops.score_vote_supported(wl.cfg, 1, 2000)
-    space = ops.SelectionWorkspace(wl.cfg, 1, 2000, dev)
-    space.reset()
-    with pytest.raises(RuntimeError, match="ts_score_vote"):
-        ops.score_vote(wl.cfg, wl.batch, fingerprint(wl, dev), wl.k_pool, space)
+    assert not ops.select_supported(wl.cfg, 1, 2000)
+    with pytest.raises(RuntimeError, match="ts_select"):
+        ops.select(wl.cfg, wl.batch, fingerprint(wl, dev), wl.k_pool)
 
 
 def test_topk_ties_and_extremes(dev):
@@ -219,12 +247,12 @@ def test_attention_soft_cap(dev):
 
 
 @pytest.fixture
-def fused_vote(request):
+def fused_select(request):
     """Runs the layer with the cooperative score + vote kernel (True) or with the
     separate kernels (False); restores the library default afterwards."""
-    previous = ops.set_fused_vote(request.param)
+    previous = ops.set_fused_select(request.param)
     yield request.param
-    ops.set_fused_vote(previous)
+    ops.set_fused_select(previous)
 
 
 def check_layer(wl, dev, tag):
@@ -249,44 +277,44 @@ def check_layer(wl, dev, tag):
 
 @pytest.mark.parametrize("shape", SHAPES[:2], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
 @pytest.mark.parametrize("page", [1, 16])
-@pytest.mark.parametrize("fused_vote", [True, False], indirect=True, ids=["fused", "separate"])
-def test_decode_layer(dev, shape, page, fused_vote):
+@pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
+def test_decode_layer(dev, shape, page, fused_select):
     lens, ks = [5000, 100, 2048, 901], [256, 256, 200, 256]
-    say(f"decode_layer H={shape['num_heads']} page={page} lens={lens} fused={fused_vote}")
+    say(f"decode_layer H={shape['num_heads']} page={page} lens={lens} fused={fused_select}")
     wl = small(dev, shape, seed=21 + page, lens=lens, ks=ks, page=page, top_k=256, n_init=16,
                n_local=32)
     check_layer(wl, dev, "decode_layer")
 
 
 @pytest.mark.parametrize("shape", SHAPES[2:], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
-@pytest.mark.parametrize("fused_vote", [True], indirect=True, ids=["fused"])
-def test_decode_layer_fused_shapes(dev, shape, fused_vote):
+@pytest.mark.parametrize("fused_select", [True], indirect=True, ids=["fused"])
+def test_decode_layer_fused_shapes(dev, shape, fused_select):
     lens, ks = [3001, 40, 1500], [128, 128, 100]
     say(f"decode_layer fused H={shape['num_heads']}kv{shape['num_kv_heads']} lens={lens}")
     wl = small(dev, shape, seed=77, lens=lens, ks=ks, page=16, top_k=128)
     check_layer(wl, dev, "decode_layer fused")
 
 
-@pytest.mark.parametrize("fused_vote", [True, False], indirect=True, ids=["fused", "separate"])
-def test_decode_layer_many_chunks(dev, fused_vote):
+@pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
+def test_decode_layer_many_chunks(dev, fused_select):
     """Long ragged batch: hundreds of workgroups per request meet at the grid-wide
     rendezvous and the statistics merge walks more than 64 chunks per head."""
     lens, ks = [70000, 9000, 33000], [1024, 512, 1024]
-    say(f"decode_layer long lens={lens} fused={fused_vote}")
+    say(f"decode_layer long lens={lens} fused={fused_select}")
     wl = small(dev, SHAPES[0], seed=5, lens=lens, ks=ks, page=16, top_k=1024, n_init=128,
                n_local=512)
     check_layer(wl, dev, "decode_layer long")
 
 
-@pytest.mark.parametrize("fused_vote", [True], indirect=True, ids=["fused"])
-def test_decode_layer_fused_full_lds(dev, fused_vote):
+@pytest.mark.parametrize("fused_select", [True], indirect=True, ids=["fused"])
+def test_decode_layer_fused_full_lds(dev, fused_select):
     """Four 64K requests: the largest batch whose scores still fit the LDS of the
     device (512 candidates per workgroup, more than 64 KB of LDS each)."""
     lens, ks = [65536, 65536, 60000, 65536], [2048, 2048, 2048, 1000]
     say(f"decode_layer fused, LDS-filling batch lens={lens}")
     wl = small(dev, SHAPES[0], seed=9, lens=lens, ks=ks, page=1, top_k=2048, n_init=128,
                n_local=512)
-    assert ops.score_vote_supported(wl.cfg, len(lens), max(lens))
+    assert ops.select_supported(wl.cfg, len(lens), max(lens))
     check_layer(wl, dev, "decode_layer full LDS")
 
 

@@ -62,19 +62,17 @@ SIGNATURES = {
     "ts_topk_workspace_bytes": (_size, [_CFG, _i32, _i32]),
     "ts_topk_ragged": (_i32, [_CFG, _BT, _ptr, _i64, _ptr, _SC, _ptr, _ptr, _i64, _ptr, _ptr,
                               _size, _ptr]),
-    "ts_topk_ragged_counted": (_i32, [_CFG, _BT, _ptr, _i64, _ptr, _SC, _ptr, _ptr, _i64, _ptr, _ptr,
-                                      _size, _ptr]),
-    "ts_topk_reset": (_i32, [_CFG, _i32, _i32, _ptr, _size, _ptr]),
-    "ts_score_vote_supported": (_i32, [_CFG, _i32, _i32]),
-    "ts_score_vote": (_i32, [_CFG, _BT, _ptr, _ptr, _i64, _ptr, _ptr, _i64, _ptr, _size, _ptr, _size,
-                             _ptr]),
+    "ts_select_supported": (_i32, [_CFG, _i32, _i32]),
+    "ts_select_workspace_bytes": (_size, [_CFG, _i32, _i32]),
+    "ts_select": (_i32, [_CFG, _BT, _ptr, _ptr, _i64, _ptr, _SC, _ptr, _ptr, _i64, _ptr, _ptr, _i64,
+                         _ptr, _size, _ptr]),
     "ts_selcache_step": (_i32, [_CFG, _BT, _ptr, _SC, _ptr, _ptr]),
     "ts_attn_workspace_bytes": (_size, [_CFG, _i32, _i32]),
     "ts_sparse_decode_attn": (_i32, [_CFG, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
                                      _ptr, _ptr, _size, _ptr]),
     "ts_kv_store": (_i32, [_CFG, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
                            _ptr]),
-    "ts_set_fused_vote": (_i32, [_i32]),
+    "ts_set_fused_select": (_i32, [_i32]),
     "ts_decode_layer_workspace_bytes": (_size, [_CFG, _i32, _i32]),
     "ts_decode_layer": (_i32, [_CFG, _BT, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _SC, _ptr, _ptr,
                                _ptr, _i64, _ptr, _ptr, _size, _ptr]),

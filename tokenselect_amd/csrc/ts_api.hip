@@ -104,7 +104,7 @@ int64_t ts_score_stride(int32_t max_seq_len) {
 
 // Workspace of ts_decode_layer, carved in this order (256-byte aligned pieces).
 struct LayerWorkspace {
-  size_t qf, hit, scores, stats, votes, pooled, partials, topk_ws, attn_ws, total;
+  size_t qf, hit, scores, stats, votes, pooled, partials, topk_ws, select_ws, attn_ws, total;
   size_t partials_bytes;
   int64_t score_stride;
   int32_t max_sel;
@@ -130,6 +130,7 @@ static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32
   w.partials_bytes = ts_score_partials_bytes(cfg, batch, max_seq_len);
   w.partials = take(w.partials_bytes);
   w.topk_ws = take(ts_topk_workspace_bytes(cfg, batch, max_seq_len));
+  w.select_ws = take(select_workspace(cfg, batch, max_seq_len).total);
   w.attn_ws = take(ts_attn_workspace_bytes(cfg, batch, w.max_sel));
   w.total = off;
   return w;
@@ -169,42 +170,33 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
   float* pooled = cfg->pool_kernel > 0 ? (float*)(ws + w.pooled) : nullptr;
 
   const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
-  const int fused_tpb = fused_tokens_per_block(cfg, bt->batch, bt->max_seq_len);
-  uint32_t* topk_words = (uint32_t*)(ws + w.topk_ws);
-  TopkArgs topk = make_topk_args(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache, sel,
-                                 sel_pos, sel_stride, sel_len, topk_words);
-  topk.clear = attn_tickets(cfg, bt->batch, w.max_sel, ws + w.attn_ws);
-  topk.clear_per_req = cfg->num_kv_heads;
+  const SelectWorkspace fused = select_workspace(cfg, bt->batch, bt->max_seq_len);
+  uint32_t* tickets = attn_tickets(cfg, bt->batch, w.max_sel, ws + w.attn_ws);
 
   // Fingerprint: every request's single decode row is rotated to n_local
   // (tr.py:381-388); the mean over one row is the row itself (tr.py:392).  The same
-  // launch clears the selection counters when the fused kernel is going to fill them.
-  ZeroRegion zero, zero_sync;
-  if (fused_tpb > 0) {
-    zero.base = topk_words;
-    zero.stride = (int64_t)topk.ws_stride;
-    zero.words = kTopkCounterWords;
-    zero.count = bt->batch;
-    zero_sync.base = topk_sync_area(topk_words, bt->batch, max_n);
-    zero_sync.stride = kSyncSlotWords;
-    zero_sync.words = 2;
-    zero_sync.count = kSyncSlots + 1;
-  }
-  TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim, zero,
-                     zero_sync, (hipStream_t)stream));
+  // launch clears the counters the fused selection is going to add to.
+  ZeroRegion zero_counters, zero_sync;
+  if (fused.tokens_per_block > 0)
+    select_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_counters, &zero_sync);
+  TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
+                     zero_counters, zero_sync, (hipStream_t)stream));
   if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
-  float* partials = (float*)(ws + w.partials);
-  if (fused_tpb > 0) {
-    const size_t topk_bytes = w.attn_ws - w.topk_ws;
-    TS_TRY(ts_score_vote(cfg, bt, qf, k_pool, pool_rows, hit, votes, w.score_stride, partials,
-                         w.partials_bytes, topk_words, topk_bytes, stream));
-    TS_TRY(launch_topk(topk, bt->batch, max_n, /*zero=*/false, /*hist=*/false, (hipStream_t)stream));
+  if (fused.tokens_per_block > 0) {
+    TS_TRY(launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,
+                         nullptr, 0, ws + w.select_ws, tickets, cfg->num_kv_heads,
+                         (hipStream_t)stream));
   } else {
+    float* partials = (float*)(ws + w.partials);
     TS_TRY(ts_score(cfg, bt, qf, k_pool, pool_rows, hit, scores, w.score_stride, partials,
                     w.partials_bytes, stream));
     TS_TRY(ts_vote(cfg, bt, scores, w.score_stride, partials, hit, stats, votes, pooled,
                    w.score_stride, stream));
-    TS_TRY(launch_topk(topk, bt->batch, max_n, /*zero=*/true, /*hist=*/true, (hipStream_t)stream));
+    TopkArgs topk = make_topk_args(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache, sel,
+                                   sel_pos, sel_stride, sel_len, (uint32_t*)(ws + w.topk_ws));
+    topk.clear = tickets;
+    topk.clear_per_req = cfg->num_kv_heads;
+    TS_TRY(launch_topk(topk, bt->batch, max_n, (hipStream_t)stream));
   }
   TS_TRY(launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, bt->batch,
                      w.max_sel, out, ws + w.attn_ws, /*tickets_clear=*/true, (hipStream_t)stream));

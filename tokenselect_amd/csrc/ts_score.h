@@ -1,8 +1,9 @@
-// Arguments of the scoring kernels, shared between the scoring entry points and
-// the per-layer driver (which launches the fused score + vote form).
+// Arguments of the scoring kernels and the workspace of the fused selection, shared
+// between the scoring entry points and the per-layer driver.
 #pragma once
 
-#include "ts_common.h"
+#include "ts_grid.h"
+#include "ts_topk.h"
 
 namespace ts {
 
@@ -14,7 +15,7 @@ struct ScoreArgs {
   const int32_t* table;
   int64_t table_stride;
   const int32_t* k_per_req;
-  const int32_t* skip;
+  const int32_t* skip;  // per request: 1 = selection-cache hit, nothing to score
   int n_init, n_local, top_k, page_size, page_shift, max_seq_len;
   int64_t direct_n;  // >= 0: paged_matmul mode, candidates are table[0..direct_n)
   void* scores;
@@ -24,18 +25,53 @@ struct ScoreArgs {
   int tokens_per_block;
   int num_heads;
   int head_map;
-  // Fused score + vote only.
-  uint32_t* sync;  // [0] arrival counter (zero at launch), [1] set when a wait gave up
-  float* stats;  // [B,H,2] merged (max, sum exp), by head
-  float* votes;
+  // Fused selection only.
+  uint32_t* sync;         // rendezvous area (ts_grid.h), live words zero at launch
+  float* stats;           // [B,H,2] merged (max, sum exp), by head
+  float* votes;           // [B,vote_stride] copy of the votes, or NULL
   int64_t vote_stride;
-  uint32_t* topk_ws;  // per-request selection counters, zero at launch
-  size_t topk_ws_stride;
-  uint64_t spin_ticks;  // bound of the grid-wide wait, in 100 MHz ticks
+  uint32_t* counters;     // [B][kSelCounterWords] zero at launch
+  uint2* block_counts;    // [B][gridDim.x] (selected for sure, ties at the k-th key)
+  int32_t* sel;           // outputs of the selection, as for ts_topk_ragged
+  int32_t* sel_pos;
+  int64_t sel_stride;
+  int32_t* sel_len;
+  int32_t* topk_cache;    // selection cache to refresh on a miss, or NULL
+  int32_t* cache_len;
+  uint32_t* clear;        // words to clear for the next kernel of the stream, or NULL
+  int clear_per_req;
+  uint64_t spin_ticks;    // bound of a grid-wide wait, in 100 MHz ticks
 };
 
-// Tokens per workgroup of the fused form for this shape, or 0 when the batch does
-// not fit one co-resident grid (the caller then runs the separate kernels).
-int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len);
+// Selection counters of one request, in 32-bit words.  The first histogram is kept
+// in kSelHistCopies copies (workgroup x adds to copy x % copies): the votes of a
+// request fall into a few dozen adjacent bins, i.e. one or two cache lines, and
+// hundreds of workgroups adding to the same line serialise in memory.
+constexpr int kSelHistCopies = 8;
+constexpr int kSelHist0 = 0;                           // 8 x 2048, top 11 key bits
+constexpr int kSelHist1 = kSelHistCopies * kTopkBins;  // 2048, next 11 bits inside bin t0
+constexpr int kSelHist2 = kSelHist1 + kTopkBins;       // 1024, last 10 bits inside (t0, t1)
+constexpr int kSelMaxBin = kSelHist2 + 1024;           // highest occupied bin of hist0
+constexpr int kSelCounterWords = kSelMaxBin + 64;
+
+// Workspace of ts_select, carved in this order (256-byte aligned pieces).
+struct SelectWorkspace {
+  size_t partials, stats, counters, block_counts, sync, total;
+  int tokens_per_block;  // 0: the shape does not fit the fused kernel
+  int blocks_per_req;
+};
+SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len);
+
+// Regions the kernel before ts_select on the stream has to clear (counters and
+// rendezvous words), in the form the rotation kernel takes them.
+void select_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* counters,
+                         ZeroRegion* sync);
+
+// Launch without the clearing pass: the regions above are known to be zero.
+int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+                  int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
+                  int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
+                  int64_t vote_stride, void* workspace, uint32_t* clear, int clear_per_req,
+                  hipStream_t stream);
 
 }  // namespace ts

@@ -70,67 +70,16 @@ constexpr int kQuadSwap2 = 0x4E;  // quad_perm [2,3,0,1]
 //     contiguous burst: trickling 64-byte pieces into 32 separate head rows while
 //     the keys stream in costs a quarter of the read bandwidth (DRAM read/write
 //     turnarounds).
-//   kScoreFused (score + vote in one launch whose workgroups are all resident at
-//     once and meet twice): the scores never leave LDS.  Every workgroup publishes
-//     its per-head (max, sum exp); after the first rendezvous the (request, head)
-//     pairs are dealt out over the grid and merged; after the second every
-//     workgroup turns its own scores into votes (tr.py:361) and into the first
-//     histogram of the selection.
+//   kScoreFused (the whole selection in one launch whose workgroups are all
+//     resident at once and meet six times): the scores never leave LDS.  Every
+//     workgroup publishes its per-head (max, sum exp); the (request, head) pairs
+//     are dealt out over the grid and merged; every workgroup turns its own scores
+//     into votes (tr.py:361); three histogram rounds (11 + 11 + 10 key bits) find
+//     the k-th largest vote exactly; the workgroups exchange their counts and
+//     each writes its selected positions, in ascending order, where they belong
+//     (tr.py:371-373, 433-449).
 constexpr int kScoreDirect = 0, kScoreTiled = 1, kScoreFused = 2;
 constexpr int kMaxHeads = 128;
-
-// Data that workgroups of one launch hand to each other goes through
-// device-coherent accesses (relaxed agent-scope atomics): the L2 of an XCD is not
-// coherent with the other seven, and the fences that would make ordinary accesses
-// visible write back and invalidate a whole L2 per workgroup, which costs several
-// times the streaming pass itself.
-__device__ __forceinline__ float2 load_coherent(const float2* p) {
-  const uint64_t v =
-      __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  return make_float2(__uint_as_float((uint32_t)v), __uint_as_float((uint32_t)(v >> 32)));
-}
-__device__ __forceinline__ void store_coherent(float2* p, float m, float l) {
-  const uint64_t v = (uint64_t)__float_as_uint(m) | ((uint64_t)__float_as_uint(l) << 32);
-  __hip_atomic_store((uint64_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Grid-wide rendezvous of a fully resident grid: every workgroup arrives once per
-// round (1, 2, ...) and those that need the others' data wait for the round to
-// complete.  Each thread first waits for its own coherent stores to be
-// acknowledged; thread 0 then counts the workgroup in.  The workgroup that
-// completes the count raises the round number in every replica slot, and the
-// waiting ones poll the replica of their own index: hundreds of early workgroups
-// polling one word would saturate the memory channel it lives in, which the
-// workgroups still streaming need for 1/128 of their keys.  The wait is bounded:
-// if the round does not complete within `ticks` of the 100 MHz clock the fault
-// word is set and the workgroup carries on, so the kernel always drains.
-__device__ __forceinline__ void grid_arrive(uint32_t* sync, bool wait, uint32_t round,
-                                            uint64_t ticks) {
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const uint32_t workgroups = gridDim.x * gridDim.y;
-    const uint32_t index = blockIdx.y * gridDim.x + blockIdx.x;
-    const uint32_t before =
-        __hip_atomic_fetch_add(&sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (before + 1 == round * workgroups) {
-      for (int r = 0; r < kSyncSlots; ++r)
-        __hip_atomic_store(&sync[(size_t)(r + 1) * kSyncSlotWords], round, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-    } else if (wait) {
-      const uint32_t* flag = &sync[(size_t)(index % kSyncSlots + 1) * kSyncSlotWords];
-      const uint64_t t0 = wall_clock64();
-      while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < round) {
-        if (wall_clock64() - t0 > ticks) {
-          __hip_atomic_store(&sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          break;
-        }
-        __builtin_amdgcn_s_sleep(16);
-      }
-    }
-  }
-  __syncthreads();
-}
 
 // Between the two rendezvous of the fused kernel: the (request, head) pairs are
 // dealt out over all wavefronts of the grid; a wavefront merges the per-workgroup
@@ -166,6 +115,83 @@ __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, int lane
   }
 }
 
+constexpr uint32_t kSelectRounds = 6;  // rendezvous of the fused kernel
+
+// The parts of the output that need no votes, written while the keys stream: a
+// dense request gets all its positions and a selection-cache hit its cached ones
+// (both spread over the request's workgroups); workgroup 0 of a request writes the
+// length, the sink and the local window, and clears the words the next kernel of
+// the stream wants cleared.
+__device__ __forceinline__ void fixed_segments(const ScoreArgs& a, int b) {
+  const ReqGeom geo =
+      request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  const int32_t* tab = a.table + (int64_t)b * a.table_stride;
+  int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
+  int32_t* sel_pos = a.sel_pos + (int64_t)b * a.sel_stride;
+  const int L = geo.seq_len;
+  const int first = blockIdx.x * 256 + threadIdx.x, step = gridDim.x * 256;
+  auto emit = [&](int out_idx, int pos) {
+    sel_pos[out_idx] = pos;
+    sel[out_idx] = (int32_t)lookup_slot(tab, pos, a.page_size, a.page_shift, a.pool_rows);
+  };
+  if (blockIdx.x == 0 && a.clear)
+    for (int i = threadIdx.x; i < a.clear_per_req; i += 256)
+      a.clear[(size_t)b * a.clear_per_req + i] = 0u;
+  if (geo.dense) {  // tr.py:377-378, 741-744: attend over every token
+    for (int i = first; i < L; i += step) emit(i, i);
+    if (first == 0) a.sel_len[b] = L;
+    return;
+  }
+  const bool is_hit = a.skip && a.skip[b];
+  const int k = is_hit ? min(a.cache_len[b], a.top_k) : geo.k;
+  if (is_hit) {  // tr.py:419: reuse the cached positions
+    const int32_t* cached = a.topk_cache + (int64_t)b * a.top_k;
+    for (int i = first; i < k; i += step) emit(a.n_init + i, cached[i]);
+  }
+  if (blockIdx.x != 0) return;
+  if (threadIdx.x == 0) {
+    a.sel_len[b] = a.n_init + k + a.n_local;
+    if (!is_hit && a.cache_len) a.cache_len[b] = k;
+  }
+  for (int i = threadIdx.x; i < a.n_init; i += 256) emit(i, i);
+  for (int i = threadIdx.x; i < a.n_local; i += 256) emit(a.n_init + k + i, L - a.n_local + i);
+}
+
+// 256 threads, thread 0 holding the highest bin: finds the thread at which the
+// running count (from thread 0 on) reaches `need`.  Returns that thread's index
+// (or -1 if the total stays below `need`), the count before it, and the total.
+// `scratch` is LDS of 8 words.
+__device__ __forceinline__ int block_threshold_scan(uint32_t mine, uint32_t need, uint32_t* scratch,
+                                                    uint32_t& before_out, uint32_t& total_out) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  uint32_t incl = mine;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63) scratch[wave] = incl;
+  if (tid == 0) scratch[4] = 0xffffffffu;
+  __syncthreads();
+  uint32_t wave_base = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    if (w < wave) wave_base += scratch[w];
+    total += scratch[w];
+  }
+  const uint32_t before = wave_base + incl - mine;
+  if (before < need && need <= before + mine) {
+    scratch[4] = (uint32_t)tid;
+    scratch[5] = before;
+  }
+  __syncthreads();
+  const uint32_t who = scratch[4];
+  before_out = scratch[5];
+  total_out = total;
+  __syncthreads();
+  return who == 0xffffffffu ? -1 : (int)who;
+}
+
 template <int HKV, int G, bool OUT_BF16, int MODE>
 __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a) {
   extern __shared__ float stage[];  // tiled / fused: [tiles of the workgroup][tile_stride]
@@ -189,11 +215,13 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     first_pos = a.n_init;
   }
   const int block_lo = blockIdx.x * a.tokens_per_block;
+  if constexpr (MODE == kScoreFused) fixed_segments(a, b);
   if (block_lo >= n) {
     if constexpr (MODE == kScoreFused) {  // no tokens here: only help with the statistics
-      grid_arrive(a.sync, true, 1, a.spin_ticks);
+      grid_arrive(a.sync, 1, true, a.spin_ticks);
       merge_request_stats(a, threadIdx.x & 63, threadIdx.x >> 6);
-      grid_arrive(a.sync, false, 2, a.spin_ticks);
+      for (uint32_t round = 2; round <= kSelectRounds; ++round)
+        grid_arrive(a.sync, round, false, a.spin_ticks);
     }
     return;
   }
@@ -420,11 +448,14 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     __shared__ float s_max[kMaxHeads];
     __shared__ float s_rz[kMaxHeads];
     __shared__ uint32_t lh[kTopkBins];
-    for (int i = threadIdx.x; i < kTopkBins; i += 256) lh[i] = 0u;
-    grid_arrive(a.sync, true, 1, a.spin_ticks);
+    __shared__ uint32_t scratch[16];
+    const int tid = threadIdx.x;
+    for (int i = tid; i < kTopkBins; i += 256) lh[i] = 0u;
+    if (tid < 16) scratch[tid] = 0u;
+    grid_arrive(a.sync, 1, true, a.spin_ticks);
     merge_request_stats(a, lane, wave);
-    grid_arrive(a.sync, true, 2, a.spin_ticks);
-    for (int slot = threadIdx.x; slot < H; slot += 256) {
+    grid_arrive(a.sync, 2, true, a.spin_ticks);
+    for (int slot = tid; slot < H; slot += 256) {
       const int h = head_of<HKV, G>(slot / G, slot % G, a.head_map);
       const float2 st = load_coherent((const float2*)a.stats + (size_t)b * H + h);
       s_max[slot] = st.x;
@@ -433,18 +464,227 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     __syncthreads();
 
     // Votes of this workgroup's tokens: fp32 sum over the head slots in slot order.
+    // The vote replaces the first score of its token in LDS (only the thread that
+    // owns a token reads its column).
+    const ReqGeom geo =
+        request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+    const uint32_t k = (uint32_t)geo.k;
     const int count = min(a.tokens_per_block, n - block_lo);
-    for (int i = threadIdx.x; i < count; i += 256) {
-      const float* sc = stage + (i >> 4) * tile_stride + (i & 15);
+    uint32_t* ctr = a.counters + (size_t)b * kSelCounterWords;
+    auto column = [&](int i) -> float* { return stage + (i >> 4) * tile_stride + (i & 15); };
+    auto key_of = [&](int i) -> uint32_t { return vote_key(*column(i)); };
+    for (int i = tid; i < count; i += 256) {
+      float* sc = column(i);
       float c = 0.f;
-      for (int slot = 0; slot < H; ++slot) c += __expf(sc[slot * 16] - s_max[slot]) * s_rz[slot];
-      a.votes[(size_t)b * a.vote_stride + block_lo + i] = c;
-      atomicAdd(&lh[key_bin0(vote_key(c))], 1u);
+#pragma unroll
+      for (int s0 = 0; s0 < HKV * G; s0 += 8) {  // H = HKV * G head slots, 8 LDS reads in flight
+        float x[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] = s0 + j < HKV * G ? sc[(s0 + j) * 16] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (s0 + j < HKV * G) c += __expf(x[j] - s_max[s0 + j]) * s_rz[s0 + j];
+      }
+      if (a.votes) a.votes[(size_t)b * a.vote_stride + block_lo + i] = c;
+      sc[0] = c;
+    }
+    // Local histogram.  The votes of a wavefront fall into a narrow range of bins, so
+    // the lanes are counted bin by bin with ballots over the 64 bins below the
+    // wavefront's highest one, lane d collecting the count of bin (highest - d);
+    // one LDS atomic per occupied bin follows.  (Atomics of one LDS address are
+    // performed a lane at a time, and a loop over the distinct bins with a shuffle
+    // per bin is no faster.)  Lanes further below add their vote on their own.
+    for (int base = 0; base < count; base += 256) {
+      const bool have = base + tid < count;
+      const uint32_t bin = have ? key_bin0(key_of(base + tid)) : 0u;
+      uint32_t top = bin;
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, off));
+      uint32_t mine = 0;
+#pragma unroll 16
+      for (int d = 0; d < 64; ++d) {
+        const uint64_t same = __ballot(have && bin + d == top);
+        if (lane == d) mine = (uint32_t)__popcll(same);
+      }
+      if (mine) atomicAdd(&lh[top - lane], mine);
+      if (have && bin + 63 < top) atomicAdd(&lh[bin], 1u);
+      if (lane == 0) atomicMax(&scratch[8], top);
     }
     __syncthreads();
-    uint32_t* hist0 = hist0_copy(topk_ws(a.topk_ws, a.topk_ws_stride, b), blockIdx.x);
-    for (int i = threadIdx.x; i < kTopkBins; i += 256)
-      if (lh[i]) atomicAdd(&hist0[i], lh[i]);
+
+    // Round 3: top 11 key bits.  The workgroups add their local histograms to one
+    // of the copies and note the highest occupied bin; afterwards each searches
+    // downwards from that bin, 256 bins at a time (one is enough unless the votes
+    // span more than 64 binades).
+    uint32_t* hist0 = ctr + kSelHist0 + (blockIdx.x % kSelHistCopies) * kTopkBins;
+    {
+      uint32_t done = 0;  // old values: waited for once, after all are on their way
+#pragma unroll
+      for (int j = 0; j < kTopkBins / 256; ++j) {
+        const int i = tid + 256 * j;
+        if (lh[i]) done += fetch_add_coherent(&hist0[i], lh[i]);
+      }
+      if (tid == 0) done += fetch_max_coherent(&ctr[kSelMaxBin], scratch[8]);
+      await(done);
+    }
+    grid_arrive(a.sync, 3, true, a.spin_ticks);
+    uint32_t t0 = 0, above0 = 0;
+    for (int top = (int)load_coherent(&ctr[kSelMaxBin]); top >= 0; top -= 256) {
+      const int bin = top - tid;
+      uint32_t part[kSelHistCopies];
+#pragma unroll
+      for (int c = 0; c < kSelHistCopies; ++c)
+        part[c] = bin >= 0 ? load_coherent(&ctr[kSelHist0 + c * kTopkBins + bin]) : 0u;
+      uint32_t mine = 0;
+#pragma unroll
+      for (int c = 0; c < kSelHistCopies; ++c) mine += part[c];
+      uint32_t before, total;
+      const int who = block_threshold_scan(mine, k - above0, scratch, before, total);
+      if (who >= 0) {
+        t0 = (uint32_t)(top - who);
+        above0 += before;
+        break;
+      }
+      above0 += total;
+    }
+
+    // Round 4: next 11 bits of the candidates inside bin t0.
+    {
+      uint32_t done = 0;
+      for (int i = tid; i < count; i += 256) {
+        const uint32_t key = key_of(i);
+        if (key_bin0(key) == t0) done += fetch_add_coherent(&ctr[kSelHist1 + key_bin1(key)], 1u);
+      }
+      await(done);
+    }
+    grid_arrive(a.sync, 4, true, a.spin_ticks);
+    {
+      uint32_t h[kTopkBins / 256];
+#pragma unroll
+      for (int j = 0; j < kTopkBins / 256; ++j) h[j] = load_coherent(&ctr[kSelHist1 + tid + 256 * j]);
+#pragma unroll
+      for (int j = 0; j < kTopkBins / 256; ++j) lh[tid + 256 * j] = h[j];
+    }
+    __syncthreads();
+    uint32_t t1, above1;
+    find_threshold_bin<kTopkBins>(lh, k - above0, scratch, t1, above1);
+    const uint32_t need2 = k - above0 - above1;
+
+    // Round 5: last 10 bits of the candidates inside (t0, t1).
+    {
+      uint32_t done = 0;
+      for (int i = tid; i < count; i += 256) {
+        const uint32_t key = key_of(i);
+        if (key_bin0(key) == t0 && key_bin1(key) == t1)
+          done += fetch_add_coherent(&ctr[kSelHist2 + key_bin2(key)], 1u);
+      }
+      await(done);
+    }
+    grid_arrive(a.sync, 5, true, a.spin_ticks);
+    {
+      uint32_t h[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) h[j] = load_coherent(&ctr[kSelHist2 + tid + 256 * j]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) lh[tid + 256 * j] = h[j];
+    }
+    __syncthreads();
+    uint32_t t2, above2;
+    find_threshold_bin<1024>(lh, need2, scratch, t2, above2);
+    const uint32_t need_eq = need2 - above2;  // ties at the k-th key still to take
+    const uint32_t kth = (t0 << 21) | (t1 << 10) | t2;
+
+    // Round 6: every workgroup publishes how many of its tokens lie above the k-th
+    // key and how many tie with it; ties are taken lowest position first, so the
+    // counts of the workgroups before this one fix where its output starts and
+    // how many of its ties still fit.
+    if (tid < 4) scratch[8 + tid] = 0u;
+    __syncthreads();
+    {
+      uint32_t sure = 0, tie = 0;
+      for (int i = tid; i < count; i += 256) {
+        const uint32_t key = key_of(i);
+        sure += key > kth ? 1u : 0u;
+        tie += key == kth ? 1u : 0u;
+      }
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) {
+        sure += __shfl_xor(sure, off);
+        tie += __shfl_xor(tie, off);
+      }
+      if (lane == 0) {
+        atomicAdd(&scratch[8], sure);
+        atomicAdd(&scratch[9], tie);
+      }
+    }
+    __syncthreads();
+    uint2* counts = a.block_counts + (size_t)b * gridDim.x;
+    if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], scratch[9]);
+    grid_arrive(a.sync, 6, true, a.spin_ticks);
+    {
+      uint32_t sure = 0, tie = 0;
+      for (int j = tid; j < (int)blockIdx.x; j += 256) {
+        const uint2 v = load_coherent(&counts[j]);
+        sure += v.x;
+        tie += v.y;
+      }
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) {
+        sure += __shfl_xor(sure, off);
+        tie += __shfl_xor(tie, off);
+      }
+      if (lane == 0) {
+        atomicAdd(&scratch[10], sure);
+        atomicAdd(&scratch[11], tie);
+      }
+    }
+    __syncthreads();
+    uint32_t tie_run = scratch[11];                          // ties at lower positions
+    uint32_t out_run = scratch[10] + min(tie_run, need_eq);  // selected at lower positions
+    __syncthreads();
+
+    // Emission in position order.
+    const int32_t* tab_b = a.table + (int64_t)b * a.table_stride;
+    int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
+    int32_t* sel_pos = a.sel_pos + (int64_t)b * a.sel_stride;
+    int32_t* cache_out = a.topk_cache ? a.topk_cache + (int64_t)b * a.top_k : nullptr;
+    const uint64_t below = (1ull << lane) - 1ull;
+    for (int base = 0; base < count; base += 256) {
+      const int i = base + tid;
+      const uint32_t key = i < count ? key_of(i) : 0u;
+      const bool tie = i < count && key == kth;
+      const uint64_t tie_mask = __ballot(tie);
+      if (lane == 0) scratch[wave] = (uint32_t)__popcll(tie_mask);
+      __syncthreads();
+      uint32_t tie_rank = tie_run + (uint32_t)__popcll(tie_mask & below);
+      uint32_t tie_total = 0;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        if (w < wave) tie_rank += scratch[w];
+        tie_total += scratch[w];
+      }
+      const bool chosen = i < count && (key > kth || (tie && tie_rank < need_eq));
+      const uint64_t chosen_mask = __ballot(chosen);
+      if (lane == 0) scratch[4 + wave] = (uint32_t)__popcll(chosen_mask);
+      __syncthreads();
+      uint32_t rank = out_run + (uint32_t)__popcll(chosen_mask & below);
+      uint32_t chosen_total = 0;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        if (w < wave) rank += scratch[4 + w];
+        chosen_total += scratch[4 + w];
+      }
+      if (chosen && rank < k) {
+        const int pos = a.n_init + block_lo + i;
+        sel_pos[a.n_init + rank] = pos;
+        sel[a.n_init + rank] =
+            (int32_t)lookup_slot(tab_b, pos, a.page_size, a.page_shift, a.pool_rows);
+        if (cache_out) cache_out[rank] = pos;
+      }
+      tie_run += tie_total;
+      out_run += chosen_total;
+      __syncthreads();
+    }
   }
 }
 
@@ -491,15 +731,15 @@ static size_t fused_lds_bytes(int tokens_per_block, int num_heads) {
 // workgroups fit the 160 KB of a CU.
 constexpr size_t kFusedStageBytes = 68 * 1024;
 
-static std::atomic<int> g_fused_vote{[] {
-  const char* e = getenv("TS_FUSED_VOTE");  // "0" starts with the separate kernels
+static std::atomic<int> g_fused_select{[] {
+  const char* e = getenv("TS_FUSED_SELECT");  // "0" starts with the separate kernels
   return (e && e[0] == '0') ? 0 : 1;
 }()};
 
-int set_fused_vote(int enable) { return g_fused_vote.exchange(enable ? 1 : 0); }
+int set_fused_select(int enable) { return g_fused_select.exchange(enable ? 1 : 0); }
 
 int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len) {
-  if (!g_fused_vote.load() || cfg->pool_kernel > 0 || cfg->num_heads > kMaxHeads) return 0;
+  if (!g_fused_select.load() || cfg->pool_kernel > 0 || cfg->num_heads > kMaxHeads) return 0;
   const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
   if (max_n <= 0) return 0;
   const int group = cfg->num_heads / cfg->num_kv_heads;
@@ -534,14 +774,51 @@ int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len) {
 
   int tpb = score_tokens_per_block((int64_t)batch * max_seq_len, cfg->num_heads);
   while ((int64_t)ceil_div(max_n, tpb) * batch > capacity) tpb += 64;
-  if (fused_lds_bytes(tpb, cfg->num_heads) > kFusedStageBytes) return 0;
+  if (fused_lds_bytes(tpb, cfg->num_heads) > kFusedStageBytes)
+    return 0;
   return tpb;
 }
 
-// Bytes of the per-workgroup partials proper; the merged statistics of the fused
-// kernel follow them.
-static size_t partials_region_bytes(const ts_config* cfg, int batch, size_t nchunks) {
-  return align_up((size_t)batch * cfg->num_heads * nchunks * 2 * sizeof(float), 256);
+SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len) {
+  SelectWorkspace w{};
+  w.tokens_per_block = fused_tokens_per_block(cfg, batch, max_seq_len);
+  if (w.tokens_per_block <= 0) return w;
+  const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
+  w.blocks_per_req = (int)ceil_div(max_n, w.tokens_per_block);
+  const size_t B = (size_t)batch, H = (size_t)cfg->num_heads;
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    const size_t at = off;
+    off += align_up(bytes, 256);
+    return at;
+  };
+  w.partials = take(B * H * (size_t)ceil_div(max_seq_len, w.tokens_per_block) * 2 * sizeof(float));
+  w.stats = take(B * H * 2 * sizeof(float));
+  w.counters = take(B * kSelCounterWords * 4);
+  w.block_counts = take(B * (size_t)w.blocks_per_req * sizeof(uint2));
+  w.sync = take(kSyncWords * 4);
+  w.total = off;
+  return w;
+}
+
+void select_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* counters,
+                         ZeroRegion* sync) {
+  counters->base = (uint32_t*)((char*)workspace + w.counters);
+  counters->stride = kSelCounterWords;
+  counters->words = kSelCounterWords;
+  counters->count = batch;
+  sync->base = (uint32_t*)((char*)workspace + w.sync);
+  sync->stride = kSyncSlotWords;
+  sync->words = kSyncLiveWords;
+  sync->count = kSyncSlots + 1;
+}
+
+__global__ __launch_bounds__(256) void select_zero_kernel(ZeroRegion r0, ZeroRegion r1) {
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x, step = (int64_t)gridDim.x * 256;
+  for (int64_t w = gid; w < (int64_t)r0.count * r0.words; w += step)
+    r0.base[(w / r0.words) * r0.stride + w % r0.words] = 0u;
+  for (int64_t w = gid; w < (int64_t)r1.count * r1.words; w += step)
+    r1.base[(w / r1.words) * r1.stride + w % r1.words] = 0u;
 }
 
 static ScoreArgs selection_args(const ts_config* cfg, const ts_batch* bt, const void* qf,
@@ -571,20 +848,60 @@ static ScoreArgs selection_args(const ts_config* cfg, const ts_batch* bt, const 
   return a;
 }
 
+int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+                  int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
+                  int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
+                  int64_t vote_stride, void* workspace, uint32_t* clear, int clear_per_req,
+                  hipStream_t stream) {
+  const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len);
+  TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE, "fused selection: unsupported shape");
+  char* ws = (char*)workspace;
+  ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, hit, (float*)(ws + w.partials),
+                               w.tokens_per_block);
+  a.sync = (uint32_t*)(ws + w.sync);
+  a.stats = (float*)(ws + w.stats);
+  a.votes = votes;
+  a.vote_stride = vote_stride;
+  a.counters = (uint32_t*)(ws + w.counters);
+  a.block_counts = (uint2*)(ws + w.block_counts);
+  a.sel = sel;
+  a.sel_pos = sel_pos;
+  a.sel_stride = sel_stride;
+  a.sel_len = sel_len;
+  a.topk_cache = cache ? cache->topk_cache : nullptr;
+  a.cache_len = cache ? cache->cache_len : nullptr;
+  a.clear = clear;
+  a.clear_per_req = clear_per_req;
+  a.spin_ticks = 200000000ull;  // 2 s of the 100 MHz clock
+  const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
+  const dim3 grid((unsigned)w.blocks_per_req, (unsigned)bt->batch);
+  void* params[] = {(void*)&a};
+  // An ordinary launch: the grid was sized to be resident all at once, which holds
+  // as long as the device runs nothing else beside this stream.  (The cooperative
+  // launch API would guarantee it, at some 25 us of extra launch latency.)
+  const hipError_t e =
+      hipLaunchKernel(fn, grid, dim3(256), params,
+                      fused_lds_bytes(w.tokens_per_block, cfg->num_heads), stream);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(TS_EHIP, "fused selection launch: %s", hipGetErrorString(e));
+  }
+  return TS_OK;
+}
+
 }  // namespace ts
 
 using namespace ts;
 
 extern "C" {
 
-int ts_set_fused_vote(int enable) { return set_fused_vote(enable); }
+int ts_set_fused_select(int enable) { return set_fused_select(enable); }
 
 size_t ts_score_partials_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
   const int tpb = score_tokens_per_block((int64_t)batch * max_seq_len, cfg->num_heads);
   const size_t nchunks = (size_t)ceil_div(max_seq_len, tpb);
-  return partials_region_bytes(cfg, batch, nchunks) +
-         align_up((size_t)batch * cfg->num_heads * 2 * sizeof(float), 256);  // + merged statistics
+  return align_up((size_t)batch * cfg->num_heads * nchunks * 2 * sizeof(float), 256);
 }
 
 int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
@@ -614,59 +931,51 @@ int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const voi
                                    (hipStream_t)stream);
 }
 
-int ts_score_vote_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+int ts_select_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
   return fused_tokens_per_block(cfg, batch, max_seq_len) > 0 ? 1 : 0;
 }
 
-int ts_score_vote(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
-                  int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
-                  float* partials, size_t partials_bytes, void* topk_workspace,
-                  size_t topk_workspace_bytes, ts_stream_t stream) {
+size_t ts_select_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+  if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
+  return select_workspace(cfg, batch, max_seq_len).total;
+}
+
+int ts_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+              int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
+              int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
+              int64_t vote_stride, void* workspace, size_t workspace_bytes, ts_stream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
-  TS_REQUIRE(qf && k_pool && votes && partials && topk_workspace, TS_EINVAL,
-             "ts_score_vote: NULL tensor argument");
+  TS_REQUIRE(qf && k_pool && sel && sel_pos && sel_len && workspace, TS_EINVAL,
+             "ts_select: NULL tensor argument");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
+  const int max_sel = cfg->n_init + cfg->top_k + cfg->n_local;
+  TS_REQUIRE(sel_stride >= max_sel, TS_EWORKSPACE, "sel_stride %lld < n_init+top_k+n_local = %d",
+             (long long)sel_stride, max_sel);
   const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
-  TS_REQUIRE(vote_stride >= max_n, TS_EWORKSPACE, "vote_stride %lld < max candidates %d",
-             (long long)vote_stride, max_n);
-  TS_REQUIRE(partials_bytes >= ts_score_partials_bytes(cfg, bt->batch, bt->max_seq_len),
-             TS_EWORKSPACE, "ts_score_vote: partials %zu bytes too small", partials_bytes);
-  TS_REQUIRE(topk_workspace_bytes >= ts_topk_workspace_bytes(cfg, bt->batch, bt->max_seq_len),
-             TS_EWORKSPACE, "ts_score_vote: top-k workspace %zu bytes too small",
-             topk_workspace_bytes);
-  const int tpb = fused_tokens_per_block(cfg, bt->batch, bt->max_seq_len);
-  TS_REQUIRE(tpb > 0, TS_ESHAPE,
-             "ts_score_vote: batch %d x %d tokens does not fit one co-resident grid (or pool_kernel "
-             "is on); use ts_score + ts_vote",
+  TS_REQUIRE(votes == nullptr || vote_stride >= max_n, TS_EWORKSPACE,
+             "vote_stride %lld < max candidates %d", (long long)vote_stride, max_n);
+  TS_REQUIRE(hit == nullptr || cache != nullptr, TS_EINVAL,
+             "ts_select: hit flags need the selection cache");
+  if (cache)
+    TS_REQUIRE(cache->topk_cache && cache->cache_len, TS_EINVAL,
+               "ts_select: selection cache has a NULL array");
+  const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len);
+  TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE,
+             "ts_select: batch %d x %d tokens does not fit one co-resident grid (or pool_kernel is "
+             "on); use ts_score + ts_vote + ts_topk_ragged",
              bt->batch, bt->max_seq_len);
-
-  ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, skip, partials, tpb);
-  const int unfused_tpb =
-      score_tokens_per_block((int64_t)bt->batch * bt->max_seq_len, cfg->num_heads);
-  a.stats = (float*)((char*)partials +
-                     partials_region_bytes(cfg, bt->batch, ceil_div(bt->max_seq_len, unfused_tpb)));
-  a.votes = votes;
-  a.vote_stride = vote_stride;
-  a.topk_ws = (uint32_t*)topk_workspace;
-  a.topk_ws_stride = topk_ws_stride_words(max_n);
-  a.sync = topk_sync_area(topk_workspace, bt->batch, max_n);
-  a.spin_ticks = 200000000ull;  // 2 s of the 100 MHz clock
-  const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
-  const dim3 grid((unsigned)ceil_div(max_n, tpb), (unsigned)bt->batch);
-  void* params[] = {(void*)&a};
-  // An ordinary launch: the grid was sized to be resident all at once, which holds
-  // as long as the device runs nothing else beside this stream.  (The cooperative
-  // launch API would guarantee it, at some 25 us of extra launch latency.)
-  const hipError_t e = hipLaunchKernel(fn, grid, dim3(256), params,
-                                       fused_lds_bytes(tpb, cfg->num_heads), (hipStream_t)stream);
-  if (e != hipSuccess) {
-    (void)hipGetLastError();
-    return fail(TS_EHIP, "ts_score_vote launch: %s", hipGetErrorString(e));
-  }
-  return TS_OK;
+  TS_REQUIRE(workspace_bytes >= w.total, TS_EWORKSPACE, "ts_select: workspace %zu bytes < required %zu",
+             workspace_bytes, w.total);
+  ZeroRegion counters, sync;
+  select_zero_regions(w, workspace, bt->batch, &counters, &sync);
+  hipLaunchKernelGGL(select_zero_kernel, dim3((unsigned)(8 * bt->batch)), dim3(256), 0,
+                     (hipStream_t)stream, counters, sync);
+  TS_TRY(check_launch("select_zero_kernel"));
+  return launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,
+                       votes, vote_stride, workspace, nullptr, 0, (hipStream_t)stream);
 }
 
 int ts_paged_matmul(const void* query, const void* token, int64_t pool_rows,

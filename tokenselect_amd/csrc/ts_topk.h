@@ -1,6 +1,6 @@
-// Shared declarations of the ragged top-k: workspace layout, kernel arguments and
-// the key transform, used by ts_topk.hip, by the vote kernel (which can fill the
-// first histogram while it writes the votes) and by the per-layer driver.
+// Shared declarations of the ragged top-k: workspace layout, kernel arguments, the
+// key transform and the histogram search, used by ts_topk.hip, by the fused
+// selection kernel and by the per-layer driver.
 #pragma once
 
 #include "ts_common.h"
@@ -11,25 +11,13 @@ constexpr int kTopkBins = 2048;          // 11-bit digits
 constexpr int kTopkSlice = 512;          // candidates per workgroup of the hist / mark grids
 constexpr int kTopkFinalThreads = 1024;
 // Per-request workspace, in 32-bit words:
-//   [hist0: 8 x 2048][hist1: 2048][cand_count: 1, padded to 64]   <- zeroed before every selection
+//   [hist0: 2048][hist1: 2048][cand_count: 1, padded to 64]   <- zeroed before every selection
 //   [bitmap: 1 bit per candidate, 64-bit words]
 //   [candidate list: (key, position) pairs, up to one per candidate]
-// The first histogram is kept in kTopkHistCopies copies that its readers add up:
-// the votes of a request fall into a few dozen adjacent bins, i.e. one or two cache
-// lines, and hundreds of workgroups adding to the same line serialise in memory.
-constexpr int kTopkHistCopies = 8;
 constexpr int kTopkHist0 = 0;
-constexpr int kTopkHist1 = kTopkHistCopies * kTopkBins;
-constexpr int kTopkCandCount = kTopkHist1 + kTopkBins;
-constexpr int kTopkCounterWords = kTopkCandCount + 64;
-// Behind the per-request pieces lies the rendezvous area of the fused score + vote
-// kernel, cleared together with the counters: kSyncSlots + 1 slots of two live
-// words, kSyncSlotWords apart so that the slots fall into different memory
-// channels.  Slot 0: [arrival counter, fault flag]; slot 1 + r: [round reached]
-// replica r, polled by the workgroups with index % kSyncSlots == r.
-constexpr int kSyncSlots = 64;
-constexpr int kSyncSlotWords = 1024;
-constexpr size_t kSyncWords = (size_t)(kSyncSlots + 1) * kSyncSlotWords;
+constexpr int kTopkHist1 = kTopkBins;
+constexpr int kTopkCandCount = 2 * kTopkBins;
+constexpr int kTopkCounterWords = 2 * kTopkBins + 64;
 
 struct TopkArgs {
   const float* votes;
@@ -66,25 +54,73 @@ __device__ __forceinline__ uint32_t vote_key(float v) {
   const uint32_t u = __float_as_uint(v);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
-// The copy of the first histogram that workgroup `block` of a request adds to.
-__device__ __forceinline__ uint32_t* hist0_copy(uint32_t* request_ws, unsigned block) {
-  return request_ws + kTopkHist0 + (block % kTopkHistCopies) * kTopkBins;
-}
 __device__ __forceinline__ uint32_t key_bin0(uint32_t key) { return key >> 21; }
 __device__ __forceinline__ uint32_t key_bin1(uint32_t key) { return (key >> 10) & 2047u; }
 __device__ __forceinline__ uint32_t key_bin2(uint32_t key) { return key & 1023u; }
 
-size_t topk_ws_stride_words(int max_n);
-// First word of the rendezvous area inside a workspace of `batch` requests.
-inline uint32_t* topk_sync_area(void* workspace, int batch, int max_n) {
-  return (uint32_t*)workspace + align_up(topk_ws_stride_words(max_n) * (size_t)batch, 64);
+// Block-wide search of a descending histogram: finds the bin t such that
+// count(bins > t) < need <= count(bins >= t).  `hist` has NB entries (global or
+// LDS) per copy, NB a multiple of blockDim.x; COPIES consecutive copies are added
+// up.  Returns t and count(bins > t) to every thread.  `scratch` is LDS of
+// blockDim.x/64 + 2 words.
+template <int NB, int COPIES = 1>
+__device__ __forceinline__ void find_threshold_bin(const uint32_t* hist, uint32_t need,
+                                                   uint32_t* scratch, uint32_t& t_out,
+                                                   uint32_t& above_out) {
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int per = NB / nthreads;  // bins per thread, thread 0 owns the highest bins
+  const int lane = tid & 63, wave = tid >> 6, nwaves = nthreads >> 6;
+  const int hi_bin = NB - 1 - tid * per;
+  uint32_t local[8];
+  uint32_t mine = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    local[i] = 0;
+    if (i < per) {
+#pragma unroll
+      for (int c = 0; c < COPIES; ++c) local[i] += hist[c * NB + hi_bin - i];
+      mine += local[i];
+    }
+  }
+  // exclusive prefix of `mine` over threads (descending bins)
+  uint32_t incl = mine;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63) scratch[wave] = incl;
+  if (tid == 0) {
+    scratch[nwaves] = 0;
+    scratch[nwaves + 1] = 0;
+  }
+  __syncthreads();
+  uint32_t wave_base = 0;
+  for (int w = 0; w < wave; ++w) wave_base += scratch[w];
+  const uint32_t before = wave_base + incl - mine;  // count in bins above this thread's range
+  if (before < need && need <= before + mine) {      // the crossing lies in this thread's bins
+    uint32_t run = before;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (i < per) {
+        if (run < need && need <= run + local[i]) {
+          scratch[nwaves] = (uint32_t)(hi_bin - i);
+          scratch[nwaves + 1] = run;
+        }
+        run += local[i];
+      }
+  }
+  __syncthreads();
+  t_out = scratch[nwaves];
+  above_out = scratch[nwaves + 1];
+  __syncthreads();
 }
+
+size_t topk_ws_stride_words(int max_n);
 TopkArgs make_topk_args(const ts_config* cfg, const ts_batch* bt, const float* votes,
                         int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
                         int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
                         uint32_t* workspace);
-// zero: clear the counters first; hist: build the first histogram here (false when
-// the vote kernel already did).
-int launch_topk(const TopkArgs& a, int batch, int max_n, bool zero, bool hist, hipStream_t stream);
+int launch_topk(const TopkArgs& a, int batch, int max_n, hipStream_t stream);
 
 }  // namespace ts

@@ -28,74 +28,8 @@ __device__ __forceinline__ int pooled_count(int n, int pool_kernel) {
   return (pool_kernel > 0 && (pool_kernel & 1) == 0) ? n - 1 : n;  // even kernel: one fewer
 }
 
-// Block-wide search of a descending histogram: finds the bin t such that
-// count(bins > t) < need <= count(bins >= t).  `hist` has NB entries (global or
-// LDS) per copy, NB a multiple of blockDim.x; COPIES consecutive copies are added
-// up.  Returns t and count(bins > t) to every thread.  `scratch` is LDS of
-// blockDim.x/64 + 2 words.
-template <int NB, int COPIES = 1>
-__device__ __forceinline__ void find_threshold_bin(const uint32_t* hist, uint32_t need,
-                                                   uint32_t* scratch, uint32_t& t_out,
-                                                   uint32_t& above_out) {
-  const int tid = threadIdx.x, nthreads = blockDim.x;
-  const int per = NB / nthreads;  // bins per thread, thread 0 owns the highest bins
-  const int lane = tid & 63, wave = tid >> 6, nwaves = nthreads >> 6;
-  const int hi_bin = NB - 1 - tid * per;
-  uint32_t local[8];
-  uint32_t mine = 0;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    local[i] = 0;
-    if (i < per) {
-#pragma unroll
-      for (int c = 0; c < COPIES; ++c) local[i] += hist[c * NB + hi_bin - i];
-      mine += local[i];
-    }
-  }
-  // exclusive prefix of `mine` over threads (descending bins)
-  uint32_t incl = mine;
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const uint32_t up = __shfl_up(incl, off);
-    if (lane >= off) incl += up;
-  }
-  if (lane == 63) scratch[wave] = incl;
-  if (tid == 0) {
-    scratch[nwaves] = 0;
-    scratch[nwaves + 1] = 0;
-  }
-  __syncthreads();
-  uint32_t wave_base = 0;
-  for (int w = 0; w < wave; ++w) wave_base += scratch[w];
-  const uint32_t before = wave_base + incl - mine;  // count in bins above this thread's range
-  if (before < need && need <= before + mine) {      // the crossing lies in this thread's bins
-    uint32_t run = before;
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-      if (i < per) {
-        if (run < need && need <= run + local[i]) {
-          scratch[nwaves] = (uint32_t)(hi_bin - i);
-          scratch[nwaves + 1] = run;
-        }
-        run += local[i];
-      }
-  }
-  __syncthreads();
-  t_out = scratch[nwaves];
-  above_out = scratch[nwaves + 1];
-  __syncthreads();
-}
-
-// Workgroup b < batch clears the counters of request b, workgroup `batch` the live
-// words of the rendezvous area.
 __global__ __launch_bounds__(256) void topk_zero_kernel(uint32_t* __restrict__ ws,
-                                                        size_t stride_words, int batch,
-                                                        uint32_t* __restrict__ sync) {
-  if ((int)blockIdx.x == batch) {
-    for (int i = threadIdx.x; i < 2 * (kSyncSlots + 1); i += 256)
-      sync[(size_t)(i >> 1) * kSyncSlotWords + (i & 1)] = 0u;
-    return;
-  }
+                                                        size_t stride_words) {
   uint32_t* p = ws + (size_t)blockIdx.x * stride_words;
   for (int i = threadIdx.x; i < kTopkCounterWords; i += 256) p[i] = 0u;
 }
@@ -115,7 +49,7 @@ __global__ __launch_bounds__(256) void topk_hist_kernel(TopkArgs a) {
   for (int i = lo + threadIdx.x; i < min(lo + kTopkSlice, n); i += 256)
     atomicAdd(&lh[key_bin0(vote_key(votes[i]))], 1u);
   __syncthreads();
-  uint32_t* hist0 = hist0_copy(topk_ws(a.ws, a.ws_stride, b), blockIdx.x);
+  uint32_t* hist0 = topk_ws(a.ws, a.ws_stride, b) + kTopkHist0;
   for (int i = threadIdx.x; i < kTopkBins; i += 256)
     if (lh[i]) atomicAdd(&hist0[i], lh[i]);
 }
@@ -133,7 +67,7 @@ __global__ __launch_bounds__(256) void topk_mark_kernel(TopkArgs a) {
   __shared__ uint32_t lh[kTopkBins];
   uint32_t* ws = topk_ws(a.ws, a.ws_stride, b);
   uint32_t t0, above0;
-  find_threshold_bin<kTopkBins, kTopkHistCopies>(ws + kTopkHist0, (uint32_t)geo.k, scratch, t0, above0);
+  find_threshold_bin<kTopkBins>(ws + kTopkHist0, (uint32_t)geo.k, scratch, t0, above0);
   for (int i = threadIdx.x; i < kTopkBins; i += 256) lh[i] = 0u;
   __syncthreads();
 
@@ -217,7 +151,7 @@ __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs 
   auto mark = [&](uint32_t pos) { atomicOr(&bitmap32[pos >> 5], 1u << (pos & 31u)); };
 
   uint32_t t0, above0, t1, above1, t2, above2;
-  find_threshold_bin<kTopkBins, kTopkHistCopies>(ws + kTopkHist0, (uint32_t)k, scratch, t0, above0);
+  find_threshold_bin<kTopkBins>(ws + kTopkHist0, (uint32_t)k, scratch, t0, above0);
   const uint32_t need1 = (uint32_t)k - above0;  // still to take inside bin t0
   find_threshold_bin<kTopkBins>(ws + kTopkHist1, need1, scratch, t1, above1);
   const uint32_t need2 = need1 - above1;  // still to take inside (t0, t1)
@@ -365,18 +299,14 @@ TopkArgs make_topk_args(const ts_config* cfg, const ts_batch* bt, const float* v
   return a;
 }
 
-int launch_topk(const TopkArgs& a, int batch, int max_n, bool zero, bool hist, hipStream_t stream) {
+int launch_topk(const TopkArgs& a, int batch, int max_n, hipStream_t stream) {
   if (max_n > 0) {
     const dim3 grid((unsigned)ceil_div(max_n, kTopkSlice), (unsigned)batch);
-    if (zero) {
-      hipLaunchKernelGGL(topk_zero_kernel, dim3((unsigned)batch), dim3(256), 0, stream, a.ws,
-                         a.ws_stride, batch, (uint32_t*)nullptr);
-      TS_TRY(check_launch("topk_zero_kernel"));
-    }
-    if (hist) {
-      hipLaunchKernelGGL(topk_hist_kernel, grid, dim3(256), 0, stream, a);
-      TS_TRY(check_launch("topk_hist_kernel"));
-    }
+    hipLaunchKernelGGL(topk_zero_kernel, dim3((unsigned)batch), dim3(256), 0, stream, a.ws,
+                       a.ws_stride);
+    TS_TRY(check_launch("topk_zero_kernel"));
+    hipLaunchKernelGGL(topk_hist_kernel, grid, dim3(256), 0, stream, a);
+    TS_TRY(check_launch("topk_hist_kernel"));
     hipLaunchKernelGGL(topk_mark_kernel, grid, dim3(256), 0, stream, a);
     TS_TRY(check_launch("topk_mark_kernel"));
   }
@@ -393,13 +323,13 @@ extern "C" {
 size_t ts_topk_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
   const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
-  return align_up(topk_ws_stride_words(max_n) * 4 * (size_t)batch, 256) + kSyncWords * 4;
+  return align_up(topk_ws_stride_words(max_n) * 4 * (size_t)batch, 256);
 }
 
-static int topk_entry(const ts_config* cfg, const ts_batch* bt, const float* votes,
-                      int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
-                      int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
-                      void* workspace, size_t workspace_bytes, bool counted, ts_stream_t stream) {
+int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
+                   int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
+                   int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
+                   void* workspace, size_t workspace_bytes, ts_stream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
   TS_REQUIRE(votes && sel && sel_pos && sel_len, TS_EINVAL, "ts_topk_ragged: NULL tensor argument");
@@ -419,38 +349,7 @@ static int topk_entry(const ts_config* cfg, const ts_batch* bt, const float* vot
              "ts_topk_ragged: workspace %zu bytes < required %zu", workspace_bytes, need);
   const TopkArgs a = make_topk_args(cfg, bt, votes, vote_stride, hit, cache, sel, sel_pos,
                                     sel_stride, sel_len, (uint32_t*)workspace);
-  return launch_topk(a, bt->batch, max_n, /*zero=*/!counted, /*hist=*/!counted, (hipStream_t)stream);
-}
-
-int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
-                   int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
-                   int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
-                   void* workspace, size_t workspace_bytes, ts_stream_t stream) {
-  return topk_entry(cfg, bt, votes, vote_stride, hit, cache, sel, sel_pos, sel_stride, sel_len,
-                    workspace, workspace_bytes, false, stream);
-}
-
-int ts_topk_ragged_counted(const ts_config* cfg, const ts_batch* bt, const float* votes,
-                           int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
-                           int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
-                           void* workspace, size_t workspace_bytes, ts_stream_t stream) {
-  return topk_entry(cfg, bt, votes, vote_stride, hit, cache, sel, sel_pos, sel_stride, sel_len,
-                    workspace, workspace_bytes, true, stream);
-}
-
-int ts_topk_reset(const ts_config* cfg, int32_t batch, int32_t max_seq_len, void* workspace,
-                  size_t workspace_bytes, ts_stream_t stream) {
-  TS_TRY(validate_config(cfg));
-  TS_REQUIRE(batch >= 1 && max_seq_len >= 1, TS_EINVAL, "ts_topk_reset: batch=%d max_seq_len=%d",
-             batch, max_seq_len);
-  TS_REQUIRE(workspace != nullptr &&
-                 workspace_bytes >= ts_topk_workspace_bytes(cfg, batch, max_seq_len),
-             TS_EWORKSPACE, "ts_topk_reset: workspace %zu bytes too small", workspace_bytes);
-  const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
-  hipLaunchKernelGGL(topk_zero_kernel, dim3((unsigned)batch + 1), dim3(256), 0, (hipStream_t)stream,
-                     (uint32_t*)workspace, topk_ws_stride_words(max_n), batch,
-                     topk_sync_area(workspace, batch, max_n));
-  return check_launch("topk_zero_kernel");
+  return launch_topk(a, bt->batch, max_n, (hipStream_t)stream);
 }
 
 }  // extern "C"

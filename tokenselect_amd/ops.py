@@ -147,10 +147,11 @@ def _c_cache(cache: Optional[SelectionCache], cfg: LayerConfig, batch: int):
                                    _p(cache.counters), float(cache.threshold)))
 
 
-def set_fused_vote(enable: bool) -> bool:
-    """Chooses between the cooperative score + vote kernel (default) and the separate
-    kernels inside :class:`DecodeLayer`; returns the previous setting."""
-    return bool(_lib.load().ts_set_fused_vote(1 if enable else 0))
+def set_fused_select(enable: bool) -> bool:
+    """Chooses between the single-launch selection (default, where the shape allows)
+    and the separate kernels inside :class:`DecodeLayer`; returns the previous
+    setting."""
+    return bool(_lib.load().ts_set_fused_select(1 if enable else 0))
 
 
 def score_stride_for(max_seq_len: int) -> int:
@@ -238,59 +239,52 @@ def score(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
     return scores, partials
 
 
-def score_vote_supported(cfg: LayerConfig, batch: int, max_seq_len: int) -> bool:
-    """Whether :func:`score_vote` can serve this shape (``ts_score_vote_supported``)."""
-    return bool(_lib.load().ts_score_vote_supported(ctypes.byref(cfg.to_c()), int(batch),
-                                                    int(max_seq_len)))
+def select_supported(cfg: LayerConfig, batch: int, max_seq_len: int) -> bool:
+    """Whether :func:`select` can serve this shape (``ts_select_supported``)."""
+    return bool(_lib.load().ts_select_supported(ctypes.byref(cfg.to_c()), int(batch),
+                                                int(max_seq_len)))
 
 
-class SelectionWorkspace:
-    """Buffers of the fused selection: votes, softmax partials and the top-k workspace
-    that :func:`score_vote` fills and :func:`topk_ragged` (``counted=``) consumes."""
-
-    def __init__(self, cfg: LayerConfig, batch: int, max_seq_len: int, device):
-        lib, c = _lib.load(), cfg.to_c()
-        self.batch, self.max_seq_len = int(batch), int(max_seq_len)
-        self.votes = torch.empty((batch, score_stride_for(max_seq_len)), dtype=torch.float32,
-                                 device=device)
-        nbytes = lib.ts_score_partials_bytes(ctypes.byref(c), batch, max_seq_len)
-        self.partials = torch.empty((max(nbytes, 256) // 4,), dtype=torch.float32, device=device)
-        nbytes = lib.ts_topk_workspace_bytes(ctypes.byref(c), batch, max_seq_len)
-        self.topk = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=device)
-        self._cfg = cfg
-
-    def reset(self) -> None:
-        """Clears the selection counters (``ts_topk_reset``); needed before every
-        :func:`score_vote`."""
-        _lib.check(_lib.load().ts_topk_reset(ctypes.byref(self._cfg.to_c()), self.batch,
-                                             self.max_seq_len, _p(self.topk), self.topk.numel(),
-                                             _stream()))
-
-    def fault(self) -> bool:
-        """True when a grid-wide wait of :func:`score_vote` gave up (synchronises)."""
-        words = self.topk.view(torch.int32)
-        return bool(words[words.numel() - 65 * 1024 + 1].item())
-
-
-def score_vote(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
-               space: SelectionWorkspace, skip: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Scoring and soft vote in one cooperative launch (tr.py:350-361): fills and returns
-    ``space.votes`` and the first histogram of the selection.  ``space.reset()`` must
-    precede every call."""
+def select(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
+           hit: Optional[torch.Tensor] = None, cache: Optional[SelectionCache] = None,
+           want_votes: bool = False, workspace: Optional[torch.Tensor] = None):
+    """The whole selection in one launch (tr.py:350-373, 424-449): scoring, soft vote,
+    exact top-k, ascending order and index assembly, the scores never leaving LDS.
+    Returns ``(sel, sel_pos, sel_len, votes, workspace)`` with the first three as
+    from :func:`topk_ragged`; ``votes`` is ``[B, stride]`` fp32 when ``want_votes``
+    else ``None``.  ``workspace`` (uint8) may be passed back in to avoid allocating."""
     c, cb = cfg.to_c(), _c_batch(cfg, bt)
     _need(qf, "qf", torch.bfloat16)
     _check_pool(cfg, k_pool, "k_pool")
-    if qf.numel() != bt.batch * cfg.num_heads * cfg.head_dim:
+    B = bt.batch
+    if qf.numel() != B * cfg.num_heads * cfg.head_dim:
         raise ValueError("qf must hold B*H*D elements")
-    if bt.batch != space.batch or bt.max_seq_len > space.max_seq_len:
-        raise ValueError("workspace was sized for another batch")
-    if skip is not None:
-        _need(skip, "skip", torch.int32, 1)
-    _lib.check(_lib.load().ts_score_vote(
-        ctypes.byref(c), ctypes.byref(cb), _p(qf), _p(k_pool), k_pool.shape[0], _p(skip),
-        _p(space.votes), space.votes.shape[1], _p(space.partials), space.partials.numel() * 4,
-        _p(space.topk), space.topk.numel(), _stream()))
-    return space.votes
+    if hit is not None:
+        _need(hit, "hit", torch.int32, 1)
+    lib = _lib.load()
+    nbytes = lib.ts_select_workspace_bytes(ctypes.byref(c), B, bt.max_seq_len)
+    if workspace is None or workspace.numel() < nbytes:
+        workspace = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=qf.device)
+    sel = torch.empty((B, cfg.max_sel), dtype=torch.int32, device=qf.device)
+    sel_pos = torch.empty_like(sel)
+    sel_len = torch.empty((B,), dtype=torch.int32, device=qf.device)
+    votes = None
+    if want_votes:
+        votes = torch.empty((B, score_stride_for(bt.max_seq_len)), dtype=torch.float32,
+                            device=qf.device)
+    _lib.check(lib.ts_select(
+        ctypes.byref(c), ctypes.byref(cb), _p(qf), _p(k_pool), k_pool.shape[0], _p(hit),
+        _c_cache(cache, cfg, B), _p(sel), _p(sel_pos), cfg.max_sel, _p(sel_len), _p(votes),
+        votes.shape[1] if votes is not None else 0, _p(workspace), workspace.numel(), _stream()))
+    return sel, sel_pos, sel_len, votes, workspace
+
+
+def select_fault(cfg: LayerConfig, bt: Batch, workspace: torch.Tensor) -> bool:
+    """True when a grid-wide wait of the last :func:`select` on ``workspace`` gave up
+    (synchronises)."""
+    nbytes = _lib.load().ts_select_workspace_bytes(ctypes.byref(cfg.to_c()), bt.batch,
+                                                   bt.max_seq_len)
+    return bool(workspace.view(torch.int32)[nbytes // 4 - 65 * 1024].item())
 
 
 def scores_head_major(cfg: LayerConfig, scores: torch.Tensor) -> torch.Tensor:
@@ -329,12 +323,10 @@ def vote(cfg: LayerConfig, bt: Batch, scores: torch.Tensor, partials: torch.Tens
 
 
 def topk_ragged(cfg: LayerConfig, bt: Batch, votes: torch.Tensor,
-                hit: Optional[torch.Tensor] = None, cache: Optional[SelectionCache] = None,
-                counted: Optional["SelectionWorkspace"] = None):
+                hit: Optional[torch.Tensor] = None, cache: Optional[SelectionCache] = None):
     """Top-k + sort + assembly (tr.py:371-373, 433-449).  Returns
     ``(sel [B,max_sel] int32 physical slots, sel_pos [B,max_sel] int32 logical
-    positions, sel_len [B] int32)``.  ``counted``: the workspace :func:`score_vote`
-    has just filled (``ts_topk_ragged_counted``)."""
+    positions, sel_len [B] int32)``."""
     c, cb = cfg.to_c(), _c_batch(cfg, bt)
     _need(votes, "votes", torch.float32, 2)
     B = bt.batch
@@ -346,13 +338,9 @@ def topk_ragged(cfg: LayerConfig, bt: Batch, votes: torch.Tensor,
     sel_pos = torch.empty_like(sel)
     sel_len = torch.empty((B,), dtype=torch.int32, device=votes.device)
     lib = _lib.load()
-    if counted is not None:
-        ws, entry = counted.topk, lib.ts_topk_ragged_counted
-    else:
-        nbytes = lib.ts_topk_workspace_bytes(ctypes.byref(c), B, bt.max_seq_len)
-        ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=votes.device)
-        entry = lib.ts_topk_ragged
-    _lib.check(entry(ctypes.byref(c), ctypes.byref(cb), _p(votes), votes.shape[1], _p(hit),
+    nbytes = lib.ts_topk_workspace_bytes(ctypes.byref(c), B, bt.max_seq_len)
+    ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=votes.device)
+    _lib.check(lib.ts_topk_ragged(ctypes.byref(c), ctypes.byref(cb), _p(votes), votes.shape[1], _p(hit),
                      _c_cache(cache, cfg, B), _p(sel), _p(sel_pos), cfg.max_sel, _p(sel_len), _p(ws),
                      ws.numel(), _stream()))
     return sel, sel_pos, sel_len
