@@ -5,16 +5,19 @@ A step is one layer of the patched decode forward after the KV store
 (fingerprint -> score -> soft vote -> top-k -> index assembly -> sparse decode
 attention) over one synthetic batch resident in HBM, issued as a single
 ``ts_decode_layer`` call.  The default workload is the Llama-3-8B layer at
-128K context in a page-16 KV pool (``--workload c2``).
+128K context in a page-16 KV pool (``--workload c2``); ``c1``, ``c3`` and
+``c5`` are the other layer shapes, ``c4`` the 64-step selection-cache trace
+(there a step also stores the new token's K/V and consults the cache).
 
 Every step reads a different copy of the K/V pool (``--pools``, default 4, as
 consecutive layers of a model do): the copies together exceed the 256 MB
 last-level cache, so the keys really stream from HBM in every timed pass.
 
 Prints one JSON line: the per-layer latency, the roofline figures of the
-scoring kernel (algorithmic bytes / HIP-event time of the call that streams the
+dominant kernel (algorithmic bytes / HIP-event time of the call that streams the
 keys: ``ts_select``, the whole selection in one kernel, when the batch fits it,
-else ``ts_score``) and the CPU oracle timed on the host cores.
+else ``ts_score``), the same for the stand-alone scoring kernel and the gather
+attention, and the CPU oracle timed on the host cores.
 """
 
 import argparse
@@ -29,6 +32,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+# HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` runs of this script (KiB per dispatch, scaled by what the same
+# counters read for the 256 MiB copy of --calibration-copy); the runs and their
+# figures are recorded under profiles/.  Workloads not measured that way give null.
+MEASURED_TRAFFIC = {"C2": 271244542}  # profiles/decode_layer_c2_hbm_traffic.txt
 
 
 def event_time_us(fn, launches: int, warmup: int, before=None):
@@ -53,22 +62,27 @@ def event_time_us(fn, launches: int, warmup: int, before=None):
     return sum(times) / len(times), min(times)
 
 
-def cpu_baseline(wl, reps: int):
-    """The CPU oracle (a restatement of the reference's PyTorch path) on the
-    host cores, same inputs as the GPU run."""
+def cpu_baseline(wl, reps: int, requests=None):
+    """The CPU oracle (a restatement of the reference's PyTorch path) on the host
+    cores, same inputs as the GPU run; `requests` restricts it to a bounded sample
+    of the batch."""
     import oracle
     c = wl.cfg
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     torch.set_num_threads(threads)
-    q, kp, vp, table = wl.q.cpu(), wl.k_pool.cpu(), wl.v_pool.cpu(), wl.table.cpu()
-    tabs = [oracle.select.expand_page_table(table[b], L, c.page_size)
-            for b, L in enumerate(wl.seq_lens)]
+    idx = list(range(len(wl.seq_lens))) if requests is None else list(requests)
+    H, D = c.num_heads, c.head_dim
+    q = wl.q.view(len(wl.seq_lens), H * D)[idx].cpu()
+    kp, vp, table = wl.k_pool.cpu(), wl.v_pool.cpu(), wl.table.cpu()
+    lens = [wl.seq_lens[b] for b in idx]
+    ks = [wl.k_list[b] for b in idx]
+    tabs = [oracle.select.expand_page_table(table[b], wl.seq_lens[b], c.page_size) for b in idx]
     sm = c.sm_scale if c.sm_scale is not None else c.head_dim ** -0.5
 
     def run():
-        return oracle.layer.decode_layer(q, kp, vp, tabs, wl.seq_lens, c.num_heads, c.head_dim,
-                                         c.n_init, c.n_local, wl.k_list, c.rope_theta, c.rope_scale,
-                                         sm, c.logit_cap, c.rope_mode, c.pool_kernel)
+        return oracle.layer.decode_layer(q, kp, vp, tabs, lens, H, D, c.n_init, c.n_local, ks,
+                                         c.rope_theta, c.rope_scale, sm, c.logit_cap, c.rope_mode,
+                                         c.pool_kernel)
 
     run()
     times = []
@@ -80,28 +94,63 @@ def cpu_baseline(wl, reps: int):
     return times[len(times) // 2] * 1e6, torch.get_num_threads(), sels, out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3"])
-    ap.add_argument("--cpu-reps", type=int, default=3)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--layers", type=int, default=32, help="layers for the tokens/s figure")
-    ap.add_argument("--pools", type=int, default=4,
-                    help="copies of the K/V pool cycled through, one per step")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build measures the one-GPU hot path only; run with --gpus 1 "
-                 "(no multi-GPU figure exists for it).")
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback.")
+def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
+    """HIP-event timings of the calls that move the bytes: the selection (or the
+    scoring kernel where the selection does not fit one launch), the stand-alone
+    scoring kernel, and the gather attention."""
+    c, bt, B = wl.cfg, wl.batch, len(wl.seq_lens)
+    dev = wl.q.device
+    n_pools = len(k_pools)
+    cos, sin = ops.scoring_cos_sin(c.head_dim, c.rope_theta, c.rope_scale, c.n_local, dev)
+    qf = ops.rope_apply(wl.q.view(B, c.num_heads, c.head_dim), cos, sin, None)
+    score_bytes, attn_bytes = wl.score_bytes(), wl.attn_bytes()
 
-    from tokenselect_amd import ops, workloads
+    bufs = ops.score(c, bt, qf, wl.k_pool)
+    score_us, score_min = event_time_us(
+        lambda i: ops.score(c, bt, qf, k_pools[i % n_pools], out=bufs), steps, warmup)
+    score_only = {"kernel": "ts::score_kernel<Hkv,G,false,1> (ts_score: scores written tile-major)",
+                  "achieved": round(score_bytes / score_us / 1e3, 1), "peak": HBM_PEAK_GBS,
+                  "unit": "GB/s", "frac": round(score_bytes / score_us / 1e3 / HBM_PEAK_GBS, 4),
+                  "bytes_per_launch": score_bytes, "us_per_launch": round(score_us, 2),
+                  "us_min": round(score_min, 2)}
+    del bufs
 
-    dev = torch.device("cuda:0")
-    wl = {"c1": workloads.config1, "c2": workloads.config2, "c3": workloads.config3}[args.workload](dev)
+    if ops.select_supported(c, B, bt.max_seq_len):
+        space = [None]
+
+        def run_select(i):
+            space[0] = ops.select(c, bt, qf, k_pools[i % n_pools], workspace=space[0])[4]
+
+        # ts_select = one small clearing kernel (about 3 us, folded into the rotation
+        # kernel inside ts_decode_layer) + the selection kernel; both are timed here.
+        dom_us, dom_min = event_time_us(run_select, steps, warmup)
+        if ops.select_fault(c, bt, space[0]):
+            sys.exit("bench.py: a grid-wide wait of the selection kernel gave up")
+        dom_kernel = "ts::score_kernel<Hkv,G,false,2> (ts_select: score + vote + top-k in one launch)"
+    else:
+        dom_us, dom_min, dom_kernel = score_us, score_min, score_only["kernel"]
+    gbs = score_bytes / dom_us / 1e3
+    roofline = {"bound": "hbm", "kernel": dom_kernel, "achieved": round(gbs, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                "traffic": MEASURED_TRAFFIC.get(wl.name.split()[0]),
+                "bytes_per_launch": score_bytes, "us_per_launch": round(dom_us, 2),
+                "us_min": round(dom_min, 2)}
+
+    sel, sel_len = layer.sel, layer.sel_len
+    attn_us, _ = event_time_us(
+        lambda i: ops.sparse_decode_attention(c, wl.q, k_pools[i % n_pools], v_pools[i % n_pools],
+                                              sel, sel_len), steps, warmup)
+    attn = {"kernel": "ts::attn_kernel<G> (+ a 1 us ticket-clearing kernel when called on its own)",
+            "achieved": round(attn_bytes / attn_us / 1e3, 1), "unit": "GB/s",
+            "frac": round(attn_bytes / attn_us / 1e3 / HBM_PEAK_GBS, 4),
+            "bytes_per_launch": attn_bytes, "us_per_launch": round(attn_us, 2)}
+    return roofline, score_only, attn
+
+
+def bench_layer(args, ops, workloads, dev):
+    make = {"c1": workloads.config1, "c2": workloads.config2, "c3": workloads.config3,
+            "c5": workloads.config5_layer}[args.workload]
+    wl = make(dev)
     c, bt, B = wl.cfg, wl.batch, len(wl.seq_lens)
     layer = ops.DecodeLayer(c, B, bt.max_seq_len, dev)
     n_pools = max(1, args.pools)
@@ -118,79 +167,134 @@ def main():
     for i in range(args.steps):
         step(i)
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    us_per_layer = elapsed / args.steps * 1e6
+    us_per_layer = (time.perf_counter() - t0) / args.steps * 1e6
 
-    # Kernel-level roofline figures: the kernel that streams the keys, and the
-    # gather attention.
-    cos, sin = ops.scoring_cos_sin(c.head_dim, c.rope_theta, c.rope_scale, c.n_local, dev)
-    qf = ops.rope_apply(wl.q.view(B, c.num_heads, c.head_dim), cos, sin, None)
-    fused = ops.select_supported(c, B, bt.max_seq_len)
-    if fused:
-        space = [None]
-
-        def run_select(i):
-            space[0] = ops.select(c, bt, qf, k_pools[i % n_pools], workspace=space[0])[4]
-
-        # ts_select = one small clearing kernel + the selection kernel; the clearing
-        # kernel (about 2 us) is inside the timed span.
-        score_us, score_min = event_time_us(run_select, args.steps, args.warmup)
-        if ops.select_fault(c, bt, space[0]):
-            sys.exit("bench.py: a grid-wide wait of the selection kernel gave up")
-        score_kernel = "ts::score_kernel<Hkv,G,false,2> (ts_select: score + vote + top-k in one launch)"
-    else:
-        bufs = ops.score(c, bt, qf, wl.k_pool)
-        score_us, score_min = event_time_us(
-            lambda i: ops.score(c, bt, qf, k_pools[i % n_pools], out=bufs), args.steps, args.warmup)
-        score_kernel = "ts::score_kernel<Hkv,G,false,1> (ts_score)"
-    sel, sel_len = layer.sel, layer.sel_len
-    attn_us, _ = event_time_us(
-        lambda i: ops.sparse_decode_attention(c, wl.q, k_pools[i % n_pools], v_pools[i % n_pools],
-                                              sel, sel_len),
-        args.steps, args.warmup)
-    score_bytes, attn_bytes = wl.score_bytes(), wl.attn_bytes()
-    score_gbs = score_bytes / score_us / 1e3
-    attn_gbs = attn_bytes / attn_us / 1e3
+    roofline, score_only, attn = kernel_rooflines(ops, wl, k_pools, v_pools, layer, args.steps,
+                                                  args.warmup)
+    if args.calibration_copy:  # a plain copy of known size for the counter runs
+        src = torch.empty((256 << 20,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     result = {
         "metric": "us_per_layer_decode (score+top-k+sparse attn)",
-        "value": round(us_per_layer, 2),
-        "unit": "us",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(us_per_layer / 1e3, 5),
-        "higher_is_better": False,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
+        "value": round(us_per_layer, 2), "unit": "us", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(us_per_layer / 1e3, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": wl.name, "batch": B, "seq_lens_max": max(wl.seq_lens),
                    "page_size": c.page_size, "top_k": c.top_k, "n_init": c.n_init,
                    "n_local": c.n_local, "kv_pool_copies": n_pools},
         "tokens_per_s": round(B / (us_per_layer * 1e-6 * args.layers), 1),
         "tokens_per_s_note": f"selection+attention only, {args.layers} layers per token",
-        "roofline": {"bound": "hbm", "kernel": score_kernel, "achieved": round(score_gbs, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(score_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": None, "bytes_per_launch": score_bytes,
-                     "us_per_launch": round(score_us, 2), "us_min": round(score_min, 2)},
-        "gather_attention": {"achieved": round(attn_gbs, 1), "unit": "GB/s",
-                             "frac": round(attn_gbs / HBM_PEAK_GBS, 4),
-                             "bytes_per_launch": attn_bytes, "us_per_launch": round(attn_us, 2)},
+        "roofline": roofline, "score_only": score_only, "gather_attention": attn,
     }
 
     if not args.no_cpu_baseline:
-        cpu_us, cores, ref_sels, ref_out = cpu_baseline(wl, args.cpu_reps)
+        # Bounded sample: the whole batch where that is a few hundred ms of CPU work,
+        # else its first two requests.
+        sample = None if sum(wl.seq_lens) <= 300000 else [0, 1]
+        cpu_us, cores, ref_sels, ref_out = cpu_baseline(wl, args.cpu_reps, sample)
+        what = f"the full {wl.name} layer" if sample is None else \
+            f"requests 0-1 (L={wl.seq_lens[0]}, {wl.seq_lens[1]}) of {wl.name}"
         result["cpu_baseline"] = {
             "value": round(cpu_us, 1), "unit": "us", "cores": cores, "kind": "port",
-            "sample": f"the full {wl.name} layer, median of {args.cpu_reps} repetitions "
-                      "after one warm-up (PyTorch CPU oracle)"}
+            "sample": f"{what}, median of {args.cpu_reps} repetitions after one warm-up "
+                      "(PyTorch CPU oracle)"}
         # Parity of this very run against the oracle.
+        idx = list(range(B)) if sample is None else sample
         S = [int(x) for x in layer.sel_len.tolist()]
-        same = all(torch.equal(layer.sel[b, :S[b]].cpu(), ref_sels[b]) for b in range(B))
-        err = (layer.out.cpu().float() - ref_out.float()).abs().max().item()
+        same = all(torch.equal(layer.sel[b, :S[b]].cpu(), ref_sels[i]) for i, b in enumerate(idx))
+        err = (layer.out[idx].cpu().float() - ref_out.float()).abs().max().item()
         result["parity"] = {"selected_slots_identical": bool(same),
                             "attn_max_abs_err": round(err, 5)}
+    return result
+
+
+def bench_trace(args, ops, workloads, dev):
+    """Selection-cache trace: `trace_steps` consecutive decode steps of one layer, the
+    new token's K/V stored first, AR(1) queries with occasional jumps, cosine reuse
+    threshold bf16(0.9).  Reports the amortised time per step and the hit rate."""
+    steps = args.trace_steps
+    wl = workloads.config4(dev, steps=steps)
+    c, B = wl.cfg, len(wl.seq_lens)
+    L0 = wl.seq_lens[0]
+    qs = workloads.ar1_queries(B, c.num_heads * c.head_dim, steps, dev)
+    gen = torch.Generator(device=dev).manual_seed(7)
+    k_new = torch.randn((steps, B, c.num_kv_heads * c.head_dim), generator=gen, device=dev).bfloat16()
+    v_new = torch.randn((steps, B, c.num_kv_heads * c.head_dim), generator=gen, device=dev).bfloat16()
+    free = torch.arange(B * L0, B * (L0 + steps), dtype=torch.int32, device=dev).view(steps, B)
+    table0 = torch.zeros((B, L0 + steps), dtype=torch.int32, device=dev)
+    table0[:, :L0] = wl.table[:, :L0]
+    layer = ops.DecodeLayer(c, B, L0 + steps, dev)
+
+    def run_trace():
+        table, seq = table0.clone(), wl.seq_lens_dev.clone()
+        cache = ops.SelectionCache.allocate(c, B, dev)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for t in range(steps):
+            ops.kv_store(c, k_new[t], v_new[t], free[t], wl.k_pool, wl.v_pool, table, seq)
+            layer(qs[t], wl.k_pool, wl.v_pool, ops.Batch(seq, table, L0 + t + 1), cache)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e6, cache
+
+    for _ in range(max(1, args.warmup // steps)):
+        run_trace()
+    reps = max(1, args.steps // steps)
+    runs = [run_trace() for _ in range(reps)]
+    us_per_step = sum(r[0] for r in runs) / reps
+    counters = runs[-1][1].counters.cpu()
+    hits, lookups = int(counters[:, 0].sum()), int(counters[:, 1].sum())
+
+    result = {
+        "metric": "us_per_layer_decode (selection-cache trace: kv store + cache + select + attn)",
+        "value": round(us_per_step, 2), "unit": "us", "n_gpus": 1, "steps": reps * steps,
+        "warmup": max(1, args.warmup // steps) * steps, "ms_per_step": round(us_per_step / 1e3, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": wl.name, "batch": B, "seq_lens_max": L0 + steps, "page_size": 1,
+                   "top_k": c.top_k, "n_init": c.n_init, "n_local": c.n_local,
+                   "trace_steps": steps, "ar1_rho": 0.95, "jump_p": 0.1,
+                   "threshold": runs[-1][1].threshold, "kv_pool_copies": 1},
+        "hit_rate": round(hits / max(lookups, 1), 4), "hits": hits, "lookups": lookups,
+        "tokens_per_s": round(B / (us_per_step * 1e-6 * args.layers), 1),
+        "tokens_per_s_note": f"selection+attention only, {args.layers} layers per token",
+        "roofline": None, "cpu_baseline": None,
+    }
+    return result
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--layers", type=int, default=32, help="layers for the tokens/s figure")
+    ap.add_argument("--pools", type=int, default=4,
+                    help="copies of the K/V pool cycled through, one per step")
+    ap.add_argument("--trace-steps", type=int, default=64, help="decode steps of the c4 trace")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run five 256 MiB device copies (reference for counter runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures the one-GPU hot path only; run with --gpus 1 "
+                 "(no multi-GPU figure exists for it).")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback.")
+
+    from tokenselect_amd import ops, workloads
+
+    dev = torch.device("cuda:0")
+    if args.workload == "c4":
+        result = bench_trace(args, ops, workloads, dev)
+    else:
+        result = bench_layer(args, ops, workloads, dev)
     print(json.dumps(result), flush=True)
 
 

@@ -162,6 +162,14 @@ def config4(device, seed: int = 3, batch: int = 4, seq_len: int = 65536, steps: 
                  [top_k] * batch, 1, device, seed, extra_pages=batch * steps)
 
 
+def config5_layer(device, seed: int = 4, batch: int = 4, seq_len: int = 262144,
+                  top_k: int = 4096) -> Workload:
+    """One layer of the full-model configuration: Llama-3-8B shape, four requests of
+    256K context each, top-k 4096, page size 16."""
+    return build("C5-layer llama3-8b B%d L%d k%d page16" % (batch, seq_len, top_k), LLAMA3_8B,
+                 [seq_len] * batch, [top_k] * batch, 16, device, seed)
+
+
 def ar1_queries(batch: int, dim: int, steps: int, device, seed: int = 3, rho: float = 0.95,
                 jump_p: float = 0.1) -> torch.Tensor:
     """``q_t = rho q_{t-1} + sqrt(1-rho^2) eps`` with a fresh N(0,1) draw per
