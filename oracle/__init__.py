@@ -20,6 +20,9 @@ a CUDA GPU, none of which are available):
 * ``assemble``  - structural invariants (prefix / suffix / length / identity table).
 * ``attend``    - ``F.scaled_dot_product_attention`` with RoPE disabled, full
                   selection == textbook attention, position-shift invariance.
+* ``prefill``   - causal attention against ``F.scaled_dot_product_attention`` with
+                  an explicit mask (RoPE off), a one-row chunk == ``attend``, row
+                  ``i`` == decode attention over the first ``S - m + i + 1`` keys.
 * ``selcache``  - pure-Python replay of the state machine.  The reference ships
                   this branch disabled and not runnable (tr.py:918, 412, 397), so
                   its behaviour is *intended* semantics: parity unpinned.
@@ -29,4 +32,4 @@ the bf16 rounding / reduction order of Triton 3.0.0's ``tl.sum`` on NVIDIA, the
 tie order of CUDA ``torch.topk``, and FlashInfer's ``__sincosf`` error.
 """
 
-from . import rope, select, attend, selcache, layer  # noqa: F401
+from . import rope, select, attend, selcache, layer, prefill  # noqa: F401

@@ -120,15 +120,19 @@ def retrieval_indices(q: torch.Tensor, k_pool: torch.Tensor, tab: torch.Tensor,
                       seq_len: int, num_heads: int, head_dim: int, n_init: int,
                       n_local: int, k: int, rope_base: float, rope_scale=1.0,
                       mode: str = "fp32", kernel_size: int = -1,
-                      detail: Optional[dict] = None) -> Optional[torch.Tensor]:
+                      detail: Optional[dict] = None,
+                      qf_override: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """tr.py:375-449 for one request with the selection cache disabled, as
     released (tr.py:918).  ``q`` is ``[rows, H*D]`` bf16 un-rotated, ``tab`` the
     request's logical->physical table with the new token already appended
     (store precedes select, tr.py:787-791).  Returns physical slots ``[S]`` int32
-    or ``None`` for the dense fallback."""
+    or ``None`` for the dense fallback.  ``qf_override`` ([H*D] bf16) stands in for
+    the fingerprint, for checks downstream of a fingerprint computed elsewhere."""
     if is_dense(seq_len, n_init, n_local, k):
         return None
     qf = _rope.scoring_query(q, num_heads, head_dim, n_local, rope_base, rope_scale)
+    if qf_override is not None:
+        qf = qf_override.reshape(-1).to(qf.dtype)
     cand = tab[n_init:seq_len - n_local]
     top, s, c = get_topk_tokens(qf, k_pool, k, cand, head_dim, mode, kernel_size,
                                 return_all=True)

@@ -346,3 +346,98 @@ def test_batched_layer_applies_single_request_semantics():
     alone = oracle.layer.decode_layer(q[1:], k_pool, v_pool, tabs[1:], [28], H, D, 4, 8, [16],
                                       1e4, 1.0, D ** -0.5)[1]
     assert torch.equal(out[1], alone[0])
+
+
+# ---------------------------------------------------------------- chunked prefill
+def _prefill_case(seed=0, m=24, S=90, H=4, Hkv=2, P=200):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(m, H, 128, generator=g).bfloat16()
+    kp = torch.randn(P, Hkv, 128, generator=g).bfloat16()
+    vp = torch.randn(P, Hkv, 128, generator=g).bfloat16()
+    slots = torch.randperm(P, generator=g)[:S].int()
+    return q, kp, vp, slots
+
+
+def test_prefill_attention_matches_sdpa_with_explicit_mask():
+    """RoPE off: the chunk attention is textbook attention under the mask
+    key j visible to row i iff j <= S - m + i."""
+    q, kp, vp, slots = _prefill_case()
+    m, H, _ = q.shape
+    S, G = slots.shape[0], H // kp.shape[1]
+    got = oracle.prefill.sparse_prefill_attention(q, kp, vp, slots, 0.11, 1e4, rope_mode="NONE")
+    k = kp[slots.long()].float().repeat_interleave(G, dim=1).permute(1, 0, 2)   # [H, S, D]
+    v = vp[slots.long()].float().repeat_interleave(G, dim=1).permute(1, 0, 2)
+    mask = torch.tril(torch.ones(m, S, dtype=torch.bool), diagonal=S - m)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.float().permute(1, 0, 2), k, v, attn_mask=mask, scale=0.11).permute(1, 0, 2)
+    assert (got.float() - ref).abs().max().item() <= 1e-2
+
+
+def test_prefill_rows_are_decode_steps_over_key_prefixes():
+    """With RoPE on, row i of a chunk equals the decode attention (query at the last
+    position) over the first S - m + i + 1 selected keys: pins the query position,
+    the key positions and the causal cut at once against the decode oracle."""
+    q, kp, vp, slots = _prefill_case(seed=1)
+    m, S = q.shape[0], slots.shape[0]
+    got = oracle.prefill.sparse_prefill_attention(q, kp, vp, slots, 0.09, 5e5)
+    for i in (0, 7, m - 1):
+        ref = oracle.attend.sparse_decode_attention(q[i], kp, vp, slots[:S - m + i + 1], 0.09, 5e5)
+        assert (got[i].float() - ref.float()).abs().max().item() <= 1e-2
+    # not causal: every row sees all keys, so the last row is unchanged and the first is not
+    full = oracle.prefill.sparse_prefill_attention(q, kp, vp, slots, 0.09, 5e5, causal=False)
+    assert torch.equal(full[m - 1], got[m - 1])
+    assert (full[0].float() - got[0].float()).abs().max().item() > 1e-3
+
+
+def test_prefill_one_row_chunk_is_the_decode_layer():
+    g = torch.Generator().manual_seed(5)
+    H, Hkv, L = 4, 2, 300
+    kp = torch.randn(L, Hkv, 128, generator=g).bfloat16()
+    vp = torch.randn(L, Hkv, 128, generator=g).bfloat16()
+    q = torch.randn(1, H * 128, generator=g).bfloat16()
+    tab = torch.randperm(L, generator=g).int()
+    slots, out = oracle.prefill.prefill_chunk(q, kp, vp, tab, L, H, 128, 4, 16, 32, 1e4, 1.0, 0.1)
+    ref_slots, ref_out = oracle.layer.decode_layer(q, kp, vp, [tab], [L], H, 128, 4, 16, [32], 1e4,
+                                                   1.0, 0.1)
+    assert torch.equal(slots, ref_slots[0])
+    assert torch.equal(out, ref_out)
+
+
+def test_prefill_fingerprint_is_the_mean_of_rows_rotated_to_consecutive_positions():
+    g = torch.Generator().manual_seed(6)
+    rows, H = 40, 2
+    q = torch.randn(rows, H * 128, generator=g).bfloat16()
+    qf = oracle.rope.scoring_query(q, H, 128, 16, 1e4)
+    x = q.view(rows, H, 128).double()
+    inv = 1.0 / (1e4 ** (torch.arange(0, 128, 2, dtype=torch.float64) / 128))
+    ang = torch.arange(16, 16 + rows, dtype=torch.float64)[:, None] * inv           # [rows, 64]
+    z = torch.complex(x[..., :64], x[..., 64:]) * torch.polar(torch.ones_like(ang), ang)[:, None, :]
+    rot = torch.cat((z.real, z.imag), dim=-1).bfloat16().double()                    # rounded per row
+    ref = rot.mean(dim=0).reshape(-1)
+    assert (qf.double() - ref).abs().max().item() <= 2.0 ** -8 * ref.abs().max().item()
+
+
+def test_prefill_loop_stores_then_selects_chunk_by_chunk():
+    """The extend loop appends each chunk before selecting for it; a later chunk
+    sees the earlier ones among its candidates and every chunk ends with itself."""
+    g = torch.Generator().manual_seed(8)
+    H, Hkv, L0, T, chunk = 4, 2, 200, 70, 32
+    P = L0 + T
+    kp = torch.randn(P, Hkv, 128, generator=g).bfloat16()
+    vp = torch.randn(P, Hkv, 128, generator=g).bfloat16()
+    tab = torch.zeros(P, dtype=torch.int32)
+    tab[:L0] = torch.randperm(L0, generator=g).int()
+    new_slots = (L0 + torch.randperm(T, generator=g)).int()
+    q = torch.randn(T, H * 128, generator=g).bfloat16()
+    k_new = torch.randn(T, Hkv, 128, generator=g).bfloat16()
+    v_new = torch.randn(T, Hkv, 128, generator=g).bfloat16()
+    details = []
+    out = oracle.prefill.prefill(q, k_new, v_new, kp, vp, tab, L0, new_slots, H, 128, 4, chunk, 16,
+                                 1e4, 1.0, 0.1, chunk=chunk, details=details)
+    assert out.shape == (T, H * 128) and len(details) == 3
+    assert torch.equal(tab[L0:], new_slots) and torch.equal(kp[new_slots.long()], k_new)
+    # chunk 2 (rows 32..63) alone, from the final pools and its own context length
+    L2 = L0 + 64
+    _, ref = oracle.prefill.prefill_chunk(q[32:64], kp, vp, tab, L2, H, 128, 4, chunk, 16, 1e4, 1.0,
+                                          0.1)
+    assert torch.equal(out[32:64], ref)
