@@ -211,6 +211,51 @@ int ts_kv_store(const ts_config* cfg, const void* k, const void* v, const int32_
                 int64_t table_stride, int32_t* seq_lens, int32_t batch, int32_t max_tokens,
                 ts_stream_t stream);
 
+/* ---- chunked prefill (patched_radix_attention_extend_forward_flashinfer,
+ * tr.py:703-775): per chunk of at most 512 rows of one request the chunk's K/V
+ * are stored, one selection is made from the mean of the chunk's rotated
+ * queries, and the chunk attends causally over the selected slots. ---- */
+
+/* store_kv_cache(start, end) + add_k_cache for a chunk (tr.py:725-733,
+ * 332-336), page size 1: k_pool[loc[r]] = k[r], v likewise,
+ * table[*seq_len + r] = loc[r] for r < rows, then *seq_len += rows.
+ * k, v: [rows, Hkv, D] bf16; table: the request's row; rows beyond max_tokens
+ * are dropped. */
+int ts_kv_store_chunk(const ts_config* cfg, const void* k, const void* v,
+                      const int32_t* out_cache_loc, int32_t rows, void* k_pool, void* v_pool,
+                      int64_t pool_rows, int32_t* table, int32_t* seq_len, int32_t max_tokens,
+                      ts_stream_t stream);
+
+/* Fingerprint of a chunk (tr.py:380-392): row i of q [rows, H, D] bf16 rotated
+ * with rows n_local + i of the [table_rows, D] fp32 cos / sin tables, rounded
+ * to bf16 (bit-identical to ts_rope_apply), then the mean over the rows, in
+ * fp32, rounded to bf16: qf [H, D]. */
+int ts_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
+                   const float* sin_table, int64_t table_rows, void* qf, ts_stream_t stream);
+
+/* FlashInfer paged prefill over the selected slots with causal=True
+ * (tr.py:759-771), page size 1, one request: query row i of q [rows, H, D] sits
+ * at position S - rows + i (S = *sel_len <= max_sel_len, S >= rows), is rotated
+ * to it, and attends to the keys sel[j], rotated to j, for j <= S - rows + i;
+ * GQA head h reads KV head h / (H/Hkv); sm_scale, logit_cap as in
+ * ts_sparse_decode_attn.  out: [rows, H, D] bf16. */
+int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, const void* k_pool,
+                           const void* v_pool, int64_t pool_rows, const int32_t* sel,
+                           const int32_t* sel_len, int32_t max_sel_len, void* out,
+                           ts_stream_t stream);
+
+/* One chunk of the extend forward after its KV store (tr.py:735-773):
+ * fingerprint -> selection -> causal sparse attention, for the single request
+ * of bt (batch 1; seq_lens[0] already counts the chunk).  rows <= n_local, so
+ * that the chunk's own tokens are the tail of the selected list.  Workspace as
+ * for ts_decode_layer (ts_decode_layer_workspace_bytes(cfg, 1, max_seq_len)).
+ * q, out: [rows, H*D] bf16. */
+int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, int32_t rows,
+                     const float* cos_table, const float* sin_table, int64_t table_rows,
+                     const void* k_pool, const void* v_pool, int64_t pool_rows, void* out,
+                     int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
+                     void* workspace, size_t workspace_bytes, ts_stream_t stream);
+
 /* One layer of patched_radix_attention_decode_forward_flashinfer after the KV
  * store (tr.py:791-825): fingerprint (q rotated with q_cos/q_sin, the [D] table
  * rows of position n_local, tr.py:380-388) -> [selection cache] -> score ->

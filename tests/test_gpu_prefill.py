@@ -1,0 +1,193 @@
+"""GPU parity of the chunked-prefill path against the CPU oracle, through the C ABI:
+chunk fingerprint within one bf16 ulp (fp32 summation order), selection identical
+for the same fingerprint up to ties at the k-th vote, causal sparse attention
+within 2e-2 absolute in bf16."""
+
+import pytest
+import torch
+
+import oracle
+from tokenselect_amd import ops, workloads
+from helpers import assert_index_sets_match, cpu_tabs, say
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    dict(num_heads=32, num_kv_heads=8, rope_theta=5e5),   # Llama-3-8B
+    dict(num_heads=28, num_kv_heads=4, rope_theta=1e6),   # Qwen2-7B
+    dict(num_heads=8, num_kv_heads=1, rope_theta=1e4),
+    dict(num_heads=4, num_kv_heads=2, rope_theta=1e4),
+    dict(num_heads=8, num_kv_heads=8, rope_theta=1e4),
+]
+IDS = [f"H{s['num_heads']}kv{s['num_kv_heads']}" for s in SHAPES]
+
+
+def _sm(c):
+    return c.sm_scale if c.sm_scale is not None else c.head_dim ** -0.5
+
+
+@pytest.mark.parametrize("rows", [1, 37, 512])
+def test_fingerprint(dev, rows):
+    say(f"chunk fingerprint rows={rows}")
+    g = torch.Generator().manual_seed(rows)
+    H, n_local = 6, 40
+    cfg = ops.LayerConfig(num_heads=8, num_kv_heads=8, n_local=n_local, rope_theta=5e5)
+    q = torch.randn(rows, 8, 128, generator=g).bfloat16()
+    cos, sin = ops.rope_tables(128, 5e5, 1.0, n_local + rows, dev)
+    got = ops.fingerprint(cfg, q.to(dev), cos, sin).cpu().float().reshape(-1)
+    ref = oracle.rope.scoring_query(q.view(rows, -1), 8, 128, n_local, 5e5).float()
+    ulp = ref.abs().clamp_min(2.0 ** -126) * 2.0 ** -7
+    assert bool(((got - ref).abs() <= ulp).all())
+    if rows == 1:  # the mean of one row is the row: bit-exact
+        assert torch.equal(got, ref)
+    assert (got != ref).float().mean().item() < 0.05
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=IDS)
+@pytest.mark.parametrize("rope_mode", ["ROPE_LLAMA", "NONE"])
+def test_sparse_prefill_attention(dev, shape, rope_mode):
+    m, S = 77, 413   # ragged tile edges on both axes
+    say(f"prefill attention H={shape['num_heads']} Hkv={shape['num_kv_heads']} m={m} S={S} {rope_mode}")
+    wl = workloads.build("pf", shape, [S + 50], [64], 1, dev, seed=3, n_init=8, n_local=m)
+    c = wl.cfg
+    c.rope_mode = rope_mode
+    g = torch.Generator(device=dev).manual_seed(4)
+    q = torch.randn((m, c.num_heads * 128), generator=g, device=dev).bfloat16()
+    sel = wl.table[0, torch.randperm(S + 50, generator=g, device=dev)[:S].long()].contiguous()
+    sel_len = torch.tensor([S], dtype=torch.int32, device=dev)
+    out = ops.sparse_prefill_attention(c, q, wl.k_pool, wl.v_pool, sel, sel_len)
+    torch.cuda.synchronize()
+    ref = oracle.prefill.sparse_prefill_attention(q.cpu().view(m, c.num_heads, 128), wl.k_pool.cpu(),
+                                                  wl.v_pool.cpu(), sel.cpu(), _sm(c), c.rope_theta,
+                                                  c.rope_scale, c.logit_cap, rope_mode)
+    err = (out.cpu().float() - ref.reshape(m, -1).float()).abs().max().item()
+    assert err <= 2e-2, err
+
+
+def test_sparse_prefill_attention_full_chunk_and_soft_cap(dev):
+    """A whole 512-row chunk over the selected-list length of the served configs, the
+    chunk starting exactly at S - m; and the soft cap."""
+    m, S = 512, 2688
+    say(f"prefill attention m={m} S={S} (+ soft cap)")
+    wl = workloads.build("pf", SHAPES[0], [S], [64], 1, dev, seed=5, n_init=8, n_local=m)
+    for cap in (0.0, 30.0):
+        c = wl.cfg
+        c.logit_cap = cap
+        g = torch.Generator(device=dev).manual_seed(6)
+        q = (3.0 * torch.randn((m, c.num_heads * 128), generator=g, device=dev)).bfloat16()
+        sel = wl.table[0, :S].contiguous()
+        sel_len = torch.tensor([S], dtype=torch.int32, device=dev)
+        out = ops.sparse_prefill_attention(c, q, wl.k_pool, wl.v_pool, sel, sel_len)
+        torch.cuda.synchronize()
+        rows = torch.tensor([0, 1, 15, 16, 255, 300, 511])
+        ref = oracle.prefill.sparse_prefill_attention(
+            q.cpu().view(m, c.num_heads, 128), wl.k_pool.cpu(), wl.v_pool.cpu(), sel.cpu(), _sm(c),
+            c.rope_theta, c.rope_scale, cap, c.rope_mode)
+        err = (out.cpu().float().view(m, -1)[rows] - ref.reshape(m, -1).float()[rows]).abs().max().item()
+        assert err <= 2e-2, (cap, err)
+
+
+def test_kv_store_chunk(dev):
+    say("kv_store_chunk")
+    wl = workloads.build("pf", SHAPES[0], [100], [16], 1, dev, seed=7, n_init=4, n_local=16,
+                         extra_pages=64)
+    c = wl.cfg
+    g = torch.Generator(device=dev).manual_seed(8)
+    rows = 40
+    k = torch.randn((rows, c.num_kv_heads, 128), generator=g, device=dev).bfloat16()
+    v = torch.randn((rows, c.num_kv_heads, 128), generator=g, device=dev).bfloat16()
+    loc = (100 + torch.randperm(64, generator=g, device=dev)[:rows]).int()
+    table = torch.zeros(200, dtype=torch.int32, device=dev)
+    table[:100] = wl.table[0, :100]
+    seq = torch.tensor([100], dtype=torch.int32, device=dev)
+    ops.kv_store_chunk(c, k, v, loc, wl.k_pool, wl.v_pool, table, seq)
+    torch.cuda.synchronize()
+    assert int(seq) == 140
+    assert torch.equal(table[100:140], loc)
+    assert torch.equal(wl.k_pool[loc.long()], k) and torch.equal(wl.v_pool[loc.long()], v)
+    assert torch.equal(table[:100], wl.table[0, :100])
+
+
+@pytest.mark.parametrize("shape", SHAPES[:2], ids=IDS[:2])
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "separate"])
+def test_prefill_chunks(dev, shape, fused):
+    """Three chunks of an extend forward (the last one ragged) on top of an existing
+    context: store, fingerprint, selection, causal attention, chunk by chunk."""
+    previous = ops.set_fused_select(fused)
+    try:
+        L0, T, chunk, top_k = 3000, 150, 64, 96
+        say(f"prefill chunks H={shape['num_heads']} L0={L0} T={T} chunk={chunk} fused={fused}")
+        wl = workloads.build("pf", shape, [L0], [top_k], 1, dev, seed=11, n_init=8, n_local=chunk,
+                             top_k=top_k, extra_pages=T)
+        c = wl.cfg
+        g = torch.Generator(device=dev).manual_seed(12)
+        q = torch.randn((T, c.num_heads * 128), generator=g, device=dev).bfloat16()
+        k_new = torch.randn((T, c.num_kv_heads, 128), generator=g, device=dev).bfloat16()
+        v_new = torch.randn((T, c.num_kv_heads, 128), generator=g, device=dev).bfloat16()
+        new_slots = (L0 + torch.randperm(T, generator=g, device=dev)).int()
+        table = torch.zeros((1, L0 + T), dtype=torch.int32, device=dev)
+        table[0, :L0] = wl.table[0, :L0]
+        seq = wl.seq_lens_dev.clone()
+        layer = ops.PrefillChunk(c, L0 + T, dev, max_rows=chunk)
+
+        kc, vc, tab_cpu = wl.k_pool.cpu(), wl.v_pool.cpu(), table[0].cpu()
+        L = L0
+        for start in range(0, T, chunk):
+            end = min(start + chunk, T)
+            m = end - start
+            ops.kv_store_chunk(c, k_new[start:end], v_new[start:end], new_slots[start:end].contiguous(),
+                               wl.k_pool, wl.v_pool, table[0], seq)
+            L += m
+            out, sel, sel_pos, sel_len = layer(q[start:end].contiguous(), wl.k_pool, wl.v_pool,
+                                               ops.Batch(seq, table, L))
+            torch.cuda.synchronize()
+            # oracle on the same pools, following the device's fingerprint
+            loc = new_slots[start:end].cpu().long()
+            kc[loc], vc[loc] = k_new[start:end].cpu(), v_new[start:end].cpu()
+            tab_cpu[L - m:L] = new_slots[start:end].cpu()
+            qf = ops.fingerprint(c, q[start:end].view(m, c.num_heads, 128).contiguous(),
+                                 layer.cos, layer.sin).cpu()
+            d = {}
+            ref_slots, ref_out = oracle.prefill.prefill_chunk(
+                q[start:end].cpu(), kc, vc, tab_cpu, L, c.num_heads, 128, c.n_init, c.n_local, top_k,
+                c.rope_theta, c.rope_scale, _sm(c), detail=d, qf_override=qf)
+            S = int(sel_len[0])
+            assert S == ref_slots.shape[0] == c.n_init + top_k + c.n_local
+            pos = sel_pos[0, :S].cpu()
+            assert_index_sets_match(pos[c.n_init:c.n_init + top_k], d["top_pos"], d["votes"], c.n_init,
+                                    f"chunk at {start}")
+            assert pos[-m:].tolist() == list(range(L - m, L))     # the chunk is the tail
+            assert torch.equal(sel[0, :S].cpu(), tab_cpu[pos.long()])
+            if torch.equal(sel[0, :S].cpu(), ref_slots):
+                err = (out.cpu().float() - ref_out.float()).abs().max().item()
+                assert err <= 2e-2, (start, err)
+    finally:
+        ops.set_fused_select(previous)
+
+
+def test_prefill_short_context_attends_densely(dev):
+    """n_init + k + n_local >= L: the chunk attends over every token so far (tr.py:741-744)."""
+    say("prefill chunk, dense context")
+    L0, m = 40, 24
+    wl = workloads.build("pf", SHAPES[3], [L0 + m], [64], 1, dev, seed=13, n_init=8, n_local=32,
+                         top_k=64)
+    c = wl.cfg
+    g = torch.Generator(device=dev).manual_seed(14)
+    q = torch.randn((m, c.num_heads * 128), generator=g, device=dev).bfloat16()
+    layer = ops.PrefillChunk(c, L0 + m, dev, max_rows=32)
+    out, sel, sel_pos, sel_len = layer(q, wl.k_pool, wl.v_pool, wl.batch)
+    torch.cuda.synchronize()
+    tab = cpu_tabs(wl)[0]
+    assert int(sel_len[0]) == L0 + m
+    assert torch.equal(sel[0, :L0 + m].cpu(), tab[:L0 + m])
+    ref = oracle.prefill.sparse_prefill_attention(q.cpu().view(m, c.num_heads, 128), wl.k_pool.cpu(),
+                                                  wl.v_pool.cpu(), tab[:L0 + m], _sm(c), c.rope_theta)
+    assert (out.cpu().float() - ref.reshape(m, -1).float()).abs().max().item() <= 2e-2
+
+
+def test_prefill_chunk_rejects_rows_beyond_the_local_window(dev):
+    wl = workloads.build("pf", SHAPES[3], [500], [16], 1, dev, seed=15, n_init=4, n_local=16)
+    layer = ops.PrefillChunk(wl.cfg, 500, dev, max_rows=64)
+    q = torch.zeros((32, wl.cfg.num_heads * 128), dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="local window"):
+        layer(q, wl.k_pool, wl.v_pool, wl.batch)

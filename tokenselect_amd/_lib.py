@@ -72,6 +72,11 @@ SIGNATURES = {
                                      _ptr, _ptr, _size, _ptr]),
     "ts_kv_store": (_i32, [_CFG, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
                            _ptr]),
+    "ts_kv_store_chunk": (_i32, [_CFG, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i32, _ptr]),
+    "ts_fingerprint": (_i32, [_CFG, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr]),
+    "ts_sparse_prefill_attn": (_i32, [_CFG, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i32, _ptr, _ptr]),
+    "ts_prefill_chunk": (_i32, [_CFG, _BT, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i64, _ptr, _ptr,
+                                _ptr, _i64, _ptr, _ptr, _size, _ptr]),
     "ts_set_fused_select": (_i32, [_i32]),
     "ts_decode_layer_workspace_bytes": (_size, [_CFG, _i32, _i32]),
     "ts_decode_layer": (_i32, [_CFG, _BT, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _SC, _ptr, _ptr,

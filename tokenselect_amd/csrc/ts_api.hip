@@ -141,15 +141,19 @@ size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int3
   return layer_workspace(cfg, batch, max_seq_len).total;
 }
 
-int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, const float* q_cos,
-                    const float* q_sin, const void* k_pool, const void* v_pool,
-                    int64_t pool_rows, const ts_selcache* cache, void* out, int32_t* sel,
-                    int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
-                    size_t workspace_bytes, ts_stream_t stream) {
+// Decode (chunk_rows == 0: one query row per request, q_cos / q_sin are the [D] rows
+// of position n_local) or one prefill chunk of a single request (chunk_rows > 0:
+// q_cos / q_sin are the whole [table_rows, D] tables).
+static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, int32_t chunk_rows,
+                     const float* q_cos, const float* q_sin, int64_t table_rows,
+                     const void* k_pool, const void* v_pool, int64_t pool_rows,
+                     const ts_selcache* cache, void* out, int32_t* sel, int32_t* sel_pos,
+                     int64_t sel_stride, int32_t* sel_len, void* workspace, size_t workspace_bytes,
+                     ts_stream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
   TS_REQUIRE(q && q_cos && q_sin && k_pool && v_pool && out && sel && sel_pos && sel_len, TS_EINVAL,
-             "ts_decode_layer: NULL tensor argument");
+             "layer: NULL tensor argument");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);
@@ -179,8 +183,18 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
   ZeroRegion zero_counters, zero_sync;
   if (fused.tokens_per_block > 0)
     select_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_counters, &zero_sync);
-  TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
-                     zero_counters, zero_sync, (hipStream_t)stream));
+  if (chunk_rows > 0) {
+    // Chunk fingerprint: row i rotated to n_local + i, mean over the rows (tr.py:380-392).
+    TS_TRY(ts_fingerprint(cfg, q, chunk_rows, q_cos, q_sin, table_rows, qf, stream));
+    if (fused.tokens_per_block > 0) {
+      hipLaunchKernelGGL(select_zero_kernel, dim3(8), dim3(256), 0, (hipStream_t)stream,
+                         zero_counters, zero_sync);
+      TS_TRY(check_launch("select_zero_kernel"));
+    }
+  } else {
+    TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
+                       zero_counters, zero_sync, (hipStream_t)stream));
+  }
   if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
   if (fused.tokens_per_block > 0) {
     TS_TRY(launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,
@@ -198,9 +212,37 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
     topk.clear_per_req = cfg->num_kv_heads;
     TS_TRY(launch_topk(topk, bt->batch, max_n, (hipStream_t)stream));
   }
-  TS_TRY(launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, bt->batch,
-                     w.max_sel, out, ws + w.attn_ws, /*tickets_clear=*/true, (hipStream_t)stream));
-  return TS_OK;
+  if (chunk_rows > 0)
+    return ts_sparse_prefill_attn(cfg, q, chunk_rows, k_pool, v_pool, pool_rows, sel, sel_len,
+                                  w.max_sel, out, stream);
+  return launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, bt->batch,
+                     w.max_sel, out, ws + w.attn_ws, /*tickets_clear=*/true, (hipStream_t)stream);
+}
+
+int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, const float* q_cos,
+                    const float* q_sin, const void* k_pool, const void* v_pool,
+                    int64_t pool_rows, const ts_selcache* cache, void* out, int32_t* sel,
+                    int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
+                    size_t workspace_bytes, ts_stream_t stream) {
+  return run_layer(cfg, bt, q, 0, q_cos, q_sin, 1, k_pool, v_pool, pool_rows, cache, out, sel,
+                   sel_pos, sel_stride, sel_len, workspace, workspace_bytes, stream);
+}
+
+int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, int32_t rows,
+                     const float* cos_table, const float* sin_table, int64_t table_rows,
+                     const void* k_pool, const void* v_pool, int64_t pool_rows, void* out,
+                     int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
+                     void* workspace, size_t workspace_bytes, ts_stream_t stream) {
+  TS_REQUIRE(bt != nullptr && bt->batch == 1, TS_EINVAL,
+             "ts_prefill_chunk serves one request at a time (batch must be 1)");
+  TS_REQUIRE(rows >= 1, TS_EINVAL, "ts_prefill_chunk: rows %d < 1", rows);
+  TS_REQUIRE(cfg != nullptr && cfg->n_local >= rows, TS_EINVAL,
+             "ts_prefill_chunk: the chunk (%d rows) must lie inside the local window (n_local %d), "
+             "otherwise its own tokens are not all attended to",
+             rows, cfg ? cfg->n_local : 0);
+  return run_layer(cfg, bt, q, rows, cos_table, sin_table, table_rows, k_pool, v_pool, pool_rows,
+                   nullptr, out, sel, sel_pos, sel_stride, sel_len, workspace, workspace_bytes,
+                   stream);
 }
 
 }  // extern "C"

@@ -47,17 +47,6 @@ __device__ __forceinline__ void unpack8(const uint4& w, float (&f)[8]) {
   f[7] = bf16_hi(w.w);
 }
 
-// sin and cos of an angle of up to some 1e5 radians: two-constant reduction by
-// 2 pi (hi + lo parts, each product exact inside the FMA), then the hardware
-// functions on [-pi, pi].
-__device__ __forceinline__ void sincos_reduced(float x, float& sn, float& cs) {
-  const float k = rintf(x * 0.15915494309189535f);
-  float r = fmaf(-k, 6.2831854820251465f, x);
-  r = fmaf(-k, -1.7484555e-07f, r);
-  sn = __sinf(r);
-  cs = __cosf(r);
-}
-
 __device__ __forceinline__ float2 load_coherent2(const float* p) {
   const uint64_t v =
       __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

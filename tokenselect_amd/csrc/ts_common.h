@@ -87,6 +87,17 @@ __device__ __forceinline__ float row16_sum(float x) {
   return x;
 }
 
+// sin and cos of an angle of up to some 1e5 radians: two-constant reduction by
+// 2 pi (hi + lo parts, each product exact inside the FMA), then the hardware
+// functions on [-pi, pi].
+__device__ __forceinline__ void sincos_reduced(float x, float& sn, float& cs) {
+  const float k = rintf(x * 0.15915494309189535f);
+  float r = fmaf(-k, 6.2831854820251465f, x);
+  r = fmaf(-k, -1.7484555e-07f, r);
+  sn = __sinf(r);
+  cs = __cosf(r);
+}
+
 // Merge two (max, sum-of-exp) softmax partials.
 __device__ __forceinline__ void softmax_merge(float& m, float& l, float m2, float l2) {
   float mm = fmaxf(m, m2);

@@ -1,0 +1,362 @@
+// Chunked prefill (patched_radix_attention_extend_forward_flashinfer, tr.py:703-775):
+// the fingerprint of a chunk (mean of its rotated query rows, tr.py:380-392) and the
+// causal attention of the chunk's rows over the selected KV slots (FlashInfer paged
+// prefill, tr.py:759-771, page size 1, in-kernel Llama RoPE).
+#include <math.h>
+
+#include "ts_common.h"
+
+namespace ts {
+
+// ------------------------------------------------------------------ fingerprint
+// One workgroup per head, 1024 threads = 64 rotation pairs x 16 row groups.  Row r
+// is rotated with table row first_pos + r exactly like the rotation kernel (every
+// product and sum rounded on its own, result rounded to bf16, tr.py:104-107); the
+// bf16 values are summed in fp32, row group by row group in a fixed order, divided
+// by the row count and rounded to bf16 (torch.mean on a bf16 tensor, tr.py:392).
+constexpr int kFpRowGroups = 16;
+
+__global__ __launch_bounds__(1024) void fingerprint_kernel(
+    const uint16_t* __restrict__ q, uint16_t* __restrict__ qf, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, int64_t table_rows, int first_pos, int rows, int heads) {
+#pragma clang fp contract(off)
+  constexpr int half = kHeadDim / 2;
+  const int h = blockIdx.x;
+  const int i = threadIdx.x % half, rg = threadIdx.x / half;
+  float lo_sum = 0.f, hi_sum = 0.f;
+  for (int r = rg; r < rows; r += kFpRowGroups) {
+    int64_t pos = (int64_t)first_pos + r;
+    pos = pos < table_rows ? pos : table_rows - 1;
+    const float* c = cos_table + pos * kHeadDim;
+    const float* s = sin_table + pos * kHeadDim;
+    const size_t base = ((size_t)r * heads + h) * kHeadDim;
+    const float x1 = bf16_to_f32(q[base + i]);
+    const float x2 = bf16_to_f32(q[base + i + half]);
+    const float lo = x1 * c[i] + (-x2) * s[i];
+    const float hi = x2 * c[i + half] + x1 * s[i + half];
+    lo_sum += bf16_to_f32(f32_to_bf16(lo));
+    hi_sum += bf16_to_f32(f32_to_bf16(hi));
+  }
+  __shared__ float part[kFpRowGroups][kHeadDim];
+  part[rg][i] = lo_sum;
+  part[rg][i + half] = hi_sum;
+  __syncthreads();
+  if (threadIdx.x < kHeadDim) {
+    float total = 0.f;
+    for (int g = 0; g < kFpRowGroups; ++g) total += part[g][threadIdx.x];
+    qf[(size_t)h * kHeadDim + threadIdx.x] = f32_to_bf16(total / (float)rows);
+  }
+}
+
+// ------------------------------------------------------------ prefill attention
+// Grid (16-row query tiles, KV heads, quads of the G query heads of a KV head);
+// four wavefronts, one query head each, share the K/V tiles of their KV head.
+//
+// Per 32-key tile: 256 threads gather the 32 K rows and V rows of the KV head (the
+// next tile's rows are requested before the current one is used), rotate the keys
+// to their index in the selected list and write K row-major and V transposed into
+// LDS.  A wavefront then computes S^T = K Q^T with v_mfma_f32_16x16x32_bf16 (A = 16
+// keys x 32 dims from LDS, B = its 16 rotated queries, held in registers), which
+// leaves lane (query l%16, key group l/16) with the logits of 8 keys; the online
+// softmax needs two cross-lane maxima per tile; the 8 probabilities, rounded to
+// bf16, are directly the B operand of O^T += V^T P^T (A = 16 dims x 32 keys from the
+// transposed V tile, keys in the order the logits came in), so no data moves
+// between the two products.  fp32 accumulation throughout.
+struct PrefillArgs {
+  const uint16_t* q;  // [rows, H, 128] bf16, un-rotated
+  const uint16_t* k_pool;
+  const uint16_t* v_pool;
+  uint32_t pool_rows;
+  const int32_t* sel;      // [S] selected slots in attention order
+  const int32_t* sel_len;  // device scalar S
+  int max_sel_len;
+  int rows;
+  int num_heads, num_kv_heads, rope_mode;
+  float log2_theta, rope_rcp_scale, sm_scale, logit_cap;
+  uint16_t* out;  // [rows, H, 128] bf16
+};
+
+typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float pf_f32x4;
+
+constexpr int kPfKeys = 32;               // keys per tile
+constexpr int kPfKRow = kHeadDim + 8;     // halfwords per K row in LDS (272 B: rows on different banks)
+constexpr int kPfVRow = kPfKeys + 4;      // halfwords per V^T row in LDS (72 B)
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+template <int G>
+__global__ __launch_bounds__(256) void prefill_attn_kernel(PrefillArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[kPfKeys * kPfKRow];
+  __shared__ __attribute__((aligned(16))) uint16_t vt_lds[kHeadDim * kPfVRow];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int qc = lane & 15, g4 = lane >> 4;  // query column / key group of the MFMA layouts
+  const int kvh = blockIdx.y;
+  const int head_in_group = blockIdx.z * 4 + wave;
+  const bool wave_active = head_in_group < G;
+  const int h = kvh * G + (wave_active ? head_in_group : 0);
+  const int H = a.num_heads;
+  const int S = min(max(*a.sel_len, 0), a.max_sel_len);
+  const int m = a.rows;
+  const int q_row0 = blockIdx.x * 16;
+  const int shift = S - m;  // query row i sits at position shift + i and sees keys <= that
+  const bool rope = a.rope_mode == TS_ROPE_LLAMA;
+  if (S < m || S <= 0) return;  // fewer keys than rows: not a prefill chunk
+
+  // ---- queries: B operand, lane (qc, g4) holds dims [32 ks + 8 g4, +8) of row q_row0 + qc,
+  // rotated to position shift + row (partner dims d and d + 64 are k-steps ks and ks + 2).
+  const int q_row = min(q_row0 + qc, m - 1);
+  pf_bf16x8 qb[4];
+  {
+    float x[4][8];
+    const uint16_t* qrow = a.q + ((size_t)q_row * H + h) * kHeadDim;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const uint4 w = *(const uint4*)(qrow + 32 * ks + 8 * g4);
+      const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x[ks][2 * e] = bf16_lo(ww[e]);
+        x[ks][2 * e + 1] = bf16_hi(ww[e]);
+      }
+    }
+    if (rope) {
+      const float pos = (float)(shift + q_row);
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int pair = 32 * ks + 8 * g4 + e;
+          const float freq = a.rope_rcp_scale * exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
+          float sn, cs;
+          sincos_reduced(pos * freq, sn, cs);
+          const float lo = x[ks][e], hi = x[ks + 2][e];
+          x[ks][e] = lo * cs - hi * sn;
+          x[ks + 2][e] = hi * cs + lo * sn;
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const uint4 w = make_uint4(pack_bf16(x[ks][0], x[ks][1]), pack_bf16(x[ks][2], x[ks][3]),
+                                 pack_bf16(x[ks][4], x[ks][5]), pack_bf16(x[ks][6], x[ks][7]));
+      qb[ks] = __builtin_bit_cast(pf_bf16x8, w);
+    }
+  }
+
+  // ---- staging role: thread (key kk, chunk c) moves dims [8c, 8c+8) and [64+8c, +8) of
+  // key j = tile + kk; its rotation state advances by one tile (32 positions) per step.
+  const int kk = tid >> 3, c8 = tid & 7;
+  float kc[8], ksn[8], dc[8], ds[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    kc[e] = 1.f;
+    ksn[e] = 0.f;
+    dc[e] = 1.f;
+    ds[e] = 0.f;
+    if (rope) {
+      const int pair = 8 * c8 + e;
+      const float freq = a.rope_rcp_scale * exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
+      sincos_reduced((float)kk * freq, ksn[e], kc[e]);
+      sincos_reduced((float)kPfKeys * freq, ds[e], dc[e]);
+    }
+  }
+  const size_t row_elems = (size_t)a.num_kv_heads * kHeadDim;
+  uint4 kraw[2], vraw[2];
+  auto request_tile = [&](int tile) {
+    const int j = min(tile + kk, S - 1);
+    uint32_t slot = (uint32_t)a.sel[j];
+    slot = slot < a.pool_rows ? slot : a.pool_rows - 1;
+    const size_t at = (size_t)slot * row_elems + (size_t)kvh * kHeadDim + 8 * c8;
+    kraw[0] = *(const uint4*)(a.k_pool + at);
+    kraw[1] = *(const uint4*)(a.k_pool + at + 64);
+    vraw[0] = *(const uint4*)(a.v_pool + at);
+    vraw[1] = *(const uint4*)(a.v_pool + at + 64);
+  };
+  auto stage_tile = [&]() {
+    const uint32_t klo[4] = {kraw[0].x, kraw[0].y, kraw[0].z, kraw[0].w};
+    const uint32_t khi[4] = {kraw[1].x, kraw[1].y, kraw[1].z, kraw[1].w};
+    float lo[8], hi[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      lo[2 * e] = bf16_lo(klo[e]);
+      lo[2 * e + 1] = bf16_hi(klo[e]);
+      hi[2 * e] = bf16_lo(khi[e]);
+      hi[2 * e + 1] = bf16_hi(khi[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float l2 = lo[e] * kc[e] - hi[e] * ksn[e];
+      const float h2 = hi[e] * kc[e] + lo[e] * ksn[e];
+      lo[e] = l2;
+      hi[e] = h2;
+      const float c2 = kc[e] * dc[e] - ksn[e] * ds[e];  // advance to the next tile
+      ksn[e] = ksn[e] * dc[e] + kc[e] * ds[e];
+      kc[e] = c2;
+    }
+    *(uint4*)(k_lds + kk * kPfKRow + 8 * c8) =
+        make_uint4(pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]), pack_bf16(lo[4], lo[5]),
+                   pack_bf16(lo[6], lo[7]));
+    *(uint4*)(k_lds + kk * kPfKRow + 64 + 8 * c8) =
+        make_uint4(pack_bf16(hi[0], hi[1]), pack_bf16(hi[2], hi[3]), pack_bf16(hi[4], hi[5]),
+                   pack_bf16(hi[6], hi[7]));
+    const uint32_t vlo[4] = {vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w};
+    const uint32_t vhi[4] = {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      vt_lds[(8 * c8 + 2 * e) * kPfVRow + kk] = (uint16_t)(vlo[e] & 0xffffu);
+      vt_lds[(8 * c8 + 2 * e + 1) * kPfVRow + kk] = (uint16_t)(vlo[e] >> 16);
+      vt_lds[(64 + 8 * c8 + 2 * e) * kPfVRow + kk] = (uint16_t)(vhi[e] & 0xffffu);
+      vt_lds[(64 + 8 * c8 + 2 * e + 1) * kPfVRow + kk] = (uint16_t)(vhi[e] >> 16);
+    }
+  };
+
+  // ---- main loop over the tiles any row of this query tile can see
+  const int last_visible = min(S - 1, shift + min(q_row0 + 15, m - 1));
+  const int my_limit = shift + q_row;  // last key this lane's query sees
+  float m_run = kNegBig, l_run = 0.f;
+  pf_f32x4 o[8];
+#pragma unroll
+  for (int db = 0; db < 8; ++db) o[db] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  request_tile(0);
+  for (int tile = 0; tile <= last_visible; tile += kPfKeys) {
+    __syncthreads();  // the previous tile's LDS reads are done
+    stage_tile();
+    if (tile + kPfKeys <= last_visible) request_tile(tile + kPfKeys);
+    __syncthreads();
+    if (!wave_active) continue;
+
+    // logits: s[blk][r] belongs to key tile + 16 blk + 4 g4 + r and query qc
+    float s[2][4];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      pf_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const uint4 kw = *(const uint4*)(k_lds + (16 * blk + qc) * kPfKRow + 32 * ks + 8 * g4);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, kw), qb[ks], acc,
+                                                      0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float x = acc[r] * a.sm_scale;
+        if (a.logit_cap > 0.f) x = a.logit_cap * tanhf(x / a.logit_cap);
+        const int key = tile + 16 * blk + 4 * g4 + r;
+        s[blk][r] = key <= my_limit ? x : kNegBig;
+      }
+    }
+    float mx = kNegBig;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[blk][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __expf(m_run - m_new);
+    float p[2][4], psum = 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        p[blk][r] = s[blk][r] > 0.5f * kNegBig ? __expf(s[blk][r] - m_new) : 0.f;
+        psum += p[blk][r];
+      }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    const uint4 pw = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]),
+                                pack_bf16(p[1][0], p[1][1]), pack_bf16(p[1][2], p[1][3]));
+    const pf_bf16x8 pb = __builtin_bit_cast(pf_bf16x8, pw);
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      const uint16_t* vrow = vt_lds + (16 * db + qc) * kPfVRow;
+      const uint2 v0 = *(const uint2*)(vrow + 4 * g4);
+      const uint2 v1 = *(const uint2*)(vrow + 16 + 4 * g4);
+      const uint4 vw = make_uint4(v0.x, v0.y, v1.x, v1.y);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[db][r] *= alpha;
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw), pb, o[db],
+                                                      0, 0, 0);
+    }
+  }
+  if (!wave_active || q_row0 + qc >= m) return;
+
+  // o[db][r] = O[query qc][dim 16 db + 4 g4 + r]; the row sum is spread over the 4 key groups.
+  float l_tot = l_run + __shfl_xor(l_run, 16);
+  l_tot += __shfl_xor(l_tot, 32);
+  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  uint16_t* orow = a.out + ((size_t)(q_row0 + qc) * H + h) * kHeadDim;
+#pragma unroll
+  for (int db = 0; db < 8; ++db)
+    *(uint2*)(orow + 16 * db + 4 * g4) = make_uint2(pack_bf16(o[db][0] * inv, o[db][1] * inv),
+                                                    pack_bf16(o[db][2] * inv, o[db][3] * inv));
+}
+
+}  // namespace ts
+
+using namespace ts;
+
+extern "C" {
+
+int ts_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
+                   const float* sin_table, int64_t table_rows, void* qf, ts_stream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_REQUIRE(q && cos_table && sin_table && qf, TS_EINVAL, "ts_fingerprint: NULL tensor argument");
+  TS_REQUIRE(rows >= 1, TS_EINVAL, "ts_fingerprint: rows %d < 1", rows);
+  TS_REQUIRE(table_rows >= (int64_t)cfg->n_local + rows, TS_EINVAL,
+             "ts_fingerprint: cos/sin tables have %lld rows, need n_local + rows = %lld",
+             (long long)table_rows, (long long)cfg->n_local + rows);
+  hipLaunchKernelGGL(fingerprint_kernel, dim3((unsigned)cfg->num_heads), dim3(1024), 0,
+                     (hipStream_t)stream, (const uint16_t*)q, (uint16_t*)qf, cos_table, sin_table,
+                     table_rows, cfg->n_local, rows, cfg->num_heads);
+  return check_launch("fingerprint_kernel");
+}
+
+int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, const void* k_pool,
+                           const void* v_pool, int64_t pool_rows, const int32_t* sel,
+                           const int32_t* sel_len, int32_t max_sel_len, void* out,
+                           ts_stream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_REQUIRE(q && k_pool && v_pool && sel && sel_len && out, TS_EINVAL,
+             "ts_sparse_prefill_attn: NULL tensor argument");
+  TS_REQUIRE(rows >= 1 && rows <= 65535 * 16, TS_EINVAL, "rows %d out of range", rows);
+  TS_REQUIRE(max_sel_len >= rows, TS_EINVAL,
+             "max_sel_len %d < rows %d: a chunk attends at least to itself", max_sel_len, rows);
+  TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
+             (long long)pool_rows);
+  PrefillArgs a;
+  a.q = (const uint16_t*)q;
+  a.k_pool = (const uint16_t*)k_pool;
+  a.v_pool = (const uint16_t*)v_pool;
+  a.pool_rows = (uint32_t)pool_rows;
+  a.sel = sel;
+  a.sel_len = sel_len;
+  a.max_sel_len = max_sel_len;
+  a.rows = rows;
+  a.num_heads = cfg->num_heads;
+  a.num_kv_heads = cfg->num_kv_heads;
+  a.rope_mode = cfg->rope_mode;
+  a.log2_theta = cfg->rope_mode == TS_ROPE_LLAMA ? (float)log2((double)cfg->rope_theta) : 0.f;
+  a.rope_rcp_scale = cfg->rope_mode == TS_ROPE_LLAMA ? 1.0f / cfg->rope_scale : 1.0f;
+  a.sm_scale = cfg->sm_scale;
+  a.logit_cap = cfg->logit_cap;
+  a.out = (uint16_t*)out;
+  const int group = cfg->num_heads / cfg->num_kv_heads;
+  const dim3 grid((unsigned)ceil_div(rows, 16), (unsigned)cfg->num_kv_heads,
+                  (unsigned)ceil_div(group, 4));
+  hipStream_t st = (hipStream_t)stream;
+  switch (group) {
+    case 1: hipLaunchKernelGGL(prefill_attn_kernel<1>, grid, dim3(256), 0, st, a); break;
+    case 2: hipLaunchKernelGGL(prefill_attn_kernel<2>, grid, dim3(256), 0, st, a); break;
+    case 4: hipLaunchKernelGGL(prefill_attn_kernel<4>, grid, dim3(256), 0, st, a); break;
+    case 7: hipLaunchKernelGGL(prefill_attn_kernel<7>, grid, dim3(256), 0, st, a); break;
+    case 8: hipLaunchKernelGGL(prefill_attn_kernel<8>, grid, dim3(256), 0, st, a); break;
+    default: return fail(TS_ESHAPE, "unsupported head group %d", group);
+  }
+  return check_launch("prefill_attn_kernel");
+}
+
+}  // extern "C"

@@ -67,6 +67,9 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
 void select_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* counters,
                          ZeroRegion* sync);
 
+// Clears two regions (the stand-alone form of what the rotation kernel does on the side).
+__global__ void select_zero_kernel(ZeroRegion r0, ZeroRegion r1);
+
 // Launch without the clearing pass: the regions above are known to be zero.
 int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
                   int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,

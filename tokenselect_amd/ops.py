@@ -461,3 +461,119 @@ class DecodeLayer:
             _p(self.sel), _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
             self.workspace.numel(), _stream()))
         return out, self.sel, self.sel_pos, self.sel_len
+
+
+# ---------------------------------------------------------------- chunked prefill
+def rope_tables(head_dim: int, rope_base: float, rope_scale, rows: int, device):
+    """The reference's cos/sin tables (tr.py:75-96) for positions ``0..rows-1``, built
+    with the same fp32 torch expressions on the host: ``(cos [rows,D], sin [rows,D])``."""
+    inv_freq = 1.0 / (rope_base ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    freqs = torch.outer(torch.arange(rows) * rope_scale, inv_freq)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.cos().to(device).contiguous(), emb.sin().to(device).contiguous()
+
+
+def kv_store_chunk(cfg: LayerConfig, k: torch.Tensor, v: torch.Tensor, out_cache_loc: torch.Tensor,
+                   k_pool: torch.Tensor, v_pool: torch.Tensor, table_row: torch.Tensor,
+                   seq_len: torch.Tensor) -> None:
+    """KV store + table append of a prefill chunk of one request (tr.py:725-733,
+    332-336): ``table_row`` [max_tokens] int32, ``seq_len`` a one-element int32 tensor."""
+    c = cfg.to_c()
+    _need(k, "k", torch.bfloat16)
+    _need(v, "v", torch.bfloat16)
+    _need(out_cache_loc, "out_cache_loc", torch.int32, 1)
+    _check_pool(cfg, k_pool, "k_pool")
+    _check_pool(cfg, v_pool, "v_pool")
+    _need(table_row, "table_row", torch.int32, 1)
+    _need(seq_len, "seq_len", torch.int32)
+    rows = out_cache_loc.shape[0]
+    row = cfg.num_kv_heads * cfg.head_dim
+    if k.numel() != rows * row or v.numel() != rows * row or seq_len.numel() != 1:
+        raise ValueError("k / v / seq_len do not match the chunk")
+    _lib.check(_lib.load().ts_kv_store_chunk(ctypes.byref(c), _p(k), _p(v), _p(out_cache_loc), rows,
+                                             _p(k_pool), _p(v_pool), k_pool.shape[0], _p(table_row),
+                                             _p(seq_len), table_row.shape[0], _stream()))
+
+
+def fingerprint(cfg: LayerConfig, q: torch.Tensor, cos_table: torch.Tensor,
+                sin_table: torch.Tensor) -> torch.Tensor:
+    """Fingerprint of a chunk (tr.py:380-392): ``q`` [rows, H, D] bf16, row ``i``
+    rotated to ``n_local + i``, mean over the rows: ``[H, D]`` bf16."""
+    _need(q, "q", torch.bfloat16, 3)
+    _need(cos_table, "cos_table", torch.float32, 2)
+    _need(sin_table, "sin_table", torch.float32, 2)
+    rows, H, D = q.shape
+    if H != cfg.num_heads or D != cfg.head_dim or cos_table.shape != sin_table.shape \
+            or cos_table.shape[1] != D:
+        raise ValueError("q must be [rows, H, D] and the tables [T, D]")
+    qf = torch.empty((H, D), dtype=torch.bfloat16, device=q.device)
+    _lib.check(_lib.load().ts_fingerprint(ctypes.byref(cfg.to_c()), _p(q), rows, _p(cos_table),
+                                          _p(sin_table), cos_table.shape[0], _p(qf), _stream()))
+    return qf
+
+
+def sparse_prefill_attention(cfg: LayerConfig, q: torch.Tensor, k_pool: torch.Tensor,
+                             v_pool: torch.Tensor, sel: torch.Tensor, sel_len: torch.Tensor,
+                             max_sel_len: Optional[int] = None) -> torch.Tensor:
+    """Causal attention of a chunk over the selected slots (tr.py:759-771): ``q``
+    [rows, H*D] bf16, ``sel`` [>= max_sel_len] int32, ``sel_len`` one-element int32."""
+    _need(q, "q", torch.bfloat16, 2)
+    _check_pool(cfg, k_pool, "k_pool")
+    _check_pool(cfg, v_pool, "v_pool")
+    _need(sel, "sel", torch.int32)
+    _need(sel_len, "sel_len", torch.int32)
+    rows = q.shape[0]
+    if q.shape[1] != cfg.num_heads * cfg.head_dim:
+        raise ValueError("q must be [rows, H*D]")
+    if max_sel_len is None:
+        max_sel_len = sel.numel()
+    if sel.numel() < max_sel_len or sel_len.numel() != 1:
+        raise ValueError("sel shorter than max_sel_len, or sel_len not a scalar")
+    out = torch.empty_like(q)
+    _lib.check(_lib.load().ts_sparse_prefill_attn(ctypes.byref(cfg.to_c()), _p(q), rows, _p(k_pool),
+                                                  _p(v_pool), k_pool.shape[0], _p(sel), _p(sel_len),
+                                                  max_sel_len, _p(out), _stream()))
+    return out
+
+
+class PrefillChunk:
+    """One chunk of the patched extend forward after its KV store (tr.py:735-773) as a
+    single library call, for one request; buffers are allocated once."""
+
+    def __init__(self, cfg: LayerConfig, max_seq_len: int, device, max_rows: int = 512):
+        self.cfg, self.max_seq_len, self.max_rows = cfg, max_seq_len, max_rows
+        self._c = cfg.to_c()
+        lib = _lib.load()
+        _lib.check(lib.ts_check_config(ctypes.byref(self._c)))
+        nbytes = lib.ts_decode_layer_workspace_bytes(ctypes.byref(self._c), 1, max_seq_len)
+        self.workspace = torch.empty((nbytes,), dtype=torch.uint8, device=device)
+        self.cos, self.sin = rope_tables(cfg.head_dim, cfg.rope_theta, cfg.rope_scale,
+                                         cfg.n_local + max_rows, device)
+        self.sel = torch.empty((1, cfg.max_sel), dtype=torch.int32, device=device)
+        self.sel_pos = torch.empty_like(self.sel)
+        self.sel_len = torch.empty((1,), dtype=torch.int32, device=device)
+
+    def __call__(self, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch,
+                 out: Optional[torch.Tensor] = None):
+        cfg = self.cfg
+        cb = _c_batch(cfg, bt)
+        _need(q, "q", torch.bfloat16, 2)
+        rows = q.shape[0]
+        if bt.batch != 1 or bt.max_seq_len > self.max_seq_len or rows > self.max_rows:
+            raise ValueError("one request, within the sizes this PrefillChunk was built for")
+        if q.shape[1] != cfg.num_heads * cfg.head_dim:
+            raise ValueError("q must be [rows, H*D]")
+        _check_pool(cfg, k_pool, "k_pool")
+        _check_pool(cfg, v_pool, "v_pool")
+        if out is None:
+            out = torch.empty_like(q)
+        else:
+            _need(out, "out", torch.bfloat16)
+            if out.numel() != q.numel():
+                raise ValueError("out must hold rows*H*D elements")
+        _lib.check(_lib.load().ts_prefill_chunk(
+            ctypes.byref(self._c), ctypes.byref(cb), _p(q), rows, _p(self.cos), _p(self.sin),
+            self.cos.shape[0], _p(k_pool), _p(v_pool), k_pool.shape[0], _p(out), _p(self.sel),
+            _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
+            self.workspace.numel(), _stream()))
+        return out, self.sel, self.sel_pos, self.sel_len
