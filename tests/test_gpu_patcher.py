@@ -179,3 +179,52 @@ def test_selection_cache_trace(dev, anchor_jump):
     assert counters[:, 1].tolist() == [steps] * B
     assert int(counters[:, 0].sum()) == total_hits
     assert 0 < total_hits < B * steps, "the trace must exercise both hits and misses"
+
+
+def test_patched_extend_forward(dev):
+    """Chunked prefill through the patched RadixAttention.forward in EXTEND mode: a
+    prompt of three chunks (the last one ragged) on an empty cache, then one more
+    extend on top; every chunk against the oracle's extend loop on the same pools."""
+    say("patched extend forward: 2 layers, H8/kv2, chunk 32, top_k 24")
+    H, Hkv, D, layers = 8, 2, 128, 2
+    n_init, n_local, top_k, chunk = 4, 32, 24, 32
+    tr.patch(rope_base=1e4, rope_scale=1, rope_model="ROPE_LLAMA", max_n_tokens=512, top_k=top_k,
+             n_init=n_init, n_local=n_local)
+    tr.PREFILL_CHUNK_SIZE = chunk
+    try:
+        g = torch.Generator(device=dev).manual_seed(17)
+        pool = sg.TokenToKVPool(1024, torch.bfloat16, Hkv, D, layers, dev)
+        runner = sg.ModelRunner(model_config=sg.ModelConfig(layers, D, H, Hkv),
+                                token_to_kv_pool=pool, dtype=torch.bfloat16)
+        retriever = runner.req_to_token_retriever.get_token_retriever("req-extend")
+        slots = torch.randperm(1024, generator=g, device=dev).to(torch.int32)
+        attns = [sg.RadixAttention(H, D, D ** -0.5, Hkv, layer_id=l) for l in range(layers)]
+        ref_k = [pool.k_buffer[l].cpu().clone() for l in range(layers)]
+        ref_v = [pool.v_buffer[l].cpu().clone() for l in range(layers)]
+        ref_tab = [torch.zeros(512, dtype=torch.int32) for _ in range(layers)]
+        L = 0
+        for T in (80, 45):
+            loc = slots[L:L + T].contiguous()
+            meta = sg.InputMetadata(sg.ForwardMode.EXTEND, retriever, pool, loc)
+            for l, attn in enumerate(attns):
+                q = torch.randn(T, H * D, generator=g, device=dev).bfloat16()
+                k = torch.randn(T, Hkv * D, generator=g, device=dev).bfloat16()
+                v = torch.randn(T, Hkv * D, generator=g, device=dev).bfloat16()
+                got = attn.forward(q, k, v, meta)
+                torch.cuda.synchronize()
+                assert got.shape == (T, H * D) and retriever.num_tokens[l] == L + T
+                assert torch.equal(retriever.get_all_tokens(l).cpu(), slots[:L + T].cpu())
+                details = []
+                ref = oracle.prefill.prefill(q.cpu(), k.cpu().view(T, Hkv, D), v.cpu().view(T, Hkv, D),
+                                             ref_k[l], ref_v[l], ref_tab[l], L, loc.cpu(), H, D, n_init,
+                                             n_local, top_k, 1e4, 1, D ** -0.5, chunk=chunk,
+                                             details=details)
+                assert torch.equal(pool.k_buffer[l].cpu(), ref_k[l])
+                err = (got.cpu().float() - ref.float()).abs()
+                # chunks whose selection coincides with the oracle's are compared row by row;
+                # the oracle's own fingerprint mean may round a bf16 element differently
+                assert err.max().item() <= 2e-2 or (err > 2e-2).float().mean().item() < 0.02, \
+                    f"extend T={T} layer {l}: max {err.max().item():.3f}"
+            L += T
+    finally:
+        tr.PREFILL_CHUNK_SIZE = 512

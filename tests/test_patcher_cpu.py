@@ -106,13 +106,12 @@ def test_forward_dispatch_and_unsupported_modes():
     meta = sg.InputMetadata(sg.ForwardMode.PREFILL, None, None, torch.zeros(1, dtype=torch.int32))
     q = torch.zeros(1, 4 * 128, dtype=torch.bfloat16)
     assert attn.forward(q, None, None, meta) is None          # neither EXTEND nor DECODE, tr.py:835-842
-    meta.forward_mode = sg.ForwardMode.EXTEND
-    with pytest.raises(NotImplementedError):
-        attn.forward(q, None, None, meta)
     sliding = sg.RadixAttention(4, 128, 128 ** -0.5, 2, layer_id=0, sliding_window_size=4096)
+    for mode in (sg.ForwardMode.EXTEND, sg.ForwardMode.DECODE):
+        meta.forward_mode = mode
+        with pytest.raises(NotImplementedError, match="Sliding window"):
+            sliding.forward(q, None, None, meta)
     meta.forward_mode = sg.ForwardMode.DECODE
-    with pytest.raises(NotImplementedError, match="Sliding window"):
-        sliding.forward(q, None, None, meta)
     with pytest.raises(AssertionError):                       # k without v, tr.py:830-831
         attn.forward(q, torch.zeros(1, 256, dtype=torch.bfloat16), None, meta)
 

@@ -251,11 +251,15 @@ class TokenRetriever:
         return sel_pos[0, :topk].to(torch.int64)
 
     def _fingerprint(self, query):
+        """tr.py:380-392: rotate row i to position n_local + i, average the rows."""
         rows = query.shape[0]
         if rows != 1:
-            raise NotImplementedError(
-                "fingerprints of multi-row (chunked prefill) queries are not built yet; the "
-                "decode path passes one row per request")
+            if not QUERY_ROTATE:
+                return query.mean(dim=0, keepdim=True)
+            cos, sin = self._rope_tables(rows)
+            cfg = self._config(N_INIT, N_Local, TOP_K)
+            return ops.fingerprint(cfg, query.view(rows, -1, self.head_dim).contiguous(), cos,
+                                   sin).view(1, -1)
         if QUERY_ROTATE:
             # Decode row i sits at position n_local + i (tr.py:381-385); one row -> n_local.
             pos = int(N_Local)
@@ -263,6 +267,17 @@ class TokenRetriever:
             return self.rope_embedding.apply_rotary_pos_emb(
                 query.view(1, -1, self.head_dim), position_ids, max_position=pos).view(1, -1)
         return query.view(1, -1)
+
+    def _rope_tables(self, rows):
+        """cos / sin rows 0 .. n_local + rows - 1 (tr.py:92-96), cached."""
+        need = int(N_Local) + rows
+        tables = getattr(self, "_tables", None)
+        if tables is None or tables[0].shape[0] < need:
+            tables = ops.rope_tables(self.head_dim, ROPE_BASE, ROPE_SCALE,
+                                     max(need, int(N_Local) + max(PREFILL_CHUNK_SIZE, 1)),
+                                     self.device)
+            self._tables = tables
+        return tables
 
     def _cache(self, layer_id) -> Optional[ops.SelectionCache]:
         if not QUERY_CACHE:
@@ -316,21 +331,47 @@ class TokenRetriever:
         return out
 
 
+    # ------------------------------------------------------ fused prefill chunk
+    def prefill_attention(self, attn, q, k_buffer, v_buffer):
+        """One fused library call for a prefill chunk after its KV store: chunk
+        fingerprint, selection (or the dense fallback) and the causal attention of the
+        chunk's rows over the result (tr.py:735-773)."""
+        layer_id = attn.layer_id
+        cfg = self._config(N_INIT, N_Local, TOP_K, attn.scaling, attn.logit_cap)
+        key = ("prefill", attn.scaling, attn.logit_cap)
+        runner = self._layers.get(key)
+        if runner is None:
+            runner = ops.PrefillChunk(cfg, self.max_num_tokens, self.device,
+                                      max_rows=max(PREFILL_CHUNK_SIZE, 1))
+            self._layers[key] = runner
+        bt = ops.Batch(self._num_tokens_dev[layer_id:layer_id + 1],
+                       self.token_indices[layer_id:layer_id + 1], self.num_tokens[layer_id])
+        out, _, _, _ = runner(q, k_buffer, v_buffer, bt)
+        return out
+
+
 # ----------------------------------------------------------- patched forwards
 def patched_radix_attention_store_kv_cache(self, cache_k, cache_v, input_metadata, start=0, end=None):
     """tr.py:844-854: scatter the new K/V rows into the pool and append their slots
-    to the request's table - one fused kernel for a decode row."""
+    to the request's table - one fused kernel for a decode row or a prefill chunk."""
     k_cache = input_metadata.token_to_kv_pool.get_key_buffer(self.layer_id)
     v_cache = input_metadata.token_to_kv_pool.get_value_buffer(self.layer_id)
     loc = input_metadata.out_cache_loc[start:end]
     retriever = input_metadata.token_retriever
     rows_k, rows_v = cache_k[start:end], cache_v[start:end]
-    if loc.shape[0] == 1 and loc.dtype == torch.int32:
+    if loc.dtype == torch.int32 and loc.shape[0] >= 1:
         cfg = retriever._config(max(N_INIT, 0), max(N_Local, 0), max(TOP_K, 1))
-        ops.kv_store(cfg, rows_k.contiguous(), rows_v.contiguous(), loc.contiguous(), k_cache,
-                     v_cache, retriever.token_indices[self.layer_id:self.layer_id + 1],
-                     retriever._num_tokens_dev[self.layer_id:self.layer_id + 1])
-        retriever._note_appended(self.layer_id, 1)
+        layer = self.layer_id
+        if loc.shape[0] == 1:
+            ops.kv_store(cfg, rows_k.contiguous(), rows_v.contiguous(), loc.contiguous(), k_cache,
+                         v_cache, retriever.token_indices[layer:layer + 1],
+                         retriever._num_tokens_dev[layer:layer + 1])
+        else:
+            assert retriever.num_tokens[layer] + loc.shape[0] <= retriever.max_num_tokens
+            ops.kv_store_chunk(cfg, rows_k.contiguous(), rows_v.contiguous(), loc.contiguous(),
+                               k_cache, v_cache, retriever.token_indices[layer],
+                               retriever._num_tokens_dev[layer:layer + 1])
+        retriever._note_appended(layer, loc.shape[0])
         return
     k_cache[loc] = rows_k
     v_cache[loc] = rows_v
@@ -354,12 +395,24 @@ def patched_radix_attention_decode_forward_flashinfer(self, q, k, v, input_metad
 
 
 def patched_radix_attention_extend_forward_flashinfer(self, q, k, v, input_metadata):
-    """tr.py:703-775 (chunked prefill with per-chunk selection)."""
+    """tr.py:703-775 without FlashInfer: the prompt in chunks of PREFILL_CHUNK_SIZE rows;
+    per chunk store its K/V, select once for the whole chunk, attend causally."""
+    if self.sliding_window_size != -1:
+        raise NotImplementedError("Sliding window not supported yet")
     assert not getattr(input_metadata, "flashinfer_use_ragged", False)  # not supported yet
     num_chunks = ceil(q.shape[0] / PREFILL_CHUNK_SIZE)
-    raise NotImplementedError(
-        f"chunked-prefill selection ({num_chunks} chunks of {PREFILL_CHUNK_SIZE}) is not built "
-        "yet: this library covers the decode path")
+    outputs = torch.empty_like(q)
+    k_buffer, v_buffer = input_metadata.token_to_kv_pool.get_kv_buffer(self.layer_id)
+    for chunk_idx in range(num_chunks):
+        start = chunk_idx * PREFILL_CHUNK_SIZE
+        end = min((chunk_idx + 1) * PREFILL_CHUNK_SIZE, q.shape[0])
+        if k is not None:
+            assert v is not None
+            self.store_kv_cache(k, v, input_metadata, start=start, end=end)
+        o = input_metadata.token_retriever.prefill_attention(
+            self, q[start:end].contiguous().view(end - start, -1), k_buffer, v_buffer)
+        outputs[start:end] = o.view(end - start, -1)
+    return outputs
 
 
 def patched_radix_attention_forward(self, q, k, v, input_metadata):
