@@ -238,11 +238,14 @@ int ts_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const floa
  * at position S - rows + i (S = *sel_len <= max_sel_len, S >= rows), is rotated
  * to it, and attends to the keys sel[j], rotated to j, for j <= S - rows + i;
  * GQA head h reads KV head h / (H/Hkv); sm_scale, logit_cap as in
- * ts_sparse_decode_attn.  out: [rows, H, D] bf16. */
+ * ts_sparse_decode_attn.  out: [rows, H, D] bf16.  The workspace receives the
+ * selected keys, rotated, and the selected values, transposed, once per call
+ * (2 * Hkv * max_sel_len * D bf16, rounded up). */
+size_t ts_prefill_attn_workspace_bytes(const ts_config* cfg, int32_t max_sel_len);
 int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, const void* k_pool,
                            const void* v_pool, int64_t pool_rows, const int32_t* sel,
-                           const int32_t* sel_len, int32_t max_sel_len, void* out,
-                           ts_stream_t stream);
+                           const int32_t* sel_len, int32_t max_sel_len, void* out, void* workspace,
+                           size_t workspace_bytes, ts_stream_t stream);
 
 /* One chunk of the extend forward after its KV store (tr.py:735-773):
  * fingerprint -> selection -> causal sparse attention, for the single request

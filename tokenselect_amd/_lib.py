@@ -74,7 +74,9 @@ SIGNATURES = {
                            _ptr]),
     "ts_kv_store_chunk": (_i32, [_CFG, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i32, _ptr]),
     "ts_fingerprint": (_i32, [_CFG, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr]),
-    "ts_sparse_prefill_attn": (_i32, [_CFG, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i32, _ptr, _ptr]),
+    "ts_prefill_attn_workspace_bytes": (_size, [_CFG, _i32]),
+    "ts_sparse_prefill_attn": (_i32, [_CFG, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i32, _ptr, _ptr,
+                                      _size, _ptr]),
     "ts_prefill_chunk": (_i32, [_CFG, _BT, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i64, _ptr, _ptr,
                                 _ptr, _i64, _ptr, _ptr, _size, _ptr]),
     "ts_set_fused_select": (_i32, [_i32]),

@@ -131,7 +131,11 @@ static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32
   w.partials = take(w.partials_bytes);
   w.topk_ws = take(ts_topk_workspace_bytes(cfg, batch, max_seq_len));
   w.select_ws = take(select_workspace(cfg, batch, max_seq_len).total);
-  w.attn_ws = take(ts_attn_workspace_bytes(cfg, batch, w.max_sel));
+  {  // decode attention partials, or the staging area of the prefill attention
+    const size_t decode = ts_attn_workspace_bytes(cfg, batch, w.max_sel);
+    const size_t prefill = ts_prefill_attn_workspace_bytes(cfg, w.max_sel);
+    w.attn_ws = take(decode > prefill ? decode : prefill);
+  }
   w.total = off;
   return w;
 }
@@ -214,7 +218,7 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
   }
   if (chunk_rows > 0)
     return ts_sparse_prefill_attn(cfg, q, chunk_rows, k_pool, v_pool, pool_rows, sel, sel_len,
-                                  w.max_sel, out, stream);
+                                  w.max_sel, out, ws + w.attn_ws, w.total - w.attn_ws, stream);
   return launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, bt->batch,
                      w.max_sel, out, ws + w.attn_ws, /*tickets_clear=*/true, (hipStream_t)stream);
 }

@@ -49,19 +49,27 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
 }
 
 // ------------------------------------------------------------ prefill attention
-// Grid (16-row query tiles, KV heads, quads of the G query heads of a KV head);
-// four wavefronts, one query head each, share the K/V tiles of their KV head.
+// Two launches.
 //
-// Per 32-key tile: 256 threads gather the 32 K rows and V rows of the KV head (the
-// next tile's rows are requested before the current one is used), rotate the keys
-// to their index in the selected list and write K row-major and V transposed into
-// LDS.  A wavefront then computes S^T = K Q^T with v_mfma_f32_16x16x32_bf16 (A = 16
-// keys x 32 dims from LDS, B = its 16 rotated queries, held in registers), which
-// leaves lane (query l%16, key group l/16) with the logits of 8 keys; the online
-// softmax needs two cross-lane maxima per tile; the 8 probabilities, rounded to
-// bf16, are directly the B operand of O^T += V^T P^T (A = 16 dims x 32 keys from the
-// transposed V tile, keys in the order the logits came in), so no data moves
-// between the two products.  fp32 accumulation throughout.
+// prefill_gather_kernel: the selected rows are gathered once per chunk into a
+// contiguous staging area, K rotated to its index in the selected list (in fp32,
+// rounded to bf16 like the queries) as kr[kvh][j][128] and V transposed as
+// vt[kvh][128][S_pad], so that the attention kernel, whose 32 query tiles would
+// otherwise each repeat the gather, the rotation and the transposition, only copies
+// tiles.  (That repetition made the first version of this kernel bound by vector
+// instructions at 5 % of the matrix peak.)
+//
+// prefill_attn_kernel<G>: grid (16-row query tiles, KV heads, quads of the G query
+// heads of a KV head); four wavefronts, one query head each, share the K/V tiles of
+// their KV head.  Per 32-key tile the workgroup copies 8 KB of kr and 8 KB of vt
+// into LDS (the next tiles' pieces already in registers).  A wavefront then computes
+// S^T = K Q^T with v_mfma_f32_16x16x32_bf16 (A = 16 keys x 32 dims from LDS, B = its
+// 16 rotated queries, held in registers), which leaves lane (query l%16, key group
+// l/16) with the logits of 8 keys; the online softmax needs two cross-lane maxima
+// per tile; the 8 probabilities, rounded to bf16, are directly the B operand of
+// O^T += V^T P^T (A = 16 dims x 32 keys from the transposed V tile, keys in the order
+// the logits came in), so no data moves between the two products.  fp32 accumulation
+// throughout.
 struct PrefillArgs {
   const uint16_t* q;  // [rows, H, 128] bf16, un-rotated
   const uint16_t* k_pool;
@@ -70,9 +78,12 @@ struct PrefillArgs {
   const int32_t* sel;      // [S] selected slots in attention order
   const int32_t* sel_len;  // device scalar S
   int max_sel_len;
+  int s_pad;               // columns of a vt row: max_sel_len rounded up to the tile
   int rows;
   int num_heads, num_kv_heads, rope_mode;
   float log2_theta, rope_rcp_scale, sm_scale, logit_cap;
+  uint16_t* kr;   // [Hkv, s_pad, 128] bf16 rotated keys
+  uint16_t* vt;   // [Hkv, 128, s_pad] bf16 transposed values
   uint16_t* out;  // [rows, H, 128] bf16
 };
 
@@ -80,11 +91,79 @@ typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float pf_f32x4;
 
 constexpr int kPfKeys = 32;               // keys per tile
+constexpr int kPfPipe = 8;                // tiles whose pieces are in flight
 constexpr int kPfKRow = kHeadDim + 8;     // halfwords per K row in LDS (272 B: rows on different banks)
-constexpr int kPfVRow = kPfKeys + 4;      // halfwords per V^T row in LDS (72 B)
+constexpr int kPfVRow = kPfKeys + 8;      // halfwords per V^T row in LDS (80 B)
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+// Grid (32-key tiles, KV heads).  Thread (key kk, chunk c) moves dims [8c, 8c+8) and
+// [64+8c, +8) of key j = tile + kk.  Keys past S are written as zeros.
+__global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t vt_lds[kHeadDim * kPfVRow];
+  const int tid = threadIdx.x;
+  const int kk = tid >> 3, c8 = tid & 7;
+  const int kvh = blockIdx.y;
+  const int S = min(max(*a.sel_len, 0), a.max_sel_len);
+  const int j = blockIdx.x * kPfKeys + kk;
+  if (blockIdx.x * kPfKeys >= S) return;
+  const bool live = j < S;
+  uint4 kraw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+  uint4 vraw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+  if (live) {
+    uint32_t slot = (uint32_t)a.sel[j];
+    slot = slot < a.pool_rows ? slot : a.pool_rows - 1;
+    const size_t at = ((size_t)slot * a.num_kv_heads + kvh) * kHeadDim + 8 * c8;
+    kraw[0] = *(const uint4*)(a.k_pool + at);
+    kraw[1] = *(const uint4*)(a.k_pool + at + 64);
+    vraw[0] = *(const uint4*)(a.v_pool + at);
+    vraw[1] = *(const uint4*)(a.v_pool + at + 64);
+  }
+  const uint32_t klo[4] = {kraw[0].x, kraw[0].y, kraw[0].z, kraw[0].w};
+  const uint32_t khi[4] = {kraw[1].x, kraw[1].y, kraw[1].z, kraw[1].w};
+  float lo[8], hi[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    lo[2 * e] = bf16_lo(klo[e]);
+    lo[2 * e + 1] = bf16_hi(klo[e]);
+    hi[2 * e] = bf16_lo(khi[e]);
+    hi[2 * e + 1] = bf16_hi(khi[e]);
+  }
+  if (a.rope_mode == TS_ROPE_LLAMA) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int pair = 8 * c8 + e;
+      const float freq = a.rope_rcp_scale * exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
+      float sn, cs;
+      sincos_reduced((float)j * freq, sn, cs);
+      const float l2 = lo[e] * cs - hi[e] * sn;
+      hi[e] = hi[e] * cs + lo[e] * sn;
+      lo[e] = l2;
+    }
+  }
+  uint16_t* krow = a.kr + ((size_t)kvh * a.s_pad + j) * kHeadDim;
+  *(uint4*)(krow + 8 * c8) = make_uint4(pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]),
+                                        pack_bf16(lo[4], lo[5]), pack_bf16(lo[6], lo[7]));
+  *(uint4*)(krow + 64 + 8 * c8) = make_uint4(pack_bf16(hi[0], hi[1]), pack_bf16(hi[2], hi[3]),
+                                             pack_bf16(hi[4], hi[5]), pack_bf16(hi[6], hi[7]));
+  // transpose the 32 x 128 V tile through LDS, then write 128 rows of 64 bytes
+  const uint32_t vlo[4] = {vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w};
+  const uint32_t vhi[4] = {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    vt_lds[(8 * c8 + 2 * e) * kPfVRow + kk] = (uint16_t)(vlo[e] & 0xffffu);
+    vt_lds[(8 * c8 + 2 * e + 1) * kPfVRow + kk] = (uint16_t)(vlo[e] >> 16);
+    vt_lds[(64 + 8 * c8 + 2 * e) * kPfVRow + kk] = (uint16_t)(vhi[e] & 0xffffu);
+    vt_lds[(64 + 8 * c8 + 2 * e + 1) * kPfVRow + kk] = (uint16_t)(vhi[e] >> 16);
+  }
+  __syncthreads();
+  const int d = tid >> 1, half = tid & 1;
+  uint16_t* vrow = a.vt + ((size_t)kvh * kHeadDim + d) * a.s_pad + blockIdx.x * kPfKeys + 16 * half;
+  const uint4* src = (const uint4*)(vt_lds + d * kPfVRow + 16 * half);
+  ((uint4*)vrow)[0] = src[0];
+  ((uint4*)vrow)[1] = src[1];
 }
 
 template <int G>
@@ -146,71 +225,22 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(PrefillArgs a) {
     }
   }
 
-  // ---- staging role: thread (key kk, chunk c) moves dims [8c, 8c+8) and [64+8c, +8) of
-  // key j = tile + kk; its rotation state advances by one tile (32 positions) per step.
-  const int kk = tid >> 3, c8 = tid & 7;
-  float kc[8], ksn[8], dc[8], ds[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    kc[e] = 1.f;
-    ksn[e] = 0.f;
-    dc[e] = 1.f;
-    ds[e] = 0.f;
-    if (rope) {
-      const int pair = 8 * c8 + e;
-      const float freq = a.rope_rcp_scale * exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
-      sincos_reduced((float)kk * freq, ksn[e], kc[e]);
-      sincos_reduced((float)kPfKeys * freq, ds[e], dc[e]);
-    }
-  }
-  const size_t row_elems = (size_t)a.num_kv_heads * kHeadDim;
-  uint4 kraw[2], vraw[2];
-  auto request_tile = [&](int tile) {
-    const int j = min(tile + kk, S - 1);
-    uint32_t slot = (uint32_t)a.sel[j];
-    slot = slot < a.pool_rows ? slot : a.pool_rows - 1;
-    const size_t at = (size_t)slot * row_elems + (size_t)kvh * kHeadDim + 8 * c8;
-    kraw[0] = *(const uint4*)(a.k_pool + at);
-    kraw[1] = *(const uint4*)(a.k_pool + at + 64);
-    vraw[0] = *(const uint4*)(a.v_pool + at);
-    vraw[1] = *(const uint4*)(a.v_pool + at + 64);
-  };
-  auto stage_tile = [&]() {
-    const uint32_t klo[4] = {kraw[0].x, kraw[0].y, kraw[0].z, kraw[0].w};
-    const uint32_t khi[4] = {kraw[1].x, kraw[1].y, kraw[1].z, kraw[1].w};
-    float lo[8], hi[8];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      lo[2 * e] = bf16_lo(klo[e]);
-      lo[2 * e + 1] = bf16_hi(klo[e]);
-      hi[2 * e] = bf16_lo(khi[e]);
-      hi[2 * e + 1] = bf16_hi(khi[e]);
-    }
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float l2 = lo[e] * kc[e] - hi[e] * ksn[e];
-      const float h2 = hi[e] * kc[e] + lo[e] * ksn[e];
-      lo[e] = l2;
-      hi[e] = h2;
-      const float c2 = kc[e] * dc[e] - ksn[e] * ds[e];  // advance to the next tile
-      ksn[e] = ksn[e] * dc[e] + kc[e] * ds[e];
-      kc[e] = c2;
-    }
-    *(uint4*)(k_lds + kk * kPfKRow + 8 * c8) =
-        make_uint4(pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]), pack_bf16(lo[4], lo[5]),
-                   pack_bf16(lo[6], lo[7]));
-    *(uint4*)(k_lds + kk * kPfKRow + 64 + 8 * c8) =
-        make_uint4(pack_bf16(hi[0], hi[1]), pack_bf16(hi[2], hi[3]), pack_bf16(hi[4], hi[5]),
-                   pack_bf16(hi[6], hi[7]));
-    const uint32_t vlo[4] = {vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w};
-    const uint32_t vhi[4] = {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      vt_lds[(8 * c8 + 2 * e) * kPfVRow + kk] = (uint16_t)(vlo[e] & 0xffffu);
-      vt_lds[(8 * c8 + 2 * e + 1) * kPfVRow + kk] = (uint16_t)(vlo[e] >> 16);
-      vt_lds[(64 + 8 * c8 + 2 * e) * kPfVRow + kk] = (uint16_t)(vhi[e] & 0xffffu);
-      vt_lds[(64 + 8 * c8 + 2 * e + 1) * kPfVRow + kk] = (uint16_t)(vhi[e] >> 16);
-    }
+  // ---- staging role: thread t copies 32 bytes of the K tile (key t/8, dims [16 (t%8), +16))
+  // and 32 bytes of the V^T tile (dim t/2, keys [16 (t%2), +16)).
+  const uint16_t* k_src = a.kr + (size_t)kvh * a.s_pad * kHeadDim + (size_t)(tid >> 3) * kHeadDim +
+                          16 * (tid & 7);
+  const uint16_t* v_src = a.vt + ((size_t)kvh * kHeadDim + (tid >> 1)) * a.s_pad + 16 * (tid & 1);
+  uint16_t* k_dst = k_lds + (tid >> 3) * kPfKRow + 16 * (tid & 7);
+  uint16_t* v_dst = vt_lds + (tid >> 1) * kPfVRow + 16 * (tid & 1);
+  uint4 kbuf[kPfPipe][2], vbuf[kPfPipe][2];
+  auto request_tile = [&](int u, int tile) {
+    tile = min(tile, a.s_pad - kPfKeys);  // past the end: harmless repeat of the last tile
+    const uint4* ks = (const uint4*)(k_src + (size_t)tile * kHeadDim);
+    const uint4* vs = (const uint4*)(v_src + tile);
+    kbuf[u][0] = ks[0];
+    kbuf[u][1] = ks[1];
+    vbuf[u][0] = vs[0];
+    vbuf[u][1] = vs[1];
   };
 
   // ---- main loop over the tiles any row of this query tile can see
@@ -221,65 +251,81 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
   for (int db = 0; db < 8; ++db) o[db] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
 
-  request_tile(0);
-  for (int tile = 0; tile <= last_visible; tile += kPfKeys) {
-    __syncthreads();  // the previous tile's LDS reads are done
-    stage_tile();
-    if (tile + kPfKeys <= last_visible) request_tile(tile + kPfKeys);
-    __syncthreads();
-    if (!wave_active) continue;
+#pragma unroll
+  for (int u = 0; u < kPfPipe; ++u) request_tile(u, kPfKeys * u);
+  for (int round = 0; round <= last_visible; round += kPfPipe * kPfKeys) {
+#pragma unroll
+    for (int u = 0; u < kPfPipe; ++u) {
+      const int tile = round + kPfKeys * u;
+      if (tile > last_visible) break;
+      __syncthreads();  // the previous tile's LDS reads are done
+      ((uint4*)k_dst)[0] = kbuf[u][0];
+      ((uint4*)k_dst)[1] = kbuf[u][1];
+      ((uint4*)v_dst)[0] = vbuf[u][0];
+      ((uint4*)v_dst)[1] = vbuf[u][1];
+      request_tile(u, tile + kPfPipe * kPfKeys);
+      __syncthreads();
+      if (!wave_active) continue;
 
-    // logits: s[blk][r] belongs to key tile + 16 blk + 4 g4 + r and query qc
-    float s[2][4];
+      // logits: s[blk][r] belongs to key tile + 16 blk + 4 g4 + r and query qc
+      float s[2][4];
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
-      pf_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      for (int blk = 0; blk < 2; ++blk) {
+        pf_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const uint4 kw = *(const uint4*)(k_lds + (16 * blk + qc) * kPfKRow + 32 * ks + 8 * g4);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, kw), qb[ks], acc,
-                                                      0, 0, 0);
+        for (int ks = 0; ks < 4; ++ks) {
+          const uint4 kw = *(const uint4*)(k_lds + (16 * blk + qc) * kPfKRow + 32 * ks + 8 * g4);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, kw), qb[ks],
+                                                        acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float x = acc[r] * a.sm_scale;
+          if (a.logit_cap > 0.f) x = a.logit_cap * tanhf(x / a.logit_cap);
+          const int key = tile + 16 * blk + 4 * g4 + r;
+          s[blk][r] = key <= my_limit ? x : kNegBig;
+        }
+      }
+      float mx = kNegBig;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[blk][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __expf(m_run - m_new);
+      float p[2][4], psum = 0.f;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          p[blk][r] = s[blk][r] > 0.5f * kNegBig ? __expf(s[blk][r] - m_new) : 0.f;
+          psum += p[blk][r];
+        }
+      l_run = l_run * alpha + psum;
+      // The accumulators only need rescaling when some query's maximum moved, which
+      // after the first tiles is rare: skip the 32 multiplications otherwise.
+      const bool rescale = __ballot(m_new != m_run) != 0ull;
+      m_run = m_new;
+      const uint4 pw = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]),
+                                  pack_bf16(p[1][0], p[1][1]), pack_bf16(p[1][2], p[1][3]));
+      const pf_bf16x8 pb = __builtin_bit_cast(pf_bf16x8, pw);
+      if (rescale) {
+#pragma unroll
+        for (int db = 0; db < 8; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[db][r] *= alpha;
       }
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float x = acc[r] * a.sm_scale;
-        if (a.logit_cap > 0.f) x = a.logit_cap * tanhf(x / a.logit_cap);
-        const int key = tile + 16 * blk + 4 * g4 + r;
-        s[blk][r] = key <= my_limit ? x : kNegBig;
+      for (int db = 0; db < 8; ++db) {
+        const uint16_t* vrow = vt_lds + (16 * db + qc) * kPfVRow;
+        const uint2 v0 = *(const uint2*)(vrow + 4 * g4);
+        const uint2 v1 = *(const uint2*)(vrow + 16 + 4 * g4);
+        const uint4 vw = make_uint4(v0.x, v0.y, v1.x, v1.y);
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw), pb, o[db],
+                                                        0, 0, 0);
       }
-    }
-    float mx = kNegBig;
-#pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[blk][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __expf(m_run - m_new);
-    float p[2][4], psum = 0.f;
-#pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        p[blk][r] = s[blk][r] > 0.5f * kNegBig ? __expf(s[blk][r] - m_new) : 0.f;
-        psum += p[blk][r];
-      }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    const uint4 pw = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]),
-                                pack_bf16(p[1][0], p[1][1]), pack_bf16(p[1][2], p[1][3]));
-    const pf_bf16x8 pb = __builtin_bit_cast(pf_bf16x8, pw);
-#pragma unroll
-    for (int db = 0; db < 8; ++db) {
-      const uint16_t* vrow = vt_lds + (16 * db + qc) * kPfVRow;
-      const uint2 v0 = *(const uint2*)(vrow + 4 * g4);
-      const uint2 v1 = *(const uint2*)(vrow + 16 + 4 * g4);
-      const uint4 vw = make_uint4(v0.x, v0.y, v1.x, v1.y);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) o[db][r] *= alpha;
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw), pb, o[db],
-                                                      0, 0, 0);
     }
   }
   if (!wave_active || q_row0 + qc >= m) return;
@@ -294,6 +340,8 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(PrefillArgs a) {
     *(uint2*)(orow + 16 * db + 4 * g4) = make_uint2(pack_bf16(o[db][0] * inv, o[db][1] * inv),
                                                     pack_bf16(o[db][2] * inv, o[db][3] * inv));
 }
+
+static int prefill_s_pad(int max_sel_len) { return (int)ceil_div(max_sel_len, kPfKeys) * kPfKeys; }
 
 }  // namespace ts
 
@@ -315,10 +363,15 @@ int ts_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const floa
   return check_launch("fingerprint_kernel");
 }
 
+size_t ts_prefill_attn_workspace_bytes(const ts_config* cfg, int32_t max_sel_len) {
+  if (validate_config(cfg) != TS_OK || max_sel_len < 1) return 0;
+  return 2 * align_up((size_t)cfg->num_kv_heads * prefill_s_pad(max_sel_len) * kHeadDim * 2, 256);
+}
+
 int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, const void* k_pool,
                            const void* v_pool, int64_t pool_rows, const int32_t* sel,
-                           const int32_t* sel_len, int32_t max_sel_len, void* out,
-                           ts_stream_t stream) {
+                           const int32_t* sel_len, int32_t max_sel_len, void* out, void* workspace,
+                           size_t workspace_bytes, ts_stream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_REQUIRE(q && k_pool && v_pool && sel && sel_len && out, TS_EINVAL,
              "ts_sparse_prefill_attn: NULL tensor argument");
@@ -327,6 +380,9 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
              "max_sel_len %d < rows %d: a chunk attends at least to itself", max_sel_len, rows);
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
+  const size_t need = ts_prefill_attn_workspace_bytes(cfg, max_sel_len);
+  TS_REQUIRE(workspace != nullptr && workspace_bytes >= need, TS_EWORKSPACE,
+             "ts_sparse_prefill_attn: workspace %zu bytes < required %zu", workspace_bytes, need);
   PrefillArgs a;
   a.q = (const uint16_t*)q;
   a.k_pool = (const uint16_t*)k_pool;
@@ -335,6 +391,7 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
   a.sel = sel;
   a.sel_len = sel_len;
   a.max_sel_len = max_sel_len;
+  a.s_pad = prefill_s_pad(max_sel_len);
   a.rows = rows;
   a.num_heads = cfg->num_heads;
   a.num_kv_heads = cfg->num_kv_heads;
@@ -343,11 +400,16 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
   a.rope_rcp_scale = cfg->rope_mode == TS_ROPE_LLAMA ? 1.0f / cfg->rope_scale : 1.0f;
   a.sm_scale = cfg->sm_scale;
   a.logit_cap = cfg->logit_cap;
+  a.kr = (uint16_t*)workspace;
+  a.vt = (uint16_t*)((char*)workspace + need / 2);
   a.out = (uint16_t*)out;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(prefill_gather_kernel, dim3((unsigned)(a.s_pad / kPfKeys), (unsigned)cfg->num_kv_heads),
+                     dim3(256), 0, st, a);
+  TS_TRY(check_launch("prefill_gather_kernel"));
   const int group = cfg->num_heads / cfg->num_kv_heads;
   const dim3 grid((unsigned)ceil_div(rows, 16), (unsigned)cfg->num_kv_heads,
                   (unsigned)ceil_div(group, 4));
-  hipStream_t st = (hipStream_t)stream;
   switch (group) {
     case 1: hipLaunchKernelGGL(prefill_attn_kernel<1>, grid, dim3(256), 0, st, a); break;
     case 2: hipLaunchKernelGGL(prefill_attn_kernel<2>, grid, dim3(256), 0, st, a); break;

@@ -530,9 +530,12 @@ def sparse_prefill_attention(cfg: LayerConfig, q: torch.Tensor, k_pool: torch.Te
     if sel.numel() < max_sel_len or sel_len.numel() != 1:
         raise ValueError("sel shorter than max_sel_len, or sel_len not a scalar")
     out = torch.empty_like(q)
-    _lib.check(_lib.load().ts_sparse_prefill_attn(ctypes.byref(cfg.to_c()), _p(q), rows, _p(k_pool),
-                                                  _p(v_pool), k_pool.shape[0], _p(sel), _p(sel_len),
-                                                  max_sel_len, _p(out), _stream()))
+    lib, c = _lib.load(), cfg.to_c()
+    nbytes = lib.ts_prefill_attn_workspace_bytes(ctypes.byref(c), max_sel_len)
+    ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=q.device)
+    _lib.check(lib.ts_sparse_prefill_attn(ctypes.byref(c), _p(q), rows, _p(k_pool), _p(v_pool),
+                                          k_pool.shape[0], _p(sel), _p(sel_len), max_sel_len, _p(out),
+                                          _p(ws), ws.numel(), _stream()))
     return out
 
 
