@@ -60,9 +60,12 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
 // instructions at 5 % of the matrix peak.)
 //
 // prefill_attn_kernel<G>: grid (16-row query tiles, KV heads, quads of the G query
-// heads of a KV head); four wavefronts, one query head each, share the K/V tiles of
-// their KV head.  Per 32-key tile the workgroup copies 8 KB of kr and 8 KB of vt
-// into LDS (the next tiles' pieces already in registers).  A wavefront then computes
+// heads of a KV head); 512 threads = two groups of four wavefronts.  The wavefronts
+// of a group serve one query head each and share the K/V tiles of their KV head;
+// group 0 takes the even 32-key tiles and group 1 the odd ones (two wavefronts per
+// SIMD hide each other's LDS and matrix latencies), and their (max, sum, acc) are
+// merged through LDS at the end.  Per tile a group copies 8 KB of kr and 8 KB of vt
+// into its LDS buffers (the next tiles' pieces already in registers).  A wavefront then computes
 // S^T = K Q^T with v_mfma_f32_16x16x32_bf16 (A = 16 keys x 32 dims from LDS, B = its
 // 16 rotated queries, held in registers), which leaves lane (query l%16, key group
 // l/16) with the logits of 8 keys; the online softmax needs two cross-lane maxima
@@ -91,7 +94,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float pf_f32x4;
 
 constexpr int kPfKeys = 32;               // keys per tile
-constexpr int kPfPipe = 8;                // tiles whose pieces are in flight
+constexpr int kPfPipe = 4;                // tiles whose pieces are in flight
 constexpr int kPfKRow = kHeadDim + 8;     // halfwords per K row in LDS (272 B: rows on different banks)
 constexpr int kPfVRow = kPfKeys + 8;      // halfwords per V^T row in LDS (80 B)
 
@@ -167,11 +170,15 @@ __global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
 }
 
 template <int G>
-__global__ __launch_bounds__(256) void prefill_attn_kernel(PrefillArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t k_lds[kPfKeys * kPfKRow];
-  __shared__ __attribute__((aligned(16))) uint16_t vt_lds[kHeadDim * kPfVRow];
+__global__ __launch_bounds__(512) void prefill_attn_kernel(PrefillArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds2[2][kPfKeys * kPfKRow];
+  __shared__ __attribute__((aligned(16))) uint16_t vt_lds2[2][kHeadDim * kPfVRow];
+  __shared__ float merge_lds[4][64][34];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int group = threadIdx.x >> 8;  // which of the two tile streams this wavefront follows
+  uint16_t* const k_lds = k_lds2[group];
+  uint16_t* const vt_lds = vt_lds2[group];
+  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
   const int qc = lane & 15, g4 = lane >> 4;  // query column / key group of the MFMA layouts
   const int kvh = blockIdx.y;
   const int head_in_group = blockIdx.z * 4 + wave;
@@ -251,21 +258,24 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
   for (int db = 0; db < 8; ++db) o[db] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // Step u of a round covers the tile pair starting at round + 64 u; this group's tile
+  // is the first or the second of the pair.
 #pragma unroll
-  for (int u = 0; u < kPfPipe; ++u) request_tile(u, kPfKeys * u);
-  for (int round = 0; round <= last_visible; round += kPfPipe * kPfKeys) {
+  for (int u = 0; u < kPfPipe; ++u) request_tile(u, kPfKeys * (2 * u + group));
+  for (int round = 0; round <= last_visible; round += 2 * kPfPipe * kPfKeys) {
 #pragma unroll
     for (int u = 0; u < kPfPipe; ++u) {
-      const int tile = round + kPfKeys * u;
-      if (tile > last_visible) break;
-      __syncthreads();  // the previous tile's LDS reads are done
+      const int pair = round + 2 * kPfKeys * u;
+      if (pair > last_visible) break;
+      const int tile = pair + kPfKeys * group;
+      __syncthreads();  // the previous tiles' LDS reads are done
       ((uint4*)k_dst)[0] = kbuf[u][0];
       ((uint4*)k_dst)[1] = kbuf[u][1];
       ((uint4*)v_dst)[0] = vbuf[u][0];
       ((uint4*)v_dst)[1] = vbuf[u][1];
-      request_tile(u, tile + kPfPipe * kPfKeys);
+      request_tile(u, tile + 2 * kPfPipe * kPfKeys);
       __syncthreads();
-      if (!wave_active) continue;
+      if (!wave_active || tile > last_visible) continue;
 
       // logits: s[blk][r] belongs to key tile + 16 blk + 4 g4 + r and query qc
       float s[2][4];
@@ -328,7 +338,28 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(PrefillArgs a) {
       }
     }
   }
-  if (!wave_active || q_row0 + qc >= m) return;
+  // Group 1 hands its partial result to group 0 (same wavefront index, same lane).
+  if (group == 1) {
+    float* mine = merge_lds[wave][lane];
+    mine[0] = m_run;
+    mine[1] = l_run;
+#pragma unroll
+    for (int db = 0; db < 8; ++db)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mine[2 + 4 * db + r] = o[db][r];
+  }
+  __syncthreads();
+  if (group == 1 || !wave_active || q_row0 + qc >= m) return;
+  {
+    const float* other = merge_lds[wave][lane];
+    const float m_new = fmaxf(m_run, other[0]);
+    const float e0 = __expf(m_run - m_new), e1 = __expf(other[0] - m_new);
+    l_run = l_run * e0 + other[1] * e1;
+#pragma unroll
+    for (int db = 0; db < 8; ++db)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[db][r] = o[db][r] * e0 + other[2 + 4 * db + r] * e1;
+  }
 
   // o[db][r] = O[query qc][dim 16 db + 4 g4 + r]; the row sum is spread over the 4 key groups.
   float l_tot = l_run + __shfl_xor(l_run, 16);
@@ -411,11 +442,11 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
   const dim3 grid((unsigned)ceil_div(rows, 16), (unsigned)cfg->num_kv_heads,
                   (unsigned)ceil_div(group, 4));
   switch (group) {
-    case 1: hipLaunchKernelGGL(prefill_attn_kernel<1>, grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL(prefill_attn_kernel<2>, grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL(prefill_attn_kernel<4>, grid, dim3(256), 0, st, a); break;
-    case 7: hipLaunchKernelGGL(prefill_attn_kernel<7>, grid, dim3(256), 0, st, a); break;
-    case 8: hipLaunchKernelGGL(prefill_attn_kernel<8>, grid, dim3(256), 0, st, a); break;
+    case 1: hipLaunchKernelGGL(prefill_attn_kernel<1>, grid, dim3(512), 0, st, a); break;
+    case 2: hipLaunchKernelGGL(prefill_attn_kernel<2>, grid, dim3(512), 0, st, a); break;
+    case 4: hipLaunchKernelGGL(prefill_attn_kernel<4>, grid, dim3(512), 0, st, a); break;
+    case 7: hipLaunchKernelGGL(prefill_attn_kernel<7>, grid, dim3(512), 0, st, a); break;
+    case 8: hipLaunchKernelGGL(prefill_attn_kernel<8>, grid, dim3(512), 0, st, a); break;
     default: return fail(TS_ESHAPE, "unsupported head group %d", group);
   }
   return check_launch("prefill_attn_kernel");
