@@ -7,7 +7,8 @@ attention) over one synthetic batch resident in HBM, issued as a single
 ``ts_decode_layer`` call.  The default workload is the Llama-3-8B layer at
 128K context in a page-16 KV pool (``--workload c2``); ``c1``, ``c3`` and
 ``c5`` are the other layer shapes, ``c4`` the 64-step selection-cache trace
-(there a step also stores the new token's K/V and consults the cache).
+(there a step also stores the new token's K/V and consults the cache),
+``prefill`` one 512-row chunk of the extend forward on top of a 128K context.
 
 Every step reads a different copy of the K/V pool (``--pools``, default 4, as
 consecutive layers of a model do): the copies together exceed the 256 MB
@@ -267,18 +268,120 @@ def bench_trace(args, ops, workloads, dev):
     return result
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix peak
+
+
+def bench_prefill(args, ops, workloads, dev):
+    """One chunk of the patched extend forward on top of a 128K context: store the
+    chunk's K/V, fingerprint of the chunk, selection, causal sparse attention of the
+    chunk's 512 rows.  Each step serves a different copy of the pool."""
+    L0, m = args.prefill_context, args.prefill_rows
+    wl = workloads.build("PREFILL llama3-8b L%d chunk%d k2048 page1" % (L0, m), workloads.LLAMA3_8B,
+                         [L0], [2048], 1, dev, seed=5, extra_pages=m)
+    c = wl.cfg
+    gen = torch.Generator(device=dev).manual_seed(6)
+    q = torch.randn((m, c.num_heads * c.head_dim), generator=gen, device=dev).bfloat16()
+    k_new = torch.randn((m, c.num_kv_heads, c.head_dim), generator=gen, device=dev).bfloat16()
+    v_new = torch.randn((m, c.num_kv_heads, c.head_dim), generator=gen, device=dev).bfloat16()
+    loc = torch.arange(L0, L0 + m, dtype=torch.int32, device=dev)
+    table0 = torch.zeros((1, L0 + m), dtype=torch.int32, device=dev)
+    table0[0, :L0] = wl.table[0, :L0]
+    n_pools = max(1, args.pools)
+    k_pools = [wl.k_pool] + [wl.k_pool.clone() for _ in range(n_pools - 1)]
+    v_pools = [wl.v_pool] + [wl.v_pool.clone() for _ in range(n_pools - 1)]
+    layer = ops.PrefillChunk(c, L0 + m, dev, max_rows=m)
+    tables = [table0.clone() for _ in range(n_pools)]
+    seqs = [wl.seq_lens_dev.clone() for _ in range(n_pools)]
+
+    def step(i):
+        p = i % n_pools
+        seqs[p].fill_(L0)          # the chunk is appended afresh every time
+        ops.kv_store_chunk(c, k_new, v_new, loc, k_pools[p], v_pools[p], tables[p][0], seqs[p])
+        return layer(q, k_pools[p], v_pools[p], ops.Batch(seqs[p], tables[p], L0 + m))
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    us_per_chunk = (time.perf_counter() - t0) / args.steps * 1e6
+
+    out, sel, _, sel_len = step(0)
+    torch.cuda.synchronize()
+    S = int(sel_len[0])
+    sel0 = sel[0].contiguous()
+    attn_us, attn_min = event_time_us(
+        lambda i: ops.sparse_prefill_attention(c, q, k_pools[i % n_pools], v_pools[i % n_pools], sel0,
+                                               sel_len, c.max_sel), args.steps, args.warmup)
+    visible = sum(S - m + i + 1 for i in range(m))                 # (row, key) pairs under the mask
+    flops = 4 * c.num_heads * c.head_dim * visible                 # QK^T and PV, 2 flops per MAC
+    tflops = flops / attn_us / 1e6
+    result = {
+        "metric": "us_per_layer_prefill_chunk (kv store+fingerprint+select+causal sparse attn)",
+        "value": round(us_per_chunk, 2), "unit": "us", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(us_per_chunk / 1e3, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": wl.name, "batch": 1, "seq_lens_max": L0 + m, "chunk_rows": m,
+                   "page_size": 1, "top_k": c.top_k, "n_init": c.n_init, "n_local": c.n_local,
+                   "kv_pool_copies": n_pools},
+        "prompt_tokens_per_s": round(m / (us_per_chunk * 1e-6 * args.layers), 1),
+        "tokens_per_s_note": f"selection+attention only, {args.layers} layers per token",
+        "roofline": {"bound": "mfma", "kernel": "ts::prefill_attn_kernel<G> (+ the 7 us gather pass)",
+                     "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "flops_per_launch": flops, "us_per_launch": round(attn_us, 2),
+                     "us_min": round(attn_min, 2)},
+    }
+    if not args.no_cpu_baseline:
+        import oracle
+        torch.set_num_threads(int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        kc, vc, tab = k_pools[0].cpu(), v_pools[0].cpu(), tables[0][0].cpu()
+        qc = q.cpu()
+        qf = ops.fingerprint(c, q.view(m, c.num_heads, c.head_dim), layer.cos, layer.sin).cpu()
+        sm = c.head_dim ** -0.5
+
+        def run():
+            return oracle.prefill.prefill_chunk(qc, kc, vc, tab, L0 + m, c.num_heads, c.head_dim,
+                                                c.n_init, c.n_local, c.top_k, c.rope_theta,
+                                                c.rope_scale, sm, qf_override=qf)
+
+        run()
+        times = []
+        for _ in range(args.cpu_reps):
+            t0 = time.perf_counter()
+            ref_slots, ref_out = run()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        result["cpu_baseline"] = {
+            "value": round(times[len(times) // 2] * 1e6, 1), "unit": "us",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"the chunk's selection + attention (no KV store), median of {args.cpu_reps} "
+                      "repetitions after one warm-up (PyTorch CPU oracle)"}
+        same = torch.equal(sel[0, :S].cpu(), ref_slots)
+        err = (out.cpu().float() - ref_out.float()).abs().max().item()
+        result["parity"] = {"selected_slots_identical": bool(same),
+                            "attn_max_abs_err": round(err, 5)}
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "prefill"])
     ap.add_argument("--cpu-reps", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layers", type=int, default=32, help="layers for the tokens/s figure")
     ap.add_argument("--pools", type=int, default=4,
                     help="copies of the K/V pool cycled through, one per step")
     ap.add_argument("--trace-steps", type=int, default=64, help="decode steps of the c4 trace")
+    ap.add_argument("--prefill-context", type=int, default=131072,
+                    help="tokens already cached when the measured prefill chunk arrives")
+    ap.add_argument("--prefill-rows", type=int, default=512, help="rows of the prefill chunk")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run five 256 MiB device copies (reference for counter runs)")
     args = ap.parse_args()
@@ -293,6 +396,8 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload == "c4":
         result = bench_trace(args, ops, workloads, dev)
+    elif args.workload == "prefill":
+        result = bench_prefill(args, ops, workloads, dev)
     else:
         result = bench_layer(args, ops, workloads, dev)
     print(json.dumps(result), flush=True)
