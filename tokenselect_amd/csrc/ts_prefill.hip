@@ -98,8 +98,12 @@ constexpr int kPfPipe = 4;                // tiles whose pieces are in flight
 constexpr int kPfKRow = kHeadDim + 8;     // halfwords per K row in LDS (272 B: rows on different banks)
 constexpr int kPfVRow = kPfKeys + 8;      // halfwords per V^T row in LDS (80 B)
 
+// Two floats to packed bf16, round to nearest even, in one v_cvt_pk_bf16_f32.
+typedef __attribute__((ext_vector_type(2))) __bf16 pf_bf16x2;
+typedef __attribute__((ext_vector_type(2))) float pf_f32x2;
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+  const pf_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, pf_bf16x2));
 }
 
 // Grid (32-key tiles, KV heads).  Thread (key kk, chunk c) moves dims [8c, 8c+8) and
@@ -169,8 +173,11 @@ __global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
   ((uint4*)vrow)[1] = src[1];
 }
 
-template <int G>
-__global__ __launch_bounds__(512) void prefill_attn_kernel(PrefillArgs a) {
+// Two wavefronts per SIMD by construction (8 per workgroup, one workgroup per CU):
+// saying so lets the compiler use 256 registers instead of spilling at 128.
+template <int G, bool CAP>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(
+    PrefillArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t k_lds2[2][kPfKeys * kPfKRow];
   __shared__ __attribute__((aligned(16))) uint16_t vt_lds2[2][kHeadDim * kPfVRow];
   __shared__ float merge_lds[4][64][34];
@@ -239,15 +246,22 @@ __global__ __launch_bounds__(512) void prefill_attn_kernel(PrefillArgs a) {
   const uint16_t* v_src = a.vt + ((size_t)kvh * kHeadDim + (tid >> 1)) * a.s_pad + 16 * (tid & 1);
   uint16_t* k_dst = k_lds + (tid >> 3) * kPfKRow + 16 * (tid & 7);
   uint16_t* v_dst = vt_lds + (tid >> 1) * kPfVRow + 16 * (tid & 1);
-  uint4 kbuf[kPfPipe][2], vbuf[kPfPipe][2];
-  auto request_tile = [&](int u, int tile) {
+  // Four register buffers, named rather than indexed: an indexed array of them is
+  // kept in scratch memory by the compiler, and the prefetch with it.
+  struct TilePiece {
+    uint4 k0, k1, v0, v1;
+  };
+  TilePiece piece0, piece1, piece2, piece3;
+  auto request_tile = [&](int tile) __attribute__((always_inline)) -> TilePiece {
     tile = min(tile, a.s_pad - kPfKeys);  // past the end: harmless repeat of the last tile
     const uint4* ks = (const uint4*)(k_src + (size_t)tile * kHeadDim);
     const uint4* vs = (const uint4*)(v_src + tile);
-    kbuf[u][0] = ks[0];
-    kbuf[u][1] = ks[1];
-    vbuf[u][0] = vs[0];
-    vbuf[u][1] = vs[1];
+    TilePiece piece;
+    piece.k0 = ks[0];
+    piece.k1 = ks[1];
+    piece.v0 = vs[0];
+    piece.v1 = vs[1];
+    return piece;
   };
 
   // ---- main loop over the tiles any row of this query tile can see
@@ -258,86 +272,100 @@ __global__ __launch_bounds__(512) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
   for (int db = 0; db < 8; ++db) o[db] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // Step u of a round covers the tile pair starting at round + 64 u; this group's tile
-  // is the first or the second of the pair.
+  // One tile of this group: logits, online softmax, output update.
+  auto compute_tile = [&](int tile) __attribute__((always_inline)) {
+    // logits: s[blk][r] belongs to key tile + 16 blk + 4 g4 + r and query qc
+    float s[2][4];
 #pragma unroll
-  for (int u = 0; u < kPfPipe; ++u) request_tile(u, kPfKeys * (2 * u + group));
-  for (int round = 0; round <= last_visible; round += 2 * kPfPipe * kPfKeys) {
+    for (int blk = 0; blk < 2; ++blk) {
+      pf_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int u = 0; u < kPfPipe; ++u) {
-      const int pair = round + 2 * kPfKeys * u;
-      if (pair > last_visible) break;
-      const int tile = pair + kPfKeys * group;
-      __syncthreads();  // the previous tiles' LDS reads are done
-      ((uint4*)k_dst)[0] = kbuf[u][0];
-      ((uint4*)k_dst)[1] = kbuf[u][1];
-      ((uint4*)v_dst)[0] = vbuf[u][0];
-      ((uint4*)v_dst)[1] = vbuf[u][1];
-      request_tile(u, tile + 2 * kPfPipe * kPfKeys);
-      __syncthreads();
-      if (!wave_active || tile > last_visible) continue;
-
-      // logits: s[blk][r] belongs to key tile + 16 blk + 4 g4 + r and query qc
-      float s[2][4];
-#pragma unroll
-      for (int blk = 0; blk < 2; ++blk) {
-        pf_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          const uint4 kw = *(const uint4*)(k_lds + (16 * blk + qc) * kPfKRow + 32 * ks + 8 * g4);
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, kw), qb[ks],
-                                                        acc, 0, 0, 0);
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float x = acc[r] * a.sm_scale;
-          if (a.logit_cap > 0.f) x = a.logit_cap * tanhf(x / a.logit_cap);
-          const int key = tile + 16 * blk + 4 * g4 + r;
-          s[blk][r] = key <= my_limit ? x : kNegBig;
-        }
-      }
-      float mx = kNegBig;
-#pragma unroll
-      for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[blk][r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 16));
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __expf(m_run - m_new);
-      float p[2][4], psum = 0.f;
-#pragma unroll
-      for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          p[blk][r] = s[blk][r] > 0.5f * kNegBig ? __expf(s[blk][r] - m_new) : 0.f;
-          psum += p[blk][r];
-        }
-      l_run = l_run * alpha + psum;
-      // The accumulators only need rescaling when some query's maximum moved, which
-      // after the first tiles is rare: skip the 32 multiplications otherwise.
-      const bool rescale = __ballot(m_new != m_run) != 0ull;
-      m_run = m_new;
-      const uint4 pw = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]),
-                                  pack_bf16(p[1][0], p[1][1]), pack_bf16(p[1][2], p[1][3]));
-      const pf_bf16x8 pb = __builtin_bit_cast(pf_bf16x8, pw);
-      if (rescale) {
-#pragma unroll
-        for (int db = 0; db < 8; ++db)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) o[db][r] *= alpha;
+      for (int ks = 0; ks < 4; ++ks) {
+        const uint4 kw = *(const uint4*)(k_lds + (16 * blk + qc) * kPfKRow + 32 * ks + 8 * g4);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, kw), qb[ks],
+                                                      acc, 0, 0, 0);
       }
 #pragma unroll
-      for (int db = 0; db < 8; ++db) {
-        const uint16_t* vrow = vt_lds + (16 * db + qc) * kPfVRow;
-        const uint2 v0 = *(const uint2*)(vrow + 4 * g4);
-        const uint2 v1 = *(const uint2*)(vrow + 16 + 4 * g4);
-        const uint4 vw = make_uint4(v0.x, v0.y, v1.x, v1.y);
-        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw), pb, o[db],
-                                                        0, 0, 0);
+      for (int r = 0; r < 4; ++r) {
+        float x = acc[r] * a.sm_scale;
+        if (CAP) x = a.logit_cap * tanhf(x / a.logit_cap);
+        const int key = tile + 16 * blk + 4 * g4 + r;
+        // Masked logits are -inf and the running maximum starts at a finite value,
+        // so exp(s - max) is 0 for them without a branch and never NaN.
+        s[blk][r] = key <= my_limit ? x : -INFINITY;
       }
     }
+    float mx = kNegBig;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[blk][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __expf(m_run - m_new);
+    float p[2][4], psum = 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        p[blk][r] = __expf(s[blk][r] - m_new);
+        psum += p[blk][r];
+      }
+    l_run = l_run * alpha + psum;
+    // The accumulators only need rescaling when some query's maximum moved, which
+    // after the first tiles is rare: skip the 32 multiplications otherwise.
+    const bool rescale = __ballot(m_new != m_run) != 0ull;
+    m_run = m_new;
+    const uint4 pw = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]),
+                                pack_bf16(p[1][0], p[1][1]), pack_bf16(p[1][2], p[1][3]));
+    const pf_bf16x8 pb = __builtin_bit_cast(pf_bf16x8, pw);
+    if (rescale) {
+#pragma unroll
+      for (int db = 0; db < 8; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[db][r] *= alpha;
+    }
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      const uint16_t* vrow = vt_lds + (16 * db + qc) * kPfVRow;
+      const uint2 v0 = *(const uint2*)(vrow + 4 * g4);
+      const uint2 v1 = *(const uint2*)(vrow + 16 + 4 * g4);
+      const uint4 vw = make_uint4(v0.x, v0.y, v1.x, v1.y);
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw), pb, o[db],
+                                                      0, 0, 0);
+    }
+  };
+
+  // Step u of a round covers the tile pair starting at round + 64 u; this group's tile
+  // is the first or the second of the pair.  The steps are written out one by one so
+  // that each uses its own register buffer.
+  static_assert(kPfPipe == 4, "the steps below are written out for four buffers");
+#define TS_PF_STEP(u)                                                         \
+  {                                                                           \
+    const int pair = round + 2 * kPfKeys * (u);                               \
+    if (pair > last_visible) break;                                           \
+    const int tile = pair + kPfKeys * group;                                  \
+    __syncthreads(); /* the previous tiles' LDS reads are done */             \
+    ((uint4*)k_dst)[0] = piece##u.k0;                                         \
+    ((uint4*)k_dst)[1] = piece##u.k1;                                         \
+    ((uint4*)v_dst)[0] = piece##u.v0;                                         \
+    ((uint4*)v_dst)[1] = piece##u.v1;                                         \
+    piece##u = request_tile(tile + 2 * kPfPipe * kPfKeys);                    \
+    __syncthreads();                                                          \
+    if (wave_active && tile <= last_visible) compute_tile(tile);              \
   }
+  piece0 = request_tile(kPfKeys * (0 + group));
+  piece1 = request_tile(kPfKeys * (2 + group));
+  piece2 = request_tile(kPfKeys * (4 + group));
+  piece3 = request_tile(kPfKeys * (6 + group));
+  for (int round = 0; round <= last_visible; round += 2 * kPfPipe * kPfKeys) {
+    TS_PF_STEP(0)
+    TS_PF_STEP(1)
+    TS_PF_STEP(2)
+    TS_PF_STEP(3)
+  }
+#undef TS_PF_STEP
   // Group 1 hands its partial result to group 0 (same wavefront index, same lane).
   if (group == 1) {
     float* mine = merge_lds[wave][lane];
@@ -441,14 +469,23 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
   const int group = cfg->num_heads / cfg->num_kv_heads;
   const dim3 grid((unsigned)ceil_div(rows, 16), (unsigned)cfg->num_kv_heads,
                   (unsigned)ceil_div(group, 4));
+  const bool cap = cfg->logit_cap > 0.f;
+#define TS_PF_CASE(G_)                                                                       \
+  case G_:                                                                                   \
+    if (cap)                                                                                 \
+      hipLaunchKernelGGL((prefill_attn_kernel<G_, true>), grid, dim3(512), 0, st, a);        \
+    else                                                                                     \
+      hipLaunchKernelGGL((prefill_attn_kernel<G_, false>), grid, dim3(512), 0, st, a);       \
+    break;
   switch (group) {
-    case 1: hipLaunchKernelGGL(prefill_attn_kernel<1>, grid, dim3(512), 0, st, a); break;
-    case 2: hipLaunchKernelGGL(prefill_attn_kernel<2>, grid, dim3(512), 0, st, a); break;
-    case 4: hipLaunchKernelGGL(prefill_attn_kernel<4>, grid, dim3(512), 0, st, a); break;
-    case 7: hipLaunchKernelGGL(prefill_attn_kernel<7>, grid, dim3(512), 0, st, a); break;
-    case 8: hipLaunchKernelGGL(prefill_attn_kernel<8>, grid, dim3(512), 0, st, a); break;
+    TS_PF_CASE(1)
+    TS_PF_CASE(2)
+    TS_PF_CASE(4)
+    TS_PF_CASE(7)
+    TS_PF_CASE(8)
     default: return fail(TS_ESHAPE, "unsupported head group %d", group);
   }
+#undef TS_PF_CASE
   return check_launch("prefill_attn_kernel");
 }
 
