@@ -24,18 +24,34 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
   const int h = blockIdx.x;
   const int i = threadIdx.x % half, rg = threadIdx.x / half;
   float lo_sum = 0.f, hi_sum = 0.f;
-  for (int r = rg; r < rows; r += kFpRowGroups) {
-    int64_t pos = (int64_t)first_pos + r;
-    pos = pos < table_rows ? pos : table_rows - 1;
-    const float* c = cos_table + pos * kHeadDim;
-    const float* s = sin_table + pos * kHeadDim;
-    const size_t base = ((size_t)r * heads + h) * kHeadDim;
-    const float x1 = bf16_to_f32(q[base + i]);
-    const float x2 = bf16_to_f32(q[base + i + half]);
-    const float lo = x1 * c[i] + (-x2) * s[i];
-    const float hi = x2 * c[i + half] + x1 * s[i + half];
-    lo_sum += bf16_to_f32(f32_to_bf16(lo));
-    hi_sum += bf16_to_f32(f32_to_bf16(hi));
+  // Four rows per step: their loads are independent and go out together; the sums
+  // are still taken in row order.
+  for (int r0 = rg; r0 < rows; r0 += 4 * kFpRowGroups) {
+    float x1[4], x2[4], c1[4], c2[4], s1[4], s2[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = min(r0 + j * kFpRowGroups, rows - 1);
+      int64_t pos = (int64_t)first_pos + r;
+      pos = pos < table_rows ? pos : table_rows - 1;
+      const float* c = cos_table + pos * kHeadDim;
+      const float* s = sin_table + pos * kHeadDim;
+      const size_t base = ((size_t)r * heads + h) * kHeadDim;
+      x1[j] = bf16_to_f32(q[base + i]);
+      x2[j] = bf16_to_f32(q[base + i + half]);
+      c1[j] = c[i];
+      c2[j] = c[i + half];
+      s1[j] = s[i];
+      s2[j] = s[i + half];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (r0 + j * kFpRowGroups < rows) {
+        const float lo = x1[j] * c1[j] + (-x2[j]) * s1[j];
+        const float hi = x2[j] * c2[j] + x1[j] * s2[j];
+        lo_sum += bf16_to_f32(f32_to_bf16(lo));
+        hi_sum += bf16_to_f32(f32_to_bf16(hi));
+      }
+    }
   }
   __shared__ float part[kFpRowGroups][kHeadDim];
   part[rg][i] = lo_sum;
