@@ -1,5 +1,6 @@
-"""Writes ``tests/golden/decode_layer_small.npz``: seeded inputs of one small
-decode layer and the outputs of the CPU oracle (``oracle/``) for them.
+"""Writes ``tests/golden/decode_layer_small.npz`` and
+``tests/golden/prefill_small.npz``: seeded inputs of one small decode layer and of
+one small chunked prefill, and the outputs of the CPU oracle (``oracle/``) for them.
 
 The reference holds no golden vectors for this path and cannot be imported, so
 these fixtures come from this repository's own oracle; they lock the oracle
@@ -67,5 +68,40 @@ def main():
     print("wrote", OUT, os.path.getsize(OUT), "bytes")
 
 
+PREFILL_OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prefill_small.npz")
+
+
+def prefill():
+    """A 70-row extend on top of 90 cached tokens, chunks of 32 rows (n_local 32)."""
+    g = torch.Generator().manual_seed(2025)
+    heads, kv, L0, T, chunk, n_init, n_local, top_k = 8, 2, 90, 70, 32, 4, 32, 12
+    rows = L0 + T
+    k_pool = torch.randn(rows, kv, D, generator=g).bfloat16()
+    v_pool = torch.randn(rows, kv, D, generator=g).bfloat16()
+    order = torch.randperm(rows, generator=g).int()
+    tab = torch.zeros(rows, dtype=torch.int32)
+    tab[:L0] = order[:L0]
+    new_slots = order[L0:]
+    q = torch.randn(T, heads * D, generator=g).bfloat16()
+    k_new = torch.randn(T, kv, D, generator=g).bfloat16()
+    v_new = torch.randn(T, kv, D, generator=g).bfloat16()
+    k0, v0 = k_pool.clone(), v_pool.clone()
+    details = []
+    out = oracle.prefill.prefill(q, k_new, v_new, k_pool, v_pool, tab, L0, new_slots, heads, D, n_init,
+                                 n_local, top_k, ROPE_BASE, 1.0, D ** -0.5, chunk=chunk,
+                                 details=details)
+    arrays = dict(
+        meta=np.array([heads, kv, D, n_init, n_local, top_k, L0, T, chunk], dtype=np.int64),
+        rope_base=np.array([ROPE_BASE]), k_pool=bits(k0), v_pool=bits(v0), table=tab[:L0].numpy(),
+        new_slots=new_slots.numpy(), q=bits(q), k_new=bits(k_new), v_new=bits(v_new), out=bits(out))
+    for i, d in enumerate(details):
+        arrays[f"qf_{i}"] = bits(d["qf"])
+        arrays[f"top_pos_{i}"] = d["top_pos"].numpy()
+        arrays[f"votes_{i}"] = d["votes"].numpy()
+    np.savez_compressed(PREFILL_OUT, **arrays)
+    print("wrote", PREFILL_OUT, os.path.getsize(PREFILL_OUT), "bytes")
+
+
 if __name__ == "__main__":
     main()
+    prefill()

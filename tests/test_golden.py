@@ -59,3 +59,73 @@ def test_hip_path_matches_the_fixture(dev):
         assert int(sel_len[b]) == want.shape[0]
         assert sel[b, :want.shape[0]].cpu().tolist() == want.tolist()
     assert (out.cpu().float() - f["out"].float()).abs().max().item() <= 2e-2
+
+
+PREFILL_FIXTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "prefill_small.npz")
+
+
+def load_prefill():
+    z = np.load(PREFILL_FIXTURE, allow_pickle=False)
+    names = ("H", "HKV", "D", "n_init", "n_local", "top_k", "L0", "T", "chunk")
+    f = dict(zip(names, (int(x) for x in z["meta"])))
+    bf = lambda name: torch.from_numpy(z[name].copy()).view(torch.bfloat16)
+    f.update(z=z, rope_base=float(z["rope_base"][0]), k_pool=bf("k_pool"), v_pool=bf("v_pool"),
+             table=torch.from_numpy(z["table"].copy()), new_slots=torch.from_numpy(z["new_slots"].copy()),
+             q=bf("q"), k_new=bf("k_new"), v_new=bf("v_new"), out=bf("out"))
+    return f
+
+
+def test_oracle_reproduces_the_prefill_fixture():
+    f = load_prefill()
+    rows = f["L0"] + f["T"]
+    tab = torch.zeros(rows, dtype=torch.int32)
+    tab[:f["L0"]] = f["table"]
+    details = []
+    out = oracle.prefill.prefill(f["q"], f["k_new"], f["v_new"], f["k_pool"].clone(), f["v_pool"].clone(),
+                                 tab, f["L0"], f["new_slots"], f["H"], f["D"], f["n_init"], f["n_local"],
+                                 f["top_k"], f["rope_base"], 1.0, f["D"] ** -0.5, chunk=f["chunk"],
+                                 details=details)
+    assert len(details) == 3                                    # 32 + 32 + 6 rows
+    for i, d in enumerate(details):
+        assert d["top_pos"].tolist() == f["z"][f"top_pos_{i}"].tolist()
+        assert torch.equal(d["qf"].view(torch.int16), torch.from_numpy(f["z"][f"qf_{i}"].copy()))
+    assert (out.float() - f["out"].float()).abs().max().item() <= 1e-2
+
+
+@pytest.mark.gpu
+def test_hip_prefill_matches_the_fixture(dev):
+    """Chunk by chunk: device fingerprint within one bf16 ulp of the fixture's, the
+    selection as in the fixture wherever the fingerprints agree bit for bit, and the
+    chunk output within tolerance wherever the selections agree."""
+    from tokenselect_amd import ops
+    f = load_prefill()
+    H, D, L0, T, chunk = f["H"], f["D"], f["L0"], f["T"], f["chunk"]
+    cfg = ops.LayerConfig(num_heads=H, num_kv_heads=f["HKV"], n_init=f["n_init"], n_local=f["n_local"],
+                          top_k=f["top_k"], rope_theta=f["rope_base"])
+    k_pool, v_pool = f["k_pool"].to(dev), f["v_pool"].to(dev)
+    table = torch.zeros((1, L0 + T), dtype=torch.int32, device=dev)
+    table[0, :L0] = f["table"].to(dev)
+    seq = torch.tensor([L0], dtype=torch.int32, device=dev)
+    layer = ops.PrefillChunk(cfg, L0 + T, dev, max_rows=chunk)
+    q, L, compared = f["q"].to(dev), L0, 0
+    for i, start in enumerate(range(0, T, chunk)):
+        end = min(start + chunk, T)
+        ops.kv_store_chunk(cfg, f["k_new"][start:end].to(dev), f["v_new"][start:end].to(dev),
+                           f["new_slots"][start:end].to(dev).contiguous(), k_pool, v_pool, table[0], seq)
+        L += end - start
+        out, sel, sel_pos, sel_len = layer(q[start:end].contiguous(), k_pool, v_pool,
+                                           ops.Batch(seq, table, L))
+        qf = ops.fingerprint(cfg, q[start:end].view(end - start, H, D).contiguous(), layer.cos, layer.sin)
+        torch.cuda.synchronize()
+        want_qf = torch.from_numpy(f["z"][f"qf_{i}"].copy()).view(torch.bfloat16).float()
+        got_qf = qf.cpu().float().reshape(-1)
+        assert bool(((got_qf - want_qf).abs() <= want_qf.abs() * 2.0 ** -7 + 1e-30).all())
+        S = int(sel_len[0])
+        assert S == f["n_init"] + f["top_k"] + f["n_local"]
+        if torch.equal(got_qf, want_qf):
+            mid = sel_pos[0, f["n_init"]:f["n_init"] + f["top_k"]].cpu()
+            if mid.tolist() == f["z"][f"top_pos_{i}"].tolist():
+                want = f["out"][start:end].float()
+                assert (out.cpu().float() - want).abs().max().item() <= 2e-2
+                compared += 1
+    assert compared >= 1
