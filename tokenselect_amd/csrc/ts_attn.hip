@@ -59,7 +59,8 @@ __device__ __forceinline__ void store_coherent2(float* p, float x, float y) {
 
 constexpr int kAttnInFlight = 8;  // tokens per lane group requested together
 
-template <int G>
+// ROPE and CAP are compile-time so that the token loop carries no branches.
+template <int G, bool ROPE, bool CAP>
 __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int S = min(max(a.sel_len[b], 0), a.max_sel_len);
@@ -72,7 +73,7 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   const int l16 = tid & 15;  // owns dims [8*l16, 8*l16+8)
   const bool upper = l16 >= 8;  // second half of the head dimension
   const int H = a.num_heads;
-  const bool rope = a.rope_mode == TS_ROPE_LLAMA;
+  constexpr bool rope = ROPE;
   const int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
   const size_t row_elems = (size_t)a.num_kv_heads * kHeadDim;
 
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const int pair = (l16 & 7) * 8 + e;
-    freq[e] = a.rope_rcp_scale * exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
+    freq[e] = a.rope_rcp_scale * __builtin_amdgcn_exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
   }
 
   // Query rows of the G heads, rotated to position S-1.
@@ -173,16 +174,17 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) p += qv[g][e] * kf[e];
         p = row16_sum(p) * a.sm_scale;
-        if (a.logit_cap > 0.f) p = a.logit_cap * tanhf(p / a.logit_cap);
-        if (valid) {
-          const float mn = fmaxf(m[g], p);
-          const float alpha = __expf(m[g] - mn);
-          const float w = __expf(p - mn);
-          l[g] = l[g] * alpha + w;
+        if (CAP) p = a.logit_cap * tanhf(p / a.logit_cap);
+        // A token past the range gets the logit -inf: weight 0, maximum unchanged
+        // (the running maximum starts at a finite value, so nothing becomes NaN).
+        p = valid ? p : -INFINITY;
+        const float mn = fmaxf(m[g], p);
+        const float alpha = __expf(m[g] - mn);
+        const float w = __expf(p - mn);
+        l[g] = l[g] * alpha + w;
 #pragma unroll
-          for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * alpha + w * vf[e];
-          m[g] = mn;
-        }
+        for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * alpha + w * vf[e];
+        m[g] = mn;
       }
     }
   }
@@ -344,14 +346,26 @@ int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const v
   }
   const dim3 grid((unsigned)a.nsplit, (unsigned)cfg->num_kv_heads, (unsigned)batch);
   const int group = cfg->num_heads / cfg->num_kv_heads;
+  const bool rope = cfg->rope_mode == TS_ROPE_LLAMA, cap = cfg->logit_cap > 0.f;
+#define TS_ATTN_LAUNCH(G_, R_, C_) \
+  hipLaunchKernelGGL((attn_kernel<G_, R_, C_>), grid, dim3(256), 0, st, a)
+#define TS_ATTN_CASE(G_)                           \
+  case G_:                                         \
+    if (rope && cap) TS_ATTN_LAUNCH(G_, true, true);        \
+    else if (rope) TS_ATTN_LAUNCH(G_, true, false);         \
+    else if (cap) TS_ATTN_LAUNCH(G_, false, true);          \
+    else TS_ATTN_LAUNCH(G_, false, false);                  \
+    break;
   switch (group) {
-    case 1: hipLaunchKernelGGL(attn_kernel<1>, grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL(attn_kernel<2>, grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL(attn_kernel<4>, grid, dim3(256), 0, st, a); break;
-    case 7: hipLaunchKernelGGL(attn_kernel<7>, grid, dim3(256), 0, st, a); break;
-    case 8: hipLaunchKernelGGL(attn_kernel<8>, grid, dim3(256), 0, st, a); break;
+    TS_ATTN_CASE(1)
+    TS_ATTN_CASE(2)
+    TS_ATTN_CASE(4)
+    TS_ATTN_CASE(7)
+    TS_ATTN_CASE(8)
     default: return fail(TS_ESHAPE, "unsupported head group %d", group);
   }
+#undef TS_ATTN_CASE
+#undef TS_ATTN_LAUNCH
   return check_launch("attn_kernel");
 }
 
