@@ -46,6 +46,12 @@ __device__ __forceinline__ uint32_t load_coherent(const uint32_t* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The workgroups of a grid that take part in its rendezvous.
+struct GridTeam {
+  uint32_t size;   // participating workgroups
+  uint32_t index;  // this workgroup among them
+};
+
 // Rendezvous area, in 32-bit words: kSyncSlots + 1 slots, kSyncSlotWords apart so
 // that the slots fall into different memory channels, the first kSyncLiveWords of
 // each zero at launch.
@@ -59,7 +65,7 @@ constexpr int kSyncLiveWords = 16;
 constexpr int kSyncMaxRounds = kSyncLiveWords - 2;
 constexpr size_t kSyncWords = (size_t)(kSyncSlots + 1) * kSyncSlotWords;
 
-// Every workgroup arrives exactly once per round; those that need the others' data
+// Every participating workgroup arrives exactly once per round; those that need the others' data
 // of that round wait for it to complete.  Each thread first waits for its
 // outstanding memory operations (what it published has been performed by then);
 // thread 0 then counts the workgroup in.  Arrivals are counted in two levels,
@@ -72,13 +78,12 @@ constexpr size_t kSyncWords = (size_t)(kSyncSlots + 1) * kSyncSlotWords;
 // still streaming need for 1/128 of their data.  The wait is bounded: if the
 // round does not complete within `ticks` of the 100 MHz clock the fault word is
 // set and the workgroup carries on, so the kernel always drains.
+// `workgroups` of the grid take part, this one as number `index` among them.
 __device__ __forceinline__ void grid_arrive(uint32_t* sync, uint32_t round, bool wait,
-                                            uint64_t ticks) {
+                                            uint64_t ticks, uint32_t workgroups, uint32_t index) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (threadIdx.x < 64) {  // the first wavefront; lane 0 counts, all lanes raise the flags
-    const uint32_t workgroups = gridDim.x * gridDim.y;
-    const uint32_t index = blockIdx.y * gridDim.x + blockIdx.x;
     uint32_t last = 0;
     if (threadIdx.x == 0) {
       uint32_t groups = 1;

@@ -84,11 +84,12 @@ constexpr int kMaxHeads = 128;
 // Between the two rendezvous of the fused kernel: the (request, head) pairs are
 // dealt out over all wavefronts of the grid; a wavefront merges the per-workgroup
 // (max, sum exp) of its pair, a lane per chunk, in a fixed order.
-__device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, int lane, int wave) {
+__device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const GridTeam& team,
+                                                    int lane, int wave) {
   const int H = a.num_heads;
   const int items = (int)gridDim.y * H;
-  const int first = ((int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x) * 4 + wave;
-  const int step = (int)gridDim.x * (int)gridDim.y * 4;
+  const int first = (int)team.index * 4 + wave;
+  const int step = (int)team.size * 4;
   for (int item = first; item < items; item += step) {
     const int b = item / H, h = item % H;
     if (a.skip && a.skip[b]) continue;
@@ -116,6 +117,42 @@ __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, int lane
 }
 
 constexpr uint32_t kSelectRounds = 6;  // rendezvous of the fused kernel
+
+// The workgroups that take part in the rendezvous of the fused kernel: all those of
+// the requests that select (neither dense nor served by the selection cache).  The
+// others write their fixed output and leave, so that a step in which every request
+// hits the cache costs a few microseconds instead of six empty rounds.
+__device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t* lds) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int B = gridDim.y, mine = blockIdx.y;
+  uint32_t before = 0, total = 0;  // selecting requests below this one / in all
+  for (int base = 0; base < B; base += 256) {
+    const int b = base + tid;
+    bool selects = false;
+    if (b < B && !(a.skip && a.skip[b]))
+      selects = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
+                                 a.max_seq_len).n > 0;
+    const uint64_t mask = __ballot(selects);
+    if (lane == 0) {
+      lds[wave] = (uint32_t)__popcll(mask);
+      // requests of this chunk below `mine` that lie in this wavefront's 64
+      const int lo = base + 64 * wave;
+      const int upto = mine - lo;  // bits [0, upto) count
+      lds[4 + wave] = upto <= 0 ? 0u
+                                : (uint32_t)__popcll(upto >= 64 ? mask : mask & ((1ull << upto) - 1ull));
+    }
+    __syncthreads();
+    for (int w = 0; w < 4; ++w) {
+      total += lds[w];
+      before += lds[4 + w];
+    }
+    __syncthreads();
+  }
+  GridTeam team;
+  team.size = total * gridDim.x;
+  team.index = before * gridDim.x + blockIdx.x;
+  return team;
+}
 
 // The parts of the output that need no votes, written while the keys stream: a
 // dense request gets all its positions and a selection-cache hit its cached ones
@@ -215,13 +252,19 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     first_pos = a.n_init;
   }
   const int block_lo = blockIdx.x * a.tokens_per_block;
-  if constexpr (MODE == kScoreFused) fixed_segments(a, b);
+  GridTeam team{0u, 0u};
+  if constexpr (MODE == kScoreFused) {
+    __shared__ uint32_t team_lds[8];
+    fixed_segments(a, b);
+    if (n <= 0) return;  // dense or served by the cache: nothing to select, not on the team
+    team = selecting_team(a, team_lds);
+  }
   if (block_lo >= n) {
     if constexpr (MODE == kScoreFused) {  // no tokens here: only help with the statistics
-      grid_arrive(a.sync, 1, true, a.spin_ticks);
-      merge_request_stats(a, threadIdx.x & 63, threadIdx.x >> 6);
+      grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
+      merge_request_stats(a, team, threadIdx.x & 63, threadIdx.x >> 6);
       for (uint32_t round = 2; round <= kSelectRounds; ++round)
-        grid_arrive(a.sync, round, false, a.spin_ticks);
+        grid_arrive(a.sync, round, false, a.spin_ticks, team.size, team.index);
     }
     return;
   }
@@ -452,9 +495,9 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     const int tid = threadIdx.x;
     for (int i = tid; i < kTopkBins; i += 256) lh[i] = 0u;
     if (tid < 16) scratch[tid] = 0u;
-    grid_arrive(a.sync, 1, true, a.spin_ticks);
-    merge_request_stats(a, lane, wave);
-    grid_arrive(a.sync, 2, true, a.spin_ticks);
+    grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
+    merge_request_stats(a, team, lane, wave);
+    grid_arrive(a.sync, 2, true, a.spin_ticks, team.size, team.index);
     for (int slot = tid; slot < H; slot += 256) {
       const int h = head_of<HKV, G>(slot / G, slot % G, a.head_map);
       const float2 st = load_coherent((const float2*)a.stats + (size_t)b * H + h);
@@ -527,7 +570,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       if (tid == 0) done += fetch_max_coherent(&ctr[kSelMaxBin], scratch[8]);
       await(done);
     }
-    grid_arrive(a.sync, 3, true, a.spin_ticks);
+    grid_arrive(a.sync, 3, true, a.spin_ticks, team.size, team.index);
     uint32_t t0 = 0, above0 = 0;
     for (int top = (int)load_coherent(&ctr[kSelMaxBin]); top >= 0; top -= 256) {
       const int bin = top - tid;
@@ -557,7 +600,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       }
       await(done);
     }
-    grid_arrive(a.sync, 4, true, a.spin_ticks);
+    grid_arrive(a.sync, 4, true, a.spin_ticks, team.size, team.index);
     {
       uint32_t h[kTopkBins / 256];
 #pragma unroll
@@ -580,7 +623,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       }
       await(done);
     }
-    grid_arrive(a.sync, 5, true, a.spin_ticks);
+    grid_arrive(a.sync, 5, true, a.spin_ticks, team.size, team.index);
     {
       uint32_t h[4];
 #pragma unroll
@@ -620,7 +663,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     __syncthreads();
     uint2* counts = a.block_counts + (size_t)b * gridDim.x;
     if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], scratch[9]);
-    grid_arrive(a.sync, 6, true, a.spin_ticks);
+    grid_arrive(a.sync, 6, true, a.spin_ticks, team.size, team.index);
     {
       uint32_t sure = 0, tie = 0;
       for (int j = tid; j < (int)blockIdx.x; j += 256) {
