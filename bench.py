@@ -8,7 +8,10 @@ attention) over one synthetic batch resident in HBM, issued as a single
 128K context in a page-16 KV pool (``--workload c2``); ``c1``, ``c3`` and
 ``c5`` are the other layer shapes, ``c4`` the 64-step selection-cache trace
 (there a step also stores the new token's K/V and consults the cache),
-``prefill`` one 512-row chunk of the extend forward on top of a 128K context.
+``prefill`` one 512-row chunk of the extend forward on top of a 128K context,
+``model`` the whole 32-layer Llama-3-8B-shaped decoder (batch 4, 256K context per
+request, 128 greedy decode steps; there a step is one decode step and the value is
+tokens/s).
 
 Every step reads a different copy of the K/V pool (``--pools``, default 4, as
 consecutive layers of a model do): the copies together exceed the 256 MB
@@ -367,15 +370,120 @@ def bench_prefill(args, ops, workloads, dev):
     return result
 
 
+def bench_model(args, ops, dev):
+    """The full-model configuration: a random-initialised Llama-3-8B-shaped decoder
+    (bf16 weights N(0, 0.02)), `model_batch` requests with `model_context` prefilled
+    random KV tokens each, TokenSelect on all layers, greedy decoding.  A step is
+    one decode step of the whole batch through all layers."""
+    from tokenselect_amd.model import Decoder, ModelConfig
+    mc = ModelConfig(layers=args.layers, top_k=args.model_top_k)
+    B, L = args.model_batch, args.model_context
+    t0 = time.perf_counter()
+    m = Decoder(mc, [L] * B, args.warmup + args.steps + 1, dev, seed=4)
+    torch.cuda.synchronize()
+    build_s = time.perf_counter() - t0
+    c = m.cfg
+    tokens = torch.arange(1, B + 1, device=dev)
+    tokens = m.generate(tokens, args.warmup)[-1] if args.warmup else tokens
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    tokens = m.generate(tokens, args.steps)[-1]
+    torch.cuda.synchronize()
+    step_s = (time.perf_counter() - t0) / args.steps
+
+    # One more step, traced, for the parity check and the kernel timings.
+    trace = []
+    m.decode_step(tokens, trace)
+    torch.cuda.synchronize()
+    Lnow = L + args.warmup + args.steps + 1
+    bt = ops.Batch(m.num_tokens[0], m.table, Lnow)
+    row = c.num_kv_heads * c.head_dim * 2
+    score_bytes = B * ((Lnow - c.n_init - c.n_local) * row + Lnow * 4 + c.num_heads * c.head_dim * 2)
+    cos, sin = ops.scoring_cos_sin(c.head_dim, c.rope_theta, c.rope_scale, c.n_local, dev)
+    qf = ops.rope_apply(trace[0][0].view(B, c.num_heads, c.head_dim), cos, sin, None)
+    bufs = ops.score(c, bt, qf, m.k_pools[0])
+    score_us, score_min = event_time_us(
+        lambda i: ops.score(c, bt, qf, m.k_pools[i % mc.layers], out=bufs), 2 * mc.layers, mc.layers)
+    del bufs
+    gbs = score_bytes / score_us / 1e3
+    weights = sum(w.numel() * 2 for ws in (m.wqkv, m.wo, m.w_gate_up, m.w_down) for w in ws) \
+        + m.lm_head.numel() * 2
+    sel_rows = B * c.max_sel
+    step_bytes = weights + mc.layers * (score_bytes + sel_rows * (2 * row + 4))
+    result = {
+        "metric": "decode tokens/s, full model (all layers TokenSelect, greedy)",
+        "value": round(B / step_s, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "C5 llama3-8b-shaped decoder B%d L%d k%d page1, %d layers"
+                               % (B, L, c.top_k, mc.layers),
+                   "batch": B, "seq_lens_max": Lnow, "page_size": 1, "top_k": c.top_k,
+                   "n_init": c.n_init, "n_local": c.n_local, "hidden": mc.hidden,
+                   "intermediate": mc.intermediate, "vocab": mc.vocab,
+                   "weights": "random N(0, 0.02) bf16", "kv": "prefilled random N(0,1) bf16"},
+        "us_per_layer": round(step_s * 1e6 / mc.layers, 2),
+        "setup_s": round(build_s, 1),
+        "hbm_bytes_per_step": step_bytes,
+        "hbm_frac_whole_step": round(step_bytes / step_s / 1e9 / HBM_PEAK_GBS, 4),
+        "roofline": {"bound": "hbm",
+                     "kernel": "ts::score_kernel<Hkv,G,false,1> (ts_score, one launch per layer)",
+                     "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": score_bytes, "us_per_launch": round(score_us, 2),
+                     "us_min": round(score_min, 2)},
+    }
+    if not args.no_cpu_baseline:
+        import oracle
+        torch.set_num_threads(int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        layer_ix = mc.layers - 1
+        q, _, _, attn, sel, sel_len = trace[layer_ix]
+        kc, vc = m.k_pools[layer_ix].cpu(), m.v_pools[layer_ix].cpu()
+        tab = m.table[0].cpu()
+        q0 = q[:1].cpu()
+
+        def run():
+            return oracle.layer.decode_layer(q0, kc, vc, [tab], [Lnow], c.num_heads, c.head_dim,
+                                             c.n_init, c.n_local, [c.top_k], c.rope_theta,
+                                             c.rope_scale, c.head_dim ** -0.5)
+
+        run()
+        times = []
+        for _ in range(args.cpu_reps):
+            t0 = time.perf_counter()
+            ref_sels, ref_out = run()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        per_request_layer = times[len(times) // 2]
+        result["cpu_baseline"] = {
+            "value": round(1.0 / (per_request_layer * mc.layers), 4), "unit": "tokens/s",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"selection + attention of request 0 on layer {layer_ix} at the last decode "
+                      f"step ({per_request_layer * 1e3:.1f} ms, median of {args.cpu_reps} after one "
+                      f"warm-up, PyTorch CPU oracle), scaled by {mc.layers} layers per token; the "
+                      "projections and the MLP are not in it"}
+        S = int(sel_len[0])
+        same = torch.equal(sel[0, :S].cpu(), ref_sels[0])
+        err = (attn[0].cpu().float() - ref_out[0].float()).abs().max().item()
+        result["parity"] = {"selected_slots_identical": bool(same),
+                            "attn_max_abs_err": round(err, 5)}
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "prefill"])
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default 200; 128 decode steps for the model workload)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps (default 20; model 4)")
+    ap.add_argument("--workload", default="c2",
+                    choices=["c1", "c2", "c3", "c4", "c5", "prefill", "model"])
     ap.add_argument("--cpu-reps", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--layers", type=int, default=32, help="layers for the tokens/s figure")
+    ap.add_argument("--layers", type=int, default=32,
+                    help="layers for the tokens/s figure; layers of the model workload")
+    ap.add_argument("--model-batch", type=int, default=4)
+    ap.add_argument("--model-context", type=int, default=262144)
+    ap.add_argument("--model-top-k", type=int, default=4096)
     ap.add_argument("--pools", type=int, default=4,
                     help="copies of the K/V pool cycled through, one per step")
     ap.add_argument("--trace-steps", type=int, default=64, help="decode steps of the c4 trace")
@@ -385,6 +493,10 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run five 256 MiB device copies (reference for counter runs)")
     args = ap.parse_args()
+    if args.steps is None:
+        args.steps = 128 if args.workload == "model" else 200
+    if args.warmup is None:
+        args.warmup = 4 if args.workload == "model" else 20
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the one-GPU hot path only; run with --gpus 1 "
                  "(no multi-GPU figure exists for it).")
@@ -398,6 +510,8 @@ def main():
         result = bench_trace(args, ops, workloads, dev)
     elif args.workload == "prefill":
         result = bench_prefill(args, ops, workloads, dev)
+    elif args.workload == "model":
+        result = bench_model(args, ops, dev)
     else:
         result = bench_layer(args, ops, workloads, dev)
     print(json.dumps(result), flush=True)

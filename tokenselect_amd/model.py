@@ -1,0 +1,155 @@
+"""A Llama-shaped decoder whose attention is the TokenSelect decode layer: the
+caller either side of the hot path, as the serving stack drives it
+(``RadixAttention.forward`` -> ``patched_radix_attention_forward`` tr.py:827-842:
+store the new token's K/V and append it to the token table, tr.py:844-854,
+332-336, then select and attend, tr.py:777-825) on every layer of the model.
+
+Only the attention goes through the library; the projections, norms and the MLP
+are torch's library GEMMs and elementwise kernels.  The model applies no rotary
+embedding of its own: keys are cached un-rotated and both the scoring query and
+the attention rotate inside the library (tr.py:381-392, 822).
+
+The KV cache is laid out as the reference's: one ``[rows, Hkv, D]`` K pool and V
+pool per layer, slot ids shared by all layers, a per-request table of slots per
+logical position (page size 1, tr.py:293-297) and a token count per layer and
+request (``num_tokens[layer]``, tr.py:298).
+"""
+
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import torch
+import torch.nn.functional as F
+
+from . import ops
+from .ops import Batch, DecodeLayer, LayerConfig, SelectionCache
+
+
+@dataclass
+class ModelConfig:
+    """Llama-3-8B by default."""
+    layers: int = 32
+    hidden: int = 4096
+    intermediate: int = 14336
+    vocab: int = 128256
+    num_heads: int = 32
+    num_kv_heads: int = 8
+    head_dim: int = 128
+    rms_eps: float = 1e-5
+    rope_theta: float = 5e5
+    init_std: float = 0.02
+    n_init: int = 128
+    n_local: int = 512
+    top_k: int = 4096
+
+    def layer_config(self) -> LayerConfig:
+        return LayerConfig(num_heads=self.num_heads, num_kv_heads=self.num_kv_heads,
+                           head_dim=self.head_dim, page_size=1, n_init=self.n_init,
+                           n_local=self.n_local, top_k=self.top_k, rope_theta=self.rope_theta)
+
+
+def _normal_bf16(shape, std: float, gen, device) -> torch.Tensor:
+    """N(0, std) in bf16, drawn in slabs so that no fp32 copy of a large tensor exists."""
+    out = torch.empty(shape, dtype=torch.bfloat16, device=device)
+    flat = out.view(-1)
+    slab = 1 << 28
+    for lo in range(0, flat.numel(), slab):
+        flat[lo:lo + slab].normal_(0.0, std, generator=gen)
+    return out
+
+
+class Decoder:
+    """Random-initialised decoder with a prefilled random KV cache.
+
+    ``contexts[b]`` tokens of request b are already cached (N(0,1) keys and
+    values, slots drawn from a random permutation); ``new_tokens`` more can be
+    decoded.  ``query_cache`` switches the selection cache on (one per layer,
+    tr.py:301-322); the reference serves with it off (tr.py:897)."""
+
+    def __init__(self, mc: ModelConfig, contexts: Sequence[int], new_tokens: int, device,
+                 seed: int = 0, query_cache: bool = False):
+        self.mc, self.cfg, self.device = mc, mc.layer_config(), device
+        self.contexts, self.new_tokens = list(contexts), new_tokens
+        B = self.batch = len(self.contexts)
+        gen = torch.Generator(device=device)
+        gen.manual_seed(seed)
+        hd, kvd = mc.num_heads * mc.head_dim, mc.num_kv_heads * mc.head_dim
+        std = mc.init_std
+        self.embed = _normal_bf16((mc.vocab, mc.hidden), std, gen, device)
+        self.lm_head = _normal_bf16((mc.vocab, mc.hidden), std, gen, device)
+        self.final_norm = torch.ones(mc.hidden, dtype=torch.bfloat16, device=device)
+        self.wqkv = [_normal_bf16((hd + 2 * kvd, mc.hidden), std, gen, device) for _ in range(mc.layers)]
+        self.wo = [_normal_bf16((mc.hidden, hd), std, gen, device) for _ in range(mc.layers)]
+        self.w_gate_up = [_normal_bf16((2 * mc.intermediate, mc.hidden), std, gen, device)
+                          for _ in range(mc.layers)]
+        self.w_down = [_normal_bf16((mc.hidden, mc.intermediate), std, gen, device)
+                       for _ in range(mc.layers)]
+        self.norm_in = [torch.ones(mc.hidden, dtype=torch.bfloat16, device=device)
+                        for _ in range(mc.layers)]
+        self.norm_post = [torch.ones(mc.hidden, dtype=torch.bfloat16, device=device)
+                          for _ in range(mc.layers)]
+
+        # KV cache: every request owns contexts[b] + new_tokens slots of the permutation.
+        self.max_len = max(self.contexts) + new_tokens
+        rows = sum(self.contexts) + B * new_tokens
+        order = torch.randperm(rows, generator=gen, device=device).to(torch.int32)
+        self.table = torch.zeros((B, self.max_len), dtype=torch.int32, device=device)
+        self.free = torch.empty((new_tokens, B), dtype=torch.int32, device=device)
+        at = 0
+        for b, L in enumerate(self.contexts):
+            self.table[b, :L] = order[at:at + L]
+            self.free[:, b] = order[at + L:at + L + new_tokens]
+            at += L + new_tokens
+        self.k_pools = [_normal_bf16((rows, mc.num_kv_heads, mc.head_dim), 1.0, gen, device)
+                        for _ in range(mc.layers)]
+        self.v_pools = [_normal_bf16((rows, mc.num_kv_heads, mc.head_dim), 1.0, gen, device)
+                        for _ in range(mc.layers)]
+        self.num_tokens = torch.tensor(self.contexts, dtype=torch.int32, device=device) \
+            .repeat(mc.layers, 1).contiguous()
+        self.decoded = 0
+        self.attention = DecodeLayer(self.cfg, B, self.max_len, device)
+        self.caches: List[Optional[SelectionCache]] = [
+            SelectionCache.allocate(self.cfg, B, device) if query_cache else None
+            for _ in range(mc.layers)]
+
+    def _norm(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        return F.rms_norm(x, (self.mc.hidden,), w, self.mc.rms_eps)
+
+    @torch.no_grad()
+    def decode_step(self, tokens: torch.Tensor, trace: Optional[list] = None) -> torch.Tensor:
+        """One forward over ``tokens`` [B] (the last token of every request): stores
+        their K/V, attends through the TokenSelect layer, returns the logits
+        ``[B, vocab]`` (bf16).  ``trace`` receives, per layer, clones of the query, key and
+        value rows, the attention output, the selected slots and their count."""
+        mc, cfg = self.mc, self.cfg
+        if self.decoded >= self.new_tokens:
+            raise RuntimeError("the KV cache has no slot left for another token")
+        loc = self.free[self.decoded]
+        max_len = max(self.contexts) + self.decoded + 1
+        hd, kvd = mc.num_heads * mc.head_dim, mc.num_kv_heads * mc.head_dim
+        x = self.embed[tokens]
+        for l in range(mc.layers):
+            qkv = F.linear(self._norm(x, self.norm_in[l]), self.wqkv[l])
+            q, k, v = qkv.split((hd, kvd, kvd), dim=-1)
+            q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+            ops.kv_store(cfg, k, v, loc, self.k_pools[l], self.v_pools[l], self.table,
+                         self.num_tokens[l])
+            attn, sel, _, sel_len = self.attention(
+                q, self.k_pools[l], self.v_pools[l], Batch(self.num_tokens[l], self.table, max_len),
+                self.caches[l])
+            if trace is not None:
+                trace.append((q.clone(), k.clone(), v.clone(), attn.clone(), sel.clone(), sel_len.clone()))
+            x = x + F.linear(attn, self.wo[l])
+            gate, up = F.linear(self._norm(x, self.norm_post[l]), self.w_gate_up[l]).chunk(2, dim=-1)
+            x = x + F.linear(F.silu(gate) * up, self.w_down[l])
+        self.decoded += 1
+        return F.linear(self._norm(x, self.final_norm), self.lm_head)
+
+    @torch.no_grad()
+    def generate(self, tokens: torch.Tensor, steps: int) -> torch.Tensor:
+        """Greedy decoding: ``[steps, B]`` token ids, no host synchronisation inside."""
+        out = torch.empty((steps, self.batch), dtype=torch.int64, device=self.device)
+        for t in range(steps):
+            tokens = self.decode_step(tokens).argmax(dim=-1)
+            out[t] = tokens
+        return out
