@@ -183,14 +183,21 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
 
   // Fingerprint: every request's single decode row is rotated to n_local
   // (tr.py:381-388); the mean over one row is the row itself (tr.py:392).  The same
-  // launch clears the counters the fused selection is going to add to.
+  // launch clears the counters the selection is going to add to.
+  const bool one_launch = fused.tokens_per_block > 0;
+  TopkArgs topk = make_topk_args(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache, sel,
+                                 sel_pos, sel_stride, sel_len, (uint32_t*)(ws + w.topk_ws));
+  topk.clear = tickets;
+  topk.clear_per_req = cfg->num_kv_heads;
   ZeroRegion zero_counters, zero_sync;
-  if (fused.tokens_per_block > 0)
+  if (one_launch)
     select_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_counters, &zero_sync);
+  else if (max_n > 0)
+    zero_counters = topk_zero_region(topk, bt->batch);
   if (chunk_rows > 0) {
     // Chunk fingerprint: row i rotated to n_local + i, mean over the rows (tr.py:380-392).
     TS_TRY(ts_fingerprint(cfg, q, chunk_rows, q_cos, q_sin, table_rows, qf, stream));
-    if (fused.tokens_per_block > 0) {
+    if (zero_counters.count > 0) {
       hipLaunchKernelGGL(select_zero_kernel, dim3(8), dim3(256), 0, (hipStream_t)stream,
                          zero_counters, zero_sync);
       TS_TRY(check_launch("select_zero_kernel"));
@@ -200,7 +207,7 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
                        zero_counters, zero_sync, (hipStream_t)stream));
   }
   if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
-  if (fused.tokens_per_block > 0) {
+  if (one_launch) {
     TS_TRY(launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,
                          nullptr, 0, ws + w.select_ws, tickets, cfg->num_kv_heads,
                          (hipStream_t)stream));
@@ -208,13 +215,14 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
     float* partials = (float*)(ws + w.partials);
     TS_TRY(ts_score(cfg, bt, qf, k_pool, pool_rows, hit, scores, w.score_stride, partials,
                     w.partials_bytes, stream));
-    TS_TRY(ts_vote(cfg, bt, scores, w.score_stride, partials, hit, stats, votes, pooled,
-                   w.score_stride, stream));
-    TopkArgs topk = make_topk_args(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache, sel,
-                                   sel_pos, sel_stride, sel_len, (uint32_t*)(ws + w.topk_ws));
-    topk.clear = tickets;
-    topk.clear_per_req = cfg->num_kv_heads;
-    TS_TRY(launch_topk(topk, bt->batch, max_n, (hipStream_t)stream));
+    // The vote kernel counts the first histogram level of the selection as it goes
+    // (not with max-pooling, which changes the votes afterwards).
+    const bool zeroed = max_n > 0;
+    TS_TRY(launch_vote(cfg, bt, scores, w.score_stride, partials, hit, stats, votes, pooled,
+                       w.score_stride, zeroed ? topk.ws : nullptr, topk.ws_stride,
+                       (hipStream_t)stream));
+    TS_TRY(launch_topk(topk, bt->batch, max_n, (hipStream_t)stream, zeroed,
+                       zeroed && cfg->pool_kernel <= 0));
   }
   if (chunk_rows > 0)
     return ts_sparse_prefill_attn(cfg, q, chunk_rows, k_pool, v_pool, pool_rows, sel, sel_len,

@@ -10,6 +10,7 @@ namespace ts {
 constexpr int kTopkBins = 2048;          // 11-bit digits
 constexpr int kTopkSlice = 512;          // candidates per workgroup of the hist / mark grids
 constexpr int kTopkFinalThreads = 1024;
+constexpr int kTopkPartWords = 1024;     // 32-bit bitmap words per workgroup of the final grid
 // Per-request workspace, in 32-bit words:
 //   [hist0: 2048][hist1: 2048][cand_count: 1, padded to 64]   <- zeroed before every selection
 //   [bitmap: 1 bit per candidate, 64-bit words]
@@ -121,6 +122,19 @@ TopkArgs make_topk_args(const ts_config* cfg, const ts_batch* bt, const float* v
                         int64_t vote_stride, const int32_t* hit, const ts_selcache* cache,
                         int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
                         uint32_t* workspace);
-int launch_topk(const TopkArgs& a, int batch, int max_n, hipStream_t stream);
+// counters_zeroed: an earlier kernel of the stream cleared the per-request counters
+// (topk_zero_region() says where they are); hist0_filled: the vote kernel was given
+// the workspace and has counted the first-level histogram already.
+int launch_topk(const TopkArgs& a, int batch, int max_n, hipStream_t stream,
+                bool counters_zeroed = false, bool hist0_filled = false);
+ZeroRegion topk_zero_region(const TopkArgs& a, int batch);
+
+// Soft vote (ts_vote.hip); with hist_ws (the top-k workspace, counters zeroed) the vote
+// kernel also fills the first-level histogram of the selection, unless max-pooling
+// comes between the votes and the selection.
+int launch_vote(const ts_config* cfg, const ts_batch* bt, const float* scores, int64_t score_stride,
+                const float* partials, const int32_t* skip, float* stats, float* votes,
+                float* pooled, int64_t vote_stride, uint32_t* hist_ws, size_t hist_ws_stride,
+                hipStream_t stream);
 
 }  // namespace ts

@@ -10,9 +10,10 @@
 //                                  store per wavefront); candidates inside bin t0
 //                                  are appended to a short list and histogrammed
 //                                  on their next 11 bits
-//   final  (one workgroup/request) resolves the remaining 21 bits on the short
-//                                  list (ties at the k-th key: lowest position
-//                                  first), sets their bits, then walks the bitmap
+//   final  (a few workgroups per request, one per slice of the bitmap) resolves
+//                                  the remaining 21 bits on the short list (ties
+//                                  at the k-th key: lowest position first), sets
+//                                  their bits, then walks its slice of the bitmap
 //                                  with a popcount prefix scan and emits the
 //                                  selected positions in ascending order, together
 //                                  with the sink and local-window segments and
@@ -106,7 +107,8 @@ __global__ __launch_bounds__(256) void topk_mark_kernel(TopkArgs a) {
 }
 
 __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs a) {
-  const int b = blockIdx.x;
+  const int b = blockIdx.y;
+  const int part = blockIdx.x, parts = gridDim.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const ReqGeom geo =
@@ -115,7 +117,9 @@ __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs 
   int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
   int32_t* sel_pos = a.sel_pos + (int64_t)b * a.sel_stride;
   const int L = geo.seq_len;
-  if (a.clear)
+  // This thread's share of a loop that the request's workgroups walk together.
+  const int first = part * kTopkFinalThreads + tid, step = parts * kTopkFinalThreads;
+  if (a.clear && part == 0)
     for (int i = tid; i < a.clear_per_req; i += kTopkFinalThreads)
       a.clear[(size_t)b * a.clear_per_req + i] = 0u;
 
@@ -125,30 +129,54 @@ __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs 
   };
 
   if (geo.dense) {  // tr.py:377-378, 741-744: attend over every token
-    for (int i = tid; i < L; i += kTopkFinalThreads) emit(i, i);
-    if (tid == 0) a.sel_len[b] = L;
+    for (int i = first; i < L; i += step) emit(i, i);
+    if (part == 0 && tid == 0) a.sel_len[b] = L;
     return;
   }
   const bool is_hit = a.hit && a.hit[b];
   const int k = is_hit ? min(a.cache_len[b], a.top_k) : geo.k;
-  if (tid == 0) a.sel_len[b] = a.n_init + k + a.n_local;
-  for (int i = tid; i < a.n_init; i += kTopkFinalThreads) emit(i, i);
-  for (int i = tid; i < a.n_local; i += kTopkFinalThreads) emit(a.n_init + k + i, L - a.n_local + i);
+  if (part == 0 && tid == 0) a.sel_len[b] = a.n_init + k + a.n_local;
+  for (int i = first; i < a.n_init; i += step) emit(i, i);
+  for (int i = first; i < a.n_local; i += step) emit(a.n_init + k + i, L - a.n_local + i);
   if (is_hit) {  // tr.py:419: reuse the cached positions
     const int32_t* cached = a.topk_cache + (int64_t)b * a.top_k;
-    for (int i = tid; i < k; i += kTopkFinalThreads) emit(a.n_init + i, cached[i]);
+    for (int i = first; i < k; i += step) emit(a.n_init + i, cached[i]);
     return;
   }
 
+  // The workgroups of a request split the position bitmap into consecutive slices
+  // of whole 32-bit words.  Each resolves the k-th key on its own (the histograms
+  // and the short list are small), sets the bits of the listed candidates that
+  // fall into its slice in an LDS copy, counts the selected positions before the
+  // slice, and emits its slice; no workgroup waits for another.
   const int n = pooled_count(geo.n, a.pool_kernel);
+  const int words = (n + 31) >> 5;
+  const int per_part = (words + parts - 1) / parts;  // <= kTopkPartWords by the launch grid
+  const int w_lo = min(part * per_part, words), w_hi = min(w_lo + per_part, words);
+  if (w_lo >= w_hi) return;
   uint32_t* ws = topk_ws(a.ws, a.ws_stride, b);
-  uint32_t* bitmap32 = ws + kTopkCounterWords;
+  const uint32_t* bitmap32 = ws + kTopkCounterWords;
   const uint2* cand = (const uint2*)(ws + kTopkCounterWords + a.bitmap_words);
   const int ncand = (int)min(ws[kTopkCandCount], (uint32_t)n);
 
   __shared__ uint32_t scratch[kTopkFinalThreads / 64 + 2];
   __shared__ uint32_t lh[1024];
-  auto mark = [&](uint32_t pos) { atomicOr(&bitmap32[pos >> 5], 1u << (pos & 31u)); };
+  __shared__ uint32_t lbits[kTopkPartWords];
+  uint32_t before = 0;  // selected positions before the slice, this thread's share
+  for (int w = tid; w < w_lo; w += kTopkFinalThreads) before += __popc(bitmap32[w]);
+  for (int w = w_lo + tid; w < w_hi; w += kTopkFinalThreads) {
+    uint32_t bits = bitmap32[w];
+    const int rem = n - (w << 5);
+    if (rem < 32) bits &= (1u << rem) - 1u;  // positions past n hold stale bits
+    lbits[w - w_lo] = bits;
+  }
+  auto mark = [&](uint32_t pos) {
+    const int w = (int)(pos >> 5);
+    if (w < w_lo)
+      ++before;
+    else if (w < w_hi)
+      atomicOr(&lbits[w - w_lo], 1u << (pos & 31u));
+  };
 
   uint32_t t0, above0, t1, above1, t2, above2;
   find_threshold_bin<kTopkBins>(ws + kTopkHist0, (uint32_t)k, scratch, t0, above0);
@@ -206,21 +234,20 @@ __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs 
         mark(c.y);
     }
   }
-  __threadfence();
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) before += __shfl_xor(before, off);
+  if (lane == 0) scratch[wave] = before;
+  __syncthreads();
+  uint32_t running = 0;  // selected positions before the words handled so far
+#pragma unroll
+  for (int x = 0; x < kTopkFinalThreads / 64; ++x) running += scratch[x];
   __syncthreads();
 
-  // Ordered emission: popcount prefix scan over the bitmap, one word per thread per round.
+  // Ordered emission: popcount prefix scan over the slice, one word per thread per round.
   int32_t* cache_out = a.topk_cache ? a.topk_cache + (int64_t)b * a.top_k : nullptr;
-  const int words = (n + 31) >> 5;
-  uint32_t running = 0;
-  for (int base = 0; base < words; base += kTopkFinalThreads) {
+  for (int base = w_lo; base < w_hi; base += kTopkFinalThreads) {
     const int w = base + tid;
-    uint32_t bits = 0;
-    if (w < words) {
-      bits = __hip_atomic_load(&bitmap32[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const int rem = n - (w << 5);
-      if (rem < 32) bits &= (1u << rem) - 1u;  // positions past n hold stale bits
-    }
+    uint32_t bits = w < w_hi ? lbits[w - w_lo] : 0u;
     const uint32_t cnt = __popc(bits);
     uint32_t incl = cnt;
 #pragma unroll
@@ -251,7 +278,7 @@ __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs 
     running += total;
     __syncthreads();
   }
-  if (tid == 0 && a.cache_len) a.cache_len[b] = k;
+  if (part == 0 && tid == 0 && a.cache_len) a.cache_len[b] = k;
 }
 
 static size_t bitmap_words_for(int max_n) {
@@ -299,18 +326,34 @@ TopkArgs make_topk_args(const ts_config* cfg, const ts_batch* bt, const float* v
   return a;
 }
 
-int launch_topk(const TopkArgs& a, int batch, int max_n, hipStream_t stream) {
+ZeroRegion topk_zero_region(const TopkArgs& a, int batch) {
+  ZeroRegion r;
+  r.base = a.ws;
+  r.stride = (int64_t)a.ws_stride;
+  r.words = kTopkCounterWords;
+  r.count = batch;
+  return r;
+}
+
+int launch_topk(const TopkArgs& a, int batch, int max_n, hipStream_t stream, bool counters_zeroed,
+                bool hist0_filled) {
   if (max_n > 0) {
     const dim3 grid((unsigned)ceil_div(max_n, kTopkSlice), (unsigned)batch);
-    hipLaunchKernelGGL(topk_zero_kernel, dim3((unsigned)batch), dim3(256), 0, stream, a.ws,
-                       a.ws_stride);
-    TS_TRY(check_launch("topk_zero_kernel"));
-    hipLaunchKernelGGL(topk_hist_kernel, grid, dim3(256), 0, stream, a);
-    TS_TRY(check_launch("topk_hist_kernel"));
+    if (!counters_zeroed) {
+      hipLaunchKernelGGL(topk_zero_kernel, dim3((unsigned)batch), dim3(256), 0, stream, a.ws,
+                         a.ws_stride);
+      TS_TRY(check_launch("topk_zero_kernel"));
+    }
+    if (!hist0_filled) {
+      hipLaunchKernelGGL(topk_hist_kernel, grid, dim3(256), 0, stream, a);
+      TS_TRY(check_launch("topk_hist_kernel"));
+    }
     hipLaunchKernelGGL(topk_mark_kernel, grid, dim3(256), 0, stream, a);
     TS_TRY(check_launch("topk_mark_kernel"));
   }
-  hipLaunchKernelGGL(topk_final_kernel, dim3((unsigned)batch), dim3(kTopkFinalThreads), 0, stream, a);
+  const int parts = max_n > 0 ? ceil_div(ceil_div(max_n, 32), kTopkPartWords) : 1;
+  hipLaunchKernelGGL(topk_final_kernel, dim3((unsigned)parts, (unsigned)batch),
+                     dim3(kTopkFinalThreads), 0, stream, a);
   return check_launch("topk_final_kernel");
 }
 

@@ -4,11 +4,12 @@
 // Scores arrive tile-major from the scoring pass: scores[b][tile][slot][16] with
 // head slot = kvh*G + g (see ts_score.hip); a thread owns one candidate and walks
 // the H slots of its tile, so a wavefront reads four contiguous 16*H*4-byte tiles.
-#include "ts_common.h"
+#include "ts_topk.h"
 
 namespace ts {
 
 constexpr int kMaxHeads = 128;
+constexpr int kVoteSlice = 1024;  // candidates per workgroup of the vote grid
 
 struct VoteArgs {
   const float* scores;
@@ -22,6 +23,10 @@ struct VoteArgs {
   int n_init, n_local, top_k, num_heads, num_kv_heads, head_map, max_seq_len;
   float* votes;
   int64_t vote_stride;
+  // Per-request top-k workspace whose first-level histogram the vote kernel fills
+  // (zero at launch), or NULL.
+  uint32_t* hist_ws;
+  size_t hist_ws_stride;
 };
 
 // Merge the per-workgroup softmax partials of one (request, head).
@@ -44,17 +49,21 @@ __global__ __launch_bounds__(64) void stats_merge_kernel(VoteArgs a) {
   }
 }
 
-// One thread per candidate; fp32 sum over the head slots in slot order.
+// A thread owns four candidates, 256 apart; fp32 sum over the head slots in slot
+// order.  With a top-k workspace attached the workgroup also counts its votes into the
+// first-level histogram of the selection (top 11 key bits) and adds its occupied bins
+// to the request's histogram at the end.
 __global__ __launch_bounds__(256) void vote_kernel(VoteArgs a) {
   const int b = blockIdx.y;
   if (a.skip && a.skip[b]) return;
   const ReqGeom geo =
       request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (blockIdx.x * 256 >= geo.n) return;
+  const int block_lo = blockIdx.x * kVoteSlice;
+  if (block_lo >= geo.n) return;
 
   __shared__ float s_max[kMaxHeads];
   __shared__ float s_rz[kMaxHeads];
+  __shared__ uint32_t lh[kTopkBins];
   const int H = a.num_heads;
   const int group = H / a.num_kv_heads;
   for (int slot = threadIdx.x; slot < H; slot += 256) {
@@ -63,21 +72,48 @@ __global__ __launch_bounds__(256) void vote_kernel(VoteArgs a) {
     s_max[slot] = a.stats[((size_t)b * H + h) * 2];
     s_rz[slot] = 1.0f / a.stats[((size_t)b * H + h) * 2 + 1];
   }
+  if (a.hist_ws)
+    for (int i = threadIdx.x; i < kTopkBins; i += 256) lh[i] = 0u;
   __syncthreads();
-  if (t >= geo.n) return;
 
-  const float* p = a.scores + ((size_t)b * a.score_stride + (size_t)(t & ~15)) * H + (t & 15);
-  float c = 0.f;
-  int slot = 0;
-  for (; slot + 8 <= H; slot += 8) {
-    float s[8];
+  constexpr int kPerThread = kVoteSlice / 256;
+  float c[kPerThread];
+  const float* p[kPerThread];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) s[i] = p[(slot + i) * 16];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) c += __expf(s[i] - s_max[slot + i]) * s_rz[slot + i];
+  for (int j = 0; j < kPerThread; ++j) {
+    const int t = min(block_lo + j * 256 + (int)threadIdx.x, geo.n - 1);  // clamped: no branch
+    p[j] = a.scores + ((size_t)b * a.score_stride + (size_t)(t & ~15)) * H + (t & 15);
+    c[j] = 0.f;
   }
-  for (; slot < H; ++slot) c += __expf(p[slot * 16] - s_max[slot]) * s_rz[slot];
-  a.votes[(size_t)b * a.vote_stride + t] = c;
+  int slot = 0;
+  for (; slot + 4 <= H; slot += 4) {
+    float s[kPerThread][4];
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[j][i] = p[j][(slot + i) * 16];
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) c[j] += __expf(s[j][i] - s_max[slot + i]) * s_rz[slot + i];
+  }
+  for (; slot < H; ++slot)
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) c[j] += __expf(p[j][slot * 16] - s_max[slot]) * s_rz[slot];
+#pragma unroll
+  for (int j = 0; j < kPerThread; ++j) {
+    const int t = block_lo + j * 256 + (int)threadIdx.x;
+    if (t < geo.n) {
+      a.votes[(size_t)b * a.vote_stride + t] = c[j];
+      if (a.hist_ws) atomicAdd(&lh[key_bin0(vote_key(c[j]))], 1u);
+    }
+  }
+  if (a.hist_ws) {
+    __syncthreads();
+    uint32_t* hist0 = topk_ws(a.hist_ws, a.hist_ws_stride, b) + kTopkHist0;
+    for (int i = threadIdx.x; i < kTopkBins; i += 256)
+      if (lh[i]) atomicAdd(&hist0[i], lh[i]);
+  }
 }
 
 struct PoolArgs {
@@ -109,14 +145,10 @@ __global__ __launch_bounds__(256) void pool_kernel(PoolArgs a) {
   a.pooled[(size_t)b * a.vote_stride + t] = m;
 }
 
-}  // namespace ts
-
-using namespace ts;
-
-extern "C" int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
-                       int64_t score_stride, const float* partials, const int32_t* skip,
-                       float* stats, float* votes, float* pooled, int64_t vote_stride,
-                       ts_stream_t stream) {
+int launch_vote(const ts_config* cfg, const ts_batch* bt, const float* scores, int64_t score_stride,
+                const float* partials, const int32_t* skip, float* stats, float* votes,
+                float* pooled, int64_t vote_stride, uint32_t* hist_ws, size_t hist_ws_stride,
+                hipStream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
   TS_REQUIRE(scores && partials && stats && votes, TS_EINVAL, "ts_vote: NULL tensor argument");
@@ -148,11 +180,13 @@ extern "C" int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* sc
   a.head_map = cfg->head_map;
   a.votes = votes;
   a.vote_stride = vote_stride;
+  a.hist_ws = cfg->pool_kernel > 0 ? nullptr : hist_ws;  // the selection sees the pooled votes
+  a.hist_ws_stride = hist_ws_stride;
   hipLaunchKernelGGL(stats_merge_kernel, dim3((unsigned)cfg->num_heads, (unsigned)bt->batch), dim3(64),
-                     0, (hipStream_t)stream, a);
+                     0, stream, a);
   TS_TRY(check_launch("stats_merge_kernel"));
-  hipLaunchKernelGGL(vote_kernel, dim3((unsigned)ceil_div(max_n, 256), (unsigned)bt->batch), dim3(256),
-                     0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(vote_kernel, dim3((unsigned)ceil_div(max_n, kVoteSlice), (unsigned)bt->batch),
+                     dim3(256), 0, stream, a);
   TS_TRY(check_launch("vote_kernel"));
 
   if (cfg->pool_kernel > 0) {
@@ -169,8 +203,20 @@ extern "C" int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* sc
     p.max_seq_len = bt->max_seq_len;
     p.kernel = cfg->pool_kernel;
     hipLaunchKernelGGL(pool_kernel, dim3((unsigned)ceil_div(max_n, 256), (unsigned)bt->batch),
-                       dim3(256), 0, (hipStream_t)stream, p);
+                       dim3(256), 0, stream, p);
     TS_TRY(check_launch("pool_kernel"));
   }
   return TS_OK;
+}
+
+}  // namespace ts
+
+using namespace ts;
+
+extern "C" int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
+                       int64_t score_stride, const float* partials, const int32_t* skip,
+                       float* stats, float* votes, float* pooled, int64_t vote_stride,
+                       ts_stream_t stream) {
+  return launch_vote(cfg, bt, scores, score_stride, partials, skip, stats, votes, pooled,
+                     vote_stride, nullptr, 0, (hipStream_t)stream);
 }
