@@ -4,10 +4,10 @@
 // Split-K in one launch: grid (splits, Hkv, B).  A workgroup owns a contiguous
 // range of the request's selected list for one KV head and keeps the G = H/Hkv
 // query heads that read it in registers.  Sixteen lanes gather one K row and one
-// V row (256 bytes each, 128-bit loads); the sixteen lane groups of a workgroup
-// walk the range with stride 16, eight tokens per lane group in flight (the slots,
-// then all sixteen rows, are requested before the first is used: the pass is
-// bound by memory latency, not bandwidth).  Keys are rotated to their index in
+// V row (256 bytes each, as two 128-byte halves); the sixteen lane groups of a
+// workgroup walk the range with stride 16, eight tokens per lane group in flight
+// (the slots, then all keys, then all values are requested before the first is
+// used: the pass is bound by memory latency, not bandwidth).  Keys are rotated to their index in
 // the selected list, the query to S-1; softmax is online in fp32.  Partial
 // (max, sum, acc) triples are merged across the lane groups and waves, written
 // with device-coherent stores, and the workgroup that draws the last ticket of
@@ -36,15 +36,11 @@ struct AttnArgs {
   uint16_t* out;      // [B,H,128] bf16
 };
 
-__device__ __forceinline__ void unpack8(const uint4& w, float (&f)[8]) {
+__device__ __forceinline__ void unpack4(const uint2& w, float* f) {
   f[0] = bf16_lo(w.x);
   f[1] = bf16_hi(w.x);
   f[2] = bf16_lo(w.y);
   f[3] = bf16_hi(w.y);
-  f[4] = bf16_lo(w.z);
-  f[5] = bf16_hi(w.z);
-  f[6] = bf16_lo(w.w);
-  f[7] = bf16_hi(w.w);
 }
 
 __device__ __forceinline__ float2 load_coherent2(const float* p) {
@@ -59,7 +55,15 @@ __device__ __forceinline__ void store_coherent2(float* p, float x, float y) {
 
 constexpr int kAttnInFlight = 8;  // tokens per lane group requested together
 
-// ROPE and CAP are compile-time so that the token loop carries no branches.
+// ROPE and CAP are compile-time so that the token loop carries no branches other
+// than the wave-uniform ones that skip tokens past the range.
+//
+// A lane owns four rotation pairs of the head dimension: dims 4*l16 .. 4*l16+3 and
+// their partners 64 dims further on, so a key row arrives as two 8-byte pieces per
+// lane (the sixteen lanes of a group still read two full 128-byte lines) and the
+// rotation needs no exchange between lanes.  The softmax runs on batches of tokens:
+// the logits of a batch are collected first, the running maximum moves once per
+// batch and every token costs one exponential per head.
 template <int G, bool ROPE, bool CAP>
 __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
@@ -70,10 +74,11 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int lg = tid >> 4;   // lane group 0..15 inside the workgroup
-  const int l16 = tid & 15;  // owns dims [8*l16, 8*l16+8)
-  const bool upper = l16 >= 8;  // second half of the head dimension
+  const int l16 = tid & 15;  // owns dims [4*l16, 4*l16+4) and [64+4*l16, 64+4*l16+4)
   const int H = a.num_heads;
   constexpr bool rope = ROPE;
+  // Tokens per softmax batch: as many as the registers allow at two waves per SIMD.
+  constexpr int kBatch = G <= 4 ? kAttnInFlight : (G == 7 ? 2 : 4);
   const int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
   const size_t row_elems = (size_t)a.num_kv_heads * kHeadDim;
 
@@ -88,21 +93,20 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   };
   load_slots(lo + lg);
 
-  // Frequencies of this lane's 8 rotation pairs (pair index = dim mod 64):
-  // theta^(-2 pair / 128) / scale.
-  float freq[8];
+  // Frequencies of this lane's 4 rotation pairs: theta^(-2 pair / 128) / scale.
+  float freq[4];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int pair = (l16 & 7) * 8 + e;
+  for (int e = 0; e < 4; ++e) {
+    const int pair = l16 * 4 + e;
     freq[e] = a.rope_rcp_scale * __builtin_amdgcn_exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
   }
 
-  // Query rows of the G heads, rotated to position S-1.
+  // Query rows of the G heads, rotated to position S-1: [0..3] low dims, [4..7] partners.
   float qv[G][8];
   {
-    float qc[8], qs[8];
+    float qc[4], qs[4];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
+    for (int e = 0; e < 4; ++e) {
       qc[e] = 1.f;
       qs[e] = 0.f;
       if (rope) sincos_reduced((float)(S - 1) * freq[e], qs[e], qc[e]);
@@ -110,19 +114,21 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       const uint16_t* qrow = a.q + ((size_t)b * H + (size_t)kvh * G + g) * kHeadDim;
-      float mine[8], other[8];
-      unpack8(*(const uint4*)(qrow + l16 * 8), mine);
-      unpack8(*(const uint4*)(qrow + (l16 ^ 8) * 8), other);
+      float x[4], y[4];
+      unpack4(*(const uint2*)(qrow + l16 * 4), x);
+      unpack4(*(const uint2*)(qrow + 64 + l16 * 4), y);
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        qv[g][e] = upper ? mine[e] * qc[e] + other[e] * qs[e] : mine[e] * qc[e] - other[e] * qs[e];
+      for (int e = 0; e < 4; ++e) {
+        qv[g][e] = x[e] * qc[e] - y[e] * qs[e];
+        qv[g][4 + e] = y[e] * qc[e] + x[e] * qs[e];
+      }
     }
   }
 
   // Key rotation state: angle of token j is j*freq; advance by 16 tokens per step.
-  float kc[8], ks[8], dc[8], ds[8];
+  float kc[4], ks[4], dc[4], ds[4];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
+  for (int e = 0; e < 4; ++e) {
     kc[e] = 1.f;
     ks[e] = 0.f;
     dc[e] = 1.f;
@@ -142,49 +148,103 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
     for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
   }
 
-  for (int j0 = lo + lg; j0 < hi; j0 += 16 * kAttnInFlight) {
-    uint4 kraw[kAttnInFlight], vraw[kAttnInFlight];
+  for (int j0 = lo + lg; j0 < hi + (lg & 3); j0 += 16 * kAttnInFlight) {
+    // The first token of the wavefront's four lane groups in this pass: a token
+    // step whose first token lies past the range is skipped by the whole wavefront.
+    const int wave_j0 = __builtin_amdgcn_readfirstlane(j0 - (lg & 3));
+    uint2 klo[kAttnInFlight], khi[kAttnInFlight], vlo[kAttnInFlight], vhi[kAttnInFlight];
 #pragma unroll
     for (int u = 0; u < kAttnInFlight; ++u) {
       const uint32_t sl = slot[u] < a.pool_rows ? slot[u] : a.pool_rows - 1;
-      const size_t at = (size_t)sl * row_elems + (size_t)kvh * kHeadDim + l16 * 8;
-      kraw[u] = *(const uint4*)(a.k_pool + at);
-      vraw[u] = *(const uint4*)(a.v_pool + at);
+      const size_t at = (size_t)sl * row_elems + (size_t)kvh * kHeadDim + l16 * 4;
+      klo[u] = *(const uint2*)(a.k_pool + at);
+      khi[u] = *(const uint2*)(a.k_pool + at + 64);
     }
-    if (j0 + 16 * kAttnInFlight < hi) load_slots(j0 + 16 * kAttnInFlight);
+    // The values after all the keys: the logits of the batch need every key, and
+    // the values arrive while they are being computed.
 #pragma unroll
     for (int u = 0; u < kAttnInFlight; ++u) {
-      const bool valid = j0 + 16 * u < hi;  // uniform over the 16 lanes of a group
-      float kf[8], vf[8];
-      unpack8(kraw[u], kf);
-      unpack8(vraw[u], vf);
-      if (rope) {
+      const uint32_t sl = slot[u] < a.pool_rows ? slot[u] : a.pool_rows - 1;
+      const size_t at = (size_t)sl * row_elems + (size_t)kvh * kHeadDim + l16 * 4;
+      vlo[u] = *(const uint2*)(a.v_pool + at);
+      vhi[u] = *(const uint2*)(a.v_pool + at + 64);
+    }
+    if (wave_j0 + 16 * kAttnInFlight < hi) load_slots(j0 + 16 * kAttnInFlight);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float partner = dpp_move<kRowRor8>(kf[e]);  // dim +-64 of the same token
-          kf[e] = upper ? kf[e] * kc[e] + partner * ks[e] : kf[e] * kc[e] - partner * ks[e];
-          const float c2 = kc[e] * dc[e] - ks[e] * ds[e];
-          ks[e] = ks[e] * dc[e] + kc[e] * ds[e];
-          kc[e] = c2;
+    for (int u0 = 0; u0 < kAttnInFlight; u0 += kBatch) {
+      if (wave_j0 + 16 * u0 >= hi) break;
+      // Logits of the batch; a token past the range gets -inf: weight 0, maximum
+      // unchanged (the running maximum starts at a finite value, so nothing becomes NaN).
+      float p[G][kBatch];
+#pragma unroll
+      for (int ub = 0; ub < kBatch; ++ub) {
+        const int u = u0 + ub;
+#pragma unroll
+        for (int g = 0; g < G; ++g) p[g][ub] = -INFINITY;
+        if (wave_j0 + 16 * u < hi) {
+          const bool valid = j0 + 16 * u < hi;  // uniform over the 16 lanes of a group
+          float kx[4], ky[4];
+          unpack4(klo[u], kx);
+          unpack4(khi[u], ky);
+          if (rope) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float x = kx[e] * kc[e] - ky[e] * ks[e];
+              ky[e] = ky[e] * kc[e] + kx[e] * ks[e];
+              kx[e] = x;
+            }
+          }
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            float d = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) d += qv[g][e] * kx[e] + qv[g][4 + e] * ky[e];
+            d = row16_sum(d) * a.sm_scale;
+            if (CAP) d = a.logit_cap * tanhf(d / a.logit_cap);
+            p[g][ub] = valid ? d : -INFINITY;
+          }
+        }
+        if (rope) {  // next token of this lane group: 16 positions further
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float c2 = kc[e] * dc[e] - ks[e] * ds[e];
+            ks[e] = ks[e] * dc[e] + kc[e] * ds[e];
+            kc[e] = c2;
+          }
         }
       }
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        float p = 0.f;
+        float mn = m[g];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) p += qv[g][e] * kf[e];
-        p = row16_sum(p) * a.sm_scale;
-        if (CAP) p = a.logit_cap * tanhf(p / a.logit_cap);
-        // A token past the range gets the logit -inf: weight 0, maximum unchanged
-        // (the running maximum starts at a finite value, so nothing becomes NaN).
-        p = valid ? p : -INFINITY;
-        const float mn = fmaxf(m[g], p);
+        for (int ub = 0; ub < kBatch; ++ub) mn = fmaxf(mn, p[g][ub]);
         const float alpha = __expf(m[g] - mn);
-        const float w = __expf(p - mn);
-        l[g] = l[g] * alpha + w;
+        float sum = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * alpha + w * vf[e];
+        for (int ub = 0; ub < kBatch; ++ub) {
+          p[g][ub] = __expf(p[g][ub] - mn);
+          sum += p[g][ub];
+        }
+        l[g] = l[g] * alpha + sum;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] *= alpha;
         m[g] = mn;
+      }
+#pragma unroll
+      for (int ub = 0; ub < kBatch; ++ub) {
+        const int u = u0 + ub;
+        if (wave_j0 + 16 * u < hi) {
+          float vx[4], vy[4];
+          unpack4(vlo[u], vx);
+          unpack4(vhi[u], vy);
+#pragma unroll
+          for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              acc[g][e] += p[g][ub] * vx[e];
+              acc[g][4 + e] += p[g][ub] * vy[e];
+            }
+        }
       }
     }
   }
@@ -207,7 +267,10 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
     }
     if (lane < 16) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sm_acc[wave][g][l16 * 8 + e] = acc[g][e];
+      for (int e = 0; e < 4; ++e) {
+        sm_acc[wave][g][l16 * 4 + e] = acc[g][e];
+        sm_acc[wave][g][64 + l16 * 4 + e] = acc[g][4 + e];
+      }
       if (lane == 0) {
         sm_m[wave][g] = m[g];
         sm_l[wave][g] = l[g];
@@ -285,9 +348,11 @@ __global__ __launch_bounds__(256) void attn_zero_kernel(uint32_t* tickets, int c
 
 static int attn_splits(int batch, int num_kv_heads, int max_sel_len) {
   // One batch of loads per lane group (16 groups x 8 tokens = 128 tokens per
-  // workgroup) as long as that keeps the grid near a thousand workgroups.
+  // workgroup) as long as the grid stays within the 512 workgroups that are
+  // resident at once (two per CU): a second round of workgroups pays the start-up
+  // and merge latencies again, which costs more than longer ranges do.
   int64_t want = ceil_div(max_sel_len, 16 * kAttnInFlight);
-  const int64_t cap = ceil_div(1024, (int64_t)batch * num_kv_heads);
+  const int64_t cap = ceil_div(512, (int64_t)batch * num_kv_heads);
   if (want > cap) want = cap;
   if (want < 1) want = 1;
   return (int)want;
