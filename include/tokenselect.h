@@ -211,6 +211,22 @@ int ts_kv_store(const ts_config* cfg, const void* k, const void* v, const int32_
                 int64_t table_stride, int32_t* seq_lens, int32_t batch, int32_t max_tokens,
                 ts_stream_t stream);
 
+/* The QKV projection of a decode step with the KV store as its epilogue: what the
+ * serving stack does in two places, qkv = x W^T (+ bias) in the model's attention
+ * module and then patched_radix_attention_store_kv_cache (tr.py:844-854) +
+ * add_k_cache (tr.py:332-336), in one pass over W.  Columns [0, H*D) of the product
+ * go to q_out [batch, H*D]; the next Hkv*D to k_pool[loc[b]], the last Hkv*D to
+ * v_pool[loc[b]]; then table[b][seq_lens[b]] = loc[b], seq_lens[b] += 1 as
+ * ts_kv_store does (a full table leaves table and length alone).  x: [batch, hidden]
+ * bf16; w: [(H + 2 Hkv) * D, hidden] bf16 row-major (torch Linear weight);
+ * bias: [(H + 2 Hkv) * D] bf16 or NULL; fp32 accumulation, bf16 outputs.
+ * batch <= 8 and hidden a multiple of 8, at most 4096 (TS_ESHAPE otherwise: use a
+ * library GEMM and ts_kv_store). */
+int ts_qkv_store(const ts_config* cfg, const void* x, const void* w, const void* bias,
+                 int32_t hidden, const int32_t* out_cache_loc, void* q_out, void* k_pool,
+                 void* v_pool, int64_t pool_rows, int32_t* table, int64_t table_stride,
+                 int32_t* seq_lens, int32_t batch, int32_t max_tokens, ts_stream_t stream);
+
 /* ---- chunked prefill (patched_radix_attention_extend_forward_flashinfer,
  * tr.py:703-775): per chunk of at most 512 rows of one request the chunk's K/V
  * are stored, one selection is made from the mean of the chunk's rotated

@@ -42,12 +42,14 @@ def _cpu_forward(m: Decoder, tokens, kc, vc, tab, lens, loc):
     return norm(x, m.final_norm) @ m.lm_head.cpu().float().T
 
 
-@pytest.mark.parametrize("query_cache", [False, True], ids=["plain", "query_cache"])
-def test_decoder_steps_match_the_oracle(dev, query_cache):
-    say(f"toy decoder, query_cache={query_cache}")
+@pytest.mark.parametrize("query_cache,fused_qkv", [(False, True), (False, False), (True, True)],
+                         ids=["plain", "plain-gemm-then-store", "query_cache"])
+def test_decoder_steps_match_the_oracle(dev, query_cache, fused_qkv):
+    say(f"toy decoder, query_cache={query_cache} fused_qkv={fused_qkv}")
     mc = ModelConfig(**TOY)
     contexts, steps = [300, 41], 3          # the second request attends densely
-    m = Decoder(mc, contexts, steps, dev, seed=21, query_cache=query_cache)
+    m = Decoder(mc, contexts, steps, dev, seed=21, query_cache=query_cache, fused_qkv=fused_qkv)
+    assert m.fused_qkv == fused_qkv
     c = m.cfg
     kc = [p.cpu().clone() for p in m.k_pools]
     vc = [p.cpu().clone() for p in m.v_pools]

@@ -72,6 +72,8 @@ SIGNATURES = {
                                      _ptr, _ptr, _size, _ptr]),
     "ts_kv_store": (_i32, [_CFG, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
                            _ptr]),
+    "ts_qkv_store": (_i32, [_CFG, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr,
+                            _i32, _i32, _ptr]),
     "ts_kv_store_chunk": (_i32, [_CFG, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i32, _ptr]),
     "ts_fingerprint": (_i32, [_CFG, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr]),
     "ts_prefill_attn_workspace_bytes": (_size, [_CFG, _i32]),

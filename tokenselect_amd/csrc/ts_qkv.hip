@@ -1,0 +1,209 @@
+// QKV projection of a decode step with the KV store as its epilogue: the step
+// before the hot path.  The serving stack computes qkv = x W^T in the model
+// (LlamaAttention.forward) and the patched attention then scatters K and V into the
+// pool and appends the slot to the token table (patched_radix_attention_store_kv_cache
+// tr.py:844-854, add_k_cache tr.py:332-336); here the projection writes the K and V
+// rows straight to their pool slot, so the [B, Hkv*D] staging rows, their copies
+// and the separate store launch disappear.
+//
+// With a handful of rows in x the product is a stream over W (bound: HBM).  A
+// wavefront owns two whole rows of W: a lane reads up to eight 16-byte pieces of
+// each (all requested before the first is used, before x is staged), multiplies
+// them with the matching pieces of x from LDS (bf16, staged once per workgroup of
+// eight wavefronts) and the wavefront reduces its 2 x B sums on its own: no
+// exchange between wavefronts.
+#include "ts_common.h"
+
+namespace ts {
+
+constexpr int kQkvMaxBatch = 8;      // rows of x
+constexpr int kQkvRows = 2;          // rows of W per wavefront
+constexpr int kQkvWaves = 8;         // wavefronts per workgroup
+constexpr int kQkvPieces = 8;        // 16-byte pieces of a row per lane
+constexpr int kQkvMaxHidden = 4096;  // 64 lanes x kQkvPieces x 8 elements
+
+struct QkvArgs {
+  const uint16_t* x;     // [B, hidden] bf16
+  const uint16_t* w;     // [n_out, hidden] bf16
+  const uint16_t* bias;  // [n_out] bf16 or NULL
+  int hidden, n_out, q_cols, kv_cols;
+  const int32_t* loc;    // [B] pool slot of the new token
+  uint16_t* q_out;       // [B, q_cols]
+  uint16_t* k_pool;
+  uint16_t* v_pool;
+  int64_t pool_rows;
+  int32_t* table;
+  int64_t table_stride;
+  int32_t* seq_lens;
+  int max_tokens;
+};
+
+__device__ __forceinline__ void unpack8(const uint4& w, float (&f)[8]) {
+  f[0] = bf16_lo(w.x);
+  f[1] = bf16_hi(w.x);
+  f[2] = bf16_lo(w.y);
+  f[3] = bf16_hi(w.y);
+  f[4] = bf16_lo(w.z);
+  f[5] = bf16_hi(w.z);
+  f[6] = bf16_lo(w.w);
+  f[7] = bf16_hi(w.w);
+}
+
+// W is read once: a non-temporal load keeps it from displacing the rest of the cache.
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+__device__ __forceinline__ uint4 load_streaming(const uint4* p) {
+  const u32x4_t v = __builtin_nontemporal_load((const u32x4_t*)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+template <int B>
+__global__ __launch_bounds__(64 * kQkvWaves) void qkv_store_kernel(QkvArgs a) {
+  extern __shared__ uint4 lds_x[];  // [B][hidden / 8]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int kvec = a.hidden >> 3;  // 16-byte pieces per row
+  const int n0 = (blockIdx.x * kQkvWaves + wave) * kQkvRows;
+
+  // The wavefront's rows first: they do not depend on the copy of x.
+  uint4 wv[kQkvRows][kQkvPieces];
+#pragma unroll
+  for (int r = 0; r < kQkvRows; ++r) {
+    const uint4* row = (const uint4*)(a.w + (size_t)min(n0 + r, a.n_out - 1) * a.hidden);
+#pragma unroll
+    for (int j = 0; j < kQkvPieces; ++j) {
+      const int v = lane + 64 * j;
+      wv[r][j] = v < kvec ? load_streaming(row + v) : make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+  for (int i = tid; i < B * kvec; i += 64 * kQkvWaves) lds_x[i] = ((const uint4*)a.x)[i];
+  __syncthreads();
+
+  float acc[kQkvRows][B];
+#pragma unroll
+  for (int r = 0; r < kQkvRows; ++r)
+#pragma unroll
+    for (int b = 0; b < B; ++b) acc[r][b] = 0.f;
+#pragma unroll
+  for (int j = 0; j < kQkvPieces; ++j) {
+    const int v = min(lane + 64 * j, kvec - 1);  // past the row: W piece is zero
+    float wf[kQkvRows][8];
+#pragma unroll
+    for (int r = 0; r < kQkvRows; ++r) unpack8(wv[r][j], wf[r]);
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      float xf[8];
+      unpack8(lds_x[b * kvec + v], xf);
+#pragma unroll
+      for (int r = 0; r < kQkvRows; ++r)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[r][b] += wf[r][e] * xf[e];
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < kQkvRows; ++r)
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) acc[r][b] += __shfl_xor(acc[r][b], off);
+    }
+  // Lane r * B + b writes y[b][n0 + r] (every lane holds every sum).
+  float y = 0.f;
+#pragma unroll
+  for (int r = 0; r < kQkvRows; ++r)
+#pragma unroll
+    for (int b = 0; b < B; ++b)
+      if (lane == r * B + b) y = acc[r][b];
+  if (lane < kQkvRows * B) {
+    const int r = lane / B, b = lane % B;
+    const int n = n0 + r;
+    if (n < a.n_out) {
+      if (a.bias) y += bf16_to_f32(a.bias[n]);
+      const uint16_t out = f32_to_bf16(y);
+      if (n < a.q_cols) {
+        a.q_out[(size_t)b * a.q_cols + n] = out;
+      } else {
+        const int64_t slot = a.loc[b];
+        if (slot >= 0 && slot < a.pool_rows) {
+          const int c = n - a.q_cols;
+          if (c < a.kv_cols)
+            a.k_pool[(size_t)slot * a.kv_cols + c] = out;
+          else
+            a.v_pool[(size_t)slot * a.kv_cols + (c - a.kv_cols)] = out;
+        }
+      }
+    }
+  }
+
+  // Table append (add_k_cache tr.py:332-336) by the first workgroup; a full table
+  // (tr.py:334 asserts) or a slot outside the pool leaves table and length alone.
+  if (blockIdx.x == 0 && tid < B) {
+    const int b = tid;
+    const int slot = a.loc[b];
+    const int len = a.seq_lens[b];
+    if (slot >= 0 && slot < a.pool_rows && len < a.max_tokens) {
+      a.table[(int64_t)b * a.table_stride + len] = slot;
+      a.seq_lens[b] = len + 1;
+    }
+  }
+}
+
+template <int B>
+static int launch_qkv(const QkvArgs& a, hipStream_t stream) {
+  const size_t lds = (size_t)B * a.hidden * 2;  // at most 64 KB
+  hipLaunchKernelGGL(qkv_store_kernel<B>,
+                     dim3((unsigned)ceil_div(a.n_out, kQkvRows * kQkvWaves)), dim3(64 * kQkvWaves),
+                     lds, stream, a);
+  return check_launch("qkv_store_kernel");
+}
+
+}  // namespace ts
+
+using namespace ts;
+
+extern "C" int ts_qkv_store(const ts_config* cfg, const void* x, const void* w, const void* bias,
+                            int32_t hidden, const int32_t* out_cache_loc, void* q_out,
+                            void* k_pool, void* v_pool, int64_t pool_rows, int32_t* table,
+                            int64_t table_stride, int32_t* seq_lens, int32_t batch,
+                            int32_t max_tokens, ts_stream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_REQUIRE(x && w && out_cache_loc && q_out && k_pool && v_pool && table && seq_lens, TS_EINVAL,
+             "ts_qkv_store: NULL tensor argument");
+  TS_REQUIRE(cfg->page_size == 1, TS_EINVAL, "ts_qkv_store appends to a per-token table (page_size 1)");
+  TS_REQUIRE(batch >= 1 && batch <= kQkvMaxBatch, TS_ESHAPE,
+             "ts_qkv_store: batch %d outside 1..%d (use a library GEMM and ts_kv_store)", batch,
+             kQkvMaxBatch);
+  TS_REQUIRE(hidden >= 8 && hidden % 8 == 0 && hidden <= kQkvMaxHidden, TS_ESHAPE,
+             "ts_qkv_store: hidden %d must be a multiple of 8, at most %d", hidden, kQkvMaxHidden);
+  TS_REQUIRE(pool_rows >= 1 && max_tokens >= 1, TS_EINVAL,
+             "ts_qkv_store: pool_rows=%lld max_tokens=%d out of range", (long long)pool_rows,
+             max_tokens);
+  TS_REQUIRE(batch == 1 || table_stride >= max_tokens, TS_EINVAL,
+             "ts_qkv_store: table_stride %lld < max_tokens %d", (long long)table_stride, max_tokens);
+  QkvArgs a;
+  a.x = (const uint16_t*)x;
+  a.w = (const uint16_t*)w;
+  a.bias = (const uint16_t*)bias;
+  a.hidden = hidden;
+  a.q_cols = cfg->num_heads * cfg->head_dim;
+  a.kv_cols = cfg->num_kv_heads * cfg->head_dim;
+  a.n_out = a.q_cols + 2 * a.kv_cols;
+  a.loc = out_cache_loc;
+  a.q_out = (uint16_t*)q_out;
+  a.k_pool = (uint16_t*)k_pool;
+  a.v_pool = (uint16_t*)v_pool;
+  a.pool_rows = pool_rows;
+  a.table = table;
+  a.table_stride = table_stride;
+  a.seq_lens = seq_lens;
+  a.max_tokens = max_tokens;
+  switch (batch) {
+    case 1: return launch_qkv<1>(a, (hipStream_t)stream);
+    case 2: return launch_qkv<2>(a, (hipStream_t)stream);
+    case 3: return launch_qkv<3>(a, (hipStream_t)stream);
+    case 4: return launch_qkv<4>(a, (hipStream_t)stream);
+    case 5: return launch_qkv<5>(a, (hipStream_t)stream);
+    case 6: return launch_qkv<6>(a, (hipStream_t)stream);
+    case 7: return launch_qkv<7>(a, (hipStream_t)stream);
+    default: return launch_qkv<8>(a, (hipStream_t)stream);
+  }
+}

@@ -64,10 +64,12 @@ class Decoder:
     ``contexts[b]`` tokens of request b are already cached (N(0,1) keys and
     values, slots drawn from a random permutation); ``new_tokens`` more can be
     decoded.  ``query_cache`` switches the selection cache on (one per layer,
-    tr.py:301-322); the reference serves with it off (tr.py:897)."""
+    tr.py:301-322); the reference serves with it off (tr.py:897).  ``fused_qkv``
+    (default: where the shape allows) runs the QKV projection with the KV store as
+    its epilogue instead of a library GEMM followed by ``ts_kv_store``."""
 
     def __init__(self, mc: ModelConfig, contexts: Sequence[int], new_tokens: int, device,
-                 seed: int = 0, query_cache: bool = False):
+                 seed: int = 0, query_cache: bool = False, fused_qkv: Optional[bool] = None):
         self.mc, self.cfg, self.device = mc, mc.layer_config(), device
         self.contexts, self.new_tokens = list(contexts), new_tokens
         B = self.batch = len(self.contexts)
@@ -107,6 +109,9 @@ class Decoder:
         self.num_tokens = torch.tensor(self.contexts, dtype=torch.int32, device=device) \
             .repeat(mc.layers, 1).contiguous()
         self.decoded = 0
+        # QKV projection + KV store in one kernel where the library serves the shape.
+        supported = ops.qkv_store_supported(B, mc.hidden)
+        self.fused_qkv = supported if fused_qkv is None else (fused_qkv and supported)
         self.attention = DecodeLayer(self.cfg, B, self.max_len, device)
         self.caches: List[Optional[SelectionCache]] = [
             SelectionCache.allocate(self.cfg, B, device) if query_cache else None
@@ -129,15 +134,23 @@ class Decoder:
         hd, kvd = mc.num_heads * mc.head_dim, mc.num_kv_heads * mc.head_dim
         x = self.embed[tokens]
         for l in range(mc.layers):
-            qkv = F.linear(self._norm(x, self.norm_in[l]), self.wqkv[l])
-            q, k, v = qkv.split((hd, kvd, kvd), dim=-1)
-            q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-            ops.kv_store(cfg, k, v, loc, self.k_pools[l], self.v_pools[l], self.table,
-                         self.num_tokens[l])
+            h = self._norm(x, self.norm_in[l])
+            if self.fused_qkv:  # projection with the KV store as its epilogue
+                q = ops.qkv_store(cfg, h, self.wqkv[l], None, loc, self.k_pools[l], self.v_pools[l],
+                                  self.table, self.num_tokens[l])
+                k = v = None
+            else:
+                q, k, v = F.linear(h, self.wqkv[l]).split((hd, kvd, kvd), dim=-1)
+                q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+                ops.kv_store(cfg, k, v, loc, self.k_pools[l], self.v_pools[l], self.table,
+                             self.num_tokens[l])
             attn, sel, _, sel_len = self.attention(
                 q, self.k_pools[l], self.v_pools[l], Batch(self.num_tokens[l], self.table, max_len),
                 self.caches[l])
             if trace is not None:
+                if k is None:   # the rows as they landed in the pools
+                    k = self.k_pools[l][loc.long()].reshape(self.batch, kvd)
+                    v = self.v_pools[l][loc.long()].reshape(self.batch, kvd)
                 trace.append((q.clone(), k.clone(), v.clone(), attn.clone(), sel.clone(), sel_len.clone()))
             x = x + F.linear(attn, self.wo[l])
             gate, up = F.linear(self._norm(x, self.norm_post[l]), self.w_gate_up[l]).chunk(2, dim=-1)

@@ -407,6 +407,54 @@ def kv_store(cfg: LayerConfig, k: torch.Tensor, v: torch.Tensor, out_cache_loc: 
                                        _p(seq_lens), B, table.shape[1], _stream()))
 
 
+QKV_STORE_MAX_BATCH = 8
+
+
+def qkv_store_supported(batch: int, hidden: int) -> bool:
+    """Shapes :func:`qkv_store` serves; others take a library GEMM and :func:`kv_store`."""
+    return 1 <= batch <= QKV_STORE_MAX_BATCH and 8 <= hidden <= 4096 and hidden % 8 == 0
+
+
+def qkv_store(cfg: LayerConfig, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+              out_cache_loc: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+              table: torch.Tensor, seq_lens: torch.Tensor,
+              q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """QKV projection of a decode step with the KV store + table append as its epilogue
+    (the model's ``qkv_proj`` followed by tr.py:844-854, 332-336) in one pass over the
+    weight.  ``x`` [B, hidden] bf16, ``weight`` [(H+2Hkv)*D, hidden] bf16 (a torch
+    ``Linear`` weight), ``bias`` [(H+2Hkv)*D] bf16 or None.  Returns ``q`` [B, H*D] bf16;
+    K and V land in the pools at ``out_cache_loc``."""
+    c = cfg.to_c()
+    _need(x, "x", torch.bfloat16, 2)
+    _need(weight, "weight", torch.bfloat16, 2)
+    if bias is not None:
+        _need(bias, "bias", torch.bfloat16, 1)
+    _need(out_cache_loc, "out_cache_loc", torch.int32, 1)
+    _check_pool(cfg, k_pool, "k_pool")
+    _check_pool(cfg, v_pool, "v_pool")
+    _need(table, "table", torch.int32, 2)
+    _need(seq_lens, "seq_lens", torch.int32, 1)
+    B, hidden = x.shape
+    n_out = (cfg.num_heads + 2 * cfg.num_kv_heads) * cfg.head_dim
+    if tuple(weight.shape) != (n_out, hidden) or (bias is not None and bias.shape[0] != n_out):
+        raise ValueError(f"weight must be [{n_out}, {hidden}] (and bias [{n_out}])")
+    if out_cache_loc.shape[0] != B or table.shape[0] != B or seq_lens.shape[0] != B:
+        raise ValueError("out_cache_loc / table / seq_lens do not match the batch")
+    if k_pool.shape != v_pool.shape:
+        raise ValueError("k_pool and v_pool must have the same shape")
+    if q_out is None:
+        q_out = torch.empty((B, cfg.num_heads * cfg.head_dim), dtype=torch.bfloat16, device=x.device)
+    else:
+        _need(q_out, "q_out", torch.bfloat16, 2)
+        if tuple(q_out.shape) != (B, cfg.num_heads * cfg.head_dim):
+            raise ValueError("q_out must be [B, H*D]")
+    _lib.check(_lib.load().ts_qkv_store(
+        ctypes.byref(c), _p(x), _p(weight), _p(bias), hidden, _p(out_cache_loc), _p(q_out), _p(k_pool),
+        _p(v_pool), k_pool.shape[0], _p(table), table.stride(0), _p(seq_lens), B, table.shape[1],
+        _stream()))
+    return q_out
+
+
 def scoring_cos_sin(head_dim: int, rope_base: float, rope_scale, n_local: int, device):
     """Row ``n_local`` of the reference's cos/sin tables (tr.py:75-96), built with
     the same fp32 torch expressions on the host: ``(cos [1,D], sin [1,D])``."""
