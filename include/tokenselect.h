@@ -163,10 +163,12 @@ int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
  * The scores stay in LDS.  The workgroups of the launch meet six times: softmax
  * partials, merged statistics, three histogram rounds over the 11 + 11 + 10
  * bits of the vote keys, and the per-workgroup counts that place each
- * workgroup's selected positions in the output.  Outputs and the hit / cache
- * arguments are those of ts_topk_ragged (same tie rule: lowest position first);
- * votes, when not NULL, also receives the [B, vote_stride] fp32 votes.
- * Usable when ts_select_supported() returns 1: pool_kernel off and batch x
+ * workgroup's selected positions in the output (seven times with
+ * cfg->pool_kernel > 0: the max-pool of tr.py:366-369 needs the votes of the
+ * neighbouring workgroups).  Outputs and the hit / cache arguments are those of
+ * ts_topk_ragged (same tie rule: lowest position first); votes, when not NULL,
+ * also receives the [B, vote_stride] fp32 votes (pooled when pool_kernel > 0).
+ * Usable when ts_select_supported() returns 1: pool_kernel at most 256 and batch x
  * candidates small enough (some 260K candidates for 32 heads) for the scores to
  * fit the LDS of the device; TS_ESHAPE otherwise, and the caller runs
  * ts_score + ts_vote + ts_topk_ragged.  The launch is an ordinary one sized so

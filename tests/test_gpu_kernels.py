@@ -175,11 +175,66 @@ def test_fused_select_ties(dev):
 
 
 def test_fused_select_rejects_unsupported(dev):
-    say("fused select: pool_kernel on -> TS_ESHAPE")
-    wl = small(dev, SHAPES[0], seed=3, lens=[2000], ks=[64], pool_kernel=5)
+    say("fused select: pool_kernel above 256 -> TS_ESHAPE")
+    wl = small(dev, SHAPES[0], seed=3, lens=[2000], ks=[64], pool_kernel=300)
     assert not ops.select_supported(wl.cfg, 1, 2000)
     with pytest.raises(RuntimeError, match="ts_select"):
         ops.select(wl.cfg, wl.batch, fingerprint(wl, dev), wl.k_pool)
+
+
+@pytest.mark.parametrize("kernel", [5, 6, 32, 128, 255])
+@pytest.mark.parametrize("page", [1, 16])
+def test_fused_select_max_pool(dev, kernel, page):
+    """Max-pooled votes inside the single-launch selection (the neighbours' votes cross
+    workgroup borders): against the oracle, and exact on the kernel's own pooled votes,
+    where runs of equal values make ties at the k-th vote the rule."""
+    lens, ks = [3000, 777, 40, 1531], [64, 100, 64, 17]
+    say(f"fused select with max-pool kernel={kernel} page={page}")
+    wl = small(dev, SHAPES[0], seed=60 + kernel, lens=lens, ks=ks, page=page, top_k=100,
+               pool_kernel=kernel)
+    c = wl.cfg
+    assert ops.select_supported(c, len(lens), max(lens))
+    qf = fingerprint(wl, dev)
+    details = []
+    oracle_layer(wl, details)
+    space = None
+    for attempt in range(2):
+        sel, sel_pos, sel_len, votes, space = ops.select(c, wl.batch, qf, wl.k_pool,
+                                                         want_votes=True, workspace=space)
+        torch.cuda.synchronize()
+        assert not ops.select_fault(c, wl.batch, space)
+        for b, (L, k) in enumerate(zip(wl.seq_lens, wl.k_list)):
+            S = int(sel_len[b])
+            if not details[b]:  # dense
+                assert S == L
+                continue
+            n_out = details[b]["votes"].shape[0]
+            assert n_out == L - c.n_init - c.n_local - (1 if kernel % 2 == 0 else 0)
+            v = votes[b, :n_out]
+            assert torch.allclose(v.cpu(), details[b]["votes"], rtol=2e-4, atol=1e-9), \
+                f"pooled votes b={b} attempt={attempt}"
+            mid = sel_pos[b, c.n_init:c.n_init + k].long()
+            assert S == c.n_init + k + c.n_local
+            assert bool((mid[1:] > mid[:-1]).all())
+            assert_index_sets_match(mid.cpu(), details[b]["top_pos"], details[b]["votes"], c.n_init,
+                                    f"fused pooled top-k b={b} attempt={attempt}", rtol=3e-4)
+            chosen = torch.zeros(n_out, dtype=torch.bool, device=dev)
+            chosen[mid - c.n_init] = True
+            lowest_in, highest_out = v[chosen].min(), v[~chosen].max()
+            assert float(lowest_in) >= float(highest_out)
+            tied_in = torch.nonzero(chosen & (v == lowest_in)).flatten()
+            tied_out = torch.nonzero(~chosen & (v == lowest_in)).flatten()
+            if tied_out.numel():
+                assert int(tied_in.max()) < int(tied_out.min()), f"tie order b={b}"
+
+
+@pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
+def test_decode_layer_max_pool(dev, fused_select):
+    lens, ks = [5000, 100, 2048, 901], [256, 256, 200, 256]
+    say(f"decode_layer with max-pool, fused={fused_select}")
+    wl = small(dev, SHAPES[0], seed=71, lens=lens, ks=ks, page=16, top_k=256, n_init=16, n_local=32,
+               pool_kernel=9)
+    check_layer(wl, dev, "decode_layer max-pool")
 
 
 def test_topk_ties_and_extremes(dev):

@@ -41,6 +41,9 @@ struct ScoreArgs {
   uint32_t* clear;        // words to clear for the next kernel of the stream, or NULL
   int clear_per_req;
   uint64_t spin_ticks;    // bound of a grid-wide wait, in 100 MHz ticks
+  int pool_kernel;        // max-pool window over the votes (tr.py:366-369), <= 0: off
+  float* pool_votes;      // [B,pool_stride] un-pooled votes exchanged between workgroups
+  int64_t pool_stride;
 };
 
 // Selection counters of one request, in 32-bit words.  The first histogram is kept
@@ -56,7 +59,8 @@ constexpr int kSelCounterWords = kSelMaxBin + 64;
 
 // Workspace of ts_select, carved in this order (256-byte aligned pieces).
 struct SelectWorkspace {
-  size_t partials, stats, counters, block_counts, sync, total;
+  size_t partials, stats, counters, block_counts, pool_votes, sync, total;  // sync stays last
+  int64_t pool_stride;
   int tokens_per_block;  // 0: the shape does not fit the fused kernel
   int blocks_per_req;
 };

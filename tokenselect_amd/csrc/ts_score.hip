@@ -263,7 +263,8 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     if constexpr (MODE == kScoreFused) {  // no tokens here: only help with the statistics
       grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
       merge_request_stats(a, team, threadIdx.x & 63, threadIdx.x >> 6);
-      for (uint32_t round = 2; round <= kSelectRounds; ++round)
+      const uint32_t rounds = kSelectRounds + (a.pool_kernel > 0 ? 1u : 0u);
+      for (uint32_t round = 2; round <= rounds; ++round)
         grid_arrive(a.sync, round, false, a.spin_ticks, team.size, team.index);
     }
     return;
@@ -528,8 +529,46 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         for (int j = 0; j < 8; ++j)
           if (s0 + j < HKV * G) c += __expf(x[j] - s_max[s0 + j]) * s_rz[s0 + j];
       }
-      if (a.votes) a.votes[(size_t)b * a.vote_stride + block_lo + i] = c;
+      if (a.votes && a.pool_kernel <= 0) a.votes[(size_t)b * a.vote_stride + block_lo + i] = c;
       sc[0] = c;
+    }
+    uint32_t round = 2;  // rendezvous passed so far
+    if (a.pool_kernel > 0) {
+      // Max-pool smoothing of the votes (tr.py:366-369): stride 1, padding (kernel-1)/2
+      // with -inf, an even kernel makes the result one shorter.  The workgroups
+      // exchange their votes through memory (one more rendezvous), gather the
+      // kernel-1 neighbours on either side of their range into LDS (the histogram
+      // array is still unused) and replace each vote by the maximum of its window.
+      float* pv = a.pool_votes + (size_t)b * a.pool_stride;
+      float* window = (float*)lh;  // [pad | own votes | kernel-1-pad]
+      const int pad = (a.pool_kernel - 1) / 2;
+      const int halo = a.pool_kernel - 1;
+      for (int i = tid; i < count; i += 256) {
+        const float c = *column(i);
+        __hip_atomic_store((uint32_t*)&pv[block_lo + i], __float_as_uint(c), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        window[pad + i] = c;
+      }
+      grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      for (int hx = tid; hx < halo; hx += 256) {
+        const int t = hx < pad ? block_lo - pad + hx : block_lo + count + (hx - pad);
+        const int at = hx < pad ? hx : count + hx;
+        window[at] = (t >= 0 && t < n) ? __uint_as_float(load_coherent((const uint32_t*)&pv[t]))
+                                       : -INFINITY;
+      }
+      __syncthreads();
+      const int n_pooled = n + 2 * pad - a.pool_kernel + 1;
+      for (int i = tid; i < count; i += 256) {
+        float m = -INFINITY;  // past the pooled length: never selected (k < n)
+        if (block_lo + i < n_pooled) {
+          for (int w = 0; w < a.pool_kernel; ++w) m = fmaxf(m, window[i + w]);
+          if (a.votes) a.votes[(size_t)b * a.vote_stride + block_lo + i] = m;
+        }
+        *column(i) = m;
+      }
+      __syncthreads();
+      for (int i = tid; i < count + halo; i += 256) lh[i] = 0u;
+      __syncthreads();
     }
     // Local histogram.  The votes of a wavefront fall into a narrow range of bins, so
     // the lanes are counted bin by bin with ballots over the 64 bins below the
@@ -575,7 +614,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       if (tid == 0) done += fetch_max_coherent(&ctr[kSelMaxBin], scratch[8]);
       await(done);
     }
-    grid_arrive(a.sync, 3, true, a.spin_ticks, team.size, team.index);
+    grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
     uint32_t t0 = 0, above0 = 0;
     for (int top = (int)load_coherent(&ctr[kSelMaxBin]); top >= 0; top -= 256) {
       const int bin = top - tid;
@@ -605,7 +644,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       }
       await(done);
     }
-    grid_arrive(a.sync, 4, true, a.spin_ticks, team.size, team.index);
+    grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
     {
       uint32_t h[kTopkBins / 256];
 #pragma unroll
@@ -628,7 +667,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       }
       await(done);
     }
-    grid_arrive(a.sync, 5, true, a.spin_ticks, team.size, team.index);
+    grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
     {
       uint32_t h[4];
 #pragma unroll
@@ -668,7 +707,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     __syncthreads();
     uint2* counts = a.block_counts + (size_t)b * gridDim.x;
     if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], scratch[9]);
-    grid_arrive(a.sync, 6, true, a.spin_ticks, team.size, team.index);
+    grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
     {
       uint32_t sure = 0, tie = 0;
       for (int j = tid; j < (int)blockIdx.x; j += 256) {
@@ -787,7 +826,8 @@ static std::atomic<int> g_fused_select{[] {
 int set_fused_select(int enable) { return g_fused_select.exchange(enable ? 1 : 0); }
 
 int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len) {
-  if (!g_fused_select.load() || cfg->pool_kernel > 0 || cfg->num_heads > kMaxHeads) return 0;
+  // Max-pool windows beyond 256 would not fit the LDS the neighbours are gathered into.
+  if (!g_fused_select.load() || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256) return 0;
   const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
   if (max_n <= 0) return 0;
   const int group = cfg->num_heads / cfg->num_kv_heads;
@@ -844,6 +884,8 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
   w.stats = take(B * H * 2 * sizeof(float));
   w.counters = take(B * kSelCounterWords * 4);
   w.block_counts = take(B * (size_t)w.blocks_per_req * sizeof(uint2));
+  w.pool_stride = (int64_t)align_up((size_t)max_n, 64);
+  w.pool_votes = take(cfg->pool_kernel > 0 ? B * (size_t)w.pool_stride * sizeof(float) : 0);
   w.sync = take(kSyncWords * 4);
   w.total = off;
   return w;
@@ -921,6 +963,9 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   a.clear = clear;
   a.clear_per_req = clear_per_req;
   a.spin_ticks = 200000000ull;  // 2 s of the 100 MHz clock
+  a.pool_kernel = cfg->pool_kernel;
+  a.pool_votes = (float*)(ws + w.pool_votes);
+  a.pool_stride = w.pool_stride;
   const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
   const dim3 grid((unsigned)w.blocks_per_req, (unsigned)bt->batch);
   void* params[] = {(void*)&a};
@@ -1013,7 +1058,7 @@ int ts_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const vo
   const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len);
   TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE,
              "ts_select: batch %d x %d tokens does not fit one co-resident grid (or pool_kernel is "
-             "on); use ts_score + ts_vote + ts_topk_ragged",
+             "above 256); use ts_score + ts_vote + ts_topk_ragged",
              bt->batch, bt->max_seq_len);
   TS_REQUIRE(workspace_bytes >= w.total, TS_EWORKSPACE, "ts_select: workspace %zu bytes < required %zu",
              workspace_bytes, w.total);

@@ -10,7 +10,7 @@ namespace ts {
 constexpr int kTopkBins = 2048;          // 11-bit digits
 constexpr int kTopkSlice = 512;          // candidates per workgroup of the hist / mark grids
 constexpr int kTopkFinalThreads = 1024;
-constexpr int kTopkPartWords = 1024;     // 32-bit bitmap words per workgroup of the final grid
+constexpr int kTopkPartWords = 512;      // 32-bit bitmap words per workgroup of the final grid
 // Per-request workspace, in 32-bit words:
 //   [hist0: 2048][hist1: 2048][cand_count: 1, padded to 64]   <- zeroed before every selection
 //   [bitmap: 1 bit per candidate, 64-bit words]

@@ -9,7 +9,6 @@
 namespace ts {
 
 constexpr int kMaxHeads = 128;
-constexpr int kVoteSlice = 1024;  // candidates per workgroup of the vote grid
 
 struct VoteArgs {
   const float* scores;
@@ -53,7 +52,9 @@ __global__ __launch_bounds__(64) void stats_merge_kernel(VoteArgs a) {
 // order.  With a top-k workspace attached the workgroup also counts its votes into the
 // first-level histogram of the selection (top 11 key bits) and adds its occupied bins
 // to the request's histogram at the end.
+template <int kPerThread>  // candidates per thread: a workgroup owns 256 * kPerThread
 __global__ __launch_bounds__(256) void vote_kernel(VoteArgs a) {
+  constexpr int kVoteSlice = 256 * kPerThread;
   const int b = blockIdx.y;
   if (a.skip && a.skip[b]) return;
   const ReqGeom geo =
@@ -76,7 +77,6 @@ __global__ __launch_bounds__(256) void vote_kernel(VoteArgs a) {
     for (int i = threadIdx.x; i < kTopkBins; i += 256) lh[i] = 0u;
   __syncthreads();
 
-  constexpr int kPerThread = kVoteSlice / 256;
   float c[kPerThread];
   const float* p[kPerThread];
 #pragma unroll
@@ -185,7 +185,10 @@ int launch_vote(const ts_config* cfg, const ts_batch* bt, const float* scores, i
   hipLaunchKernelGGL(stats_merge_kernel, dim3((unsigned)cfg->num_heads, (unsigned)bt->batch), dim3(64),
                      0, stream, a);
   TS_TRY(check_launch("stats_merge_kernel"));
-  hipLaunchKernelGGL(vote_kernel, dim3((unsigned)ceil_div(max_n, kVoteSlice), (unsigned)bt->batch),
+  // Four candidates per thread: the workgroups' histogram flushes (a scan of 2048 LDS
+  // bins and an atomic per occupied one) cost more than the parallelism of smaller
+  // workgroup ranges brings, also at 128K candidates.
+  hipLaunchKernelGGL(vote_kernel<4>, dim3((unsigned)ceil_div(max_n, 1024), (unsigned)bt->batch),
                      dim3(256), 0, stream, a);
   TS_TRY(check_launch("vote_kernel"));
 
