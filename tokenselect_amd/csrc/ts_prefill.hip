@@ -108,11 +108,14 @@ struct PrefillArgs {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float pf_f32x4;
+constexpr float kLog2e = 1.4426950408889634f;
 
 constexpr int kPfKeys = 32;               // keys per tile
 constexpr int kPfPipe = 4;                // tiles whose pieces are in flight
 constexpr int kPfKRow = kHeadDim + 8;     // halfwords per K row in LDS (272 B: rows on different banks)
-constexpr int kPfVRow = kPfKeys + 8;      // halfwords per V^T row in LDS (80 B)
+constexpr int kPfVRow = kPfKeys + 8;      // halfwords per V^T row in the gather kernel's LDS (80 B)
+constexpr int kPfVRowA = kPfKeys + 4;     // in the attention kernel's LDS: 72 B = 18 banks, the 16
+                                          // rows a wavefront reads together fall on distinct banks
 
 // Two floats to packed bf16, round to nearest even, in one v_cvt_pk_bf16_f32.
 typedef __attribute__((ext_vector_type(2))) __bf16 pf_bf16x2;
@@ -195,7 +198,7 @@ template <int G, bool CAP>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(
     PrefillArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t k_lds2[2][kPfKeys * kPfKRow];
-  __shared__ __attribute__((aligned(16))) uint16_t vt_lds2[2][kHeadDim * kPfVRow];
+  __shared__ __attribute__((aligned(16))) uint16_t vt_lds2[2][kHeadDim * kPfVRowA];
   __shared__ float merge_lds[4][64][34];
 
   const int group = threadIdx.x >> 8;  // which of the two tile streams this wavefront follows
@@ -247,21 +250,29 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           x[ks + 2][e] = hi * cs + lo * sn;
         }
     }
+    // Without a soft cap the softmax scale and log2(e) go into the query, so that the
+    // products come out as base-2 logits and every key costs one exp2 and no multiply.
+    const float qs = CAP ? 1.0f : a.sm_scale * kLog2e;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[ks][e] *= qs;
       const uint4 w = make_uint4(pack_bf16(x[ks][0], x[ks][1]), pack_bf16(x[ks][2], x[ks][3]),
                                  pack_bf16(x[ks][4], x[ks][5]), pack_bf16(x[ks][6], x[ks][7]));
       qb[ks] = __builtin_bit_cast(pf_bf16x8, w);
     }
   }
 
-  // ---- staging role: thread t copies 32 bytes of the K tile (key t/8, dims [16 (t%8), +16))
-  // and 32 bytes of the V^T tile (dim t/2, keys [16 (t%2), +16)).
+  // ---- staging role: thread t copies two 16-byte pieces of the K tile (key t/8, dims
+  // [8 (t%8), +8) and the same 64 dims further on: consecutive lanes write consecutive 16
+  // bytes of a K row, which the LDS banks take without conflicts) and 32 bytes of the V^T
+  // tile (dim t/2, keys [16 (t%2), +16): two lanes per 64-byte row of the staging area;
+  // one row per lane would suit the LDS banks better but costs more on the global side).
   const uint16_t* k_src = a.kr + (size_t)kvh * a.s_pad * kHeadDim + (size_t)(tid >> 3) * kHeadDim +
-                          16 * (tid & 7);
+                          8 * (tid & 7);
   const uint16_t* v_src = a.vt + ((size_t)kvh * kHeadDim + (tid >> 1)) * a.s_pad + 16 * (tid & 1);
-  uint16_t* k_dst = k_lds + (tid >> 3) * kPfKRow + 16 * (tid & 7);
-  uint16_t* v_dst = vt_lds + (tid >> 1) * kPfVRow + 16 * (tid & 1);
+  uint16_t* k_dst = k_lds + (tid >> 3) * kPfKRow + 8 * (tid & 7);
+  uint16_t* v_dst = vt_lds + (tid >> 1) * kPfVRowA + 16 * (tid & 1);  // 8-byte aligned
   // Four register buffers, named rather than indexed: an indexed array of them is
   // kept in scratch memory by the compiler, and the prefetch with it.
   struct TilePiece {
@@ -274,7 +285,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint4* vs = (const uint4*)(v_src + tile);
     TilePiece piece;
     piece.k0 = ks[0];
-    piece.k1 = ks[1];
+    piece.k1 = ks[8];  // 64 dims further on
     piece.v0 = vs[0];
     piece.v1 = vs[1];
     return piece;
@@ -290,7 +301,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   // One tile of this group: logits, online softmax, output update.
   auto compute_tile = [&](int tile) __attribute__((always_inline)) {
-    // logits: s[blk][r] belongs to key tile + 16 blk + 4 g4 + r and query qc
+    // logits (base 2): s[blk][r] belongs to key tile + 16 blk + 4 g4 + r and query qc.
+    // Only the tiles on the diagonal hold keys that some query of the tile must not see.
+    const bool diagonal = tile + kPfKeys - 1 > shift + q_row0;
     float s[2][4];
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
@@ -303,12 +316,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float x = acc[r] * a.sm_scale;
-        if (CAP) x = a.logit_cap * tanhf(x / a.logit_cap);
+        float x = acc[r];
+        if (CAP) x = a.logit_cap * tanhf(x * a.sm_scale / a.logit_cap) * kLog2e;
         const int key = tile + 16 * blk + 4 * g4 + r;
         // Masked logits are -inf and the running maximum starts at a finite value,
-        // so exp(s - max) is 0 for them without a branch and never NaN.
-        s[blk][r] = key <= my_limit ? x : -INFINITY;
+        // so exp2(s - max) is 0 for them without a branch and never NaN.
+        s[blk][r] = (!diagonal || key <= my_limit) ? x : -INFINITY;
       }
     }
     float mx = kNegBig;
@@ -319,13 +332,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_run, mx);
-    const float alpha = __expf(m_run - m_new);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     float p[2][4], psum = 0.f;
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        p[blk][r] = __expf(s[blk][r] - m_new);
+        p[blk][r] = __builtin_amdgcn_exp2f(s[blk][r] - m_new);
         psum += p[blk][r];
       }
     l_run = l_run * alpha + psum;
@@ -344,7 +357,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
-      const uint16_t* vrow = vt_lds + (16 * db + qc) * kPfVRow;
+      const uint16_t* vrow = vt_lds + (16 * db + qc) * kPfVRowA;
       const uint2 v0 = *(const uint2*)(vrow + 4 * g4);
       const uint2 v1 = *(const uint2*)(vrow + 16 + 4 * g4);
       const uint4 vw = make_uint4(v0.x, v0.y, v1.x, v1.y);
@@ -364,9 +377,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int tile = pair + kPfKeys * group;                                  \
     __syncthreads(); /* the previous tiles' LDS reads are done */             \
     ((uint4*)k_dst)[0] = piece##u.k0;                                         \
-    ((uint4*)k_dst)[1] = piece##u.k1;                                         \
-    ((uint4*)v_dst)[0] = piece##u.v0;                                         \
-    ((uint4*)v_dst)[1] = piece##u.v1;                                         \
+    ((uint4*)k_dst)[8] = piece##u.k1;                                         \
+    ((uint2*)v_dst)[0] = make_uint2(piece##u.v0.x, piece##u.v0.y);            \
+    ((uint2*)v_dst)[1] = make_uint2(piece##u.v0.z, piece##u.v0.w);            \
+    ((uint2*)v_dst)[2] = make_uint2(piece##u.v1.x, piece##u.v1.y);            \
+    ((uint2*)v_dst)[3] = make_uint2(piece##u.v1.z, piece##u.v1.w);            \
     piece##u = request_tile(tile + 2 * kPfPipe * kPfKeys);                    \
     __syncthreads();                                                          \
     if (wave_active && tile <= last_visible) compute_tile(tile);              \
@@ -397,7 +412,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   {
     const float* other = merge_lds[wave][lane];
     const float m_new = fmaxf(m_run, other[0]);
-    const float e0 = __expf(m_run - m_new), e1 = __expf(other[0] - m_new);
+    const float e0 = __builtin_amdgcn_exp2f(m_run - m_new), e1 = __builtin_amdgcn_exp2f(other[0] - m_new);
     l_run = l_run * e0 + other[1] * e1;
 #pragma unroll
     for (int db = 0; db < 8; ++db)
