@@ -174,6 +174,31 @@ def test_fused_select_ties(dev):
         assert torch.equal(sel_pos[0, :int(sel_len[0])], pos_sep[0, :int(sel_len[0])])
 
 
+@pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
+def test_select_with_all_votes_equal(dev, fused_select):
+    """A zero query makes every vote H/n: one histogram bin at every level, every
+    candidate tied at the k-th vote; the k lowest positions win.  (Also a guard against
+    the selection serialising on one counter: the layer must not take milliseconds.)"""
+    say(f"selection with all votes equal, fused={fused_select}")
+    L, k = 70000, 1000
+    wl = small(dev, SHAPES[0], seed=81, lens=[L], ks=[k], page=16, top_k=k, n_init=128, n_local=512)
+    wl.q.zero_()
+    c = wl.cfg
+    layer = ops.DecodeLayer(c, 1, L, dev)
+    layer(wl.q, wl.k_pool, wl.v_pool, wl.batch)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    out, sel, sel_pos, sel_len = layer(wl.q, wl.k_pool, wl.v_pool, wl.batch)
+    end.record()
+    torch.cuda.synchronize()
+    S = int(sel_len[0])
+    assert S == c.n_init + k + c.n_local
+    expect = torch.cat([torch.arange(c.n_init + k), torch.arange(L - c.n_local, L)]).int()
+    assert torch.equal(sel_pos[0, :S].cpu(), expect)
+    assert start.elapsed_time(end) < 1.0, "the selection serialised on a single counter"
+
+
 def test_fused_select_rejects_unsupported(dev):
     say("fused select: pool_kernel above 256 -> TS_ESHAPE")
     wl = small(dev, SHAPES[0], seed=3, lens=[2000], ks=[64], pool_kernel=300)

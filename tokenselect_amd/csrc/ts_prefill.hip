@@ -78,17 +78,21 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
 // prefill_attn_kernel<G>: grid (16-row query tiles, KV heads, quads of the G query
 // heads of a KV head); 512 threads = two groups of four wavefronts.  The wavefronts
 // of a group serve one query head each and share the K/V tiles of their KV head;
-// group 0 takes the even 32-key tiles and group 1 the odd ones (two wavefronts per
+// group 0 takes the even 64-key tiles and group 1 the odd ones (two wavefronts per
 // SIMD hide each other's LDS and matrix latencies), and their (max, sum, acc) are
-// merged through LDS at the end.  Per tile a group copies 8 KB of kr and 8 KB of vt
-// into its LDS buffers (the next tiles' pieces already in registers).  A wavefront then computes
-// S^T = K Q^T with v_mfma_f32_16x16x32_bf16 (A = 16 keys x 32 dims from LDS, B = its
-// 16 rotated queries, held in registers), which leaves lane (query l%16, key group
-// l/16) with the logits of 8 keys; the online softmax needs two cross-lane maxima
-// per tile; the 8 probabilities, rounded to bf16, are directly the B operand of
-// O^T += V^T P^T (A = 16 dims x 32 keys from the transposed V tile, keys in the order
-// the logits came in), so no data moves between the two products.  fp32 accumulation
-// throughout.
+// merged through LDS at the end.  Per tile a group copies 16 KB of kr and 16 KB of vt
+// into one of its two LDS buffers (the pieces of the next two tiles already in
+// registers) while the wavefronts compute on the other: one barrier per tile.  A
+// wavefront computes S^T = K Q^T with v_mfma_f32_16x16x32_bf16 (A = 16 keys x 32 dims
+// from LDS, B = its 16 rotated queries, held in registers, pre-multiplied by the softmax
+// scale and log2 e), which leaves lane (query l%16, key group l/16) with the base-2
+// logits of 16 keys; the online softmax needs two cross-lane maxima per tile; the 16
+// probabilities, rounded to bf16, are directly the B operands of O^T += V^T P^T (A = 16
+// dims x 32 keys from the transposed V tile, keys in the order the logits came in), so
+// no data moves between the two products.  fp32 accumulation throughout.
+// What the time went into, by the counters: neither the matrix units (17 % busy), nor
+// the vector ALU, nor LDS bandwidth, but waiting: bank conflicts of the V^T rows (now
+// padded to 34 banks), and the two barriers per tile of the single-buffered version.
 struct PrefillArgs {
   const uint16_t* q;  // [rows, H, 128] bf16, un-rotated
   const uint16_t* k_pool;
@@ -110,12 +114,14 @@ typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float pf_f32x4;
 constexpr float kLog2e = 1.4426950408889634f;
 
-constexpr int kPfKeys = 32;               // keys per tile
-constexpr int kPfPipe = 4;                // tiles whose pieces are in flight
+constexpr int kPfKeys = 32;               // keys per workgroup of the gather kernel
 constexpr int kPfKRow = kHeadDim + 8;     // halfwords per K row in LDS (272 B: rows on different banks)
 constexpr int kPfVRow = kPfKeys + 8;      // halfwords per V^T row in the gather kernel's LDS (80 B)
-constexpr int kPfVRowA = kPfKeys + 4;     // in the attention kernel's LDS: 72 B = 18 banks, the 16
-                                          // rows a wavefront reads together fall on distinct banks
+constexpr int kPfTile = 64;               // keys per tile of the attention kernel
+constexpr int kPfPipeA = 2;               // attention tiles whose pieces are in flight
+constexpr int kPfVRowA = kPfTile + 4;     // halfwords per V^T row in the attention kernel's LDS:
+                                          // 136 B = 34 banks, the 16 rows a wavefront reads together
+                                          // (8 bytes each) fall on distinct banks
 
 // Two floats to packed bf16, round to nearest even, in one v_cvt_pk_bf16_f32.
 typedef __attribute__((ext_vector_type(2))) __bf16 pf_bf16x2;
@@ -134,7 +140,9 @@ __global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
   const int kvh = blockIdx.y;
   const int S = min(max(*a.sel_len, 0), a.max_sel_len);
   const int j = blockIdx.x * kPfKeys + kk;
-  if (blockIdx.x * kPfKeys >= S) return;
+  // Whole tiles of the attention kernel: the keys between S and the next multiple of
+  // its tile are written as zeros too (their weights are zero, but 0 x garbage is not).
+  if (blockIdx.x * kPfKeys >= (S + kPfTile - 1) / kPfTile * kPfTile) return;
   const bool live = j < S;
   uint4 kraw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
   uint4 vraw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
@@ -197,13 +205,16 @@ __global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
 template <int G, bool CAP>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(
     PrefillArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t k_lds2[2][kPfKeys * kPfKRow];
-  __shared__ __attribute__((aligned(16))) uint16_t vt_lds2[2][kHeadDim * kPfVRowA];
-  __shared__ float merge_lds[4][64][34];
-
+  // Dynamic LDS: per group two buffers of a K tile [kPfTile * kPfKRow] followed by a V^T
+  // tile [kHeadDim * kPfVRowA]; the merge of the two groups at the end reuses the space.
+  extern __shared__ __attribute__((aligned(16))) uint16_t pf_lds[];
+  constexpr int kBuf = kPfTile * kPfKRow + kHeadDim * kPfVRowA;  // halfwords per buffer
   const int group = threadIdx.x >> 8;  // which of the two tile streams this wavefront follows
-  uint16_t* const k_lds = k_lds2[group];
-  uint16_t* const vt_lds = vt_lds2[group];
+  uint16_t* const k_lds = pf_lds + group * (2 * kBuf);
+  uint16_t* const vt_lds = k_lds + kPfTile * kPfKRow;
+  float(*merge_lds)[64][34] = (float(*)[64][34])pf_lds;  // [4][64][34]
+  static_assert(4 * 64 * 34 * 4 <= 4 * kBuf * 2, "the merge area fits the tiles");
+
   const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
   const int qc = lane & 15, g4 = lane >> 4;  // query column / key group of the MFMA layouts
   const int kvh = blockIdx.y;
@@ -263,31 +274,34 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
   }
 
-  // ---- staging role: thread t copies two 16-byte pieces of the K tile (key t/8, dims
-  // [8 (t%8), +8) and the same 64 dims further on: consecutive lanes write consecutive 16
-  // bytes of a K row, which the LDS banks take without conflicts) and 32 bytes of the V^T
-  // tile (dim t/2, keys [16 (t%2), +16): two lanes per 64-byte row of the staging area;
-  // one row per lane would suit the LDS banks better but costs more on the global side).
+  // ---- staging role: thread t copies four 16-byte pieces of the K tile (keys t/8 and
+  // t/8 + 32, dims [8 (t%8), +8) and the same 64 dims further on: consecutive lanes write
+  // consecutive 16 bytes of a K row, which the LDS banks take without conflicts) and 64
+  // bytes of the V^T tile (dim t/2, keys [32 (t%2), +32)).
   const uint16_t* k_src = a.kr + (size_t)kvh * a.s_pad * kHeadDim + (size_t)(tid >> 3) * kHeadDim +
                           8 * (tid & 7);
-  const uint16_t* v_src = a.vt + ((size_t)kvh * kHeadDim + (tid >> 1)) * a.s_pad + 16 * (tid & 1);
+  const uint16_t* v_src = a.vt + ((size_t)kvh * kHeadDim + (tid >> 1)) * a.s_pad + 32 * (tid & 1);
   uint16_t* k_dst = k_lds + (tid >> 3) * kPfKRow + 8 * (tid & 7);
-  uint16_t* v_dst = vt_lds + (tid >> 1) * kPfVRowA + 16 * (tid & 1);  // 8-byte aligned
-  // Four register buffers, named rather than indexed: an indexed array of them is
+  uint16_t* v_dst = vt_lds + (tid >> 1) * kPfVRowA + 32 * (tid & 1);  // 8-byte aligned
+  // Two register buffers, named rather than indexed: an indexed array of them is
   // kept in scratch memory by the compiler, and the prefetch with it.
   struct TilePiece {
-    uint4 k0, k1, v0, v1;
+    uint4 k0, k1, k2, k3, v0, v1, v2, v3;
   };
-  TilePiece piece0, piece1, piece2, piece3;
+  TilePiece piece0, piece1;
   auto request_tile = [&](int tile) __attribute__((always_inline)) -> TilePiece {
-    tile = min(tile, a.s_pad - kPfKeys);  // past the end: harmless repeat of the last tile
+    tile = min(tile, a.s_pad - kPfTile);  // past the end: harmless repeat of the last tile
     const uint4* ks = (const uint4*)(k_src + (size_t)tile * kHeadDim);
     const uint4* vs = (const uint4*)(v_src + tile);
     TilePiece piece;
     piece.k0 = ks[0];
-    piece.k1 = ks[8];  // 64 dims further on
+    piece.k1 = ks[8];                      // 64 dims further on
+    piece.k2 = ks[32 * kHeadDim / 8];      // 32 keys further on
+    piece.k3 = ks[32 * kHeadDim / 8 + 8];
     piece.v0 = vs[0];
     piece.v1 = vs[1];
+    piece.v2 = vs[2];
+    piece.v3 = vs[3];
     return piece;
   };
 
@@ -299,18 +313,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
   for (int db = 0; db < 8; ++db) o[db] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // One tile of this group: logits, online softmax, output update.
-  auto compute_tile = [&](int tile) __attribute__((always_inline)) {
+  // One 64-key tile of this group: logits, online softmax, output update.
+  auto compute_tile = [&](int tile, int buf) __attribute__((always_inline)) {
+    const uint16_t* const kt = k_lds + buf * kBuf;
+    const uint16_t* const vt = vt_lds + buf * kBuf;
     // logits (base 2): s[blk][r] belongs to key tile + 16 blk + 4 g4 + r and query qc.
     // Only the tiles on the diagonal hold keys that some query of the tile must not see.
-    const bool diagonal = tile + kPfKeys - 1 > shift + q_row0;
-    float s[2][4];
+    const bool diagonal = tile + kPfTile - 1 > shift + q_row0;
+    float s[4][4];
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
+    for (int blk = 0; blk < 4; ++blk) {
       pf_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
-        const uint4 kw = *(const uint4*)(k_lds + (16 * blk + qc) * kPfKRow + 32 * ks + 8 * g4);
+        const uint4 kw = *(const uint4*)(kt + (16 * blk + qc) * kPfKRow + 32 * ks + 8 * g4);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, kw), qb[ks],
                                                       acc, 0, 0, 0);
       }
@@ -326,16 +342,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     float mx = kNegBig;
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
+    for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
       for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[blk][r]);
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_run, mx);
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    float p[2][4], psum = 0.f;
+    float p[4][4], psum = 0.f;
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
+    for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         p[blk][r] = __builtin_amdgcn_exp2f(s[blk][r] - m_new);
@@ -346,9 +362,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // after the first tiles is rare: skip the 32 multiplications otherwise.
     const bool rescale = __ballot(m_new != m_run) != 0ull;
     m_run = m_new;
-    const uint4 pw = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]),
-                                pack_bf16(p[1][0], p[1][1]), pack_bf16(p[1][2], p[1][3]));
-    const pf_bf16x8 pb = __builtin_bit_cast(pf_bf16x8, pw);
+    pf_bf16x8 pb[2];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const uint4 pw = make_uint4(pack_bf16(p[2 * hf][0], p[2 * hf][1]),
+                                  pack_bf16(p[2 * hf][2], p[2 * hf][3]),
+                                  pack_bf16(p[2 * hf + 1][0], p[2 * hf + 1][1]),
+                                  pack_bf16(p[2 * hf + 1][2], p[2 * hf + 1][3]));
+      pb[hf] = __builtin_bit_cast(pf_bf16x8, pw);
+    }
     if (rescale) {
 #pragma unroll
       for (int db = 0; db < 8; ++db)
@@ -357,46 +379,66 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
-      const uint16_t* vrow = vt_lds + (16 * db + qc) * kPfVRowA;
-      const uint2 v0 = *(const uint2*)(vrow + 4 * g4);
-      const uint2 v1 = *(const uint2*)(vrow + 16 + 4 * g4);
-      const uint4 vw = make_uint4(v0.x, v0.y, v1.x, v1.y);
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw), pb, o[db],
-                                                      0, 0, 0);
+      const uint16_t* vrow = vt + (16 * db + qc) * kPfVRowA;
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const uint2 v0 = *(const uint2*)(vrow + 32 * hf + 4 * g4);
+        const uint2 v1 = *(const uint2*)(vrow + 32 * hf + 16 + 4 * g4);
+        const uint4 vw = make_uint4(v0.x, v0.y, v1.x, v1.y);
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw), pb[hf],
+                                                        o[db], 0, 0, 0);
+      }
     }
   };
 
-  // Step u of a round covers the tile pair starting at round + 64 u; this group's tile
-  // is the first or the second of the pair.  The steps are written out one by one so
-  // that each uses its own register buffer.
-  static_assert(kPfPipe == 4, "the steps below are written out for four buffers");
-#define TS_PF_STEP(u)                                                         \
-  {                                                                           \
-    const int pair = round + 2 * kPfKeys * (u);                               \
-    if (pair > last_visible) break;                                           \
-    const int tile = pair + kPfKeys * group;                                  \
-    __syncthreads(); /* the previous tiles' LDS reads are done */             \
-    ((uint4*)k_dst)[0] = piece##u.k0;                                         \
-    ((uint4*)k_dst)[8] = piece##u.k1;                                         \
-    ((uint2*)v_dst)[0] = make_uint2(piece##u.v0.x, piece##u.v0.y);            \
-    ((uint2*)v_dst)[1] = make_uint2(piece##u.v0.z, piece##u.v0.w);            \
-    ((uint2*)v_dst)[2] = make_uint2(piece##u.v1.x, piece##u.v1.y);            \
-    ((uint2*)v_dst)[3] = make_uint2(piece##u.v1.z, piece##u.v1.w);            \
-    piece##u = request_tile(tile + 2 * kPfPipe * kPfKeys);                    \
-    __syncthreads();                                                          \
-    if (wave_active && tile <= last_visible) compute_tile(tile);              \
+  // The LDS tiles are double-buffered: while the wavefronts compute on one buffer, the
+  // next tile (its pieces already in registers) is written to the other, and one
+  // barrier per tile separates "everybody has read buffer b" from its next overwrite.
+  // Tile number i of this group (keys (2 i + group) * 64 ...) travels through register
+  // buffer i % 2 and LDS buffer i % 2; the steps are written out for the two parities so
+  // that each uses its own named registers.
+  static_assert(kPfPipeA == 2, "the steps below are written out for two buffers");
+#define TS_PF_STORE(u, buf)                                                                  \
+  {                                                                                          \
+    uint16_t* const kd = k_dst + (buf) * kBuf;                                               \
+    uint16_t* const vd = v_dst + (buf) * kBuf;                                               \
+    ((uint4*)kd)[0] = piece##u.k0;                                                           \
+    ((uint4*)kd)[8] = piece##u.k1;                                                           \
+    ((uint4*)(kd + 32 * kPfKRow))[0] = piece##u.k2;                                          \
+    ((uint4*)(kd + 32 * kPfKRow))[8] = piece##u.k3;                                          \
+    ((uint2*)vd)[0] = make_uint2(piece##u.v0.x, piece##u.v0.y);                              \
+    ((uint2*)vd)[1] = make_uint2(piece##u.v0.z, piece##u.v0.w);                              \
+    ((uint2*)vd)[2] = make_uint2(piece##u.v1.x, piece##u.v1.y);                              \
+    ((uint2*)vd)[3] = make_uint2(piece##u.v1.z, piece##u.v1.w);                              \
+    ((uint2*)vd)[4] = make_uint2(piece##u.v2.x, piece##u.v2.y);                              \
+    ((uint2*)vd)[5] = make_uint2(piece##u.v2.z, piece##u.v2.w);                              \
+    ((uint2*)vd)[6] = make_uint2(piece##u.v3.x, piece##u.v3.y);                              \
+    ((uint2*)vd)[7] = make_uint2(piece##u.v3.z, piece##u.v3.w);                              \
   }
-  piece0 = request_tile(kPfKeys * (0 + group));
-  piece1 = request_tile(kPfKeys * (2 + group));
-  piece2 = request_tile(kPfKeys * (4 + group));
-  piece3 = request_tile(kPfKeys * (6 + group));
-  for (int round = 0; round <= last_visible; round += 2 * kPfPipe * kPfKeys) {
-    TS_PF_STEP(0)
-    TS_PF_STEP(1)
-    TS_PF_STEP(2)
-    TS_PF_STEP(3)
+  // Step for the tile in LDS buffer `cur`: stage the following tile from register buffer
+  // `nxt` into LDS buffer `nxt`, request the tile after that, compute, barrier.
+#define TS_PF_STEP(cur, nxt)                                                                 \
+  {                                                                                          \
+    const int pair = round + 2 * kPfTile * (cur);                                            \
+    if (pair > last_visible) break;                                                          \
+    const int tile = pair + kPfTile * group;                                                 \
+    TS_PF_STORE(nxt, nxt)                                                                    \
+    piece##nxt = request_tile(tile + 3 * 2 * kPfTile);                                       \
+    if (wave_active && tile <= last_visible) compute_tile(tile, cur);                        \
+    __syncthreads();                                                                         \
+  }
+  piece0 = request_tile(kPfTile * (0 + group));
+  piece1 = request_tile(kPfTile * (2 + group));
+  TS_PF_STORE(0, 0)
+  piece0 = request_tile(kPfTile * (4 + group));
+  __syncthreads();
+  for (int round = 0; round <= last_visible; round += 2 * kPfPipeA * kPfTile) {
+    TS_PF_STEP(0, 1)
+    TS_PF_STEP(1, 0)
   }
 #undef TS_PF_STEP
+#undef TS_PF_STORE
+  // (the barrier that ended the last step also freed the tiles' space for the merge)
   // Group 1 hands its partial result to group 0 (same wavefront index, same lane).
   if (group == 1) {
     float* mine = merge_lds[wave][lane];
@@ -431,7 +473,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                                                     pack_bf16(o[db][2] * inv, o[db][3] * inv));
 }
 
-static int prefill_s_pad(int max_sel_len) { return (int)ceil_div(max_sel_len, kPfKeys) * kPfKeys; }
+constexpr size_t kPfLdsBytes = 2 * 2 * (size_t)(kPfTile * kPfKRow + kHeadDim * kPfVRowA) * 2;
+
+static int prefill_s_pad(int max_sel_len) { return (int)ceil_div(max_sel_len, kPfTile) * kPfTile; }
 
 }  // namespace ts
 
@@ -501,12 +545,18 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
   const dim3 grid((unsigned)ceil_div(rows, 16), (unsigned)cfg->num_kv_heads,
                   (unsigned)ceil_div(group, 4));
   const bool cap = cfg->logit_cap > 0.f;
-#define TS_PF_CASE(G_)                                                                       \
-  case G_:                                                                                   \
-    if (cap)                                                                                 \
-      hipLaunchKernelGGL((prefill_attn_kernel<G_, true>), grid, dim3(512), 0, st, a);        \
-    else                                                                                     \
-      hipLaunchKernelGGL((prefill_attn_kernel<G_, false>), grid, dim3(512), 0, st, a);       \
+#define TS_PF_LAUNCH(G_, C_)                                                                  \
+  {                                                                                           \
+    static const hipError_t lds_ok = hipFuncSetAttribute(                                     \
+        (const void*)prefill_attn_kernel<G_, C_>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+        (int)kPfLdsBytes);                                                                    \
+    if (lds_ok != hipSuccess) return fail(TS_EHIP, "prefill attention: %zu bytes of LDS refused", kPfLdsBytes); \
+    hipLaunchKernelGGL((prefill_attn_kernel<G_, C_>), grid, dim3(512), kPfLdsBytes, st, a);   \
+  }
+#define TS_PF_CASE(G_)               \
+  case G_:                           \
+    if (cap) TS_PF_LAUNCH(G_, true)  \
+    else TS_PF_LAUNCH(G_, false)     \
     break;
   switch (group) {
     TS_PF_CASE(1)
@@ -517,6 +567,7 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
     default: return fail(TS_ESHAPE, "unsupported head group %d", group);
   }
 #undef TS_PF_CASE
+#undef TS_PF_LAUNCH
   return check_launch("prefill_attn_kernel");
 }
 

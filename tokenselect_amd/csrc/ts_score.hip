@@ -198,6 +198,26 @@ __device__ __forceinline__ void fixed_segments(const ScoreArgs& a, int b) {
 // running count (from thread 0 on) reaches `need`.  Returns that thread's index
 // (or -1 if the total stays below `need`), the count before it, and the total.
 // `scratch` is LDS of 8 words.
+// Adds the wavefront's candidates to a histogram in memory with one fetch-add per
+// distinct bin: normally a wavefront has a few candidates in different bins, but
+// nearly uniform votes (a query of small norm) put all 64 lanes, of every wavefront,
+// into the same bin, and that many single increments of one address take
+// milliseconds.  Returns the old values (to be awaited).  Every lane of the wavefront
+// must call it.
+__device__ __forceinline__ uint32_t wave_histogram_add(uint32_t* hist, bool have, uint32_t bin,
+                                                      int lane) {
+  uint32_t done = 0;
+  uint64_t todo = __ballot(have);
+  while (todo) {
+    const int leader = __ffsll((unsigned long long)todo) - 1;
+    const uint32_t leader_bin = (uint32_t)__shfl((int)bin, leader);
+    const uint64_t same = __ballot(have && bin == leader_bin);
+    if (lane == leader) done += fetch_add_coherent(&hist[leader_bin], (uint32_t)__popcll(same));
+    todo &= ~same;
+  }
+  return done;
+}
+
 __device__ __forceinline__ int block_threshold_scan(uint32_t mine, uint32_t need, uint32_t* scratch,
                                                     uint32_t& before_out, uint32_t& total_out) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -638,9 +658,10 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     // Round 4: next 11 bits of the candidates inside bin t0.
     {
       uint32_t done = 0;
-      for (int i = tid; i < count; i += 256) {
-        const uint32_t key = key_of(i);
-        if (key_bin0(key) == t0) done += fetch_add_coherent(&ctr[kSelHist1 + key_bin1(key)], 1u);
+      for (int base = 0; base < count; base += 256) {
+        const uint32_t key = base + tid < count ? key_of(base + tid) : 0u;
+        done += wave_histogram_add(ctr + kSelHist1, base + tid < count && key_bin0(key) == t0,
+                                   key_bin1(key), lane);
       }
       await(done);
     }
@@ -660,10 +681,11 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     // Round 5: last 10 bits of the candidates inside (t0, t1).
     {
       uint32_t done = 0;
-      for (int i = tid; i < count; i += 256) {
-        const uint32_t key = key_of(i);
-        if (key_bin0(key) == t0 && key_bin1(key) == t1)
-          done += fetch_add_coherent(&ctr[kSelHist2 + key_bin2(key)], 1u);
+      for (int base = 0; base < count; base += 256) {
+        const uint32_t key = base + tid < count ? key_of(base + tid) : 0u;
+        done += wave_histogram_add(
+            ctr + kSelHist2, base + tid < count && key_bin0(key) == t0 && key_bin1(key) == t1,
+            key_bin2(key), lane);
       }
       await(done);
     }
