@@ -196,12 +196,8 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
     zero_counters = topk_zero_region(topk, bt->batch);
   if (chunk_rows > 0) {
     // Chunk fingerprint: row i rotated to n_local + i, mean over the rows (tr.py:380-392).
-    TS_TRY(ts_fingerprint(cfg, q, chunk_rows, q_cos, q_sin, table_rows, qf, stream));
-    if (zero_counters.count > 0) {
-      hipLaunchKernelGGL(select_zero_kernel, dim3(8), dim3(256), 0, (hipStream_t)stream,
-                         zero_counters, zero_sync);
-      TS_TRY(check_launch("select_zero_kernel"));
-    }
+    TS_TRY(launch_fingerprint(cfg, q, chunk_rows, q_cos, q_sin, table_rows, qf, zero_counters,
+                              zero_sync, (hipStream_t)stream));
   } else {
     TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
                        zero_counters, zero_sync, (hipStream_t)stream));

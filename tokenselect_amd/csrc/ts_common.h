@@ -42,6 +42,11 @@ struct ZeroRegion {
   int words = 0;
   int count = 0;
 };
+// Chunk fingerprint (ts_prefill.hip) with the same side job as launch_rope: the two
+// regions are cleared by the same launch.
+int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
+                       const float* sin_table, int64_t table_rows, void* qf, const ZeroRegion& zero,
+                       const ZeroRegion& zero2, hipStream_t stream);
 int launch_rope(const void* x, void* out, const float* cos_table, const float* sin_table,
                 const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
                 const ZeroRegion& zero, const ZeroRegion& zero2, hipStream_t stream);

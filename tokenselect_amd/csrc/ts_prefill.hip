@@ -16,20 +16,32 @@ namespace ts {
 // by the row count and rounded to bf16 (torch.mean on a bf16 tensor, tr.py:392).
 constexpr int kFpRowGroups = 16;
 
+constexpr int kFpInFlight = 8;  // rows per step of a row group
+
 __global__ __launch_bounds__(1024) void fingerprint_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ qf, const float* __restrict__ cos_table,
-    const float* __restrict__ sin_table, int64_t table_rows, int first_pos, int rows, int heads) {
+    const float* __restrict__ sin_table, int64_t table_rows, int first_pos, int rows, int heads,
+    ZeroRegion zero, ZeroRegion zero2) {
 #pragma clang fp contract(off)
   constexpr int half = kHeadDim / 2;
   const int h = blockIdx.x;
   const int i = threadIdx.x % half, rg = threadIdx.x / half;
+  // On the side: clear the words the selection kernel after this one counts into.
+  {
+    const int64_t gid = (int64_t)blockIdx.x * 1024 + threadIdx.x, step = (int64_t)gridDim.x * 1024;
+    for (int64_t w = gid; w < (int64_t)zero.count * zero.words; w += step)
+      zero.base[(w / zero.words) * zero.stride + w % zero.words] = 0u;
+    for (int64_t w = gid; w < (int64_t)zero2.count * zero2.words; w += step)
+      zero2.base[(w / zero2.words) * zero2.stride + w % zero2.words] = 0u;
+  }
   float lo_sum = 0.f, hi_sum = 0.f;
-  // Four rows per step: their loads are independent and go out together; the sums
+  // Eight rows per step: their loads are independent and go out together; the sums
   // are still taken in row order.
-  for (int r0 = rg; r0 < rows; r0 += 4 * kFpRowGroups) {
-    float x1[4], x2[4], c1[4], c2[4], s1[4], s2[4];
+  for (int r0 = rg; r0 < rows; r0 += kFpInFlight * kFpRowGroups) {
+    float x1[kFpInFlight], x2[kFpInFlight], c1[kFpInFlight], c2[kFpInFlight], s1[kFpInFlight],
+        s2[kFpInFlight];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kFpInFlight; ++j) {
       const int r = min(r0 + j * kFpRowGroups, rows - 1);
       int64_t pos = (int64_t)first_pos + r;
       pos = pos < table_rows ? pos : table_rows - 1;
@@ -44,7 +56,7 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
       s2[j] = s[i + half];
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kFpInFlight; ++j) {
       if (r0 + j * kFpRowGroups < rows) {
         const float lo = x1[j] * c1[j] + (-x2[j]) * s1[j];
         const float hi = x2[j] * c2[j] + x1[j] * s2[j];
@@ -475,6 +487,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 constexpr size_t kPfLdsBytes = 2 * 2 * (size_t)(kPfTile * kPfKRow + kHeadDim * kPfVRowA) * 2;
 
+int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
+                       const float* sin_table, int64_t table_rows, void* qf, const ZeroRegion& zero,
+                       const ZeroRegion& zero2, hipStream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_REQUIRE(q && cos_table && sin_table && qf, TS_EINVAL, "ts_fingerprint: NULL tensor argument");
+  TS_REQUIRE(rows >= 1, TS_EINVAL, "ts_fingerprint: rows %d < 1", rows);
+  TS_REQUIRE(table_rows >= (int64_t)cfg->n_local + rows, TS_EINVAL,
+             "ts_fingerprint: cos/sin tables have %lld rows, need n_local + rows = %lld",
+             (long long)table_rows, (long long)cfg->n_local + rows);
+  hipLaunchKernelGGL(fingerprint_kernel, dim3((unsigned)cfg->num_heads), dim3(1024), 0, stream,
+                     (const uint16_t*)q, (uint16_t*)qf, cos_table, sin_table, table_rows,
+                     cfg->n_local, rows, cfg->num_heads, zero, zero2);
+  return check_launch("fingerprint_kernel");
+}
+
 static int prefill_s_pad(int max_sel_len) { return (int)ceil_div(max_sel_len, kPfTile) * kPfTile; }
 
 }  // namespace ts
@@ -485,16 +512,8 @@ extern "C" {
 
 int ts_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
                    const float* sin_table, int64_t table_rows, void* qf, ts_stream_t stream) {
-  TS_TRY(validate_config(cfg));
-  TS_REQUIRE(q && cos_table && sin_table && qf, TS_EINVAL, "ts_fingerprint: NULL tensor argument");
-  TS_REQUIRE(rows >= 1, TS_EINVAL, "ts_fingerprint: rows %d < 1", rows);
-  TS_REQUIRE(table_rows >= (int64_t)cfg->n_local + rows, TS_EINVAL,
-             "ts_fingerprint: cos/sin tables have %lld rows, need n_local + rows = %lld",
-             (long long)table_rows, (long long)cfg->n_local + rows);
-  hipLaunchKernelGGL(fingerprint_kernel, dim3((unsigned)cfg->num_heads), dim3(1024), 0,
-                     (hipStream_t)stream, (const uint16_t*)q, (uint16_t*)qf, cos_table, sin_table,
-                     table_rows, cfg->n_local, rows, cfg->num_heads);
-  return check_launch("fingerprint_kernel");
+  return launch_fingerprint(cfg, q, rows, cos_table, sin_table, table_rows, qf, ZeroRegion{},
+                            ZeroRegion{}, (hipStream_t)stream);
 }
 
 size_t ts_prefill_attn_workspace_bytes(const ts_config* cfg, int32_t max_sel_len) {

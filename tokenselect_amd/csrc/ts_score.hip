@@ -211,10 +211,14 @@ __device__ __forceinline__ uint32_t wave_histogram_add(uint32_t* hist, bool have
   while (todo) {
     const int leader = __ffsll((unsigned long long)todo) - 1;
     const uint32_t leader_bin = (uint32_t)__shfl((int)bin, leader);
-    const uint64_t same = __ballot(have && bin == leader_bin);
+    const uint64_t same = __ballot(have && bin == leader_bin) & todo;
+    // Little sharing: the remaining lanes add on their own, in one instruction (a
+    // wavefront whose 64 candidates sit in 64 bins must not issue 64 of them).
+    if (__popcll(same) < 4) break;
     if (lane == leader) done += fetch_add_coherent(&hist[leader_bin], (uint32_t)__popcll(same));
     todo &= ~same;
   }
+  if ((todo >> lane) & 1ull) done += fetch_add_coherent(&hist[bin], 1u);
   return done;
 }
 
