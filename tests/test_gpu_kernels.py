@@ -253,6 +253,73 @@ def test_fused_select_max_pool(dev, kernel, page):
                 assert int(tied_in.max()) < int(tied_out.min()), f"tie order b={b}"
 
 
+@pytest.mark.parametrize("case", ["wide", "narrow", "tie_groups_small", "tie_groups_large"])
+def test_fused_select_every_resolution_path(dev, case):
+    """The single-launch selection resolves the k-th vote by histogram levels until the
+    threshold bin holds at most 256 candidates, which it then lists and ranks: a
+    heavy-tailed vote distribution lists after the first level, a narrow one (tiny
+    query) after the second, many exact ties (keys drawn from a few distinct rows) go
+    through all three levels and the count of ties.  Checked exactly on the kernel's
+    own votes: no unselected vote above a selected one, ties lowest position first."""
+    say(f"fused select resolution path: {case}")
+    L, k = 60000, 1000
+    wl = small(dev, SHAPES[0], seed=90, lens=[L, 9000], ks=[k, 300], page=16, top_k=k, n_init=128,
+               n_local=512)
+    c = wl.cfg
+    g = torch.Generator(device=dev).manual_seed(91)
+    if case == "narrow":
+        wl.q.mul_(0.02)
+    if case.startswith("tie_groups"):
+        groups = 400 if case == "tie_groups_small" else 3
+        distinct = torch.randn(groups, c.num_kv_heads, c.head_dim, device=dev, generator=g).bfloat16()
+        which = torch.randint(groups, (wl.k_pool.shape[0],), device=dev, generator=g)
+        wl.k_pool.copy_(distinct[which])
+    qf = fingerprint(wl, dev)
+    space = None
+    for attempt in range(2):
+        sel, sel_pos, sel_len, votes, space = ops.select(c, wl.batch, qf, wl.k_pool,
+                                                         want_votes=True, workspace=space)
+        torch.cuda.synchronize()
+        assert not ops.select_fault(c, wl.batch, space)
+        for b, (Lb, kb) in enumerate(zip(wl.seq_lens, wl.k_list)):
+            n = Lb - c.n_init - c.n_local
+            assert int(sel_len[b]) == c.n_init + kb + c.n_local
+            v = votes[b, :n]
+            mid = sel_pos[b, c.n_init:c.n_init + kb].long()
+            assert bool((mid[1:] > mid[:-1]).all()), f"{case} b={b}: not ascending"
+            assert int(mid.min()) >= c.n_init and int(mid.max()) < Lb - c.n_local
+            chosen = torch.zeros(n, dtype=torch.bool, device=dev)
+            chosen[mid - c.n_init] = True
+            lowest_in, highest_out = v[chosen].min(), v[~chosen].max()
+            assert float(lowest_in) >= float(highest_out), f"{case} b={b} attempt={attempt}"
+            tied_in = torch.nonzero(chosen & (v == lowest_in)).flatten()
+            tied_out = torch.nonzero(~chosen & (v == lowest_in)).flatten()
+            if tied_out.numel():
+                assert int(tied_in.max()) < int(tied_out.min()), f"{case} b={b}: tie order"
+            # the table translation of the selected positions
+            slots = wl.batch.table[b].long()[mid // c.page_size] * c.page_size + mid % c.page_size
+            assert torch.equal(sel[b, c.n_init:c.n_init + kb].long(), slots)
+        # the case is in the regime it is meant to exercise (request 0)
+        keys = votes[0, :L - 640].view(torch.int32).long() | (1 << 31)
+        kth = keys.sort(descending=True).values[k - 1]
+        in_bin = {bits: int(((keys >> (32 - bits)) == (kth >> (32 - bits))).sum()) for bits in (11, 22)}
+        if case == "wide":
+            assert in_bin[11] <= 256, in_bin
+        elif case == "tie_groups_large":
+            assert in_bin[22] > 256, in_bin
+        else:
+            assert in_bin[11] > 256 >= in_bin[22], in_bin
+    # same inputs through the separate kernels: identical positions
+    scores, partials = ops.score(c, wl.batch, qf, wl.k_pool)
+    votes_sep, _ = ops.vote(c, wl.batch, scores, partials)
+    _, pos_sep, len_sep = ops.topk_ragged(c, wl.batch, votes_sep)
+    assert torch.equal(len_sep, sel_len)
+    for b, Lb in enumerate(wl.seq_lens):
+        n = Lb - c.n_init - c.n_local
+        if torch.equal(votes_sep[b, :n], votes[b, :n]):
+            assert torch.equal(pos_sep[b, :int(len_sep[b])], sel_pos[b, :int(sel_len[b])])
+
+
 @pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
 def test_decode_layer_max_pool(dev, fused_select):
     lens, ks = [5000, 100, 2048, 901], [256, 256, 200, 256]

@@ -32,6 +32,7 @@ struct ScoreArgs {
   int64_t vote_stride;
   uint32_t* counters;     // [B][kSelCounterWords] zero at launch
   uint2* block_counts;    // [B][gridDim.x] (selected for sure, ties at the k-th key)
+  uint2* short_list;      // [B][kSelListParts][kSelListCap] (key, position) of the threshold bin
   int32_t* sel;           // outputs of the selection, as for ts_topk_ragged
   int32_t* sel_pos;
   int64_t sel_stride;
@@ -54,12 +55,20 @@ constexpr int kSelHistCopies = 8;
 constexpr int kSelHist0 = 0;                           // 8 x 2048, top 11 key bits
 constexpr int kSelHist1 = kSelHistCopies * kTopkBins;  // 2048, next 11 bits inside bin t0
 constexpr int kSelHist2 = kSelHist1 + kTopkBins;       // 1024, last 10 bits inside (t0, t1)
-constexpr int kSelMaxBin = kSelHist2 + 1024;           // highest occupied bin of hist0
-constexpr int kSelCounterWords = kSelMaxBin + 64;
+// Highest occupied bin of hist0, one word per copy, 128 bytes apart (hundreds of
+// read-modify-writes of one address, or one line, take microseconds).
+constexpr int kSelMaxBin = kSelHist2 + 1024;
+// Once at most kSelListCap candidates are left in the threshold bin they are listed
+// instead of being resolved by further histogram levels; the list is kept in parts
+// with a fill counter each (128 bytes apart), workgroup x appending to part x % parts.
+constexpr int kSelListCap = 256;
+constexpr int kSelListParts = 8;
+constexpr int kSelListCount = kSelMaxBin + kSelHistCopies * 32;
+constexpr int kSelCounterWords = kSelListCount + kSelListParts * 32;
 
 // Workspace of ts_select, carved in this order (256-byte aligned pieces).
 struct SelectWorkspace {
-  size_t partials, stats, counters, block_counts, pool_votes, sync, total;  // sync stays last
+  size_t partials, stats, counters, block_counts, short_list, pool_votes, sync, total;  // sync stays last
   int64_t pool_stride;
   int tokens_per_block;  // 0: the shape does not fit the fused kernel
   int blocks_per_req;

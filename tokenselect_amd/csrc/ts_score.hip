@@ -194,10 +194,6 @@ __device__ __forceinline__ void fixed_segments(const ScoreArgs& a, int b) {
   for (int i = threadIdx.x; i < a.n_local; i += 256) emit(a.n_init + k + i, L - a.n_local + i);
 }
 
-// 256 threads, thread 0 holding the highest bin: finds the thread at which the
-// running count (from thread 0 on) reaches `need`.  Returns that thread's index
-// (or -1 if the total stays below `need`), the count before it, and the total.
-// `scratch` is LDS of 8 words.
 // Adds the wavefront's candidates to a histogram in memory with one fetch-add per
 // distinct bin: normally a wavefront has a few candidates in different bins, but
 // nearly uniform votes (a query of small norm) put all 64 lanes, of every wavefront,
@@ -222,8 +218,13 @@ __device__ __forceinline__ uint32_t wave_histogram_add(uint32_t* hist, bool have
   return done;
 }
 
+// 256 threads, thread 0 holding the highest bin: finds the thread at which the
+// running count (from thread 0 on) reaches `need`.  Returns that thread's index
+// (or -1 if the total stays below `need`), the count before it, the total, and
+// that thread's own count.  `scratch` is LDS of 8 words.
 __device__ __forceinline__ int block_threshold_scan(uint32_t mine, uint32_t need, uint32_t* scratch,
-                                                    uint32_t& before_out, uint32_t& total_out) {
+                                                    uint32_t& before_out, uint32_t& total_out,
+                                                    uint32_t& count_out) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   uint32_t incl = mine;
 #pragma unroll
@@ -244,10 +245,12 @@ __device__ __forceinline__ int block_threshold_scan(uint32_t mine, uint32_t need
   if (before < need && need <= before + mine) {
     scratch[4] = (uint32_t)tid;
     scratch[5] = before;
+    scratch[6] = mine;
   }
   __syncthreads();
   const uint32_t who = scratch[4];
   before_out = scratch[5];
+  count_out = scratch[6];
   total_out = total;
   __syncthreads();
   return who == 0xffffffffu ? -1 : (int)who;
@@ -594,26 +597,15 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       for (int i = tid; i < count + halo; i += 256) lh[i] = 0u;
       __syncthreads();
     }
-    // Local histogram.  The votes of a wavefront fall into a narrow range of bins, so
-    // the lanes are counted bin by bin with ballots over the 64 bins below the
-    // wavefront's highest one, lane d collecting the count of bin (highest - d);
-    // one LDS atomic per occupied bin follows.  (Atomics of one LDS address are
-    // performed a lane at a time, and a loop over the distinct bins with a shuffle
-    // per bin is no faster.)  Lanes further below add their vote on their own.
+    // Local histogram: one LDS atomic per candidate (lanes that hit the same bin are
+    // performed one after the other, which for 256 candidates is a few hundred cycles).
     for (int base = 0; base < count; base += 256) {
       const bool have = base + tid < count;
       const uint32_t bin = have ? key_bin0(key_of(base + tid)) : 0u;
+      if (have) atomicAdd(&lh[bin], 1u);
       uint32_t top = bin;
 #pragma unroll
       for (int off = 32; off >= 1; off >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, off));
-      uint32_t mine = 0;
-#pragma unroll 16
-      for (int d = 0; d < 64; ++d) {
-        const uint64_t same = __ballot(have && bin + d == top);
-        if (lane == d) mine = (uint32_t)__popcll(same);
-      }
-      if (mine) atomicAdd(&lh[top - lane], mine);
-      if (have && bin + 63 < top) atomicAdd(&lh[bin], 1u);
       if (lane == 0) atomicMax(&scratch[8], top);
     }
     __syncthreads();
@@ -635,12 +627,22 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
           done += __hip_atomic_fetch_add((uint64_t*)&hist0[i], pair, __ATOMIC_RELAXED,
                                          __HIP_MEMORY_SCOPE_AGENT);
       }
-      if (tid == 0) done += fetch_max_coherent(&ctr[kSelMaxBin], scratch[8]);
+      if (tid == 0)
+        done += fetch_max_coherent(&ctr[kSelMaxBin + (blockIdx.x % kSelHistCopies) * 32], scratch[8]);
       await(done);
     }
     grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
-    uint32_t t0 = 0, above0 = 0;
-    for (int top = (int)load_coherent(&ctr[kSelMaxBin]); top >= 0; top -= 256) {
+    uint32_t t0 = 0, above0 = 0, in_bin0 = 0;
+    int top_bin = 0;
+    {
+      uint32_t m = tid < kSelHistCopies ? load_coherent(&ctr[kSelMaxBin + tid * 32]) : 0u;
+#pragma unroll
+      for (int off = kSelHistCopies / 2; off >= 1; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off));
+      if (tid == 0) scratch[8] = m;
+      __syncthreads();
+      top_bin = (int)scratch[8];
+    }
+    for (int top = top_bin; top >= 0; top -= 256) {
       const int bin = top - tid;
       uint32_t part[kSelHistCopies];
 #pragma unroll
@@ -649,18 +651,25 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       uint32_t mine = 0;
 #pragma unroll
       for (int c = 0; c < kSelHistCopies; ++c) mine += part[c];
-      uint32_t before, total;
-      const int who = block_threshold_scan(mine, k - above0, scratch, before, total);
+      uint32_t before, total, in_bin;
+      const int who = block_threshold_scan(mine, k - above0, scratch, before, total, in_bin);
       if (who >= 0) {
         t0 = (uint32_t)(top - who);
         above0 += before;
+        in_bin0 = in_bin;
         break;
       }
       above0 += total;
     }
 
-    // Round 4: next 11 bits of the candidates inside bin t0.
-    {
+    // What is left: `need` of the `in_bin` candidates whose key >> shift equals `prefix`.
+    // As soon as they are few enough, they go to a short list that every workgroup
+    // ranks on its own (the usual case: heavy-tailed votes leave a hundred candidates
+    // in the threshold bin of the first level); otherwise the next histogram level.
+    uint32_t need = k - above0, in_bin = in_bin0, prefix = t0;
+    int shift = 21;
+    if (in_bin > (uint32_t)kSelListCap) {
+      // Round 4: next 11 bits of the candidates inside bin t0.
       uint32_t done = 0;
       for (int base = 0; base < count; base += 256) {
         const uint32_t key = base + tid < count ? key_of(base + tid) : 0u;
@@ -668,52 +677,141 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
                                    key_bin1(key), lane);
       }
       await(done);
-    }
-    grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
-    {
-      uint32_t h[kTopkBins / 256];
+      grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      {
+        uint32_t h[kTopkBins / 256];
 #pragma unroll
-      for (int j = 0; j < kTopkBins / 256; ++j) h[j] = load_coherent(&ctr[kSelHist1 + tid + 256 * j]);
+        for (int j = 0; j < kTopkBins / 256; ++j) h[j] = load_coherent(&ctr[kSelHist1 + tid + 256 * j]);
 #pragma unroll
-      for (int j = 0; j < kTopkBins / 256; ++j) lh[tid + 256 * j] = h[j];
-    }
-    __syncthreads();
-    uint32_t t1, above1;
-    find_threshold_bin<kTopkBins>(lh, k - above0, scratch, t1, above1);
-    const uint32_t need2 = k - above0 - above1;
-
-    // Round 5: last 10 bits of the candidates inside (t0, t1).
-    {
-      uint32_t done = 0;
-      for (int base = 0; base < count; base += 256) {
-        const uint32_t key = base + tid < count ? key_of(base + tid) : 0u;
-        done += wave_histogram_add(
-            ctr + kSelHist2, base + tid < count && key_bin0(key) == t0 && key_bin1(key) == t1,
-            key_bin2(key), lane);
+        for (int j = 0; j < kTopkBins / 256; ++j) lh[tid + 256 * j] = h[j];
       }
-      await(done);
+      __syncthreads();
+      uint32_t t1, above1;
+      find_threshold_bin<kTopkBins>(lh, need, scratch, t1, above1);
+      need -= above1;
+      in_bin = lh[t1];
+      prefix = (t0 << 11) | t1;
+      shift = 10;
+      __syncthreads();
     }
-    grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
-    {
-      uint32_t h[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) h[j] = load_coherent(&ctr[kSelHist2 + tid + 256 * j]);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) lh[tid + 256 * j] = h[j];
-    }
-    __syncthreads();
-    uint32_t t2, above2;
-    find_threshold_bin<1024>(lh, need2, scratch, t2, above2);
-    const uint32_t need_eq = need2 - above2;  // ties at the k-th key still to take
-    const uint32_t kth = (t0 << 21) | (t1 << 10) | t2;
 
-    // Round 6: every workgroup publishes how many of its tokens lie above the k-th
-    // key and how many tie with it; ties are taken lowest position first, so the
-    // counts of the workgroups before this one fix where its output starts and
-    // how many of its ties still fit.
-    if (tid < 4) scratch[8 + tid] = 0u;
+    uint2* counts = a.block_counts + (size_t)b * gridDim.x;
+    const bool listed = in_bin <= (uint32_t)kSelListCap;
+    uint32_t kth, need_eq = 0, pos_thr = 0;
+    if (tid < 8) scratch[8 + tid] = 0u;
     __syncthreads();
-    {
+    if (listed) {
+      // Last round, short form: the candidates of the threshold bin are appended to
+      // the list (in kSelListParts parts with a counter each, a wavefront reserving
+      // its entries with one add), and every workgroup publishes how many of its
+      // tokens lie above the bin.
+      uint2* list = a.short_list + (size_t)b * kSelListParts * kSelListCap;
+      const int part = blockIdx.x % kSelListParts;
+      const uint64_t below_mask = (1ull << lane) - 1ull;
+      uint32_t above = 0;
+      for (int base = 0; base < count; base += 256) {
+        const int i = base + tid;
+        const uint32_t key = i < count ? key_of(i) : 0u;
+        const uint32_t top = key >> shift;
+        above += (i < count && top > prefix) ? 1u : 0u;
+        const bool match = i < count && top == prefix;
+        const uint64_t mm = __ballot(match);
+        if (mm) {
+          const int leader = __ffsll((unsigned long long)mm) - 1;
+          uint32_t slot = 0;
+          if (lane == leader)
+            slot = fetch_add_coherent(&ctr[kSelListCount + part * 32], (uint32_t)__popcll(mm));
+          slot = (uint32_t)__shfl((int)slot, leader) + (uint32_t)__popcll(mm & below_mask);
+          if (match && slot < (uint32_t)kSelListCap)
+            store_coherent(&list[part * kSelListCap + slot], key, (uint32_t)(block_lo + i));
+        }
+      }
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) above += __shfl_xor(above, off);
+      if (lane == 0) atomicAdd(&scratch[8], above);
+      __syncthreads();
+      if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], 0u);
+      grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+
+      // Every workgroup ranks the list on its own: entry t goes to thread t; the order
+      // is (key descending, position ascending), packed into one 64-bit word.
+      uint64_t* ranked = (uint64_t*)lh;
+      if (tid < kSelListParts) scratch[tid] = load_coherent(&ctr[kSelListCount + tid * 32]);
+      __syncthreads();
+      uint32_t entries = 0, at = (uint32_t)tid, from = 0;
+      bool has = false;
+#pragma unroll
+      for (int p = 0; p < kSelListParts; ++p) {
+        const uint32_t c = min(scratch[p], (uint32_t)kSelListCap);
+        if (!has && at < c) {
+          has = true;
+          from = (uint32_t)p;
+        } else if (!has) {
+          at -= c;
+        }
+        entries += c;
+      }
+      entries = min(entries, (uint32_t)kSelListCap);
+      has = has && (uint32_t)tid < entries;
+      uint64_t mine = 0;
+      uint32_t my_pos = 0;
+      if (has) {
+        const uint2 e = load_coherent(&list[from * kSelListCap + at]);
+        mine = ((uint64_t)e.x << 32) | (uint64_t)(0xffffffffu - e.y);
+        my_pos = e.y;
+      }
+      ranked[tid] = mine;
+      if (tid < 8) ranked[256 + tid] = 0ull;  // the ranking loop reads in steps of 8
+      __syncthreads();
+      uint32_t rank = 0;
+      for (uint32_t u0 = 0; u0 < entries; u0 += 8) {
+        uint64_t other[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) other[j] = ranked[u0 + j];  // zero beyond the entries
+#pragma unroll
+        for (int j = 0; j < 8; ++j) rank += other[j] > mine ? 1u : 0u;
+      }
+      const bool taken = has && rank < need;
+      if (has && rank + 1 == need) {  // the k-th of the request
+        scratch[9] = (uint32_t)(mine >> 32);
+        scratch[12] = my_pos;
+      }
+      const uint64_t lower = __ballot(taken && my_pos < (uint32_t)block_lo);
+      if (lane == 0 && lower) atomicAdd(&scratch[13], (uint32_t)__popcll(lower));
+      __syncthreads();
+      kth = scratch[9];
+      pos_thr = scratch[12];
+    } else {
+      // Round 5: last 10 bits of the candidates inside (t0, t1).
+      const uint32_t t1 = prefix & 2047u;
+      {
+        uint32_t done = 0;
+        for (int base = 0; base < count; base += 256) {
+          const uint32_t key = base + tid < count ? key_of(base + tid) : 0u;
+          done += wave_histogram_add(
+              ctr + kSelHist2, base + tid < count && key_bin0(key) == t0 && key_bin1(key) == t1,
+              key_bin2(key), lane);
+        }
+        await(done);
+      }
+      grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      {
+        uint32_t h[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) h[j] = load_coherent(&ctr[kSelHist2 + tid + 256 * j]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) lh[tid + 256 * j] = h[j];
+      }
+      __syncthreads();
+      uint32_t t2, above2;
+      find_threshold_bin<1024>(lh, need, scratch, t2, above2);
+      need_eq = need - above2;  // ties at the k-th key still to take
+      kth = (t0 << 21) | (t1 << 10) | t2;
+
+      // Round 6: every workgroup publishes how many of its tokens lie above the k-th
+      // key and how many tie with it; ties are taken lowest position first, so the
+      // counts of the workgroups before this one fix where its output starts and
+      // how many of its ties still fit.
       uint32_t sure = 0, tie = 0;
       for (int i = tid; i < count; i += 256) {
         const uint32_t key = key_of(i);
@@ -729,12 +827,19 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         atomicAdd(&scratch[8], sure);
         atomicAdd(&scratch[9], tie);
       }
+      __syncthreads();
+      if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], scratch[9]);
+      grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
     }
-    __syncthreads();
-    uint2* counts = a.block_counts + (size_t)b * gridDim.x;
-    if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], scratch[9]);
-    grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+    // The requests of a batch may need different numbers of rounds, and the rendezvous
+    // spans them all: whoever is through counts itself in for the rounds it skipped.
+    if (team.size != gridDim.x) {
+      const uint32_t rounds = kSelectRounds + (a.pool_kernel > 0 ? 1u : 0u);
+      while (round < rounds)
+        grid_arrive(a.sync, ++round, false, a.spin_ticks, team.size, team.index);
+    }
     {
+      // Counts of the workgroups before this one.
       uint32_t sure = 0, tie = 0;
       for (int j = tid; j < (int)blockIdx.x; j += 256) {
         const uint2 v = load_coherent(&counts[j]);
@@ -752,8 +857,9 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       }
     }
     __syncthreads();
-    uint32_t tie_run = scratch[11];                          // ties at lower positions
-    uint32_t out_run = scratch[10] + min(tie_run, need_eq);  // selected at lower positions
+    uint32_t tie_run = scratch[11];  // ties at lower positions
+    // selected at lower positions
+    uint32_t out_run = scratch[10] + (listed ? scratch[13] : min(tie_run, need_eq));
     __syncthreads();
 
     // Emission in position order.
@@ -776,7 +882,10 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         if (w < wave) tie_rank += scratch[w];
         tie_total += scratch[w];
       }
-      const bool chosen = i < count && (key > kth || (tie && tie_rank < need_eq));
+      // A tie is taken if it is among the first need_eq in position order; with the
+      // short list that is: not beyond the position of the k-th entry.
+      const bool tie_taken = listed ? (uint32_t)(block_lo + i) <= pos_thr : tie_rank < need_eq;
+      const bool chosen = i < count && (key > kth || (tie && tie_taken));
       const uint64_t chosen_mask = __ballot(chosen);
       if (lane == 0) scratch[4 + wave] = (uint32_t)__popcll(chosen_mask);
       __syncthreads();
@@ -910,6 +1019,7 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
   w.stats = take(B * H * 2 * sizeof(float));
   w.counters = take(B * kSelCounterWords * 4);
   w.block_counts = take(B * (size_t)w.blocks_per_req * sizeof(uint2));
+  w.short_list = take(B * kSelListParts * kSelListCap * sizeof(uint2));
   w.pool_stride = (int64_t)align_up((size_t)max_n, 64);
   w.pool_votes = take(cfg->pool_kernel > 0 ? B * (size_t)w.pool_stride * sizeof(float) : 0);
   w.sync = take(kSyncWords * 4);
@@ -980,6 +1090,7 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   a.vote_stride = vote_stride;
   a.counters = (uint32_t*)(ws + w.counters);
   a.block_counts = (uint2*)(ws + w.block_counts);
+  a.short_list = (uint2*)(ws + w.short_list);
   a.sel = sel;
   a.sel_pos = sel_pos;
   a.sel_stride = sel_stride;
