@@ -633,24 +633,36 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     }
     grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
     uint32_t t0 = 0, above0 = 0, in_bin0 = 0;
-    int top_bin = 0;
-    {
-      uint32_t m = tid < kSelHistCopies ? load_coherent(&ctr[kSelMaxBin + tid * 32]) : 0u;
-#pragma unroll
-      for (int off = kSelHistCopies / 2; off >= 1; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off));
-      if (tid == 0) scratch[8] = m;
-      __syncthreads();
-      top_bin = (int)scratch[8];
-    }
-    for (int top = top_bin; top >= 0; top -= 256) {
+    // The search starts at the highest occupied bin of the request.  Together with the
+    // words that hold it, the 256 bins below a guess (a little above this workgroup's
+    // own highest bin) are fetched; the guess serves if no bin above it is occupied.
+    const int guess = min((int)scratch[8] + 64, kTopkBins - 1);
+    auto bins_below = [&](int top) {
       const int bin = top - tid;
       uint32_t part[kSelHistCopies];
 #pragma unroll
       for (int c = 0; c < kSelHistCopies; ++c)
         part[c] = bin >= 0 ? load_coherent(&ctr[kSelHist0 + c * kTopkBins + bin]) : 0u;
-      uint32_t mine = 0;
+      uint32_t sum = 0;
 #pragma unroll
-      for (int c = 0; c < kSelHistCopies; ++c) mine += part[c];
+      for (int c = 0; c < kSelHistCopies; ++c) sum += part[c];
+      return sum;
+    };
+    uint32_t mine = bins_below(guess);
+    int top = guess;
+    {
+      uint32_t m = tid < kSelHistCopies ? load_coherent(&ctr[kSelMaxBin + tid * 32]) : 0u;
+#pragma unroll
+      for (int off = kSelHistCopies / 2; off >= 1; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off));
+      __syncthreads();  // every thread has read this workgroup's own highest bin
+      if (tid == 0) scratch[8] = m;
+      __syncthreads();
+      if ((int)scratch[8] > guess) {
+        top = (int)scratch[8];
+        mine = bins_below(top);
+      }
+    }
+    for (;;) {
       uint32_t before, total, in_bin;
       const int who = block_threshold_scan(mine, k - above0, scratch, before, total, in_bin);
       if (who >= 0) {
@@ -660,6 +672,9 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         break;
       }
       above0 += total;
+      top -= 256;
+      if (top < 0) break;
+      mine = bins_below(top);
     }
 
     // What is left: `need` of the `in_bin` candidates whose key >> shift equals `prefix`.
@@ -733,47 +748,74 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], 0u);
       grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
 
-      // Every workgroup ranks the list on its own: entry t goes to thread t; the order
-      // is (key descending, position ascending), packed into one 64-bit word.
-      uint64_t* ranked = (uint64_t*)lh;
-      if (tid < kSelListParts) scratch[tid] = load_coherent(&ctr[kSelListCount + tid * 32]);
+      // Every workgroup ranks the list on its own, one entry per thread, in the order
+      // (key descending, position ascending) packed into one 64-bit word.  The fill
+      // counters, the entries (thread t guesses entry t / parts of part t % parts,
+      // which is right unless a part holds more than 256 / parts) and the counts of
+      // the workgroups before this one are fetched together.
+      constexpr uint32_t kPerPart = kSelListCap / kSelListParts;
+      const uint32_t fill =
+          tid < kSelListParts ? load_coherent(&ctr[kSelListCount + tid * 32]) : 0u;
+      uint2 e = load_coherent(&list[(tid % kSelListParts) * kSelListCap + tid / kSelListParts]);
+      {
+        uint32_t sure = 0;
+        for (int j = tid; j < (int)blockIdx.x; j += 256) sure += load_coherent(&counts[j]).x;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) sure += __shfl_xor(sure, off);
+        if (lane == 0) atomicAdd(&scratch[10], sure);
+      }
+      if (tid < kSelListParts) scratch[tid] = min(fill, (uint32_t)kSelListCap);
       __syncthreads();
-      uint32_t entries = 0, at = (uint32_t)tid, from = 0;
-      bool has = false;
+      uint32_t entries = 0, longest = 0;
 #pragma unroll
       for (int p = 0; p < kSelListParts; ++p) {
-        const uint32_t c = min(scratch[p], (uint32_t)kSelListCap);
-        if (!has && at < c) {
-          has = true;
-          from = (uint32_t)p;
-        } else if (!has) {
-          at -= c;
+        entries += scratch[p];
+        longest = max(longest, scratch[p]);
+      }
+      bool has;
+      if (longest <= kPerPart) {
+        has = (uint32_t)tid / kSelListParts < scratch[tid % kSelListParts];
+      } else {  // uneven parts: entry t of the concatenation
+        uint32_t at = (uint32_t)tid, from = 0;
+        has = false;
+#pragma unroll
+        for (int p = 0; p < kSelListParts; ++p) {
+          if (!has && at < scratch[p]) {
+            has = true;
+            from = (uint32_t)p;
+          } else if (!has) {
+            at -= scratch[p];
+          }
         }
-        entries += c;
+        has = has && (uint32_t)tid < min(entries, (uint32_t)kSelListCap);
+        if (has) e = load_coherent(&list[from * kSelListCap + at]);
       }
-      entries = min(entries, (uint32_t)kSelListCap);
-      has = has && (uint32_t)tid < entries;
-      uint64_t mine = 0;
-      uint32_t my_pos = 0;
-      if (has) {
-        const uint2 e = load_coherent(&list[from * kSelListCap + at]);
-        mine = ((uint64_t)e.x << 32) | (uint64_t)(0xffffffffu - e.y);
-        my_pos = e.y;
-      }
-      ranked[tid] = mine;
-      if (tid < 8) ranked[256 + tid] = 0ull;  // the ranking loop reads in steps of 8
+      const uint64_t mine = has ? ((uint64_t)e.x << 32) | (uint64_t)(0xffffffffu - e.y) : 0ull;
+      const uint32_t my_pos = e.y;
+      // The need-th largest entry: one more histogram level, over the next 8 key bits
+      // and in LDS, leaves the entries of one digit, which rank themselves against
+      // each other (ranking all entries against all would cost 64 K comparisons).
+      uint32_t* digits = lh;                    // [256]
+      uint64_t* peers = (uint64_t*)(lh + 256);  // [kSelListCap] entries of the threshold digit
+      const uint32_t digit = (e.x >> (shift - 8)) & 255u;
+      digits[tid] = 0u;
+      __syncthreads();
+      if (has) atomicAdd(&digits[digit], 1u);
+      __syncthreads();
+      uint32_t above_digit, all_digits, in_digit;
+      const int down = block_threshold_scan(digits[255 - tid], need, scratch, above_digit,
+                                            all_digits, in_digit);
+      const uint32_t threshold_digit = 255u - (uint32_t)down;  // down >= 0: the bin holds the k-th
+      const bool peer = has && digit == threshold_digit;
+      if (peer) peers[atomicAdd(&scratch[14], 1u)] = mine;
       __syncthreads();
       uint32_t rank = 0;
-      for (uint32_t u0 = 0; u0 < entries; u0 += 8) {
-        uint64_t other[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) other[j] = ranked[u0 + j];  // zero beyond the entries
-#pragma unroll
-        for (int j = 0; j < 8; ++j) rank += other[j] > mine ? 1u : 0u;
-      }
-      const bool taken = has && rank < need;
-      if (has && rank + 1 == need) {  // the k-th of the request
-        scratch[9] = (uint32_t)(mine >> 32);
+      if (peer)
+        for (uint32_t u = 0; u < in_digit; ++u) rank += peers[u] > mine ? 1u : 0u;
+      const uint32_t need_here = need - above_digit;
+      const bool taken = has && (digit > threshold_digit || (peer && rank < need_here));
+      if (peer && rank + 1 == need_here) {  // the k-th of the request
+        scratch[9] = e.x;
         scratch[12] = my_pos;
       }
       const uint64_t lower = __ballot(taken && my_pos < (uint32_t)block_lo);
@@ -838,7 +880,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       while (round < rounds)
         grid_arrive(a.sync, ++round, false, a.spin_ticks, team.size, team.index);
     }
-    {
+    if (!listed) {
       // Counts of the workgroups before this one.
       uint32_t sure = 0, tie = 0;
       for (int j = tid; j < (int)blockIdx.x; j += 256) {
