@@ -41,7 +41,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # `--pmc WRITE_SIZE` runs of this script (KiB per dispatch, scaled by what the same
 # counters read for the 256 MiB copy of --calibration-copy); the runs and their
 # figures are recorded under profiles/.  Workloads not measured that way give null.
-MEASURED_TRAFFIC = {"C2": 271244542}  # profiles/decode_layer_c2_hbm_traffic.txt
+MEASURED_TRAFFIC = {"C2": 271191716}  # profiles/decode_layer_c2_hbm_traffic.txt
 
 
 def event_time_us(fn, launches: int, warmup: int, before=None):

@@ -160,12 +160,14 @@ int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
 /* The whole selection in one launch (tr.py:350-373, 424-449 without the [H, n]
  * score tensor, the [n] vote vector or the sort in between): score, per-head
  * softmax, vote, exact k-th largest vote, ascending positions, index assembly.
- * The scores stay in LDS.  The workgroups of the launch meet six times: softmax
- * partials, merged statistics, three histogram rounds over the 11 + 11 + 10
- * bits of the vote keys, and the per-workgroup counts that place each
- * workgroup's selected positions in the output (seven times with
- * cfg->pool_kernel > 0: the max-pool of tr.py:366-369 needs the votes of the
- * neighbouring workgroups).  Outputs and the hit / cache arguments are those of
+ * The scores stay in LDS.  The workgroups of the launch meet four to six times:
+ * softmax partials, merged statistics, then histogram rounds over the 11 + 11 +
+ * 10 bits of the vote keys until at most 256 candidates are left around the k-th
+ * vote, which are listed and ranked by every workgroup in a last round together
+ * with the per-workgroup counts that place its selected positions in the output
+ * (masses of exact ties take all three histogram rounds and a count round; one
+ * more round with cfg->pool_kernel > 0: the max-pool of tr.py:366-369 needs the
+ * votes of the neighbouring workgroups).  Outputs and the hit / cache arguments are those of
  * ts_topk_ragged (same tie rule: lowest position first); votes, when not NULL,
  * also receives the [B, vote_stride] fp32 votes (pooled when pool_kernel > 0).
  * Usable when ts_select_supported() returns 1: pool_kernel at most 256 and batch x

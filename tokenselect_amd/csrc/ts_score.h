@@ -51,8 +51,8 @@ struct ScoreArgs {
 // in kSelHistCopies copies (workgroup x adds to copy x % copies): the votes of a
 // request fall into a few dozen adjacent bins, i.e. one or two cache lines, and
 // hundreds of workgroups adding to the same line serialise in memory.
-constexpr int kSelHistCopies = 8;
-constexpr int kSelHist0 = 0;                           // 8 x 2048, top 11 key bits
+constexpr int kSelHistCopies = 16;
+constexpr int kSelHist0 = 0;                           // copies x 2048, top 11 key bits
 constexpr int kSelHist1 = kSelHistCopies * kTopkBins;  // 2048, next 11 bits inside bin t0
 constexpr int kSelHist2 = kSelHist1 + kTopkBins;       // 1024, last 10 bits inside (t0, t1)
 // Highest occupied bin of hist0, one word per copy, 128 bytes apart (hundreds of

@@ -634,19 +634,22 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
     uint32_t t0 = 0, above0 = 0, in_bin0 = 0;
     // The search starts at the highest occupied bin of the request.  Together with the
-    // words that hold it, the 256 bins below a guess (a little above this workgroup's
+    // words that hold it, the 128 bins below a guess (a little above this workgroup's
     // own highest bin) are fetched; the guess serves if no bin above it is occupied.
-    const int guess = min((int)scratch[8] + 64, kTopkBins - 1);
+    constexpr int kWindow = 128;  // bins per step: two threads per bin, half the copies each
+    const int guess = min((int)scratch[8] + 32, kTopkBins - 1);
     auto bins_below = [&](int top) {
-      const int bin = top - tid;
-      uint32_t part[kSelHistCopies];
+      const int bin = top - (tid >> 1);
+      const int first = (tid & 1) * (kSelHistCopies / 2);
+      uint32_t part[kSelHistCopies / 2];
 #pragma unroll
-      for (int c = 0; c < kSelHistCopies; ++c)
-        part[c] = bin >= 0 ? load_coherent(&ctr[kSelHist0 + c * kTopkBins + bin]) : 0u;
+      for (int c = 0; c < kSelHistCopies / 2; ++c)
+        part[c] = bin >= 0 ? load_coherent(&ctr[kSelHist0 + (first + c) * kTopkBins + bin]) : 0u;
       uint32_t sum = 0;
 #pragma unroll
-      for (int c = 0; c < kSelHistCopies; ++c) sum += part[c];
-      return sum;
+      for (int c = 0; c < kSelHistCopies / 2; ++c) sum += part[c];
+      sum += (uint32_t)__shfl_xor((int)sum, 1);
+      return (tid & 1) ? 0u : sum;  // the even thread of a pair stands for the bin
     };
     uint32_t mine = bins_below(guess);
     int top = guess;
@@ -666,13 +669,13 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       uint32_t before, total, in_bin;
       const int who = block_threshold_scan(mine, k - above0, scratch, before, total, in_bin);
       if (who >= 0) {
-        t0 = (uint32_t)(top - who);
+        t0 = (uint32_t)(top - (who >> 1));
         above0 += before;
         in_bin0 = in_bin;
         break;
       }
       above0 += total;
-      top -= 256;
+      top -= kWindow;
       if (top < 0) break;
       mine = bins_below(top);
     }
