@@ -9,14 +9,17 @@
 namespace ts {
 
 // ------------------------------------------------------------------ fingerprint
-// One workgroup per head, 1024 threads = 64 rotation pairs x 16 row groups.  Row r
+// Two workgroups per head (32 rotation pairs each), 1024 threads = 8 quads of pairs
+// x 128 row groups, so that a chunk of 512 rows is one step of four independent rows
+// per thread (the kernel is bound by the latency of its loads).  Row r
 // is rotated with table row first_pos + r exactly like the rotation kernel (every
 // product and sum rounded on its own, result rounded to bf16, tr.py:104-107); the
 // bf16 values are summed in fp32, row group by row group in a fixed order, divided
 // by the row count and rounded to bf16 (torch.mean on a bf16 tensor, tr.py:392).
-constexpr int kFpRowGroups = 16;
-
-constexpr int kFpInFlight = 8;  // rows per step of a row group
+constexpr int kFpRowGroups = 128;
+constexpr int kFpInFlight = 4;  // rows per step of a row group
+constexpr int kFpVec = 4;       // rotation pairs per thread
+constexpr int kFpSplit = 2;     // workgroups per head
 
 __global__ __launch_bounds__(1024) void fingerprint_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ qf, const float* __restrict__ cos_table,
@@ -24,22 +27,27 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
     ZeroRegion zero, ZeroRegion zero2) {
 #pragma clang fp contract(off)
   constexpr int half = kHeadDim / 2;
+  constexpr int kPairs = half / kFpSplit;   // rotation pairs of this workgroup
+  constexpr int kLanes = kPairs / kFpVec;   // threads per row
+  static_assert(kLanes * kFpRowGroups == 1024, "1024 threads per workgroup");
   const int h = blockIdx.x;
-  const int i = threadIdx.x % half, rg = threadIdx.x / half;
+  const int first_pair = blockIdx.y * kPairs;
+  const int i = first_pair + (threadIdx.x % kLanes) * kFpVec, rg = threadIdx.x / kLanes;
   // On the side: clear the words the selection kernel after this one counts into.
   {
-    const int64_t gid = (int64_t)blockIdx.x * 1024 + threadIdx.x, step = (int64_t)gridDim.x * 1024;
+    const int64_t gid = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 1024 + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * gridDim.y * 1024;
     for (int64_t w = gid; w < (int64_t)zero.count * zero.words; w += step)
       zero.base[(w / zero.words) * zero.stride + w % zero.words] = 0u;
     for (int64_t w = gid; w < (int64_t)zero2.count * zero2.words; w += step)
       zero2.base[(w / zero2.words) * zero2.stride + w % zero2.words] = 0u;
   }
-  float lo_sum = 0.f, hi_sum = 0.f;
-  // Eight rows per step: their loads are independent and go out together; the sums
+  float lo_sum[kFpVec] = {0.f, 0.f, 0.f, 0.f}, hi_sum[kFpVec] = {0.f, 0.f, 0.f, 0.f};
+  // Four rows per step: their loads are independent and go out together; the sums
   // are still taken in row order.
   for (int r0 = rg; r0 < rows; r0 += kFpInFlight * kFpRowGroups) {
-    float x1[kFpInFlight], x2[kFpInFlight], c1[kFpInFlight], c2[kFpInFlight], s1[kFpInFlight],
-        s2[kFpInFlight];
+    uint2 x1[kFpInFlight], x2[kFpInFlight];
+    float4 c1[kFpInFlight], c2[kFpInFlight], s1[kFpInFlight], s2[kFpInFlight];
 #pragma unroll
     for (int j = 0; j < kFpInFlight; ++j) {
       const int r = min(r0 + j * kFpRowGroups, rows - 1);
@@ -48,31 +56,59 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
       const float* c = cos_table + pos * kHeadDim;
       const float* s = sin_table + pos * kHeadDim;
       const size_t base = ((size_t)r * heads + h) * kHeadDim;
-      x1[j] = bf16_to_f32(q[base + i]);
-      x2[j] = bf16_to_f32(q[base + i + half]);
-      c1[j] = c[i];
-      c2[j] = c[i + half];
-      s1[j] = s[i];
-      s2[j] = s[i + half];
+      x1[j] = *(const uint2*)(q + base + i);
+      x2[j] = *(const uint2*)(q + base + i + half);
+      c1[j] = *(const float4*)(c + i);
+      c2[j] = *(const float4*)(c + i + half);
+      s1[j] = *(const float4*)(s + i);
+      s2[j] = *(const float4*)(s + i + half);
     }
 #pragma unroll
     for (int j = 0; j < kFpInFlight; ++j) {
       if (r0 + j * kFpRowGroups < rows) {
-        const float lo = x1[j] * c1[j] + (-x2[j]) * s1[j];
-        const float hi = x2[j] * c2[j] + x1[j] * s2[j];
-        lo_sum += bf16_to_f32(f32_to_bf16(lo));
-        hi_sum += bf16_to_f32(f32_to_bf16(hi));
+        const float a1[kFpVec] = {bf16_to_f32((uint16_t)x1[j].x), bf16_to_f32((uint16_t)(x1[j].x >> 16)),
+                                  bf16_to_f32((uint16_t)x1[j].y), bf16_to_f32((uint16_t)(x1[j].y >> 16))};
+        const float a2[kFpVec] = {bf16_to_f32((uint16_t)x2[j].x), bf16_to_f32((uint16_t)(x2[j].x >> 16)),
+                                  bf16_to_f32((uint16_t)x2[j].y), bf16_to_f32((uint16_t)(x2[j].y >> 16))};
+        const float cc1[kFpVec] = {c1[j].x, c1[j].y, c1[j].z, c1[j].w};
+        const float cc2[kFpVec] = {c2[j].x, c2[j].y, c2[j].z, c2[j].w};
+        const float ss1[kFpVec] = {s1[j].x, s1[j].y, s1[j].z, s1[j].w};
+        const float ss2[kFpVec] = {s2[j].x, s2[j].y, s2[j].z, s2[j].w};
+#pragma unroll
+        for (int e = 0; e < kFpVec; ++e) {
+          const float lo = a1[e] * cc1[e] + (-a2[e]) * ss1[e];
+          const float hi = a2[e] * cc2[e] + a1[e] * ss2[e];
+          lo_sum[e] += bf16_to_f32(f32_to_bf16(lo));
+          hi_sum[e] += bf16_to_f32(f32_to_bf16(hi));
+        }
       }
     }
   }
-  __shared__ float part[kFpRowGroups][kHeadDim];
-  part[rg][i] = lo_sum;
-  part[rg][i + half] = hi_sum;
+  // Columns of this workgroup: its kPairs low halves, then its kPairs high halves.
+  // The row groups are added in order, eight at a time and then the sixteen eights.
+  __shared__ float part[kFpRowGroups][2 * kPairs];
+  __shared__ float part8[kFpRowGroups / 8][2 * kPairs];
+  const int col = i - first_pair;
+#pragma unroll
+  for (int e = 0; e < kFpVec; ++e) {
+    part[rg][col + e] = lo_sum[e];
+    part[rg][col + e + kPairs] = hi_sum[e];
+  }
   __syncthreads();
-  if (threadIdx.x < kHeadDim) {
+  {
+    const int c = threadIdx.x % (2 * kPairs), set = threadIdx.x / (2 * kPairs);
+    float sum = 0.f;
+#pragma unroll
+    for (int g = 0; g < 8; ++g) sum += part[set * 8 + g][c];
+    part8[set][c] = sum;
+  }
+  __syncthreads();
+  if (threadIdx.x < 2 * kPairs) {
     float total = 0.f;
-    for (int g = 0; g < kFpRowGroups; ++g) total += part[g][threadIdx.x];
-    qf[(size_t)h * kHeadDim + threadIdx.x] = f32_to_bf16(total / (float)rows);
+    for (int g = 0; g < kFpRowGroups / 8; ++g) total += part8[g][threadIdx.x];
+    const int c = threadIdx.x;
+    const int dim = c < kPairs ? first_pair + c : half + first_pair + (c - kPairs);
+    qf[(size_t)h * kHeadDim + dim] = f32_to_bf16(total / (float)rows);
   }
 }
 
@@ -496,7 +532,7 @@ int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const 
   TS_REQUIRE(table_rows >= (int64_t)cfg->n_local + rows, TS_EINVAL,
              "ts_fingerprint: cos/sin tables have %lld rows, need n_local + rows = %lld",
              (long long)table_rows, (long long)cfg->n_local + rows);
-  hipLaunchKernelGGL(fingerprint_kernel, dim3((unsigned)cfg->num_heads), dim3(1024), 0, stream,
+  hipLaunchKernelGGL(fingerprint_kernel, dim3((unsigned)cfg->num_heads, kFpSplit), dim3(1024), 0, stream,
                      (const uint16_t*)q, (uint16_t*)qf, cos_table, sin_table, table_rows,
                      cfg->n_local, rows, cfg->num_heads, zero, zero2);
   return check_launch("fingerprint_kernel");
