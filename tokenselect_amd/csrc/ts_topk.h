@@ -8,7 +8,7 @@
 namespace ts {
 
 constexpr int kTopkBins = 2048;          // 11-bit digits
-constexpr int kTopkSlice = 512;          // candidates per workgroup of the hist / mark grids
+constexpr int kTopkSlice = 512;          // least candidates per workgroup of the hist / mark grids
 constexpr int kTopkFinalThreads = 1024;
 constexpr int kTopkPartWords = 512;      // 32-bit bitmap words per workgroup of the final grid
 // Per-request workspace, in 32-bit words:
@@ -40,6 +40,7 @@ struct TopkArgs {
   size_t ws_stride;   // words per request
   int bitmap_words;   // 32-bit words of the bitmap region
   uint32_t cand_cap;  // entries of the candidate list
+  int slice;          // candidates per workgroup of the hist / mark grids (set by launch_topk)
   // Words the last kernel clears for whoever runs next on the stream (the
   // attention's tickets): clear_per_req words per request, or NULL.
   uint32_t* clear;

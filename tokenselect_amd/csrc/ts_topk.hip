@@ -21,6 +21,8 @@
 //
 // The output is sorted without a sort and bit-stable across runs (no result
 // depends on the order in which atomics land).
+#include <stdlib.h>
+
 #include "ts_topk.h"
 
 namespace ts {
@@ -41,13 +43,13 @@ __global__ __launch_bounds__(256) void topk_hist_kernel(TopkArgs a) {
   const ReqGeom geo =
       request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
   const int n = pooled_count(geo.n, a.pool_kernel);
-  const int lo = blockIdx.x * kTopkSlice;
+  const int lo = blockIdx.x * a.slice;
   if (lo >= n) return;
   __shared__ uint32_t lh[kTopkBins];
   for (int i = threadIdx.x; i < kTopkBins; i += 256) lh[i] = 0u;
   __syncthreads();
   const float* votes = a.votes + (int64_t)b * a.vote_stride;
-  for (int i = lo + threadIdx.x; i < min(lo + kTopkSlice, n); i += 256)
+  for (int i = lo + threadIdx.x; i < min(lo + a.slice, n); i += 256)
     atomicAdd(&lh[key_bin0(vote_key(votes[i]))], 1u);
   __syncthreads();
   uint32_t* hist0 = topk_ws(a.ws, a.ws_stride, b) + kTopkHist0;
@@ -61,7 +63,7 @@ __global__ __launch_bounds__(256) void topk_mark_kernel(TopkArgs a) {
   const ReqGeom geo =
       request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
   const int n = pooled_count(geo.n, a.pool_kernel);
-  const int lo = blockIdx.x * kTopkSlice;
+  const int lo = blockIdx.x * a.slice;
   if (lo >= n) return;
 
   __shared__ uint32_t scratch[8];
@@ -77,7 +79,7 @@ __global__ __launch_bounds__(256) void topk_mark_kernel(TopkArgs a) {
   uint2* cand = (uint2*)(ws + kTopkCounterWords + a.bitmap_words);
   const int lane = threadIdx.x & 63;
   // Whole 64-position groups per wave iteration so that a bitmap word has one writer.
-  for (int base = lo + (threadIdx.x & ~63); base < min(lo + kTopkSlice, n); base += 256) {
+  for (int base = lo + (threadIdx.x & ~63); base < min(lo + a.slice, n); base += 256) {
     const int i = base + lane;
     uint32_t key = 0;
     bool gt = false, eq = false;
@@ -323,6 +325,7 @@ TopkArgs make_topk_args(const ts_config* cfg, const ts_batch* bt, const float* v
   a.ws_stride = topk_ws_stride_words(max_n);
   a.clear = nullptr;
   a.clear_per_req = 0;
+  a.slice = kTopkSlice;
   return a;
 }
 
@@ -335,10 +338,26 @@ ZeroRegion topk_zero_region(const TopkArgs& a, int batch) {
   return r;
 }
 
-int launch_topk(const TopkArgs& a, int batch, int max_n, hipStream_t stream, bool counters_zeroed,
+// Candidates per workgroup of the hist / mark grids: every workgroup first searches
+// the first-level histogram on its own, so a large batch gets larger slices (about a
+// thousand workgroups in all), in multiples of the 256 candidates of a pass.
+static int topk_slice(int batch, int max_n) {
+  static const int forced = [] {
+    const char* e = getenv("TS_TOPK_SLICE");  // tuning override, multiple of 256
+    const int v = e ? atoi(e) : 0;
+    return (v >= 256 && v <= 65536) ? v / 256 * 256 : 0;
+  }();
+  if (forced) return forced;
+  const int64_t per = ceil_div(ceil_div((int64_t)batch * max_n, 1024), 256) * 256;
+  return (int)(per < kTopkSlice ? kTopkSlice : (per > 4096 ? 4096 : per));
+}
+
+int launch_topk(const TopkArgs& args, int batch, int max_n, hipStream_t stream, bool counters_zeroed,
                 bool hist0_filled) {
+  TopkArgs a = args;
+  a.slice = topk_slice(batch, max_n);
   if (max_n > 0) {
-    const dim3 grid((unsigned)ceil_div(max_n, kTopkSlice), (unsigned)batch);
+    const dim3 grid((unsigned)ceil_div(max_n, a.slice), (unsigned)batch);
     if (!counters_zeroed) {
       hipLaunchKernelGGL(topk_zero_kernel, dim3((unsigned)batch), dim3(256), 0, stream, a.ws,
                          a.ws_stride);
