@@ -320,6 +320,70 @@ def test_fused_select_every_resolution_path(dev, case):
             assert torch.equal(pos_sep[b, :int(len_sep[b])], sel_pos[b, :int(sel_len[b])])
 
 
+def test_select_randomised(dev):
+    """Both forms of the selection (single launch; score + vote + ragged top-k).  Seeded sweep over shapes, ragged batches, page sizes, sink / local sizes, k (zero
+    included), max-pool windows and vote distributions (heavy-tailed, nearly uniform,
+    tie groups of about 256 = the capacity of the short candidate list, all equal):
+    the middle segment is exactly the k best of the kernel's own votes, ties lowest
+    position first; the sink, the local window and the slot translation are exact."""
+    import random
+    for seed in range(60):
+        rnd = random.Random(1000 + seed)
+        shape = rnd.choice(SHAPES)
+        B = rnd.choice([1, 1, 2, 3, 5])
+        lens = [rnd.randint(30, 40000 if seed % 4 == 0 else 6000) for _ in range(B)]
+        top_k = rnd.choice([1, 17, 100, 256, 1000, 2048])
+        ks = [rnd.randint(0, top_k) if rnd.random() < 0.2 else top_k for _ in range(B)]
+        page = rnd.choice([1, 16])
+        n_init, n_local = rnd.choice([(0, 1), (8, 16), (128, 512)])
+        pool = rnd.choice([-1, -1, 5, 6, 32])
+        mode = rnd.choice(["wide", "narrow", "ties", "ties256", "zero"])
+        say(f"randomised select seed={seed} H={shape['num_heads']}/{shape['num_kv_heads']} lens={lens} "
+            f"ks={ks} page={page} sink/local={n_init}/{n_local} pool={pool} votes={mode}")
+        wl = small(dev, shape, seed=seed, lens=lens, ks=ks, page=page, n_init=n_init, n_local=n_local,
+                   top_k=top_k, pool_kernel=pool)
+        c = wl.cfg
+        if not ops.select_supported(c, B, max(lens)):
+            continue
+        g = torch.Generator(device=dev).manual_seed(seed)
+        if mode == "narrow":
+            wl.q.mul_(rnd.choice([0.02, 0.1]))
+        elif mode == "zero":
+            wl.q.zero_()
+        elif mode in ("ties", "ties256"):
+            n0 = max(lens[0] - n_init - n_local, 1)
+            groups = (max(1, n0 // rnd.choice([250, 256, 257, 300])) if mode == "ties256"
+                      else rnd.choice([2, 7, 40, 400]))
+            distinct = torch.randn(groups, c.num_kv_heads, c.head_dim, device=dev, generator=g).bfloat16()
+            which = torch.randint(groups, (wl.k_pool.shape[0],), device=dev, generator=g)
+            wl.k_pool.copy_(distinct[which])
+        qf = fingerprint(wl, dev)
+        sel, sel_pos, sel_len, votes, space = ops.select(c, wl.batch, qf, wl.k_pool, want_votes=True)
+        torch.cuda.synchronize()
+        assert not ops.select_fault(c, wl.batch, space)
+        votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool))
+        separate = ops.topk_ragged(c, wl.batch, votes_sep)
+        for path, (sel, sel_pos, sel_len), votes in (("fused", (sel, sel_pos, sel_len), votes),
+                                                     ("separate", separate, votes_sep)):
+            for b, (L, k) in enumerate(zip(lens, ks)):
+                what = f"seed={seed} b={b} {path}"
+                S = int(sel_len[b])
+                if n_init + k + n_local >= L:
+                    assert S == L and torch.equal(sel_pos[b, :L].cpu(), torch.arange(L, dtype=torch.int32))
+                    continue
+                n_out = L - n_init - n_local - (1 if (pool > 0 and pool % 2 == 0) else 0)
+                assert S == n_init + k + n_local, what
+                best = torch.sort(votes[b, :n_out], descending=True, stable=True).indices[:k]
+                expect = torch.sort(best).values + n_init
+                assert torch.equal(sel_pos[b, n_init:n_init + k].long(), expect), what
+                assert torch.equal(sel_pos[b, :n_init].cpu(), torch.arange(n_init, dtype=torch.int32))
+                assert torch.equal(sel_pos[b, n_init + k:S].cpu(),
+                                   torch.arange(L - n_local, L, dtype=torch.int32))
+                pos = sel_pos[b, :S].long()
+                slots = wl.batch.table[b].long()[pos // page] * page + pos % page
+                assert torch.equal(sel[b, :S].long(), slots), what
+
+
 @pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
 def test_decode_layer_max_pool(dev, fused_select):
     lens, ks = [5000, 100, 2048, 901], [256, 256, 200, 256]
