@@ -65,6 +65,20 @@ constexpr int kSyncLiveWords = 16;
 constexpr int kSyncMaxRounds = kSyncLiveWords - 2;
 constexpr size_t kSyncWords = (size_t)(kSyncSlots + 1) * kSyncSlotWords;
 
+// One thread polls the replica of its workgroup until `round` is complete.
+__device__ __forceinline__ void grid_poll(uint32_t* sync, uint32_t round, uint64_t ticks,
+                                          uint32_t index) {
+  const uint32_t* flag = &sync[(size_t)(index % kSyncSlots + 1) * kSyncSlotWords];
+  const uint64_t t0 = wall_clock64();
+  for (uint32_t polls = 1; load_coherent(flag) < round; ++polls) {
+    if ((polls & 255u) == 0 && wall_clock64() - t0 > ticks) {
+      __hip_atomic_store(&sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(2);
+  }
+}
+
 // Every participating workgroup arrives exactly once per round; those that need the others' data
 // of that round wait for it to complete.  Each thread first waits for its
 // outstanding memory operations (what it published has been performed by then);
@@ -101,17 +115,17 @@ __device__ __forceinline__ void grid_arrive(uint32_t* sync, uint32_t round, bool
       __hip_atomic_fetch_max(&sync[(size_t)(threadIdx.x + 1) * kSyncSlotWords], round,
                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else if (wait && threadIdx.x == 0) {
-      const uint32_t* flag = &sync[(size_t)(index % kSyncSlots + 1) * kSyncSlotWords];
-      const uint64_t t0 = wall_clock64();
-      for (uint32_t polls = 1; load_coherent(flag) < round; ++polls) {
-        if ((polls & 255u) == 0 && wall_clock64() - t0 > ticks) {
-          __hip_atomic_store(&sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          break;
-        }
-        __builtin_amdgcn_s_sleep(2);
-      }
+      grid_poll(sync, round, ticks, index);
     }
   }
+  __syncthreads();
+}
+
+// The second half of a rendezvous for a workgroup that arrived without waiting and
+// did other work in the meantime.
+__device__ __forceinline__ void grid_wait(uint32_t* sync, uint32_t round, uint64_t ticks,
+                                          uint32_t index) {
+  if (threadIdx.x == 0) grid_poll(sync, round, ticks, index);
   __syncthreads();
 }
 

@@ -483,6 +483,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   if (a.partials == nullptr) return;
 
   // Per-workgroup (max, sum exp) of every head: 16 lanes of a row, then 4 waves.
+  __shared__ float local_max[MODE == kScoreFused ? kMaxHeads : 1];  // by head slot
   __shared__ float sm_m[4][4][HKV][NA];
   __shared__ float sm_l[4][4][HKV][NA];
 #pragma unroll
@@ -508,15 +509,16 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       for (int w = 1; w < 4; ++w) softmax_merge(m, l, sm_m[w][g4][kvh][na], sm_l[w][g4][kvh][na]);
       const int h = head_of<HKV, G>(kvh, g, a.head_map);
       float2* out = (float2*)a.partials + ((size_t)b * H + h) * a.nchunks + blockIdx.x;
-      if (MODE == kScoreFused)
+      if (MODE == kScoreFused) {
         store_coherent(out, m, l);
-      else
+        local_max[kvh * G + g] = m;
+      } else {
         *out = make_float2(m, l);
+      }
     }
   }
 
   if constexpr (MODE == kScoreFused) {
-    __shared__ float s_max[kMaxHeads];
     __shared__ float s_rz[kMaxHeads];
     __shared__ uint32_t lh[kTopkBins];
     __shared__ uint32_t scratch[16];
@@ -525,18 +527,9 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     if (tid < 16) scratch[tid] = 0u;
     grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
     merge_request_stats(a, team, lane, wave);
-    grid_arrive(a.sync, 2, true, a.spin_ticks, team.size, team.index);
-    for (int slot = tid; slot < H; slot += 256) {
-      const int h = head_of<HKV, G>(slot / G, slot % G, a.head_map);
-      const float2 st = load_coherent((const float2*)a.stats + (size_t)b * H + h);
-      s_max[slot] = st.x;
-      s_rz[slot] = 1.0f / st.y;
-    }
-    __syncthreads();
-
-    // Votes of this workgroup's tokens: fp32 sum over the head slots in slot order.
-    // The vote replaces the first score of its token in LDS (only the thread that
-    // owns a token reads its column).
+    grid_arrive(a.sync, 2, false, a.spin_ticks, team.size, team.index);
+    // While the merged statistics are on their way: the exponentials, relative to this
+    // workgroup's own maxima; exp(s - max) / sum = exp(s - own max) * exp(own max - max) / sum.
     const ReqGeom geo =
         request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
     const uint32_t k = (uint32_t)geo.k;
@@ -546,7 +539,6 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     auto key_of = [&](int i) -> uint32_t { return vote_key(*column(i)); };
     for (int i = tid; i < count; i += 256) {
       float* sc = column(i);
-      float c = 0.f;
 #pragma unroll
       for (int s0 = 0; s0 < HKV * G; s0 += 8) {  // H = HKV * G head slots, 8 LDS reads in flight
         float x[8];
@@ -554,7 +546,31 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         for (int j = 0; j < 8; ++j) x[j] = s0 + j < HKV * G ? sc[(s0 + j) * 16] : 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-          if (s0 + j < HKV * G) c += __expf(x[j] - s_max[s0 + j]) * s_rz[s0 + j];
+          if (s0 + j < HKV * G) sc[(s0 + j) * 16] = __expf(x[j] - local_max[s0 + j]);
+      }
+    }
+    grid_wait(a.sync, 2, a.spin_ticks, team.index);
+    for (int slot = tid; slot < H; slot += 256) {
+      const int h = head_of<HKV, G>(slot / G, slot % G, a.head_map);
+      const float2 st = load_coherent((const float2*)a.stats + (size_t)b * H + h);
+      s_rz[slot] = __expf(local_max[slot] - st.x) / st.y;
+    }
+    __syncthreads();
+
+    // Votes of this workgroup's tokens: fp32 sum over the head slots in slot order.
+    // The vote replaces the first score of its token in LDS (only the thread that
+    // owns a token reads its column).
+    for (int i = tid; i < count; i += 256) {
+      float* sc = column(i);
+      float c = 0.f;
+#pragma unroll
+      for (int s0 = 0; s0 < HKV * G; s0 += 8) {
+        float x[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] = s0 + j < HKV * G ? sc[(s0 + j) * 16] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (s0 + j < HKV * G) c += x[j] * s_rz[s0 + j];
       }
       if (a.votes && a.pool_kernel <= 0) a.votes[(size_t)b * a.vote_stride + block_lo + i] = c;
       sc[0] = c;
