@@ -1,4 +1,6 @@
 // Rotation of the scoring query: RotaryEmbedding.apply_rotary_pos_emb, tr.py:98-107.
+#include <algorithm>
+
 #include "ts_common.h"
 
 namespace ts {
@@ -48,7 +50,9 @@ int launch_rope(const void* x, void* out, const float* cos_table, const float* s
                 const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
                 const ZeroRegion& zero, const ZeroRegion& zero2, hipStream_t stream) {
   const int64_t pairs = rows * heads * (dim / 2);
-  const int64_t blocks = ceil_div(pairs, 256);
+  // Enough workgroups for the clearing on the side as well: four words per thread.
+  const int64_t to_clear = (int64_t)zero.count * zero.words + (int64_t)zero2.count * zero2.words;
+  const int64_t blocks = std::max(ceil_div(pairs, 256), ceil_div(to_clear, 1024));
   TS_REQUIRE(blocks <= 0x7fffffff, TS_EINVAL, "ts_rope_apply: too many rows");
   hipLaunchKernelGGL(rope_apply_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
                      (const uint16_t*)x, (uint16_t*)out, cos_table, sin_table, position_ids,
