@@ -497,6 +497,31 @@ def test_decode_layer(dev, shape, page, fused_select):
     check_layer(wl, dev, "decode_layer")
 
 
+@pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
+def test_decode_layer_object_serves_smaller_batches(dev, fused_select):
+    """A layer object sized for the largest batch and context is called with batches of
+    changing size and length, as a serving loop does; every call gives what a fresh
+    object of exactly that size gives."""
+    say(f"decode_layer: one object, changing batches, fused={fused_select}")
+    shape = SHAPES[0]
+    big = None
+    for seed, lens, ks in ((31, [5000, 100, 2048, 901], [256, 256, 200, 256]),
+                           (32, [700], [256]),
+                           (33, [6000, 3000, 5999, 64, 1200], [256, 100, 256, 256, 7]),
+                           (34, [2500, 2600], [256, 256])):
+        wl = small(dev, shape, seed=seed, lens=lens, ks=ks, page=16, top_k=256, n_init=16, n_local=32)
+        big = big or ops.DecodeLayer(wl.cfg, 5, 6000, dev)
+        out, sel, sel_pos, sel_len = [t.clone() for t in big(wl.q, wl.k_pool, wl.v_pool, wl.batch)]
+        fresh = ops.DecodeLayer(wl.cfg, len(lens), max(lens), dev)
+        out2, sel2, pos2, len2 = fresh(wl.q, wl.k_pool, wl.v_pool, wl.batch)
+        torch.cuda.synchronize()
+        assert torch.equal(sel_len, len2), f"lens={lens}"
+        for b in range(len(lens)):
+            S = int(sel_len[b])
+            assert torch.equal(sel_pos[b, :S], pos2[b, :S]) and torch.equal(sel[b, :S], sel2[b, :S])
+        assert torch.equal(out.view(torch.int16), out2.view(torch.int16)), f"lens={lens}"
+
+
 @pytest.mark.parametrize("shape", SHAPES[2:], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
 @pytest.mark.parametrize("fused_select", [True], indirect=True, ids=["fused"])
 def test_decode_layer_fused_shapes(dev, shape, fused_select):

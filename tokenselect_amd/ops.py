@@ -488,27 +488,28 @@ class DecodeLayer:
                  cache: Optional[SelectionCache] = None, out: Optional[torch.Tensor] = None):
         cfg = self.cfg
         cb = _c_batch(cfg, bt)
-        if bt.batch != self.batch or bt.max_seq_len > self.max_seq_len:
+        if bt.batch > self.batch or bt.max_seq_len > self.max_seq_len:
             raise ValueError("batch / max_seq_len exceed what this DecodeLayer was sized for")
         _need(q, "q", torch.bfloat16)
-        if q.numel() != self.batch * cfg.num_heads * cfg.head_dim:
+        B = bt.batch
+        if q.numel() != B * cfg.num_heads * cfg.head_dim:
             raise ValueError("q must hold B*H*D elements")
         _check_pool(cfg, k_pool, "k_pool")
         _check_pool(cfg, v_pool, "v_pool")
         if k_pool.shape != v_pool.shape:
             raise ValueError("k_pool and v_pool must have the same shape")
         if out is None:
-            out = self.out
+            out = self.out[:B]
         else:
             _need(out, "out", torch.bfloat16)
-            if out.numel() != self.out.numel():
+            if out.numel() != q.numel():
                 raise ValueError("out must hold B*H*D elements")
         _lib.check(_lib.load().ts_decode_layer(
             ctypes.byref(self._c), ctypes.byref(cb), _p(q), _p(self.q_cos), _p(self.q_sin),
-            _p(k_pool), _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, self.batch), _p(out),
+            _p(k_pool), _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, B), _p(out),
             _p(self.sel), _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
             self.workspace.numel(), _stream()))
-        return out, self.sel, self.sel_pos, self.sel_len
+        return out, self.sel[:B], self.sel_pos[:B], self.sel_len[:B]
 
 
 # ---------------------------------------------------------------- chunked prefill
