@@ -199,7 +199,9 @@ int ts_selcache_step(const ts_config* cfg, const ts_batch* bt, const void* qf,
  * tr.py:815-823.  Head h reads KV head h/(H/Hkv); with TS_ROPE_LLAMA the query
  * is rotated to position S-1 and selected key j to position j inside the kernel.
  * q, out: [B,H,D] bf16; k_pool, v_pool: [pool_rows,Hkv,D] bf16;
- * sel [B, sel_stride] int32 with sel_len[b] valid entries (<= max_sel_len). */
+ * sel [B, sel_stride] int32 with sel_len[b] valid entries (<= max_sel_len); every
+ * row holds at least max_sel_len entries, those past sel_len[b] are read (the
+ * slots are requested together with the length) but not used. */
 size_t ts_attn_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_sel_len);
 int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_pool,
                           const void* v_pool, int64_t pool_rows, const int32_t* sel,

@@ -67,10 +67,11 @@ constexpr int kAttnInFlight = 8;  // tokens per lane group requested together
 template <int G, bool ROPE, bool CAP>
 __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
-  const int S = min(max(a.sel_len[b], 0), a.max_sel_len);
-  const int chunk = (S + a.nsplit - 1) / a.nsplit;
+  // The ranges are cut from the longest list the launch was sized for, not from this
+  // request's own length: the first slots can then be requested together with the
+  // length instead of after it (a shorter request leaves its last workgroups idle).
+  const int chunk = (a.max_sel_len + a.nsplit - 1) / a.nsplit;
   const int lo = split * chunk;
-  const int hi = min(S, lo + chunk);
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int lg = tid >> 4;   // lane group 0..15 inside the workgroup
@@ -82,16 +83,17 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   const int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
   const size_t row_elems = (size_t)a.num_kv_heads * kHeadDim;
 
-  // First batch of slots: requested before the rotation set-up below.
+  // First batch of slots: requested before the rotation set-up below.  Entries past
+  // the request's length are read (they lie inside its row of `sel`) and never used.
   uint32_t slot[kAttnInFlight];
   auto load_slots = [&](int j0) {
 #pragma unroll
-    for (int u = 0; u < kAttnInFlight; ++u) {
-      const int j = min(j0 + 16 * u, max(hi - 1, 0));
-      slot[u] = hi > lo ? (uint32_t)sel[j] : 0u;
-    }
+    for (int u = 0; u < kAttnInFlight; ++u)
+      slot[u] = (uint32_t)sel[min(j0 + 16 * u, a.max_sel_len - 1)];
   };
   load_slots(lo + lg);
+  const int S = min(max(a.sel_len[b], 0), a.max_sel_len);
+  const int hi = min(S, lo + chunk);
 
   // Frequencies of this lane's 4 rotation pairs: theta^(-2 pair / 128) / scale.
   float freq[4];
@@ -310,21 +312,21 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   if (!s_last) return;
 
   // out[b,h,:] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s, rounded to
-  // bf16; splits in index order, 16 of them in flight.
+  // bf16; splits in index order, 32 of them in flight.
   for (int idx = tid; idx < G * (kHeadDim / 2); idx += 256) {
     const int g = idx / (kHeadDim / 2), d = (idx % (kHeadDim / 2)) * 2;
     const size_t ph = ((size_t)b * H + (size_t)kvh * G + g) * a.nsplit;
     float mm = kNegBig, ll = 0.f, o0 = 0.f, o1 = 0.f;
-    for (int s0 = 0; s0 < a.nsplit; s0 += 16) {
-      float2 ml[16], ac[16];
+    for (int s0 = 0; s0 < a.nsplit; s0 += 32) {
+      float2 ml[32], ac[32];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
+      for (int i = 0; i < 32; ++i) {
         const int sp = min(s0 + i, a.nsplit - 1);
         ml[i] = load_coherent2(a.part_ml + (ph + sp) * 2);
         ac[i] = load_coherent2(a.part_acc + (ph + sp) * kHeadDim + d);
       }
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
+      for (int i = 0; i < 32; ++i) {
         if (s0 + i < a.nsplit) {
           const float mn = fmaxf(mm, ml[i].x);
           const float a1 = __expf(mm - mn), a2 = __expf(ml[i].x - mn);
