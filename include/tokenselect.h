@@ -186,6 +186,20 @@ int ts_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const vo
               int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
               int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
               int64_t vote_stride, void* workspace, size_t workspace_bytes, ts_stream_t stream);
+/* ts_select is two launches: a small kernel that clears the counters and rendezvous
+ * words in the workspace, and the selection kernel.  A caller that has another
+ * kernel of its own clear them (ts_decode_layer folds the clearing into its rotation
+ * kernel), or that wants to time the selection kernel alone, makes the two calls
+ * itself: ts_select_clear() once before every ts_select_cleared() on the same
+ * workspace, for the same cfg, batch and max_seq_len.  Same arguments, results and
+ * errors as ts_select.  No counterpart in the reference. */
+int ts_select_clear(const ts_config* cfg, const ts_batch* bt, void* workspace,
+                    size_t workspace_bytes, ts_stream_t stream);
+int ts_select_cleared(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+                      int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
+                      int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
+                      int64_t vote_stride, void* workspace, size_t workspace_bytes,
+                      ts_stream_t stream);
 
 /* Selection-cache decision (tr.py:394-401, 416-421) for one layer, no host
  * sync: hit[b] = cache_len[b] > 0 && cos(q_cache[b], qf[b]) >= threshold; on a

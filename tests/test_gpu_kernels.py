@@ -149,6 +149,32 @@ def test_fused_select(dev, shape, page):
             assert torch.equal(sel[b, :S].cpu(), tabs[b][pos.long()])
 
 
+def test_select_clear_then_cleared_equals_select(dev):
+    """ts_select is ts_select_clear + ts_select_cleared: the two calls made by hand,
+    twice in a row on one workspace, give what the single call gives."""
+    say("select_clear + select(cleared) against select")
+    lens, ks = [3000, 777, 40, 1531], [64, 100, 64, 1]
+    wl = small(dev, SHAPES[0], seed=5, lens=lens, ks=ks, page=16, top_k=100)
+    c = wl.cfg
+    qf = fingerprint(wl, dev)
+    want = ops.select(c, wl.batch, qf, wl.k_pool, want_votes=True)
+    space = ops.select_workspace(c, wl.batch, dev)
+    for attempt in range(2):
+        ops.select_clear(c, wl.batch, space)
+        got = ops.select(c, wl.batch, qf, wl.k_pool, want_votes=True, workspace=space, cleared=True)
+        torch.cuda.synchronize()
+        assert not ops.select_fault(c, wl.batch, space)
+        assert torch.equal(got[2], want[2])
+        for b, L in enumerate(lens):
+            S = int(want[2][b])
+            assert torch.equal(got[0][b, :S], want[0][b, :S]) and torch.equal(got[1][b, :S], want[1][b, :S])
+            n = L - c.n_init - c.n_local
+            if n > 0 and S < L:
+                assert torch.equal(got[3][b, :n], want[3][b, :n])
+    with pytest.raises(ValueError, match="cleared"):
+        ops.select(c, wl.batch, qf, wl.k_pool, cleared=True)
+
+
 def test_fused_select_ties(dev):
     """Duplicated key rows give exactly equal votes: the k-th vote is shared by many
     candidates and the ones at the lowest positions must win, as in the separate

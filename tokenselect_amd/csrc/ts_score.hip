@@ -1232,14 +1232,42 @@ size_t ts_select_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t ma
   return select_workspace(cfg, batch, max_seq_len).total;
 }
 
-int ts_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
-              int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
-              int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
-              int64_t vote_stride, void* workspace, size_t workspace_bytes, ts_stream_t stream) {
+// Argument checks shared by the three forms of the call.
+static int check_select(const ts_config* cfg, const ts_batch* bt, const void* workspace,
+                        size_t workspace_bytes, SelectWorkspace* w_out) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
-  TS_REQUIRE(qf && k_pool && sel && sel_pos && sel_len && workspace, TS_EINVAL,
-             "ts_select: NULL tensor argument");
+  TS_REQUIRE(workspace != nullptr, TS_EINVAL, "ts_select: NULL workspace");
+  const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len);
+  TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE,
+             "ts_select: batch %d x %d tokens does not fit one co-resident grid (or pool_kernel is "
+             "above 256); use ts_score + ts_vote + ts_topk_ragged",
+             bt->batch, bt->max_seq_len);
+  TS_REQUIRE(workspace_bytes >= w.total, TS_EWORKSPACE, "ts_select: workspace %zu bytes < required %zu",
+             workspace_bytes, w.total);
+  *w_out = w;
+  return TS_OK;
+}
+
+int ts_select_clear(const ts_config* cfg, const ts_batch* bt, void* workspace,
+                    size_t workspace_bytes, ts_stream_t stream) {
+  SelectWorkspace w;
+  TS_TRY(check_select(cfg, bt, workspace, workspace_bytes, &w));
+  ZeroRegion counters, sync;
+  select_zero_regions(w, workspace, bt->batch, &counters, &sync);
+  hipLaunchKernelGGL(select_zero_kernel, dim3((unsigned)(8 * bt->batch)), dim3(256), 0,
+                     (hipStream_t)stream, counters, sync);
+  return check_launch("select_zero_kernel");
+}
+
+int ts_select_cleared(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+                      int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
+                      int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
+                      int64_t vote_stride, void* workspace, size_t workspace_bytes,
+                      ts_stream_t stream) {
+  SelectWorkspace w;
+  TS_TRY(check_select(cfg, bt, workspace, workspace_bytes, &w));
+  TS_REQUIRE(qf && k_pool && sel && sel_pos && sel_len, TS_EINVAL, "ts_select: NULL tensor argument");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   const int max_sel = cfg->n_init + cfg->top_k + cfg->n_local;
@@ -1253,20 +1281,17 @@ int ts_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const vo
   if (cache)
     TS_REQUIRE(cache->topk_cache && cache->cache_len, TS_EINVAL,
                "ts_select: selection cache has a NULL array");
-  const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len);
-  TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE,
-             "ts_select: batch %d x %d tokens does not fit one co-resident grid (or pool_kernel is "
-             "above 256); use ts_score + ts_vote + ts_topk_ragged",
-             bt->batch, bt->max_seq_len);
-  TS_REQUIRE(workspace_bytes >= w.total, TS_EWORKSPACE, "ts_select: workspace %zu bytes < required %zu",
-             workspace_bytes, w.total);
-  ZeroRegion counters, sync;
-  select_zero_regions(w, workspace, bt->batch, &counters, &sync);
-  hipLaunchKernelGGL(select_zero_kernel, dim3((unsigned)(8 * bt->batch)), dim3(256), 0,
-                     (hipStream_t)stream, counters, sync);
-  TS_TRY(check_launch("select_zero_kernel"));
   return launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,
                        votes, vote_stride, workspace, nullptr, 0, (hipStream_t)stream);
+}
+
+int ts_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+              int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
+              int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
+              int64_t vote_stride, void* workspace, size_t workspace_bytes, ts_stream_t stream) {
+  TS_TRY(ts_select_clear(cfg, bt, workspace, workspace_bytes, stream));
+  return ts_select_cleared(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride,
+                           sel_len, votes, vote_stride, workspace, workspace_bytes, stream);
 }
 
 int ts_paged_matmul(const void* query, const void* token, int64_t pool_rows,

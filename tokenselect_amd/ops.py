@@ -245,14 +245,28 @@ def select_supported(cfg: LayerConfig, batch: int, max_seq_len: int) -> bool:
                                                 int(max_seq_len)))
 
 
+def select_clear(cfg: LayerConfig, bt: Batch, workspace: torch.Tensor) -> None:
+    """Clears what :func:`select` with ``cleared=True`` wants zero in ``workspace``."""
+    _lib.check(_lib.load().ts_select_clear(ctypes.byref(cfg.to_c()), ctypes.byref(_c_batch(cfg, bt)),
+                                           _p(workspace), workspace.numel(), _stream()))
+
+
+def select_workspace(cfg: LayerConfig, bt: Batch, device) -> torch.Tensor:
+    nbytes = _lib.load().ts_select_workspace_bytes(ctypes.byref(cfg.to_c()), bt.batch, bt.max_seq_len)
+    return torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=device)
+
+
 def select(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
            hit: Optional[torch.Tensor] = None, cache: Optional[SelectionCache] = None,
-           want_votes: bool = False, workspace: Optional[torch.Tensor] = None):
+           want_votes: bool = False, workspace: Optional[torch.Tensor] = None,
+           cleared: bool = False):
     """The whole selection in one launch (tr.py:350-373, 424-449): scoring, soft vote,
     exact top-k, ascending order and index assembly, the scores never leaving LDS.
     Returns ``(sel, sel_pos, sel_len, votes, workspace)`` with the first three as
     from :func:`topk_ragged`; ``votes`` is ``[B, stride]`` fp32 when ``want_votes``
-    else ``None``.  ``workspace`` (uint8) may be passed back in to avoid allocating."""
+    else ``None``.  ``workspace`` (uint8) may be passed back in to avoid allocating;
+    with ``cleared`` the caller has run :func:`select_clear` on it since its last use
+    and only the selection kernel is launched."""
     c, cb = cfg.to_c(), _c_batch(cfg, bt)
     _need(qf, "qf", torch.bfloat16)
     _check_pool(cfg, k_pool, "k_pool")
@@ -263,6 +277,8 @@ def select(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
         _need(hit, "hit", torch.int32, 1)
     lib = _lib.load()
     nbytes = lib.ts_select_workspace_bytes(ctypes.byref(c), B, bt.max_seq_len)
+    if cleared and (workspace is None or workspace.numel() < nbytes):
+        raise ValueError("cleared=True needs the workspace that select_clear was run on")
     if workspace is None or workspace.numel() < nbytes:
         workspace = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=qf.device)
     sel = torch.empty((B, cfg.max_sel), dtype=torch.int32, device=qf.device)
@@ -272,7 +288,7 @@ def select(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
     if want_votes:
         votes = torch.empty((B, score_stride_for(bt.max_seq_len)), dtype=torch.float32,
                             device=qf.device)
-    _lib.check(lib.ts_select(
+    _lib.check((lib.ts_select_cleared if cleared else lib.ts_select)(
         ctypes.byref(c), ctypes.byref(cb), _p(qf), _p(k_pool), k_pool.shape[0], _p(hit),
         _c_cache(cache, cfg, B), _p(sel), _p(sel_pos), cfg.max_sel, _p(sel_len), _p(votes),
         votes.shape[1] if votes is not None else 0, _p(workspace), workspace.numel(), _stream()))
