@@ -53,8 +53,12 @@ struct ScoreArgs {
 // hundreds of workgroups adding to the same line serialise in memory.
 constexpr int kSelHistCopies = 16;
 constexpr int kSelHist0 = 0;                           // copies x 2048, top 11 key bits
-constexpr int kSelHist1 = kSelHistCopies * kTopkBins;  // 2048, next 11 bits inside bin t0
-constexpr int kSelHist2 = kSelHist1 + kTopkBins;       // 1024, last 10 bits inside (t0, t1)
+// Second level (next 11 bits inside bin t0), needed when the votes are nearly uniform
+// and t0 holds tens of thousands of candidates: that many adds to the 64 lines of a
+// single copy take 20 us, hence copies here as well.
+constexpr int kSelHist1Copies = 8;
+constexpr int kSelHist1 = kSelHistCopies * kTopkBins;             // copies x 2048
+constexpr int kSelHist2 = kSelHist1 + kSelHist1Copies * kTopkBins;  // 1024, last 10 bits inside (t0, t1)
 // Highest occupied bin of hist0, one word per copy, 128 bytes apart (hundreds of
 // read-modify-writes of one address, or one line, take microseconds).
 constexpr int kSelMaxBin = kSelHist2 + 1024;

@@ -707,15 +707,23 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       uint32_t done = 0;
       for (int base = 0; base < count; base += 256) {
         const uint32_t key = base + tid < count ? key_of(base + tid) : 0u;
-        done += wave_histogram_add(ctr + kSelHist1, base + tid < count && key_bin0(key) == t0,
-                                   key_bin1(key), lane);
+        done += wave_histogram_add(ctr + kSelHist1 + (blockIdx.x % kSelHist1Copies) * kTopkBins,
+                                   base + tid < count && key_bin0(key) == t0, key_bin1(key), lane);
       }
       await(done);
       grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
       {
         uint32_t h[kTopkBins / 256];
 #pragma unroll
-        for (int j = 0; j < kTopkBins / 256; ++j) h[j] = load_coherent(&ctr[kSelHist1 + tid + 256 * j]);
+        for (int j = 0; j < kTopkBins / 256; ++j) {
+          uint32_t part[kSelHist1Copies];
+#pragma unroll
+          for (int c = 0; c < kSelHist1Copies; ++c)
+            part[c] = load_coherent(&ctr[kSelHist1 + c * kTopkBins + tid + 256 * j]);
+          h[j] = 0u;
+#pragma unroll
+          for (int c = 0; c < kSelHist1Copies; ++c) h[j] += part[c];
+        }
 #pragma unroll
         for (int j = 0; j < kTopkBins / 256; ++j) lh[tid + 256 * j] = h[j];
       }
