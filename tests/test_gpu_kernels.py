@@ -374,6 +374,11 @@ def test_select_randomised(dev):
         g = torch.Generator(device=dev).manual_seed(seed)
         if mode == "narrow":
             wl.q.mul_(rnd.choice([0.02, 0.1]))
+        elif mode == "wide" and B > 1:
+            # a scale per request: the requests of one launch then need different numbers
+            # of histogram levels
+            scale = torch.tensor([rnd.choice([1.0, 0.02, 0.2, 0.0]) for _ in range(B)], device=dev)
+            wl.q.copy_((wl.q.view(B, -1).float() * scale.view(B, 1)).to(wl.q.dtype).view(wl.q.shape))
         elif mode == "zero":
             wl.q.zero_()
         elif mode in ("ties", "ties256"):
