@@ -71,13 +71,14 @@ constexpr int kQuadSwap2 = 0x4E;  // quad_perm [2,3,0,1]
 //     the keys stream in costs a quarter of the read bandwidth (DRAM read/write
 //     turnarounds).
 //   kScoreFused (the whole selection in one launch whose workgroups are all
-//     resident at once and meet six times): the scores never leave LDS.  Every
-//     workgroup publishes its per-head (max, sum exp); the (request, head) pairs
-//     are dealt out over the grid and merged; every workgroup turns its own scores
-//     into votes (tr.py:361); three histogram rounds (11 + 11 + 10 key bits) find
-//     the k-th largest vote exactly; the workgroups exchange their counts and
-//     each writes its selected positions, in ascending order, where they belong
-//     (tr.py:371-373, 433-449).
+//     resident at once and meet four to six times): the scores never leave LDS.
+//     Every workgroup publishes its per-head (max, sum exp); the (request, head)
+//     pairs are dealt out over the grid and merged; every workgroup turns its own
+//     scores into votes (tr.py:361); histogram rounds (11 + 11 + 10 key bits) narrow
+//     the k-th largest vote down until at most 256 candidates are left, which are
+//     listed and ranked by every workgroup together with the counts that tell it
+//     where its selected positions, in ascending order, belong (tr.py:371-373,
+//     433-449); masses of exact ties go through all three levels and a count round.
 constexpr int kScoreDirect = 0, kScoreTiled = 1, kScoreFused = 2;
 constexpr int kMaxHeads = 128;
 
@@ -121,7 +122,7 @@ constexpr uint32_t kSelectRounds = 6;  // rendezvous of the fused kernel
 // The workgroups that take part in the rendezvous of the fused kernel: all those of
 // the requests that select (neither dense nor served by the selection cache).  The
 // others write their fixed output and leave, so that a step in which every request
-// hits the cache costs a few microseconds instead of six empty rounds.
+// hits the cache costs a few microseconds instead of empty rounds.
 __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t* lds) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int B = gridDim.y, mine = blockIdx.y;
