@@ -223,6 +223,23 @@ int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_poo
                           int32_t max_sel_len, void* out, void* workspace,
                           size_t workspace_bytes, ts_stream_t stream);
 
+/* ts_sparse_decode_attn for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops and harnesses that forbid hipMalloc): same
+ * arguments, kernels and results, but the split-K partials and tickets live in a
+ * buffer built into the library (ts_attn_static_scratch_bytes() = 4 MiB of device
+ * memory per GPU the library runs on, held until the process ends) instead of a
+ * caller's workspace.  The call allocates and frees nothing.  TS_EWORKSPACE when
+ * batch x heads x splits needs more than the buffer holds (about 7900 partial rows
+ * of 520 bytes; with 32 query / 8 KV heads: every batch up to 251).  All calls on one GPU share the buffer:
+ * calls that overlap on one GPU (two streams, two threads) race and must be
+ * serialised by the caller; calls on one stream are ordered by the stream.
+ * No counterpart in the reference. */
+size_t ts_attn_static_scratch_bytes(void);
+int ts_sparse_decode_attn_static(const ts_config* cfg, const void* q, const void* k_pool,
+                                 const void* v_pool, int64_t pool_rows, const int32_t* sel,
+                                 int64_t sel_stride, const int32_t* sel_len, int32_t batch,
+                                 int32_t max_sel_len, void* out, ts_stream_t stream);
+
 /* KV store + table append (patched_radix_attention_store_kv_cache tr.py:844-854,
  * add_k_cache tr.py:332-336) for page_size 1: k_pool[loc[b]] = k[b],
  * v_pool[loc[b]] = v[b], table[b][seq_lens[b]] = loc[b], seq_lens[b] += 1. */

@@ -114,6 +114,17 @@ def test_null_and_range_errors_need_no_gpu(lib):
     assert "workspace" in err(lib)
 
 
+def test_static_scratch_entry_point_rejects_what_does_not_fit(lib):
+    assert lib.ts_attn_static_scratch_bytes() == 4 << 20
+    one = ctypes.c_void_p(0x1000)  # never dereferenced: the size check fails first
+    wide = cfg(num_heads=64, num_kv_heads=8, top_k=4096)
+    assert lib.ts_sparse_decode_attn_static(ctypes.byref(wide), one, one, one, 10, one, 4736, one,
+                                            63, 4736, one, None) == _lib.TS_EWORKSPACE
+    assert "scratch" in err(lib)
+    assert lib.ts_sparse_decode_attn_static(ctypes.byref(cfg()), one, one, one, 10, None, 2688, one,
+                                            1, 2688, one, None) == _lib.TS_EINVAL
+
+
 def test_python_layer_refuses_cpu_tensors(lib):
     c = ops.LayerConfig(num_heads=4, num_kv_heads=2, n_init=1, n_local=2, top_k=4)
     x = torch.zeros(1, 4, 128, dtype=torch.bfloat16)

@@ -73,6 +73,9 @@ SIGNATURES = {
     "ts_attn_workspace_bytes": (_size, [_CFG, _i32, _i32]),
     "ts_sparse_decode_attn": (_i32, [_CFG, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
                                      _ptr, _ptr, _size, _ptr]),
+    "ts_attn_static_scratch_bytes": (_size, []),
+    "ts_sparse_decode_attn_static": (_i32, [_CFG, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
+                                            _ptr, _ptr]),
     "ts_kv_store": (_i32, [_CFG, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
                            _ptr]),
     "ts_qkv_store": (_i32, [_CFG, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr,

@@ -14,6 +14,8 @@
 // its (request, KV head) merges the splits and writes the bf16 output.
 #include <math.h>
 
+#include <mutex>
+
 #include "ts_common.h"
 
 namespace ts {
@@ -436,6 +438,38 @@ int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const v
   return check_launch("attn_kernel");
 }
 
+// Scratch of ts_sparse_decode_attn_static: the split-K partials and tickets of one
+// launch, held by every device the library runs on until the process ends.
+constexpr size_t kStaticScratchBytes = 4u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device, looked up once per device (each
+// device holds its own copy at its own address); NULL with the error set on failure.
+constexpr int kMaxDevices = 64;
+static void* static_scratch() {
+  static std::mutex mu;
+  static void* ptr_of_device[kMaxDevices] = {};
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess || device < 0 || device >= kMaxDevices) {
+    (void)hipGetLastError();
+    fail(TS_EHIP, "ts_sparse_decode_attn_static: no current device (%s)", hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptr_of_device[device] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      fail(TS_EHIP, "ts_sparse_decode_attn_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    ptr_of_device[device] = ptr;
+  }
+  return ptr_of_device[device];
+}
+
 }  // namespace ts
 
 using namespace ts;
@@ -466,6 +500,34 @@ int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_poo
              "ts_sparse_decode_attn: workspace %zu bytes < required %zu", workspace_bytes, need);
   return launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, batch, max_sel_len,
                      out, workspace, /*tickets_clear=*/false, (hipStream_t)stream);
+}
+
+size_t ts_attn_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int ts_sparse_decode_attn_static(const ts_config* cfg, const void* q, const void* k_pool,
+                                 const void* v_pool, int64_t pool_rows, const int32_t* sel,
+                                 int64_t sel_stride, const int32_t* sel_len, int32_t batch,
+                                 int32_t max_sel_len, void* out, ts_stream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_REQUIRE(q && k_pool && v_pool && sel && sel_len && out, TS_EINVAL,
+             "ts_sparse_decode_attn_static: NULL tensor argument");
+  TS_REQUIRE(batch >= 1 && batch <= 65535, TS_EINVAL, "batch %d out of range", batch);
+  TS_REQUIRE(max_sel_len >= 1, TS_EINVAL, "max_sel_len %d < 1", max_sel_len);
+  TS_REQUIRE(sel_stride >= max_sel_len || batch == 1, TS_EWORKSPACE,
+             "sel_stride %lld < max_sel_len %d", (long long)sel_stride, max_sel_len);
+  TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
+             (long long)pool_rows);
+  const size_t need = attn_workspace(cfg, batch, max_sel_len).total;
+  TS_REQUIRE(need <= kStaticScratchBytes, TS_EWORKSPACE,
+             "ts_sparse_decode_attn_static: batch %d x %d heads x %d selected needs %zu bytes of "
+             "scratch, the built-in buffer holds %zu; use ts_sparse_decode_attn with a workspace",
+             batch, cfg->num_heads, max_sel_len, need, kStaticScratchBytes);
+  void* ptr = static_scratch();
+  if (ptr == nullptr) return TS_EHIP;
+  // The tickets are cleared by a fill kernel on the caller's stream (the previous call
+  // may have been interrupted), so the call can be captured into a HIP graph.
+  return launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, batch, max_sel_len,
+                     out, ptr, /*tickets_clear=*/false, (hipStream_t)stream);
 }
 
 }  // extern "C"

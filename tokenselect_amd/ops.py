@@ -645,3 +645,30 @@ class PrefillChunk:
             _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
             self.workspace.numel(), _stream()))
         return out, self.sel, self.sel_pos, self.sel_len
+
+
+def sparse_decode_attention_static(cfg: LayerConfig, q: torch.Tensor, k_pool: torch.Tensor,
+                                   v_pool: torch.Tensor, sel: torch.Tensor, sel_len: torch.Tensor,
+                                   out: torch.Tensor, max_sel_len: Optional[int] = None) -> torch.Tensor:
+    """:func:`sparse_decode_attention` through ``ts_sparse_decode_attn_static``: the
+    split-K partials live in a buffer built into the library, and neither this wrapper
+    nor the library allocates (``out`` [B, H*D] bf16 is the caller's)."""
+    c = cfg.to_c()
+    _need(q, "q", torch.bfloat16)
+    _check_pool(cfg, k_pool, "k_pool")
+    _check_pool(cfg, v_pool, "v_pool")
+    _need(sel, "sel", torch.int32, 2)
+    _need(sel_len, "sel_len", torch.int32, 1)
+    _need(out, "out", torch.bfloat16)
+    B = sel.shape[0]
+    if k_pool.shape != v_pool.shape:
+        raise ValueError("k_pool and v_pool must have the same shape")
+    if q.numel() != B * cfg.num_heads * cfg.head_dim or sel_len.shape[0] != B or out.numel() != q.numel():
+        raise ValueError("q / sel_len / out do not match the batch of sel")
+    max_sel_len = sel.shape[1] if max_sel_len is None else int(max_sel_len)
+    if max_sel_len > sel.shape[1]:
+        raise ValueError("max_sel_len exceeds the width of sel")
+    _lib.check(_lib.load().ts_sparse_decode_attn_static(
+        ctypes.byref(c), _p(q), _p(k_pool), _p(v_pool), k_pool.shape[0], _p(sel), sel.stride(0),
+        _p(sel_len), B, max_sel_len, _p(out), _stream()))
+    return out
