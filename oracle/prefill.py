@@ -88,11 +88,13 @@ def prefill(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, k_pool: t
             num_heads: int, head_dim: int, n_init: int, n_local: int, k: int, rope_base: float,
             rope_scale: float, sm_scale: float, logit_cap: float = 0.0,
             rope_mode: str = "ROPE_LLAMA", chunk: int = PREFILL_CHUNK_SIZE,
-            details: Optional[List[dict]] = None):
+            details: Optional[List[dict]] = None,
+            qf_overrides: Optional[List[torch.Tensor]] = None):
     """The whole extend forward of one layer for one request: ``q`` [T, H*D],
     ``k_new`` / ``v_new`` [T, Hkv, D] written to ``new_slots`` [T] and appended to
     ``tab`` (which must have room for ``seq_len + T`` entries) chunk by chunk.
-    Pools and ``tab`` are modified in place.  Returns ``out`` [T, H*D]."""
+    Pools and ``tab`` are modified in place.  ``qf_overrides[i]`` replaces the
+    fingerprint of chunk i (see ``prefill_chunk``).  Returns ``out`` [T, H*D]."""
     total = q.shape[0]
     outs = []
     for start in range(0, total, chunk):
@@ -105,7 +107,8 @@ def prefill(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, k_pool: t
         d = {} if details is not None else None
         _, o = prefill_chunk(q[start:end], k_pool, v_pool, tab, seq_len, num_heads, head_dim,
                              n_init, n_local, k, rope_base, rope_scale, sm_scale, logit_cap,
-                             rope_mode, detail=d)
+                             rope_mode, detail=d,
+                             qf_override=None if qf_overrides is None else qf_overrides[start // chunk])
         if details is not None:
             details.append(d)
         outs.append(o)

@@ -26,20 +26,16 @@ import torch
 THRESHOLD = float(torch.tensor(0.9, dtype=torch.bfloat16))  # 0.8984375
 
 
-def cosine(a: torch.Tensor, b: torch.Tensor, mode: str = "fp32") -> float:
-    if mode == "ref_rounding":
-        return float(torch.cosine_similarity(a, b, dim=0))
+def cosine(a: torch.Tensor, b: torch.Tensor) -> float:
     a64, b64 = a.double(), b.double()
     return float((a64 @ b64) / max(float(a64.norm() * b64.norm()), 1e-8))
 
 
 class SelectionCache:
-    def __init__(self, threshold: float = THRESHOLD, anchor: str = "last_miss",
-                 mode: str = "fp32"):
+    def __init__(self, threshold: float = THRESHOLD, anchor: str = "last_miss"):
         assert anchor in ("last_miss", "previous")
         self.threshold = threshold
         self.anchor = anchor
-        self.mode = mode
         self.q_cached = None
         self.top_cached = None
         self.skip_count = 0
@@ -47,7 +43,7 @@ class SelectionCache:
 
     def step(self, qf: torch.Tensor, select: Callable[[], torch.Tensor]):
         """Returns ``(top_pos, hit)``; ``select()`` yields positions incl. ``+n_init``."""
-        miss = self.q_cached is None or cosine(self.q_cached, qf, self.mode) < self.threshold
+        miss = self.q_cached is None or cosine(self.q_cached, qf) < self.threshold
         if miss:
             top = select()
             self.top_cached = top.clone()

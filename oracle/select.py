@@ -6,13 +6,10 @@ sum tr.py:361, max-pool smoothing tr.py:366-369, top-k + sort tr.py:371-373,
 the short-context fallback and index assembly tr.py:375-449, and the
 logical->physical token table tr.py:324-336.
 
-Two numeric modes:
-
-``fp32``          canonical for parity: exact bf16 products accumulated in fp32,
-                  fp32 scores, fp32 softmax and vote.
-``ref_rounding``  restates the rounding chain of the reference as released:
-                  each product rounded to bf16, fp32 sum, bf16 scores
-                  (tr.py:345-347), bf16 softmax and bf16 head sum (tr.py:361).
+Numerics: exact bf16 products accumulated in fp32, fp32 scores, fp32 softmax and
+vote.  (The reference as released rounds the scores, the softmax and the head sum to
+bf16, tr.py:345-347, 361, in an order its Triton version fixes; that chain is not
+restated here.)
 """
 
 from typing import Optional
@@ -35,13 +32,13 @@ def expand_page_table(page_table: torch.Tensor, seq_len: int, page_size: int) ->
 
 
 def score(qf: torch.Tensor, k_pool: torch.Tensor, cand_slots: torch.Tensor,
-          mode: str = "fp32", head_map: str = "mod") -> torch.Tensor:
+          head_map: str = "mod") -> torch.Tensor:
     """``scores[h, t] = sum_d qf[h, d] * K[cand[t], kv(h), d]`` with no scaling
     (tr.py:216-224).  ``kv(h) = h % Hkv`` in the reference (tr.py:202);
     ``head_map="div"`` gives the conventional ``h // (H/Hkv)`` for comparison.
 
     ``qf`` is ``[H, D]`` bf16, ``k_pool`` ``[P, Hkv, D]`` bf16, ``cand_slots``
-    ``[n]`` integer.  Returns ``[H, n]`` fp32 (bf16 in ``ref_rounding`` mode).
+    ``[n]`` integer.  Returns ``[H, n]`` fp32.
     """
     num_heads, _ = qf.shape
     num_kv = k_pool.shape[1]
@@ -53,21 +50,13 @@ def score(qf: torch.Tensor, k_pool: torch.Tensor, cand_slots: torch.Tensor,
     for lo in range(0, n, _CHUNK):
         rows = k_pool[slots[lo:lo + _CHUNK]]            # [c, Hkv, D]
         per_head = rows[:, kv_of_head]                   # [c, H, D]
-        if mode == "fp32":
-            out[:, lo:lo + _CHUNK] = torch.einsum("hd,chd->hc", qf.float(), per_head.float())
-        elif mode == "ref_rounding":
-            prod = (qf[None] * per_head)                 # bf16 x bf16 -> bf16
-            out[:, lo:lo + _CHUNK] = prod.float().sum(-1).transpose(0, 1)
-        else:
-            raise ValueError(mode)
-    if mode == "ref_rounding":
-        return out.to(torch.bfloat16)
+        out[:, lo:lo + _CHUNK] = torch.einsum("hd,chd->hc", qf.float(), per_head.float())
     return out
 
 
 def vote(scores: torch.Tensor) -> torch.Tensor:
     """Per-head softmax over the candidates, summed over heads (tr.py:361).
-    Keeps the dtype of ``scores`` (fp32 canonical, bf16 in ``ref_rounding``)."""
+    fp32 in, fp32 out."""
     return torch.softmax(scores, dim=-1).sum(dim=0)
 
 
@@ -89,11 +78,11 @@ def topk_sorted(votes: torch.Tensor, k: int) -> torch.Tensor:
 
 
 def get_topk_tokens(qf: torch.Tensor, k_pool: torch.Tensor, k: int,
-                    cand_slots: torch.Tensor, head_dim: int, mode: str = "fp32",
+                    cand_slots: torch.Tensor, head_dim: int,
                     kernel_size: int = -1, return_all: bool = False):
     """tr.py:338-373 for one request: score -> vote -> [pool] -> top-k -> sort.
     ``qf`` is the flat ``[H*D]`` fingerprint."""
-    s = score(qf.view(-1, head_dim), k_pool, cand_slots, mode)
+    s = score(qf.view(-1, head_dim), k_pool, cand_slots)
     c = max_pool(vote(s), kernel_size)
     top = topk_sorted(c, k)
     if return_all:
@@ -119,7 +108,7 @@ def is_dense(seq_len: int, n_init: int, n_local: int, k: int) -> bool:
 def retrieval_indices(q: torch.Tensor, k_pool: torch.Tensor, tab: torch.Tensor,
                       seq_len: int, num_heads: int, head_dim: int, n_init: int,
                       n_local: int, k: int, rope_base: float, rope_scale=1.0,
-                      mode: str = "fp32", kernel_size: int = -1,
+                      kernel_size: int = -1,
                       detail: Optional[dict] = None,
                       qf_override: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """tr.py:375-449 for one request with the selection cache disabled, as
@@ -134,7 +123,7 @@ def retrieval_indices(q: torch.Tensor, k_pool: torch.Tensor, tab: torch.Tensor,
     if qf_override is not None:
         qf = qf_override.reshape(-1).to(qf.dtype)
     cand = tab[n_init:seq_len - n_local]
-    top, s, c = get_topk_tokens(qf, k_pool, k, cand, head_dim, mode, kernel_size,
+    top, s, c = get_topk_tokens(qf, k_pool, k, cand, head_dim, kernel_size,
                                 return_all=True)
     top = top + n_init
     if detail is not None:

@@ -94,10 +94,11 @@ def test_oracle_reproduces_the_prefill_fixture():
 
 @pytest.mark.gpu
 def test_hip_prefill_matches_the_fixture(dev):
-    """Chunk by chunk: device fingerprint within one bf16 ulp of the fixture's, the
-    selection as in the fixture wherever the fingerprints agree bit for bit, and the
-    chunk output within tolerance wherever the selections agree."""
+    """Chunk by chunk: device fingerprint within one bf16 ulp of the fixture's; every
+    chunk's selection and output against the oracle following the device's fingerprint;
+    and, wherever the fingerprints agree bit for bit, against the fixture itself."""
     from tokenselect_amd import ops
+    from helpers import assert_index_sets_match
     f = load_prefill()
     H, D, L0, T, chunk = f["H"], f["D"], f["L0"], f["T"], f["chunk"]
     cfg = ops.LayerConfig(num_heads=H, num_kv_heads=f["HKV"], n_init=f["n_init"], n_local=f["n_local"],
@@ -107,25 +108,40 @@ def test_hip_prefill_matches_the_fixture(dev):
     table[0, :L0] = f["table"].to(dev)
     seq = torch.tensor([L0], dtype=torch.int32, device=dev)
     layer = ops.PrefillChunk(cfg, L0 + T, dev, max_rows=chunk)
-    q, L, compared = f["q"].to(dev), L0, 0
+    kc, vc = f["k_pool"].clone(), f["v_pool"].clone()
+    tab_cpu = torch.zeros(L0 + T, dtype=torch.int32)
+    tab_cpu[:L0] = f["table"]
+    q, L = f["q"].to(dev), L0
     for i, start in enumerate(range(0, T, chunk)):
         end = min(start + chunk, T)
+        m = end - start
         ops.kv_store_chunk(cfg, f["k_new"][start:end].to(dev), f["v_new"][start:end].to(dev),
                            f["new_slots"][start:end].to(dev).contiguous(), k_pool, v_pool, table[0], seq)
-        L += end - start
+        L += m
         out, sel, sel_pos, sel_len = layer(q[start:end].contiguous(), k_pool, v_pool,
                                            ops.Batch(seq, table, L))
-        qf = ops.fingerprint(cfg, q[start:end].view(end - start, H, D).contiguous(), layer.cos, layer.sin)
+        qf = ops.fingerprint(cfg, q[start:end].view(m, H, D).contiguous(), layer.cos, layer.sin)
         torch.cuda.synchronize()
         want_qf = torch.from_numpy(f["z"][f"qf_{i}"].copy()).view(torch.bfloat16).float()
         got_qf = qf.cpu().float().reshape(-1)
         assert bool(((got_qf - want_qf).abs() <= want_qf.abs() * 2.0 ** -7 + 1e-30).all())
         S = int(sel_len[0])
         assert S == f["n_init"] + f["top_k"] + f["n_local"]
-        if torch.equal(got_qf, want_qf):
-            mid = sel_pos[0, f["n_init"]:f["n_init"] + f["top_k"]].cpu()
-            if mid.tolist() == f["z"][f"top_pos_{i}"].tolist():
-                want = f["out"][start:end].float()
-                assert (out.cpu().float() - want).abs().max().item() <= 2e-2
-                compared += 1
-    assert compared >= 1
+        # the oracle on the same pools, with the device's fingerprint
+        loc = f["new_slots"][start:end].long()
+        kc[loc], vc[loc] = f["k_new"][start:end], f["v_new"][start:end]
+        tab_cpu[L - m:L] = f["new_slots"][start:end].to(torch.int32)
+        d = {}
+        ref_slots, ref_out = oracle.prefill.prefill_chunk(
+            f["q"][start:end], kc, vc, tab_cpu, L, H, D, f["n_init"], f["n_local"], f["top_k"],
+            f["rope_base"], 1.0, D ** -0.5, detail=d, qf_override=qf.cpu())
+        mid = sel_pos[0, f["n_init"]:f["n_init"] + f["top_k"]].cpu()
+        assert_index_sets_match(mid, d["top_pos"], d["votes"], f["n_init"], f"fixture chunk {i}")
+        got_slots = sel[0, :S].cpu()
+        if not torch.equal(got_slots, ref_slots):               # a tie went the other way
+            ref_out = oracle.prefill.sparse_prefill_attention(
+                f["q"][start:end].view(m, H, D), kc, vc, got_slots, D ** -0.5,
+                f["rope_base"]).reshape(m, -1)
+        assert (out.cpu().float() - ref_out.float()).abs().max().item() <= 2e-2, f"chunk {i}"
+        if torch.equal(got_qf, want_qf) and mid.tolist() == f["z"][f"top_pos_{i}"].tolist():
+            assert (out.cpu().float() - f["out"][start:end].float()).abs().max().item() <= 2e-2

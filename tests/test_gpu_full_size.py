@@ -11,7 +11,7 @@ import torch
 
 import oracle
 from tokenselect_amd import ops, workloads
-from helpers import assert_index_sets_match, say
+from helpers import assert_attention_close, assert_index_sets_match, say
 
 pytestmark = pytest.mark.gpu
 
@@ -87,9 +87,7 @@ def _check_against_oracle(wl, layer_out, requests, tag):
         if details[i]:
             assert_index_sets_match(sel_pos[b, c.n_init:S - c.n_local].cpu(), details[i]["top_pos"],
                                     details[i]["votes"], c.n_init, f"{tag} b={b}")
-        if torch.equal(sel[b, :S].cpu(), ref_sel[i]):
-            err = (out[b].cpu().float() - ref_out[i].float()).abs().max().item()
-            assert err <= 2e-2, f"{tag} b={b}: attention error {err}"
+        assert_attention_close(wl, b, out[b], sel[b, :S], ref_sel[i], ref_out[i], f"{tag} b={b}")
 
 
 def _run(wl, dev):
@@ -183,6 +181,8 @@ def test_selection_cache_trace_config(dev):
     cache = ops.SelectionCache.allocate(c, B, dev)
     layer = ops.DecodeLayer(c, B, L0 + steps, dev)
     previous_mid, hits_seen, last_miss = None, 0, None
+    cos_t, sin_t = ops.scoring_cos_sin(c.head_dim, c.rope_theta, c.rope_scale, c.n_local, dev)
+    anchors = [None] * B          # the oracle's state machine: fingerprint of the last miss
     for t in range(steps):
         before = cache.counters.clone()
         ops.kv_store(c, k_new[t], v_new[t], free[t], wl.k_pool, wl.v_pool, table, seq)
@@ -197,6 +197,19 @@ def test_selection_cache_trace_config(dev):
                            torch.arange(L - c.n_local, L, dtype=torch.int32).repeat(B, 1))
         hit = (cache.counters[:, 0] - before[:, 0]).tolist()
         assert (cache.counters[:, 1] - before[:, 1]).tolist() == [1] * B
+        # every step's decision against the oracle's cosine rule on the same fingerprints
+        qf = ops.rope_apply(qs[t].view(B, c.num_heads, c.head_dim), cos_t, sin_t, None).cpu()
+        for b in range(B):
+            fp = qf[b].reshape(-1)
+            if anchors[b] is None:
+                assert not hit[b], f"step {t} b={b}: the first lookup must miss"
+            else:
+                cos = oracle.selcache.cosine(anchors[b], fp)
+                want = cos >= oracle.selcache.THRESHOLD
+                if want != bool(hit[b]):            # only a cosine on the threshold may differ
+                    assert abs(cos - oracle.selcache.THRESHOLD) < 1e-5, (t, b, cos, hit[b])
+            if not hit[b]:
+                anchors[b] = fp.clone()
         for b in range(B):
             if hit[b]:
                 hits_seen += 1

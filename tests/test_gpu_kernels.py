@@ -8,7 +8,8 @@ import torch
 
 import oracle
 from tokenselect_amd import ops, workloads
-from helpers import assert_index_sets_match, assert_scores_close, cpu_tabs, oracle_layer, say
+from helpers import (assert_attention_close, assert_index_sets_match, assert_scores_close, cpu_tabs,
+                     oracle_layer, say)
 
 pytestmark = pytest.mark.gpu
 
@@ -511,9 +512,7 @@ def check_layer(wl, dev, tag):
             c = wl.cfg
             assert_index_sets_match(sel_pos[b, c.n_init:S - c.n_local].cpu(), details[b]["top_pos"],
                                     details[b]["votes"], c.n_init, f"{tag} top-k b={b}")
-        if torch.equal(sel[b, :S].cpu(), ref_sel[b]):
-            err = (out[b].cpu().float() - ref_out[b].float()).abs().max().item()
-            assert err <= 2e-2, f"{tag} out b={b}: {err}"
+        assert_attention_close(wl, b, out[b], sel[b, :S], ref_sel[b], ref_out[b], f"{tag} b={b}")
     return sel_pos, sel_len
 
 

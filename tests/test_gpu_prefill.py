@@ -158,9 +158,12 @@ def test_prefill_chunks(dev, shape, fused):
                                     f"chunk at {start}")
             assert pos[-m:].tolist() == list(range(L - m, L))     # the chunk is the tail
             assert torch.equal(sel[0, :S].cpu(), tab_cpu[pos.long()])
-            if torch.equal(sel[0, :S].cpu(), ref_slots):
-                err = (out.cpu().float() - ref_out.float()).abs().max().item()
-                assert err <= 2e-2, (start, err)
+            if not torch.equal(sel[0, :S].cpu(), ref_slots):   # a tie went the other way
+                ref_out = oracle.prefill.sparse_prefill_attention(
+                    q[start:end].cpu().view(m, c.num_heads, 128), kc, vc, sel[0, :S].cpu(), _sm(c),
+                    c.rope_theta, c.rope_scale).reshape(m, -1)
+            err = (out.cpu().float() - ref_out.float()).abs().max().item()
+            assert err <= 2e-2, (start, err)
     finally:
         ops.set_fused_select(previous)
 

@@ -131,16 +131,6 @@ def test_score_follows_the_table_not_the_pool_order():
     assert torch.equal(select.score(qf, shuffled_pool, perm[:40].int()), base)
 
 
-def test_ref_rounding_mode_is_bf16_and_close():
-    qf, k_pool = rnd(4, 128, seed=12), rnd(50, 2, 128, seed=13)
-    cand = torch.arange(50, dtype=torch.int32)
-    s32 = select.score(qf, k_pool, cand)
-    s16 = select.score(qf, k_pool, cand, mode="ref_rounding")
-    assert s16.dtype == torch.bfloat16
-    assert (s16.float() - s32).abs().max() < 0.02 * s32.abs().max()
-    assert select.vote(s16).dtype == torch.bfloat16
-
-
 # ------------------------------------------------------------- vote / pool
 def test_vote_mass_shift_invariance_and_single_head():
     s = rnd(6, 300, seed=14, dtype=torch.float32) * 5
