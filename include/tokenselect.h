@@ -6,8 +6,10 @@
  * device pointers unless a parameter says "host".  bf16 tensors are passed as
  * `const void*` (16-bit brain floats, row-major, innermost dimension
  * contiguous).  Launches are asynchronous on the given HIP stream; the library
- * never synchronises, never allocates device memory and keeps no mutable
- * global state, so calls are re-entrant across streams.
+ * never synchronises and never allocates device memory.  Its only mutable
+ * process-wide state is the ts_set_fused_select() switch (and the built-in
+ * scratch buffer of ts_sparse_decode_attn_static); everything else lives in the
+ * caller's buffers, so calls are re-entrant across streams.
  *
  * Return value: TS_OK or a negative TS_E* code; ts_last_error() then holds a
  * thread-local message.  Arguments are validated on the host before anything
@@ -77,6 +79,12 @@ typedef struct ts_batch {
                                of logical token t: table[t/ps]*ps + t%ps       */
   int64_t table_stride;     /* elements between rows                           */
   const int32_t* k_per_req; /* [B] per-request k (<= top_k), or NULL = top_k   */
+  uint32_t* fault;          /* NULL, or one 32-bit word the device can write
+                               (device memory, or pinned host memory that the
+                               device maps, which the host may read at any time
+                               without synchronising): set to 1 when a grid-wide
+                               wait of a ts_select launch gave up, never cleared
+                               by the library                                   */
 } ts_batch;
 
 /* Optional selection-cache state for one layer (tr.py:301-322, 394-421).
@@ -177,8 +185,13 @@ int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
  * that all its workgroups are resident together; that holds while nothing else
  * runs on the device beside the caller's stream (a cooperative launch would
  * enforce it, at about 25 us per call).  Every grid-wide wait is bounded (2 s);
- * if one ever gives up, the first 32-bit word of the last 65 * 4096 bytes of
- * the workspace is set to 1 and the outputs of that launch are not valid.
+ * once one has given up the others return at once, the kernel drains, and the
+ * launch reports it without any host synchronisation: sel_len[b] = -1 for
+ * every request that was selecting (the other outputs of those requests are
+ * not valid; ts_sparse_decode_attn treats a negative length as an empty list),
+ * *bt->fault = 1 when bt->fault is given, and the first 32-bit word of the
+ * last 65 * 4096 bytes of the workspace is 1 until the next clearing.  A
+ * caller that sees it reruns the step with the separate kernels.
  * No counterpart in the reference, which materialises every intermediate. */
 int ts_select_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
 size_t ts_select_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
@@ -200,6 +213,19 @@ int ts_select_cleared(const ts_config* cfg, const ts_batch* bt, const void* qf, 
                       int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
                       int64_t vote_stride, void* workspace, size_t workspace_bytes,
                       ts_stream_t stream);
+
+/* ts_select_cleared with an explicit bound for the grid-wide waits, in ticks of
+ * the device's 100 MHz clock (ts_select uses 200 000 000 = 2 s), and a number of
+ * workgroups that are counted as members of the rendezvous but never arrive
+ * (0 in production): with absent_workgroups > 0 every wait gives up after
+ * wait_ticks, which is how the give-up path is tested without hanging a GPU.
+ * No counterpart in the reference. */
+int ts_select_cleared_bounded(const ts_config* cfg, const ts_batch* bt, const void* qf,
+                              const void* k_pool, int64_t pool_rows, const int32_t* hit,
+                              const ts_selcache* cache, int32_t* sel, int32_t* sel_pos,
+                              int64_t sel_stride, int32_t* sel_len, float* votes,
+                              int64_t vote_stride, void* workspace, size_t workspace_bytes,
+                              uint64_t wait_ticks, int32_t absent_workgroups, ts_stream_t stream);
 
 /* Selection-cache decision (tr.py:394-401, 416-421) for one layer, no host
  * sync: hit[b] = cache_len[b] > 0 && cos(q_cache[b], qf[b]) >= threshold; on a

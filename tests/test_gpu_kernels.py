@@ -226,6 +226,57 @@ def test_select_with_all_votes_equal(dev, fused_select):
     assert start.elapsed_time(end) < 1.0, "the selection serialised on a single counter"
 
 
+def test_fused_select_reports_a_wait_that_gave_up(dev):
+    """The give-up path, forced from the host so that every kernel still exits normally: one
+    team member that never arrives and a 20 us bound.  Every wait runs into the bound, the
+    kernel drains, and the launch says so without a synchronisation of its own: sel_len = -1
+    for the selecting requests, the caller's word, the word in the workspace.  The next
+    launch on the same workspace is correct."""
+    import time
+    lens, ks = [3000, 40, 1531], [64, 64, 100]
+    say(f"fused select, forced give-up lens={lens}")
+    wl = small(dev, SHAPES[0], seed=77, lens=lens, ks=ks, page=16, top_k=100)
+    c = wl.cfg
+    qf = fingerprint(wl, dev)
+    word = ops.fault_word()
+    bt = ops.Batch(wl.batch.seq_lens, wl.batch.table, wl.batch.max_seq_len, wl.batch.k_per_req, word)
+    space = ops.select_workspace(c, bt, dev)
+    torch.cuda.synchronize()
+    t0 = time.time()
+    sel, sel_pos, sel_len, _, _ = ops.select(c, bt, qf, wl.k_pool, workspace=space, wait_ticks=2000,
+                                             absent_workgroups=1)
+    torch.cuda.synchronize()
+    assert time.time() - t0 < 1.0, "a wait that gave up must not be waited for again"
+    assert sel_len.tolist() == [-1, 40, -1]          # the dense request needs no rendezvous
+    assert torch.equal(sel[1, :40].cpu(), cpu_tabs(wl)[1][:40])
+    assert int(word[0]) == 1 and ops.select_fault(c, bt, space)
+    with pytest.raises(ops.SelectionGaveUp):
+        ops.raise_if_gave_up(word)
+    # an attention over the reported lengths reads nothing of the invalid lists
+    out = ops.sparse_decode_attention(c, wl.q, wl.k_pool, wl.v_pool, sel, sel_len)
+    torch.cuda.synchronize()
+    assert out.shape[0] == 3
+    # the same workspace, cleared by the next call: the selection of the separate kernels
+    word.zero_()
+    votes_sep, _ = ops.vote(c, bt, *ops.score(c, bt, qf, wl.k_pool))
+    sel_sep, pos_sep, len_sep = ops.topk_ragged(c, bt, votes_sep)
+    sel, sel_pos, sel_len, _, _ = ops.select(c, bt, qf, wl.k_pool, workspace=space)
+    torch.cuda.synchronize()
+    assert int(word[0]) == 0 and not ops.select_fault(c, bt, space)
+    assert torch.equal(sel_len, len_sep)
+    for b in range(3):
+        S = int(sel_len[b])
+        assert torch.equal(sel[b, :S], sel_sep[b, :S]) and torch.equal(sel_pos[b, :S], pos_sep[b, :S])
+    # the layer object refuses to go on once its word is set
+    layer = ops.DecodeLayer(c, 3, max(lens), dev)
+    layer(wl.q, wl.k_pool, wl.v_pool, wl.batch)
+    torch.cuda.synchronize()
+    layer.check()
+    layer.fault[0] = 1
+    with pytest.raises(ops.SelectionGaveUp):
+        layer(wl.q, wl.k_pool, wl.v_pool, wl.batch)
+
+
 def test_fused_select_rejects_unsupported(dev):
     say("fused select: pool_kernel above 256 -> TS_ESHAPE")
     wl = small(dev, SHAPES[0], seed=3, lens=[2000], ks=[64], pool_kernel=300)

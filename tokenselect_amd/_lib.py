@@ -35,7 +35,7 @@ class TsConfig(ctypes.Structure):
 class TsBatch(ctypes.Structure):
     _fields_ = [
         ("batch", _i32), ("max_seq_len", _i32), ("seq_lens", _ptr), ("table", _ptr),
-        ("table_stride", _i64), ("k_per_req", _ptr),
+        ("table_stride", _i64), ("k_per_req", _ptr), ("fault", _ptr),
     ]
 
 
@@ -68,6 +68,8 @@ SIGNATURES = {
                          _ptr, _size, _ptr]),
     "ts_select_cleared": (_i32, [_CFG, _BT, _ptr, _ptr, _i64, _ptr, _SC, _ptr, _ptr, _i64, _ptr, _ptr, _i64,
                          _ptr, _size, _ptr]),
+    "ts_select_cleared_bounded": (_i32, [_CFG, _BT, _ptr, _ptr, _i64, _ptr, _SC, _ptr, _ptr, _i64, _ptr,
+                                         _ptr, _i64, _ptr, _size, ctypes.c_uint64, _i32, _ptr]),
     "ts_select_clear": (_i32, [_CFG, _BT, _ptr, _size, _ptr]),
     "ts_selcache_step": (_i32, [_CFG, _BT, _ptr, _SC, _ptr, _ptr]),
     "ts_attn_workspace_bytes": (_size, [_CFG, _i32, _i32]),

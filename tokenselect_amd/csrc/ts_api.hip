@@ -73,14 +73,9 @@ int score_tokens_per_block(int64_t total_candidates, int num_heads) {
   // Two workgroups per CU are resident (register budget), so aim for 512
   // workgroups on 256 CUs, in 64-row steps (every wave on whole 16-row tiles).  A
   // workgroup stages its fp32 scores in LDS, tokens * heads * 4 bytes <= 64 KB.
-  static const int forced = [] {
-    const char* e = getenv("TS_SCORE_TOKENS_PER_BLOCK");  // tuning override, multiple of 64
-    const int v = e ? atoi(e) : 0;
-    return (v >= 64 && v <= 8192) ? v / 64 * 64 : 0;
-  }();
   int64_t cap = (16384 / (num_heads > 0 ? num_heads : 1)) / 64 * 64;
   if (cap < 64) cap = 64;
-  int64_t per = forced ? forced : ceil_div(ceil_div(total_candidates, 512), 64) * 64;
+  int64_t per = ceil_div(ceil_div(total_candidates, 512), 64) * 64;
   if (per < 64) per = 64;
   if (per > cap) per = cap;
   return (int)per;

@@ -71,9 +71,13 @@ __device__ __forceinline__ void grid_poll(uint32_t* sync, uint32_t round, uint64
   const uint32_t* flag = &sync[(size_t)(index % kSyncSlots + 1) * kSyncSlotWords];
   const uint64_t t0 = wall_clock64();
   for (uint32_t polls = 1; load_coherent(flag) < round; ++polls) {
-    if ((polls & 255u) == 0 && wall_clock64() - t0 > ticks) {
-      __hip_atomic_store(&sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      break;
+    if ((polls & 15u) == 0) {
+      // Some workgroup has given up already: the launch is lost, do not wait again.
+      if (load_coherent(&sync[0]) != 0u) break;
+      if (wall_clock64() - t0 > ticks) {
+        __hip_atomic_store(&sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
     }
     __builtin_amdgcn_s_sleep(2);
   }

@@ -42,6 +42,8 @@ struct ScoreArgs {
   uint32_t* clear;        // words to clear for the next kernel of the stream, or NULL
   int clear_per_req;
   uint64_t spin_ticks;    // bound of a grid-wide wait, in 100 MHz ticks
+  uint32_t absent;        // team members that never arrive (tests of the give-up path)
+  uint32_t* fault_out;    // caller's word, set to 1 when a wait gave up, or NULL
   int pool_kernel;        // max-pool window over the votes (tr.py:366-369), <= 0: off
   float* pool_votes;      // [B,pool_stride] un-pooled votes exchanged between workgroups
   int64_t pool_stride;
@@ -87,11 +89,14 @@ void select_zero_regions(const SelectWorkspace& w, void* workspace, int batch, Z
 // Clears two regions (the stand-alone form of what the rotation kernel does on the side).
 __global__ void select_zero_kernel(ZeroRegion r0, ZeroRegion r1);
 
+// Bound of a grid-wide wait of the fused selection: 2 s of the 100 MHz clock.
+constexpr uint64_t kSelectWaitTicks = 200000000ull;
+
 // Launch without the clearing pass: the regions above are known to be zero.
 int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
                   int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
                   int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
                   int64_t vote_stride, void* workspace, uint32_t* clear, int clear_per_req,
-                  hipStream_t stream);
+                  hipStream_t stream, uint64_t wait_ticks = kSelectWaitTicks, uint32_t absent = 0);
 
 }  // namespace ts

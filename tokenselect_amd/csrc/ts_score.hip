@@ -150,7 +150,7 @@ __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t*
     __syncthreads();
   }
   GridTeam team;
-  team.size = total * gridDim.x;
+  team.size = total * gridDim.x + a.absent;
   team.index = before * gridDim.x + blockIdx.x;
   return team;
 }
@@ -977,6 +977,14 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       out_run += chosen_total;
       __syncthreads();
     }
+    // A grid-wide wait of this launch gave up (the workgroups were not all resident
+    // within the bound): what was selected is not valid.  The first workgroup of every
+    // selecting request says so in place of the length, and in the caller's word.
+    if (blockIdx.x == 0 && tid == 0 && load_coherent(&a.sync[0]) != 0u) {
+      a.sel_len[b] = -1;
+      if (a.fault_out)
+        __hip_atomic_store(a.fault_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
   }
 }
 
@@ -1023,10 +1031,8 @@ static size_t fused_lds_bytes(int tokens_per_block, int num_heads) {
 // workgroups fit the 160 KB of a CU.
 constexpr size_t kFusedStageBytes = 68 * 1024;
 
-static std::atomic<int> g_fused_select{[] {
-  const char* e = getenv("TS_FUSED_SELECT");  // "0" starts with the separate kernels
-  return (e && e[0] == '0') ? 0 : 1;
-}()};
+// The one process-wide switch of the library (ts_set_fused_select).
+static std::atomic<int> g_fused_select{1};
 
 int set_fused_select(int enable) { return g_fused_select.exchange(enable ? 1 : 0); }
 
@@ -1148,7 +1154,7 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
                   int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
                   int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
                   int64_t vote_stride, void* workspace, uint32_t* clear, int clear_per_req,
-                  hipStream_t stream) {
+                  hipStream_t stream, uint64_t wait_ticks, uint32_t absent) {
   const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len);
   TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE, "fused selection: unsupported shape");
   char* ws = (char*)workspace;
@@ -1169,7 +1175,9 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   a.cache_len = cache ? cache->cache_len : nullptr;
   a.clear = clear;
   a.clear_per_req = clear_per_req;
-  a.spin_ticks = 200000000ull;  // 2 s of the 100 MHz clock
+  a.spin_ticks = wait_ticks;
+  a.absent = absent;
+  a.fault_out = bt->fault;
   a.pool_kernel = cfg->pool_kernel;
   a.pool_votes = (float*)(ws + w.pool_votes);
   a.pool_stride = w.pool_stride;
@@ -1269,12 +1277,16 @@ int ts_select_clear(const ts_config* cfg, const ts_batch* bt, void* workspace,
   return check_launch("select_zero_kernel");
 }
 
-int ts_select_cleared(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
-                      int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
-                      int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
-                      int64_t vote_stride, void* workspace, size_t workspace_bytes,
-                      ts_stream_t stream) {
+int ts_select_cleared_bounded(const ts_config* cfg, const ts_batch* bt, const void* qf,
+                              const void* k_pool, int64_t pool_rows, const int32_t* hit,
+                              const ts_selcache* cache, int32_t* sel, int32_t* sel_pos,
+                              int64_t sel_stride, int32_t* sel_len, float* votes,
+                              int64_t vote_stride, void* workspace, size_t workspace_bytes,
+                              uint64_t wait_ticks, int32_t absent_workgroups, ts_stream_t stream) {
   SelectWorkspace w;
+  TS_REQUIRE(wait_ticks >= 1 && absent_workgroups >= 0, TS_EINVAL,
+             "ts_select: wait_ticks %llu / absent_workgroups %d out of range",
+             (unsigned long long)wait_ticks, absent_workgroups);
   TS_TRY(check_select(cfg, bt, workspace, workspace_bytes, &w));
   TS_REQUIRE(qf && k_pool && sel && sel_pos && sel_len, TS_EINVAL, "ts_select: NULL tensor argument");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
@@ -1291,7 +1303,18 @@ int ts_select_cleared(const ts_config* cfg, const ts_batch* bt, const void* qf, 
     TS_REQUIRE(cache->topk_cache && cache->cache_len, TS_EINVAL,
                "ts_select: selection cache has a NULL array");
   return launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,
-                       votes, vote_stride, workspace, nullptr, 0, (hipStream_t)stream);
+                       votes, vote_stride, workspace, nullptr, 0, (hipStream_t)stream, wait_ticks,
+                       (uint32_t)absent_workgroups);
+}
+
+int ts_select_cleared(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+                      int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
+                      int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
+                      int64_t vote_stride, void* workspace, size_t workspace_bytes,
+                      ts_stream_t stream) {
+  return ts_select_cleared_bounded(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride,
+                                   sel_len, votes, vote_stride, workspace, workspace_bytes,
+                                   kSelectWaitTicks, 0, stream);
 }
 
 int ts_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,

@@ -61,10 +61,35 @@ class Batch:
     table: torch.Tensor
     max_seq_len: int
     k_per_req: Optional[torch.Tensor] = None
+    # One int32 word of pinned host memory (see fault_word()) that the single-launch
+    # selection sets to 1 when one of its grid-wide waits gave up, or None.
+    fault: Optional[torch.Tensor] = None
 
     @property
     def batch(self) -> int:
         return int(self.seq_lens.shape[0])
+
+
+class SelectionGaveUp(RuntimeError):
+    """A grid-wide wait of the single-launch selection ran into its bound: the launch
+    did not have the device to itself (its workgroups were not all resident together)
+    and what it selected, and what was attended over, is not valid."""
+
+
+def fault_word() -> torch.Tensor:
+    """A zeroed int32 word of pinned host memory.  The device maps such memory, so a
+    kernel can set it and the host can read it at any time without synchronising."""
+    return torch.zeros((1,), dtype=torch.int32).pin_memory()
+
+
+def raise_if_gave_up(word: Optional[torch.Tensor]) -> None:
+    """Raises SelectionGaveUp when ``word`` has been set by an earlier launch.  A plain
+    host read: a set word is seen at the latest after the next synchronisation."""
+    if word is not None and int(word[0]) != 0:
+        raise SelectionGaveUp(
+            "ts_select gave up waiting for its workgroups (is another stream or process using the "
+            "GPU?); results since the last check are not valid.  Serialise the GPU work, or call "
+            "ops.set_fused_select(False) to use the separate kernels, clear the word and rerun")
 
 
 @dataclass
@@ -128,8 +153,11 @@ def _c_batch(cfg: LayerConfig, bt: Batch) -> TsBatch:
         _need(bt.k_per_req, "k_per_req", torch.int32, 1)
         if bt.k_per_req.shape[0] != bt.batch:
             raise ValueError("k_per_req must have one entry per request")
+    if bt.fault is not None and (bt.fault.dtype != torch.int32 or bt.fault.numel() != 1 or
+                                 not (bt.fault.is_cuda or bt.fault.is_pinned())):
+        raise ValueError("fault must be one int32 word of device or pinned host memory")
     return TsBatch(bt.batch, int(bt.max_seq_len), _p(bt.seq_lens), _p(bt.table),
-                   int(bt.table.stride(0)), _p(bt.k_per_req))
+                   int(bt.table.stride(0)), _p(bt.k_per_req), _p(bt.fault))
 
 
 def _c_cache(cache: Optional[SelectionCache], cfg: LayerConfig, batch: int):
@@ -259,14 +287,16 @@ def select_workspace(cfg: LayerConfig, bt: Batch, device) -> torch.Tensor:
 def select(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
            hit: Optional[torch.Tensor] = None, cache: Optional[SelectionCache] = None,
            want_votes: bool = False, workspace: Optional[torch.Tensor] = None,
-           cleared: bool = False):
+           cleared: bool = False, wait_ticks: Optional[int] = None, absent_workgroups: int = 0):
     """The whole selection in one launch (tr.py:350-373, 424-449): scoring, soft vote,
     exact top-k, ascending order and index assembly, the scores never leaving LDS.
     Returns ``(sel, sel_pos, sel_len, votes, workspace)`` with the first three as
     from :func:`topk_ragged`; ``votes`` is ``[B, stride]`` fp32 when ``want_votes``
     else ``None``.  ``workspace`` (uint8) may be passed back in to avoid allocating;
     with ``cleared`` the caller has run :func:`select_clear` on it since its last use
-    and only the selection kernel is launched."""
+    and only the selection kernel is launched.  ``wait_ticks`` / ``absent_workgroups``
+    go to ``ts_select_cleared_bounded`` (tests of the give-up path).  A launch that gave
+    up reports ``sel_len[b] == -1`` and sets ``bt.fault``."""
     c, cb = cfg.to_c(), _c_batch(cfg, bt)
     _need(qf, "qf", torch.bfloat16)
     _check_pool(cfg, k_pool, "k_pool")
@@ -288,10 +318,18 @@ def select(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
     if want_votes:
         votes = torch.empty((B, score_stride_for(bt.max_seq_len)), dtype=torch.float32,
                             device=qf.device)
-    _lib.check((lib.ts_select_cleared if cleared else lib.ts_select)(
-        ctypes.byref(c), ctypes.byref(cb), _p(qf), _p(k_pool), k_pool.shape[0], _p(hit),
-        _c_cache(cache, cfg, B), _p(sel), _p(sel_pos), cfg.max_sel, _p(sel_len), _p(votes),
-        votes.shape[1] if votes is not None else 0, _p(workspace), workspace.numel(), _stream()))
+    args = (ctypes.byref(c), ctypes.byref(cb), _p(qf), _p(k_pool), k_pool.shape[0], _p(hit),
+            _c_cache(cache, cfg, B), _p(sel), _p(sel_pos), cfg.max_sel, _p(sel_len), _p(votes),
+            votes.shape[1] if votes is not None else 0, _p(workspace), workspace.numel())
+    if wait_ticks is not None or absent_workgroups:
+        if not cleared:
+            _lib.check(lib.ts_select_clear(ctypes.byref(c), ctypes.byref(cb), _p(workspace),
+                                           workspace.numel(), _stream()))
+        _lib.check(lib.ts_select_cleared_bounded(
+            *args, int(wait_ticks if wait_ticks is not None else 200_000_000),
+            int(absent_workgroups), _stream()))
+    else:
+        _lib.check((lib.ts_select_cleared if cleared else lib.ts_select)(*args, _stream()))
     return sel, sel_pos, sel_len, votes, workspace
 
 
@@ -499,10 +537,20 @@ class DecodeLayer:
         self.sel = torch.empty((batch, cfg.max_sel), dtype=torch.int32, device=device)
         self.sel_pos = torch.empty_like(self.sel)
         self.sel_len = torch.empty((batch,), dtype=torch.int32, device=device)
+        self.fault = fault_word()
+
+    def check(self) -> None:
+        """Raises SelectionGaveUp if a selection of this layer gave up since the last
+        check.  Costs a host memory read; call it wherever the stream has been
+        synchronised anyway (it also runs at the start of every call)."""
+        raise_if_gave_up(self.fault)
 
     def __call__(self, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch,
                  cache: Optional[SelectionCache] = None, out: Optional[torch.Tensor] = None):
         cfg = self.cfg
+        self.check()
+        if bt.fault is None:
+            bt = Batch(bt.seq_lens, bt.table, bt.max_seq_len, bt.k_per_req, self.fault)
         cb = _c_batch(cfg, bt)
         if bt.batch > self.batch or bt.max_seq_len > self.max_seq_len:
             raise ValueError("batch / max_seq_len exceed what this DecodeLayer was sized for")
@@ -620,10 +668,18 @@ class PrefillChunk:
         self.sel = torch.empty((1, cfg.max_sel), dtype=torch.int32, device=device)
         self.sel_pos = torch.empty_like(self.sel)
         self.sel_len = torch.empty((1,), dtype=torch.int32, device=device)
+        self.fault = fault_word()
+
+    def check(self) -> None:
+        """As DecodeLayer.check()."""
+        raise_if_gave_up(self.fault)
 
     def __call__(self, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch,
                  out: Optional[torch.Tensor] = None):
         cfg = self.cfg
+        self.check()
+        if bt.fault is None:
+            bt = Batch(bt.seq_lens, bt.table, bt.max_seq_len, bt.k_per_req, self.fault)
         cb = _c_batch(cfg, bt)
         _need(q, "q", torch.bfloat16, 2)
         rows = q.shape[0]
