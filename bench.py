@@ -164,9 +164,9 @@ def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
     return roofline, score_only, attn
 
 
-def bench_layer(args, ops, workloads, dev):
+def bench_layer(args, ops, workloads, dev, which=None):
     make = {"c1": workloads.config1, "c2": workloads.config2, "c3": workloads.config3,
-            "c5": workloads.config5_layer}[args.workload]
+            "c5": workloads.config5_layer}[which or args.workload]
     wl = make(dev)
     c, bt, B = wl.cfg, wl.batch, len(wl.seq_lens)
     layer = ops.DecodeLayer(c, B, bt.max_seq_len, dev)
@@ -212,10 +212,10 @@ def bench_layer(args, ops, workloads, dev):
     if not args.no_cpu_baseline:
         # Bounded sample: the whole batch where that is a few hundred ms of CPU work,
         # else its first two requests.
-        sample = None if sum(wl.seq_lens) <= 300000 else [0, 1]
+        sample = None if sum(wl.seq_lens) <= 300000 else [0, 1][:args.cpu_requests]
         cpu_us, cores, ref_sels, ref_out = cpu_baseline(wl, args.cpu_reps, sample)
         what = f"the full {wl.name} layer" if sample is None else \
-            f"requests 0-1 (L={wl.seq_lens[0]}, {wl.seq_lens[1]}) of {wl.name}"
+            f"requests {sample} (L={[wl.seq_lens[b] for b in sample]}) of {wl.name}"
         result["cpu_baseline"] = {
             "value": round(cpu_us, 1), "unit": "us", "cores": cores, "kind": "port",
             "sample": f"{what}, median of {args.cpu_reps} repetitions after one warm-up "
@@ -235,25 +235,30 @@ def bench_trace(args, ops, workloads, dev):
     new token's K/V stored first, AR(1) queries with occasional jumps, cosine reuse
     threshold bf16(0.9).  Reports the amortised time per step and the hit rate."""
     steps = args.trace_steps
-    wl = workloads.config4(dev, steps=steps)
+    ps = args.page_size
+    wl = workloads.config4(dev, steps=steps, page_size=ps)
     c, B = wl.cfg, len(wl.seq_lens)
     L0 = wl.seq_lens[0]
     qs = workloads.ar1_queries(B, c.num_heads * c.head_dim, steps, dev)
     gen = torch.Generator(device=dev).manual_seed(7)
     k_new = torch.randn((steps, B, c.num_kv_heads * c.head_dim), generator=gen, device=dev).bfloat16()
     v_new = torch.randn((steps, B, c.num_kv_heads * c.head_dim), generator=gen, device=dev).bfloat16()
-    free = torch.arange(B * L0, B * (L0 + steps), dtype=torch.int32, device=dev).view(steps, B)
-    table0 = torch.zeros((B, L0 + steps), dtype=torch.int32, device=dev)
-    table0[:, :L0] = wl.table[:, :L0]
+    # New tokens go to the slots a serving framework would hand over (per-token table),
+    # or, with pages, to fresh pages the store kernel takes from the device-side free list.
+    free = wl.free_pages[:B * steps].view(steps, B) if ps == 1 else None
+    table0 = torch.zeros((B, -(-(L0 + steps) // ps)), dtype=torch.int32, device=dev)
+    table0[:, :wl.table.shape[1]] = wl.table
     layer = ops.DecodeLayer(c, B, L0 + steps, dev)
 
     def run_trace():
         table, seq = table0.clone(), wl.seq_lens_dev.clone()
         cache = ops.SelectionCache.allocate(c, B, dev)
+        pages = ops.PagePool.of(wl.free_pages) if ps > 1 else None
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for t in range(steps):
-            ops.kv_store(c, k_new[t], v_new[t], free[t], wl.k_pool, wl.v_pool, table, seq)
+            ops.kv_store(c, k_new[t], v_new[t], None if pages else free[t], wl.k_pool, wl.v_pool, table,
+                         seq, pages=pages)
             layer(qs[t], wl.k_pool, wl.v_pool, ops.Batch(seq, table, L0 + t + 1), cache)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps * 1e6, cache
@@ -272,7 +277,7 @@ def bench_trace(args, ops, workloads, dev):
         "warmup": max(1, args.warmup // steps) * steps, "ms_per_step": round(us_per_step / 1e3, 5),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": wl.name, "batch": B, "seq_lens_max": L0 + steps, "page_size": 1,
+        "config": {"workload": wl.name, "batch": B, "seq_lens_max": L0 + steps, "page_size": ps,
                    "top_k": c.top_k, "n_init": c.n_init, "n_local": c.n_local,
                    "trace_steps": steps, "ar1_rho": 0.95, "jump_p": 0.1,
                    "threshold": runs[-1][1].threshold, "kv_pool_copies": 1},
@@ -483,6 +488,40 @@ def bench_model(args, ops, dev):
     return result
 
 
+def extra_workloads(args, ops, workloads, dev):
+    """Compact lines for the other configurations, appended to the default run so that one
+    driver-run command measures them all: fewer steps, two pool copies, the oracle on one
+    request (parity only)."""
+    import copy
+    lines = []
+    small = copy.copy(args)
+    small.steps, small.warmup, small.pools = 50, 10, 2
+    small.cpu_reps, small.cpu_requests = 1, 1
+    for which in ("c1", "c3", "c5"):
+        t0 = time.perf_counter()
+        r = bench_layer(small, ops, workloads, dev, which)
+        roof = r["roofline"]
+        lines.append({
+            "workload": r["config"]["workload"], "us_per_layer": r["value"],
+            "dominant_kernel": roof["kernel"].split(" ")[0], "us_per_launch": roof["us_per_launch"],
+            "bytes_per_launch": roof["bytes_per_launch"], "frac": roof["frac"],
+            "score_only_frac": r["score_only"]["frac"],
+            "attn_us": r["gather_attention"]["us_per_launch"], "parity": r.get("parity"),
+            "wall_s": round(time.perf_counter() - t0, 1)})
+        torch.cuda.empty_cache()
+    t0 = time.perf_counter()
+    small.steps, small.warmup = 64, 64
+    r = bench_trace(small, ops, workloads, dev)
+    lines.append({"workload": r["config"]["workload"], "us_per_step": r["value"],
+                  "hit_rate": r["hit_rate"], "wall_s": round(time.perf_counter() - t0, 1)})
+    small.page_size = 16
+    t0 = time.perf_counter()
+    r = bench_trace(small, ops, workloads, dev)
+    lines.append({"workload": r["config"]["workload"], "us_per_step": r["value"],
+                  "hit_rate": r["hit_rate"], "wall_s": round(time.perf_counter() - t0, 1)})
+    return lines
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -501,6 +540,12 @@ def main():
     ap.add_argument("--pools", type=int, default=4,
                     help="copies of the K/V pool cycled through, one per step")
     ap.add_argument("--trace-steps", type=int, default=64, help="decode steps of the c4 trace")
+    ap.add_argument("--page-size", type=int, default=1,
+                    help="tokens per KV page of the c4 trace (above 1: appends through the page pool)")
+    ap.add_argument("--cpu-requests", type=int, default=2,
+                    help="requests of a large batch the CPU oracle is run on")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="default run: only the headline workload, not the compact lines of the others")
     ap.add_argument("--prefill-context", type=int, default=131072,
                     help="tokens already cached when the measured prefill chunk arrives")
     ap.add_argument("--prefill-rows", type=int, default=512, help="rows of the prefill chunk")
@@ -528,6 +573,8 @@ def main():
         result = bench_model(args, ops, dev)
     else:
         result = bench_layer(args, ops, workloads, dev)
+        if args.workload == "c2" and not args.no_extra:
+            result["extra_workloads"] = extra_workloads(args, ops, workloads, dev)
     print(json.dumps(result), flush=True)
 
 

@@ -97,6 +97,20 @@ typedef struct ts_selcache {
   float threshold;      /* similarity_threshold, bf16(0.9)=0.8984375 (tr.py:313) */
 } ts_selcache;
 
+/* Free pages of a paged KV pool, for the store entry points when the library and
+ * not the serving framework places new tokens (any page_size; required when
+ * page_size > 1).  All arrays are device memory owned by the caller.  The list is a
+ * stack: entries [0, *free_count) are free and a store takes them from the top,
+ * free_pages[*free_count - 1] first, for the requests that need one in request
+ * order; the host returns pages by writing them at the top and raising the count
+ * between launches.  ticket is one word that is zero before the first call and
+ * between calls; the store kernels count their workgroups in it and reset it. */
+typedef struct ts_page_pool {
+  const int32_t* free_pages; /* [capacity] physical page numbers                 */
+  int32_t* free_count;       /* [1]                                              */
+  uint32_t* ticket;          /* [1]                                              */
+} ts_page_pool;
+
 int ts_version(void);
 const char* ts_last_error(void);
 
@@ -267,12 +281,21 @@ int ts_sparse_decode_attn_static(const ts_config* cfg, const void* q, const void
                                  int32_t max_sel_len, void* out, ts_stream_t stream);
 
 /* KV store + table append (patched_radix_attention_store_kv_cache tr.py:844-854,
- * add_k_cache tr.py:332-336) for page_size 1: k_pool[loc[b]] = k[b],
- * v_pool[loc[b]] = v[b], table[b][seq_lens[b]] = loc[b], seq_lens[b] += 1. */
+ * add_k_cache tr.py:332-336).
+ * pages == NULL, page_size 1 (the reference): the framework has chosen the slots,
+ *   k_pool[loc[b]] = k[b], v_pool[loc[b]] = v[b], table[b][seq_lens[b]] = loc[b],
+ *   seq_lens[b] += 1.
+ * pages != NULL (any page_size; out_cache_loc is not read): the new token of request
+ *   b, at position L = seq_lens[b], goes to slot table[b][L/ps]*ps + L%ps; when
+ *   L % ps == 0 the request first takes a fresh page from the pool (in request
+ *   order, top of the stack first) and table[b][L/ps] receives it.  A request
+ *   whose table is full (L >= max_tokens) or that finds no page left is left
+ *   untouched; *free_count drops by the pages taken.
+ * k, v: [batch, Hkv, D] bf16; table rows hold ceil(max_tokens / ps) entries. */
 int ts_kv_store(const ts_config* cfg, const void* k, const void* v, const int32_t* out_cache_loc,
-                void* k_pool, void* v_pool, int64_t pool_rows, int32_t* table,
-                int64_t table_stride, int32_t* seq_lens, int32_t batch, int32_t max_tokens,
-                ts_stream_t stream);
+                const ts_page_pool* pages, void* k_pool, void* v_pool, int64_t pool_rows,
+                int32_t* table, int64_t table_stride, int32_t* seq_lens, int32_t batch,
+                int32_t max_tokens, ts_stream_t stream);
 
 /* The QKV projection of a decode step with the KV store as its epilogue: what the
  * serving stack does in two places, qkv = x W^T (+ bias) in the model's attention
@@ -280,13 +303,16 @@ int ts_kv_store(const ts_config* cfg, const void* k, const void* v, const int32_
  * add_k_cache (tr.py:332-336), in one pass over W.  Columns [0, H*D) of the product
  * go to q_out [batch, H*D]; the next Hkv*D to k_pool[loc[b]], the last Hkv*D to
  * v_pool[loc[b]]; then table[b][seq_lens[b]] = loc[b], seq_lens[b] += 1 as
- * ts_kv_store does (a full table leaves table and length alone).  x: [batch, hidden]
+ * ts_kv_store does, with the caller's slots (pages == NULL, page_size 1; a full
+ * table leaves table and length alone) or with slots from the table / the page
+ * pool (pages != NULL, as for ts_kv_store).  x: [batch, hidden]
  * bf16; w: [(H + 2 Hkv) * D, hidden] bf16 row-major (torch Linear weight);
  * bias: [(H + 2 Hkv) * D] bf16 or NULL; fp32 accumulation, bf16 outputs.
  * batch <= 8 and hidden a multiple of 8, at most 4096 (TS_ESHAPE otherwise: use a
  * library GEMM and ts_kv_store). */
 int ts_qkv_store(const ts_config* cfg, const void* x, const void* w, const void* bias,
-                 int32_t hidden, const int32_t* out_cache_loc, void* q_out, void* k_pool,
+                 int32_t hidden, const int32_t* out_cache_loc, const ts_page_pool* pages,
+                 void* q_out, void* k_pool,
                  void* v_pool, int64_t pool_rows, int32_t* table, int64_t table_stride,
                  int32_t* seq_lens, int32_t batch, int32_t max_tokens, ts_stream_t stream);
 
@@ -296,12 +322,16 @@ int ts_qkv_store(const ts_config* cfg, const void* x, const void* w, const void*
  * queries, and the chunk attends causally over the selected slots. ---- */
 
 /* store_kv_cache(start, end) + add_k_cache for a chunk (tr.py:725-733,
- * 332-336), page size 1: k_pool[loc[r]] = k[r], v likewise,
+ * 332-336).  pages == NULL, page size 1: k_pool[loc[r]] = k[r], v likewise,
  * table[*seq_len + r] = loc[r] for r < rows, then *seq_len += rows.
+ * pages != NULL: row r goes to position *seq_len + r of the paged table, the
+ * request's last page first and then fresh pages from the top of the pool, in
+ * order; one launch.
  * k, v: [rows, Hkv, D] bf16; table: the request's row; rows beyond max_tokens
- * are dropped. */
+ * (or beyond the pages left) are dropped. */
 int ts_kv_store_chunk(const ts_config* cfg, const void* k, const void* v,
-                      const int32_t* out_cache_loc, int32_t rows, void* k_pool, void* v_pool,
+                      const int32_t* out_cache_loc, const ts_page_pool* pages, int32_t rows,
+                      void* k_pool, void* v_pool,
                       int64_t pool_rows, int32_t* table, int32_t* seq_len, int32_t max_tokens,
                       ts_stream_t stream);
 

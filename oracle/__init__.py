@@ -23,6 +23,12 @@ a CUDA GPU, none of which are available):
 * ``prefill``   - causal attention against ``F.scaled_dot_product_attention`` with
                   an explicit mask (RoPE off), a one-row chunk == ``attend``, row
                   ``i`` == decode attention over the first ``S - m + i + 1`` keys.
+* ``store``     - the per-token append is a slice assignment (tr.py:332-336); the
+                  paged append (no reference counterpart: an extension, like
+                  batches) is pinned by what the page arithmetic fixes: a chunk
+                  equals the same tokens appended one by one, slots equal the
+                  expanded page table, pages taken = ceil((L+m)/ps) - ceil(L/ps),
+                  a page size of 1 reduces to popping one slot per token.
 * ``selcache``  - pure-Python replay of the state machine.  The reference ships
                   this branch disabled and not runnable (tr.py:918, 412, 397), so
                   its behaviour is *intended* semantics: parity unpinned.
@@ -32,4 +38,4 @@ the bf16 rounding / reduction order of Triton 3.0.0's ``tl.sum`` on NVIDIA, the
 tie order of CUDA ``torch.topk``, and FlashInfer's ``__sincosf`` error.
 """
 
-from . import rope, select, attend, selcache, layer, prefill  # noqa: F401
+from . import rope, select, attend, selcache, layer, prefill, store  # noqa: F401

@@ -108,8 +108,14 @@ def test_null_and_range_errors_need_no_gpu(lib):
     assert lib.ts_paged_matmul(one, one, 10, one, one, 5, 10, 32, 8, 128, None) == _lib.TS_EINVAL
     assert lib.ts_paged_matmul(one, one, 10, one, one, 0, 10, 32, 8, 64, None) == _lib.TS_ESHAPE
     assert lib.ts_rope_apply(one, one, one, one, None, 1, 1, 4, 127, None) == _lib.TS_ESHAPE
-    assert lib.ts_kv_store(ctypes.byref(cfg(page_size=16)), one, one, one, one, one, 10, one, 100,
+    # pages of 16 tokens without a page pool
+    assert lib.ts_kv_store(ctypes.byref(cfg(page_size=16)), one, one, one, None, one, one, 10, one, 100,
                            one, 1, 100, None) == _lib.TS_EINVAL
+    assert "page pool" in err(lib)
+    # more than 2^20 candidates per request
+    huge = _lib.TsBatch(1, (1 << 20) + 641, one, one, 1 << 21, None)
+    assert lib.ts_topk_ragged(ctypes.byref(c), ctypes.byref(huge), one, 1 << 21, None, None, one, one,
+                              4096, one, one, 1 << 30, None) == _lib.TS_ESHAPE
     assert lib.ts_decode_layer(ctypes.byref(c), ctypes.byref(bt), one, one, one, one, one, 10, None,
                                one, one, one, 4096, one, one, 64, None) == _lib.TS_EWORKSPACE
     assert "workspace" in err(lib)

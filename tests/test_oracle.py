@@ -431,3 +431,70 @@ def test_prefill_loop_stores_then_selects_chunk_by_chunk():
     _, ref = oracle.prefill.prefill_chunk(q[32:64], kp, vp, tab, L2, H, 128, 4, chunk, 16, 1e4, 1.0,
                                           0.1)
     assert torch.equal(out[32:64], ref)
+
+
+# ------------------------------------------------------------- store / paged append
+def test_append_slots_is_the_reference_slice_assignment():
+    tab = torch.zeros(10, dtype=torch.int32)
+    L = oracle.store.append_slots(tab, 3, torch.tensor([7, 8, 9]), 10)
+    assert L == 6 and tab.tolist() == [0, 0, 0, 7, 8, 9, 0, 0, 0, 0]
+    assert oracle.store.append_slots(tab, 8, torch.tensor([1, 2, 3]), 10) == 10   # tail dropped
+    assert tab[8:].tolist() == [1, 2]
+
+
+def test_paged_append_matches_what_the_page_arithmetic_fixes():
+    ps, pages_cap = 4, 12
+    g = torch.Generator().manual_seed(5)
+    free = torch.randperm(40, generator=g).tolist()
+    table = torch.full((3, pages_cap), -1, dtype=torch.int32)
+    lens = [0, 0, 0]
+    given = {b: [] for b in range(3)}
+    start = len(free)
+    for step in range(19):
+        slots = oracle.store.append_token_paged(table, lens, free, ps, pages_cap * ps, 40 * ps)
+        for b, s in enumerate(slots):
+            given[b].append(s)
+    assert lens == [19, 19, 19]
+    for b in range(3):     # slots are exactly the expanded page table
+        assert oracle.select.expand_page_table(table[b], 19, ps).tolist() == given[b]
+    used = table[table >= 0].tolist()
+    assert len(set(used)) == len(used) == 3 * 5            # ceil(19 / 4) pages each, all distinct
+    assert start - len(free) == 15 and not set(used) & set(free)
+    # request order, top of the stack first
+    free2 = [10, 11, 12]
+    t2 = torch.full((2, 4), -1, dtype=torch.int32)
+    assert oracle.store.append_token_paged(t2, [0, 4], free2, 4, 16, 1000) == [12 * 4, 11 * 4]
+    assert free2 == [10] and t2[0, 0] == 12 and t2[1, 1] == 11
+    # page size 1: one slot popped per token
+    t3 = torch.full((1, 8), -1, dtype=torch.int32)
+    free3 = [5, 6, 7]
+    assert oracle.store.append_token_paged(t3, [2], free3, 1, 8, 100) == [7] and free3 == [5, 6]
+
+
+def test_paged_chunk_equals_token_by_token_and_drops_what_does_not_fit():
+    ps = 16
+    for L0, rows in ((0, 80), (37, 45), (48, 3), (15, 1), (16, 33)):
+        free_a, free_b = list(range(100, 120)), list(range(100, 120))
+        row_a = torch.full((16,), -1, dtype=torch.int32)
+        row_a[:(L0 + ps - 1) // ps] = torch.arange(50, 50 + (L0 + ps - 1) // ps, dtype=torch.int32)
+        row_b = row_a.clone()
+        slots, L = oracle.store.append_chunk_paged(row_a, L0, rows, free_a, ps, 256)
+        one_by_one = []
+        lens = [L0]
+        tab_b = row_b.view(1, -1)
+        for _ in range(rows):
+            one_by_one += oracle.store.append_token_paged(tab_b, lens, free_b, ps, 256, 10 ** 6)
+        assert slots == one_by_one and L == lens[0] == L0 + rows
+        assert torch.equal(row_a, row_b) and free_a == free_b
+        assert 20 - len(free_a) == -(-(L0 + rows) // ps) - (-(-L0 // ps))     # closed form
+    # two pages left for a chunk that wants three; the table ends at 40 tokens
+    row = torch.full((4,), -1, dtype=torch.int32)
+    slots, L = oracle.store.append_chunk_paged(row, 0, 48, [3, 9], ps, 64)
+    assert L == 32 and slots[:16] == list(range(9 * 16, 10 * 16)) and slots[16:] == list(range(48, 64))
+    row = torch.full((4,), -1, dtype=torch.int32)
+    assert oracle.store.append_chunk_paged(row, 0, 48, [1, 2, 3, 4], ps, 40)[1] == 40
+    # a full table or an empty stack leaves a request untouched
+    t = torch.full((2, 2), -1, dtype=torch.int32)
+    lens = [32, 16]
+    assert oracle.store.append_token_paged(t, lens, [], ps, 32, 10 ** 6) == [None, None]
+    assert lens == [32, 16] and bool((t == -1).all())

@@ -46,7 +46,12 @@ class TsSelCache(ctypes.Structure):
     ]
 
 
+class TsPagePool(ctypes.Structure):
+    _fields_ = [("free_pages", _ptr), ("free_count", _ptr), ("ticket", _ptr)]
+
+
 _CFG, _BT, _SC = ctypes.POINTER(TsConfig), ctypes.POINTER(TsBatch), ctypes.POINTER(TsSelCache)
+_PP = ctypes.POINTER(TsPagePool)
 
 # name -> (restype, argtypes); mirrors include/tokenselect.h one to one.
 SIGNATURES = {
@@ -78,11 +83,12 @@ SIGNATURES = {
     "ts_attn_static_scratch_bytes": (_size, []),
     "ts_sparse_decode_attn_static": (_i32, [_CFG, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
                                             _ptr, _ptr]),
-    "ts_kv_store": (_i32, [_CFG, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
+    "ts_kv_store": (_i32, [_CFG, _ptr, _ptr, _ptr, _PP, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
                            _ptr]),
-    "ts_qkv_store": (_i32, [_CFG, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr,
-                            _i32, _i32, _ptr]),
-    "ts_kv_store_chunk": (_i32, [_CFG, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i32, _ptr]),
+    "ts_qkv_store": (_i32, [_CFG, _ptr, _ptr, _ptr, _i32, _ptr, _PP, _ptr, _ptr, _ptr, _i64, _ptr, _i64,
+                            _ptr, _i32, _i32, _ptr]),
+    "ts_kv_store_chunk": (_i32, [_CFG, _ptr, _ptr, _ptr, _PP, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i32,
+                                 _ptr]),
     "ts_fingerprint": (_i32, [_CFG, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr]),
     "ts_prefill_attn_workspace_bytes": (_size, [_CFG, _i32]),
     "ts_sparse_prefill_attn": (_i32, [_CFG, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i32, _ptr, _ptr,

@@ -105,7 +105,8 @@ struct LayerWorkspace {
   int32_t max_sel;
 };
 
-static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32_t max_seq_len,
+                                      bool ignore_switch = false) {
   LayerWorkspace w;
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -125,7 +126,7 @@ static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32
   w.partials_bytes = ts_score_partials_bytes(cfg, batch, max_seq_len);
   w.partials = take(w.partials_bytes);
   w.topk_ws = take(ts_topk_workspace_bytes(cfg, batch, max_seq_len));
-  w.select_ws = take(select_workspace(cfg, batch, max_seq_len).total);
+  w.select_ws = take(select_workspace(cfg, batch, max_seq_len, ignore_switch).total);
   {  // decode attention partials, or the staging area of the prefill attention
     const size_t decode = ts_attn_workspace_bytes(cfg, batch, w.max_sel);
     const size_t prefill = ts_prefill_attn_workspace_bytes(cfg, w.max_sel);
@@ -137,7 +138,15 @@ static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32
 
 size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
-  return layer_workspace(cfg, batch, max_seq_len).total;
+  // A workspace sized for `batch` serves every smaller batch and both settings of
+  // ts_set_fused_select: the pieces do not all grow with the batch (attention splits,
+  // candidates per workgroup of the fused selection), so the largest layout is taken.
+  size_t most = 0;
+  for (int32_t b = 1; b <= batch; ++b) {
+    const size_t need = layer_workspace(cfg, b, max_seq_len, /*ignore_switch=*/true).total;
+    if (need > most) most = need;
+  }
+  return most;
 }
 
 // Decode (chunk_rows == 0: one query row per request, q_cos / q_sin are the [D] rows
@@ -156,6 +165,9 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);
+  // The tie-break of the ragged top-k orders positions by two 10-bit digits.
+  TS_REQUIRE(bt->max_seq_len - cfg->n_init - cfg->n_local <= (1 << 20), TS_ESHAPE,
+             "layer: at most 2^20 candidates per request (max_seq_len %d)", bt->max_seq_len);
   TS_REQUIRE(sel_stride >= w.max_sel, TS_EWORKSPACE, "sel_stride %lld < n_init+top_k+n_local = %d",
              (long long)sel_stride, w.max_sel);
   TS_REQUIRE(workspace != nullptr && workspace_bytes >= w.total, TS_EWORKSPACE,

@@ -275,7 +275,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int q_row0 = blockIdx.x * 16;
   const int shift = S - m;  // query row i sits at position shift + i and sees keys <= that
   const bool rope = a.rope_mode == TS_ROPE_LLAMA;
-  if (S < m || S <= 0) return;  // fewer keys than rows: not a prefill chunk
+  if (S < m || S <= 0) {
+    // Fewer keys than rows (not a prefill chunk, or a selection that reported a
+    // fault): the rows attend to nothing and the output is defined as zero.
+    if (wave_active)
+      for (int i = lane; i < 16 * (kHeadDim / 8); i += 64) {
+        const int row = q_row0 + i / (kHeadDim / 8);
+        if (row < m)
+          *(uint4*)(a.out + ((size_t)row * H + h) * kHeadDim + 8 * (i % (kHeadDim / 8))) =
+              make_uint4(0u, 0u, 0u, 0u);
+      }
+    return;
+  }
 
   // ---- queries: B operand, lane (qc, g4) holds dims [32 ks + 8 g4, +8) of row q_row0 + qc,
   // rotated to position shift + row (partner dims d and d + 64 are k-steps ks and ks + 2).

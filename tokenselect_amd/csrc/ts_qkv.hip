@@ -12,7 +12,7 @@
 // them with the matching pieces of x from LDS (bf16, staged once per workgroup of
 // eight wavefronts) and the wavefront reduces its 2 x B sums on its own: no
 // exchange between wavefronts.
-#include "ts_common.h"
+#include "ts_pages.h"
 
 namespace ts {
 
@@ -36,6 +36,8 @@ struct QkvArgs {
   int64_t table_stride;
   int32_t* seq_lens;
   int max_tokens;
+  PagePool pool;  // free_pages != NULL: slots come from the table / the free list (ts_pages.h)
+  int page_shift;
 };
 
 __device__ __forceinline__ void unpack8(const uint4& w, float (&f)[8]) {
@@ -122,7 +124,27 @@ __global__ __launch_bounds__(64 * kQkvWaves) void qkv_store_kernel(QkvArgs a) {
       if (n < a.q_cols) {
         a.q_out[(size_t)b * a.q_cols + n] = out;
       } else {
-        const int64_t slot = a.loc[b];
+        int64_t slot = -1;
+        if (a.pool.free_pages) {
+          // The plan of request b, from the lengths as they were at launch: the
+          // requests before it that take a page decide which page it takes.
+          const int page_mask = (1 << a.page_shift) - 1;
+          uint32_t rank = 0;
+#pragma unroll
+          for (int c = 0; c < B; ++c) {
+            const int lc = a.seq_lens[c];
+            rank += (c < b && lc >= 0 && lc < a.max_tokens && (lc & page_mask) == 0) ? 1u : 0u;
+          }
+          const int len = a.seq_lens[b];
+          const bool room = len >= 0 && len < a.max_tokens;
+          const AppendPlan plan = make_append_plan(
+              a.table + (int64_t)b * a.table_stride, len, room, room && (len & page_mask) == 0, rank,
+              max(*a.pool.free_count, 0), a.pool.free_pages, a.page_shift, page_mask,
+              (uint32_t)a.pool_rows);
+          if (plan.ok) slot = plan.slot;
+        } else {
+          slot = a.loc[b];
+        }
         if (slot >= 0 && slot < a.pool_rows) {
           const int c = n - a.q_cols;
           if (c < a.kv_cols)
@@ -134,8 +156,21 @@ __global__ __launch_bounds__(64 * kQkvWaves) void qkv_store_kernel(QkvArgs a) {
     }
   }
 
+  // Paged table: the launch's last workgroup commits the appends (nothing of the
+  // snapshot the plans are made from changes before every workgroup is through).
+  if (a.pool.free_pages) {
+    __syncthreads();
+    if (tid < 64)
+      commit_appends(a.seq_lens, a.table, a.table_stride, B, a.pool, a.page_shift, a.max_tokens,
+                     (uint32_t)a.pool_rows, lane, gridDim.x);
+    return;
+  }
   // Table append (add_k_cache tr.py:332-336) by the first workgroup; a full table
   // (tr.py:334 asserts) or a slot outside the pool leaves table and length alone.
+  // (The K and V rows of a request whose table is full are still written to the
+  // caller's slot: the other workgroups cannot consult a length that this one is
+  // changing.  The reference asserts on the host before it appends, tr.py:334, and so
+  // do the callers of this library.)
   if (blockIdx.x == 0 && tid < B) {
     const int b = tid;
     const int slot = a.loc[b];
@@ -161,14 +196,22 @@ static int launch_qkv(const QkvArgs& a, hipStream_t stream) {
 using namespace ts;
 
 extern "C" int ts_qkv_store(const ts_config* cfg, const void* x, const void* w, const void* bias,
-                            int32_t hidden, const int32_t* out_cache_loc, void* q_out,
+                            int32_t hidden, const int32_t* out_cache_loc,
+                            const ts_page_pool* pages, void* q_out,
                             void* k_pool, void* v_pool, int64_t pool_rows, int32_t* table,
                             int64_t table_stride, int32_t* seq_lens, int32_t batch,
                             int32_t max_tokens, ts_stream_t stream) {
   TS_TRY(validate_config(cfg));
-  TS_REQUIRE(x && w && out_cache_loc && q_out && k_pool && v_pool && table && seq_lens, TS_EINVAL,
+  TS_REQUIRE(x && w && q_out && k_pool && v_pool && table && seq_lens, TS_EINVAL,
              "ts_qkv_store: NULL tensor argument");
-  TS_REQUIRE(cfg->page_size == 1, TS_EINVAL, "ts_qkv_store appends to a per-token table (page_size 1)");
+  if (pages) {
+    TS_REQUIRE(pages->free_pages && pages->free_count && pages->ticket, TS_EINVAL,
+               "ts_qkv_store: page pool has a NULL array");
+  } else {
+    TS_REQUIRE(cfg->page_size == 1, TS_EINVAL,
+               "ts_qkv_store: page_size %d needs a page pool", cfg->page_size);
+    TS_REQUIRE(out_cache_loc != nullptr, TS_EINVAL, "ts_qkv_store: NULL out_cache_loc and no page pool");
+  }
   TS_REQUIRE(batch >= 1 && batch <= kQkvMaxBatch, TS_ESHAPE,
              "ts_qkv_store: batch %d outside 1..%d (use a library GEMM and ts_kv_store)", batch,
              kQkvMaxBatch);
@@ -177,9 +220,12 @@ extern "C" int ts_qkv_store(const ts_config* cfg, const void* x, const void* w, 
   TS_REQUIRE(pool_rows >= 1 && max_tokens >= 1, TS_EINVAL,
              "ts_qkv_store: pool_rows=%lld max_tokens=%d out of range", (long long)pool_rows,
              max_tokens);
-  TS_REQUIRE(batch == 1 || table_stride >= max_tokens, TS_EINVAL,
-             "ts_qkv_store: table_stride %lld < max_tokens %d", (long long)table_stride, max_tokens);
+  TS_REQUIRE(batch == 1 || table_stride * (int64_t)cfg->page_size >= max_tokens, TS_EINVAL,
+             "ts_qkv_store: table_stride %lld x page_size %d < max_tokens %d", (long long)table_stride,
+             cfg->page_size, max_tokens);
   QkvArgs a;
+  a.pool = page_pool_of(pages);
+  a.page_shift = page_shift_of(cfg->page_size);
   a.x = (const uint16_t*)x;
   a.w = (const uint16_t*)w;
   a.bias = (const uint16_t*)bias;

@@ -79,7 +79,10 @@ struct SelectWorkspace {
   int tokens_per_block;  // 0: the shape does not fit the fused kernel
   int blocks_per_req;
 };
-SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len);
+// ignore_switch: lay out as if ts_set_fused_select were on (for sizing a workspace that
+// must serve both settings).
+SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len,
+                                 bool ignore_switch = false);
 
 // Regions the kernel before ts_select on the stream has to clear (counters and
 // rendezvous words), in the form the rotation kernel takes them.

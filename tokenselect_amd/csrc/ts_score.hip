@@ -1036,9 +1036,10 @@ static std::atomic<int> g_fused_select{1};
 
 int set_fused_select(int enable) { return g_fused_select.exchange(enable ? 1 : 0); }
 
-int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len) {
+int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch) {
   // Max-pool windows beyond 256 would not fit the LDS the neighbours are gathered into.
-  if (!g_fused_select.load() || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256) return 0;
+  if ((!ignore_switch && !g_fused_select.load()) || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256)
+    return 0;
   const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
   if (max_n <= 0) return 0;
   const int group = cfg->num_heads / cfg->num_kv_heads;
@@ -1078,9 +1079,9 @@ int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len) {
   return tpb;
 }
 
-SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len) {
+SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch) {
   SelectWorkspace w{};
-  w.tokens_per_block = fused_tokens_per_block(cfg, batch, max_seq_len);
+  w.tokens_per_block = fused_tokens_per_block(cfg, batch, max_seq_len, ignore_switch);
   if (w.tokens_per_block <= 0) return w;
   const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
   w.blocks_per_req = (int)ceil_div(max_n, w.tokens_per_block);
@@ -1241,7 +1242,7 @@ int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const voi
 
 int ts_select_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
-  return fused_tokens_per_block(cfg, batch, max_seq_len) > 0 ? 1 : 0;
+  return fused_tokens_per_block(cfg, batch, max_seq_len, false) > 0 ? 1 : 0;
 }
 
 size_t ts_select_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {

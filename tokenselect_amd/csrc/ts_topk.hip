@@ -401,6 +401,9 @@ int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
   const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
   TS_REQUIRE(vote_stride >= max_n, TS_EWORKSPACE, "vote_stride %lld < max candidates %d",
              (long long)vote_stride, max_n);
+  // Ties at the k-th vote are cut by position, resolved as two 10-bit digits.
+  TS_REQUIRE(max_n <= (1 << 20), TS_ESHAPE,
+             "ts_topk_ragged: at most 2^20 candidates per request (max_seq_len %d)", bt->max_seq_len);
   TS_REQUIRE(hit == nullptr || cache != nullptr, TS_EINVAL,
              "ts_topk_ragged: hit flags need the selection cache");
   if (cache)

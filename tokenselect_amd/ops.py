@@ -13,7 +13,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._lib import TsBatch, TsConfig, TsSelCache
+from ._lib import TsBatch, TsConfig, TsPagePool, TsSelCache
 
 HEAD_DIM = 128
 
@@ -440,25 +440,65 @@ def sparse_decode_attention(cfg: LayerConfig, q: torch.Tensor, k_pool: torch.Ten
     return out
 
 
-def kv_store(cfg: LayerConfig, k: torch.Tensor, v: torch.Tensor, out_cache_loc: torch.Tensor,
+@dataclass
+class PagePool:
+    """Free pages of a paged KV pool (``ts_page_pool``): a stack of physical page
+    numbers on the device, ``free_pages[:free_count]`` being free and the top taken
+    first, plus the ticket word the store kernels count their workgroups in."""
+    free_pages: torch.Tensor   # [capacity] int32
+    free_count: torch.Tensor   # [1] int32
+    ticket: torch.Tensor       # [1] int32, zero between calls
+
+    @classmethod
+    def of(cls, pages: torch.Tensor):
+        """A pool whose free pages are ``pages`` (int32, on the device; the last one is
+        taken first)."""
+        _need(pages, "pages", torch.int32, 1)
+        return cls(pages.clone(), torch.tensor([pages.shape[0]], dtype=torch.int32, device=pages.device),
+                   torch.zeros((1,), dtype=torch.int32, device=pages.device))
+
+    def to_c(self) -> TsPagePool:
+        _need(self.free_pages, "free_pages", torch.int32, 1)
+        _need(self.free_count, "free_count", torch.int32, 1)
+        _need(self.ticket, "ticket", torch.int32, 1)
+        return TsPagePool(_p(self.free_pages), _p(self.free_count), _p(self.ticket))
+
+
+def _c_pages(cfg: LayerConfig, out_cache_loc, pages: Optional[PagePool]):
+    """(out_cache_loc pointer, ts_page_pool*) for the store entry points: the caller's
+    slots with a per-token table (the reference), or slots the library takes from the
+    table / the page pool."""
+    if pages is not None:
+        c_pool = pages.to_c()
+        return None, ctypes.byref(c_pool), c_pool
+    if cfg.page_size != 1:
+        raise ValueError(f"page_size {cfg.page_size} needs a PagePool")
+    _need(out_cache_loc, "out_cache_loc", torch.int32, 1)
+    return _p(out_cache_loc), None, None
+
+
+def kv_store(cfg: LayerConfig, k: torch.Tensor, v: torch.Tensor, out_cache_loc: Optional[torch.Tensor],
              k_pool: torch.Tensor, v_pool: torch.Tensor, table: torch.Tensor,
-             seq_lens: torch.Tensor) -> None:
-    """KV store + table append of a decode step (tr.py:844-854, 332-336)."""
+             seq_lens: torch.Tensor, pages: Optional[PagePool] = None) -> None:
+    """KV store + table append of a decode step (tr.py:844-854, 332-336): to the
+    caller's ``out_cache_loc`` (page size 1, the reference), or, with ``pages``, to the
+    next position of each request's paged table, fresh pages coming from the pool."""
     c = cfg.to_c()
     _need(k, "k", torch.bfloat16)
     _need(v, "v", torch.bfloat16)
-    _need(out_cache_loc, "out_cache_loc", torch.int32, 1)
+    loc, pool, _keep = _c_pages(cfg, out_cache_loc, pages)
     _check_pool(cfg, k_pool, "k_pool")
     _check_pool(cfg, v_pool, "v_pool")
     _need(table, "table", torch.int32, 2)
     _need(seq_lens, "seq_lens", torch.int32, 1)
-    B = out_cache_loc.shape[0]
+    B = seq_lens.shape[0]
     row = cfg.num_kv_heads * cfg.head_dim
-    if k.numel() != B * row or v.numel() != B * row or table.shape[0] != B or seq_lens.shape[0] != B:
-        raise ValueError("k / v / table / seq_lens do not match the batch")
-    _lib.check(_lib.load().ts_kv_store(ctypes.byref(c), _p(k), _p(v), _p(out_cache_loc), _p(k_pool),
+    if k.numel() != B * row or v.numel() != B * row or table.shape[0] != B or \
+            (pages is None and out_cache_loc.shape[0] != B):
+        raise ValueError("k / v / out_cache_loc / table / seq_lens do not match the batch")
+    _lib.check(_lib.load().ts_kv_store(ctypes.byref(c), _p(k), _p(v), loc, pool, _p(k_pool),
                                        _p(v_pool), k_pool.shape[0], _p(table), table.stride(0),
-                                       _p(seq_lens), B, table.shape[1], _stream()))
+                                       _p(seq_lens), B, table.shape[1] * cfg.page_size, _stream()))
 
 
 QKV_STORE_MAX_BATCH = 8
@@ -470,20 +510,21 @@ def qkv_store_supported(batch: int, hidden: int) -> bool:
 
 
 def qkv_store(cfg: LayerConfig, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
-              out_cache_loc: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+              out_cache_loc: Optional[torch.Tensor], k_pool: torch.Tensor, v_pool: torch.Tensor,
               table: torch.Tensor, seq_lens: torch.Tensor,
-              q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+              q_out: Optional[torch.Tensor] = None, pages: Optional[PagePool] = None) -> torch.Tensor:
     """QKV projection of a decode step with the KV store + table append as its epilogue
     (the model's ``qkv_proj`` followed by tr.py:844-854, 332-336) in one pass over the
     weight.  ``x`` [B, hidden] bf16, ``weight`` [(H+2Hkv)*D, hidden] bf16 (a torch
     ``Linear`` weight), ``bias`` [(H+2Hkv)*D] bf16 or None.  Returns ``q`` [B, H*D] bf16;
-    K and V land in the pools at ``out_cache_loc``."""
+    K and V land in the pools at ``out_cache_loc`` or, with ``pages``, where
+    :func:`kv_store` would put them."""
     c = cfg.to_c()
     _need(x, "x", torch.bfloat16, 2)
     _need(weight, "weight", torch.bfloat16, 2)
     if bias is not None:
         _need(bias, "bias", torch.bfloat16, 1)
-    _need(out_cache_loc, "out_cache_loc", torch.int32, 1)
+    loc, pool, _keep = _c_pages(cfg, out_cache_loc, pages)
     _check_pool(cfg, k_pool, "k_pool")
     _check_pool(cfg, v_pool, "v_pool")
     _need(table, "table", torch.int32, 2)
@@ -492,7 +533,7 @@ def qkv_store(cfg: LayerConfig, x: torch.Tensor, weight: torch.Tensor, bias: Opt
     n_out = (cfg.num_heads + 2 * cfg.num_kv_heads) * cfg.head_dim
     if tuple(weight.shape) != (n_out, hidden) or (bias is not None and bias.shape[0] != n_out):
         raise ValueError(f"weight must be [{n_out}, {hidden}] (and bias [{n_out}])")
-    if out_cache_loc.shape[0] != B or table.shape[0] != B or seq_lens.shape[0] != B:
+    if (pages is None and out_cache_loc.shape[0] != B) or table.shape[0] != B or seq_lens.shape[0] != B:
         raise ValueError("out_cache_loc / table / seq_lens do not match the batch")
     if k_pool.shape != v_pool.shape:
         raise ValueError("k_pool and v_pool must have the same shape")
@@ -503,9 +544,9 @@ def qkv_store(cfg: LayerConfig, x: torch.Tensor, weight: torch.Tensor, bias: Opt
         if tuple(q_out.shape) != (B, cfg.num_heads * cfg.head_dim):
             raise ValueError("q_out must be [B, H*D]")
     _lib.check(_lib.load().ts_qkv_store(
-        ctypes.byref(c), _p(x), _p(weight), _p(bias), hidden, _p(out_cache_loc), _p(q_out), _p(k_pool),
-        _p(v_pool), k_pool.shape[0], _p(table), table.stride(0), _p(seq_lens), B, table.shape[1],
-        _stream()))
+        ctypes.byref(c), _p(x), _p(weight), _p(bias), hidden, loc, pool, _p(q_out), _p(k_pool),
+        _p(v_pool), k_pool.shape[0], _p(table), table.stride(0), _p(seq_lens), B,
+        table.shape[1] * cfg.page_size, _stream()))
     return q_out
 
 
@@ -586,26 +627,31 @@ def rope_tables(head_dim: int, rope_base: float, rope_scale, rows: int, device):
     return emb.cos().to(device).contiguous(), emb.sin().to(device).contiguous()
 
 
-def kv_store_chunk(cfg: LayerConfig, k: torch.Tensor, v: torch.Tensor, out_cache_loc: torch.Tensor,
-                   k_pool: torch.Tensor, v_pool: torch.Tensor, table_row: torch.Tensor,
-                   seq_len: torch.Tensor) -> None:
+def kv_store_chunk(cfg: LayerConfig, k: torch.Tensor, v: torch.Tensor,
+                   out_cache_loc: Optional[torch.Tensor], k_pool: torch.Tensor, v_pool: torch.Tensor,
+                   table_row: torch.Tensor, seq_len: torch.Tensor,
+                   pages: Optional[PagePool] = None) -> None:
     """KV store + table append of a prefill chunk of one request (tr.py:725-733,
-    332-336): ``table_row`` [max_tokens] int32, ``seq_len`` a one-element int32 tensor."""
+    332-336): ``table_row`` [pages of the request] int32, ``seq_len`` a one-element int32
+    tensor; slots from ``out_cache_loc`` (page size 1) or, with ``pages``, from the table
+    and the page pool."""
     c = cfg.to_c()
     _need(k, "k", torch.bfloat16)
     _need(v, "v", torch.bfloat16)
-    _need(out_cache_loc, "out_cache_loc", torch.int32, 1)
+    loc, pool, _keep = _c_pages(cfg, out_cache_loc, pages)
     _check_pool(cfg, k_pool, "k_pool")
     _check_pool(cfg, v_pool, "v_pool")
     _need(table_row, "table_row", torch.int32, 1)
     _need(seq_len, "seq_len", torch.int32)
-    rows = out_cache_loc.shape[0]
     row = cfg.num_kv_heads * cfg.head_dim
-    if k.numel() != rows * row or v.numel() != rows * row or seq_len.numel() != 1:
-        raise ValueError("k / v / seq_len do not match the chunk")
-    _lib.check(_lib.load().ts_kv_store_chunk(ctypes.byref(c), _p(k), _p(v), _p(out_cache_loc), rows,
+    rows = k.numel() // row
+    if k.numel() != rows * row or v.numel() != rows * row or seq_len.numel() != 1 or \
+            (pages is None and out_cache_loc.shape[0] != rows):
+        raise ValueError("k / v / out_cache_loc / seq_len do not match the chunk")
+    _lib.check(_lib.load().ts_kv_store_chunk(ctypes.byref(c), _p(k), _p(v), loc, pool, rows,
                                              _p(k_pool), _p(v_pool), k_pool.shape[0], _p(table_row),
-                                             _p(seq_len), table_row.shape[0], _stream()))
+                                             _p(seq_len), table_row.shape[0] * cfg.page_size,
+                                             _stream()))
 
 
 def fingerprint(cfg: LayerConfig, q: torch.Tensor, cos_table: torch.Tensor,

@@ -33,6 +33,7 @@ class Workload:
     k_list: List[int]
     k_per_req: Optional[torch.Tensor] = None
     planted: List[torch.Tensor] = field(default_factory=list)  # per request: logical positions
+    free_pages: Optional[torch.Tensor] = None   # [extra_pages] int32: pages no request holds
 
     @property
     def batch(self) -> Batch:
@@ -128,7 +129,7 @@ def build(name: str, shape: dict, seq_lens: List[int], k_list: List[int], page_s
     if any(k != cfg.top_k for k in k_list):
         k_dev = torch.tensor(k_list, dtype=torch.int32, device=device)
     return Workload(name, cfg, q, k_pool, v_pool, table, list(seq_lens), seq_dev, list(k_list),
-                    k_dev, planted)
+                    k_dev, planted, order[at:].to(torch.int32).contiguous())
 
 
 def config1(device, seed: int = 0, seq_len: int = 32768, top_k: int = 2048) -> Workload:
@@ -156,10 +157,12 @@ def config3(device, seed: int = 2, batch: int = 16, lo: int = 4096, hi: int = 13
 
 
 def config4(device, seed: int = 3, batch: int = 4, seq_len: int = 65536, steps: int = 64,
-            top_k: int = 2048) -> Workload:
-    """Selection-cache trace base: per-token tables with room for ``steps`` appended tokens."""
-    return build("C4 llama3-8b B%d L%d trace" % (batch, seq_len), LLAMA3_8B, [seq_len] * batch,
-                 [top_k] * batch, 1, device, seed, extra_pages=batch * steps)
+            top_k: int = 2048, page_size: int = 1) -> Workload:
+    """Selection-cache trace base: tables (per token, or pages of ``page_size`` tokens)
+    with free pages for ``steps`` appended tokens per request."""
+    extra = batch * (-(-steps // page_size) + 1)
+    return build("C4 llama3-8b B%d L%d trace page%d" % (batch, seq_len, page_size), LLAMA3_8B,
+                 [seq_len] * batch, [top_k] * batch, page_size, device, seed, extra_pages=extra)
 
 
 def config5_layer(device, seed: int = 4, batch: int = 4, seq_len: int = 262144,
