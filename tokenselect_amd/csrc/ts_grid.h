@@ -125,6 +125,24 @@ __device__ __forceinline__ void grid_arrive(uint32_t* sync, uint32_t round, bool
   __syncthreads();
 }
 
+// One lane waits until the 64-bit word at `p` is no longer zero and returns it; 0 when
+// the wait ran into its bound (the fault word is then set) or another one did.
+__device__ __forceinline__ uint64_t poll_nonzero(const uint64_t* p, uint32_t* sync, uint64_t ticks) {
+  const uint64_t t0 = wall_clock64();
+  for (uint32_t polls = 1;; ++polls) {
+    const uint64_t v = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (v != 0ull) return v;
+    if ((polls & 15u) == 0) {
+      if (load_coherent(&sync[0]) != 0u) return 0ull;
+      if (wall_clock64() - t0 > ticks) {
+        __hip_atomic_store(&sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return 0ull;
+      }
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+
 // The second half of a rendezvous for a workgroup that arrived without waiting and
 // did other work in the meantime.
 __device__ __forceinline__ void grid_wait(uint32_t* sync, uint32_t round, uint64_t ticks,

@@ -27,7 +27,9 @@ struct ScoreArgs {
   int head_map;
   // Fused selection only.
   uint32_t* sync;         // rendezvous area (ts_grid.h), live words zero at launch
-  float* stats;           // [B,H,2] merged (max, sum exp), by head
+  float* stats;           // [kSyncSlots replicas][stats_stride]: [B,H,2] merged (max, sum exp), by
+                          // head, zero at launch
+  int64_t stats_stride;   // floats between replicas
   float* votes;           // [B,vote_stride] copy of the votes, or NULL
   int64_t vote_stride;
   uint32_t* counters;     // [B][kSelCounterWords] zero at launch
@@ -74,7 +76,8 @@ constexpr int kSelCounterWords = kSelListCount + kSelListParts * 32;
 
 // Workspace of ts_select, carved in this order (256-byte aligned pieces).
 struct SelectWorkspace {
-  size_t partials, stats, counters, block_counts, short_list, pool_votes, sync, total;  // sync stays last
+  size_t partials, counters, stats, block_counts, short_list, pool_votes, sync, total;  // sync stays last
+  int64_t stats_stride;
   int64_t pool_stride;
   int tokens_per_block;  // 0: the shape does not fit the fused kernel
   int blocks_per_req;

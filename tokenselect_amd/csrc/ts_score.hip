@@ -82,9 +82,12 @@ constexpr int kQuadSwap2 = 0x4E;  // quad_perm [2,3,0,1]
 constexpr int kScoreDirect = 0, kScoreTiled = 1, kScoreFused = 2;
 constexpr int kMaxHeads = 128;
 
-// Between the two rendezvous of the fused kernel: the (request, head) pairs are
-// dealt out over all wavefronts of the grid; a wavefront merges the per-workgroup
-// (max, sum exp) of its pair, a lane per chunk, in a fixed order.
+// After the first rendezvous of the fused kernel: the (request, head) pairs are dealt
+// out over all wavefronts of the grid; a wavefront merges the per-workgroup (max, sum
+// exp) of its pair, a lane per chunk, in a fixed order, and writes the result into 64
+// replicas, lane r into replica r.  The workgroups poll the words of the replica of
+// their index until they are there (a sum of exponentials is never zero): the data is
+// its own flag, which saves a rendezvous.
 __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const GridTeam& team,
                                                     int lane, int wave) {
   const int H = a.num_heads;
@@ -113,11 +116,11 @@ __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const Gr
     row16_softmax_merge(m, l);
     softmax_merge(m, l, __shfl_xor(m, 16), __shfl_xor(l, 16));
     softmax_merge(m, l, __shfl_xor(m, 32), __shfl_xor(l, 32));
-    if (lane == 0) store_coherent((float2*)a.stats + (size_t)b * H + h, m, l);
+    store_coherent((float2*)(a.stats + (size_t)lane * a.stats_stride) + (size_t)b * H + h, m, l);
   }
 }
 
-constexpr uint32_t kSelectRounds = 6;  // rendezvous of the fused kernel
+constexpr uint32_t kSelectRounds = 5;  // rendezvous of the fused kernel
 
 // The workgroups that take part in the rendezvous of the fused kernel: all those of
 // the requests that select (neither dense nor served by the selection cache).  The
@@ -528,7 +531,6 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     if (tid < 16) scratch[tid] = 0u;
     grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
     merge_request_stats(a, team, lane, wave);
-    grid_arrive(a.sync, 2, false, a.spin_ticks, team.size, team.index);
     // While the merged statistics are on their way: the exponentials, relative to this
     // workgroup's own maxima; exp(s - max) / sum = exp(s - own max) * exp(own max - max) / sum.
     const ReqGeom geo =
@@ -550,11 +552,13 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
           if (s0 + j < HKV * G) sc[(s0 + j) * 16] = __expf(x[j] - local_max[s0 + j]);
       }
     }
-    grid_wait(a.sync, 2, a.spin_ticks, team.index);
-    for (int slot = tid; slot < H; slot += 256) {
-      const int h = head_of<HKV, G>(slot / G, slot % G, a.head_map);
-      const float2 st = load_coherent((const float2*)a.stats + (size_t)b * H + h);
-      s_rz[slot] = __expf(local_max[slot] - st.x) / st.y;
+    if (tid < H) {  // H <= kMaxHeads < 256
+      const int h = head_of<HKV, G>(tid / G, tid % G, a.head_map);
+      const uint64_t* rep = (const uint64_t*)(a.stats + (size_t)(team.index % kSyncSlots) * a.stats_stride) +
+                            (size_t)b * H + h;
+      const uint64_t st = poll_nonzero(rep, a.sync, a.spin_ticks);
+      const float mx = __uint_as_float((uint32_t)st), sum = __uint_as_float((uint32_t)(st >> 32));
+      s_rz[tid] = st ? __expf(local_max[tid] - mx) / sum : 0.f;  // 0: the wait gave up
     }
     __syncthreads();
 
@@ -576,7 +580,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       if (a.votes && a.pool_kernel <= 0) a.votes[(size_t)b * a.vote_stride + block_lo + i] = c;
       sc[0] = c;
     }
-    uint32_t round = 2;  // rendezvous passed so far
+    uint32_t round = 1;  // rendezvous passed so far
     if (a.pool_kernel > 0) {
       // Max-pool smoothing of the votes (tr.py:366-369): stride 1, padding (kernel-1)/2
       // with -inf, an even kernel makes the result one shorter.  The workgroups
@@ -1093,8 +1097,11 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
     return at;
   };
   w.partials = take(B * H * (size_t)ceil_div(max_seq_len, w.tokens_per_block) * 2 * sizeof(float));
-  w.stats = take(B * H * 2 * sizeof(float));
+  // The counters and, right behind them, the replicas of the statistics are cleared
+  // together before every launch.
   w.counters = take(B * kSelCounterWords * 4);
+  w.stats_stride = (int64_t)align_up(B * H * 2, 1024);
+  w.stats = take((size_t)kSyncSlots * w.stats_stride * sizeof(float));
   w.block_counts = take(B * (size_t)w.blocks_per_req * sizeof(uint2));
   w.short_list = take(B * kSelListParts * kSelListCap * sizeof(uint2));
   w.pool_stride = (int64_t)align_up((size_t)max_n, 64);
@@ -1107,9 +1114,9 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
 void select_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* counters,
                          ZeroRegion* sync) {
   counters->base = (uint32_t*)((char*)workspace + w.counters);
-  counters->stride = kSelCounterWords;
-  counters->words = kSelCounterWords;
-  counters->count = batch;
+  counters->words = (int)((w.stats - w.counters) / 4 + (size_t)kSyncSlots * w.stats_stride);
+  counters->stride = counters->words;
+  counters->count = 1;
   sync->base = (uint32_t*)((char*)workspace + w.sync);
   sync->stride = kSyncSlotWords;
   sync->words = kSyncLiveWords;
@@ -1163,6 +1170,7 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
                                w.tokens_per_block);
   a.sync = (uint32_t*)(ws + w.sync);
   a.stats = (float*)(ws + w.stats);
+  a.stats_stride = w.stats_stride;
   a.votes = votes;
   a.vote_stride = vote_stride;
   a.counters = (uint32_t*)(ws + w.counters);
