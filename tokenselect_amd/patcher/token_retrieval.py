@@ -520,7 +520,24 @@ def patch_input_metadata():
             return ret
 
     found[1].InputMetadata = PatchedInputMetadata
+    found[1].update_flashinfer_indices = patched_forward_batch_info_update_flashinfer_indices
     return PatchedInputMetadata
+
+
+def patched_forward_batch_info_update_flashinfer_indices(
+        forward_mode, model_runner, req_pool_indices, seq_lens, prefix_lens,
+        flashinfer_decode_wrapper=None, flashinfer_use_ragged=False):
+    """Stands in for the function the reference installs as
+    ``forward_batch_info.update_flashinfer_indices`` (tr.py:570-655), with its signature
+    and the configurations it refuses (tr.py:589, 635, 650).  The reference rebuilds the
+    dense ``kv_indptr`` / ``kv_indices`` on the host here and re-plans the FlashInfer
+    wrappers; the library plans its split-K schedule on the device from ``sel_len``, so
+    nothing is left to do."""
+    if getattr(model_runner, "sliding_window_size", None) is not None:
+        raise NotImplementedError("Sliding window not supported yet")
+    if flashinfer_use_ragged:
+        raise NotImplementedError("Ragged attention not supported yet")
+    return None
 
 
 def patch_model():
