@@ -150,3 +150,19 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libtokenselect_hip.so"))
     with pytest.raises(ImportError, match="no CPU fallback"):
         _lib.load()
+
+
+def test_workspace_sizes_never_shrink_with_the_context_or_the_batch(lib):
+    """A workspace sized for (batch, max_seq_len) must serve every smaller batch and every
+    shorter context: the candidates per workgroup move in steps, so the sizes are taken
+    from bounds that do not."""
+    for heads, kv in ((32, 8), (28, 4), (8, 1)):
+        c = cfg(num_heads=heads, num_kv_heads=kv)
+        lens = list(range(700, 70000, 997)) + [32768, 32769, 131072, 131073, 262144, 262145, 1048576]
+        for fn in (lib.ts_decode_layer_workspace_bytes, lib.ts_score_partials_bytes,
+                   lib.ts_select_workspace_bytes, lib.ts_topk_workspace_bytes):
+            sizes = [fn(ctypes.byref(c), 4, L) for L in sorted(lens)]
+            assert all(x > 0 for x in sizes)
+            assert sizes == sorted(sizes), fn.__name__
+        by_batch = [lib.ts_decode_layer_workspace_bytes(ctypes.byref(c), B, 65536) for B in range(1, 33)]
+        assert by_batch == sorted(by_batch)

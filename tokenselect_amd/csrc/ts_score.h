@@ -74,6 +74,10 @@ constexpr int kSelListParts = 8;
 constexpr int kSelListCount = kSelMaxBin + kSelHistCopies * 32;
 constexpr int kSelCounterWords = kSelListCount + kSelListParts * 32;
 
+// Workgroups of one request the workspace of ts_select is laid out for (the device keeps
+// some 510 resident at once).
+constexpr int kSelMaxChunks = 1024;
+
 // Workspace of ts_select, carved in this order (256-byte aligned pieces).
 struct SelectWorkspace {
   size_t partials, counters, stats, block_counts, short_list, pool_votes, sync, total;  // sync stays last

@@ -30,6 +30,7 @@
 // ahead.
 #include <stdlib.h>
 
+#include <algorithm>
 #include <atomic>
 
 #include "ts_score.h"
@@ -1080,15 +1081,19 @@ int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, boo
   while ((int64_t)ceil_div(max_n, tpb) * batch > capacity) tpb += 64;
   if (fused_lds_bytes(tpb, cfg->num_heads) > kFusedStageBytes)
     return 0;
+  if (ceil_div(max_seq_len, tpb) > kSelMaxChunks) return 0;  // what the workspace is laid out for
   return tpb;
 }
 
 SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch) {
   SelectWorkspace w{};
+  // The layout depends on the batch, the head count and (for the pooled votes) the
+  // length, not on how the candidates are dealt out, and is the same whether or not
+  // this shape is served: a workspace sized for the longest context serves every
+  // shorter one.
   w.tokens_per_block = fused_tokens_per_block(cfg, batch, max_seq_len, ignore_switch);
-  if (w.tokens_per_block <= 0) return w;
-  const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
-  w.blocks_per_req = (int)ceil_div(max_n, w.tokens_per_block);
+  const int max_n = std::max(max_seq_len - cfg->n_init - cfg->n_local, 0);
+  w.blocks_per_req = w.tokens_per_block > 0 ? (int)ceil_div(max_n, w.tokens_per_block) : 0;
   const size_t B = (size_t)batch, H = (size_t)cfg->num_heads;
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -1096,15 +1101,15 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
     off += align_up(bytes, 256);
     return at;
   };
-  w.partials = take(B * H * (size_t)ceil_div(max_seq_len, w.tokens_per_block) * 2 * sizeof(float));
+  w.partials = take(B * H * (size_t)kSelMaxChunks * 2 * sizeof(float));
   // The counters and, right behind them, the replicas of the statistics are cleared
   // together before every launch.
   w.counters = take(B * kSelCounterWords * 4);
   w.stats_stride = (int64_t)align_up(B * H * 2, 1024);
   w.stats = take((size_t)kSyncSlots * w.stats_stride * sizeof(float));
-  w.block_counts = take(B * (size_t)w.blocks_per_req * sizeof(uint2));
+  w.block_counts = take(B * (size_t)kSelMaxChunks * sizeof(uint2));
   w.short_list = take(B * kSelListParts * kSelListCap * sizeof(uint2));
-  w.pool_stride = (int64_t)align_up((size_t)max_n, 64);
+  w.pool_stride = (int64_t)align_up((size_t)std::max(max_n, 1), 64);
   w.pool_votes = take(cfg->pool_kernel > 0 ? B * (size_t)w.pool_stride * sizeof(float) : 0);
   w.sync = take(kSyncWords * 4);
   w.total = off;
@@ -1216,8 +1221,12 @@ int ts_set_fused_select(int enable) { return set_fused_select(enable); }
 
 size_t ts_score_partials_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
-  const int tpb = score_tokens_per_block((int64_t)batch * max_seq_len, cfg->num_heads);
-  const size_t nchunks = (size_t)ceil_div(max_seq_len, tpb);
+  // A bound that never shrinks when max_seq_len grows, unlike the number of workgroups
+  // itself (the candidates per workgroup move in steps of 64), so that a buffer sized
+  // for the longest context serves every shorter one: 512 workgroups are aimed at, more
+  // only once a workgroup holds as many candidates as its LDS takes.
+  const int64_t cap = std::max<int64_t>((16384 / cfg->num_heads) / 64 * 64, 64);
+  const size_t nchunks = (size_t)std::max<int64_t>(520, ceil_div(max_seq_len, cap) + 8);
   return align_up((size_t)batch * cfg->num_heads * nchunks * 2 * sizeof(float), 256);
 }
 

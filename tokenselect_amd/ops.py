@@ -267,6 +267,17 @@ def score(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
     return scores, partials
 
 
+def score_buffers(cfg: LayerConfig, bt: Batch, device):
+    """``(scores, partials)`` for :func:`score`'s ``out``, sized for ``bt.max_seq_len``
+    (serves every shorter batch of the same size)."""
+    c = cfg.to_c()
+    stride = score_stride_for(bt.max_seq_len)
+    scores = torch.empty((bt.batch, stride // 16, cfg.num_heads, 16), dtype=torch.float32, device=device)
+    nbytes = _lib.load().ts_score_partials_bytes(ctypes.byref(c), bt.batch, bt.max_seq_len)
+    partials = torch.empty((max(nbytes, 256) // 4,), dtype=torch.float32, device=device)
+    return scores, partials
+
+
 def select_supported(cfg: LayerConfig, batch: int, max_seq_len: int) -> bool:
     """Whether :func:`select` can serve this shape (``ts_select_supported``)."""
     return bool(_lib.load().ts_select_supported(ctypes.byref(cfg.to_c()), int(batch),

@@ -303,9 +303,29 @@ class TokenRetriever:
                        self.token_indices[layer_id:layer_id + 1], current_num_tokens)
         cache = self._cache(layer_id)
         hit = ops.selcache_step(cfg, bt, qf, cache) if cache is not None else None
-        scores, partials = ops.score(cfg, bt, qf, self.token_fingerprints[layer_id], skip=hit)
-        votes, _ = ops.vote(cfg, bt, scores, partials, skip=hit)
-        sel, _, _ = ops.topk_ragged(cfg, bt, votes, hit=hit, cache=cache)
+        k_buffer = self.token_fingerprints[layer_id]
+        # The large buffers are kept between calls, sized for the longest table.
+        key = ("select", n_init, n_local, topk, KERNEL_SIZE)
+        sized = ops.Batch(bt.seq_lens, bt.table, self.max_num_tokens)
+        if ops.select_supported(cfg, 1, self.max_num_tokens):
+            # the whole selection in one launch
+            held = self._layers.get(key)
+            if held is None:
+                held = (ops.select_workspace(cfg, sized, self.device), ops.fault_word())
+                self._layers[key] = held
+            workspace, fault = held
+            ops.raise_if_gave_up(fault)
+            bt.fault = fault
+            sel, _, _, _, _ = ops.select(cfg, bt, qf, k_buffer, hit=hit, cache=cache,
+                                         workspace=workspace)
+        else:
+            held = self._layers.get(key)
+            if held is None:
+                held = ops.score_buffers(cfg, sized, self.device)
+                self._layers[key] = held
+            scores, partials = ops.score(cfg, bt, qf, k_buffer, skip=hit, out=held)
+            votes, _ = ops.vote(cfg, bt, scores, partials, skip=hit)
+            sel, _, _ = ops.topk_ragged(cfg, bt, votes, hit=hit, cache=cache)
         if cache is not None:
             self.is_first_query[layer_id] = False
         return sel[0, : n_init + topk + n_local]
