@@ -164,6 +164,23 @@ int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
             int64_t score_stride, const float* partials, const int32_t* skip, float* stats,
             float* votes, float* pooled, int64_t vote_stride, ts_stream_t stream);
 
+/* ts_score + ts_vote without the [H, n] scores in memory (tr.py:350-361): the
+ * requests are served in groups whose fp32 scores fit the LDS of the device, one
+ * launch per group in which the workgroups meet once to merge the softmax
+ * statistics (twice with cfg->pool_kernel > 0) and then write the votes; a batch of
+ * any size is served as long as one request fits (some 260K candidates for 32
+ * heads) and pool_kernel is at most 256 (ts_score_vote_supported).  votes
+ * [B, vote_stride] fp32 receives what ts_vote's votes (pooled with pool_kernel > 0)
+ * would hold, up to the last bit of an fp32 sum taken in another order.  workspace:
+ * ts_select_workspace_bytes().  The launches are ordinary ones whose workgroups must
+ * be resident together, as for ts_select, with the same bounded waits; a wait that
+ * gave up sets *bt->fault and the workspace's fault word (ts_select).
+ * No counterpart in the reference, which materialises the scores. */
+int ts_score_vote_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+int ts_score_vote(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+                  int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
+                  void* workspace, size_t workspace_bytes, ts_stream_t stream);
+
 /* Ragged top-k + sort + index assembly (tr.py:371-373, 433-449).  Per request:
  * the k_b largest votes (ties: lowest position first), ascending, offset by
  * n_init, between the n_init sink positions and the n_local newest positions;
@@ -204,7 +221,7 @@ int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
  * every request that was selecting (the other outputs of those requests are
  * not valid; ts_sparse_decode_attn treats a negative length as an empty list),
  * *bt->fault = 1 when bt->fault is given, and the first 32-bit word of the
- * last 65 * 4096 bytes of the workspace is 1 until the next clearing.  A
+ * last batch * 65 * 4096 bytes of the workspace is 1 until the next clearing.  A
  * caller that sees it reruns the step with the separate kernels.
  * No counterpart in the reference, which materialises every intermediate. */
 int ts_select_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
@@ -375,8 +392,10 @@ int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, in
  * cache may be NULL (QUERY_CACHE=False as released, tr.py:918).
  *
  * When ts_select_supported() holds, the selection runs as the single ts_select
- * kernel; otherwise ts_score, ts_vote and ts_topk_ragged run as they do on
- * their own.  Both forms give the same selection.
+ * kernel; a larger batch is scored and voted on in groups of requests as by
+ * ts_score_vote and then ranked by the kernels of ts_topk_ragged; where not even one
+ * request fits, ts_score, ts_vote and ts_topk_ragged run as they do on their own.
+ * All forms give the same selection.
  * ts_set_fused_select(0) forces the separate kernels for the calling process
  * (1 restores the default); it returns the previous setting and has no
  * counterpart in the reference. */
@@ -387,6 +406,29 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
                     int64_t pool_rows, const ts_selcache* cache, void* out, int32_t* sel,
                     int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
                     size_t workspace_bytes, ts_stream_t stream);
+
+/* ts_decode_layer split at the vote, for tensor parallelism (tr.py:361-364: every rank
+ * scores its own heads, the ranks add up their partial votes with one all-reduce, and
+ * all then select the same tokens): ts_decode_layer_votes runs fingerprint ->
+ * [selection cache] -> score -> per-head softmax -> sum over this rank's heads and
+ * leaves the un-pooled votes in votes [B, vote_stride] fp32 (requests that are dense
+ * or hit the cache are not written); the caller adds the ranks' votes in place (an
+ * all-reduce(SUM) over xGMI; nothing to do on one rank); ts_decode_layer_attend runs
+ * [max-pool, tr.py:366-369] -> top-k -> assembly -> sparse attention over this rank's
+ * heads.  Both calls take the same cfg (this rank's num_heads / num_kv_heads), batch,
+ * cache and workspace (ts_decode_layer_workspace_bytes; the hit flags of the cache
+ * travel in it).  On one rank the two calls give what ts_decode_layer gives.
+ * The selection cache compares this rank's slice of the query, so ranks may disagree
+ * on a hit: use it with one rank only. */
+int ts_decode_layer_votes(const ts_config* cfg, const ts_batch* bt, const void* q, const float* q_cos,
+                          const float* q_sin, const void* k_pool, int64_t pool_rows,
+                          const ts_selcache* cache, float* votes, int64_t vote_stride,
+                          void* workspace, size_t workspace_bytes, ts_stream_t stream);
+int ts_decode_layer_attend(const ts_config* cfg, const ts_batch* bt, const void* q, const float* votes,
+                           int64_t vote_stride, const void* k_pool, const void* v_pool,
+                           int64_t pool_rows, const ts_selcache* cache, void* out, int32_t* sel,
+                           int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
+                           size_t workspace_bytes, ts_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -39,6 +39,8 @@ def _votes_on_device(wl):
     qf = ops.rope_apply(wl.q.view(B, c.num_heads, c.head_dim), cos, sin, None)
     if ops.select_supported(c, B, bt.max_seq_len):
         return ops.select(c, bt, qf, wl.k_pool, want_votes=True)[3], qf
+    if ops.score_vote_supported(c, B, bt.max_seq_len):
+        return ops.score_vote(c, bt, qf, wl.k_pool), qf
     scores, partials = ops.score(c, bt, qf, wl.k_pool)
     return ops.vote(c, bt, scores, partials)[0], qf
 

@@ -669,3 +669,88 @@ def test_kv_store(dev):
     assert table[0, 100].item() == loc[0].item() and table[1, 50].item() == loc[1].item()
     assert torch.equal(wl.k_pool[loc[0].item()].reshape(-1), k[0])
     assert torch.equal(wl.v_pool[loc[1].item()].reshape(-1), v[1])
+
+
+@pytest.mark.parametrize("pool_kernel", [-1, 6])
+def test_score_vote_in_groups_of_requests(dev, pool_kernel):
+    """ts_score_vote (scores never in memory, the batch served in groups of requests)
+    against the oracle's votes and against ts_score + ts_vote; ragged, with a dense
+    request and a skipped one."""
+    lens, ks = [3000, 777, 40, 1531, 2048, 900], [64] * 6
+    say(f"score_vote lens={lens} pool={pool_kernel}")
+    wl = small(dev, SHAPES[0], seed=41, lens=lens, ks=ks, page=16, top_k=64, pool_kernel=pool_kernel)
+    c = wl.cfg
+    assert ops.score_vote_supported(c, len(lens), max(lens))
+    qf = fingerprint(wl, dev)
+    skip = torch.tensor([0, 0, 0, 1, 0, 0], dtype=torch.int32, device=dev)
+    details = []
+    oracle_layer(wl, details)
+    votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool, skip=skip), skip=skip)
+    votes = ops.score_vote(c, wl.batch, qf, wl.k_pool, skip=skip)
+    torch.cuda.synchronize()
+    for b, L in enumerate(lens):
+        if not details[b] or b == 3:
+            continue
+        n = L - c.n_init - c.n_local
+        if pool_kernel > 0 and pool_kernel % 2 == 0:
+            n -= 1
+        ref = details[b]["votes"][:n]
+        got = votes[b, :n].cpu()
+        assert (got - ref).abs().max().item() <= 2e-4 * ref.abs().max().item(), f"b={b}"
+        assert (got - votes_sep[b, :n].cpu()).abs().max().item() <= 1e-5 * ref.abs().max().item()
+
+
+@pytest.mark.parametrize("pool_kernel", [-1, 5])
+@pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
+def test_layer_split_at_the_vote(dev, fused_select, pool_kernel):
+    """ts_decode_layer_votes + ts_decode_layer_attend give what ts_decode_layer gives; and two
+    ranks that hold half of the heads each select, from the sum of their votes, what one
+    rank with all heads selects (tr.py:361-364), each attending with its own heads."""
+    lens, ks = [2500, 100, 1800], [128, 128, 100]
+    say(f"layer split at the vote, fused={fused_select} pool={pool_kernel}")
+    wl = small(dev, SHAPES[0], seed=43, lens=lens, ks=ks, page=16, top_k=128, n_init=16, n_local=32,
+               pool_kernel=pool_kernel)
+    c, B = wl.cfg, 3
+    c.head_map = "div"      # a rank holds whole GQA groups: heads [r*H/2, (r+1)*H/2) and their KV heads
+    whole = ops.DecodeLayer(c, B, max(lens), dev)
+    out, sel, sel_pos, sel_len = [t.clone() for t in whole(wl.q, wl.k_pool, wl.v_pool, wl.batch)]
+    halves = ops.DecodeLayer(c, B, max(lens), dev)
+    votes = halves.votes(wl.q, wl.k_pool, wl.batch)
+    out2, sel2, pos2, len2 = halves.attend(wl.q, votes, wl.k_pool, wl.v_pool, wl.batch)
+    torch.cuda.synchronize()
+    assert torch.equal(sel_len, len2)
+    for b in range(B):
+        S = int(sel_len[b])
+        assert torch.equal(sel[b, :S], sel2[b, :S]) and torch.equal(sel_pos[b, :S], pos2[b, :S])
+    assert (out.float() - out2.float()).abs().max().item() <= 1e-3
+    # two ranks
+    H, Hkv, D = c.num_heads, c.num_kv_heads, c.head_dim
+    import copy
+    rc = copy.copy(c)
+    rc.num_heads, rc.num_kv_heads = H // 2, Hkv // 2
+    ranks = []
+    for r in range(2):
+        q_r = wl.q.view(B, H, D)[:, r * H // 2:(r + 1) * H // 2].contiguous().view(B, -1)
+        k_r = wl.k_pool[:, r * Hkv // 2:(r + 1) * Hkv // 2].contiguous()
+        v_r = wl.v_pool[:, r * Hkv // 2:(r + 1) * Hkv // 2].contiguous()
+        layer = ops.DecodeLayer(rc, B, max(lens), dev)
+        ranks.append((layer, q_r, k_r, v_r, layer.votes(q_r, k_r, wl.batch).clone()))
+    total = ranks[0][4] + ranks[1][4]               # the all-reduce
+    details = []
+    oracle_layer(wl, details) if False else None
+    for r, (layer, q_r, k_r, v_r, _) in enumerate(ranks):
+        out_r, sel_r, pos_r, len_r = layer.attend(q_r, total, k_r, v_r, wl.batch)
+        torch.cuda.synchronize()
+        assert torch.equal(len_r, sel_len)
+        for b in range(B):
+            S = int(sel_len[b])
+            same = torch.equal(pos_r[b, :S], sel_pos[b, :S])
+            if not same:   # the sum over heads in another order may move a tie at the k-th vote
+                n = lens[b] - c.n_init - c.n_local
+                v = total[b, :n].cpu()
+                assert_index_sets_match(pos_r[b, c.n_init:S - c.n_local].cpu(),
+                                        sel_pos[b, c.n_init:S - c.n_local].cpu().long(), v, c.n_init,
+                                        f"rank {r} b={b}") if pool_kernel <= 0 else None
+            else:
+                want = out.view(B, H, D)[b, r * H // 2:(r + 1) * H // 2].reshape(-1).float()
+                assert (out_r[b].float() - want).abs().max().item() <= 2e-2

@@ -64,6 +64,8 @@ SIGNATURES = {
     "ts_score_stride": (_i64, [_i32]),
     "ts_score": (_i32, [_CFG, _BT, _ptr, _ptr, _i64, _ptr, _ptr, _i64, _ptr, _size, _ptr]),
     "ts_vote": (_i32, [_CFG, _BT, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
+    "ts_score_vote_supported": (_i32, [_CFG, _i32, _i32]),
+    "ts_score_vote": (_i32, [_CFG, _BT, _ptr, _ptr, _i64, _ptr, _ptr, _i64, _ptr, _size, _ptr]),
     "ts_topk_workspace_bytes": (_size, [_CFG, _i32, _i32]),
     "ts_topk_ragged": (_i32, [_CFG, _BT, _ptr, _i64, _ptr, _SC, _ptr, _ptr, _i64, _ptr, _ptr,
                               _size, _ptr]),
@@ -97,6 +99,10 @@ SIGNATURES = {
                                 _ptr, _i64, _ptr, _ptr, _size, _ptr]),
     "ts_set_fused_select": (_i32, [_i32]),
     "ts_decode_layer_workspace_bytes": (_size, [_CFG, _i32, _i32]),
+    "ts_decode_layer_votes": (_i32, [_CFG, _BT, _ptr, _ptr, _ptr, _ptr, _i64, _SC, _ptr, _i64, _ptr,
+                                     _size, _ptr]),
+    "ts_decode_layer_attend": (_i32, [_CFG, _BT, _ptr, _ptr, _i64, _ptr, _ptr, _i64, _SC, _ptr, _ptr,
+                                      _ptr, _i64, _ptr, _ptr, _size, _ptr]),
     "ts_decode_layer": (_i32, [_CFG, _BT, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _SC, _ptr, _ptr,
                                _ptr, _i64, _ptr, _ptr, _size, _ptr]),
 }

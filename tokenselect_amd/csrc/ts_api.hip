@@ -196,24 +196,42 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
                                  sel_pos, sel_stride, sel_len, (uint32_t*)(ws + w.topk_ws));
   topk.clear = tickets;
   topk.clear_per_req = cfg->num_kv_heads;
-  ZeroRegion zero_counters, zero_sync;
-  if (one_launch)
+  // A batch too large for one launch of the selection: scores and votes still without
+  // the [H, n] scores in memory, one launch per request, then the top-k kernels on the
+  // votes.  Taken when a request of max_seq_len needs the device to itself (4 x 256K:
+  // 463 us per layer against 481 us): the grids are sized by max_seq_len, so with
+  // several requests per launch a ragged batch (16 x 4K..128K: 617 against 534 us)
+  // leaves most workgroups of a launch without tokens.
+  const int vote_group =
+      (!one_launch && max_n > 0 && cfg->pool_kernel <= 256 &&
+       score_votes_group(cfg, bt->batch, bt->max_seq_len) == 1) ? 1 : 0;
+  ZeroRegion zero_counters, zero_sync, zero_stats;
+  if (one_launch) {
     select_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_counters, &zero_sync);
-  else if (max_n > 0)
+  } else if (max_n > 0) {
     zero_counters = topk_zero_region(topk, bt->batch);
+    if (vote_group > 0) score_votes_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_stats, &zero_sync);
+  }
   if (chunk_rows > 0) {
     // Chunk fingerprint: row i rotated to n_local + i, mean over the rows (tr.py:380-392).
     TS_TRY(launch_fingerprint(cfg, q, chunk_rows, q_cos, q_sin, table_rows, qf, zero_counters,
-                              zero_sync, (hipStream_t)stream));
+                              zero_sync, (hipStream_t)stream, zero_stats));
   } else {
     TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
-                       zero_counters, zero_sync, (hipStream_t)stream));
+                       zero_counters, zero_sync, (hipStream_t)stream, zero_stats));
   }
   if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
   if (one_launch) {
     TS_TRY(launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,
                          nullptr, 0, ws + w.select_ws, tickets, cfg->num_kv_heads,
                          (hipStream_t)stream));
+  } else if (vote_group > 0) {
+    // With max-pooling the kernel writes the pooled votes (there is no un-pooled copy).
+    TS_TRY(launch_score_votes(cfg, bt, qf, k_pool, pool_rows, hit, votes, w.score_stride, topk.ws,
+                              topk.ws_stride, ws + w.select_ws, (hipStream_t)stream));
+    topk.votes = votes;
+    topk.fault = score_votes_fault_word(cfg, bt->batch, bt->max_seq_len, ws + w.select_ws);
+    TS_TRY(launch_topk(topk, bt->batch, max_n, (hipStream_t)stream, true, true));
   } else {
     float* partials = (float*)(ws + w.partials);
     TS_TRY(ts_score(cfg, bt, qf, k_pool, pool_rows, hit, scores, w.score_stride, partials,
@@ -241,6 +259,96 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
                     size_t workspace_bytes, ts_stream_t stream) {
   return run_layer(cfg, bt, q, 0, q_cos, q_sin, 1, k_pool, v_pool, pool_rows, cache, out, sel,
                    sel_pos, sel_stride, sel_len, workspace, workspace_bytes, stream);
+}
+
+// The layer split at the vote, for tensor parallelism (tr.py:361-364): every rank scores
+// its own heads and holds partial votes; the ranks add them up (one all-reduce of the
+// [B, vote_stride] votes, the caller's); every rank then selects the same tokens from
+// the summed votes and attends with its own heads.
+int ts_decode_layer_votes(const ts_config* cfg, const ts_batch* bt, const void* q, const float* q_cos,
+                          const float* q_sin, const void* k_pool, int64_t pool_rows,
+                          const ts_selcache* cache, float* votes, int64_t vote_stride,
+                          void* workspace, size_t workspace_bytes, ts_stream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_TRY(validate_batch(cfg, bt));
+  TS_REQUIRE(q && q_cos && q_sin && k_pool && votes, TS_EINVAL, "layer votes: NULL tensor argument");
+  TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
+             (long long)pool_rows);
+  const LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);
+  TS_REQUIRE(workspace != nullptr && workspace_bytes >= w.total, TS_EWORKSPACE,
+             "workspace %zu bytes < required %zu", workspace_bytes, w.total);
+  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
+  TS_REQUIRE(vote_stride >= max_n, TS_EWORKSPACE, "vote_stride %lld < max candidates %d",
+             (long long)vote_stride, max_n);
+  if (cache)
+    TS_REQUIRE(cache->q_cache && cache->topk_cache && cache->cache_len && cache->counters, TS_EINVAL,
+               "selection cache has a NULL array");
+  ts_config plain = *cfg;  // the max-pool comes after the ranks' votes are added up
+  plain.pool_kernel = -1;
+  char* ws = (char*)workspace;
+  void* qf = ws + w.qf;
+  int32_t* hit = cache ? (int32_t*)(ws + w.hit) : nullptr;
+  const SelectWorkspace fused = select_workspace(&plain, bt->batch, bt->max_seq_len);
+  const int group = max_n > 0 ? score_votes_group(&plain, bt->batch, bt->max_seq_len) : 0;
+  ZeroRegion zero_stats, zero_sync;
+  if (group > 0) score_votes_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_stats, &zero_sync);
+  TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
+                     zero_stats, zero_sync, (hipStream_t)stream));
+  if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
+  if (max_n <= 0) return TS_OK;
+  if (group > 0)
+    return launch_score_votes(&plain, bt, qf, k_pool, pool_rows, hit, votes, vote_stride, nullptr, 0,
+                              ws + w.select_ws, (hipStream_t)stream);
+  float* partials = (float*)(ws + w.partials);
+  TS_TRY(ts_score(&plain, bt, qf, k_pool, pool_rows, hit, (float*)(ws + w.scores), w.score_stride,
+                  partials, w.partials_bytes, stream));
+  return launch_vote(&plain, bt, (const float*)(ws + w.scores), w.score_stride, partials, hit,
+                     (float*)(ws + w.stats), votes, nullptr, vote_stride, nullptr, 0, (hipStream_t)stream);
+}
+
+int ts_decode_layer_attend(const ts_config* cfg, const ts_batch* bt, const void* q, const float* votes,
+                           int64_t vote_stride, const void* k_pool, const void* v_pool,
+                           int64_t pool_rows, const ts_selcache* cache, void* out, int32_t* sel,
+                           int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
+                           size_t workspace_bytes, ts_stream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_TRY(validate_batch(cfg, bt));
+  TS_REQUIRE(q && votes && k_pool && v_pool && out && sel && sel_pos && sel_len, TS_EINVAL,
+             "layer attend: NULL tensor argument");
+  TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
+             (long long)pool_rows);
+  const LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);
+  TS_REQUIRE(workspace != nullptr && workspace_bytes >= w.total, TS_EWORKSPACE,
+             "workspace %zu bytes < required %zu", workspace_bytes, w.total);
+  TS_REQUIRE(sel_stride >= w.max_sel, TS_EWORKSPACE, "sel_stride %lld < n_init+top_k+n_local = %d",
+             (long long)sel_stride, w.max_sel);
+  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
+  TS_REQUIRE(vote_stride >= max_n, TS_EWORKSPACE, "vote_stride %lld < max candidates %d",
+             (long long)vote_stride, max_n);
+  TS_REQUIRE(max_n <= (1 << 20), TS_ESHAPE, "layer: at most 2^20 candidates per request (max_seq_len %d)",
+             bt->max_seq_len);
+  char* ws = (char*)workspace;
+  // The hit flags are those the votes call left in this workspace.
+  int32_t* hit = cache ? (int32_t*)(ws + w.hit) : nullptr;
+  const float* ranked = votes;
+  int64_t ranked_stride = vote_stride;
+  if (cfg->pool_kernel > 0 && max_n > 0) {  // tr.py:366-369, after the all-reduce of tr.py:363-364
+    TS_TRY(launch_pool(cfg, bt, votes, vote_stride, (float*)(ws + w.pooled), w.score_stride, hit,
+                       (hipStream_t)stream));
+    ranked = (const float*)(ws + w.pooled);
+    ranked_stride = w.score_stride;
+  }
+  TopkArgs topk = make_topk_args(cfg, bt, ranked, ranked_stride, hit, cache, sel, sel_pos, sel_stride,
+                                 sel_len, (uint32_t*)(ws + w.topk_ws));
+  topk.clear = attn_tickets(cfg, bt->batch, w.max_sel, ws + w.attn_ws);
+  topk.clear_per_req = cfg->num_kv_heads;
+  ts_config plain = *cfg;
+  plain.pool_kernel = -1;
+  if (max_n > 0 && score_votes_group(&plain, bt->batch, bt->max_seq_len) > 0)
+    topk.fault = score_votes_fault_word(&plain, bt->batch, bt->max_seq_len, ws + w.select_ws);
+  TS_TRY(launch_topk(topk, bt->batch, max_n, (hipStream_t)stream));
+  return launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, bt->batch, w.max_sel,
+                     out, ws + w.attn_ws, /*tickets_clear=*/true, (hipStream_t)stream);
 }
 
 int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, int32_t rows,

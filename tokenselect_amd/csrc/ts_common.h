@@ -33,7 +33,7 @@ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // the statistics merge and the workspace query.
 int score_tokens_per_block(int64_t total_candidates, int num_heads);
 
-// Words the rotation kernel clears on the side (two such regions per launch):
+// Words the rotation kernel clears on the side (up to three such regions per launch):
 // `count` pieces of `words` 32-bit words, `stride` words apart (all zero: nothing
 // to clear).
 struct ZeroRegion {
@@ -46,10 +46,11 @@ struct ZeroRegion {
 // regions are cleared by the same launch.
 int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
                        const float* sin_table, int64_t table_rows, void* qf, const ZeroRegion& zero,
-                       const ZeroRegion& zero2, hipStream_t stream);
+                       const ZeroRegion& zero2, hipStream_t stream, const ZeroRegion& zero3 = ZeroRegion{});
 int launch_rope(const void* x, void* out, const float* cos_table, const float* sin_table,
                 const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
-                const ZeroRegion& zero, const ZeroRegion& zero2, hipStream_t stream);
+                const ZeroRegion& zero, const ZeroRegion& zero2, hipStream_t stream,
+                const ZeroRegion& zero3 = ZeroRegion{});
 
 // Sparse decode attention (ts_attn.hip).  The kernel counts its workgroups in per
 // (request, KV head) tickets inside the workspace, which must be zero at launch:

@@ -44,6 +44,14 @@ struct ScoreArgs {
   uint32_t* clear;        // words to clear for the next kernel of the stream, or NULL
   int clear_per_req;
   uint64_t spin_ticks;    // bound of a grid-wide wait, in 100 MHz ticks
+  // Votes-only form of the fused kernel (groups of requests of a large batch, one
+  // launch each): request index of the launch's first request; the launch ends with
+  // the votes in memory and their first-level histogram added to the top-k workspace.
+  int batch_offset;
+  int votes_only;
+  uint32_t* hist_ws;      // per-request top-k workspace (ts_topk.h) whose hist0 is counted into, or NULL
+  size_t hist_ws_stride;
+  uint32_t* fault_word;   // votes-only: the word the kernels after this one consult
   uint32_t absent;        // team members that never arrive (tests of the give-up path)
   uint32_t* fault_out;    // caller's word, set to 1 when a wait gave up, or NULL
   int pool_kernel;        // max-pool window over the votes (tr.py:366-369), <= 0: off
@@ -101,6 +109,24 @@ __global__ void select_zero_kernel(ZeroRegion r0, ZeroRegion r1);
 
 // Bound of a grid-wide wait of the fused selection: 2 s of the 100 MHz clock.
 constexpr uint64_t kSelectWaitTicks = 200000000ull;
+
+// Scores and votes of a batch of any size without the [H, n] scores in memory: the
+// requests are served in groups whose scores fit the LDS of the device, one launch of
+// the fused kernel in its votes-only form per group (score, statistics rendezvous,
+// votes, [max-pool]); each launch also counts the first histogram level of the top-k
+// into hist_ws.  score_votes_group() is the number of requests per launch, 0 when not
+// even one request fits (or the fused kernels are switched off): then the separate
+// kernels serve.  The workspace is that of ts_select for the whole batch; the
+// statistics replicas and the rendezvous areas (score_votes_zero_regions) are zero.
+int score_votes_group(const ts_config* cfg, int batch, int max_seq_len);
+void score_votes_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* stats,
+                              ZeroRegion* sync);
+int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+                       int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
+                       uint32_t* hist_ws, size_t hist_ws_stride, void* workspace, hipStream_t stream);
+// The word the votes-only launches leave non-zero when a wait of theirs gave up.
+const uint32_t* score_votes_fault_word(const ts_config* cfg, int batch, int max_seq_len,
+                                       const void* workspace);
 
 // Launch without the clearing pass: the regions above are known to be zero.
 int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,

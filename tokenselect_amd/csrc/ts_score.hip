@@ -96,7 +96,7 @@ __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const Gr
   const int first = (int)team.index * 4 + wave;
   const int step = (int)team.size * 4;
   for (int item = first; item < items; item += step) {
-    const int b = item / H, h = item % H;
+    const int b = a.batch_offset + item / H, h = item % H;
     if (a.skip && a.skip[b]) continue;
     const ReqGeom geo =
         request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
@@ -132,9 +132,9 @@ __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t*
   const int B = gridDim.y, mine = blockIdx.y;
   uint32_t before = 0, total = 0;  // selecting requests below this one / in all
   for (int base = 0; base < B; base += 256) {
-    const int b = base + tid;
+    const int b = a.batch_offset + base + tid;  // requests of this launch
     bool selects = false;
-    if (b < B && !(a.skip && a.skip[b]))
+    if (base + tid < B && !(a.skip && a.skip[b]))
       selects = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
                                  a.max_seq_len).n > 0;
     const uint64_t mask = __ballot(selects);
@@ -272,7 +272,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   constexpr int ITER = 16 * TG;    // tokens per iteration
   constexpr uint32_t ROW_BYTES = HKV * kHeadDim * 2;
 
-  const int b = blockIdx.y;
+  const int b = blockIdx.y + a.batch_offset;
   int n, first_pos;
   if (a.direct_n >= 0) {
     n = (int)a.direct_n;
@@ -287,7 +287,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   GridTeam team{0u, 0u};
   if constexpr (MODE == kScoreFused) {
     __shared__ uint32_t team_lds[8];
-    fixed_segments(a, b);
+    if (!a.votes_only) fixed_segments(a, b);
     if (n <= 0) return;  // dense or served by the cache: nothing to select, not on the team
     team = selecting_team(a, team_lds);
   }
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     if constexpr (MODE == kScoreFused) {  // no tokens here: only help with the statistics
       grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
       merge_request_stats(a, team, threadIdx.x & 63, threadIdx.x >> 6);
-      const uint32_t rounds = kSelectRounds + (a.pool_kernel > 0 ? 1u : 0u);
+      const uint32_t rounds = (a.votes_only ? 1u : kSelectRounds) + (a.pool_kernel > 0 ? 1u : 0u);
       for (uint32_t round = 2; round <= rounds; ++round)
         grid_arrive(a.sync, round, false, a.spin_ticks, team.size, team.index);
     }
@@ -618,6 +618,23 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       __syncthreads();
       for (int i = tid; i < count + halo; i += 256) lh[i] = 0u;
       __syncthreads();
+    }
+    if (a.votes_only) {
+      // The launch ends here: the votes are in memory, and their first histogram level
+      // goes to the top-k workspace, where the kernels after this one pick it up.
+      if (a.hist_ws) {
+        for (int i = tid; i < count; i += 256) atomicAdd(&lh[key_bin0(key_of(i))], 1u);
+        __syncthreads();
+        uint32_t* hist0 = topk_ws(a.hist_ws, a.hist_ws_stride, b) + kTopkHist0;
+        for (int i = tid; i < kTopkBins; i += 256)
+          if (lh[i]) atomicAdd(&hist0[i], lh[i]);
+      }
+      if (blockIdx.x == 0 && tid == 0 && load_coherent(&a.sync[0]) != 0u) {
+        __hip_atomic_store(a.fault_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (a.fault_out)
+          __hip_atomic_store(a.fault_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+      return;
     }
     // Local histogram: one LDS atomic per candidate (lanes that hit the same bin are
     // performed one after the other, which for 256 candidates is a few hundred cycles).
@@ -1111,7 +1128,7 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
   w.short_list = take(B * kSelListParts * kSelListCap * sizeof(uint2));
   w.pool_stride = (int64_t)align_up((size_t)std::max(max_n, 1), 64);
   w.pool_votes = take(cfg->pool_kernel > 0 ? B * (size_t)w.pool_stride * sizeof(float) : 0);
-  w.sync = take(kSyncWords * 4);
+  w.sync = take(B * kSyncWords * 4);  // one rendezvous area per launch of a batch served in groups
   w.total = off;
   return w;
 }
@@ -1126,6 +1143,29 @@ void select_zero_regions(const SelectWorkspace& w, void* workspace, int batch, Z
   sync->stride = kSyncSlotWords;
   sync->words = kSyncLiveWords;
   sync->count = kSyncSlots + 1;
+}
+
+void score_votes_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* stats,
+                              ZeroRegion* sync) {
+  stats->base = (uint32_t*)((char*)workspace + w.stats);
+  stats->words = (int)((size_t)kSyncSlots * w.stats_stride);
+  stats->stride = stats->words;
+  stats->count = 1;
+  sync->base = (uint32_t*)((char*)workspace + w.sync);
+  sync->stride = kSyncSlotWords;
+  sync->words = kSyncLiveWords;
+  sync->count = (kSyncSlots + 1) * batch;
+}
+
+int score_votes_group(const ts_config* cfg, int batch, int max_seq_len) {
+  for (int g = batch; g >= 1; --g)
+    if (fused_tokens_per_block(cfg, g, max_seq_len, false) > 0) return g;
+  return 0;
+}
+
+const uint32_t* score_votes_fault_word(const ts_config* cfg, int batch, int max_seq_len,
+                                       const void* workspace) {
+  return (const uint32_t*)((const char*)workspace + select_workspace(cfg, batch, max_seq_len, true).sync);
 }
 
 __global__ __launch_bounds__(256) void select_zero_kernel(ZeroRegion r0, ZeroRegion r1) {
@@ -1211,6 +1251,52 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   return TS_OK;
 }
 
+int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+                       int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
+                       uint32_t* hist_ws, size_t hist_ws_stride, void* workspace, hipStream_t stream) {
+  const int group = score_votes_group(cfg, bt->batch, bt->max_seq_len);
+  TS_REQUIRE(group > 0, TS_ESHAPE, "fused scoring + vote: not even one request of %d tokens fits",
+             bt->max_seq_len);
+  // Offsets of the pieces: those of the whole batch's workspace, whatever the groups.
+  const SelectWorkspace all = select_workspace(cfg, bt->batch, bt->max_seq_len, true);
+  char* ws = (char*)workspace;
+  const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
+  int launch = 0;
+  for (int first = 0; first < bt->batch; first += group, ++launch) {
+    const int requests = std::min(group, bt->batch - first);
+    const SelectWorkspace w = select_workspace(cfg, requests, bt->max_seq_len, true);
+    TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE, "fused scoring + vote: group of %d does not fit",
+               requests);
+    ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, skip, (float*)(ws + all.partials),
+                                 w.tokens_per_block);
+    a.sync = (uint32_t*)(ws + all.sync) + (size_t)launch * kSyncWords;
+    a.fault_word = (uint32_t*)(ws + all.sync);
+    a.stats = (float*)(ws + all.stats);
+    a.stats_stride = all.stats_stride;
+    a.votes = votes;
+    a.vote_stride = vote_stride;
+    a.counters = (uint32_t*)(ws + all.counters);
+    a.spin_ticks = kSelectWaitTicks;
+    a.fault_out = bt->fault;
+    a.pool_kernel = cfg->pool_kernel;
+    a.pool_votes = (float*)(ws + all.pool_votes);
+    a.pool_stride = all.pool_stride;
+    a.batch_offset = first;
+    a.votes_only = 1;
+    a.hist_ws = hist_ws;
+    a.hist_ws_stride = hist_ws_stride;
+    const dim3 grid((unsigned)w.blocks_per_req, (unsigned)requests);
+    void* params[] = {(void*)&a};
+    const hipError_t e = hipLaunchKernel(fn, grid, dim3(256), params,
+                                         fused_lds_bytes(w.tokens_per_block, cfg->num_heads), stream);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(TS_EHIP, "fused scoring + vote launch: %s", hipGetErrorString(e));
+    }
+  }
+  return TS_OK;
+}
+
 }  // namespace ts
 
 using namespace ts;
@@ -1255,6 +1341,39 @@ int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const voi
   const dim3 grid((unsigned)ceil_div(max_n, a.tokens_per_block), (unsigned)bt->batch);
   return launch_score<false, kScoreTiled>(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, a, grid,
                                    (hipStream_t)stream);
+}
+
+int ts_score_vote_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+  if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
+  return (cfg->pool_kernel <= 256 && score_votes_group(cfg, batch, max_seq_len) > 0) ? 1 : 0;
+}
+
+int ts_score_vote(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
+                  int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
+                  void* workspace, size_t workspace_bytes, ts_stream_t stream) {
+  TS_TRY(validate_config(cfg));
+  TS_TRY(validate_batch(cfg, bt));
+  TS_REQUIRE(qf && k_pool && votes && workspace, TS_EINVAL, "ts_score_vote: NULL argument");
+  TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
+             (long long)pool_rows);
+  TS_REQUIRE(ts_score_vote_supported(cfg, bt->batch, bt->max_seq_len), TS_ESHAPE,
+             "ts_score_vote: not even one request of %d tokens fits the LDS of the device (or "
+             "pool_kernel is above 256, or the fused kernels are switched off); use ts_score + ts_vote",
+             bt->max_seq_len);
+  const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len, true);
+  TS_REQUIRE(workspace_bytes >= w.total, TS_EWORKSPACE, "ts_score_vote: workspace %zu bytes < required %zu",
+             workspace_bytes, w.total);
+  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
+  TS_REQUIRE(vote_stride >= max_n, TS_EWORKSPACE, "vote_stride %lld < max candidates %d",
+             (long long)vote_stride, max_n);
+  if (max_n <= 0) return TS_OK;
+  ZeroRegion stats, sync;
+  score_votes_zero_regions(w, workspace, bt->batch, &stats, &sync);
+  hipLaunchKernelGGL(select_zero_kernel, dim3((unsigned)(8 * bt->batch)), dim3(256), 0,
+                     (hipStream_t)stream, stats, sync);
+  TS_TRY(check_launch("select_zero_kernel"));
+  return launch_score_votes(cfg, bt, qf, k_pool, pool_rows, skip, votes, vote_stride, nullptr, 0,
+                            workspace, (hipStream_t)stream);
 }
 
 int ts_select_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {

@@ -45,6 +45,9 @@ struct TopkArgs {
   // attention's tickets): clear_per_req words per request, or NULL.
   uint32_t* clear;
   int clear_per_req;
+  // A word an earlier kernel of the stream leaves non-zero when the votes are not
+  // valid (a wait of the fused scoring gave up): sel_len then reports -1.  Or NULL.
+  const uint32_t* fault;
 };
 
 __device__ __host__ __forceinline__ uint32_t* topk_ws(uint32_t* ws, size_t stride, int b) {
@@ -129,6 +132,10 @@ TopkArgs make_topk_args(const ts_config* cfg, const ts_batch* bt, const float* v
 int launch_topk(const TopkArgs& a, int batch, int max_n, hipStream_t stream,
                 bool counters_zeroed = false, bool hist0_filled = false);
 ZeroRegion topk_zero_region(const TopkArgs& a, int batch);
+
+// Max-pool of the votes (ts_vote.hip, tr.py:366-369): pooled[t] over votes[t - pad, t - pad + kernel).
+int launch_pool(const ts_config* cfg, const ts_batch* bt, const float* votes, int64_t vote_stride,
+                float* pooled, int64_t pooled_stride, const int32_t* skip, hipStream_t stream);
 
 // Soft vote (ts_vote.hip); with hist_ws (the top-k workspace, counters zeroed) the vote
 // kernel also fills the first-level histogram of the selection, unless max-pooling

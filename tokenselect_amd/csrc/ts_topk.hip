@@ -137,7 +137,8 @@ __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs 
   }
   const bool is_hit = a.hit && a.hit[b];
   const int k = is_hit ? min(a.cache_len[b], a.top_k) : geo.k;
-  if (part == 0 && tid == 0) a.sel_len[b] = a.n_init + k + a.n_local;
+  if (part == 0 && tid == 0)
+    a.sel_len[b] = (a.fault && !is_hit && *a.fault) ? -1 : a.n_init + k + a.n_local;
   for (int i = first; i < a.n_init; i += step) emit(i, i);
   for (int i = first; i < a.n_local; i += step) emit(a.n_init + k + i, L - a.n_local + i);
   if (is_hit) {  // tr.py:419: reuse the cached positions
@@ -325,6 +326,7 @@ TopkArgs make_topk_args(const ts_config* cfg, const ts_batch* bt, const float* v
   a.ws_stride = topk_ws_stride_words(max_n);
   a.clear = nullptr;
   a.clear_per_req = 0;
+  a.fault = nullptr;
   a.slice = kTopkSlice;
   return a;
 }
@@ -342,12 +344,6 @@ ZeroRegion topk_zero_region(const TopkArgs& a, int batch) {
 // the first-level histogram on its own, so a large batch gets larger slices (about a
 // thousand workgroups in all), in multiples of the 256 candidates of a pass.
 static int topk_slice(int batch, int max_n) {
-  static const int forced = [] {
-    const char* e = getenv("TS_TOPK_SLICE");  // tuning override, multiple of 256
-    const int v = e ? atoi(e) : 0;
-    return (v >= 256 && v <= 65536) ? v / 256 * 256 : 0;
-  }();
-  if (forced) return forced;
   const int64_t per = ceil_div(ceil_div((int64_t)batch * max_n, 1024), 256) * 256;
   return (int)(per < kTopkSlice ? kTopkSlice : (per > 4096 ? 4096 : per));
 }

@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256) void vote_kernel(VoteArgs a) {
 struct PoolArgs {
   const float* votes;
   float* pooled;
-  int64_t vote_stride;
+  int64_t vote_stride, pooled_stride;
   const int32_t* seq_lens;
   const int32_t* k_per_req;
   const int32_t* skip;
@@ -142,7 +142,29 @@ __global__ __launch_bounds__(256) void pool_kernel(PoolArgs a) {
   const int lo = max(t - pad, 0), hi = min(t - pad + a.kernel, geo.n);
   float m = v[lo];
   for (int i = lo + 1; i < hi; ++i) m = fmaxf(m, v[i]);
-  a.pooled[(size_t)b * a.vote_stride + t] = m;
+  a.pooled[(size_t)b * a.pooled_stride + t] = m;
+}
+
+int launch_pool(const ts_config* cfg, const ts_batch* bt, const float* votes, int64_t vote_stride,
+                float* pooled, int64_t pooled_stride, const int32_t* skip, hipStream_t stream) {
+  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
+  if (max_n <= 0) return TS_OK;
+  PoolArgs p;
+  p.votes = votes;
+  p.pooled = pooled;
+  p.vote_stride = vote_stride;
+  p.pooled_stride = pooled_stride;
+  p.seq_lens = bt->seq_lens;
+  p.k_per_req = bt->k_per_req;
+  p.skip = skip;
+  p.n_init = cfg->n_init;
+  p.n_local = cfg->n_local;
+  p.top_k = cfg->top_k;
+  p.max_seq_len = bt->max_seq_len;
+  p.kernel = cfg->pool_kernel;
+  hipLaunchKernelGGL(pool_kernel, dim3((unsigned)ceil_div(max_n, 256), (unsigned)bt->batch), dim3(256),
+                     0, stream, p);
+  return check_launch("pool_kernel");
 }
 
 int launch_vote(const ts_config* cfg, const ts_batch* bt, const float* scores, int64_t score_stride,
@@ -192,23 +214,8 @@ int launch_vote(const ts_config* cfg, const ts_batch* bt, const float* scores, i
                      dim3(256), 0, stream, a);
   TS_TRY(check_launch("vote_kernel"));
 
-  if (cfg->pool_kernel > 0) {
-    PoolArgs p;
-    p.votes = votes;
-    p.pooled = pooled;
-    p.vote_stride = vote_stride;
-    p.seq_lens = bt->seq_lens;
-    p.k_per_req = bt->k_per_req;
-    p.skip = skip;
-    p.n_init = cfg->n_init;
-    p.n_local = cfg->n_local;
-    p.top_k = cfg->top_k;
-    p.max_seq_len = bt->max_seq_len;
-    p.kernel = cfg->pool_kernel;
-    hipLaunchKernelGGL(pool_kernel, dim3((unsigned)ceil_div(max_n, 256), (unsigned)bt->batch),
-                       dim3(256), 0, stream, p);
-    TS_TRY(check_launch("pool_kernel"));
-  }
+  if (cfg->pool_kernel > 0)
+    TS_TRY(launch_pool(cfg, bt, votes, vote_stride, pooled, vote_stride, skip, stream));
   return TS_OK;
 }
 

@@ -349,7 +349,9 @@ def select_fault(cfg: LayerConfig, bt: Batch, workspace: torch.Tensor) -> bool:
     (synchronises)."""
     nbytes = _lib.load().ts_select_workspace_bytes(ctypes.byref(cfg.to_c()), bt.batch,
                                                    bt.max_seq_len)
-    return bool(workspace.view(torch.int32)[nbytes // 4 - 65 * 1024].item())
+    # the rendezvous areas (one of 65 x 4096 bytes per request) end the workspace; the
+    # fault word is the first word of the first
+    return bool(workspace.view(torch.int32)[nbytes // 4 - bt.batch * 65 * 1024].item())
 
 
 def scores_head_major(cfg: LayerConfig, scores: torch.Tensor) -> torch.Tensor:
@@ -385,6 +387,36 @@ def vote(cfg: LayerConfig, bt: Batch, scores: torch.Tensor, partials: torch.Tens
     _lib.check(lib.ts_vote(ctypes.byref(c), ctypes.byref(cb), _p(scores), stride, _p(partials),
                            _p(skip), _p(stats), _p(votes), _p(pooled), stride, _stream()))
     return (pooled if pooled is not None else votes), stats
+
+
+def score_vote_supported(cfg: LayerConfig, batch: int, max_seq_len: int) -> bool:
+    """Whether :func:`score_vote` can serve this shape (``ts_score_vote_supported``)."""
+    return bool(_lib.load().ts_score_vote_supported(ctypes.byref(cfg.to_c()), int(batch),
+                                                    int(max_seq_len)))
+
+
+def score_vote(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
+               skip: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):
+    """:func:`score` + :func:`vote` without the scores in memory (``ts_score_vote``), a
+    batch of any size in groups of requests that fit the LDS of the device.  Returns
+    ``votes [B, stride]`` fp32 (pooled when ``cfg.pool_kernel > 0``)."""
+    c, cb = cfg.to_c(), _c_batch(cfg, bt)
+    _need(qf, "qf", torch.bfloat16)
+    _check_pool(cfg, k_pool, "k_pool")
+    B = bt.batch
+    if qf.numel() != B * cfg.num_heads * cfg.head_dim:
+        raise ValueError("qf must hold B*H*D elements")
+    if skip is not None:
+        _need(skip, "skip", torch.int32, 1)
+    lib = _lib.load()
+    nbytes = lib.ts_select_workspace_bytes(ctypes.byref(c), B, bt.max_seq_len)
+    if workspace is None or workspace.numel() < nbytes:
+        workspace = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=qf.device)
+    votes = torch.empty((B, score_stride_for(bt.max_seq_len)), dtype=torch.float32, device=qf.device)
+    _lib.check(lib.ts_score_vote(ctypes.byref(c), ctypes.byref(cb), _p(qf), _p(k_pool), k_pool.shape[0],
+                                 _p(skip), _p(votes), votes.shape[1], _p(workspace), workspace.numel(),
+                                 _stream()))
+    return votes
 
 
 def topk_ragged(cfg: LayerConfig, bt: Batch, votes: torch.Tensor,
@@ -624,6 +656,54 @@ class DecodeLayer:
             ctypes.byref(self._c), ctypes.byref(cb), _p(q), _p(self.q_cos), _p(self.q_sin),
             _p(k_pool), _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, B), _p(out),
             _p(self.sel), _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
+            self.workspace.numel(), _stream()))
+        return out, self.sel[:B], self.sel_pos[:B], self.sel_len[:B]
+
+    # The layer split at the vote (tensor parallelism, tr.py:361-364): votes() leaves this
+    # rank's partial votes, the caller adds the ranks' votes in place (all-reduce), attend()
+    # selects from the sum and attends with this rank's heads.
+    def votes(self, q: torch.Tensor, k_pool: torch.Tensor, bt: Batch,
+              cache: Optional[SelectionCache] = None) -> torch.Tensor:
+        cfg = self.cfg
+        self.check()
+        if bt.fault is None:
+            bt = Batch(bt.seq_lens, bt.table, bt.max_seq_len, bt.k_per_req, self.fault)
+        cb = _c_batch(cfg, bt)
+        if bt.batch > self.batch or bt.max_seq_len > self.max_seq_len:
+            raise ValueError("batch / max_seq_len exceed what this DecodeLayer was sized for")
+        _need(q, "q", torch.bfloat16)
+        _check_pool(cfg, k_pool, "k_pool")
+        B = bt.batch
+        if q.numel() != B * cfg.num_heads * cfg.head_dim:
+            raise ValueError("q must hold B*H*D elements")
+        if getattr(self, "_votes", None) is None:
+            self._votes = torch.zeros((self.batch, score_stride_for(self.max_seq_len)),
+                                      dtype=torch.float32, device=q.device)
+        _lib.check(_lib.load().ts_decode_layer_votes(
+            ctypes.byref(self._c), ctypes.byref(cb), _p(q), _p(self.q_cos), _p(self.q_sin), _p(k_pool),
+            k_pool.shape[0], _c_cache(cache, cfg, B), _p(self._votes), self._votes.shape[1],
+            _p(self.workspace), self.workspace.numel(), _stream()))
+        return self._votes[:B]
+
+    def attend(self, q: torch.Tensor, votes: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+               bt: Batch, cache: Optional[SelectionCache] = None, out: Optional[torch.Tensor] = None):
+        cfg = self.cfg
+        if bt.fault is None:
+            bt = Batch(bt.seq_lens, bt.table, bt.max_seq_len, bt.k_per_req, self.fault)
+        cb = _c_batch(cfg, bt)
+        _need(q, "q", torch.bfloat16)
+        _need(votes, "votes", torch.float32, 2)
+        _check_pool(cfg, k_pool, "k_pool")
+        _check_pool(cfg, v_pool, "v_pool")
+        B = bt.batch
+        if q.numel() != B * cfg.num_heads * cfg.head_dim or votes.shape[0] != B:
+            raise ValueError("q / votes do not match the batch")
+        if out is None:
+            out = self.out[:B]
+        _lib.check(_lib.load().ts_decode_layer_attend(
+            ctypes.byref(self._c), ctypes.byref(cb), _p(q), _p(votes), votes.stride(0), _p(k_pool),
+            _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, B), _p(out), _p(self.sel),
+            _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
             self.workspace.numel(), _stream()))
         return out, self.sel[:B], self.sel_pos[:B], self.sel_len[:B]
 
