@@ -392,14 +392,18 @@ int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, in
  * cache may be NULL (QUERY_CACHE=False as released, tr.py:918).
  *
  * When ts_select_supported() holds, the selection runs as the single ts_select
- * kernel; a larger batch is scored and voted on in groups of requests as by
- * ts_score_vote and then ranked by the kernels of ts_topk_ragged; where not even one
- * request fits, ts_score, ts_vote and ts_topk_ragged run as they do on their own.
- * All forms give the same selection.
+ * kernel; a batch of contexts so long that each request needs the device to itself
+ * is scored and voted on request by request as by ts_score_vote and then ranked by
+ * the kernels of ts_topk_ragged; otherwise ts_score, ts_vote and ts_topk_ragged run
+ * as they do on their own.  All forms give the same selection.
  * ts_set_fused_select(0) forces the separate kernels for the calling process
  * (1 restores the default); it returns the previous setting and has no
  * counterpart in the reference. */
 int ts_set_fused_select(int enable);
+/* Which form ts_decode_layer takes for a shape: 2 = ts_select, 1 = ts_score_vote's
+ * launches (one request each) + top-k kernels, 0 = ts_score + ts_vote + top-k
+ * kernels; -1 for an unsupported configuration. */
+int ts_decode_layer_selection(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
 size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
 int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, const float* q_cos,
                     const float* q_sin, const void* k_pool, const void* v_pool,

@@ -37,9 +37,10 @@ def _votes_on_device(wl):
     c, bt, B = wl.cfg, wl.batch, len(wl.seq_lens)
     cos, sin = ops.scoring_cos_sin(c.head_dim, c.rope_theta, c.rope_scale, c.n_local, wl.q.device)
     qf = ops.rope_apply(wl.q.view(B, c.num_heads, c.head_dim), cos, sin, None)
-    if ops.select_supported(c, B, bt.max_seq_len):
+    form = ops.layer_selection_form(c, B, bt.max_seq_len)
+    if form == 2:
         return ops.select(c, bt, qf, wl.k_pool, want_votes=True)[3], qf
-    if ops.score_vote_supported(c, B, bt.max_seq_len):
+    if form == 1:
         return ops.score_vote(c, bt, qf, wl.k_pool), qf
     scores, partials = ops.score(c, bt, qf, wl.k_pool)
     return ops.vote(c, bt, scores, partials)[0], qf

@@ -98,6 +98,7 @@ SIGNATURES = {
     "ts_prefill_chunk": (_i32, [_CFG, _BT, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i64, _ptr, _ptr,
                                 _ptr, _i64, _ptr, _ptr, _size, _ptr]),
     "ts_set_fused_select": (_i32, [_i32]),
+    "ts_decode_layer_selection": (_i32, [_CFG, _i32, _i32]),
     "ts_decode_layer_workspace_bytes": (_size, [_CFG, _i32, _i32]),
     "ts_decode_layer_votes": (_i32, [_CFG, _BT, _ptr, _ptr, _ptr, _ptr, _i64, _SC, _ptr, _i64, _ptr,
                                      _size, _ptr]),

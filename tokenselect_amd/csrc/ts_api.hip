@@ -136,6 +136,13 @@ static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32
   return w;
 }
 
+static int layer_selection_form(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+
+int ts_decode_layer_selection(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+  if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return -1;
+  return layer_selection_form(cfg, batch, max_seq_len);
+}
+
 size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
   // A workspace sized for `batch` serves every smaller batch and both settings of
@@ -147,6 +154,20 @@ size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int3
     if (need > most) most = need;
   }
   return most;
+}
+
+// How ts_decode_layer selects for a shape: 2 = the single ts_select kernel, 1 = scores and
+// votes per request as by ts_score_vote, then the top-k kernels, 0 = ts_score, ts_vote
+// and the top-k kernels.
+static int layer_selection_form(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+  if (select_workspace(cfg, batch, max_seq_len).tokens_per_block > 0) return 2;
+  const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
+  // A request of max_seq_len needs the device to itself (4 x 256K: 463 us per layer
+  // against 481 us with the separate kernels).  The grids are sized by max_seq_len, so
+  // with several requests per launch a ragged batch (16 x 4K..128K: 617 against 534 us)
+  // leaves most workgroups of a launch without tokens: those take the separate kernels.
+  if (max_n > 0 && cfg->pool_kernel <= 256 && score_votes_group(cfg, batch, max_seq_len) == 1) return 1;
+  return 0;
 }
 
 // Decode (chunk_rows == 0: one query row per request, q_cos / q_sin are the [D] rows
@@ -197,14 +218,8 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
   topk.clear = tickets;
   topk.clear_per_req = cfg->num_kv_heads;
   // A batch too large for one launch of the selection: scores and votes still without
-  // the [H, n] scores in memory, one launch per request, then the top-k kernels on the
-  // votes.  Taken when a request of max_seq_len needs the device to itself (4 x 256K:
-  // 463 us per layer against 481 us): the grids are sized by max_seq_len, so with
-  // several requests per launch a ragged batch (16 x 4K..128K: 617 against 534 us)
-  // leaves most workgroups of a launch without tokens.
-  const int vote_group =
-      (!one_launch && max_n > 0 && cfg->pool_kernel <= 256 &&
-       score_votes_group(cfg, bt->batch, bt->max_seq_len) == 1) ? 1 : 0;
+  // the [H, n] scores in memory, one launch per request, then the top-k kernels.
+  const int vote_group = layer_selection_form(cfg, bt->batch, bt->max_seq_len) == 1 ? 1 : 0;
   ZeroRegion zero_counters, zero_sync, zero_stats;
   if (one_launch) {
     select_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_counters, &zero_sync);

@@ -389,6 +389,13 @@ def vote(cfg: LayerConfig, bt: Batch, scores: torch.Tensor, partials: torch.Tens
     return (pooled if pooled is not None else votes), stats
 
 
+def layer_selection_form(cfg: LayerConfig, batch: int, max_seq_len: int) -> int:
+    """How :class:`DecodeLayer` selects for a shape: 2 = one ``ts_select`` launch, 1 =
+    ``ts_score_vote`` request by request + the top-k kernels, 0 = the separate kernels."""
+    return int(_lib.load().ts_decode_layer_selection(ctypes.byref(cfg.to_c()), int(batch),
+                                                     int(max_seq_len)))
+
+
 def score_vote_supported(cfg: LayerConfig, batch: int, max_seq_len: int) -> bool:
     """Whether :func:`score_vote` can serve this shape (``ts_score_vote_supported``)."""
     return bool(_lib.load().ts_score_vote_supported(ctypes.byref(cfg.to_c()), int(batch),
