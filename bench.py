@@ -144,6 +144,16 @@ def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
         if any(ops.select_fault(c, bt, space) for space in spaces):
             sys.exit("bench.py: a grid-wide wait of the selection kernel gave up")
         dom_kernel = "ts::score_kernel<Hkv,G,false,2> (ts_select: score + vote + top-k in one launch)"
+    elif ops.layer_selection_form(c, B, bt.max_seq_len) == 1:
+        # Scores and votes request by request, the scores never in memory: B launches of
+        # the fused kernel in its votes-only form (+ one small clearing kernel); the
+        # figure is the bytes of all of them over the time of all of them.
+        space = ops.select_workspace(c, bt, dev)
+        dom_us, dom_min = event_time_us(
+            lambda i: ops.score_vote(c, bt, qf, k_pools[i % n_pools], workspace=space), steps, warmup,
+            burst=4)
+        dom_kernel = (f"ts::score_kernel<Hkv,G,false,2> votes-only form x {B} launches "
+                      "(ts_score_vote: score + statistics + vote, one request per launch)")
     else:
         dom_us, dom_min, dom_kernel = score_us, score_min, score_only["kernel"]
     gbs = score_bytes / dom_us / 1e3

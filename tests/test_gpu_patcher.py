@@ -230,3 +230,66 @@ def test_patched_extend_forward(dev):
             L += T
     finally:
         tr.PREFILL_CHUNK_SIZE = 512
+
+
+def test_patched_decode_forward_for_a_batch(dev):
+    """Two requests prefilled one by one through the patched extend forward, then decoded
+    together through the patched decode forward with a BatchTokenRetriever: per request
+    the store, the table and the attention output against the oracle."""
+    say("patched decode forward, batch of 2")
+    H, Hkv, D, layers = 8, 2, 128, 2
+    n_init, n_local, top_k, chunk = 4, 32, 24, 32
+    tr.patch(rope_base=1e4, rope_scale=1, rope_model="ROPE_LLAMA", max_n_tokens=512, top_k=top_k,
+             n_init=n_init, n_local=n_local)
+    tr.PREFILL_CHUNK_SIZE = chunk
+    try:
+        g = torch.Generator(device=dev).manual_seed(23)
+        pool = sg.TokenToKVPool(1024, torch.bfloat16, Hkv, D, layers, dev)
+        runner = sg.ModelRunner(model_config=sg.ModelConfig(layers, D, H, Hkv),
+                                token_to_kv_pool=pool, dtype=torch.bfloat16)
+        owner = runner.req_to_token_retriever
+        slots = torch.randperm(1024, generator=g, device=dev).to(torch.int32)
+        attns = [sg.RadixAttention(H, D, D ** -0.5, Hkv, layer_id=l) for l in range(layers)]
+        prompts, used, singles = [150, 70], 0, []
+        for T in prompts:                      # prefill, one request at a time
+            r = owner.new_token_retriever()
+            loc = slots[used:used + T].contiguous()
+            meta = sg.InputMetadata(sg.ForwardMode.EXTEND, r, pool, loc)
+            for attn in attns:
+                q = torch.randn(T, H * D, generator=g, device=dev).bfloat16()
+                k = torch.randn(T, Hkv * D, generator=g, device=dev).bfloat16()
+                v = torch.randn(T, Hkv * D, generator=g, device=dev).bfloat16()
+                attn.forward(q, k, v, meta)
+            used += T
+            singles.append(r)
+        batch = owner.get_batch_token_retriever(("a", "b"), singles)
+        assert batch is owner.get_batch_token_retriever(("a", "b"))       # same batch, same object
+        with pytest.raises(ValueError):
+            owner.get_batch_token_retriever(("a", "c"))                    # new composition, no tables
+        lens = list(prompts)
+        for step in range(6):
+            loc = slots[used:used + 2].contiguous()
+            used += 2
+            meta = sg.InputMetadata(sg.ForwardMode.DECODE, batch, pool, loc, batch_size=2)
+            for l, attn in enumerate(attns):
+                q = torch.randn(2, H * D, generator=g, device=dev).bfloat16()
+                k = torch.randn(2, Hkv * D, generator=g, device=dev).bfloat16()
+                v = torch.randn(2, Hkv * D, generator=g, device=dev).bfloat16()
+                got = attn.forward(q, k, v, meta)
+                torch.cuda.synchronize()
+                assert got.shape == (2, H * D)
+                kc, vc = pool.k_buffer[l].cpu(), pool.v_buffer[l].cpu()
+                tabs = [t.cpu() for t in batch.get_all_tokens(l)]
+                assert [t.shape[0] for t in tabs] == [n + 1 for n in lens]
+                for b in range(2):
+                    assert tabs[b][-1].item() == loc[b].item()
+                    assert torch.equal(kc[loc[b].item()].reshape(-1), k[b].cpu())
+                _, ref_out = oracle.layer.decode_layer(q.cpu(), kc, vc, tabs, [n + 1 for n in lens], H, D,
+                                                       n_init, n_local, [top_k] * 2, 1e4, 1, D ** -0.5)
+                err = (got.cpu().float() - ref_out.float()).abs().max().item()
+                assert err <= 2e-2, f"step {step} layer {l}: {err}"
+            lens = [n + 1 for n in lens]
+        with pytest.raises(NotImplementedError):                           # wrong number of rows
+            attns[0].forward(torch.zeros(3, H * D, dtype=torch.bfloat16, device=dev), None, None, meta)
+    finally:
+        tr.PREFILL_CHUNK_SIZE = 512

@@ -148,6 +148,91 @@ class ReqToTokenRetriever:
             self.current_token_retriever = TokenRetriever(**self.kwargs)
         return self.current_token_retriever
 
+    def new_token_retriever(self):
+        """A retriever for one more request of a batch (the reference keeps a single one)."""
+        return TokenRetriever(**self.kwargs)
+
+    def get_batch_token_retriever(self, req_ids, retrievers=None):
+        """The batched twin of ``get_token_retriever``: the ``BatchTokenRetriever`` of the
+        running requests ``req_ids``, started afresh (from ``retrievers``, one prefilled
+        ``TokenRetriever`` per request) whenever the composition of the batch changes."""
+        key = tuple(req_ids)
+        if self.current_req_id != key:
+            if retrievers is None or len(retrievers) != len(key):
+                raise ValueError("a new batch needs one prefilled TokenRetriever per request")
+            self.current_req_id = key
+            self.current_token_retriever = BatchTokenRetriever(list(retrievers),
+                                                               self.kwargs["token_to_kv_pool"])
+        return self.current_token_retriever
+
+
+class BatchTokenRetriever:
+    """Several running requests decoded together: the batched twin of ``TokenRetriever``
+    (the reference serves one running request, tr.py:130, and starts a fresh retriever
+    when the request id changes; a batch is the same thing per request).  Built from the
+    retrievers of requests that were prefilled one by one: their token tables and lengths
+    are copied once into ``[layers, B, max_tokens]`` / ``[layers, B]`` tensors that the
+    library reads as a batch; the K / V pools stay aliased.  The batch lives as long as
+    its composition does (``ReqToTokenRetriever.get_batch_token_retriever`` starts a new
+    one when the request ids change)."""
+
+    def __init__(self, retrievers, token_to_kv_pool):
+        first = retrievers[0]
+        self.batch = len(retrievers)
+        self.num_layers, self.head_dim = first.num_layers, first.head_dim
+        self.num_heads, self.num_kv_heads = first.num_heads, first.num_kv_heads
+        self.max_num_tokens, self.dtype, self.device = first.max_num_tokens, first.dtype, first.device
+        self.token_fingerprints = first.token_fingerprints
+        self._value_buffers = [token_to_kv_pool.get_value_buffer(l) for l in range(first.num_layers)]
+        self.token_indices = torch.stack([r.token_indices for r in retrievers], dim=1).contiguous()
+        self.num_tokens = [[r.num_tokens[l] for r in retrievers] for l in range(self.num_layers)]
+        self._num_tokens_dev = torch.stack([r._num_tokens_dev for r in retrievers], dim=1).contiguous()
+        self._layers = {}
+        self._caches = None
+        if QUERY_CACHE:
+            self._caches = [ops.SelectionCache(
+                torch.stack([r.query_fingerprints_cache[l] for r in retrievers]).contiguous(),
+                torch.stack([r.topk_indices_cache[l] for r in retrievers]).contiguous(),
+                torch.stack([r._cache_len_dev[l] for r in retrievers]).contiguous(),
+                torch.stack([r._counters_dev[l] for r in retrievers]).contiguous(),
+                first._threshold_host) for l in range(self.num_layers)]
+
+    def _config(self, n_init, n_local, topk, scaling=None, logit_cap=0.0) -> ops.LayerConfig:
+        return TokenRetriever._config(self, n_init, n_local, topk, scaling, logit_cap)
+
+    def get_all_tokens(self, layer_id):
+        """Per request, as ``TokenRetriever.get_all_tokens``."""
+        return [self.token_indices[layer_id, b, : n] for b, n in enumerate(self.num_tokens[layer_id])]
+
+    def _note_appended(self, layer_id, count: int):
+        assert count == self.batch, "one new token per running request"
+        assert max(self.num_tokens[layer_id]) + 1 <= self.max_num_tokens   # tr.py:334
+        self.num_tokens[layer_id] = [n + 1 for n in self.num_tokens[layer_id]]
+
+    def store(self, attn, rows_k, rows_v, loc):
+        """store_kv_cache + add_k_cache (tr.py:844-854, 332-336) for one new token per request."""
+        layer = attn.layer_id
+        cfg = self._config(max(N_INIT, 0), max(N_Local, 0), max(TOP_K, 1))
+        ops.kv_store(cfg, rows_k.contiguous(), rows_v.contiguous(), loc.to(torch.int32).contiguous(),
+                     self.token_fingerprints[layer], self._value_buffers[layer],
+                     self.token_indices[layer], self._num_tokens_dev[layer])
+        self._note_appended(layer, loc.shape[0])
+
+    def decode_attention(self, attn, q, k_buffer, v_buffer):
+        """One fused library call for a decode layer of the whole batch (tr.py:791-825 per request)."""
+        layer_id = attn.layer_id
+        cfg = self._config(N_INIT, N_Local, TOP_K, attn.scaling, attn.logit_cap)
+        key = (attn.scaling, attn.logit_cap)
+        runner = self._layers.get(key)
+        if runner is None:
+            runner = ops.DecodeLayer(cfg, self.batch, self.max_num_tokens, self.device)
+            self._layers[key] = runner
+        bt = ops.Batch(self._num_tokens_dev[layer_id], self.token_indices[layer_id],
+                       max(self.num_tokens[layer_id]))
+        out = torch.empty((self.batch, self.num_heads * self.head_dim), dtype=q.dtype, device=q.device)
+        runner(q, k_buffer, v_buffer, bt, self._caches[layer_id] if self._caches else None, out=out)
+        return out
+
 
 def paged_matmul(query, token, indices, scores, num_relevant_tokens, num_heads, num_kv_heads,
                  head_dim, BLOCK_SIZE_TOKENS=128):
@@ -379,6 +464,9 @@ def patched_radix_attention_store_kv_cache(self, cache_k, cache_v, input_metadat
     loc = input_metadata.out_cache_loc[start:end]
     retriever = input_metadata.token_retriever
     rows_k, rows_v = cache_k[start:end], cache_v[start:end]
+    if isinstance(retriever, BatchTokenRetriever):
+        retriever.store(self, rows_k, rows_v, loc)
+        return
     if loc.dtype == torch.int32 and loc.shape[0] >= 1:
         cfg = retriever._config(max(N_INIT, 0), max(N_Local, 0), max(TOP_K, 1))
         layer = self.layer_id
@@ -405,10 +493,12 @@ def patched_radix_attention_decode_forward_flashinfer(self, q, k, v, input_metad
     if k is not None:
         assert v is not None
         self.store_kv_cache(k, v, input_metadata)
-    if q.shape[0] != 1:
+    batched = isinstance(input_metadata.token_retriever, BatchTokenRetriever)
+    if q.shape[0] != (input_metadata.token_retriever.batch if batched else 1):
         raise NotImplementedError(
-            "the patched decode forward serves one running request, as the reference does; "
-            "use tokenselect_amd.ops.DecodeLayer for batches")
+            "the patched decode forward serves one running request, as the reference does "
+            "(tr.py:130), or the requests of a BatchTokenRetriever "
+            "(ReqToTokenRetriever.get_batch_token_retriever)")
     k_buffer, v_buffer = input_metadata.token_to_kv_pool.get_kv_buffer(self.layer_id)
     o = input_metadata.token_retriever.decode_attention(self, q.contiguous(), k_buffer, v_buffer)
     return o.view(-1, self.tp_q_head_num * self.head_dim)
