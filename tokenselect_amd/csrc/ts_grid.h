@@ -79,7 +79,9 @@ __device__ __forceinline__ void grid_poll(uint32_t* sync, uint32_t round, uint64
         break;
       }
     }
-    __builtin_amdgcn_s_sleep(2);
+    // About 0.5 us between polls: polling faster costs more (the early workgroups' polls
+    // compete with the key stream of the late ones) than seeing the flag sooner brings.
+    __builtin_amdgcn_s_sleep(20);
   }
 }
 

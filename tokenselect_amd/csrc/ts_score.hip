@@ -123,6 +123,21 @@ __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const Gr
 
 constexpr uint32_t kSelectRounds = 5;  // rendezvous of the fused kernel
 
+#ifdef TS_TRACE  // development builds: per-workgroup phase timestamps of the fused kernel
+__device__ uint64_t g_trace[4096 * 24];
+extern "C" int ts_debug_trace(void* out, size_t bytes) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), bytes);
+}
+#define TS_MARK(i)                                                                              \
+  do {                                                                                          \
+    if (threadIdx.x == 0) g_trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 24 + (i)] = wall_clock64(); \
+  } while (0)
+#else
+#define TS_MARK(i) \
+  do {             \
+  } while (0)
+#endif
+
 // The workgroups that take part in the rendezvous of the fused kernel: all those of
 // the requests that select (neither dense nor served by the selection cache).  The
 // others write their fixed output and leave, so that a step in which every request
@@ -287,6 +302,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   GridTeam team{0u, 0u};
   if constexpr (MODE == kScoreFused) {
     __shared__ uint32_t team_lds[8];
+    TS_MARK(0);
     if (!a.votes_only) fixed_segments(a, b);
     if (n <= 0) return;  // dense or served by the cache: nothing to select, not on the team
     team = selecting_team(a, team_lds);
@@ -530,8 +546,11 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     const int tid = threadIdx.x;
     for (int i = tid; i < kTopkBins; i += 256) lh[i] = 0u;
     if (tid < 16) scratch[tid] = 0u;
+    TS_MARK(1);
     grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
+    TS_MARK(2);
     merge_request_stats(a, team, lane, wave);
+    TS_MARK(3);
     // While the merged statistics are on their way: the exponentials, relative to this
     // workgroup's own maxima; exp(s - max) / sum = exp(s - own max) * exp(own max - max) / sum.
     const ReqGeom geo =
@@ -562,6 +581,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       s_rz[tid] = st ? __expf(local_max[tid] - mx) / sum : 0.f;  // 0: the wait gave up
     }
     __syncthreads();
+    TS_MARK(4);
 
     // Votes of this workgroup's tokens: fp32 sum over the head slots in slot order.
     // The vote replaces the first score of its token in LDS (only the thread that
@@ -581,6 +601,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       if (a.votes && a.pool_kernel <= 0) a.votes[(size_t)b * a.vote_stride + block_lo + i] = c;
       sc[0] = c;
     }
+    TS_MARK(5);
     uint32_t round = 1;  // rendezvous passed so far
     if (a.pool_kernel > 0) {
       // Max-pool smoothing of the votes (tr.py:366-369): stride 1, padding (kernel-1)/2
@@ -649,6 +670,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     }
     __syncthreads();
 
+    TS_MARK(6);
     // Round 3: top 11 key bits.  The workgroups add their local histograms to one
     // of the copies and note the highest occupied bin; afterwards each searches
     // downwards from that bin, 256 bins at a time (one is enough unless the votes
@@ -670,7 +692,9 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         done += fetch_max_coherent(&ctr[kSelMaxBin + (blockIdx.x % kSelHistCopies) * 32], scratch[8]);
       await(done);
     }
+    TS_MARK(7);
     grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+    TS_MARK(8);
     uint32_t t0 = 0, above0 = 0, in_bin0 = 0;
     // The search starts at the highest occupied bin of the request.  Together with the
     // words that hold it, the 128 bins below a guess (a little above this workgroup's
@@ -719,6 +743,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       mine = bins_below(top);
     }
 
+    TS_MARK(9);
     // What is left: `need` of the `in_bin` candidates whose key >> shift equals `prefix`.
     // As soon as they are few enough, they go to a short list that every workgroup
     // ranks on its own (the usual case: heavy-tailed votes leave a hundred candidates
@@ -796,7 +821,9 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       if (lane == 0) atomicAdd(&scratch[8], above);
       __syncthreads();
       if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], 0u);
+      TS_MARK(10);
       grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      TS_MARK(11);
 
       // Every workgroup ranks the list on its own, one entry per thread, in the order
       // (key descending, position ascending) packed into one 64-bit word.  The fill
@@ -873,6 +900,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       __syncthreads();
       kth = scratch[9];
       pos_thr = scratch[12];
+      TS_MARK(12);
     } else {
       // Round 5: last 10 bits of the candidates inside (t0, t1).
       const uint32_t t1 = prefix & 2047u;
@@ -949,6 +977,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       }
     }
     __syncthreads();
+    TS_MARK(13);
     uint32_t tie_run = scratch[11];  // ties at lower positions
     // selected at lower positions
     uint32_t out_run = scratch[10] + (listed ? scratch[13] : min(tie_run, need_eq));
@@ -999,6 +1028,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       out_run += chosen_total;
       __syncthreads();
     }
+    TS_MARK(14);
     // A grid-wide wait of this launch gave up (the workgroups were not all resident
     // within the bound): what was selected is not valid.  The first workgroup of every
     // selecting request says so in place of the length, and in the caller's word.
