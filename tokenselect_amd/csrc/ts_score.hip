@@ -72,9 +72,10 @@ constexpr int kQuadSwap2 = 0x4E;  // quad_perm [2,3,0,1]
 //     the keys stream in costs a quarter of the read bandwidth (DRAM read/write
 //     turnarounds).
 //   kScoreFused (the whole selection in one launch whose workgroups are all
-//     resident at once and meet four to six times): the scores never leave LDS.
+//     resident at once and meet three to five times): the scores never leave LDS.
 //     Every workgroup publishes its per-head (max, sum exp); the (request, head)
-//     pairs are dealt out over the grid and merged; every workgroup turns its own
+//     pairs are dealt out over the grid, merged and written to replicas that the
+//     workgroups poll; every workgroup turns its own
 //     scores into votes (tr.py:361); histogram rounds (11 + 11 + 10 key bits) narrow
 //     the k-th largest vote down until at most 256 candidates are left, which are
 //     listed and ranked by every workgroup together with the counts that tell it
