@@ -29,7 +29,7 @@ def _mirror(wl, extra_tokens):
 
 
 def test_kv_store_paged(dev):
-    """Lengths on and off page boundaries, a full table, three steps in a row: table,
+    """Lengths on and off page boundaries, a full table, fourteen steps in a row: table,
     lengths, free list and the rows in the pools against the oracle."""
     say("paged kv_store: page 16, B=6")
     ps, lens = 16, [32, 15, 16, 31, 100, 47]

@@ -33,15 +33,41 @@ __global__ __launch_bounds__(256) void kv_store_kernel(const uint4* __restrict__
 }
 
 // Chunked prefill (tr.py:725-733): workgroup r copies row r of the chunk to pool
-// slot loc[r] and writes table[len + r]; a second one-thread launch bumps the
-// length, so that every workgroup of the first reads the same old length.  Rows
-// that would not fit the table are dropped; slots are clamped to the pool.
+// slot loc[r] and writes table[len + r].  Every workgroup must read the same old
+// length, and the new one must be there when the launch ends: the workgroups count
+// themselves in the upper bits of the length word itself (a length stays below 2^21,
+// the count below 2^10), everybody masks those bits off, and the workgroup that
+// completes the count writes the new length.  No second launch, no other memory.
+// Rows that would not fit the table are dropped; slots are clamped to the pool.
+constexpr int kLenBits = 21;
+constexpr int kLenMask = (1 << kLenBits) - 1;
+constexpr int kChunkCountedRows = 1023;  // more rows take the two-launch form below
+
+template <bool COUNTED>
 __global__ __launch_bounds__(256) void kv_store_chunk_kernel(
     const uint4* __restrict__ k, const uint4* __restrict__ v, const int32_t* __restrict__ loc,
     uint4* __restrict__ k_pool, uint4* __restrict__ v_pool, int64_t pool_rows,
-    int32_t* __restrict__ table, const int32_t* __restrict__ seq_len, int row_vec, int max_tokens) {
+    int32_t* __restrict__ table, int32_t* seq_len, int row_vec, int max_tokens) {
   const int r = blockIdx.x;
-  const int at = *seq_len + r;
+  int len;
+  if (COUNTED) {
+    // One thread reads the word and then counts the workgroup in; the others take the
+    // length from LDS, so that nobody looks at the word after the last count.
+    __shared__ int s_len;
+    if (threadIdx.x == 0) {
+      s_len = __hip_atomic_load(seq_len, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kLenMask;
+      const int before = __hip_atomic_fetch_add(seq_len, 1 << kLenBits, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+      if ((before >> kLenBits) + 1 == (int)gridDim.x)  // every workgroup has read the length
+        __hip_atomic_store(seq_len, min(s_len + (int)gridDim.x, max_tokens), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    len = s_len;
+  } else {
+    len = *seq_len;
+  }
+  const int at = len + r;
   if (at < 0 || at >= max_tokens) return;
   int64_t slot = loc[r];
   slot = slot < 0 ? 0 : (slot >= pool_rows ? pool_rows - 1 : slot);
@@ -212,9 +238,15 @@ extern "C" int ts_kv_store_chunk(const ts_config* cfg, const void* k, const void
                        page_shift_of(cfg->page_size), page_pool_of(pages));
     return check_launch("kv_store_chunk_paged_kernel");
   }
-  hipLaunchKernelGGL(kv_store_chunk_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream,
-                     (const uint4*)k, (const uint4*)v, out_cache_loc, (uint4*)k_pool, (uint4*)v_pool,
-                     pool_rows, table, seq_len, row_vec, max_tokens);
+  if (rows <= kChunkCountedRows && max_tokens <= kLenMask) {
+    hipLaunchKernelGGL(kv_store_chunk_kernel<true>, dim3((unsigned)rows), dim3(256), 0,
+                       (hipStream_t)stream, (const uint4*)k, (const uint4*)v, out_cache_loc,
+                       (uint4*)k_pool, (uint4*)v_pool, pool_rows, table, seq_len, row_vec, max_tokens);
+    return check_launch("kv_store_chunk_kernel");
+  }
+  hipLaunchKernelGGL(kv_store_chunk_kernel<false>, dim3((unsigned)rows), dim3(256), 0,
+                     (hipStream_t)stream, (const uint4*)k, (const uint4*)v, out_cache_loc,
+                     (uint4*)k_pool, (uint4*)v_pool, pool_rows, table, seq_len, row_vec, max_tokens);
   TS_TRY(check_launch("kv_store_chunk_kernel"));
   hipLaunchKernelGGL(seq_len_add_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, seq_len, rows,
                      max_tokens);
