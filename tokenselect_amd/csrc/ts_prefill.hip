@@ -122,27 +122,36 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
 // rounded to bf16 like the queries) as kr[kvh][j][128] and V transposed as
 // vt[kvh][128][S_pad], so that the attention kernel, whose 32 query tiles would
 // otherwise each repeat the gather, the rotation and the transposition, only copies
-// tiles.  (That repetition made the first version of this kernel bound by vector
-// instructions at 5 % of the matrix peak.)
+// tiles.  Within every block of 32 keys a V^T row is stored in the order in which the
+// attention kernel's matrix instructions want the keys (see kv_pos below).
 //
-// prefill_attn_kernel<G>: grid (16-row query tiles, KV heads, quads of the G query
-// heads of a KV head); 512 threads = two groups of four wavefronts.  The wavefronts
-// of a group serve one query head each and share the K/V tiles of their KV head;
-// group 0 takes the even 64-key tiles and group 1 the odd ones (two wavefronts per
-// SIMD hide each other's LDS and matrix latencies), and their (max, sum, acc) are
-// merged through LDS at the end.  Per tile a group copies 16 KB of kr and 16 KB of vt
-// into one of its two LDS buffers (the pieces of the next two tiles already in
-// registers) while the wavefronts compute on the other: one barrier per tile.  A
-// wavefront computes S^T = K Q^T with v_mfma_f32_16x16x32_bf16 (A = 16 keys x 32 dims
-// from LDS, B = its 16 rotated queries, held in registers, pre-multiplied by the softmax
-// scale and log2 e), which leaves lane (query l%16, key group l/16) with the base-2
-// logits of 16 keys; the online softmax needs two cross-lane maxima per tile; the 16
-// probabilities, rounded to bf16, are directly the B operands of O^T += V^T P^T (A = 16
-// dims x 32 keys from the transposed V tile, keys in the order the logits came in), so
-// no data moves between the two products.  fp32 accumulation throughout.
-// What the time went into, by the counters: neither the matrix units (17 % busy), nor
-// the vector ALU, nor LDS bandwidth, but waiting: bank conflicts of the V^T rows (now
-// padded to 34 banks), and the two barriers per tile of the single-buffered version.
+// prefill_attn_kernel<G>: grid (KV heads, 16-row query tiles, quads of the G query
+// heads of a KV head); 512 threads = four key groups of two wavefronts.  Key group g
+// takes the 32-key tiles g, g + 4, g + 8, ...; its two wavefronts serve two query heads
+// each (two 16 x 128 query blocks held in registers), so that every K and V^T operand
+// read from LDS feeds two matrix instructions.  The four groups' (max, sum, acc) are
+// merged through LDS at the end.
+//
+// Staging: a group's 128 threads bring the next tile of their group (8 KB of kr, 8 KB
+// of vt) from global memory straight into LDS (global_load_lds_dwordx4: 16 bytes per
+// lane, a wavefront fills 1 KB of consecutive LDS; no registers, no LDS store
+// instructions) while the group computes on the tile that arrived during the previous
+// step; one barrier per step, two LDS buffers per group.  Rows are not padded in LDS;
+// instead the 16-byte pieces of a row are permuted (XOR with row bits) so that the 16
+// lanes the hardware serves together when a wavefront reads a matrix operand fall on
+// distinct banks: which global piece a lane fetches is free, where it lands is not.
+//
+// A wavefront computes S^T = K Q^T with v_mfma_f32_16x16x32_bf16 (A = 16 keys x 32 dims
+// from LDS, B = 16 rotated queries of one head, pre-multiplied by the softmax scale and
+// log2 e), which leaves lane (query l%16, key group l/16) with base-2 logits of 8 keys of
+// the tile.  The accumulator starts at minus the running maximum of the row, so the
+// products come out already shifted; the running maximum is only raised when a logit
+// exceeds it by more than 8 (the weights then stay below 2^8, harmless in fp32 sums
+// and invisible after the final division), so the common path per logit is one
+// maximum, one exp2 and half a conversion.  The 8 probabilities, rounded to bf16, are
+// directly the B operand of O^T += V^T P^T (A = 16 dims x 32 keys from the V^T tile);
+// a ninth product with an all-ones A operand accumulates the row sums.  fp32
+// accumulation throughout.
 struct PrefillArgs {
   const uint16_t* q;  // [rows, H, 128] bf16, un-rotated
   const uint16_t* k_pool;
@@ -151,12 +160,12 @@ struct PrefillArgs {
   const int32_t* sel;      // [S] selected slots in attention order
   const int32_t* sel_len;  // device scalar S
   int max_sel_len;
-  int s_pad;               // columns of a vt row: max_sel_len rounded up to the tile
+  int s_pad;               // columns of a vt row: max_sel_len rounded up to kPfPadKeys
   int rows;
   int num_heads, num_kv_heads, rope_mode;
   float log2_theta, rope_rcp_scale, sm_scale, logit_cap;
   uint16_t* kr;   // [Hkv, s_pad, 128] bf16 rotated keys
-  uint16_t* vt;   // [Hkv, 128, s_pad] bf16 transposed values
+  uint16_t* vt;   // [Hkv, 128, s_pad] bf16 transposed values, keys permuted within blocks of 32
   uint16_t* out;  // [rows, H, 128] bf16
 };
 
@@ -164,14 +173,19 @@ typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float pf_f32x4;
 constexpr float kLog2e = 1.4426950408889634f;
 
-constexpr int kPfKeys = 32;               // keys per workgroup of the gather kernel
-constexpr int kPfKRow = kHeadDim + 8;     // halfwords per K row in LDS (272 B: rows on different banks)
-constexpr int kPfVRow = kPfKeys + 8;      // halfwords per V^T row in the gather kernel's LDS (80 B)
-constexpr int kPfTile = 64;               // keys per tile of the attention kernel
-constexpr int kPfPipeA = 2;               // attention tiles whose pieces are in flight
-constexpr int kPfVRowA = kPfTile + 4;     // halfwords per V^T row in the attention kernel's LDS:
-                                          // 136 B = 34 banks, the 16 rows a wavefront reads together
-                                          // (8 bytes each) fall on distinct banks
+constexpr int kPfKeys = 32;            // keys per tile: of the gather kernel and of the attention kernel
+constexpr int kPfVRow = kPfKeys + 8;   // halfwords per V^T row in the gather kernel's LDS (80 B)
+constexpr int kPfPadKeys = 64;         // the staging area holds whole multiples of this many keys
+constexpr int kPfGroups = 4;           // key groups of an attention workgroup
+constexpr int kPfTileBytes = kPfKeys * kHeadDim * 2;  // 8 KB: a K tile; a V^T tile is as large
+constexpr int kPfBufBytes = 2 * kPfTileBytes;         // K tile, then V^T tile
+constexpr size_t kPfLdsBytes = (size_t)kPfGroups * 2 * kPfBufBytes;  // 128 KB
+constexpr float kPfRaise = 8.0f;       // a row's maximum is raised when a logit exceeds it by this much
+
+// Position of key kk (0..31 within its block) in a V^T row: the matrix instruction
+// that made the logits left lane group g4 with keys 16 kb + 4 g4 + r (kb < 2, r < 4),
+// and the next one wants those 8 as one 16-byte operand, in the order 4 kb + r.
+__device__ __forceinline__ int kv_pos(int kk) { return 8 * ((kk >> 2) & 3) + 4 * (kk >> 4) + (kk & 3); }
 
 // Two floats to packed bf16, round to nearest even, in one v_cvt_pk_bf16_f32.
 typedef __attribute__((ext_vector_type(2))) __bf16 pf_bf16x2;
@@ -190,9 +204,9 @@ __global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
   const int kvh = blockIdx.y;
   const int S = min(max(*a.sel_len, 0), a.max_sel_len);
   const int j = blockIdx.x * kPfKeys + kk;
-  // Whole tiles of the attention kernel: the keys between S and the next multiple of
-  // its tile are written as zeros too (their weights are zero, but 0 x garbage is not).
-  if (blockIdx.x * kPfKeys >= (S + kPfTile - 1) / kPfTile * kPfTile) return;
+  // Whole blocks of kPfPadKeys: the keys between S and the next multiple are written as
+  // zeros too (their weights are zero, but 0 x garbage is not).
+  if (blockIdx.x * kPfKeys >= (S + kPfPadKeys - 1) / kPfPadKeys * kPfPadKeys) return;
   const bool live = j < S;
   uint4 kraw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
   uint4 vraw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
@@ -232,15 +246,17 @@ __global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
                                         pack_bf16(lo[4], lo[5]), pack_bf16(lo[6], lo[7]));
   *(uint4*)(krow + 64 + 8 * c8) = make_uint4(pack_bf16(hi[0], hi[1]), pack_bf16(hi[2], hi[3]),
                                              pack_bf16(hi[4], hi[5]), pack_bf16(hi[6], hi[7]));
-  // transpose the 32 x 128 V tile through LDS, then write 128 rows of 64 bytes
+  // transpose the 32 x 128 V tile through LDS (key kk to column kv_pos(kk)), then write
+  // 128 rows of 64 bytes
   const uint32_t vlo[4] = {vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w};
   const uint32_t vhi[4] = {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w};
+  const int col = kv_pos(kk);
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    vt_lds[(8 * c8 + 2 * e) * kPfVRow + kk] = (uint16_t)(vlo[e] & 0xffffu);
-    vt_lds[(8 * c8 + 2 * e + 1) * kPfVRow + kk] = (uint16_t)(vlo[e] >> 16);
-    vt_lds[(64 + 8 * c8 + 2 * e) * kPfVRow + kk] = (uint16_t)(vhi[e] & 0xffffu);
-    vt_lds[(64 + 8 * c8 + 2 * e + 1) * kPfVRow + kk] = (uint16_t)(vhi[e] >> 16);
+    vt_lds[(8 * c8 + 2 * e) * kPfVRow + col] = (uint16_t)(vlo[e] & 0xffffu);
+    vt_lds[(8 * c8 + 2 * e + 1) * kPfVRow + col] = (uint16_t)(vlo[e] >> 16);
+    vt_lds[(64 + 8 * c8 + 2 * e) * kPfVRow + col] = (uint16_t)(vhi[e] & 0xffffu);
+    vt_lds[(64 + 8 * c8 + 2 * e + 1) * kPfVRow + col] = (uint16_t)(vhi[e] >> 16);
   }
   __syncthreads();
   const int d = tid >> 1, half = tid & 1;
@@ -250,61 +266,136 @@ __global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
   ((uint4*)vrow)[1] = src[1];
 }
 
+typedef void __attribute__((address_space(3)))* pf_lds_ptr;
+
+// 16 bytes per lane from global memory straight into LDS: lane l's piece lands at LDS
+// byte address lds_dst + 16 l (lds_dst the same for the whole wavefront, passed in M0).
+// Written as assembly and not through the compiler's builtin on purpose: the compiler
+// makes every later LDS read wait for all such loads (it cannot tell that they fill the
+// other buffer), which serialises exactly what is meant to overlap.  The waits are
+// explicit instead: s_waitcnt vmcnt(0) before the barrier that hands a buffer over.
+__device__ __forceinline__ void load_to_lds16(const void* src, uint32_t lds_dst) {
+  uint32_t saved_m0;  // M0 is the compiler's; it gets it back
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+      : "=&s"(saved_m0)
+      : "s"(lds_dst), "v"(src)
+      : "memory");
+}
+
+// Largest of three, without the NaN-quieting copies fmaxf brings along.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float d;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+  return d;
+}
+
 // Two wavefronts per SIMD by construction (8 per workgroup, one workgroup per CU):
-// saying so lets the compiler use 256 registers instead of spilling at 128.
+// saying so lets the compiler use 256 registers.
 template <int G, bool CAP>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(
     PrefillArgs a) {
-  // Dynamic LDS: per group two buffers of a K tile [kPfTile * kPfKRow] followed by a V^T
-  // tile [kHeadDim * kPfVRowA]; the merge of the two groups at the end reuses the space.
+  // Dynamic LDS: per key group two buffers, each a K tile [32 keys][256 B] followed by a
+  // V^T tile [128 dims][64 B]; the merge of the groups at the end reuses the space.
   extern __shared__ __attribute__((aligned(16))) uint16_t pf_lds[];
-  constexpr int kBuf = kPfTile * kPfKRow + kHeadDim * kPfVRowA;  // halfwords per buffer
-  const int group = threadIdx.x >> 8;  // which of the two tile streams this wavefront follows
-  uint16_t* const k_lds = pf_lds + group * (2 * kBuf);
-  uint16_t* const vt_lds = k_lds + kPfTile * kPfKRow;
-  float(*merge_lds)[64][34] = (float(*)[64][34])pf_lds;  // [4][64][34]
-  static_assert(4 * 64 * 34 * 4 <= 4 * kBuf * 2, "the merge area fits the tiles");
-
-  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
-  const int qc = lane & 15, g4 = lane >> 4;  // query column / key group of the MFMA layouts
-  const int kvh = blockIdx.y;
-  const int head_in_group = blockIdx.z * 4 + wave;
-  const bool wave_active = head_in_group < G;
-  const int h = kvh * G + (wave_active ? head_in_group : 0);
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int lane = threadIdx.x & 63;
+  const int group = wave >> 1;  // which of the four tile streams this wavefront follows
+  const int hp = wave & 1;      // which pair of the quad's heads it serves
+  const int qc = lane & 15, g4 = lane >> 4;  // query column / key group of the matrix layouts
+  // The KV head is the fastest-moving workgroup index: consecutive workgroups go to
+  // consecutive XCDs, so with eight KV heads each XCD's L2 holds the keys and values of one
+  // head (1.4 MB of 11 MB) and every query tile of that head finds them there.  The last
+  // query tiles, which see the most keys, start first.
+  const int kvh = blockIdx.x;
+  const int q_row0 = (int)(gridDim.y - 1 - blockIdx.y) * 16;
   const int H = a.num_heads;
+  char* const group_lds = (char*)pf_lds + group * (2 * kPfBufBytes);
+  const uint32_t group_lds_at = (uint32_t)(uintptr_t)(pf_lds_ptr)pf_lds + (uint32_t)(group * (2 * kPfBufBytes));
+
+  // ---- staging role.  K tile: wavefront hp of the group fills the 1 KB blocks 4 hp + i
+  // (i < 4; a block is 4 keys), lane l the piece (key l/16 of the block, slot l%16), which
+  // holds the dims [8 c, 8 c + 8) with c = slot ^ (key & 15).  V^T tile: blocks of 16 dims,
+  // lane l the piece (dim l/4 of the block, slot l%4) = keys [8 c, +8) of the tile in vt's
+  // order, c = slot ^ ((dim / 4) & 3).
+  uint32_t k_src[4], v_src[4];
+  {
+    const int key_in_block = lane >> 4, slot = lane & 15;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = 4 * (4 * hp + i) + key_in_block;
+      k_src[i] = (uint32_t)(key * kHeadDim + 8 * (slot ^ (key & 15))) * 2u;
+    }
+    const int dim_in_block = lane >> 2, vslot = lane & 3;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int dim = 16 * (4 * hp + i) + dim_in_block;
+      v_src[i] = (uint32_t)(dim * a.s_pad + 8 * (vslot ^ ((dim >> 2) & 3))) * 2u;
+    }
+  }
+  const char* const k_base = (const char*)(a.kr + (size_t)kvh * a.s_pad * kHeadDim);
+  const char* const v_base = (const char*)(a.vt + (size_t)kvh * kHeadDim * a.s_pad);
+  auto request_tile = [&](int step, int buf) __attribute__((always_inline)) {
+    // past the end: a harmless repeat of the last tile
+    const int tile = min((step * kPfGroups + group) * kPfKeys, a.s_pad - kPfKeys);
+    const uint32_t dst = group_lds_at + (uint32_t)(buf * kPfBufBytes + (4 * hp) * 1024);
+    const char* const ks = k_base + (size_t)tile * (kHeadDim * 2);
+    const char* const vs = v_base + (size_t)tile * 2;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_to_lds16(ks + k_src[i], dst + (uint32_t)(i * 1024));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_to_lds16(vs + v_src[i], dst + (uint32_t)(kPfTileBytes + i * 1024));
+  };
+  request_tile(0, 0);  // on its way while the queries are prepared
+
   const int S = min(max(*a.sel_len, 0), a.max_sel_len);
   const int m = a.rows;
-  const int q_row0 = blockIdx.x * 16;
   const int shift = S - m;  // query row i sits at position shift + i and sees keys <= that
   const bool rope = a.rope_mode == TS_ROPE_LLAMA;
+  int head[2];
+  bool head_active[2];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+    const int head_in_group = blockIdx.z * 4 + 2 * hp + rb;
+    head_active[rb] = head_in_group < G;
+    head[rb] = kvh * G + (head_active[rb] ? head_in_group : 0);
+  }
+  const bool wave_active = head_active[0];
   if (S < m || S <= 0) {
     // Fewer keys than rows (not a prefill chunk, or a selection that reported a
     // fault): the rows attend to nothing and the output is defined as zero.
-    if (wave_active)
-      for (int i = lane; i < 16 * (kHeadDim / 8); i += 64) {
-        const int row = q_row0 + i / (kHeadDim / 8);
-        if (row < m)
-          *(uint4*)(a.out + ((size_t)row * H + h) * kHeadDim + 8 * (i % (kHeadDim / 8))) =
-              make_uint4(0u, 0u, 0u, 0u);
-      }
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+      if (head_active[rb])
+        for (int i = lane; i < 16 * (kHeadDim / 8); i += 64) {
+          const int row = q_row0 + i / (kHeadDim / 8);
+          if (row < m)
+            *(uint4*)(a.out + ((size_t)row * H + head[rb]) * kHeadDim + 8 * (i % (kHeadDim / 8))) =
+                make_uint4(0u, 0u, 0u, 0u);
+        }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the tile on its way lands before the LDS is given up
     return;
   }
 
-  // ---- queries: B operand, lane (qc, g4) holds dims [32 ks + 8 g4, +8) of row q_row0 + qc,
-  // rotated to position shift + row (partner dims d and d + 64 are k-steps ks and ks + 2).
+  // ---- queries: B operand, lane (qc, g4) holds dims [32 ks + 8 g4, +8) of row q_row0 + qc
+  // of each of its two heads, rotated to position shift + row (partner dims d and d + 64 are
+  // k-steps ks and ks + 2; the angles are the same for both heads).
   const int q_row = min(q_row0 + qc, m - 1);
-  pf_bf16x8 qb[4];
+  pf_bf16x8 qb[2][4];
   {
-    float x[4][8];
-    const uint16_t* qrow = a.q + ((size_t)q_row * H + h) * kHeadDim;
+    float x[2][4][8];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const uint4 w = *(const uint4*)(qrow + 32 * ks + 8 * g4);
-      const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+    for (int rb = 0; rb < 2; ++rb) {
+      const uint16_t* qrow = a.q + ((size_t)q_row * H + head[rb]) * kHeadDim;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        x[ks][2 * e] = bf16_lo(ww[e]);
-        x[ks][2 * e + 1] = bf16_hi(ww[e]);
+      for (int ks = 0; ks < 4; ++ks) {
+        const uint4 w = *(const uint4*)(qrow + 32 * ks + 8 * g4);
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          x[rb][ks][2 * e] = bf16_lo(ww[e]);
+          x[rb][ks][2 * e + 1] = bf16_hi(ww[e]);
+        }
       }
     }
     if (rope) {
@@ -317,224 +408,218 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           const float freq = a.rope_rcp_scale * exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
           float sn, cs;
           sincos_reduced(pos * freq, sn, cs);
-          const float lo = x[ks][e], hi = x[ks + 2][e];
-          x[ks][e] = lo * cs - hi * sn;
-          x[ks + 2][e] = hi * cs + lo * sn;
+#pragma unroll
+          for (int rb = 0; rb < 2; ++rb) {
+            const float lo = x[rb][ks][e], hi = x[rb][ks + 2][e];
+            x[rb][ks][e] = lo * cs - hi * sn;
+            x[rb][ks + 2][e] = hi * cs + lo * sn;
+          }
         }
     }
     // Without a soft cap the softmax scale and log2(e) go into the query, so that the
     // products come out as base-2 logits and every key costs one exp2 and no multiply.
     const float qs = CAP ? 1.0f : a.sm_scale * kLog2e;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
+    for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) x[ks][e] *= qs;
-      const uint4 w = make_uint4(pack_bf16(x[ks][0], x[ks][1]), pack_bf16(x[ks][2], x[ks][3]),
-                                 pack_bf16(x[ks][4], x[ks][5]), pack_bf16(x[ks][6], x[ks][7]));
-      qb[ks] = __builtin_bit_cast(pf_bf16x8, w);
-    }
+      for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[rb][ks][e] *= qs;
+        const uint4 w = make_uint4(pack_bf16(x[rb][ks][0], x[rb][ks][1]), pack_bf16(x[rb][ks][2], x[rb][ks][3]),
+                                   pack_bf16(x[rb][ks][4], x[rb][ks][5]), pack_bf16(x[rb][ks][6], x[rb][ks][7]));
+        qb[rb][ks] = __builtin_bit_cast(pf_bf16x8, w);
+      }
   }
 
-  // ---- staging role: thread t copies four 16-byte pieces of the K tile (keys t/8 and
-  // t/8 + 32, dims [8 (t%8), +8) and the same 64 dims further on: consecutive lanes write
-  // consecutive 16 bytes of a K row, which the LDS banks take without conflicts) and 64
-  // bytes of the V^T tile (dim t/2, keys [32 (t%2), +32)).
-  const uint16_t* k_src = a.kr + (size_t)kvh * a.s_pad * kHeadDim + (size_t)(tid >> 3) * kHeadDim +
-                          8 * (tid & 7);
-  const uint16_t* v_src = a.vt + ((size_t)kvh * kHeadDim + (tid >> 1)) * a.s_pad + 32 * (tid & 1);
-  uint16_t* k_dst = k_lds + (tid >> 3) * kPfKRow + 8 * (tid & 7);
-  uint16_t* v_dst = vt_lds + (tid >> 1) * kPfVRowA + 32 * (tid & 1);  // 8-byte aligned
-  // Two register buffers, named rather than indexed: an indexed array of them is
-  // kept in scratch memory by the compiler, and the prefetch with it.
-  struct TilePiece {
-    uint4 k0, k1, k2, k3, v0, v1, v2, v3;
-  };
-  TilePiece piece0, piece1;
-  auto request_tile = [&](int tile) __attribute__((always_inline)) -> TilePiece {
-    tile = min(tile, a.s_pad - kPfTile);  // past the end: harmless repeat of the last tile
-    const uint4* ks = (const uint4*)(k_src + (size_t)tile * kHeadDim);
-    const uint4* vs = (const uint4*)(v_src + tile);
-    TilePiece piece;
-    piece.k0 = ks[0];
-    piece.k1 = ks[8];                      // 64 dims further on
-    piece.k2 = ks[32 * kHeadDim / 8];      // 32 keys further on
-    piece.k3 = ks[32 * kHeadDim / 8 + 8];
-    piece.v0 = vs[0];
-    piece.v1 = vs[1];
-    piece.v2 = vs[2];
-    piece.v3 = vs[3];
-    return piece;
-  };
+  // ---- reading role: where this lane's operands sit in a buffer.  K operand (kb, ks): key
+  // 16 kb + qc, dims [32 ks + 8 g4, +8) = piece 4 ks + g4, in slot (4 ks + g4) ^ qc.  V^T
+  // operand db: dim 16 db + qc, piece g4, in slot g4 ^ ((qc / 4) & 3).
+  uint32_t k_at[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) k_at[ks] = (uint32_t)(qc * (kHeadDim * 2) + 16 * ((4 * ks + g4) ^ qc));
+  const uint32_t v_at = (uint32_t)(kPfTileBytes + qc * (kPfKeys * 2) + 16 * (g4 ^ ((qc >> 2) & 3)));
 
   // ---- main loop over the tiles any row of this query tile can see
   const int last_visible = min(S - 1, shift + min(q_row0 + 15, m - 1));
   const int my_limit = shift + q_row;  // last key this lane's query sees
-  float m_run = kNegBig, l_run = 0.f;
-  pf_f32x4 o[8];
+  const int steps = last_visible / (kPfGroups * kPfKeys) + 1;
+  float m_run[2] = {kNegBig, kNegBig};  // kNegBig: no maximum yet
+  pf_f32x4 o[2][8], row_sum[2];
 #pragma unroll
-  for (int db = 0; db < 8; ++db) o[db] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rb = 0; rb < 2; ++rb) {
+    row_sum[rb] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int db = 0; db < 8; ++db) o[rb][db] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const pf_bf16x8 ones = __builtin_bit_cast(pf_bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
 
-  // One 64-key tile of this group: logits, online softmax, output update.
+  // One 32-key tile of this group: logits, online softmax, output update, for both heads.
   auto compute_tile = [&](int tile, int buf) __attribute__((always_inline)) {
-    const uint16_t* const kt = k_lds + buf * kBuf;
-    const uint16_t* const vt = vt_lds + buf * kBuf;
-    // logits (base 2): s[blk][r] belongs to key tile + 16 blk + 4 g4 + r and query qc.
+    const char* const base = group_lds + buf * kPfBufBytes;
     // Only the tiles on the diagonal hold keys that some query of the tile must not see.
-    const bool diagonal = tile + kPfTile - 1 > shift + q_row0;
-    float s[4][4];
+    const bool diagonal = tile + kPfKeys - 1 > shift + q_row0;
+    pf_f32x4 s[2][2];  // [head][key block]: key tile + 16 kb + 4 g4 + r, query qc
+    float m_base[2];
 #pragma unroll
-    for (int blk = 0; blk < 4; ++blk) {
-      pf_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int rb = 0; rb < 2; ++rb) {
+      m_base[rb] = m_run[rb] == kNegBig ? 0.f : m_run[rb];
+      const float c0 = CAP ? 0.f : -m_base[rb];
+      s[rb][0] = pf_f32x4{c0, c0, c0, c0};
+      s[rb][1] = s[rb][0];
+    }
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
-        const uint4 kw = *(const uint4*)(kt + (16 * blk + qc) * kPfKRow + 32 * ks + 8 * g4);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, kw), qb[ks],
-                                                      acc, 0, 0, 0);
+        const uint4 kw = *(const uint4*)(base + kb * (16 * kHeadDim * 2) + k_at[ks]);
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+          s[rb][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, kw), qb[rb][ks],
+                                                             s[rb][kb], 0, 0, 0);
       }
+    uint4 vw[8];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float x = acc[r];
-        if (CAP) x = a.logit_cap * tanhf(x * a.sm_scale / a.logit_cap) * kLog2e;
-        const int key = tile + 16 * blk + 4 * g4 + r;
-        // Masked logits are -inf and the running maximum starts at a finite value,
-        // so exp2(s - max) is 0 for them without a branch and never NaN.
-        s[blk][r] = (!diagonal || key <= my_limit) ? x : -INFINITY;
+    for (int db = 0; db < 8; ++db) vw[db] = *(const uint4*)(base + db * (16 * kPfKeys * 2) + v_at);
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+      if (CAP) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            s[rb][kb][r] = a.logit_cap * tanhf(s[rb][kb][r] * a.sm_scale / a.logit_cap) * kLog2e - m_base[rb];
       }
-    }
-    float mx = kNegBig;
+      if (diagonal) {
+        // Masked logits are -inf: exp2 makes them 0 without a branch.
 #pragma unroll
-    for (int blk = 0; blk < 4; ++blk)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[blk][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    float p[4][4], psum = 0.f;
-#pragma unroll
-    for (int blk = 0; blk < 4; ++blk)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        p[blk][r] = __builtin_amdgcn_exp2f(s[blk][r] - m_new);
-        psum += p[blk][r];
+          for (int r = 0; r < 4; ++r)
+            if (tile + 16 * kb + 4 * g4 + r > my_limit) s[rb][kb][r] = -INFINITY;
       }
-    l_run = l_run * alpha + psum;
-    // The accumulators only need rescaling when some query's maximum moved, which
-    // after the first tiles is rare: skip the 32 multiplications otherwise.
-    const bool rescale = __ballot(m_new != m_run) != 0ull;
-    m_run = m_new;
-    pf_bf16x8 pb[2];
+      float mx = max3(s[rb][0][0], s[rb][0][1], s[rb][0][2]);
+      mx = max3(mx, s[rb][0][3], s[rb][1][0]);
+      mx = max3(mx, s[rb][1][1], s[rb][1][2]);
+      mx = fmaxf(mx, s[rb][1][3]);
+      const bool unset = m_run[rb] == kNegBig;
+      if (__ballot(unset || mx > kPfRaise) != 0ull) {
+        // Some row of this head has no maximum yet, or outgrew it: agree on the row's
+        // maximum over the four key groups of lanes and move to it.
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const bool take = unset ? mx > -INFINITY : mx > kPfRaise;
+        const float delta = take ? mx : 0.f;
+        // (a row without a maximum has only zeros in its accumulators)
+        const float scale = unset ? 1.0f : __builtin_amdgcn_exp2f(-delta);
+        if (take) m_run[rb] = m_base[rb] + delta;
 #pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      const uint4 pw = make_uint4(pack_bf16(p[2 * hf][0], p[2 * hf][1]),
-                                  pack_bf16(p[2 * hf][2], p[2 * hf][3]),
-                                  pack_bf16(p[2 * hf + 1][0], p[2 * hf + 1][1]),
-                                  pack_bf16(p[2 * hf + 1][2], p[2 * hf + 1][3]));
-      pb[hf] = __builtin_bit_cast(pf_bf16x8, pw);
-    }
-    if (rescale) {
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[rb][kb][r] -= delta;
+#pragma unroll
+        for (int db = 0; db < 8; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[rb][db][r] *= scale;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) row_sum[rb][r] *= scale;
+      }
+      float p[2][4];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) p[kb][r] = __builtin_amdgcn_exp2f(s[rb][kb][r]);
+      const uint4 pw = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]),
+                                  pack_bf16(p[1][0], p[1][1]), pack_bf16(p[1][2], p[1][3]));
+      const pf_bf16x8 pb = __builtin_bit_cast(pf_bf16x8, pw);
 #pragma unroll
       for (int db = 0; db < 8; ++db)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[db][r] *= alpha;
-    }
-#pragma unroll
-    for (int db = 0; db < 8; ++db) {
-      const uint16_t* vrow = vt + (16 * db + qc) * kPfVRowA;
-#pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        const uint2 v0 = *(const uint2*)(vrow + 32 * hf + 4 * g4);
-        const uint2 v1 = *(const uint2*)(vrow + 32 * hf + 16 + 4 * g4);
-        const uint4 vw = make_uint4(v0.x, v0.y, v1.x, v1.y);
-        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw), pb[hf],
-                                                        o[db], 0, 0, 0);
-      }
+        o[rb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw[db]), pb,
+                                                           o[rb][db], 0, 0, 0);
+      row_sum[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb, row_sum[rb], 0, 0, 0);
     }
   };
 
-  // The LDS tiles are double-buffered: while the wavefronts compute on one buffer, the
-  // next tile (its pieces already in registers) is written to the other, and one
-  // barrier per tile separates "everybody has read buffer b" from its next overwrite.
-  // Tile number i of this group (keys (2 i + group) * 64 ...) travels through register
-  // buffer i % 2 and LDS buffer i % 2; the steps are written out for the two parities so
-  // that each uses its own named registers.
-  static_assert(kPfPipeA == 2, "the steps below are written out for two buffers");
-#define TS_PF_STORE(u, buf)                                                                  \
-  {                                                                                          \
-    uint16_t* const kd = k_dst + (buf) * kBuf;                                               \
-    uint16_t* const vd = v_dst + (buf) * kBuf;                                               \
-    ((uint4*)kd)[0] = piece##u.k0;                                                           \
-    ((uint4*)kd)[8] = piece##u.k1;                                                           \
-    ((uint4*)(kd + 32 * kPfKRow))[0] = piece##u.k2;                                          \
-    ((uint4*)(kd + 32 * kPfKRow))[8] = piece##u.k3;                                          \
-    ((uint2*)vd)[0] = make_uint2(piece##u.v0.x, piece##u.v0.y);                              \
-    ((uint2*)vd)[1] = make_uint2(piece##u.v0.z, piece##u.v0.w);                              \
-    ((uint2*)vd)[2] = make_uint2(piece##u.v1.x, piece##u.v1.y);                              \
-    ((uint2*)vd)[3] = make_uint2(piece##u.v1.z, piece##u.v1.w);                              \
-    ((uint2*)vd)[4] = make_uint2(piece##u.v2.x, piece##u.v2.y);                              \
-    ((uint2*)vd)[5] = make_uint2(piece##u.v2.z, piece##u.v2.w);                              \
-    ((uint2*)vd)[6] = make_uint2(piece##u.v3.x, piece##u.v3.y);                              \
-    ((uint2*)vd)[7] = make_uint2(piece##u.v3.z, piece##u.v3.w);                              \
-  }
-  // Step for the tile in LDS buffer `cur`: stage the following tile from register buffer
-  // `nxt` into LDS buffer `nxt`, request the tile after that, compute, barrier.
-#define TS_PF_STEP(cur, nxt)                                                                 \
-  {                                                                                          \
-    const int pair = round + 2 * kPfTile * (cur);                                            \
-    if (pair > last_visible) break;                                                          \
-    const int tile = pair + kPfTile * group;                                                 \
-    TS_PF_STORE(nxt, nxt)                                                                    \
-    piece##nxt = request_tile(tile + 3 * 2 * kPfTile);                                       \
-    if (wave_active && tile <= last_visible) compute_tile(tile, cur);                        \
-    __syncthreads();                                                                         \
-  }
-  piece0 = request_tile(kPfTile * (0 + group));
-  piece1 = request_tile(kPfTile * (2 + group));
-  TS_PF_STORE(0, 0)
-  piece0 = request_tile(kPfTile * (4 + group));
+  // The tile requested during step i - 1 is computed on in step i.  The two wavefronts of
+  // a key group keep in step through two counters in LDS and no barrier, so that the four
+  // groups drift apart and the two wavefronts of a SIMD (which belong to different
+  // groups) are rarely in the same phase: one's matrix instructions run under the other's
+  // softmax.  landed = pieces of tiles that have arrived (each wavefront counts its own
+  // after waiting for them), read = tiles a wavefront has finished reading.  Tile i may be
+  // read when landed >= 2 (i + 1); the buffer of tile i - 1 may be overwritten (by the
+  // request for tile i + 1) when read >= 2 i.  Neither wait can last: a partner is at most
+  // one step behind.  The waits are bounded all the same, so that a mistake here would
+  // show as a wrong result and not as a hang.
+  __shared__ uint32_t pf_sync[kPfGroups][2];
+  if (threadIdx.x < 2 * kPfGroups) (&pf_sync[0][0])[threadIdx.x] = 0u;
   __syncthreads();
-  for (int round = 0; round <= last_visible; round += 2 * kPfPipeA * kPfTile) {
-    TS_PF_STEP(0, 1)
-    TS_PF_STEP(1, 0)
-  }
-#undef TS_PF_STEP
-#undef TS_PF_STORE
-  // (the barrier that ended the last step also freed the tiles' space for the merge)
-  // Group 1 hands its partial result to group 0 (same wavefront index, same lane).
-  if (group == 1) {
-    float* mine = merge_lds[wave][lane];
-    mine[0] = m_run;
-    mine[1] = l_run;
-#pragma unroll
-    for (int db = 0; db < 8; ++db)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) mine[2 + 4 * db + r] = o[db][r];
+  uint32_t* const landed = &pf_sync[group][0];
+  uint32_t* const was_read = &pf_sync[group][1];
+  for (int step = 0; step < steps; ++step) {
+    const int buf = step & 1;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (lane == 0) __hip_atomic_fetch_add(landed, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    for (int spin = 0; spin < (1 << 20); ++spin) {
+      const uint32_t have = __hip_atomic_load(landed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      const uint32_t freed = __hip_atomic_load(was_read, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (have >= 2u * (uint32_t)(step + 1) && freed >= 2u * (uint32_t)step) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (step + 1 < steps) request_tile(step + 1, buf ^ 1);
+    const int tile = (step * kPfGroups + group) * kPfKeys;
+    if (wave_active && tile <= last_visible) compute_tile(tile, buf);
+    if (lane == 0) __hip_atomic_fetch_add(was_read, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
   }
   __syncthreads();
-  if (group == 1 || !wave_active || q_row0 + qc >= m) return;
-  {
-    const float* other = merge_lds[wave][lane];
-    const float m_new = fmaxf(m_run, other[0]);
-    const float e0 = __builtin_amdgcn_exp2f(m_run - m_new), e1 = __builtin_amdgcn_exp2f(other[0] - m_new);
-    l_run = l_run * e0 + other[1] * e1;
+
+  // ---- merge of the four key groups (the barrier that ended the last step also freed
+  // the tiles' space): groups 1..3 hand their partial results to group 0 (same head pair,
+  // same lane), 18 vectors of four floats per lane: per head 8 of acc and (max, sum).
+  pf_f32x4* const merge = (pf_f32x4*)pf_lds;  // [(group - 1) * 2 + hp][18][64 lanes]
+  static_assert(6 * 18 * 64 * 16 <= kPfLdsBytes, "the merge area fits the tiles");
+  if (group != 0) {
+    pf_f32x4* const mine = merge + ((group - 1) * 2 + hp) * (18 * 64) + lane;
 #pragma unroll
-    for (int db = 0; db < 8; ++db)
+    for (int rb = 0; rb < 2; ++rb) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[db][r] = o[db][r] * e0 + other[2 + 4 * db + r] * e1;
+      for (int db = 0; db < 8; ++db) mine[(9 * rb + db) * 64] = o[rb][db];
+      mine[(9 * rb + 8) * 64] = pf_f32x4{m_run[rb], row_sum[rb][0], 0.f, 0.f};
+    }
+  }
+  __syncthreads();
+  if (group != 0 || !wave_active) return;
+  float l_run[2] = {row_sum[0][0], row_sum[1][0]};
+#pragma unroll
+  for (int g = 1; g < kPfGroups; ++g) {
+    const pf_f32x4* const other = merge + ((g - 1) * 2 + hp) * (18 * 64) + lane;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+      const pf_f32x4 ml = other[(9 * rb + 8) * 64];
+      const float m_new = fmaxf(m_run[rb], ml[0]);
+      const float e0 = __builtin_amdgcn_exp2f(m_run[rb] - m_new), e1 = __builtin_amdgcn_exp2f(ml[0] - m_new);
+      m_run[rb] = m_new;
+      l_run[rb] = l_run[rb] * e0 + ml[1] * e1;
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+        const pf_f32x4 od = other[(9 * rb + db) * 64];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[rb][db][r] = o[rb][db][r] * e0 + od[r] * e1;
+      }
+    }
   }
 
-  // o[db][r] = O[query qc][dim 16 db + 4 g4 + r]; the row sum is spread over the 4 key groups.
-  float l_tot = l_run + __shfl_xor(l_run, 16);
-  l_tot += __shfl_xor(l_tot, 32);
-  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-  uint16_t* orow = a.out + ((size_t)(q_row0 + qc) * H + h) * kHeadDim;
+  // o[rb][db][r] = O[query qc][dim 16 db + 4 g4 + r] of head rb; the row sum is complete in every lane.
+  if (q_row0 + qc >= m) return;
 #pragma unroll
-  for (int db = 0; db < 8; ++db)
-    *(uint2*)(orow + 16 * db + 4 * g4) = make_uint2(pack_bf16(o[db][0] * inv, o[db][1] * inv),
-                                                    pack_bf16(o[db][2] * inv, o[db][3] * inv));
+  for (int rb = 0; rb < 2; ++rb) {
+    if (!head_active[rb]) continue;
+    const float inv = l_run[rb] > 0.f ? 1.0f / l_run[rb] : 0.f;
+    uint16_t* orow = a.out + ((size_t)(q_row0 + qc) * H + head[rb]) * kHeadDim;
+#pragma unroll
+    for (int db = 0; db < 8; ++db)
+      *(uint2*)(orow + 16 * db + 4 * g4) = make_uint2(pack_bf16(o[rb][db][0] * inv, o[rb][db][1] * inv),
+                                                      pack_bf16(o[rb][db][2] * inv, o[rb][db][3] * inv));
+  }
 }
-
-constexpr size_t kPfLdsBytes = 2 * 2 * (size_t)(kPfTile * kPfKRow + kHeadDim * kPfVRowA) * 2;
 
 int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
                        const float* sin_table, int64_t table_rows, void* qf, const ZeroRegion& zero,
@@ -551,7 +636,7 @@ int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const 
   return check_launch("fingerprint_kernel");
 }
 
-static int prefill_s_pad(int max_sel_len) { return (int)ceil_div(max_sel_len, kPfTile) * kPfTile; }
+static int prefill_s_pad(int max_sel_len) { return (int)ceil_div(max_sel_len, kPfPadKeys) * kPfPadKeys; }
 
 }  // namespace ts
 
@@ -610,7 +695,7 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
                      dim3(256), 0, st, a);
   TS_TRY(check_launch("prefill_gather_kernel"));
   const int group = cfg->num_heads / cfg->num_kv_heads;
-  const dim3 grid((unsigned)ceil_div(rows, 16), (unsigned)cfg->num_kv_heads,
+  const dim3 grid((unsigned)cfg->num_kv_heads, (unsigned)ceil_div(rows, 16),
                   (unsigned)ceil_div(group, 4));
   const bool cap = cfg->logit_cap > 0.f;
 #define TS_PF_LAUNCH(G_, C_)                                                                  \
