@@ -4,6 +4,8 @@
 // prefill, tr.py:759-771, page size 1, in-kernel Llama RoPE).
 #include <math.h>
 
+#include <type_traits>
+
 #include "ts_common.h"
 
 namespace ts {
@@ -180,6 +182,7 @@ constexpr int kPfGroups = 4;           // key groups of an attention workgroup
 constexpr int kPfTileBytes = kPfKeys * kHeadDim * 2;  // 8 KB: a K tile; a V^T tile is as large
 constexpr int kPfBufBytes = 2 * kPfTileBytes;         // K tile, then V^T tile
 constexpr size_t kPfLdsBytes = (size_t)kPfGroups * 2 * kPfBufBytes;  // 128 KB
+constexpr int kPfHeads = 2;            // query heads per wavefront of the attention kernel
 constexpr float kPfRaise = 8.0f;       // a row's maximum is raised when a logit exceeds it by this much
 
 // Position of key kk (0..31 within its block) in a V^T row: the matrix instruction
@@ -274,13 +277,46 @@ typedef void __attribute__((address_space(3)))* pf_lds_ptr;
 // makes every later LDS read wait for all such loads (it cannot tell that they fill the
 // other buffer), which serialises exactly what is meant to overlap.  The waits are
 // explicit instead: s_waitcnt vmcnt(0) before the barrier that hands a buffer over.
-__device__ __forceinline__ void load_to_lds16(const void* src, uint32_t lds_dst) {
+// The source is base (the same for the whole wavefront) + offset (per lane).  N pieces per
+// lane with one write of M0: the instruction's offset field moves both addresses, so piece
+// i lands 1 KB after piece i - 1, and its source offset is passed 1024 i too small.
+// A wavefront issues one instruction per four cycles at best, whatever its kind, and
+// the loop around these loads is bound by exactly that: every scalar instruction counts.
+template <int N>
+__device__ __forceinline__ void load_to_lds16(const void* base, const uint32_t (&offset)[N], uint32_t lds_dst) {
+  static_assert(N == 2 || N == 4, "two or four pieces");
   uint32_t saved_m0;  // M0 is the compiler's; it gets it back
-  asm volatile(
-      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
-      : "=&s"(saved_m0)
-      : "s"(lds_dst), "v"(src)
-      : "memory");
+  if (N == 4)
+    asm volatile(
+        "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+        "global_load_lds_dwordx4 %2, %6\n\t"
+        "global_load_lds_dwordx4 %3, %6 offset:1024\n\t"
+        "global_load_lds_dwordx4 %4, %6 offset:2048\n\t"
+        "global_load_lds_dwordx4 %5, %6 offset:3072\n\t"
+        "s_mov_b32 m0, %0"
+        : "=&s"(saved_m0)
+        : "s"(lds_dst), "v"(offset[0]), "v"(offset[1]), "v"(offset[N == 4 ? 2 : 0]), "v"(offset[N == 4 ? 3 : 1]),
+          "s"(base)
+        : "memory");
+  else
+    asm volatile(
+        "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+        "global_load_lds_dwordx4 %2, %4\n\t"
+        "global_load_lds_dwordx4 %3, %4 offset:1024\n\t"
+        "s_mov_b32 m0, %0"
+        : "=&s"(saved_m0)
+        : "s"(lds_dst), "v"(offset[0]), "v"(offset[1]), "s"(base)
+        : "memory");
+}
+
+// One lane adds 1 to a counter in LDS.  LDS instructions of a wavefront are carried out in
+// order, so the reads before it have been served when the addition is.
+__device__ __forceinline__ void lds_count(uint32_t lds_at_vgpr, uint32_t one_vgpr) {
+  uint64_t saved_exec;
+  asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 1\n\tds_add_u32 %1, %2\n\ts_mov_b64 exec, %0"
+               : "=&s"(saved_exec)
+               : "v"(lds_at_vgpr), "v"(one_vgpr)
+               : "memory");
 }
 
 // Largest of three, without the NaN-quieting copies fmaxf brings along.
@@ -290,18 +326,22 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return d;
 }
 
-// Two wavefronts per SIMD by construction (8 per workgroup, one workgroup per CU):
-// saying so lets the compiler use 256 registers.
-template <int G, bool CAP>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(
-    PrefillArgs a) {
+// HEADS = query heads per wavefront: 2 (8 wavefronts, two per SIMD, 256 registers each) or
+// 1 (16 wavefronts, four per SIMD, 128 registers each; twice the LDS reads, and more
+// wavefronts to hide the chain logits -> softmax -> output of each).  One workgroup per CU
+// either way, and saying how many wavefronts share a SIMD lets the compiler use the registers.
+template <int G, bool CAP, int HEADS>
+__global__ __launch_bounds__(1024 / HEADS) __attribute__((amdgpu_waves_per_eu(4 / HEADS, 4 / HEADS))) void
+prefill_attn_kernel(PrefillArgs a) {
+  constexpr int kWaves = 4 / HEADS;      // wavefronts of a key group
+  constexpr int kBlocks = 8 / kWaves;    // 1 KB blocks of a K tile (and of a V^T tile) a wavefront brings in
   // Dynamic LDS: per key group two buffers, each a K tile [32 keys][256 B] followed by a
   // V^T tile [128 dims][64 B]; the merge of the groups at the end reuses the space.
   extern __shared__ __attribute__((aligned(16))) uint16_t pf_lds[];
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int lane = threadIdx.x & 63;
-  const int group = wave >> 1;  // which of the four tile streams this wavefront follows
-  const int hp = wave & 1;      // which pair of the quad's heads it serves
+  const int group = wave / kWaves;  // which of the four tile streams this wavefront follows
+  const int hp = wave % kWaves;     // which HEADS of the quad's heads it serves
   const int qc = lane & 15, g4 = lane >> 4;  // query column / key group of the matrix layouts
   // The KV head is the fastest-moving workgroup index: consecutive workgroups go to
   // consecutive XCDs, so with eight KV heads each XCD's L2 holds the keys and values of one
@@ -313,59 +353,70 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   char* const group_lds = (char*)pf_lds + group * (2 * kPfBufBytes);
   const uint32_t group_lds_at = (uint32_t)(uintptr_t)(pf_lds_ptr)pf_lds + (uint32_t)(group * (2 * kPfBufBytes));
 
-  // ---- staging role.  K tile: wavefront hp of the group fills the 1 KB blocks 4 hp + i
-  // (i < 4; a block is 4 keys), lane l the piece (key l/16 of the block, slot l%16), which
+  // ---- staging role.  K tile: wavefront hp of the group fills the 1 KB blocks kBlocks hp + i
+  // (i < kBlocks; a block is 4 keys), lane l the piece (key l/16 of the block, slot l%16), which
   // holds the dims [8 c, 8 c + 8) with c = slot ^ (key & 15).  V^T tile: blocks of 16 dims,
   // lane l the piece (dim l/4 of the block, slot l%4) = keys [8 c, +8) of the tile in vt's
   // order, c = slot ^ ((dim / 4) & 3).
-  uint32_t k_src[4], v_src[4];
+  uint32_t k_src[kBlocks], v_src[kBlocks];
   {
     const int key_in_block = lane >> 4, slot = lane & 15;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = 4 * (4 * hp + i) + key_in_block;
-      k_src[i] = (uint32_t)(key * kHeadDim + 8 * (slot ^ (key & 15))) * 2u;
+    for (int i = 0; i < kBlocks; ++i) {
+      const int key = 4 * (kBlocks * hp + i) + key_in_block;
+      k_src[i] = (uint32_t)(key * kHeadDim + 8 * (slot ^ (key & 15))) * 2u - (uint32_t)(i * 1024);
     }
     const int dim_in_block = lane >> 2, vslot = lane & 3;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int dim = 16 * (4 * hp + i) + dim_in_block;
-      v_src[i] = (uint32_t)(dim * a.s_pad + 8 * (vslot ^ ((dim >> 2) & 3))) * 2u;
+    for (int i = 0; i < kBlocks; ++i) {
+      const int dim = 16 * (kBlocks * hp + i) + dim_in_block;
+      v_src[i] = (uint32_t)(dim * a.s_pad + 8 * (vslot ^ ((dim >> 2) & 3))) * 2u - (uint32_t)(i * 1024);
     }
   }
   const char* const k_base = (const char*)(a.kr + (size_t)kvh * a.s_pad * kHeadDim);
   const char* const v_base = (const char*)(a.vt + (size_t)kvh * kHeadDim * a.s_pad);
-  auto request_tile = [&](int step, int buf) __attribute__((always_inline)) {
+  // Tile t of this group holds the keys [(t kPfGroups + group) kPfKeys, + kPfKeys); K tile t
+  // lives in K buffer t % 2, V^T tile t in V buffer t % 2.
+  auto request_k = [&](int t) __attribute__((always_inline)) {
     // past the end: a harmless repeat of the last tile
-    const int tile = min((step * kPfGroups + group) * kPfKeys, a.s_pad - kPfKeys);
-    const uint32_t dst = group_lds_at + (uint32_t)(buf * kPfBufBytes + (4 * hp) * 1024);
-    const char* const ks = k_base + (size_t)tile * (kHeadDim * 2);
-    const char* const vs = v_base + (size_t)tile * 2;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) load_to_lds16(ks + k_src[i], dst + (uint32_t)(i * 1024));
-#pragma unroll
-    for (int i = 0; i < 4; ++i) load_to_lds16(vs + v_src[i], dst + (uint32_t)(kPfTileBytes + i * 1024));
+    const int tile = min((t * kPfGroups + group) * kPfKeys, a.s_pad - kPfKeys);
+    const uint32_t dst = group_lds_at + (uint32_t)((t & 1) * kPfBufBytes + (kBlocks * hp) * 1024);
+    load_to_lds16<kBlocks>(k_base + (size_t)tile * (kHeadDim * 2), k_src, dst);
   };
-  request_tile(0, 0);  // on its way while the queries are prepared
+  auto request_v = [&](int t) __attribute__((always_inline)) {
+    const int tile = min((t * kPfGroups + group) * kPfKeys, a.s_pad - kPfKeys);
+    const uint32_t dst = group_lds_at + (uint32_t)((t & 1) * kPfBufBytes + kPfTileBytes + (kBlocks * hp) * 1024);
+    load_to_lds16<kBlocks>(v_base + (size_t)tile * 2, v_src, dst);
+  };
+  request_k(0);  // on its way while the queries are prepared
 
-  const int S = min(max(*a.sel_len, 0), a.max_sel_len);
   const int m = a.rows;
-  const int shift = S - m;  // query row i sits at position shift + i and sees keys <= that
-  const bool rope = a.rope_mode == TS_ROPE_LLAMA;
-  int head[2];
-  bool head_active[2];
+  int head[HEADS];
+  bool head_active[HEADS];
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
-    const int head_in_group = blockIdx.z * 4 + 2 * hp + rb;
+  for (int rb = 0; rb < HEADS; ++rb) {
+    const int head_in_group = blockIdx.z * 4 + HEADS * hp + rb;
     head_active[rb] = head_in_group < G;
     head[rb] = kvh * G + (head_active[rb] ? head_in_group : 0);
   }
+  // The queries' loads do not wait for the selection's length.
+  const int q_row = min(q_row0 + qc, m - 1);
+  uint4 q_raw[HEADS][4];
+#pragma unroll
+  for (int rb = 0; rb < HEADS; ++rb) {
+    const uint16_t* qrow = a.q + ((size_t)q_row * H + head[rb]) * kHeadDim;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) q_raw[rb][ks] = *(const uint4*)(qrow + 32 * ks + 8 * g4);
+  }
+  const int S = min(max(*a.sel_len, 0), a.max_sel_len);
+  const int shift = S - m;  // query row i sits at position shift + i and sees keys <= that
+  const bool rope = a.rope_mode == TS_ROPE_LLAMA;
   const bool wave_active = head_active[0];
   if (S < m || S <= 0) {
     // Fewer keys than rows (not a prefill chunk, or a selection that reported a
     // fault): the rows attend to nothing and the output is defined as zero.
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int rb = 0; rb < HEADS; ++rb)
       if (head_active[rb])
         for (int i = lane; i < 16 * (kHeadDim / 8); i += 64) {
           const int row = q_row0 + i / (kHeadDim / 8);
@@ -380,16 +431,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // ---- queries: B operand, lane (qc, g4) holds dims [32 ks + 8 g4, +8) of row q_row0 + qc
   // of each of its two heads, rotated to position shift + row (partner dims d and d + 64 are
   // k-steps ks and ks + 2; the angles are the same for both heads).
-  const int q_row = min(q_row0 + qc, m - 1);
-  pf_bf16x8 qb[2][4];
+  pf_bf16x8 qb[HEADS][4];
   {
-    float x[2][4][8];
+    float x[HEADS][4][8];
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
-      const uint16_t* qrow = a.q + ((size_t)q_row * H + head[rb]) * kHeadDim;
+    for (int rb = 0; rb < HEADS; ++rb) {
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
-        const uint4 w = *(const uint4*)(qrow + 32 * ks + 8 * g4);
+        const uint4 w = q_raw[rb][ks];
         const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -409,7 +458,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           float sn, cs;
           sincos_reduced(pos * freq, sn, cs);
 #pragma unroll
-          for (int rb = 0; rb < 2; ++rb) {
+          for (int rb = 0; rb < HEADS; ++rb) {
             const float lo = x[rb][ks][e], hi = x[rb][ks + 2][e];
             x[rb][ks][e] = lo * cs - hi * sn;
             x[rb][ks + 2][e] = hi * cs + lo * sn;
@@ -420,7 +469,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // products come out as base-2 logits and every key costs one exp2 and no multiply.
     const float qs = CAP ? 1.0f : a.sm_scale * kLog2e;
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int rb = 0; rb < HEADS; ++rb)
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
@@ -442,29 +491,46 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // ---- main loop over the tiles any row of this query tile can see
   const int last_visible = min(S - 1, shift + min(q_row0 + 15, m - 1));
   const int my_limit = shift + q_row;  // last key this lane's query sees
-  const int steps = last_visible / (kPfGroups * kPfKeys) + 1;
-  float m_run[2] = {kNegBig, kNegBig};  // kNegBig: no maximum yet
-  pf_f32x4 o[2][8], row_sum[2];
+  // tiles of this group that hold a visible key
+  const int n_tiles = last_visible >= group * kPfKeys
+                          ? (last_visible - group * kPfKeys) / (kPfGroups * kPfKeys) + 1
+                          : 0;
+  // Running maximum of each head's row: m_run (kNegBig: none yet), minus that as the
+  // four-register start value of the logits' accumulators (0 while there is none), and the
+  // excess over it that makes the row move (-inf while there is none: any finite logit does).
+  float m_run[HEADS], raise_at[HEADS];
+  pf_f32x4 minus_m[HEADS];
+  pf_f32x4 o[HEADS][8], row_sum[HEADS];
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
+  for (int rb = 0; rb < HEADS; ++rb) {
+    m_run[rb] = kNegBig;
+    raise_at[rb] = -INFINITY;
+    minus_m[rb] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
     row_sum[rb] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int db = 0; db < 8; ++db) o[rb][db] = pf_f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const pf_bf16x8 ones = __builtin_bit_cast(pf_bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
 
-  // One 32-key tile of this group: logits, online softmax, output update, for both heads.
-  auto compute_tile = [&](int tile, int buf) __attribute__((always_inline)) {
-    const char* const base = group_lds + buf * kPfBufBytes;
-    // Only the tiles on the diagonal hold keys that some query of the tile must not see.
-    const bool diagonal = tile + kPfKeys - 1 > shift + q_row0;
-    pf_f32x4 s[2][2];  // [head][key block]: key tile + 16 kb + 4 g4 + r, query qc
-    float m_base[2];
+  // The work on a tile comes in three parts, and the loop below is a software pipeline
+  // over them, because a wavefront issues in order and the matrix unit and the vector
+  // ALU only run side by side when their instructions alternate in one stream (two
+  // wavefronts of a SIMD, each doing first one kind and then the other, were measured to
+  // overlap in 15 % of the matrix cycles):
+  //   logits(t):  S^T = K_t Q^T for both heads (16 matrix instructions), shifted by the
+  //               running maximum through the accumulator's start value;
+  //   settle(t):  the causal mask on the diagonal, the largest logit of a row, and, when
+  //               a row outgrew its maximum by kPfRaise, the move to a new one (vector);
+  //   output(t):  P = exp2 (vector, 16 exp2), O^T += V_t^T P^T and the row sums (18 matrix).
+  // Iteration t runs logits(t + 1) with the exp2 of tile t in between, then output(t),
+  // then settle(t + 1).
+  pf_f32x4 s_cur[HEADS][2];  // logits of the tile whose output comes next: [head][key block]
+
+  auto logits = [&](int t, pf_f32x4 (&s)[HEADS][2]) __attribute__((always_inline)) {
+    const char* const base = group_lds + (t & 1) * kPfBufBytes;
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
-      m_base[rb] = m_run[rb] == kNegBig ? 0.f : m_run[rb];
-      const float c0 = CAP ? 0.f : -m_base[rb];
-      s[rb][0] = pf_f32x4{c0, c0, c0, c0};
+    for (int rb = 0; rb < HEADS; ++rb) {
+      s[rb][0] = CAP ? pf_f32x4{0.f, 0.f, 0.f, 0.f} : minus_m[rb];
       s[rb][1] = s[rb][0];
     }
 #pragma unroll
@@ -473,21 +539,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int ks = 0; ks < 4; ++ks) {
         const uint4 kw = *(const uint4*)(base + kb * (16 * kHeadDim * 2) + k_at[ks]);
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
+        for (int rb = 0; rb < HEADS; ++rb)
           s[rb][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, kw), qb[rb][ks],
                                                              s[rb][kb], 0, 0, 0);
       }
-    uint4 vw[8];
+  };
+
+  auto settle = [&](int t, pf_f32x4 (&s)[HEADS][2]) __attribute__((always_inline)) {
+    const int tile = (t * kPfGroups + group) * kPfKeys;
+    // Only the tiles on the diagonal hold keys that some query of the tile must not see.
+    const bool diagonal = tile + kPfKeys - 1 > shift + q_row0;
 #pragma unroll
-    for (int db = 0; db < 8; ++db) vw[db] = *(const uint4*)(base + db * (16 * kPfKeys * 2) + v_at);
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
+    for (int rb = 0; rb < HEADS; ++rb) {
       if (CAP) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            s[rb][kb][r] = a.logit_cap * tanhf(s[rb][kb][r] * a.sm_scale / a.logit_cap) * kLog2e - m_base[rb];
+            s[rb][kb][r] = a.logit_cap * tanhf(s[rb][kb][r] * a.sm_scale / a.logit_cap) * kLog2e + minus_m[rb][0];
       }
       if (diagonal) {
         // Masked logits are -inf: exp2 makes them 0 without a branch.
@@ -501,17 +570,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       mx = max3(mx, s[rb][0][3], s[rb][1][0]);
       mx = max3(mx, s[rb][1][1], s[rb][1][2]);
       mx = fmaxf(mx, s[rb][1][3]);
-      const bool unset = m_run[rb] == kNegBig;
-      if (__ballot(unset || mx > kPfRaise) != 0ull) {
+      if (__ballot(mx > raise_at[rb]) != 0ull) {
         // Some row of this head has no maximum yet, or outgrew it: agree on the row's
         // maximum over the four key groups of lanes and move to it.
+        const bool unset = m_run[rb] == kNegBig;
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const bool take = unset ? mx > -INFINITY : mx > kPfRaise;
         const float delta = take ? mx : 0.f;
         // (a row without a maximum has only zeros in its accumulators)
         const float scale = unset ? 1.0f : __builtin_amdgcn_exp2f(-delta);
-        if (take) m_run[rb] = m_base[rb] + delta;
+        if (take) {
+          m_run[rb] = delta - minus_m[rb][0];
+          raise_at[rb] = kPfRaise;
+          const float nm = -m_run[rb];
+          minus_m[rb] = pf_f32x4{nm, nm, nm, nm};
+        }
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -523,63 +597,109 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int r = 0; r < 4; ++r) row_sum[rb][r] *= scale;
       }
+    }
+  };
+
+  // One iteration of the pipeline: NEXT = there is a tile t + 1.
+  auto iteration = [&](int t, auto next) __attribute__((always_inline)) {
+    constexpr bool NEXT = decltype(next)::value;
+    const char* const vbase = group_lds + (t & 1) * kPfBufBytes;
+    pf_f32x4 s_next[HEADS][2];
+    if (NEXT) logits(t + 1, s_next);
+    pf_bf16x8 pb[HEADS];
+#pragma unroll
+    for (int rb = 0; rb < HEADS; ++rb) {
       float p[2][4];
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) p[kb][r] = __builtin_amdgcn_exp2f(s[rb][kb][r]);
+        for (int r = 0; r < 4; ++r) p[kb][r] = __builtin_amdgcn_exp2f(s_cur[rb][kb][r]);
       const uint4 pw = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]),
                                   pack_bf16(p[1][0], p[1][1]), pack_bf16(p[1][2], p[1][3]));
-      const pf_bf16x8 pb = __builtin_bit_cast(pf_bf16x8, pw);
+      pb[rb] = __builtin_bit_cast(pf_bf16x8, pw);
+    }
 #pragma unroll
-      for (int db = 0; db < 8; ++db)
-        o[rb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw[db]), pb,
+    for (int db = 0; db < 8; ++db) {
+      const uint4 vw = *(const uint4*)(vbase + db * (16 * kPfKeys * 2) + v_at);
+#pragma unroll
+      for (int rb = 0; rb < HEADS; ++rb)
+        o[rb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw), pb[rb],
                                                            o[rb][db], 0, 0, 0);
-      row_sum[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb, row_sum[rb], 0, 0, 0);
+    }
+#pragma unroll
+    for (int rb = 0; rb < HEADS; ++rb)
+      row_sum[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[rb], row_sum[rb], 0, 0, 0);
+    if (NEXT) {
+      settle(t + 1, s_next);
+#pragma unroll
+      for (int rb = 0; rb < HEADS; ++rb) {
+        s_cur[rb][0] = s_next[rb][0];
+        s_cur[rb][1] = s_next[rb][1];
+      }
     }
   };
 
-  // The tile requested during step i - 1 is computed on in step i.  The two wavefronts of
-  // a key group keep in step through two counters in LDS and no barrier, so that the four
-  // groups drift apart and the two wavefronts of a SIMD (which belong to different
-  // groups) are rarely in the same phase: one's matrix instructions run under the other's
-  // softmax.  landed = pieces of tiles that have arrived (each wavefront counts its own
-  // after waiting for them), read = tiles a wavefront has finished reading.  Tile i may be
-  // read when landed >= 2 (i + 1); the buffer of tile i - 1 may be overwritten (by the
-  // request for tile i + 1) when read >= 2 i.  Neither wait can last: a partner is at most
-  // one step behind.  The waits are bounded all the same, so that a mistake here would
-  // show as a wrong result and not as a hang.
-  __shared__ uint32_t pf_sync[kPfGroups][2];
+  // The wavefronts of a key group keep in step through two counters in LDS and no
+  // barrier, so that the four groups drift apart.  landed = requests that have arrived
+  // (after each round of requests a wavefront waits for its own pieces and counts once),
+  // done = rounds of reading a wavefront has finished.  Round -1 brings K tile 0 and reads
+  // nothing; round t >= 0 is iteration t: it needs K tile t + 1 and V tile t, requested in
+  // round t - 1, and requests K tile t + 2 and V tile t + 1 into the buffers that round
+  // t - 1 read (K tile t, V tile t - 1): so it starts when landed >= kWaves (t + 2) and
+  // done >= kWaves (t + 1).  Neither wait can last: a partner is at most one round behind.
+  // The waits are bounded all the same, so that a mistake here would show as a wrong
+  // result and not as a hang.
+  __shared__ __attribute__((aligned(8))) uint32_t pf_sync[kPfGroups][2];
   if (threadIdx.x < 2 * kPfGroups) (&pf_sync[0][0])[threadIdx.x] = 0u;
   __syncthreads();
-  uint32_t* const landed = &pf_sync[group][0];
-  uint32_t* const was_read = &pf_sync[group][1];
-  for (int step = 0; step < steps; ++step) {
-    const int buf = step & 1;
+  const uint64_t* const both = (const uint64_t*)&pf_sync[group][0];  // one read for the two
+  const uint32_t landed_at = (uint32_t)(uintptr_t)(pf_lds_ptr)&pf_sync[group][0], done_at = landed_at + 4u;
+  const uint32_t one = 1u;
+  auto await = [&](uint32_t need_landed, uint32_t need_done) __attribute__((always_inline)) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (lane == 0) __hip_atomic_fetch_add(landed, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    lds_count(landed_at, one);
     for (int spin = 0; spin < (1 << 20); ++spin) {
-      const uint32_t have = __hip_atomic_load(landed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
-      const uint32_t freed = __hip_atomic_load(was_read, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
-      if (have >= 2u * (uint32_t)(step + 1) && freed >= 2u * (uint32_t)step) break;
+      const uint64_t counters = __hip_atomic_load(both, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if ((uint32_t)counters >= need_landed && (uint32_t)(counters >> 32) >= need_done) break;
       __builtin_amdgcn_s_sleep(1);
     }
-    if (step + 1 < steps) request_tile(step + 1, buf ^ 1);
-    const int tile = (step * kPfGroups + group) * kPfKeys;
-    if (wave_active && tile <= last_visible) compute_tile(tile, buf);
-    if (lane == 0) __hip_atomic_fetch_add(was_read, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+  };
+  auto finish_round = [&]() __attribute__((always_inline)) {
+    lds_count(done_at, one);
+  };
+  if (n_tiles > 0) {
+    await((uint32_t)kWaves, 0u);
+    if (1 < n_tiles) request_k(1);
+    request_v(0);
+    if (wave_active) {
+      logits(0, s_cur);
+      settle(0, s_cur);
+    }
+    finish_round();
+    for (int t = 0; t + 1 < n_tiles; ++t) {
+      await((uint32_t)(kWaves * (t + 2)), (uint32_t)(kWaves * (t + 1)));
+      if (t + 2 < n_tiles) request_k(t + 2);
+      request_v(t + 1);
+      if (wave_active) iteration(t, std::true_type{});
+      finish_round();
+    }
+    // the last tile: nothing follows it
+    await((uint32_t)(kWaves * (n_tiles + 1)), (uint32_t)(kWaves * n_tiles));
+    if (wave_active) iteration(n_tiles - 1, std::false_type{});
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
   // ---- merge of the four key groups (the barrier that ended the last step also freed
-  // the tiles' space): groups 1..3 hand their partial results to group 0 (same head pair,
-  // same lane), 18 vectors of four floats per lane: per head 8 of acc and (max, sum).
-  pf_f32x4* const merge = (pf_f32x4*)pf_lds;  // [(group - 1) * 2 + hp][18][64 lanes]
-  static_assert(6 * 18 * 64 * 16 <= kPfLdsBytes, "the merge area fits the tiles");
+  // the tiles' space): groups 1..3 hand their partial results to group 0 (same heads,
+  // same lane), per head 9 vectors of four floats per lane: 8 of acc and (max, sum).
+  constexpr int kVecs = 9 * HEADS;
+  pf_f32x4* const merge = (pf_f32x4*)pf_lds;  // [(group - 1) * kWaves + hp][kVecs][64 lanes]
+  static_assert(3 * kWaves * kVecs * 64 * 16 <= kPfLdsBytes, "the merge area fits the tiles");
   if (group != 0) {
-    pf_f32x4* const mine = merge + ((group - 1) * 2 + hp) * (18 * 64) + lane;
+    pf_f32x4* const mine = merge + ((group - 1) * kWaves + hp) * (kVecs * 64) + lane;
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
+    for (int rb = 0; rb < HEADS; ++rb) {
 #pragma unroll
       for (int db = 0; db < 8; ++db) mine[(9 * rb + db) * 64] = o[rb][db];
       mine[(9 * rb + 8) * 64] = pf_f32x4{m_run[rb], row_sum[rb][0], 0.f, 0.f};
@@ -587,12 +707,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   __syncthreads();
   if (group != 0 || !wave_active) return;
-  float l_run[2] = {row_sum[0][0], row_sum[1][0]};
+  float l_run[HEADS];
+#pragma unroll
+  for (int rb = 0; rb < HEADS; ++rb) l_run[rb] = row_sum[rb][0];
 #pragma unroll
   for (int g = 1; g < kPfGroups; ++g) {
-    const pf_f32x4* const other = merge + ((g - 1) * 2 + hp) * (18 * 64) + lane;
+    const pf_f32x4* const other = merge + ((g - 1) * kWaves + hp) * (kVecs * 64) + lane;
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
+    for (int rb = 0; rb < HEADS; ++rb) {
       const pf_f32x4 ml = other[(9 * rb + 8) * 64];
       const float m_new = fmaxf(m_run[rb], ml[0]);
       const float e0 = __builtin_amdgcn_exp2f(m_run[rb] - m_new), e1 = __builtin_amdgcn_exp2f(ml[0] - m_new);
@@ -610,7 +732,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // o[rb][db][r] = O[query qc][dim 16 db + 4 g4 + r] of head rb; the row sum is complete in every lane.
   if (q_row0 + qc >= m) return;
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
+  for (int rb = 0; rb < HEADS; ++rb) {
     if (!head_active[rb]) continue;
     const float inv = l_run[rb] > 0.f ? 1.0f / l_run[rb] : 0.f;
     uint16_t* orow = a.out + ((size_t)(q_row0 + qc) * H + head[rb]) * kHeadDim;
@@ -701,10 +823,10 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
 #define TS_PF_LAUNCH(G_, C_)                                                                  \
   {                                                                                           \
     static const hipError_t lds_ok = hipFuncSetAttribute(                                     \
-        (const void*)prefill_attn_kernel<G_, C_>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+        (const void*)prefill_attn_kernel<G_, C_, kPfHeads>, hipFuncAttributeMaxDynamicSharedMemorySize, \
         (int)kPfLdsBytes);                                                                    \
     if (lds_ok != hipSuccess) return fail(TS_EHIP, "prefill attention: %zu bytes of LDS refused", kPfLdsBytes); \
-    hipLaunchKernelGGL((prefill_attn_kernel<G_, C_>), grid, dim3(512), kPfLdsBytes, st, a);   \
+    hipLaunchKernelGGL((prefill_attn_kernel<G_, C_, kPfHeads>), grid, dim3(1024 / kPfHeads), kPfLdsBytes, st, a); \
   }
 #define TS_PF_CASE(G_)               \
   case G_:                           \

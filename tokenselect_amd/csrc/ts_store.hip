@@ -49,33 +49,32 @@ __global__ __launch_bounds__(256) void kv_store_chunk_kernel(
     uint4* __restrict__ k_pool, uint4* __restrict__ v_pool, int64_t pool_rows,
     int32_t* __restrict__ table, int32_t* seq_len, int row_vec, int max_tokens) {
   const int r = blockIdx.x;
-  int len;
+  // Counted: the upper bits may already hold other workgroups' counts.
+  const int len = COUNTED ? (__hip_atomic_load(seq_len, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kLenMask)
+                          : *seq_len;
+  const int at = len + r;
+  if (at >= 0 && at < max_tokens) {
+    int64_t slot = loc[r];
+    slot = slot < 0 ? 0 : (slot >= pool_rows ? pool_rows - 1 : slot);
+    for (int i = threadIdx.x; i < row_vec; i += blockDim.x) {
+      k_pool[(size_t)slot * row_vec + i] = k[(size_t)r * row_vec + i];
+      v_pool[(size_t)slot * row_vec + i] = v[(size_t)r * row_vec + i];
+    }
+    if (threadIdx.x == 0) table[at] = (int32_t)slot;
+  }
   if (COUNTED) {
-    // One thread reads the word and then counts the workgroup in; the others take the
-    // length from LDS, so that nobody looks at the word after the last count.
-    __shared__ int s_len;
+    // A workgroup counts itself in when all its wavefronts have read the length, at its
+    // end, where nobody waits for the answer; whoever completes the count knows that
+    // every workgroup has read the old length, and writes the new one.
+    __syncthreads();
     if (threadIdx.x == 0) {
-      s_len = __hip_atomic_load(seq_len, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kLenMask;
       const int before = __hip_atomic_fetch_add(seq_len, 1 << kLenBits, __ATOMIC_RELAXED,
                                                 __HIP_MEMORY_SCOPE_AGENT);
-      if ((before >> kLenBits) + 1 == (int)gridDim.x)  // every workgroup has read the length
-        __hip_atomic_store(seq_len, min(s_len + (int)gridDim.x, max_tokens), __ATOMIC_RELAXED,
+      if ((before >> kLenBits) + 1 == (int)gridDim.x)
+        __hip_atomic_store(seq_len, min(len + (int)gridDim.x, max_tokens), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     }
-    __syncthreads();
-    len = s_len;
-  } else {
-    len = *seq_len;
   }
-  const int at = len + r;
-  if (at < 0 || at >= max_tokens) return;
-  int64_t slot = loc[r];
-  slot = slot < 0 ? 0 : (slot >= pool_rows ? pool_rows - 1 : slot);
-  for (int i = threadIdx.x; i < row_vec; i += blockDim.x) {
-    k_pool[(size_t)slot * row_vec + i] = k[(size_t)r * row_vec + i];
-    v_pool[(size_t)slot * row_vec + i] = v[(size_t)r * row_vec + i];
-  }
-  if (threadIdx.x == 0) table[at] = (int32_t)slot;
 }
 
 __global__ void seq_len_add_kernel(int32_t* seq_len, int rows, int max_tokens) {
