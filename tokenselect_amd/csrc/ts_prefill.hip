@@ -137,8 +137,9 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
 // Staging: a group's 128 threads bring the next tile of their group (8 KB of kr, 8 KB
 // of vt) from global memory straight into LDS (global_load_lds_dwordx4: 16 bytes per
 // lane, a wavefront fills 1 KB of consecutive LDS; no registers, no LDS store
-// instructions) while the group computes on the tile that arrived during the previous
-// step; one barrier per step, two LDS buffers per group.  Rows are not padded in LDS;
+// instructions) while the group computes on the tiles that arrived during the previous
+// step; two LDS buffers per group, and two counters in LDS per group instead of a
+// workgroup barrier per step (see the loop).  Rows are not padded in LDS;
 // instead the 16-byte pieces of a row are permuted (XOR with row bits) so that the 16
 // lanes the hardware serves together when a wavefront reads a matrix operand fall on
 // distinct banks: which global piece a lane fetches is free, where it lands is not.
@@ -154,6 +155,15 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
 // directly the B operand of O^T += V^T P^T (A = 16 dims x 32 keys from the V^T tile);
 // a ninth product with an all-ones A operand accumulates the row sums.  fp32
 // accumulation throughout.
+//
+// Where the time goes (512 rows over 2688 selected keys, 36.5 us): 4.6 us until the
+// queries are rotated and the first tile is there, 2 us for the merge and the output, the
+// rest in some 19 rounds of 2100 cycles per wavefront, of which the matrix unit of a SIMD
+// is busy 1090 (its two wavefronts' 68 instructions of 16 cycles).  A round is some 250
+// instructions, a wavefront issues one per four cycles at best, and every wait (for LDS
+// data, for a matrix result, for the partner's counter) stalls the wavefront's whole
+// stream: two wavefronts per SIMD cover each other only partly.  Four wavefronts per SIMD
+// with one head each (HEADS = 1) double the LDS reads and come out the same.
 struct PrefillArgs {
   const uint16_t* q;  // [rows, H, 128] bf16, un-rotated
   const uint16_t* k_pool;
@@ -559,12 +569,16 @@ prefill_attn_kernel(PrefillArgs a) {
             s[rb][kb][r] = a.logit_cap * tanhf(s[rb][kb][r] * a.sm_scale / a.logit_cap) * kLog2e + minus_m[rb][0];
       }
       if (diagonal) {
-        // Masked logits are -inf: exp2 makes them 0 without a branch.
+        // Masked logits are -inf: exp2 makes them 0 without a branch.  (The tile's
+        // number passes through an empty asm so that the comparisons stay in here: the
+        // compiler otherwise computes all of them before the branch, on every tile.)
+        int tile_here = tile;
+        asm volatile("" : "+s"(tile_here));
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            if (tile + 16 * kb + 4 * g4 + r > my_limit) s[rb][kb][r] = -INFINITY;
+            if (tile_here + 16 * kb + 4 * g4 + r > my_limit) s[rb][kb][r] = -INFINITY;
       }
       float mx = max3(s[rb][0][0], s[rb][0][1], s[rb][0][2]);
       mx = max3(mx, s[rb][0][3], s[rb][1][0]);
