@@ -87,6 +87,77 @@ def test_sparse_prefill_attention_full_chunk_and_soft_cap(dev):
         assert err <= 2e-2, (cap, err)
 
 
+@pytest.mark.parametrize("m,S", [(1, 1), (20, 20), (100, 100), (5, 31), (16, 33), (40, 129), (130, 131)])
+def test_sparse_prefill_attention_short_selections(dev, m, S):
+    """The first chunk of a request (S = m: every row sees only the chunk up to itself,
+    the first rows a single key) and selections shorter than one round of the kernel's
+    four tile streams, where some streams have no tile at all."""
+    say(f"prefill attention short selection m={m} S={S}")
+    wl = workloads.build("pf", SHAPES[0], [S + 8], [8], 1, dev, seed=21, n_init=1, n_local=m)
+    c = wl.cfg
+    g = torch.Generator(device=dev).manual_seed(22)
+    q = torch.randn((m, c.num_heads * 128), generator=g, device=dev).bfloat16()
+    sel = wl.table[0, :S].contiguous()
+    sel_len = torch.tensor([S], dtype=torch.int32, device=dev)
+    out = ops.sparse_prefill_attention(c, q, wl.k_pool, wl.v_pool, sel, sel_len)
+    torch.cuda.synchronize()
+    ref = oracle.prefill.sparse_prefill_attention(q.cpu().view(m, c.num_heads, 128), wl.k_pool.cpu(),
+                                                  wl.v_pool.cpu(), sel.cpu(), _sm(c), c.rope_theta)
+    err = (out.cpu().float() - ref.reshape(m, -1).float()).abs().max().item()
+    assert err <= 2e-2, err
+
+
+@pytest.mark.parametrize("direction", ["growing", "shrinking"])
+def test_sparse_prefill_attention_moving_maximum(dev, direction):
+    """Logits that grow (or fall) steadily along the selected list, by far more than the
+    excess at which the kernel raises a row's running maximum: with growing logits every
+    round of tiles raises it, with falling ones the first tile's maximum stays and the
+    weights of the later keys become tiny."""
+    m, S = 48, 700
+    say(f"prefill attention with {direction} logits m={m} S={S}")
+    wl = workloads.build("pf", SHAPES[0], [S], [8], 1, dev, seed=23, n_init=1, n_local=m)
+    c = wl.cfg
+    c.rope_mode = "NONE"
+    g = torch.Generator(device=dev).manual_seed(24)
+    # keys along one direction with a length that moves with the position; values random
+    u = torch.ones(128, device=dev)
+    ramp = torch.arange(S, device=dev, dtype=torch.float32) * 0.006
+    if direction == "shrinking":
+        ramp = ramp.flip(0)
+    slots = wl.table[0, :S].long()
+    k_pool = wl.k_pool.clone()
+    k_pool[slots] = (ramp[:, None, None] * u[None, None, :]
+                     + 0.05 * torch.randn((S, c.num_kv_heads, 128), generator=g, device=dev)).bfloat16()
+    q = (0.5 * u[None, :].repeat(m, c.num_heads)
+         + 0.05 * torch.randn((m, c.num_heads * 128), generator=g, device=dev)).bfloat16()
+    sel = wl.table[0, :S].contiguous()
+    sel_len = torch.tensor([S], dtype=torch.int32, device=dev)
+    out = ops.sparse_prefill_attention(c, q, k_pool, wl.v_pool, sel, sel_len)
+    torch.cuda.synchronize()
+    ref = oracle.prefill.sparse_prefill_attention(q.cpu().view(m, c.num_heads, 128), k_pool.cpu(),
+                                                  wl.v_pool.cpu(), sel.cpu(), _sm(c), c.rope_theta,
+                                                  rope_mode="NONE")
+    # base-2 logits span 0.5 * 0.006 * 128 / sqrt(128) * log2(e) * 700 = 34 over the list
+    err = (out.cpu().float() - ref.reshape(m, -1).float()).abs().max().item()
+    assert err <= 2e-2, err
+
+
+def test_sparse_prefill_attention_fewer_keys_than_rows(dev):
+    """A selection that reports fewer keys than the chunk has rows (a selection that gave
+    up reports -1) leaves a defined output: zeros."""
+    m = 40
+    say("prefill attention with fewer keys than rows")
+    wl = workloads.build("pf", SHAPES[1], [100], [8], 1, dev, seed=25, n_init=1, n_local=m)
+    c = wl.cfg
+    q = torch.ones((m, c.num_heads * 128), dtype=torch.bfloat16, device=dev)
+    sel = wl.table[0, :100].contiguous()
+    for reported in (-1, 0, m - 1):
+        sel_len = torch.tensor([reported], dtype=torch.int32, device=dev)
+        out = ops.sparse_prefill_attention(c, q, wl.k_pool, wl.v_pool, sel, sel_len)
+        torch.cuda.synchronize()
+        assert torch.count_nonzero(out).item() == 0, reported
+
+
 def test_kv_store_chunk(dev):
     say("kv_store_chunk")
     wl = workloads.build("pf", SHAPES[0], [100], [16], 1, dev, seed=7, n_init=4, n_local=16,

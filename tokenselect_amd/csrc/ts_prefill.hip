@@ -163,7 +163,7 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
 // instructions, a wavefront issues one per four cycles at best, and every wait (for LDS
 // data, for a matrix result, for the partner's counter) stalls the wavefront's whole
 // stream: two wavefronts per SIMD cover each other only partly.  Four wavefronts per SIMD
-// with one head each (HEADS = 1) double the LDS reads and come out the same.
+// with one head each double the LDS reads and came out the same.
 struct PrefillArgs {
   const uint16_t* q;  // [rows, H, 128] bf16, un-rotated
   const uint16_t* k_pool;
@@ -287,36 +287,23 @@ typedef void __attribute__((address_space(3)))* pf_lds_ptr;
 // makes every later LDS read wait for all such loads (it cannot tell that they fill the
 // other buffer), which serialises exactly what is meant to overlap.  The waits are
 // explicit instead: s_waitcnt vmcnt(0) before the barrier that hands a buffer over.
-// The source is base (the same for the whole wavefront) + offset (per lane).  N pieces per
+// The source is base (the same for the whole wavefront) + offset (per lane).  Four pieces per
 // lane with one write of M0: the instruction's offset field moves both addresses, so piece
 // i lands 1 KB after piece i - 1, and its source offset is passed 1024 i too small.
 // A wavefront issues one instruction per four cycles at best, whatever its kind, and
 // the loop around these loads is bound by exactly that: every scalar instruction counts.
-template <int N>
-__device__ __forceinline__ void load_to_lds16(const void* base, const uint32_t (&offset)[N], uint32_t lds_dst) {
-  static_assert(N == 2 || N == 4, "two or four pieces");
+__device__ __forceinline__ void load_to_lds16(const void* base, const uint32_t (&offset)[4], uint32_t lds_dst) {
   uint32_t saved_m0;  // M0 is the compiler's; it gets it back
-  if (N == 4)
-    asm volatile(
-        "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
-        "global_load_lds_dwordx4 %2, %6\n\t"
-        "global_load_lds_dwordx4 %3, %6 offset:1024\n\t"
-        "global_load_lds_dwordx4 %4, %6 offset:2048\n\t"
-        "global_load_lds_dwordx4 %5, %6 offset:3072\n\t"
-        "s_mov_b32 m0, %0"
-        : "=&s"(saved_m0)
-        : "s"(lds_dst), "v"(offset[0]), "v"(offset[1]), "v"(offset[N == 4 ? 2 : 0]), "v"(offset[N == 4 ? 3 : 1]),
-          "s"(base)
-        : "memory");
-  else
-    asm volatile(
-        "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
-        "global_load_lds_dwordx4 %2, %4\n\t"
-        "global_load_lds_dwordx4 %3, %4 offset:1024\n\t"
-        "s_mov_b32 m0, %0"
-        : "=&s"(saved_m0)
-        : "s"(lds_dst), "v"(offset[0]), "v"(offset[1]), "s"(base)
-        : "memory");
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %2, %6\n\t"
+      "global_load_lds_dwordx4 %3, %6 offset:1024\n\t"
+      "global_load_lds_dwordx4 %4, %6 offset:2048\n\t"
+      "global_load_lds_dwordx4 %5, %6 offset:3072\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0)
+      : "s"(lds_dst), "v"(offset[0]), "v"(offset[1]), "v"(offset[2]), "v"(offset[3]), "s"(base)
+      : "memory");
 }
 
 // One lane adds 1 to a counter in LDS.  LDS instructions of a wavefront are carried out in
@@ -336,15 +323,15 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return d;
 }
 
-// HEADS = query heads per wavefront: 2 (8 wavefronts, two per SIMD, 256 registers each) or
-// 1 (16 wavefronts, four per SIMD, 128 registers each; twice the LDS reads, and more
-// wavefronts to hide the chain logits -> softmax -> output of each).  One workgroup per CU
-// either way, and saying how many wavefronts share a SIMD lets the compiler use the registers.
-template <int G, bool CAP, int HEADS>
-__global__ __launch_bounds__(1024 / HEADS) __attribute__((amdgpu_waves_per_eu(4 / HEADS, 4 / HEADS))) void
-prefill_attn_kernel(PrefillArgs a) {
+// Two wavefronts per SIMD by construction (8 per workgroup, one workgroup per CU): saying
+// so lets the compiler use 256 registers.
+template <int G, bool CAP>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(
+    PrefillArgs a) {
+  constexpr int HEADS = kPfHeads;        // query heads per wavefront
   constexpr int kWaves = 4 / HEADS;      // wavefronts of a key group
   constexpr int kBlocks = 8 / kWaves;    // 1 KB blocks of a K tile (and of a V^T tile) a wavefront brings in
+  static_assert(HEADS == 2 && kBlocks == 4, "the staging loads come four per wavefront");
   // Dynamic LDS: per key group two buffers, each a K tile [32 keys][256 B] followed by a
   // V^T tile [128 dims][64 B]; the merge of the groups at the end reuses the space.
   extern __shared__ __attribute__((aligned(16))) uint16_t pf_lds[];
@@ -391,12 +378,12 @@ prefill_attn_kernel(PrefillArgs a) {
     // past the end: a harmless repeat of the last tile
     const int tile = min((t * kPfGroups + group) * kPfKeys, a.s_pad - kPfKeys);
     const uint32_t dst = group_lds_at + (uint32_t)((t & 1) * kPfBufBytes + (kBlocks * hp) * 1024);
-    load_to_lds16<kBlocks>(k_base + (size_t)tile * (kHeadDim * 2), k_src, dst);
+    load_to_lds16(k_base + (size_t)tile * (kHeadDim * 2), k_src, dst);
   };
   auto request_v = [&](int t) __attribute__((always_inline)) {
     const int tile = min((t * kPfGroups + group) * kPfKeys, a.s_pad - kPfKeys);
     const uint32_t dst = group_lds_at + (uint32_t)((t & 1) * kPfBufBytes + kPfTileBytes + (kBlocks * hp) * 1024);
-    load_to_lds16<kBlocks>(v_base + (size_t)tile * 2, v_src, dst);
+    load_to_lds16(v_base + (size_t)tile * 2, v_src, dst);
   };
   request_k(0);  // on its way while the queries are prepared
 
@@ -837,10 +824,10 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
 #define TS_PF_LAUNCH(G_, C_)                                                                  \
   {                                                                                           \
     static const hipError_t lds_ok = hipFuncSetAttribute(                                     \
-        (const void*)prefill_attn_kernel<G_, C_, kPfHeads>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+        (const void*)prefill_attn_kernel<G_, C_>, hipFuncAttributeMaxDynamicSharedMemorySize, \
         (int)kPfLdsBytes);                                                                    \
     if (lds_ok != hipSuccess) return fail(TS_EHIP, "prefill attention: %zu bytes of LDS refused", kPfLdsBytes); \
-    hipLaunchKernelGGL((prefill_attn_kernel<G_, C_, kPfHeads>), grid, dim3(1024 / kPfHeads), kPfLdsBytes, st, a); \
+    hipLaunchKernelGGL((prefill_attn_kernel<G_, C_>), grid, dim3(512), kPfLdsBytes, st, a); \
   }
 #define TS_PF_CASE(G_)               \
   case G_:                           \
