@@ -342,7 +342,7 @@ int ts_qkv_store(const ts_config* cfg, const void* x, const void* w, const void*
 /* store_kv_cache(start, end) + add_k_cache for a chunk (tr.py:725-733,
  * 332-336).  pages == NULL, page size 1: k_pool[loc[r]] = k[r], v likewise,
  * table[*seq_len + r] = loc[r] for r < rows, then *seq_len += rows (one
- * launch for rows <= 1023 and max_tokens < 2^21: the upper bits of *seq_len
+ * launch for rows <= 8184 and max_tokens < 2^21: the upper bits of *seq_len
  * count the workgroups while the kernel runs, and are zero again when it ends).
  * pages != NULL: row r goes to position *seq_len + r of the paged table, the
  * request's last page first and then fresh pages from the top of the pool, in

@@ -32,8 +32,8 @@ __global__ __launch_bounds__(256) void kv_store_kernel(const uint4* __restrict__
   }
 }
 
-// Chunked prefill (tr.py:725-733): workgroup r copies row r of the chunk to pool
-// slot loc[r] and writes table[len + r].  Every workgroup must read the same old
+// Chunked prefill (tr.py:725-733): a workgroup copies kChunkRowsPerWg rows of the chunk
+// (row r to pool slot loc[r]) and writes table[len + r] for them.  Every workgroup must read the same old
 // length, and the new one must be there when the launch ends: the workgroups count
 // themselves in the upper bits of the length word itself (a length stays below 2^21,
 // the count below 2^10), everybody masks those bits off, and the workgroup that
@@ -41,26 +41,29 @@ __global__ __launch_bounds__(256) void kv_store_kernel(const uint4* __restrict__
 // Rows that would not fit the table are dropped; slots are clamped to the pool.
 constexpr int kLenBits = 21;
 constexpr int kLenMask = (1 << kLenBits) - 1;
-constexpr int kChunkCountedRows = 1023;  // more rows take the two-launch form below
+constexpr int kChunkRowsPerWg = 8;        // 32 threads per row: few workgroups, few counts on one word
+constexpr int kChunkCountedWgs = 1023;    // more workgroups take the two-launch form below
 
 template <bool COUNTED>
 __global__ __launch_bounds__(256) void kv_store_chunk_kernel(
     const uint4* __restrict__ k, const uint4* __restrict__ v, const int32_t* __restrict__ loc,
     uint4* __restrict__ k_pool, uint4* __restrict__ v_pool, int64_t pool_rows,
-    int32_t* __restrict__ table, int32_t* seq_len, int row_vec, int max_tokens) {
-  const int r = blockIdx.x;
+    int32_t* __restrict__ table, int32_t* seq_len, int rows, int row_vec, int max_tokens) {
   // Counted: the upper bits may already hold other workgroups' counts.
   const int len = COUNTED ? (__hip_atomic_load(seq_len, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kLenMask)
                           : *seq_len;
+  constexpr int kThreadsPerRow = 256 / kChunkRowsPerWg;
+  const int r = blockIdx.x * kChunkRowsPerWg + threadIdx.x / kThreadsPerRow;
+  const int t = threadIdx.x % kThreadsPerRow;
   const int at = len + r;
-  if (at >= 0 && at < max_tokens) {
+  if (r < rows && at >= 0 && at < max_tokens) {
     int64_t slot = loc[r];
     slot = slot < 0 ? 0 : (slot >= pool_rows ? pool_rows - 1 : slot);
-    for (int i = threadIdx.x; i < row_vec; i += blockDim.x) {
+    for (int i = t; i < row_vec; i += kThreadsPerRow) {
       k_pool[(size_t)slot * row_vec + i] = k[(size_t)r * row_vec + i];
       v_pool[(size_t)slot * row_vec + i] = v[(size_t)r * row_vec + i];
     }
-    if (threadIdx.x == 0) table[at] = (int32_t)slot;
+    if (t == 0) table[at] = (int32_t)slot;
   }
   if (COUNTED) {
     // A workgroup counts itself in when all its wavefronts have read the length, at its
@@ -71,7 +74,7 @@ __global__ __launch_bounds__(256) void kv_store_chunk_kernel(
       const int before = __hip_atomic_fetch_add(seq_len, 1 << kLenBits, __ATOMIC_RELAXED,
                                                 __HIP_MEMORY_SCOPE_AGENT);
       if ((before >> kLenBits) + 1 == (int)gridDim.x)
-        __hip_atomic_store(seq_len, min(len + (int)gridDim.x, max_tokens), __ATOMIC_RELAXED,
+        __hip_atomic_store(seq_len, min(len + rows, max_tokens), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     }
   }
@@ -237,15 +240,16 @@ extern "C" int ts_kv_store_chunk(const ts_config* cfg, const void* k, const void
                        page_shift_of(cfg->page_size), page_pool_of(pages));
     return check_launch("kv_store_chunk_paged_kernel");
   }
-  if (rows <= kChunkCountedRows && max_tokens <= kLenMask) {
-    hipLaunchKernelGGL(kv_store_chunk_kernel<true>, dim3((unsigned)rows), dim3(256), 0,
-                       (hipStream_t)stream, (const uint4*)k, (const uint4*)v, out_cache_loc,
-                       (uint4*)k_pool, (uint4*)v_pool, pool_rows, table, seq_len, row_vec, max_tokens);
+  const unsigned wgs = (unsigned)ceil_div(rows, kChunkRowsPerWg);
+  if (wgs <= (unsigned)kChunkCountedWgs && max_tokens <= kLenMask) {
+    hipLaunchKernelGGL(kv_store_chunk_kernel<true>, dim3(wgs), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4*)k, (const uint4*)v, out_cache_loc, (uint4*)k_pool, (uint4*)v_pool,
+                       pool_rows, table, seq_len, rows, row_vec, max_tokens);
     return check_launch("kv_store_chunk_kernel");
   }
-  hipLaunchKernelGGL(kv_store_chunk_kernel<false>, dim3((unsigned)rows), dim3(256), 0,
-                     (hipStream_t)stream, (const uint4*)k, (const uint4*)v, out_cache_loc,
-                     (uint4*)k_pool, (uint4*)v_pool, pool_rows, table, seq_len, row_vec, max_tokens);
+  hipLaunchKernelGGL(kv_store_chunk_kernel<false>, dim3(wgs), dim3(256), 0, (hipStream_t)stream,
+                     (const uint4*)k, (const uint4*)v, out_cache_loc, (uint4*)k_pool, (uint4*)v_pool,
+                     pool_rows, table, seq_len, rows, row_vec, max_tokens);
   TS_TRY(check_launch("kv_store_chunk_kernel"));
   hipLaunchKernelGGL(seq_len_add_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, seq_len, rows,
                      max_tokens);
