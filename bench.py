@@ -41,7 +41,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # `--pmc WRITE_SIZE` runs of this script (KiB per dispatch, scaled by what the same
 # counters read for the 256 MiB copy of --calibration-copy); the runs and their
 # figures are recorded under profiles/.  Workloads not measured that way give null.
-MEASURED_TRAFFIC = {"C2": 271191716}  # profiles/decode_layer_c2_hbm_traffic.txt
+# Each figure carries the commit of the kernels it was measured on: a later change to the
+# kernel makes it stale until the two counter runs are repeated.
+MEASURED_TRAFFIC = {"C2": (271354153, "015f14b")}  # profiles/decode_layer_c2_hbm_traffic.txt
 
 
 def event_time_us(fn, launches: int, warmup: int, before=None, burst: int = 1):
@@ -159,7 +161,8 @@ def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
     gbs = score_bytes / dom_us / 1e3
     roofline = {"bound": "hbm", "kernel": dom_kernel, "achieved": round(gbs, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC.get(wl.name.split()[0]),
+                "traffic": MEASURED_TRAFFIC.get(wl.name.split()[0], (None, None))[0],
+                "traffic_measured_at": MEASURED_TRAFFIC.get(wl.name.split()[0], (None, None))[1],
                 "bytes_per_launch": score_bytes, "us_per_launch": round(dom_us, 2),
                 "us_min": round(dom_min, 2)}
 
