@@ -215,8 +215,10 @@ __global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
   const int tid = threadIdx.x;
   const int kk = tid >> 3, c8 = tid & 7;
   const int kvh = blockIdx.y;
-  const int S = min(max(*a.sel_len, 0), a.max_sel_len);
   const int j = blockIdx.x * kPfKeys + kk;
+  // (the slot is asked for together with the length, not after it)
+  uint32_t slot = (uint32_t)a.sel[min(j, a.max_sel_len - 1)];
+  const int S = min(max(*a.sel_len, 0), a.max_sel_len);
   // Whole blocks of kPfPadKeys: the keys between S and the next multiple are written as
   // zeros too (their weights are zero, but 0 x garbage is not).
   if (blockIdx.x * kPfKeys >= (S + kPfPadKeys - 1) / kPfPadKeys * kPfPadKeys) return;
@@ -224,7 +226,6 @@ __global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
   uint4 kraw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
   uint4 vraw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
   if (live) {
-    uint32_t slot = (uint32_t)a.sel[j];
     slot = slot < a.pool_rows ? slot : a.pool_rows - 1;
     const size_t at = ((size_t)slot * a.num_kv_heads + kvh) * kHeadDim + 8 * c8;
     kraw[0] = *(const uint4*)(a.k_pool + at);
@@ -606,6 +607,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr bool NEXT = decltype(next)::value;
     const char* const vbase = group_lds + (t & 1) * kPfBufBytes;
     pf_f32x4 s_next[HEADS][2];
+    // The V^T operands are asked for first: they arrive under the logits' products.
+    uint4 vw[8];
+#pragma unroll
+    for (int db = 0; db < 8; ++db) vw[db] = *(const uint4*)(vbase + db * (16 * kPfKeys * 2) + v_at);
     if (NEXT) logits(t + 1, s_next);
     pf_bf16x8 pb[HEADS];
 #pragma unroll
@@ -621,10 +626,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
-      const uint4 vw = *(const uint4*)(vbase + db * (16 * kPfKeys * 2) + v_at);
 #pragma unroll
       for (int rb = 0; rb < HEADS; ++rb)
-        o[rb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw), pb[rb],
+        o[rb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, vw[db]), pb[rb],
                                                            o[rb][db], 0, 0, 0);
     }
 #pragma unroll
