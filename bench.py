@@ -437,6 +437,21 @@ def bench_model(args, ops, dev):
         lambda i: ops.score(c, bt, qf, m.k_pools[i % mc.layers], out=bufs), 2 * mc.layers, mc.layers,
         burst=4)
     del bufs
+    score_only = {"kernel": "ts::score_kernel<Hkv,G,false,1> (ts_score, stand-alone)",
+                  "achieved": round(score_bytes / score_us / 1e3, 1), "unit": "GB/s",
+                  "frac": round(score_bytes / score_us / 1e3 / HBM_PEAK_GBS, 4),
+                  "us_per_launch": round(score_us, 2), "us_min": round(score_min, 2)}
+    dom_kernel = "ts::score_kernel<Hkv,G,false,1> (ts_score, one launch per layer)"
+    if ops.layer_selection_form(c, B, bt.max_seq_len) == 1:
+        # What the layers of this model run: scores and votes request by request, the
+        # scores never in memory (B launches; the figure is all their bytes over all their time).
+        space = ops.select_workspace(c, bt, dev)
+        score_us, score_min = event_time_us(
+            lambda i: ops.score_vote(c, bt, qf, m.k_pools[i % mc.layers], workspace=space),
+            2 * mc.layers, mc.layers, burst=4)
+        dom_kernel = (f"ts::score_kernel<Hkv,G,false,2> votes-only form x {B} launches per layer "
+                      "(ts_score_vote: score + statistics + vote, one request per launch)")
+        del space
     gbs = score_bytes / score_us / 1e3
     weights = sum(w.numel() * 2 for ws in (m.wqkv, m.wo, m.w_gate_up, m.w_down) for w in ws) \
         + m.lm_head.numel() * 2
@@ -457,12 +472,12 @@ def bench_model(args, ops, dev):
         "setup_s": round(build_s, 1),
         "hbm_bytes_per_step": step_bytes,
         "hbm_frac_whole_step": round(step_bytes / step_s / 1e9 / HBM_PEAK_GBS, 4),
-        "roofline": {"bound": "hbm",
-                     "kernel": "ts::score_kernel<Hkv,G,false,1> (ts_score, one launch per layer)",
+        "roofline": {"bound": "hbm", "kernel": dom_kernel,
                      "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "bytes_per_launch": score_bytes, "us_per_launch": round(score_us, 2),
                      "us_min": round(score_min, 2)},
+        "score_only": score_only,
     }
     if not args.no_cpu_baseline:
         import oracle
