@@ -146,7 +146,7 @@ def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
         if any(ops.select_fault(c, bt, space) for space in spaces):
             sys.exit("bench.py: a grid-wide wait of the selection kernel gave up")
         dom_kernel = "ts::score_kernel<Hkv,G,false,2> (ts_select: score + vote + top-k in one launch)"
-    elif ops.layer_selection_form(c, B, bt.max_seq_len) == 1:
+    elif ops.layer_selection_form(c, bt) == 1:
         # Scores and votes request by request, the scores never in memory: B launches of
         # the fused kernel in its votes-only form (+ one small clearing kernel); the
         # figure is the bytes of all of them over the time of all of them.
@@ -154,8 +154,10 @@ def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
         dom_us, dom_min = event_time_us(
             lambda i: ops.score_vote(c, bt, qf, k_pools[i % n_pools], workspace=space), steps, warmup,
             burst=4)
-        dom_kernel = (f"ts::score_kernel<Hkv,G,false,2> votes-only form x {B} launches "
-                      "(ts_score_vote: score + statistics + vote, one request per launch)")
+        dom_kernel = ("ts::score_kernel<Hkv,G,false,2> votes-only form, launches packed by the host's "
+                      "lengths (ts_score_vote: score + statistics + vote)" if bt.host_seq_lens is not None
+                      else f"ts::score_kernel<Hkv,G,false,2> votes-only form x {B} launches "
+                           "(ts_score_vote: score + statistics + vote, one request per launch)")
     else:
         dom_us, dom_min, dom_kernel = score_us, score_min, score_only["kernel"]
     gbs = score_bytes / dom_us / 1e3
@@ -181,6 +183,9 @@ def bench_layer(args, ops, workloads, dev, which=None):
     make = {"c1": workloads.config1, "c2": workloads.config2, "c3": workloads.config3,
             "c5": workloads.config5_layer}[which or args.workload]
     wl = make(dev)
+    # A ragged batch: the lengths are handed over on the host as well (a serving framework
+    # holds them there), so that the launches are packed by what the requests hold.
+    wl.host_lengths = (which or args.workload) == "c3" and not args.device_lengths_only
     c, bt, B = wl.cfg, wl.batch, len(wl.seq_lens)
     layer = ops.DecodeLayer(c, B, bt.max_seq_len, dev)
     n_pools = max(1, args.pools)
@@ -216,7 +221,8 @@ def bench_layer(args, ops, workloads, dev, which=None):
         "data": "synthetic",
         "config": {"workload": wl.name, "batch": B, "seq_lens_max": max(wl.seq_lens),
                    "page_size": c.page_size, "top_k": c.top_k, "n_init": c.n_init,
-                   "n_local": c.n_local, "kv_pool_copies": n_pools},
+                   "n_local": c.n_local, "kv_pool_copies": n_pools,
+                   "lengths_on_host_too": bool(wl.host_lengths)},
         "tokens_per_s": round(B / (us_per_layer * 1e-6 * args.layers), 1),
         "tokens_per_s_note": f"selection+attention only, {args.layers} layers per token",
         "roofline": roofline, "score_only": score_only, "gather_attention": attn,
@@ -572,6 +578,8 @@ def main():
                     help="tokens per KV page of the c4 trace (above 1: appends through the page pool)")
     ap.add_argument("--cpu-requests", type=int, default=2,
                     help="requests of a large batch the CPU oracle is run on")
+    ap.add_argument("--device-lengths-only", action="store_true",
+                    help="c3: do not hand the lengths to the library on the host")
     ap.add_argument("--no-extra", action="store_true",
                     help="default run: only the headline workload, not the compact lines of the others")
     ap.add_argument("--prefill-context", type=int, default=131072,

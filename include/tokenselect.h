@@ -85,6 +85,17 @@ typedef struct ts_batch {
                                without synchronising): set to 1 when a grid-wide
                                wait of a ts_select launch gave up, never cleared
                                by the library                                   */
+  const int32_t* host_seq_lens; /* NULL, or [B] in host memory: upper bounds of
+                               seq_lens[] that the host knows (a serving
+                               framework's CPU copy of the lengths), each <=
+                               max_seq_len.  Only sizes launches: a ragged batch
+                               that is too large for one ts_select launch is then
+                               scored and voted on in launches packed by what
+                               the requests hold (as by ts_score_vote) instead of
+                               by max_seq_len.  The device's seq_lens[] still
+                               rule; a bound below the device's value is an
+                               error the library cannot see (workgroups of the
+                               request would be missing)                        */
 } ts_batch;
 
 /* Optional selection-cache state for one layer (tr.py:301-322, 394-421).
@@ -169,7 +180,9 @@ int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
  * launch per group in which the workgroups meet once to merge the softmax
  * statistics (twice with cfg->pool_kernel > 0) and then write the votes; a batch of
  * any size is served as long as one request fits (some 260K candidates for 32
- * heads) and pool_kernel is at most 256 (ts_score_vote_supported).  votes
+ * heads) and pool_kernel is at most 256 (ts_score_vote_supported).  The groups are
+ * sized by max_seq_len, or, with ts_batch.host_seq_lens, packed by what the requests
+ * hold (up to 16 consecutive requests per launch).  votes
  * [B, vote_stride] fp32 receives what ts_vote's votes (pooled with pool_kernel > 0)
  * would hold, up to the last bit of an fp32 sum taken in another order.  workspace:
  * ts_select_workspace_bytes().  The launches are ordinary ones whose workgroups must
@@ -397,7 +410,8 @@ int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, in
  * When ts_select_supported() holds, the selection runs as the single ts_select
  * kernel; a batch of contexts so long that each request needs the device to itself
  * is scored and voted on request by request as by ts_score_vote and then ranked by
- * the kernels of ts_topk_ragged; otherwise ts_score, ts_vote and ts_topk_ragged run
+ * the kernels of ts_topk_ragged (so is a ragged batch whose lengths the host passes
+ * in ts_batch.host_seq_lens, several requests per launch); otherwise ts_score, ts_vote and ts_topk_ragged run
  * as they do on their own.  All forms give the same selection.
  * ts_set_fused_select(0) forces the separate kernels for the calling process
  * (1 restores the default); it returns the previous setting and has no
@@ -405,8 +419,11 @@ int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, in
 int ts_set_fused_select(int enable);
 /* Which form ts_decode_layer takes for a shape: 2 = ts_select, 1 = ts_score_vote's
  * launches (one request each) + top-k kernels, 0 = ts_score + ts_vote + top-k
- * kernels; -1 for an unsupported configuration. */
+ * kernels; -1 for an unsupported configuration.  The second form answers for a batch
+ * descriptor: with host_seq_lens, a ragged batch too large for one ts_select launch
+ * takes form 1 with several requests per launch, packed by those lengths. */
 int ts_decode_layer_selection(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+int ts_decode_layer_selection_of(const ts_config* cfg, const ts_batch* bt);
 size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
 int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, const float* q_cos,
                     const float* q_sin, const void* k_pool, const void* v_pool,

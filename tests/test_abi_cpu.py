@@ -46,8 +46,8 @@ def test_header_symbols_are_exported_and_bound(lib):
 
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.TsConfig) == 14 * 4
-    assert ctypes.sizeof(_lib.TsBatch) == 8 + 8 + 8 + 8 + 8 + 8
-    assert _lib.TsBatch.fault.offset == 40
+    assert ctypes.sizeof(_lib.TsBatch) == 8 + 8 + 8 + 8 + 8 + 8 + 8
+    assert _lib.TsBatch.fault.offset == 40 and _lib.TsBatch.host_seq_lens.offset == 48
     assert _lib.TsBatch.seq_lens.offset == 8 and _lib.TsBatch.table_stride.offset == 24
     assert ctypes.sizeof(_lib.TsSelCache) == 4 * 8 + 8
 
@@ -92,6 +92,11 @@ def test_null_and_range_errors_need_no_gpu(lib):
                         None) == _lib.TS_EWORKSPACE
     bad = _lib.TsBatch(0, 4096, one, one, 4096, None)
     assert lib.ts_vote(ctypes.byref(c), ctypes.byref(bad), one, 4096, one, None, one, one, None,
+                       4096, None) == _lib.TS_EINVAL
+    # a host-side length beyond max_seq_len
+    lens = (ctypes.c_int32 * 1)(5000)
+    beyond = _lib.TsBatch(1, 4096, one, one, 4096, None, None, ctypes.cast(lens, ctypes.c_void_p))
+    assert lib.ts_vote(ctypes.byref(c), ctypes.byref(beyond), one, 4096, one, None, one, one, None,
                        4096, None) == _lib.TS_EINVAL
     # table rows too short for a batch of 2
     short = _lib.TsBatch(2, 4096, one, one, 100, None)

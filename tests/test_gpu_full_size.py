@@ -37,7 +37,7 @@ def _votes_on_device(wl):
     c, bt, B = wl.cfg, wl.batch, len(wl.seq_lens)
     cos, sin = ops.scoring_cos_sin(c.head_dim, c.rope_theta, c.rope_scale, c.n_local, wl.q.device)
     qf = ops.rope_apply(wl.q.view(B, c.num_heads, c.head_dim), cos, sin, None)
-    form = ops.layer_selection_form(c, B, bt.max_seq_len)
+    form = ops.layer_selection_form(c, bt)
     if form == 2:
         return ops.select(c, bt, qf, wl.k_pool, want_votes=True)[3], qf
     if form == 1:
@@ -147,9 +147,14 @@ def test_scores_at_full_size_against_a_dense_product(dev):
     assert (got - ref).abs().max().item() <= 1e-3 * scale
 
 
-def test_ragged_batch_config(dev):
+@pytest.mark.parametrize("host_lengths", [False, True], ids=["device-lengths", "host-lengths"])
+def test_ragged_batch_config(dev, host_lengths):
+    """With the lengths known on the host as well, the batch is scored and voted on in a few
+    launches packed by those lengths (form 1); without, by the separate kernels (form 0)."""
     wl = workloads.config3(dev)
-    say(f"full size {wl.name} lens={wl.seq_lens}")
+    wl.host_lengths = host_lengths
+    say(f"full size {wl.name} lens={wl.seq_lens} host_lengths={host_lengths}")
+    assert ops.layer_selection_form(wl.cfg, wl.batch) == (1 if host_lengths else 0)
     result = _run(wl, dev)
     votes, _ = _votes_on_device(wl)
     _check_properties(wl, result, votes, wl.name)

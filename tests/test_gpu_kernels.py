@@ -687,6 +687,12 @@ def test_score_vote_in_groups_of_requests(dev, pool_kernel):
     oracle_layer(wl, details)
     votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool, skip=skip), skip=skip)
     votes = ops.score_vote(c, wl.batch, qf, wl.k_pool, skip=skip)
+    # the same with the lengths (here: upper bounds of them) known on the host: the launches are
+    # then packed by what the requests hold, and workgroups without candidates stay out
+    bounds = torch.tensor([min(L + 100, max(lens)) for L in lens], dtype=torch.int32)
+    packed = ops.Batch(wl.batch.seq_lens, wl.batch.table, max(lens), wl.batch.k_per_req,
+                       host_seq_lens=bounds)
+    votes_packed = ops.score_vote(c, packed, qf, wl.k_pool, skip=skip)
     torch.cuda.synchronize()
     for b, L in enumerate(lens):
         if not details[b] or b == 3:
@@ -695,9 +701,10 @@ def test_score_vote_in_groups_of_requests(dev, pool_kernel):
         if pool_kernel > 0 and pool_kernel % 2 == 0:
             n -= 1
         ref = details[b]["votes"][:n]
-        got = votes[b, :n].cpu()
-        assert (got - ref).abs().max().item() <= 2e-4 * ref.abs().max().item(), f"b={b}"
-        assert (got - votes_sep[b, :n].cpu()).abs().max().item() <= 1e-5 * ref.abs().max().item()
+        for name, v in (("grouped", votes), ("packed", votes_packed)):
+            got = v[b, :n].cpu()
+            assert (got - ref).abs().max().item() <= 2e-4 * ref.abs().max().item(), f"{name} b={b}"
+            assert (got - votes_sep[b, :n].cpu()).abs().max().item() <= 1e-5 * ref.abs().max().item()
 
 
 @pytest.mark.parametrize("pool_kernel", [-1, 5])

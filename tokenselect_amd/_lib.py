@@ -35,7 +35,7 @@ class TsConfig(ctypes.Structure):
 class TsBatch(ctypes.Structure):
     _fields_ = [
         ("batch", _i32), ("max_seq_len", _i32), ("seq_lens", _ptr), ("table", _ptr),
-        ("table_stride", _i64), ("k_per_req", _ptr), ("fault", _ptr),
+        ("table_stride", _i64), ("k_per_req", _ptr), ("fault", _ptr), ("host_seq_lens", _ptr),
     ]
 
 
@@ -99,6 +99,7 @@ SIGNATURES = {
                                 _ptr, _i64, _ptr, _ptr, _size, _ptr]),
     "ts_set_fused_select": (_i32, [_i32]),
     "ts_decode_layer_selection": (_i32, [_CFG, _i32, _i32]),
+    "ts_decode_layer_selection_of": (_i32, [_CFG, _BT]),
     "ts_decode_layer_workspace_bytes": (_size, [_CFG, _i32, _i32]),
     "ts_decode_layer_votes": (_i32, [_CFG, _BT, _ptr, _ptr, _ptr, _ptr, _i64, _SC, _ptr, _i64, _ptr,
                                      _size, _ptr]),

@@ -66,6 +66,11 @@ int validate_batch(const ts_config* cfg, const ts_batch* bt) {
   TS_REQUIRE(bt->batch == 1 || bt->table_stride * (int64_t)cfg->page_size >= bt->max_seq_len,
              TS_EINVAL, "table_stride %lld too small for max_seq_len %d at page_size %d",
              (long long)bt->table_stride, bt->max_seq_len, cfg->page_size);
+  if (bt->host_seq_lens)
+    for (int b = 0; b < bt->batch; ++b)
+      TS_REQUIRE(bt->host_seq_lens[b] >= 0 && bt->host_seq_lens[b] <= bt->max_seq_len, TS_EINVAL,
+                 "host_seq_lens[%d] = %d outside [0, max_seq_len %d]", b, bt->host_seq_lens[b],
+                 bt->max_seq_len);
   return TS_OK;
 }
 
@@ -137,10 +142,16 @@ static LayerWorkspace layer_workspace(const ts_config* cfg, int32_t batch, int32
 }
 
 static int layer_selection_form(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
+static int layer_selection_form(const ts_config* cfg, const ts_batch* bt);
 
 int ts_decode_layer_selection(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return -1;
   return layer_selection_form(cfg, batch, max_seq_len);
+}
+
+int ts_decode_layer_selection_of(const ts_config* cfg, const ts_batch* bt) {
+  if (validate_config(cfg) != TS_OK || validate_batch(cfg, bt) != TS_OK) return -1;
+  return layer_selection_form(cfg, bt);
 }
 
 size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
@@ -168,6 +179,16 @@ static int layer_selection_form(const ts_config* cfg, int32_t batch, int32_t max
   // leaves most workgroups of a launch without tokens: those take the separate kernels.
   if (max_n > 0 && cfg->pool_kernel <= 256 && score_votes_group(cfg, batch, max_seq_len) == 1) return 1;
   return 0;
+}
+
+// The same for a batch whose descriptor may carry the host's lengths: a ragged batch too
+// large for one launch then takes form 1 with its launches packed by those lengths (16 x
+// 4K..128K: five launches instead of the fp32 scores written and read back).
+static int layer_selection_form(const ts_config* cfg, const ts_batch* bt) {
+  const int form = layer_selection_form(cfg, bt->batch, bt->max_seq_len);
+  if (form != 0 || !bt->host_seq_lens) return form;
+  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
+  return (max_n > 0 && cfg->pool_kernel <= 256 && score_votes_packed(cfg, bt)) ? 1 : 0;
 }
 
 // Decode (chunk_rows == 0: one query row per request, q_cos / q_sin are the [D] rows
@@ -219,7 +240,7 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
   topk.clear_per_req = cfg->num_kv_heads;
   // A batch too large for one launch of the selection: scores and votes still without
   // the [H, n] scores in memory, one launch per request, then the top-k kernels.
-  const int vote_group = layer_selection_form(cfg, bt->batch, bt->max_seq_len) == 1 ? 1 : 0;
+  const int vote_group = layer_selection_form(cfg, bt) == 1 ? 1 : 0;
   ZeroRegion zero_counters, zero_sync, zero_stats;
   if (one_launch) {
     select_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_counters, &zero_sync);

@@ -7,6 +7,8 @@
 
 namespace ts {
 
+constexpr int kMaxPacked = 16;  // requests per packed launch of the votes-only form
+
 struct ScoreArgs {
   const uint16_t* qf;      // [B,H,128] bf16 rotated fingerprints
   const uint16_t* k_pool;  // [pool_rows,Hkv,128] bf16
@@ -49,6 +51,12 @@ struct ScoreArgs {
   // the votes in memory and their first-level histogram added to the top-k workspace.
   int batch_offset;
   int votes_only;
+  // Votes-only launches packed by the host's lengths: `packed` requests (0: the grid is
+  // [chunks, requests]) share a one-dimensional grid, request r of the launch owning the
+  // workgroups [pack_first[r], pack_first[r + 1]); a workgroup without candidates (the
+  // host's length was an upper bound) leaves at once and is not on the rendezvous team.
+  int packed;
+  int pack_first[kMaxPacked + 1];
   uint32_t* hist_ws;      // per-request top-k workspace (ts_topk.h) whose hist0 is counted into, or NULL
   size_t hist_ws_stride;
   uint32_t* fault_word;   // votes-only: the word the kernels after this one consult
@@ -118,6 +126,9 @@ constexpr uint64_t kSelectWaitTicks = 200000000ull;
 // even one request fits (or the fused kernels are switched off): then the separate
 // kernels serve.  The workspace is that of ts_select for the whole batch; the
 // statistics replicas and the rendezvous areas (score_votes_zero_regions) are zero.
+// Whether the batch is served by votes-only launches packed by the host's lengths
+// (ts_batch.host_seq_lens given, every request fits the device).
+bool score_votes_packed(const ts_config* cfg, const ts_batch* bt);
 int score_votes_group(const ts_config* cfg, int batch, int max_seq_len);
 void score_votes_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* stats,
                               ZeroRegion* sync);

@@ -32,6 +32,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <vector>
 
 #include "ts_score.h"
 #include "ts_topk.h"
@@ -93,7 +94,7 @@ constexpr int kMaxHeads = 128;
 __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const GridTeam& team,
                                                     int lane, int wave) {
   const int H = a.num_heads;
-  const int items = (int)gridDim.y * H;
+  const int items = (a.packed ? a.packed : (int)gridDim.y) * H;
   const int first = (int)team.index * 4 + wave;
   const int step = (int)team.size * 4;
   for (int item = first; item < items; item += step) {
@@ -143,24 +144,31 @@ extern "C" int ts_debug_trace(void* out, size_t bytes) {
 // the requests that select (neither dense nor served by the selection cache).  The
 // others write their fixed output and leave, so that a step in which every request
 // hits the cache costs a few microseconds instead of empty rounds.
-__device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t* lds) {
+// (req, chunk: this workgroup's request within the launch and its chunk of that request.)
+__device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t* lds, int req, int chunk) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int B = gridDim.y, mine = blockIdx.y;
-  uint32_t before = 0, total = 0;  // selecting requests below this one / in all
+  const int B = a.packed ? a.packed : (int)gridDim.y, mine = req;
+  // Members per selecting request: the whole row of the grid, or (packed launches) only
+  // the workgroups that hold candidates.
+  uint32_t before = 0, total = 0;  // members of the requests below this one / of all
   for (int base = 0; base < B; base += 256) {
     const int b = a.batch_offset + base + tid;  // requests of this launch
-    bool selects = false;
-    if (base + tid < B && !(a.skip && a.skip[b]))
-      selects = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
-                                 a.max_seq_len).n > 0;
-    const uint64_t mask = __ballot(selects);
+    uint32_t members = 0;
+    if (base + tid < B && !(a.skip && a.skip[b])) {
+      const int n = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
+                                     a.max_seq_len).n;
+      if (n > 0)
+        members = a.packed ? (uint32_t)((n + a.tokens_per_block - 1) / a.tokens_per_block) : gridDim.x;
+    }
+    uint32_t sum = members, below = base + tid < mine ? members : 0u;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      sum += (uint32_t)__shfl_xor((int)sum, off);
+      below += (uint32_t)__shfl_xor((int)below, off);
+    }
     if (lane == 0) {
-      lds[wave] = (uint32_t)__popcll(mask);
-      // requests of this chunk below `mine` that lie in this wavefront's 64
-      const int lo = base + 64 * wave;
-      const int upto = mine - lo;  // bits [0, upto) count
-      lds[4 + wave] = upto <= 0 ? 0u
-                                : (uint32_t)__popcll(upto >= 64 ? mask : mask & ((1ull << upto) - 1ull));
+      lds[wave] = sum;
+      lds[4 + wave] = below;
     }
     __syncthreads();
     for (int w = 0; w < 4; ++w) {
@@ -170,8 +178,8 @@ __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t*
     __syncthreads();
   }
   GridTeam team;
-  team.size = total * gridDim.x + a.absent;
-  team.index = before * gridDim.x + blockIdx.x;
+  team.size = total + a.absent;
+  team.index = before + (uint32_t)chunk;
   return team;
 }
 
@@ -288,7 +296,14 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   constexpr int ITER = 16 * TG;    // tokens per iteration
   constexpr uint32_t ROW_BYTES = HKV * kHeadDim * 2;
 
-  const int b = blockIdx.y + a.batch_offset;
+  // This workgroup's request within the launch, and its chunk of that request.
+  int req = blockIdx.y, chunk = blockIdx.x;
+  if (a.packed) {
+    req = 0;
+    while (req + 1 < a.packed && (int)blockIdx.x >= a.pack_first[req + 1]) ++req;
+    chunk = (int)blockIdx.x - a.pack_first[req];
+  }
+  const int b = req + a.batch_offset;
   int n, first_pos;
   if (a.direct_n >= 0) {
     n = (int)a.direct_n;
@@ -299,14 +314,15 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     n = (a.skip && a.skip[b]) ? 0 : geo.n;
     first_pos = a.n_init;
   }
-  const int block_lo = blockIdx.x * a.tokens_per_block;
+  const int block_lo = chunk * a.tokens_per_block;
   GridTeam team{0u, 0u};
   if constexpr (MODE == kScoreFused) {
     __shared__ uint32_t team_lds[8];
     TS_MARK(0);
     if (!a.votes_only) fixed_segments(a, b);
     if (n <= 0) return;  // dense or served by the cache: nothing to select, not on the team
-    team = selecting_team(a, team_lds);
+    if (a.packed && block_lo >= n) return;  // no candidates here, and the team is made without it
+    team = selecting_team(a, team_lds, req, chunk);
   }
   if (block_lo >= n) {
     if constexpr (MODE == kScoreFused) {  // no tokens here: only help with the statistics
@@ -530,7 +546,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
 #pragma unroll
       for (int w = 1; w < 4; ++w) softmax_merge(m, l, sm_m[w][g4][kvh][na], sm_l[w][g4][kvh][na]);
       const int h = head_of<HKV, G>(kvh, g, a.head_map);
-      float2* out = (float2*)a.partials + ((size_t)b * H + h) * a.nchunks + blockIdx.x;
+      float2* out = (float2*)a.partials + ((size_t)b * H + h) * a.nchunks + chunk;
       if (MODE == kScoreFused) {
         store_coherent(out, m, l);
         local_max[kvh * G + g] = m;
@@ -651,7 +667,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         for (int i = tid; i < kTopkBins; i += 256)
           if (lh[i]) atomicAdd(&hist0[i], lh[i]);
       }
-      if (blockIdx.x == 0 && tid == 0 && load_coherent(&a.sync[0]) != 0u) {
+      if (chunk == 0 && tid == 0 && load_coherent(&a.sync[0]) != 0u) {
         __hip_atomic_store(a.fault_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (a.fault_out)
           __hip_atomic_store(a.fault_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -1089,17 +1105,11 @@ static std::atomic<int> g_fused_select{1};
 
 int set_fused_select(int enable) { return g_fused_select.exchange(enable ? 1 : 0); }
 
-int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch) {
-  // Max-pool windows beyond 256 would not fit the LDS the neighbours are gathered into.
-  if ((!ignore_switch && !g_fused_select.load()) || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256)
-    return 0;
-  const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
-  if (max_n <= 0) return 0;
-  const int group = cfg->num_heads / cfg->num_kv_heads;
-  const void* fn = fused_kernel_of(cfg->num_kv_heads, group);
+// Workgroups of the fused kernel that the current device keeps resident at once (0: the
+// shape has no fused kernel, or the runtime refused); depends on the kernel only.
+static int fused_capacity(const ts_config* cfg) {
+  const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
   if (!fn) return 0;
-
-  // Workgroups the device keeps resident at once; depends on the kernel only.
   struct Entry { const void* fn; int device; int capacity; };
   static thread_local Entry memo[4] = {};
   int device = 0;
@@ -1124,6 +1134,17 @@ int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, boo
     static thread_local int next = 0;
     memo[next++ % 4] = Entry{fn, device, capacity};
   }
+  return capacity;
+}
+
+int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch) {
+  // Max-pool windows beyond 256 would not fit the LDS the neighbours are gathered into.
+  if ((!ignore_switch && !g_fused_select.load()) || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256)
+    return 0;
+  const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
+  if (max_n <= 0) return 0;
+  const int capacity = fused_capacity(cfg);
+  if (capacity <= 0) return 0;
 
   int tpb = score_tokens_per_block((int64_t)batch * max_seq_len, cfg->num_heads);
   while ((int64_t)ceil_div(max_n, tpb) * batch > capacity) tpb += 64;
@@ -1282,9 +1303,108 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   return TS_OK;
 }
 
+// Launches of the votes-only form when the host knows upper bounds of the lengths
+// (ts_batch.host_seq_lens): consecutive requests are packed into a launch by what they
+// hold, not by max_seq_len -- as many as fit the device with the most tokens per
+// workgroup that the LDS takes, then the fewest tokens per workgroup with which they
+// still fit.  The grid of such a launch is one-dimensional and has no more workgroups
+// than the device keeps resident, every one of them with candidates by the host's
+// count: a grid [chunks of the longest, requests] with the short requests' surplus
+// workgroups leaving at once would hold no more members, but the workgroups of a grid go
+// to the XCDs (and further down) in turn by their number, and members with gaps between
+// them do not spread evenly: such launches were seen to wait for room that never came.
+struct VoteLaunch {
+  int first, requests, tokens_per_block, workgroups, table_chunks;
+};
+
+bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<VoteLaunch>* plan) {
+  plan->clear();
+  if (!bt->host_seq_lens || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256) return false;
+  const int capacity = fused_capacity(cfg);
+  if (capacity <= 0) return false;
+  int tpb_max = 64;
+  while (fused_lds_bytes(tpb_max + 64, cfg->num_heads) <= kFusedStageBytes) tpb_max += 64;
+  if (fused_lds_bytes(tpb_max, cfg->num_heads) > kFusedStageBytes) return false;
+  const int fixed = cfg->n_init + cfg->n_local;
+  auto candidates = [&](int b) { return std::max(std::min(bt->host_seq_lens[b], bt->max_seq_len) - fixed, 0); };
+  for (int first = 0; first < bt->batch;) {
+    int64_t wgs = 0;
+    int last = first, longest = 0;
+    for (; last < bt->batch && last - first < kMaxPacked; ++last) {
+      const int64_t more = ceil_div(candidates(last), tpb_max);
+      if (wgs + more > capacity) break;
+      wgs += more;
+      longest = std::max(longest, std::min(bt->host_seq_lens[last], bt->max_seq_len));
+    }
+    if (last == first) return false;  // a single request does not fit the device
+    // the statistics' table of a request holds at most kSelMaxChunks chunks
+    int tpb = (int)std::max<int64_t>(64, ceil_div(ceil_div(longest, kSelMaxChunks), 64) * 64);
+    if (tpb > tpb_max) return false;
+    for (; tpb <= tpb_max; tpb += 64) {
+      wgs = 0;
+      for (int b = first; b < last; ++b) wgs += ceil_div(candidates(b), tpb);
+      if (wgs <= capacity) break;
+    }
+    if (tpb > tpb_max) return false;
+    if (wgs > 0)  // (nothing to launch for requests that are all sink and local window)
+      plan->push_back(VoteLaunch{first, last - first, tpb, (int)wgs, (int)ceil_div(longest, tpb)});
+    first = last;
+  }
+  return true;
+}
+
+bool score_votes_packed(const ts_config* cfg, const ts_batch* bt) {
+  std::vector<VoteLaunch> plan;
+  return plan_vote_launches(cfg, bt, &plan);
+}
+
 int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
                        int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
                        uint32_t* hist_ws, size_t hist_ws_stride, void* workspace, hipStream_t stream) {
+  std::vector<VoteLaunch> plan;
+  if (plan_vote_launches(cfg, bt, &plan)) {
+    const SelectWorkspace all = select_workspace(cfg, bt->batch, bt->max_seq_len, true);
+    char* ws = (char*)workspace;
+    const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
+    int launch = 0;
+    for (const VoteLaunch& v : plan) {
+      ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, skip, (float*)(ws + all.partials),
+                                   v.tokens_per_block);
+      a.nchunks = v.table_chunks;
+      a.sync = (uint32_t*)(ws + all.sync) + (size_t)launch++ * kSyncWords;
+      a.fault_word = (uint32_t*)(ws + all.sync);
+      a.stats = (float*)(ws + all.stats);
+      a.stats_stride = all.stats_stride;
+      a.votes = votes;
+      a.vote_stride = vote_stride;
+      a.counters = (uint32_t*)(ws + all.counters);
+      a.spin_ticks = kSelectWaitTicks;
+      a.fault_out = bt->fault;
+      a.pool_kernel = cfg->pool_kernel;
+      a.pool_votes = (float*)(ws + all.pool_votes);
+      a.pool_stride = all.pool_stride;
+      a.batch_offset = v.first;
+      a.votes_only = 1;
+      a.packed = v.requests;
+      a.pack_first[0] = 0;
+      const int fixed = cfg->n_init + cfg->n_local;
+      for (int r = 0; r < v.requests; ++r) {
+        const int cand = std::max(std::min(bt->host_seq_lens[v.first + r], bt->max_seq_len) - fixed, 0);
+        a.pack_first[r + 1] = a.pack_first[r] + (int)ceil_div(cand, v.tokens_per_block);
+      }
+      a.hist_ws = hist_ws;
+      a.hist_ws_stride = hist_ws_stride;
+      const dim3 grid((unsigned)v.workgroups, 1u);
+      void* params[] = {(void*)&a};
+      const hipError_t e = hipLaunchKernel(fn, grid, dim3(256), params,
+                                           fused_lds_bytes(v.tokens_per_block, cfg->num_heads), stream);
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(TS_EHIP, "fused scoring + vote launch: %s", hipGetErrorString(e));
+      }
+    }
+    return TS_OK;
+  }
   const int group = score_votes_group(cfg, bt->batch, bt->max_seq_len);
   TS_REQUIRE(group > 0, TS_ESHAPE, "fused scoring + vote: not even one request of %d tokens fits",
              bt->max_seq_len);

@@ -7,6 +7,7 @@ and there is no fallback path.
 """
 
 import ctypes
+import dataclasses
 from dataclasses import dataclass
 from typing import Optional, Tuple
 
@@ -64,6 +65,10 @@ class Batch:
     # One int32 word of pinned host memory (see fault_word()) that the single-launch
     # selection sets to 1 when one of its grid-wide waits gave up, or None.
     fault: Optional[torch.Tensor] = None
+    # Upper bounds of seq_lens that the host knows ([B] int32 on the CPU, e.g. a serving
+    # framework's CPU copy of the lengths), or None: a ragged batch too large for one
+    # selection launch is then served in launches packed by what the requests hold.
+    host_seq_lens: Optional[torch.Tensor] = None
 
     @property
     def batch(self) -> int:
@@ -156,8 +161,14 @@ def _c_batch(cfg: LayerConfig, bt: Batch) -> TsBatch:
     if bt.fault is not None and (bt.fault.dtype != torch.int32 or bt.fault.numel() != 1 or
                                  not (bt.fault.is_cuda or bt.fault.is_pinned())):
         raise ValueError("fault must be one int32 word of device or pinned host memory")
+    if bt.host_seq_lens is not None and (
+            bt.host_seq_lens.dtype != torch.int32 or bt.host_seq_lens.is_cuda or
+            bt.host_seq_lens.dim() != 1 or bt.host_seq_lens.shape[0] != bt.batch or
+            not bt.host_seq_lens.is_contiguous()):
+        raise ValueError("host_seq_lens must be a contiguous [B] int32 tensor on the CPU")
+    host = bt.host_seq_lens.data_ptr() if bt.host_seq_lens is not None else None
     return TsBatch(bt.batch, int(bt.max_seq_len), _p(bt.seq_lens), _p(bt.table),
-                   int(bt.table.stride(0)), _p(bt.k_per_req), _p(bt.fault))
+                   int(bt.table.stride(0)), _p(bt.k_per_req), _p(bt.fault), host)
 
 
 def _c_cache(cache: Optional[SelectionCache], cfg: LayerConfig, batch: int):
@@ -389,9 +400,13 @@ def vote(cfg: LayerConfig, bt: Batch, scores: torch.Tensor, partials: torch.Tens
     return (pooled if pooled is not None else votes), stats
 
 
-def layer_selection_form(cfg: LayerConfig, batch: int, max_seq_len: int) -> int:
-    """How :class:`DecodeLayer` selects for a shape: 2 = one ``ts_select`` launch, 1 =
-    ``ts_score_vote`` request by request + the top-k kernels, 0 = the separate kernels."""
+def layer_selection_form(cfg: LayerConfig, batch, max_seq_len: Optional[int] = None) -> int:
+    """How :class:`DecodeLayer` selects for a shape ``(batch, max_seq_len)`` or for a
+    :class:`Batch` (whose ``host_seq_lens`` count): 2 = one ``ts_select`` launch, 1 =
+    ``ts_score_vote``'s launches + the top-k kernels, 0 = the separate kernels."""
+    if isinstance(batch, Batch):
+        cb = _c_batch(cfg, batch)
+        return int(_lib.load().ts_decode_layer_selection_of(ctypes.byref(cfg.to_c()), ctypes.byref(cb)))
     return int(_lib.load().ts_decode_layer_selection(ctypes.byref(cfg.to_c()), int(batch),
                                                      int(max_seq_len)))
 
@@ -641,7 +656,7 @@ class DecodeLayer:
         cfg = self.cfg
         self.check()
         if bt.fault is None:
-            bt = Batch(bt.seq_lens, bt.table, bt.max_seq_len, bt.k_per_req, self.fault)
+            bt = dataclasses.replace(bt, fault=self.fault)
         cb = _c_batch(cfg, bt)
         if bt.batch > self.batch or bt.max_seq_len > self.max_seq_len:
             raise ValueError("batch / max_seq_len exceed what this DecodeLayer was sized for")
@@ -674,7 +689,7 @@ class DecodeLayer:
         cfg = self.cfg
         self.check()
         if bt.fault is None:
-            bt = Batch(bt.seq_lens, bt.table, bt.max_seq_len, bt.k_per_req, self.fault)
+            bt = dataclasses.replace(bt, fault=self.fault)
         cb = _c_batch(cfg, bt)
         if bt.batch > self.batch or bt.max_seq_len > self.max_seq_len:
             raise ValueError("batch / max_seq_len exceed what this DecodeLayer was sized for")
@@ -696,7 +711,7 @@ class DecodeLayer:
                bt: Batch, cache: Optional[SelectionCache] = None, out: Optional[torch.Tensor] = None):
         cfg = self.cfg
         if bt.fault is None:
-            bt = Batch(bt.seq_lens, bt.table, bt.max_seq_len, bt.k_per_req, self.fault)
+            bt = dataclasses.replace(bt, fault=self.fault)
         cb = _c_batch(cfg, bt)
         _need(q, "q", torch.bfloat16)
         _need(votes, "votes", torch.float32, 2)
@@ -823,7 +838,7 @@ class PrefillChunk:
         cfg = self.cfg
         self.check()
         if bt.fault is None:
-            bt = Batch(bt.seq_lens, bt.table, bt.max_seq_len, bt.k_per_req, self.fault)
+            bt = dataclasses.replace(bt, fault=self.fault)
         cb = _c_batch(cfg, bt)
         _need(q, "q", torch.bfloat16, 2)
         rows = q.shape[0]

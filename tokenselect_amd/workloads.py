@@ -34,10 +34,13 @@ class Workload:
     k_per_req: Optional[torch.Tensor] = None
     planted: List[torch.Tensor] = field(default_factory=list)  # per request: logical positions
     free_pages: Optional[torch.Tensor] = None   # [extra_pages] int32: pages no request holds
+    host_lengths: bool = False                  # hand the lengths to the library on the host too
 
     @property
     def batch(self) -> Batch:
-        return Batch(self.seq_lens_dev, self.table, max(self.seq_lens), self.k_per_req)
+        host = torch.tensor(self.seq_lens, dtype=torch.int32) if self.host_lengths else None
+        return Batch(self.seq_lens_dev, self.table, max(self.seq_lens), self.k_per_req,
+                     host_seq_lens=host)
 
     def score_bytes(self) -> int:
         """Algorithmic bytes of the scoring pass: every candidate K row once,
