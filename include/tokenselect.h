@@ -182,7 +182,7 @@ int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
  * any size is served as long as one request fits (some 260K candidates for 32
  * heads) and pool_kernel is at most 256 (ts_score_vote_supported).  The groups are
  * sized by max_seq_len, or, with ts_batch.host_seq_lens, packed by what the requests
- * hold (up to 16 consecutive requests per launch).  votes
+ * hold (up to 8 consecutive requests per launch).  votes
  * [B, vote_stride] fp32 receives what ts_vote's votes (pooled with pool_kernel > 0)
  * would hold, up to the last bit of an fp32 sum taken in another order.  workspace:
  * ts_select_workspace_bytes().  The launches are ordinary ones whose workgroups must

@@ -7,7 +7,7 @@
 
 namespace ts {
 
-constexpr int kMaxPacked = 16;  // requests per packed launch of the votes-only form
+constexpr int kMaxPacked = 8;   // requests per packed launch of the votes-only form
 
 struct ScoreArgs {
   const uint16_t* qf;      // [B,H,128] bf16 rotated fingerprints

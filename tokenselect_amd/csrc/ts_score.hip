@@ -83,6 +83,9 @@ constexpr int kQuadSwap2 = 0x4E;  // quad_perm [2,3,0,1]
 //     where its selected positions, in ascending order, belong (tr.py:371-373,
 //     433-449); masses of exact ties go through all three levels and a count round.
 constexpr int kScoreDirect = 0, kScoreTiled = 1, kScoreFused = 2;
+// The fused kernel's votes-only form for launches packed by the host's lengths: a kernel
+// of its own, so that the single-launch selection does not carry the bookkeeping.
+constexpr int kScorePacked = 3;
 constexpr int kMaxHeads = 128;
 
 // After the first rendezvous of the fused kernel: the (request, head) pairs are dealt
@@ -91,10 +94,11 @@ constexpr int kMaxHeads = 128;
 // replicas, lane r into replica r.  The workgroups poll the words of the replica of
 // their index until they are there (a sum of exponentials is never zero): the data is
 // its own flag, which saves a rendezvous.
+template <bool PACKED>
 __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const GridTeam& team,
                                                     int lane, int wave) {
   const int H = a.num_heads;
-  const int items = (a.packed ? a.packed : (int)gridDim.y) * H;
+  const int items = (PACKED ? a.packed : (int)gridDim.y) * H;
   const int first = (int)team.index * 4 + wave;
   const int step = (int)team.size * 4;
   for (int item = first; item < items; item += step) {
@@ -145,30 +149,43 @@ extern "C" int ts_debug_trace(void* out, size_t bytes) {
 // others write their fixed output and leave, so that a step in which every request
 // hits the cache costs a few microseconds instead of empty rounds.
 // (req, chunk: this workgroup's request within the launch and its chunk of that request.)
+template <bool PACKED>
 __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t* lds, int req, int chunk) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int B = a.packed ? a.packed : (int)gridDim.y, mine = req;
-  // Members per selecting request: the whole row of the grid, or (packed launches) only
-  // the workgroups that hold candidates.
-  uint32_t before = 0, total = 0;  // members of the requests below this one / of all
-  for (int base = 0; base < B; base += 256) {
-    const int b = a.batch_offset + base + tid;  // requests of this launch
-    uint32_t members = 0;
-    if (base + tid < B && !(a.skip && a.skip[b])) {
+  GridTeam team;
+  if (PACKED) {
+    // A packed launch holds a handful of requests and its members are the workgroups
+    // that hold candidates: every thread adds them up for itself.
+    uint32_t before = 0, total = 0;
+    for (int r = 0; r < a.packed; ++r) {
+      const int b = a.batch_offset + r;
+      if (a.skip && a.skip[b]) continue;
       const int n = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
                                      a.max_seq_len).n;
-      if (n > 0)
-        members = a.packed ? (uint32_t)((n + a.tokens_per_block - 1) / a.tokens_per_block) : gridDim.x;
+      const uint32_t members = n > 0 ? (uint32_t)((n + a.tokens_per_block - 1) / a.tokens_per_block) : 0u;
+      total += members;
+      if (r < req) before += members;
     }
-    uint32_t sum = members, below = base + tid < mine ? members : 0u;
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-      sum += (uint32_t)__shfl_xor((int)sum, off);
-      below += (uint32_t)__shfl_xor((int)below, off);
-    }
+    team.size = total + a.absent;
+    team.index = before + (uint32_t)chunk;
+    return team;
+  }
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int B = gridDim.y, mine = req;
+  uint32_t before = 0, total = 0;  // selecting requests below this one / in all
+  for (int base = 0; base < B; base += 256) {
+    const int b = a.batch_offset + base + tid;  // requests of this launch
+    bool selects = false;
+    if (base + tid < B && !(a.skip && a.skip[b]))
+      selects = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
+                                 a.max_seq_len).n > 0;
+    const uint64_t mask = __ballot(selects);
     if (lane == 0) {
-      lds[wave] = sum;
-      lds[4 + wave] = below;
+      lds[wave] = (uint32_t)__popcll(mask);
+      // requests of this chunk below `mine` that lie in this wavefront's 64
+      const int lo = base + 64 * wave;
+      const int upto = mine - lo;  // bits [0, upto) count
+      lds[4 + wave] = upto <= 0 ? 0u
+                                : (uint32_t)__popcll(upto >= 64 ? mask : mask & ((1ull << upto) - 1ull));
     }
     __syncthreads();
     for (int w = 0; w < 4; ++w) {
@@ -177,9 +194,8 @@ __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t*
     }
     __syncthreads();
   }
-  GridTeam team;
-  team.size = total + a.absent;
-  team.index = before + (uint32_t)chunk;
+  team.size = total * gridDim.x + a.absent;
+  team.index = before * gridDim.x + (uint32_t)chunk;
   return team;
 }
 
@@ -289,6 +305,8 @@ template <int HKV, int G, bool OUT_BF16, int MODE>
 __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a) {
   extern __shared__ float stage[];  // tiled / fused: [tiles of the workgroup][tile_stride]
   constexpr bool TILED = MODE != kScoreDirect;
+  constexpr bool FUSED = MODE == kScoreFused || MODE == kScorePacked;
+  constexpr bool PACKED = MODE == kScorePacked;
   constexpr int TG = 8 / HKV;
   constexpr int UNITS = 8;
   constexpr int HALF = UNITS / 2;
@@ -298,7 +316,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
 
   // This workgroup's request within the launch, and its chunk of that request.
   int req = blockIdx.y, chunk = blockIdx.x;
-  if (a.packed) {
+  if (PACKED) {
     req = 0;
     while (req + 1 < a.packed && (int)blockIdx.x >= a.pack_first[req + 1]) ++req;
     chunk = (int)blockIdx.x - a.pack_first[req];
@@ -316,18 +334,18 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   }
   const int block_lo = chunk * a.tokens_per_block;
   GridTeam team{0u, 0u};
-  if constexpr (MODE == kScoreFused) {
+  if constexpr (FUSED) {
     __shared__ uint32_t team_lds[8];
     TS_MARK(0);
     if (!a.votes_only) fixed_segments(a, b);
     if (n <= 0) return;  // dense or served by the cache: nothing to select, not on the team
-    if (a.packed && block_lo >= n) return;  // no candidates here, and the team is made without it
-    team = selecting_team(a, team_lds, req, chunk);
+    if (PACKED && block_lo >= n) return;  // no candidates here, and the team is made without it
+    team = selecting_team<PACKED>(a, team_lds, req, chunk);
   }
   if (block_lo >= n) {
-    if constexpr (MODE == kScoreFused) {  // no tokens here: only help with the statistics
+    if constexpr (FUSED) {  // no tokens here: only help with the statistics
       grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
-      merge_request_stats(a, team, threadIdx.x & 63, threadIdx.x >> 6);
+      merge_request_stats<PACKED>(a, team, threadIdx.x & 63, threadIdx.x >> 6);
       const uint32_t rounds = (a.votes_only ? 1u : kSelectRounds) + (a.pool_kernel > 0 ? 1u : 0u);
       for (uint32_t round = 2; round <= rounds; ++round)
         grid_arrive(a.sync, round, false, a.spin_ticks, team.size, team.index);
@@ -344,7 +362,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   const int H = a.num_heads;
   // Fused: one spare row per tile keeps the four tiles a wavefront reads in the
   // vote phase on different LDS banks.
-  const int tile_stride = MODE == kScoreFused ? 16 * H + 16 : 16 * H;
+  const int tile_stride = FUSED ? 16 * H + 16 : 16 * H;
   const int32_t* tab = a.table + (int64_t)b * a.table_stride;
 
   // A operands: query 4*na + t4 of each KV head, same byte offsets as the keys.
@@ -521,7 +539,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   if (a.partials == nullptr) return;
 
   // Per-workgroup (max, sum exp) of every head: 16 lanes of a row, then 4 waves.
-  __shared__ float local_max[MODE == kScoreFused ? kMaxHeads : 1];  // by head slot
+  __shared__ float local_max[FUSED ? kMaxHeads : 1];  // by head slot
   __shared__ float sm_m[4][4][HKV][NA];
   __shared__ float sm_l[4][4][HKV][NA];
 #pragma unroll
@@ -547,7 +565,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       for (int w = 1; w < 4; ++w) softmax_merge(m, l, sm_m[w][g4][kvh][na], sm_l[w][g4][kvh][na]);
       const int h = head_of<HKV, G>(kvh, g, a.head_map);
       float2* out = (float2*)a.partials + ((size_t)b * H + h) * a.nchunks + chunk;
-      if (MODE == kScoreFused) {
+      if (FUSED) {
         store_coherent(out, m, l);
         local_max[kvh * G + g] = m;
       } else {
@@ -556,7 +574,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     }
   }
 
-  if constexpr (MODE == kScoreFused) {
+  if constexpr (FUSED) {
     __shared__ float s_rz[kMaxHeads];
     __shared__ uint32_t lh[kTopkBins];
     __shared__ uint32_t scratch[16];
@@ -566,7 +584,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     TS_MARK(1);
     grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
     TS_MARK(2);
-    merge_request_stats(a, team, lane, wave);
+    merge_request_stats<PACKED>(a, team, lane, wave);
     TS_MARK(3);
     // While the merged statistics are on their way: the exponentials, relative to this
     // workgroup's own maxima; exp(s - max) / sum = exp(s - own max) * exp(own max - max) / sum.
@@ -657,7 +675,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       for (int i = tid; i < count + halo; i += 256) lh[i] = 0u;
       __syncthreads();
     }
-    if (a.votes_only) {
+    if (PACKED || a.votes_only) {
       // The launch ends here: the votes are in memory, and their first histogram level
       // goes to the top-k workspace, where the kernels after this one pick it up.
       if (a.hist_ws) {
@@ -1077,10 +1095,12 @@ static int launch_score(int hkv, int group, const ScoreArgs& a, dim3 grid, hipSt
   return fail(TS_ESHAPE, "unsupported head shape: num_kv_heads=%d group=%d", hkv, group);
 }
 
-// The fused kernel of a head shape, or NULL.
-static const void* fused_kernel_of(int hkv, int group) {
-#define TS_SCORE_CASE(HKV_, G_) \
-  if (hkv == HKV_ && group == G_) return (const void*)&score_kernel<HKV_, G_, false, kScoreFused>;
+// The fused kernel of a head shape (its packed votes-only form), or NULL.
+static const void* fused_kernel_of(int hkv, int group, bool packed = false) {
+#define TS_SCORE_CASE(HKV_, G_)                                                        \
+  if (hkv == HKV_ && group == G_)                                                      \
+    return packed ? (const void*)&score_kernel<HKV_, G_, false, kScorePacked>          \
+                  : (const void*)&score_kernel<HKV_, G_, false, kScoreFused>;
 #define TS_SCORE_ROW(HKV_) \
   TS_SCORE_CASE(HKV_, 1) TS_SCORE_CASE(HKV_, 2) TS_SCORE_CASE(HKV_, 4) TS_SCORE_CASE(HKV_, 7) TS_SCORE_CASE(HKV_, 8)
   TS_SCORE_ROW(1)
@@ -1107,11 +1127,11 @@ int set_fused_select(int enable) { return g_fused_select.exchange(enable ? 1 : 0
 
 // Workgroups of the fused kernel that the current device keeps resident at once (0: the
 // shape has no fused kernel, or the runtime refused); depends on the kernel only.
-static int fused_capacity(const ts_config* cfg) {
-  const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
+static int fused_capacity(const ts_config* cfg, bool packed = false) {
+  const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, packed);
   if (!fn) return 0;
   struct Entry { const void* fn; int device; int capacity; };
-  static thread_local Entry memo[4] = {};
+  static thread_local Entry memo[8] = {};
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return 0;
   int capacity = 0;
@@ -1132,7 +1152,7 @@ static int fused_capacity(const ts_config* cfg) {
     capacity = per_cu * cus;
     if (capacity <= 0) return 0;
     static thread_local int next = 0;
-    memo[next++ % 4] = Entry{fn, device, capacity};
+    memo[next++ % 8] = Entry{fn, device, capacity};
   }
   return capacity;
 }
@@ -1320,7 +1340,7 @@ struct VoteLaunch {
 bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<VoteLaunch>* plan) {
   plan->clear();
   if (!bt->host_seq_lens || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256) return false;
-  const int capacity = fused_capacity(cfg);
+  const int capacity = fused_capacity(cfg, /*packed=*/true);
   if (capacity <= 0) return false;
   int tpb_max = 64;
   while (fused_lds_bytes(tpb_max + 64, cfg->num_heads) <= kFusedStageBytes) tpb_max += 64;
@@ -1365,7 +1385,7 @@ int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf,
   if (plan_vote_launches(cfg, bt, &plan)) {
     const SelectWorkspace all = select_workspace(cfg, bt->batch, bt->max_seq_len, true);
     char* ws = (char*)workspace;
-    const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
+    const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, true);
     int launch = 0;
     for (const VoteLaunch& v : plan) {
       ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, skip, (float*)(ws + all.partials),
