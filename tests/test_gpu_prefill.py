@@ -158,6 +158,35 @@ def test_sparse_prefill_attention_fewer_keys_than_rows(dev):
         assert torch.count_nonzero(out).item() == 0, reported
 
 
+@pytest.mark.parametrize("rows", [1, 7, 8, 9, 513, 8184, 8200])
+def test_kv_store_chunk_sizes(dev, rows):
+    """Chunks around the eight rows of a workgroup, a chunk that overflows the table, and
+    chunks on both sides of the size up to which the store also writes the length (larger
+    ones take a second launch for it)."""
+    say(f"kv_store_chunk rows={rows}")
+    cfg = ops.LayerConfig(num_heads=4, num_kv_heads=2, n_local=16, top_k=16, rope_theta=1e4)
+    g = torch.Generator(device=dev).manual_seed(rows)
+    L0, pool_rows = 30, 30 + 8200
+    max_tokens = L0 + rows if rows != 513 else L0 + 500      # 513 rows: the last 13 do not fit
+    k_pool = torch.zeros((pool_rows, 2, 128), dtype=torch.bfloat16, device=dev)
+    v_pool = torch.zeros_like(k_pool)
+    k = torch.randn((rows, 2, 128), generator=g, device=dev).bfloat16()
+    v = torch.randn((rows, 2, 128), generator=g, device=dev).bfloat16()
+    loc = (L0 + torch.randperm(8200, generator=g, device=dev)[:rows]).int()
+    table = torch.full((max_tokens,), -1, dtype=torch.int32, device=dev)
+    table[:L0] = torch.arange(L0, dtype=torch.int32, device=dev)
+    seq = torch.tensor([L0], dtype=torch.int32, device=dev)
+    for _ in range(2):      # twice: the length word is left clean for the next call
+        seq.fill_(L0)
+        ops.kv_store_chunk(cfg, k, v, loc, k_pool, v_pool, table, seq)
+        torch.cuda.synchronize()
+        kept = min(rows, max_tokens - L0)
+        assert int(seq) == L0 + kept
+        assert torch.equal(table[L0:L0 + kept], loc[:kept])
+        assert torch.equal(k_pool[loc[:kept].long()], k[:kept]) and torch.equal(v_pool[loc[:kept].long()], v[:kept])
+        assert torch.equal(table[:L0], torch.arange(L0, dtype=torch.int32, device=dev))
+
+
 def test_kv_store_chunk(dev):
     say("kv_store_chunk")
     wl = workloads.build("pf", SHAPES[0], [100], [16], 1, dev, seed=7, n_init=4, n_local=16,
