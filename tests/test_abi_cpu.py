@@ -130,8 +130,9 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit(lib):
     assert lib.ts_attn_static_scratch_bytes() == 4 << 20
     one = ctypes.c_void_p(0x1000)  # never dereferenced: the size check fails first
     wide = cfg(num_heads=64, num_kv_heads=8, top_k=4096)
+    # 130 requests x 64 heads x 512 bytes of partials per head and split: above 4 MiB
     assert lib.ts_sparse_decode_attn_static(ctypes.byref(wide), one, one, one, 10, one, 4736, one,
-                                            63, 4736, one, None) == _lib.TS_EWORKSPACE
+                                            130, 4736, one, None) == _lib.TS_EWORKSPACE
     assert "scratch" in err(lib)
     assert lib.ts_sparse_decode_attn_static(ctypes.byref(cfg()), one, one, one, 10, None, 2688, one,
                                             1, 2688, one, None) == _lib.TS_EINVAL

@@ -237,7 +237,7 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
   TopkArgs topk = make_topk_args(cfg, bt, pooled ? pooled : votes, w.score_stride, hit, cache, sel,
                                  sel_pos, sel_stride, sel_len, (uint32_t*)(ws + w.topk_ws));
   topk.clear = tickets;
-  topk.clear_per_req = cfg->num_kv_heads;
+  topk.clear_per_req = attn_tickets_per_request(cfg);
   // A batch too large for one launch of the selection: scores and votes still without
   // the [H, n] scores in memory, one launch per request, then the top-k kernels.
   const int vote_group = layer_selection_form(cfg, bt) == 1 ? 1 : 0;
@@ -259,7 +259,7 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
   if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
   if (one_launch) {
     TS_TRY(launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,
-                         nullptr, 0, ws + w.select_ws, tickets, cfg->num_kv_heads,
+                         nullptr, 0, ws + w.select_ws, tickets, attn_tickets_per_request(cfg),
                          (hipStream_t)stream));
   } else if (vote_group > 0) {
     // With max-pooling the kernel writes the pooled votes (there is no un-pooled copy).
@@ -377,7 +377,7 @@ int ts_decode_layer_attend(const ts_config* cfg, const ts_batch* bt, const void*
   TopkArgs topk = make_topk_args(cfg, bt, ranked, ranked_stride, hit, cache, sel, sel_pos, sel_stride,
                                  sel_len, (uint32_t*)(ws + w.topk_ws));
   topk.clear = attn_tickets(cfg, bt->batch, w.max_sel, ws + w.attn_ws);
-  topk.clear_per_req = cfg->num_kv_heads;
+  topk.clear_per_req = attn_tickets_per_request(cfg);
   ts_config plain = *cfg;
   plain.pool_kernel = -1;
   if (max_n > 0 && score_votes_group(&plain, bt->batch, bt->max_seq_len) > 0)

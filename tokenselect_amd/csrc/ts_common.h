@@ -57,6 +57,8 @@ int launch_rope(const void* x, void* out, const float* cos_table, const float* s
 // tickets_clear = false makes the launcher clear them first, true says an earlier
 // kernel of the stream already did (attn_tickets() tells it where they are).
 uint32_t* attn_tickets(const ts_config* cfg, int batch, int max_sel_len, void* workspace);
+// Tickets per request (the words to clear): one per workgroup row of the attention's grid.
+int attn_tickets_per_request(const ts_config* cfg);
 int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const void* v_pool,
                 int64_t pool_rows, const int32_t* sel, int64_t sel_stride, const int32_t* sel_len,
                 int batch, int max_sel_len, void* out, void* workspace, bool tickets_clear,
