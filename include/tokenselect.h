@@ -212,10 +212,10 @@ int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
 /* The whole selection in one launch (tr.py:350-373, 424-449 without the [H, n]
  * score tensor, the [n] vote vector or the sort in between): score, per-head
  * softmax, vote, exact k-th largest vote, ascending positions, index assembly.
- * The scores stay in LDS.  The workgroups of the launch meet three to five times:
- * softmax partials (the merged statistics are polled for, not met for), then
- * histogram rounds over the 11 + 11 +
- * 10 bits of the vote keys until at most 256 candidates are left around the k-th
+ * The scores stay in LDS.  The softmax statistics need no meeting (the
+ * per-workgroup partials and the merged statistics are polled for: the data
+ * is its own flag); the workgroups of the launch then meet two to four times:
+ * histogram rounds over the 11 + 11 + 10 bits of the vote keys until at most 256 candidates are left around the k-th
  * vote, which are listed and ranked by every workgroup in a last round together
  * with the per-workgroup counts that place its selected positions in the output
  * (masses of exact ties take all three histogram rounds and a count round; one

@@ -241,20 +241,20 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
   // A batch too large for one launch of the selection: scores and votes still without
   // the [H, n] scores in memory, one launch per request, then the top-k kernels.
   const int vote_group = layer_selection_form(cfg, bt) == 1 ? 1 : 0;
-  ZeroRegion zero_counters, zero_sync, zero_stats;
+  ZeroSet zero;
   if (one_launch) {
-    select_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_counters, &zero_sync);
+    select_zero_regions(cfg, fused, ws + w.select_ws, bt->batch, &zero);
   } else if (max_n > 0) {
-    zero_counters = topk_zero_region(topk, bt->batch);
-    if (vote_group > 0) score_votes_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_stats, &zero_sync);
+    zero.add(topk_zero_region(topk, bt->batch));
+    if (vote_group > 0) score_votes_zero_regions(cfg, bt, fused, ws + w.select_ws, &zero);
   }
   if (chunk_rows > 0) {
     // Chunk fingerprint: row i rotated to n_local + i, mean over the rows (tr.py:380-392).
-    TS_TRY(launch_fingerprint(cfg, q, chunk_rows, q_cos, q_sin, table_rows, qf, zero_counters,
-                              zero_sync, (hipStream_t)stream, zero_stats));
+    TS_TRY(launch_fingerprint(cfg, q, chunk_rows, q_cos, q_sin, table_rows, qf, zero,
+                              (hipStream_t)stream));
   } else {
     TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
-                       zero_counters, zero_sync, (hipStream_t)stream, zero_stats));
+                       zero, (hipStream_t)stream));
   }
   if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
   if (one_launch) {
@@ -326,10 +326,10 @@ int ts_decode_layer_votes(const ts_config* cfg, const ts_batch* bt, const void* 
   int32_t* hit = cache ? (int32_t*)(ws + w.hit) : nullptr;
   const SelectWorkspace fused = select_workspace(&plain, bt->batch, bt->max_seq_len);
   const int group = max_n > 0 ? score_votes_group(&plain, bt->batch, bt->max_seq_len) : 0;
-  ZeroRegion zero_stats, zero_sync;
-  if (group > 0) score_votes_zero_regions(fused, ws + w.select_ws, bt->batch, &zero_stats, &zero_sync);
+  ZeroSet zero;
+  if (group > 0) score_votes_zero_regions(&plain, bt, fused, ws + w.select_ws, &zero);
   TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
-                     zero_stats, zero_sync, (hipStream_t)stream));
+                     zero, (hipStream_t)stream));
   if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
   if (max_n <= 0) return TS_OK;
   if (group > 0)

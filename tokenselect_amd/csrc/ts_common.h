@@ -33,24 +33,46 @@ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // the statistics merge and the workspace query.
 int score_tokens_per_block(int64_t total_candidates, int num_heads);
 
-// Words the rotation kernel clears on the side (up to three such regions per launch):
-// `count` pieces of `words` 32-bit words, `stride` words apart (all zero: nothing
-// to clear).
+// Words the rotation kernel clears on the side: `count` pieces of `words` 32-bit
+// words, `stride` words apart (all zero: nothing to clear).
 struct ZeroRegion {
   uint32_t* base = nullptr;
   int64_t stride = 0;
   int words = 0;
   int count = 0;
 };
-// Chunk fingerprint (ts_prefill.hip) with the same side job as launch_rope: the two
+// What one such launch clears: up to four regions.
+constexpr int kZeroRegions = 4;
+struct ZeroSet {
+  ZeroRegion r[kZeroRegions];
+  int used = 0;
+  void add(const ZeroRegion& region) {
+    if (region.count > 0 && region.words > 0 && used < kZeroRegions) r[used++] = region;
+  }
+  int64_t total() const {
+    int64_t t = 0;
+    for (int i = 0; i < used; ++i) t += (int64_t)r[i].count * r[i].words;
+    return t;
+  }
+};
+// Thread `gid` of `threads` clears its share of every region.
+__device__ __forceinline__ void clear_regions(const ZeroSet& zero, int64_t gid, int64_t threads) {
+#pragma unroll
+  for (int i = 0; i < kZeroRegions; ++i) {
+    if (i >= zero.used) break;
+    const ZeroRegion& z = zero.r[i];
+    for (int64_t w = gid; w < (int64_t)z.count * z.words; w += threads)
+      z.base[(w / z.words) * z.stride + w % z.words] = 0u;
+  }
+}
+// Chunk fingerprint (ts_prefill.hip) with the same side job as launch_rope: the
 // regions are cleared by the same launch.
 int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
-                       const float* sin_table, int64_t table_rows, void* qf, const ZeroRegion& zero,
-                       const ZeroRegion& zero2, hipStream_t stream, const ZeroRegion& zero3 = ZeroRegion{});
+                       const float* sin_table, int64_t table_rows, void* qf, const ZeroSet& zero,
+                       hipStream_t stream);
 int launch_rope(const void* x, void* out, const float* cos_table, const float* sin_table,
                 const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
-                const ZeroRegion& zero, const ZeroRegion& zero2, hipStream_t stream,
-                const ZeroRegion& zero3 = ZeroRegion{});
+                const ZeroSet& zero, hipStream_t stream);
 
 // Sparse decode attention (ts_attn.hip).  The kernel counts its workgroups in per
 // (request, KV head) tickets inside the workspace, which must be zero at launch:

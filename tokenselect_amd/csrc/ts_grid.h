@@ -128,7 +128,10 @@ __device__ __forceinline__ void grid_arrive(uint32_t* sync, uint32_t round, bool
 }
 
 // One lane waits until the 64-bit word at `p` is no longer zero and returns it; 0 when
-// the wait ran into its bound (the fault word is then set) or another one did.
+// the wait ran into its bound (the fault word is then set) or another one did.  SLEEP
+// spaces the polls (in units of 64 clocks): a wait that begins while other workgroups
+// still stream must not compete with them.
+template <int SLEEP>
 __device__ __forceinline__ uint64_t poll_nonzero(const uint64_t* p, uint32_t* sync, uint64_t ticks) {
   const uint64_t t0 = wall_clock64();
   for (uint32_t polls = 1;; ++polls) {
@@ -141,16 +144,8 @@ __device__ __forceinline__ uint64_t poll_nonzero(const uint64_t* p, uint32_t* sy
         return 0ull;
       }
     }
-    __builtin_amdgcn_s_sleep(1);
+    __builtin_amdgcn_s_sleep(SLEEP);
   }
-}
-
-// The second half of a rendezvous for a workgroup that arrived without waiting and
-// did other work in the meantime.
-__device__ __forceinline__ void grid_wait(uint32_t* sync, uint32_t round, uint64_t ticks,
-                                          uint32_t index) {
-  if (threadIdx.x == 0) grid_poll(sync, round, ticks, index);
-  __syncthreads();
 }
 
 }  // namespace ts

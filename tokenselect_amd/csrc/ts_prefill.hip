@@ -26,7 +26,7 @@ constexpr int kFpSplit = 2;     // workgroups per head
 __global__ __launch_bounds__(1024) void fingerprint_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ qf, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int64_t table_rows, int first_pos, int rows, int heads,
-    ZeroRegion zero, ZeroRegion zero2, ZeroRegion zero3) {
+    ZeroSet zero) {
 #pragma clang fp contract(off)
   constexpr int half = kHeadDim / 2;
   constexpr int kPairs = half / kFpSplit;   // rotation pairs of this workgroup
@@ -39,12 +39,7 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
   {
     const int64_t gid = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 1024 + threadIdx.x;
     const int64_t step = (int64_t)gridDim.x * gridDim.y * 1024;
-    for (int64_t w = gid; w < (int64_t)zero.count * zero.words; w += step)
-      zero.base[(w / zero.words) * zero.stride + w % zero.words] = 0u;
-    for (int64_t w = gid; w < (int64_t)zero2.count * zero2.words; w += step)
-      zero2.base[(w / zero2.words) * zero2.stride + w % zero2.words] = 0u;
-    for (int64_t w = gid; w < (int64_t)zero3.count * zero3.words; w += step)
-      zero3.base[(w / zero3.words) * zero3.stride + w % zero3.words] = 0u;
+    clear_regions(zero, gid, step);
   }
   float lo_sum[kFpVec] = {0.f, 0.f, 0.f, 0.f}, hi_sum[kFpVec] = {0.f, 0.f, 0.f, 0.f};
   // Four rows per step: their loads are independent and go out together; the sums
@@ -749,8 +744,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 }
 
 int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
-                       const float* sin_table, int64_t table_rows, void* qf, const ZeroRegion& zero,
-                       const ZeroRegion& zero2, hipStream_t stream, const ZeroRegion& zero3) {
+                       const float* sin_table, int64_t table_rows, void* qf, const ZeroSet& zero,
+                       hipStream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_REQUIRE(q && cos_table && sin_table && qf, TS_EINVAL, "ts_fingerprint: NULL tensor argument");
   TS_REQUIRE(rows >= 1, TS_EINVAL, "ts_fingerprint: rows %d < 1", rows);
@@ -759,7 +754,7 @@ int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const 
              (long long)table_rows, (long long)cfg->n_local + rows);
   hipLaunchKernelGGL(fingerprint_kernel, dim3((unsigned)cfg->num_heads, kFpSplit), dim3(1024), 0, stream,
                      (const uint16_t*)q, (uint16_t*)qf, cos_table, sin_table, table_rows,
-                     cfg->n_local, rows, cfg->num_heads, zero, zero2, zero3);
+                     cfg->n_local, rows, cfg->num_heads, zero);
   return check_launch("fingerprint_kernel");
 }
 
@@ -773,8 +768,8 @@ extern "C" {
 
 int ts_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
                    const float* sin_table, int64_t table_rows, void* qf, ts_stream_t stream) {
-  return launch_fingerprint(cfg, q, rows, cos_table, sin_table, table_rows, qf, ZeroRegion{},
-                            ZeroRegion{}, (hipStream_t)stream);
+  return launch_fingerprint(cfg, q, rows, cos_table, sin_table, table_rows, qf, ZeroSet{},
+                            (hipStream_t)stream);
 }
 
 size_t ts_prefill_attn_workspace_bytes(const ts_config* cfg, int32_t max_sel_len) {

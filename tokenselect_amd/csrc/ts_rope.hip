@@ -15,23 +15,13 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(const uint16_t* __restr
                                                          const float* __restrict__ sin_table,
                                                          const int64_t* __restrict__ position_ids,
                                                          int64_t table_rows, int64_t rows, int heads,
-                                                         int dim, ZeroRegion zero, ZeroRegion zero2,
-                                                         ZeroRegion zero3) {
+                                                         int dim, ZeroSet zero) {
 #pragma clang fp contract(off)
   const int half = dim >> 1;
   const int64_t pairs = rows * heads * half;
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  // Counters the later kernels of a decode step accumulate into: `count` pieces
-  // of `words` words, `stride` words apart.
-  const int64_t zero_total = (int64_t)zero.count * zero.words;
-  for (int64_t w = gid; w < zero_total; w += (int64_t)gridDim.x * blockDim.x)
-    zero.base[(w / zero.words) * zero.stride + w % zero.words] = 0u;
-  const int64_t zero2_total = (int64_t)zero2.count * zero2.words;
-  for (int64_t w = gid; w < zero2_total; w += (int64_t)gridDim.x * blockDim.x)
-    zero2.base[(w / zero2.words) * zero2.stride + w % zero2.words] = 0u;
-  const int64_t zero3_total = (int64_t)zero3.count * zero3.words;
-  for (int64_t w = gid; w < zero3_total; w += (int64_t)gridDim.x * blockDim.x)
-    zero3.base[(w / zero3.words) * zero3.stride + w % zero3.words] = 0u;
+  // Counters the later kernels of a decode step accumulate into.
+  clear_regions(zero, gid, (int64_t)gridDim.x * blockDim.x);
   if (gid >= pairs) return;
   const int i = (int)(gid % half);
   const int64_t rh = gid / half;
@@ -52,17 +42,15 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(const uint16_t* __restr
 
 int launch_rope(const void* x, void* out, const float* cos_table, const float* sin_table,
                 const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
-                const ZeroRegion& zero, const ZeroRegion& zero2, hipStream_t stream,
-                const ZeroRegion& zero3) {
+                const ZeroSet& zero, hipStream_t stream) {
   const int64_t pairs = rows * heads * (dim / 2);
   // Enough workgroups for the clearing on the side as well: four words per thread.
-  const int64_t to_clear = (int64_t)zero.count * zero.words + (int64_t)zero2.count * zero2.words +
-                           (int64_t)zero3.count * zero3.words;
+  const int64_t to_clear = zero.total();
   const int64_t blocks = std::max(ceil_div(pairs, 256), ceil_div(to_clear, 1024));
   TS_REQUIRE(blocks <= 0x7fffffff, TS_EINVAL, "ts_rope_apply: too many rows");
   hipLaunchKernelGGL(rope_apply_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
                      (const uint16_t*)x, (uint16_t*)out, cos_table, sin_table, position_ids,
-                     table_rows, rows, heads, dim, zero, zero2, zero3);
+                     table_rows, rows, heads, dim, zero);
   return check_launch("rope_apply_kernel");
 }
 
@@ -81,5 +69,5 @@ extern "C" int ts_rope_apply(const void* x, void* out, const float* cos_table,
   TS_REQUIRE(dim >= 2 && dim % 2 == 0, TS_ESHAPE, "ts_rope_apply: dim %d must be even", dim);
   if (rows == 0) return TS_OK;
   return launch_rope(x, out, cos_table, sin_table, position_ids, table_rows, rows, heads, dim,
-                     ZeroRegion{}, ZeroRegion{}, (hipStream_t)stream);
+                     ZeroSet{}, (hipStream_t)stream);
 }

@@ -107,13 +107,14 @@ struct SelectWorkspace {
 SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len,
                                  bool ignore_switch = false);
 
-// Regions the kernel before ts_select on the stream has to clear (counters and
-// rendezvous words), in the form the rotation kernel takes them.
-void select_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* counters,
-                         ZeroRegion* sync);
+// Regions the kernel before ts_select on the stream has to clear (counters, replicas
+// of the merged statistics, rendezvous words, the per-workgroup statistics), in the form
+// the rotation kernel takes them.
+void select_zero_regions(const ts_config* cfg, const SelectWorkspace& w, void* workspace, int batch,
+                         ZeroSet* zero);
 
-// Clears two regions (the stand-alone form of what the rotation kernel does on the side).
-__global__ void select_zero_kernel(ZeroRegion r0, ZeroRegion r1);
+// Clears the regions (the stand-alone form of what the rotation kernel does on the side).
+int launch_select_zero(const ZeroSet& zero, hipStream_t stream);
 
 // Bound of a grid-wide wait of the fused selection: 2 s of the 100 MHz clock.
 constexpr uint64_t kSelectWaitTicks = 200000000ull;
@@ -125,13 +126,14 @@ constexpr uint64_t kSelectWaitTicks = 200000000ull;
 // into hist_ws.  score_votes_group() is the number of requests per launch, 0 when not
 // even one request fits (or the fused kernels are switched off): then the separate
 // kernels serve.  The workspace is that of ts_select for the whole batch; the
-// statistics replicas and the rendezvous areas (score_votes_zero_regions) are zero.
+// statistics (per workgroup and merged) and the rendezvous areas (score_votes_zero_regions)
+// are zero.
 // Whether the batch is served by votes-only launches packed by the host's lengths
 // (ts_batch.host_seq_lens given, every request fits the device).
 bool score_votes_packed(const ts_config* cfg, const ts_batch* bt);
 int score_votes_group(const ts_config* cfg, int batch, int max_seq_len);
-void score_votes_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* stats,
-                              ZeroRegion* sync);
+void score_votes_zero_regions(const ts_config* cfg, const ts_batch* bt, const SelectWorkspace& w,
+                              void* workspace, ZeroSet* zero);
 int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
                        int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
                        uint32_t* hist_ws, size_t hist_ws_stride, void* workspace, hipStream_t stream);

@@ -73,7 +73,7 @@ constexpr int kQuadSwap2 = 0x4E;  // quad_perm [2,3,0,1]
 //     the keys stream in costs a quarter of the read bandwidth (DRAM read/write
 //     turnarounds).
 //   kScoreFused (the whole selection in one launch whose workgroups are all
-//     resident at once and meet three to five times): the scores never leave LDS.
+//     resident at once and meet two to four times): the scores never leave LDS.
 //     Every workgroup publishes its per-head (max, sum exp); the (request, head)
 //     pairs are dealt out over the grid, merged and written to replicas that the
 //     workgroups poll; every workgroup turns its own
@@ -88,12 +88,14 @@ constexpr int kScoreDirect = 0, kScoreTiled = 1, kScoreFused = 2;
 constexpr int kScorePacked = 3;
 constexpr int kMaxHeads = 128;
 
-// After the first rendezvous of the fused kernel: the (request, head) pairs are dealt
-// out over all wavefronts of the grid; a wavefront merges the per-workgroup (max, sum
-// exp) of its pair, a lane per chunk, in a fixed order, and writes the result into 64
-// replicas, lane r into replica r.  The workgroups poll the words of the replica of
-// their index until they are there (a sum of exponentials is never zero): the data is
-// its own flag, which saves a rendezvous.
+// The softmax statistics of the fused kernel, without a rendezvous: every workgroup
+// publishes its per-head (max, sum exp) into a table that was zero at launch; the
+// (request, head) pairs are dealt out over all wavefronts of the team; a wavefront polls
+// the entries of its pair, a lane per chunk, until none is zero any more (a sum of
+// exponentials never is: the data is its own flag), merges them in a fixed order and
+// writes the result into 64 replicas, lane r into replica r.  The workgroups poll the
+// words of the replica of their index in the same way.  The wait is bounded like those
+// of the rendezvous: on giving up it sets the fault word and merges what is there.
 template <bool PACKED>
 __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const GridTeam& team,
                                                     int lane, int wave) {
@@ -110,15 +112,34 @@ __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const Gr
     const int chunks = (geo.n + a.tokens_per_block - 1) / a.tokens_per_block;
     const float2* part = (const float2*)a.partials + ((size_t)b * H + h) * a.nchunks;
     float m = kNegBig, l = 0.f;
+    const uint64_t t0 = wall_clock64();
+    bool lost = false;
     for (int base = 0; base < chunks; base += 8 * 64) {  // 8 loads in flight per lane
       float2 v[8];
+      for (uint32_t polls = 1;; ++polls) {
+        bool there = true;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int c = base + 64 * i + lane;
+          v[i] = c < chunks ? load_coherent(part + c) : make_float2(kNegBig, 1.f);
+          there = there && __float_as_uint(v[i].y) != 0u;
+        }
+        if (__all(there) || lost) break;
+        if ((polls & 7u) == 0) {
+          if (load_coherent(&a.sync[0]) != 0u) {
+            lost = true;
+          } else if (wall_clock64() - t0 > a.spin_ticks) {
+            __hip_atomic_store(&a.sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            lost = true;
+          }
+        }
+        __builtin_amdgcn_s_sleep(8);  // some 0.2 us between the polls of a few dozen wavefronts
+      }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int c = base + 64 * i + lane;
-        v[i] = c < chunks ? load_coherent(part + c) : make_float2(kNegBig, 0.f);
+        if (c < chunks) softmax_merge(m, l, v[i].x, v[i].y);
       }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) softmax_merge(m, l, v[i].x, v[i].y);
     }
     row16_softmax_merge(m, l);
     softmax_merge(m, l, __shfl_xor(m, 16), __shfl_xor(l, 16));
@@ -127,7 +148,8 @@ __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const Gr
   }
 }
 
-constexpr uint32_t kSelectRounds = 5;  // rendezvous of the fused kernel
+constexpr int kStatsPollSleep = 12;     // x 64 clocks between a workgroup's polls for the merged statistics
+constexpr uint32_t kSelectRounds = 4;  // rendezvous of the fused kernel at most (without the max-pool's)
 
 #ifdef TS_TRACE  // development builds: per-workgroup phase timestamps of the fused kernel
 __device__ uint64_t g_trace[4096 * 24];
@@ -344,10 +366,9 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   }
   if (block_lo >= n) {
     if constexpr (FUSED) {  // no tokens here: only help with the statistics
-      grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
       merge_request_stats<PACKED>(a, team, threadIdx.x & 63, threadIdx.x >> 6);
-      const uint32_t rounds = (a.votes_only ? 1u : kSelectRounds) + (a.pool_kernel > 0 ? 1u : 0u);
-      for (uint32_t round = 2; round <= rounds; ++round)
+      const uint32_t rounds = (a.votes_only ? 0u : kSelectRounds) + (a.pool_kernel > 0 ? 1u : 0u);
+      for (uint32_t round = 1; round <= rounds; ++round)
         grid_arrive(a.sync, round, false, a.spin_ticks, team.size, team.index);
     }
     return;
@@ -582,7 +603,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     for (int i = tid; i < kTopkBins; i += 256) lh[i] = 0u;
     if (tid < 16) scratch[tid] = 0u;
     TS_MARK(1);
-    grid_arrive(a.sync, 1, true, a.spin_ticks, team.size, team.index);
+    __syncthreads();  // scores, own maxima and the cleared histogram are in LDS for all
     TS_MARK(2);
     merge_request_stats<PACKED>(a, team, lane, wave);
     TS_MARK(3);
@@ -611,7 +632,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       const int h = head_of<HKV, G>(tid / G, tid % G, a.head_map);
       const uint64_t* rep = (const uint64_t*)(a.stats + (size_t)(team.index % kSyncSlots) * a.stats_stride) +
                             (size_t)b * H + h;
-      const uint64_t st = poll_nonzero(rep, a.sync, a.spin_ticks);
+      const uint64_t st = poll_nonzero<kStatsPollSleep>(rep, a.sync, a.spin_ticks);
       const float mx = __uint_as_float((uint32_t)st), sum = __uint_as_float((uint32_t)(st >> 32));
       s_rz[tid] = st ? __expf(local_max[tid] - mx) / sum : 0.f;  // 0: the wait gave up
     }
@@ -637,7 +658,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       sc[0] = c;
     }
     TS_MARK(5);
-    uint32_t round = 1;  // rendezvous passed so far
+    uint32_t round = 0;  // rendezvous passed so far
     if (a.pool_kernel > 0) {
       // Max-pool smoothing of the votes (tr.py:366-369): stride 1, padding (kernel-1)/2
       // with -inf, an even kernel makes the result one shorter.  The workgroups
@@ -1205,28 +1226,66 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
   return w;
 }
 
-void select_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* counters,
-                         ZeroRegion* sync) {
-  counters->base = (uint32_t*)((char*)workspace + w.counters);
-  counters->words = (int)((w.stats - w.counters) / 4 + (size_t)kSyncSlots * w.stats_stride);
-  counters->stride = counters->words;
-  counters->count = 1;
-  sync->base = (uint32_t*)((char*)workspace + w.sync);
-  sync->stride = kSyncSlotWords;
-  sync->words = kSyncLiveWords;
-  sync->count = kSyncSlots + 1;
+// One launch of the votes-only form: requests [first, first + requests), `workgroups`
+// along x (packed: all of the launch's; else per request), `table_chunks` an upper bound
+// of the chunks of any of its requests.
+struct VoteLaunch {
+  int first, requests, tokens_per_block, workgroups, table_chunks;
+  bool packed;
+};
+bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<VoteLaunch>* plan);
+
+// The per-workgroup statistics are their own flags (a sum of exponentials is never
+// zero): the chunks a launch may fill have to be zero before it, `chunks` of every
+// (request, head) row.
+static ZeroRegion partials_zero_region(const SelectWorkspace& w, void* workspace, int batch, int heads,
+                                       int chunks) {
+  ZeroRegion z;
+  z.base = (uint32_t*)((char*)workspace + w.partials);
+  z.stride = (int64_t)kSelMaxChunks * 2;
+  z.words = std::min(chunks, kSelMaxChunks) * 2;
+  z.count = batch * heads;
+  return z;
+}
+static ZeroRegion stats_zero_region(const SelectWorkspace& w, void* workspace, int batch, int heads) {
+  ZeroRegion z;  // the live words of the 64 replicas
+  z.base = (uint32_t*)((char*)workspace + w.stats);
+  z.stride = w.stats_stride;
+  z.words = batch * heads * 2;
+  z.count = kSyncSlots;
+  return z;
+}
+static ZeroRegion sync_zero_region(const SelectWorkspace& w, void* workspace, int areas) {
+  ZeroRegion z;
+  z.base = (uint32_t*)((char*)workspace + w.sync);
+  z.stride = kSyncSlotWords;
+  z.words = kSyncLiveWords;
+  z.count = (kSyncSlots + 1) * areas;
+  return z;
 }
 
-void score_votes_zero_regions(const SelectWorkspace& w, void* workspace, int batch, ZeroRegion* stats,
-                              ZeroRegion* sync) {
-  stats->base = (uint32_t*)((char*)workspace + w.stats);
-  stats->words = (int)((size_t)kSyncSlots * w.stats_stride);
-  stats->stride = stats->words;
-  stats->count = 1;
-  sync->base = (uint32_t*)((char*)workspace + w.sync);
-  sync->stride = kSyncSlotWords;
-  sync->words = kSyncLiveWords;
-  sync->count = (kSyncSlots + 1) * batch;
+void select_zero_regions(const ts_config* cfg, const SelectWorkspace& w, void* workspace, int batch,
+                         ZeroSet* zero) {
+  ZeroRegion counters;
+  counters.base = (uint32_t*)((char*)workspace + w.counters);
+  counters.words = batch * kSelCounterWords;
+  counters.stride = counters.words;
+  counters.count = 1;
+  zero->add(counters);
+  zero->add(stats_zero_region(w, workspace, batch, cfg->num_heads));
+  zero->add(sync_zero_region(w, workspace, 1));
+  zero->add(partials_zero_region(w, workspace, batch, cfg->num_heads, w.blocks_per_req));
+}
+
+void score_votes_zero_regions(const ts_config* cfg, const ts_batch* bt, const SelectWorkspace& w,
+                              void* workspace, ZeroSet* zero) {
+  std::vector<VoteLaunch> plan;
+  int chunks = 0;
+  if (plan_vote_launches(cfg, bt, &plan))
+    for (const VoteLaunch& v : plan) chunks = std::max(chunks, v.table_chunks);
+  zero->add(stats_zero_region(w, workspace, bt->batch, cfg->num_heads));
+  zero->add(sync_zero_region(w, workspace, bt->batch));
+  zero->add(partials_zero_region(w, workspace, bt->batch, cfg->num_heads, chunks));
 }
 
 int score_votes_group(const ts_config* cfg, int batch, int max_seq_len) {
@@ -1240,12 +1299,13 @@ const uint32_t* score_votes_fault_word(const ts_config* cfg, int batch, int max_
   return (const uint32_t*)((const char*)workspace + select_workspace(cfg, batch, max_seq_len, true).sync);
 }
 
-__global__ __launch_bounds__(256) void select_zero_kernel(ZeroRegion r0, ZeroRegion r1) {
-  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x, step = (int64_t)gridDim.x * 256;
-  for (int64_t w = gid; w < (int64_t)r0.count * r0.words; w += step)
-    r0.base[(w / r0.words) * r0.stride + w % r0.words] = 0u;
-  for (int64_t w = gid; w < (int64_t)r1.count * r1.words; w += step)
-    r1.base[(w / r1.words) * r1.stride + w % r1.words] = 0u;
+__global__ __launch_bounds__(256) void select_zero_kernel(ZeroSet zero) {
+  clear_regions(zero, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
+}
+int launch_select_zero(const ZeroSet& zero, hipStream_t stream) {
+  const int64_t blocks = std::max<int64_t>(1, std::min<int64_t>(1024, ceil_div(zero.total(), 1024)));
+  hipLaunchKernelGGL(select_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, zero);
+  return check_launch("select_zero_kernel");
 }
 
 static ScoreArgs selection_args(const ts_config* cfg, const ts_batch* bt, const void* qf,
@@ -1285,6 +1345,7 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   char* ws = (char*)workspace;
   ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, hit, (float*)(ws + w.partials),
                                w.tokens_per_block);
+  a.nchunks = kSelMaxChunks;  // the row of a (request, head) pair in the statistics' table
   a.sync = (uint32_t*)(ws + w.sync);
   a.stats = (float*)(ws + w.stats);
   a.stats_stride = w.stats_stride;
@@ -1333,11 +1394,7 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
 // workgroups leaving at once would hold no more members, but the workgroups of a grid go
 // to the XCDs (and further down) in turn by their number, and members with gaps between
 // them do not spread evenly: such launches were seen to wait for room that never came.
-struct VoteLaunch {
-  int first, requests, tokens_per_block, workgroups, table_chunks;
-};
-
-bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<VoteLaunch>* plan) {
+static bool plan_packed_launches(const ts_config* cfg, const ts_batch* bt, std::vector<VoteLaunch>* plan) {
   plan->clear();
   if (!bt->host_seq_lens || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256) return false;
   const int capacity = fused_capacity(cfg, /*packed=*/true);
@@ -1367,7 +1424,7 @@ bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<Vo
     }
     if (tpb > tpb_max) return false;
     if (wgs > 0)  // (nothing to launch for requests that are all sink and local window)
-      plan->push_back(VoteLaunch{first, last - first, tpb, (int)wgs, (int)ceil_div(longest, tpb)});
+      plan->push_back(VoteLaunch{first, last - first, tpb, (int)wgs, (int)ceil_div(longest, tpb), true});
     first = last;
   }
   return true;
@@ -1375,72 +1432,43 @@ bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<Vo
 
 bool score_votes_packed(const ts_config* cfg, const ts_batch* bt) {
   std::vector<VoteLaunch> plan;
-  return plan_vote_launches(cfg, bt, &plan);
+  return plan_packed_launches(cfg, bt, &plan);
+}
+
+// The launches of the votes-only form for a batch: packed by the host's lengths where
+// it has them, else groups of as many requests of max_seq_len as fit the device, each
+// launch a grid [chunks of max_seq_len, requests].  False: not even one request fits.
+bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<VoteLaunch>* plan) {
+  if (plan_packed_launches(cfg, bt, plan)) return true;
+  plan->clear();
+  const int group = score_votes_group(cfg, bt->batch, bt->max_seq_len);
+  if (group <= 0) return false;
+  for (int first = 0; first < bt->batch; first += group) {
+    const int requests = std::min(group, bt->batch - first);
+    const SelectWorkspace w = select_workspace(cfg, requests, bt->max_seq_len, true);
+    if (w.tokens_per_block <= 0) return false;
+    if (w.blocks_per_req > 0)
+      plan->push_back(VoteLaunch{first, requests, w.tokens_per_block, w.blocks_per_req, w.blocks_per_req, false});
+  }
+  return true;
 }
 
 int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
                        int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
                        uint32_t* hist_ws, size_t hist_ws_stride, void* workspace, hipStream_t stream) {
   std::vector<VoteLaunch> plan;
-  if (plan_vote_launches(cfg, bt, &plan)) {
-    const SelectWorkspace all = select_workspace(cfg, bt->batch, bt->max_seq_len, true);
-    char* ws = (char*)workspace;
-    const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, true);
-    int launch = 0;
-    for (const VoteLaunch& v : plan) {
-      ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, skip, (float*)(ws + all.partials),
-                                   v.tokens_per_block);
-      a.nchunks = v.table_chunks;
-      a.sync = (uint32_t*)(ws + all.sync) + (size_t)launch++ * kSyncWords;
-      a.fault_word = (uint32_t*)(ws + all.sync);
-      a.stats = (float*)(ws + all.stats);
-      a.stats_stride = all.stats_stride;
-      a.votes = votes;
-      a.vote_stride = vote_stride;
-      a.counters = (uint32_t*)(ws + all.counters);
-      a.spin_ticks = kSelectWaitTicks;
-      a.fault_out = bt->fault;
-      a.pool_kernel = cfg->pool_kernel;
-      a.pool_votes = (float*)(ws + all.pool_votes);
-      a.pool_stride = all.pool_stride;
-      a.batch_offset = v.first;
-      a.votes_only = 1;
-      a.packed = v.requests;
-      a.pack_first[0] = 0;
-      const int fixed = cfg->n_init + cfg->n_local;
-      for (int r = 0; r < v.requests; ++r) {
-        const int cand = std::max(std::min(bt->host_seq_lens[v.first + r], bt->max_seq_len) - fixed, 0);
-        a.pack_first[r + 1] = a.pack_first[r] + (int)ceil_div(cand, v.tokens_per_block);
-      }
-      a.hist_ws = hist_ws;
-      a.hist_ws_stride = hist_ws_stride;
-      const dim3 grid((unsigned)v.workgroups, 1u);
-      void* params[] = {(void*)&a};
-      const hipError_t e = hipLaunchKernel(fn, grid, dim3(256), params,
-                                           fused_lds_bytes(v.tokens_per_block, cfg->num_heads), stream);
-      if (e != hipSuccess) {
-        (void)hipGetLastError();
-        return fail(TS_EHIP, "fused scoring + vote launch: %s", hipGetErrorString(e));
-      }
-    }
-    return TS_OK;
-  }
-  const int group = score_votes_group(cfg, bt->batch, bt->max_seq_len);
-  TS_REQUIRE(group > 0, TS_ESHAPE, "fused scoring + vote: not even one request of %d tokens fits",
-             bt->max_seq_len);
-  // Offsets of the pieces: those of the whole batch's workspace, whatever the groups.
+  TS_REQUIRE(plan_vote_launches(cfg, bt, &plan), TS_ESHAPE,
+             "fused scoring + vote: not even one request of %d tokens fits", bt->max_seq_len);
+  // Offsets of the pieces: those of the whole batch's workspace, whatever the launches.
   const SelectWorkspace all = select_workspace(cfg, bt->batch, bt->max_seq_len, true);
   char* ws = (char*)workspace;
-  const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
   int launch = 0;
-  for (int first = 0; first < bt->batch; first += group, ++launch) {
-    const int requests = std::min(group, bt->batch - first);
-    const SelectWorkspace w = select_workspace(cfg, requests, bt->max_seq_len, true);
-    TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE, "fused scoring + vote: group of %d does not fit",
-               requests);
+  for (const VoteLaunch& v : plan) {
+    const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, v.packed);
     ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, skip, (float*)(ws + all.partials),
-                                 w.tokens_per_block);
-    a.sync = (uint32_t*)(ws + all.sync) + (size_t)launch * kSyncWords;
+                                 v.tokens_per_block);
+    a.nchunks = kSelMaxChunks;
+    a.sync = (uint32_t*)(ws + all.sync) + (size_t)launch++ * kSyncWords;
     a.fault_word = (uint32_t*)(ws + all.sync);
     a.stats = (float*)(ws + all.stats);
     a.stats_stride = all.stats_stride;
@@ -1452,14 +1480,24 @@ int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf,
     a.pool_kernel = cfg->pool_kernel;
     a.pool_votes = (float*)(ws + all.pool_votes);
     a.pool_stride = all.pool_stride;
-    a.batch_offset = first;
+    a.batch_offset = v.first;
     a.votes_only = 1;
     a.hist_ws = hist_ws;
     a.hist_ws_stride = hist_ws_stride;
-    const dim3 grid((unsigned)w.blocks_per_req, (unsigned)requests);
+    dim3 grid((unsigned)v.workgroups, (unsigned)v.requests);
+    if (v.packed) {
+      a.packed = v.requests;
+      a.pack_first[0] = 0;
+      const int fixed = cfg->n_init + cfg->n_local;
+      for (int r = 0; r < v.requests; ++r) {
+        const int cand = std::max(std::min(bt->host_seq_lens[v.first + r], bt->max_seq_len) - fixed, 0);
+        a.pack_first[r + 1] = a.pack_first[r] + (int)ceil_div(cand, v.tokens_per_block);
+      }
+      grid = dim3((unsigned)v.workgroups, 1u);
+    }
     void* params[] = {(void*)&a};
     const hipError_t e = hipLaunchKernel(fn, grid, dim3(256), params,
-                                         fused_lds_bytes(w.tokens_per_block, cfg->num_heads), stream);
+                                         fused_lds_bytes(v.tokens_per_block, cfg->num_heads), stream);
     if (e != hipSuccess) {
       (void)hipGetLastError();
       return fail(TS_EHIP, "fused scoring + vote launch: %s", hipGetErrorString(e));
@@ -1538,11 +1576,9 @@ int ts_score_vote(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   TS_REQUIRE(vote_stride >= max_n, TS_EWORKSPACE, "vote_stride %lld < max candidates %d",
              (long long)vote_stride, max_n);
   if (max_n <= 0) return TS_OK;
-  ZeroRegion stats, sync;
-  score_votes_zero_regions(w, workspace, bt->batch, &stats, &sync);
-  hipLaunchKernelGGL(select_zero_kernel, dim3((unsigned)(8 * bt->batch)), dim3(256), 0,
-                     (hipStream_t)stream, stats, sync);
-  TS_TRY(check_launch("select_zero_kernel"));
+  ZeroSet zero;
+  score_votes_zero_regions(cfg, bt, w, workspace, &zero);
+  TS_TRY(launch_select_zero(zero, (hipStream_t)stream));
   return launch_score_votes(cfg, bt, qf, k_pool, pool_rows, skip, votes, vote_stride, nullptr, 0,
                             workspace, (hipStream_t)stream);
 }
@@ -1578,11 +1614,9 @@ int ts_select_clear(const ts_config* cfg, const ts_batch* bt, void* workspace,
                     size_t workspace_bytes, ts_stream_t stream) {
   SelectWorkspace w;
   TS_TRY(check_select(cfg, bt, workspace, workspace_bytes, &w));
-  ZeroRegion counters, sync;
-  select_zero_regions(w, workspace, bt->batch, &counters, &sync);
-  hipLaunchKernelGGL(select_zero_kernel, dim3((unsigned)(8 * bt->batch)), dim3(256), 0,
-                     (hipStream_t)stream, counters, sync);
-  return check_launch("select_zero_kernel");
+  ZeroSet zero;
+  select_zero_regions(cfg, w, workspace, bt->batch, &zero);
+  return launch_select_zero(zero, (hipStream_t)stream);
 }
 
 int ts_select_cleared_bounded(const ts_config* cfg, const ts_batch* bt, const void* qf,
