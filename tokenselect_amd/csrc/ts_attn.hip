@@ -52,6 +52,9 @@ __device__ __forceinline__ float2 load_coherent2(const float* p) {
       __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return make_float2(__uint_as_float((uint32_t)v), __uint_as_float((uint32_t)(v >> 32)));
 }
+// (Plain stores, waited for before the ticket is drawn: exchanges whose old value is
+// awaited, the faster way to publish a few words elsewhere, are slower for a
+// workgroup's 2 KB of partials.)
 __device__ __forceinline__ void store_coherent2(float* p, float x, float y) {
   const uint64_t v = (uint64_t)__float_as_uint(x) | ((uint64_t)__float_as_uint(y) << 32);
   __hip_atomic_store((uint64_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -327,31 +330,48 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   __syncthreads();
   if (!s_last) return;
 
-  // out[b,h,:] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s, rounded to
-  // bf16; splits in index order, 32 of them in flight.
+  // out[b,h,:] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s, rounded to bf16.
+  // A wavefront per head slot (a thread owns two adjacent dims, and a head has 64 such
+  // pairs): lane s fetches the (max, sum) of split s, the wave takes the maximum and
+  // lane s the weight of its split, so that the accumulators, all requested at once, are
+  // added up with weights that are ready (read lane by lane): no chain of dependent
+  // exponentials, and one statistics load per wave instead of one per split and thread.
+  static_assert(kHeadDim / 2 == 64, "one wavefront per head slot");
   for (int idx = tid; idx < G * (kHeadDim / 2); idx += 256) {
     const int g = idx / (kHeadDim / 2), d = (idx % (kHeadDim / 2)) * 2;
-    if (!slot_active(g)) continue;
+    if (!slot_active(g)) continue;  // (uniform over the wave)
     const size_t ph = ((size_t)b * H + head_of_slot(g)) * a.nsplit;
     float mm = kNegBig, ll = 0.f, o0 = 0.f, o1 = 0.f;
     for (int s0 = 0; s0 < a.nsplit; s0 += 32) {
-      float2 ml[32], ac[32];
+      // 32 splits at a time, branch-free: loads past the last split repeat it and get
+      // the weight zero.
+      float2 ac[32];
+#pragma unroll
+      for (int i = 0; i < 32; ++i)
+        ac[i] = load_coherent2(a.part_acc + (ph + min(s0 + i, a.nsplit - 1)) * kHeadDim + d);
+      const float2 ml = (lane < 32 && s0 + lane < a.nsplit)
+                            ? load_coherent2(a.part_ml + (ph + s0 + lane) * 2)
+                            : make_float2(kNegBig, 0.f);
+      float mx = ml.x;
+      mx = fmaxf(mx, dpp_move<kRowRor8>(mx));
+      mx = fmaxf(mx, dpp_move<kRowRor4>(mx));
+      mx = fmaxf(mx, dpp_move<kRowRor2>(mx));
+      mx = fmaxf(mx, dpp_move<kRowRor1>(mx));
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      const float mn = fmaxf(mm, __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(mx))));
+      const float keep = __expf(mm - mn);  // what earlier batches hold
+      const float w = (lane < 32 && s0 + lane < a.nsplit) ? __expf(ml.x - mn) : 0.f;
+      const float wl = ml.y * w;
+      o0 *= keep;
+      o1 *= keep;
+      ll *= keep;
+      mm = mn;
 #pragma unroll
       for (int i = 0; i < 32; ++i) {
-        const int sp = min(s0 + i, a.nsplit - 1);
-        ml[i] = load_coherent2(a.part_ml + (ph + sp) * 2);
-        ac[i] = load_coherent2(a.part_acc + (ph + sp) * kHeadDim + d);
-      }
-#pragma unroll
-      for (int i = 0; i < 32; ++i) {
-        if (s0 + i < a.nsplit) {
-          const float mn = fmaxf(mm, ml[i].x);
-          const float a1 = __expf(mm - mn), a2 = __expf(ml[i].x - mn);
-          ll = ll * a1 + ml[i].y * a2;
-          o0 = o0 * a1 + ac[i].x * a2;
-          o1 = o1 * a1 + ac[i].y * a2;
-          mm = mn;
-        }
+        const float wi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), i));
+        ll += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wl), i));
+        o0 += ac[i].x * wi;
+        o1 += ac[i].y * wi;
       }
     }
     const uint32_t packed = (uint32_t)f32_to_bf16(ll > 0.f ? o0 / ll : 0.f) |
