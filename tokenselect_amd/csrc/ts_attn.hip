@@ -168,7 +168,24 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
     for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
   }
 
-  for (int j0 = lo + lg; j0 < hi + (lg & 3); j0 += 16 * kAttnInFlight) {
+  // Two workgroups share a CU and the older one is served first: left alone it finishes
+  // well ahead and the other one then runs by itself, its memory waits uncovered.  A
+  // wavefront therefore lowers its priority as it advances through its range, so that
+  // whichever workgroup is behind is the one served first.
+  const int passes = (chunk + 16 * kAttnInFlight - 1) / (16 * kAttnInFlight);
+  int pass = 0;
+  for (int j0 = lo + lg; j0 < hi + (lg & 3); j0 += 16 * kAttnInFlight, ++pass) {
+    if (passes > 1) {
+      const int level = __builtin_amdgcn_readfirstlane(3 - (4 * pass) / passes);
+      if (level >= 3)
+        __builtin_amdgcn_s_setprio(3);
+      else if (level == 2)
+        __builtin_amdgcn_s_setprio(2);
+      else if (level == 1)
+        __builtin_amdgcn_s_setprio(1);
+      else
+        __builtin_amdgcn_s_setprio(0);
+    }
     // The first token of the wavefront's four lane groups in this pass: a token
     // step whose first token lies past the range is skipped by the whole wavefront.
     const int wave_j0 = __builtin_amdgcn_readfirstlane(j0 - (lg & 3));
@@ -269,6 +286,7 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
     }
   }
 
+  __builtin_amdgcn_s_setprio(0);
   // Merge the four lane groups of a wave (rows of 16 lanes), then the four waves.
   __shared__ float sm_acc[4][G][kHeadDim];
   __shared__ float sm_m[4][G], sm_l[4][G];
