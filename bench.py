@@ -185,7 +185,7 @@ def bench_layer(args, ops, workloads, dev, which=None):
     wl = make(dev)
     # A ragged batch: the lengths are handed over on the host as well (a serving framework
     # holds them there), so that the launches are packed by what the requests hold.
-    wl.host_lengths = (which or args.workload) == "c3" and not args.device_lengths_only
+    wl.host_lengths = (which or args.workload) in ("c3", "c5") and not args.device_lengths_only
     c, bt, B = wl.cfg, wl.batch, len(wl.seq_lens)
     layer = ops.DecodeLayer(c, B, bt.max_seq_len, dev)
     n_pools = max(1, args.pools)

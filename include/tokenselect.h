@@ -177,12 +177,15 @@ int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
 
 /* ts_score + ts_vote without the [H, n] scores in memory (tr.py:350-361): the
  * requests are served in groups whose fp32 scores fit the LDS of the device, one
- * launch per group in which the workgroups meet once to merge the softmax
- * statistics (twice with cfg->pool_kernel > 0) and then write the votes; a batch of
+ * launch per group in which the workgroups poll for each other's softmax
+ * statistics (and meet once with cfg->pool_kernel > 0) and then write the votes; a batch of
  * any size is served as long as one request fits (some 260K candidates for 32
  * heads) and pool_kernel is at most 256 (ts_score_vote_supported).  The groups are
  * sized by max_seq_len, or, with ts_batch.host_seq_lens, packed by what the requests
- * hold (up to 8 consecutive requests per launch).  votes
+ * hold: phases of up to 8 consecutive requests that fit half the device (all of it
+ * for a request that needs more), the workgroups of up to 24 phases in one launch,
+ * which the device works through in order, so that one phase streams keys while
+ * another waits for its statistics.  votes
  * [B, vote_stride] fp32 receives what ts_vote's votes (pooled with pool_kernel > 0)
  * would hold, up to the last bit of an fp32 sum taken in another order.  workspace:
  * ts_select_workspace_bytes().  The launches are ordinary ones whose workgroups must
@@ -411,7 +414,8 @@ int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, in
  * kernel; a batch of contexts so long that each request needs the device to itself
  * is scored and voted on request by request as by ts_score_vote and then ranked by
  * the kernels of ts_topk_ragged (so is a ragged batch whose lengths the host passes
- * in ts_batch.host_seq_lens, several requests per launch); otherwise ts_score, ts_vote and ts_topk_ragged run
+ * in ts_batch.host_seq_lens, the whole batch in one launch as a rule); otherwise ts_score, ts_vote and
+ * ts_topk_ragged run
  * as they do on their own.  All forms give the same selection.
  * ts_set_fused_select(0) forces the separate kernels for the calling process
  * (1 restores the default); it returns the previous setting and has no
@@ -421,7 +425,7 @@ int ts_set_fused_select(int enable);
  * launches (one request each) + top-k kernels, 0 = ts_score + ts_vote + top-k
  * kernels; -1 for an unsupported configuration.  The second form answers for a batch
  * descriptor: with host_seq_lens, a ragged batch too large for one ts_select launch
- * takes form 1 with several requests per launch, packed by those lengths. */
+ * takes form 1 with its requests packed into one launch by those lengths. */
 int ts_decode_layer_selection(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
 int ts_decode_layer_selection_of(const ts_config* cfg, const ts_batch* bt);
 size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);

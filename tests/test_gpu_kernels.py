@@ -3,6 +3,8 @@ the C ABI.  Tolerances: fp32 scores 1e-3 relative (to the score RMS); selected
 positions identical up to ties at the k-th vote; bf16 attention output 2e-2
 absolute."""
 
+import random
+
 import pytest
 import torch
 
@@ -705,6 +707,46 @@ def test_score_vote_in_groups_of_requests(dev, pool_kernel):
             got = v[b, :n].cpu()
             assert (got - ref).abs().max().item() <= 2e-4 * ref.abs().max().item(), f"{name} b={b}"
             assert (got - votes_sep[b, :n].cpu()).abs().max().item() <= 1e-5 * ref.abs().max().item()
+
+
+@pytest.mark.parametrize("case", ["many small requests", "a dozen long requests"])
+@pytest.mark.parametrize("pool_kernel", [-1, 5])
+def test_score_vote_phases_of_one_launch(dev, case, pool_kernel):
+    """With the lengths on the host the votes-only form packs the requests into phases and
+    puts the workgroups of many phases into one grid, which the device works through in
+    order: 200 small requests make more phases than one launch holds (eight requests to a
+    phase), a dozen long ones make phases of a few requests that take turns on the device.
+    Against ts_score + ts_vote on the same inputs; the host's lengths are upper bounds, two
+    requests are dense, some are skipped."""
+    rnd = random.Random(5)
+    if case == "many small requests":
+        lens = [rnd.randrange(700, 3000) for _ in range(200)]
+        lens[17], lens[150] = 40, 80
+    else:
+        lens = [rnd.randrange(20000, 60000) for _ in range(12)]
+        lens[5] = 300
+    B = len(lens)
+    say(f"score_vote in phases: {case}, pool={pool_kernel}")
+    wl = small(dev, SHAPES[0], seed=47, lens=lens, ks=[64] * B, page=16, top_k=64, pool_kernel=pool_kernel)
+    c = wl.cfg
+    qf = fingerprint(wl, dev)
+    skip = torch.tensor([1 if b % 11 == 3 else 0 for b in range(B)], dtype=torch.int32, device=dev)
+    votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool, skip=skip), skip=skip)
+    bounds = torch.tensor([min(L + rnd.randrange(0, 700), max(lens)) for L in lens], dtype=torch.int32)
+    packed = ops.Batch(wl.batch.seq_lens, wl.batch.table, max(lens), wl.batch.k_per_req,
+                       host_seq_lens=bounds)
+    for attempt in range(2):  # (the second call finds the workspace as the first one left it)
+        votes = ops.score_vote(c, packed, qf, wl.k_pool, skip=skip)
+        torch.cuda.synchronize()
+        for b, L in enumerate(lens):
+            n = L - c.n_init - c.n_local
+            if pool_kernel > 0 and pool_kernel % 2 == 0:
+                n -= 1
+            if L <= c.n_init + 64 + c.n_local or skip[b]:   # dense: no votes are taken
+                continue
+            want = votes_sep[b, :n]
+            assert (votes[b, :n] - want).abs().max().item() <= 1e-5 * want.abs().max().item(), \
+                f"b={b} L={L} attempt={attempt}"
 
 
 @pytest.mark.parametrize("pool_kernel", [-1, 5])

@@ -7,7 +7,16 @@
 
 namespace ts {
 
-constexpr int kMaxPacked = 8;   // requests per packed launch of the votes-only form
+constexpr int kMaxPacked = 8;   // requests per phase of a packed launch of the votes-only form
+constexpr int kMaxPhases = 24;  // phases per packed launch
+
+// One phase of a packed launch: `requests` requests from `first` on share the workgroups
+// [first_workgroup, next phase's first_workgroup) of the grid, request r owning those from
+// pack_first[r] on (relative to the phase).
+struct VotePhase {
+  int tokens_per_block, first, requests, first_workgroup;
+  int pack_first[kMaxPacked + 1];
+};
 
 struct ScoreArgs {
   const uint16_t* qf;      // [B,H,128] bf16 rotated fingerprints
@@ -51,12 +60,14 @@ struct ScoreArgs {
   // the votes in memory and their first-level histogram added to the top-k workspace.
   int batch_offset;
   int votes_only;
-  // Votes-only launches packed by the host's lengths: `packed` requests (0: the grid is
-  // [chunks, requests]) share a one-dimensional grid, request r of the launch owning the
-  // workgroups [pack_first[r], pack_first[r + 1]); a workgroup without candidates (the
-  // host's length was an upper bound) leaves at once and is not on the rendezvous team.
-  int packed;
-  int pack_first[kMaxPacked + 1];
+  // Votes-only launches packed by the host's lengths (a kernel instantiation of their
+  // own): a one-dimensional grid that holds the workgroups of `nphases` phases one after
+  // the other, each phase a group of requests that fits half the device (or all of it).
+  // A workgroup serves one phase; one without candidates (the host's length was an upper
+  // bound) leaves at once and is not on the phase's team.  Phase p's rendezvous area is
+  // sync + p * kSyncWords.
+  int nphases;
+  VotePhase phases[kMaxPhases];
   uint32_t* hist_ws;      // per-request top-k workspace (ts_topk.h) whose hist0 is counted into, or NULL
   size_t hist_ws_stride;
   uint32_t* fault_word;   // votes-only: the word the kernels after this one consult

@@ -96,20 +96,31 @@ constexpr int kMaxHeads = 128;
 // writes the result into 64 replicas, lane r into replica r.  The workgroups poll the
 // words of the replica of their index in the same way.  The wait is bounded like those
 // of the rendezvous: on giving up it sets the fault word and merges what is there.
+// What a workgroup of the fused kernel serves: the whole launch, or one phase of a
+// packed launch.
+struct LaunchPart {
+  int tokens_per_block;
+  int batch_offset;       // first request
+  int packed;             // requests of the phase (0: the grid is [chunks, requests])
+  const int* pack_first;  // first workgroup of each of them
+  int x;                  // this workgroup along x
+  uint32_t* sync;         // rendezvous area
+};
+
 template <bool PACKED>
-__device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const GridTeam& team,
-                                                    int lane, int wave) {
+__device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const LaunchPart& lp,
+                                                    const GridTeam& team, int lane, int wave) {
   const int H = a.num_heads;
-  const int items = (PACKED ? a.packed : (int)gridDim.y) * H;
+  const int items = (PACKED ? lp.packed : (int)gridDim.y) * H;
   const int first = (int)team.index * 4 + wave;
   const int step = (int)team.size * 4;
   for (int item = first; item < items; item += step) {
-    const int b = a.batch_offset + item / H, h = item % H;
+    const int b = lp.batch_offset + item / H, h = item % H;
     if (a.skip && a.skip[b]) continue;
     const ReqGeom geo =
         request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
     if (geo.n <= 0) continue;
-    const int chunks = (geo.n + a.tokens_per_block - 1) / a.tokens_per_block;
+    const int chunks = (geo.n + lp.tokens_per_block - 1) / lp.tokens_per_block;
     const float2* part = (const float2*)a.partials + ((size_t)b * H + h) * a.nchunks;
     float m = kNegBig, l = 0.f;
     const uint64_t t0 = wall_clock64();
@@ -126,10 +137,10 @@ __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const Gr
         }
         if (__all(there) || lost) break;
         if ((polls & 7u) == 0) {
-          if (load_coherent(&a.sync[0]) != 0u) {
+          if (load_coherent(&lp.sync[0]) != 0u) {
             lost = true;
           } else if (wall_clock64() - t0 > a.spin_ticks) {
-            __hip_atomic_store(&a.sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&lp.sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             lost = true;
           }
         }
@@ -172,18 +183,20 @@ extern "C" int ts_debug_trace(void* out, size_t bytes) {
 // hits the cache costs a few microseconds instead of empty rounds.
 // (req, chunk: this workgroup's request within the launch and its chunk of that request.)
 template <bool PACKED>
-__device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t* lds, int req, int chunk) {
+__device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, const LaunchPart& lp,
+                                                   uint32_t* lds, int req, int chunk) {
   GridTeam team;
   if (PACKED) {
     // A packed launch holds a handful of requests and its members are the workgroups
     // that hold candidates: every thread adds them up for itself.
     uint32_t before = 0, total = 0;
-    for (int r = 0; r < a.packed; ++r) {
-      const int b = a.batch_offset + r;
+    for (int r = 0; r < lp.packed; ++r) {
+      const int b = lp.batch_offset + r;
       if (a.skip && a.skip[b]) continue;
       const int n = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
                                      a.max_seq_len).n;
-      const uint32_t members = n > 0 ? (uint32_t)((n + a.tokens_per_block - 1) / a.tokens_per_block) : 0u;
+      const uint32_t members =
+          n > 0 ? (uint32_t)((n + lp.tokens_per_block - 1) / lp.tokens_per_block) : 0u;
       total += members;
       if (r < req) before += members;
     }
@@ -195,7 +208,7 @@ __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, uint32_t*
   const int B = gridDim.y, mine = req;
   uint32_t before = 0, total = 0;  // selecting requests below this one / in all
   for (int base = 0; base < B; base += 256) {
-    const int b = a.batch_offset + base + tid;  // requests of this launch
+    const int b = lp.batch_offset + base + tid;  // requests of this launch
     bool selects = false;
     if (base + tid < B && !(a.skip && a.skip[b]))
       selects = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
@@ -337,13 +350,20 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   constexpr uint32_t ROW_BYTES = HKV * kHeadDim * 2;
 
   // This workgroup's request within the launch, and its chunk of that request.
+  LaunchPart lp{a.tokens_per_block, a.batch_offset, 0, nullptr, (int)blockIdx.x, a.sync};
   int req = blockIdx.y, chunk = blockIdx.x;
   if (PACKED) {
+    // This workgroup's phase, and its request and chunk within the phase.
+    int phase = 0;
+    while (phase + 1 < a.nphases && (int)blockIdx.x >= a.phases[phase + 1].first_workgroup) ++phase;
+    const VotePhase& ph = a.phases[phase];
+    lp = LaunchPart{ph.tokens_per_block, ph.first, ph.requests, ph.pack_first,
+                      (int)blockIdx.x - ph.first_workgroup, a.sync + (size_t)phase * kSyncWords};
     req = 0;
-    while (req + 1 < a.packed && (int)blockIdx.x >= a.pack_first[req + 1]) ++req;
-    chunk = (int)blockIdx.x - a.pack_first[req];
+    while (req + 1 < lp.packed && lp.x >= lp.pack_first[req + 1]) ++req;
+    chunk = lp.x - lp.pack_first[req];
   }
-  const int b = req + a.batch_offset;
+  const int b = req + lp.batch_offset;
   int n, first_pos;
   if (a.direct_n >= 0) {
     n = (int)a.direct_n;
@@ -354,7 +374,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     n = (a.skip && a.skip[b]) ? 0 : geo.n;
     first_pos = a.n_init;
   }
-  const int block_lo = chunk * a.tokens_per_block;
+  const int block_lo = chunk * lp.tokens_per_block;
   GridTeam team{0u, 0u};
   if constexpr (FUSED) {
     __shared__ uint32_t team_lds[8];
@@ -362,14 +382,14 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     if (!a.votes_only) fixed_segments(a, b);
     if (n <= 0) return;  // dense or served by the cache: nothing to select, not on the team
     if (PACKED && block_lo >= n) return;  // no candidates here, and the team is made without it
-    team = selecting_team<PACKED>(a, team_lds, req, chunk);
+    team = selecting_team<PACKED>(a, lp, team_lds, req, chunk);
   }
   if (block_lo >= n) {
     if constexpr (FUSED) {  // no tokens here: only help with the statistics
-      merge_request_stats<PACKED>(a, team, threadIdx.x & 63, threadIdx.x >> 6);
+      merge_request_stats<PACKED>(a, lp, team, threadIdx.x & 63, threadIdx.x >> 6);
       const uint32_t rounds = (a.votes_only ? 0u : kSelectRounds) + (a.pool_kernel > 0 ? 1u : 0u);
       for (uint32_t round = 1; round <= rounds; ++round)
-        grid_arrive(a.sync, round, false, a.spin_ticks, team.size, team.index);
+        grid_arrive(lp.sync, round, false, a.spin_ticks, team.size, team.index);
     }
     return;
   }
@@ -408,7 +428,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       run_l[kvh][na] = 0.f;
     }
 
-  const int per_wave = a.tokens_per_block >> 2;
+  const int per_wave = lp.tokens_per_block >> 2;
   const int wave_lo = block_lo + wave * per_wave;
   const int wave_hi = min(wave_lo + per_wave, n);
 
@@ -552,7 +572,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
 
   if (MODE == kScoreTiled) {  // one contiguous burst per workgroup
     __syncthreads();
-    const int tiles = (min(a.tokens_per_block, n - block_lo) + 15) >> 4;
+    const int tiles = (min(lp.tokens_per_block, n - block_lo) + 15) >> 4;
     float4* dst = (float4*)((float*)a.scores + ((size_t)b * a.score_stride + block_lo) * H);
     const float4* src = (const float4*)stage;
     for (int i = threadIdx.x; i < tiles * H * 4; i += 256) dst[i] = src[i];
@@ -605,14 +625,14 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     TS_MARK(1);
     __syncthreads();  // scores, own maxima and the cleared histogram are in LDS for all
     TS_MARK(2);
-    merge_request_stats<PACKED>(a, team, lane, wave);
+    merge_request_stats<PACKED>(a, lp, team, lane, wave);
     TS_MARK(3);
     // While the merged statistics are on their way: the exponentials, relative to this
     // workgroup's own maxima; exp(s - max) / sum = exp(s - own max) * exp(own max - max) / sum.
     const ReqGeom geo =
         request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
     const uint32_t k = (uint32_t)geo.k;
-    const int count = min(a.tokens_per_block, n - block_lo);
+    const int count = min(lp.tokens_per_block, n - block_lo);
     uint32_t* ctr = a.counters + (size_t)b * kSelCounterWords;
     auto column = [&](int i) -> float* { return stage + (i >> 4) * tile_stride + (i & 15); };
     auto key_of = [&](int i) -> uint32_t { return vote_key(*column(i)); };
@@ -632,7 +652,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       const int h = head_of<HKV, G>(tid / G, tid % G, a.head_map);
       const uint64_t* rep = (const uint64_t*)(a.stats + (size_t)(team.index % kSyncSlots) * a.stats_stride) +
                             (size_t)b * H + h;
-      const uint64_t st = poll_nonzero<kStatsPollSleep>(rep, a.sync, a.spin_ticks);
+      const uint64_t st = poll_nonzero<kStatsPollSleep>(rep, lp.sync, a.spin_ticks);
       const float mx = __uint_as_float((uint32_t)st), sum = __uint_as_float((uint32_t)(st >> 32));
       s_rz[tid] = st ? __expf(local_max[tid] - mx) / sum : 0.f;  // 0: the wait gave up
     }
@@ -675,7 +695,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
                            __HIP_MEMORY_SCOPE_AGENT);
         window[pad + i] = c;
       }
-      grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
       for (int hx = tid; hx < halo; hx += 256) {
         const int t = hx < pad ? block_lo - pad + hx : block_lo + count + (hx - pad);
         const int at = hx < pad ? hx : count + hx;
@@ -706,7 +726,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         for (int i = tid; i < kTopkBins; i += 256)
           if (lh[i]) atomicAdd(&hist0[i], lh[i]);
       }
-      if (chunk == 0 && tid == 0 && load_coherent(&a.sync[0]) != 0u) {
+      if (chunk == 0 && tid == 0 && load_coherent(&lp.sync[0]) != 0u) {
         __hip_atomic_store(a.fault_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (a.fault_out)
           __hip_atomic_store(a.fault_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -749,7 +769,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       await(done);
     }
     TS_MARK(7);
-    grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+    grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
     TS_MARK(8);
     uint32_t t0 = 0, above0 = 0, in_bin0 = 0;
     // The search starts at the highest occupied bin of the request.  Together with the
@@ -815,7 +835,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
                                    base + tid < count && key_bin0(key) == t0, key_bin1(key), lane);
       }
       await(done);
-      grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
       {
         uint32_t h[kTopkBins / 256];
 #pragma unroll
@@ -878,7 +898,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       __syncthreads();
       if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], 0u);
       TS_MARK(10);
-      grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
       TS_MARK(11);
 
       // Every workgroup ranks the list on its own, one entry per thread, in the order
@@ -970,7 +990,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         }
         await(done);
       }
-      grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
       {
         uint32_t h[4];
 #pragma unroll
@@ -1005,14 +1025,14 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       }
       __syncthreads();
       if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], scratch[9]);
-      grid_arrive(a.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
     }
     // The requests of a batch may need different numbers of rounds, and the rendezvous
     // spans them all: whoever is through counts itself in for the rounds it skipped.
     if (team.size != gridDim.x) {
       const uint32_t rounds = kSelectRounds + (a.pool_kernel > 0 ? 1u : 0u);
       while (round < rounds)
-        grid_arrive(a.sync, ++round, false, a.spin_ticks, team.size, team.index);
+        grid_arrive(lp.sync, ++round, false, a.spin_ticks, team.size, team.index);
     }
     if (!listed) {
       // Counts of the workgroups before this one.
@@ -1088,7 +1108,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     // A grid-wide wait of this launch gave up (the workgroups were not all resident
     // within the bound): what was selected is not valid.  The first workgroup of every
     // selecting request says so in place of the length, and in the caller's word.
-    if (blockIdx.x == 0 && tid == 0 && load_coherent(&a.sync[0]) != 0u) {
+    if (blockIdx.x == 0 && tid == 0 && load_coherent(&lp.sync[0]) != 0u) {
       a.sel_len[b] = -1;
       if (a.fault_out)
         __hip_atomic_store(a.fault_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -1226,14 +1246,20 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
   return w;
 }
 
-// One launch of the votes-only form: requests [first, first + requests), `workgroups`
-// along x (packed: all of the launch's; else per request), `table_chunks` an upper bound
-// of the chunks of any of its requests.
+// One part of the votes-only form (a launch, or a phase of a packed launch): requests
+// [first, first + requests), `workgroups` along x (packed: all of the part's; else per
+// request), `table_chunks` an upper bound of the chunks of any of its requests.
 struct VoteLaunch {
   int first, requests, tokens_per_block, workgroups, table_chunks;
-  bool packed;
 };
-bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<VoteLaunch>* plan);
+// The parts of a batch.  packed: phases, up to phases_per_launch of them to a launch;
+// else one launch each.
+struct VotePlan {
+  std::vector<VoteLaunch> parts;
+  bool packed = false;
+  int phases_per_launch = 1;
+};
+bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan);
 
 // The per-workgroup statistics are their own flags (a sum of exponentials is never
 // zero): the chunks a launch may fill have to be zero before it, `chunks` of every
@@ -1279,10 +1305,10 @@ void select_zero_regions(const ts_config* cfg, const SelectWorkspace& w, void* w
 
 void score_votes_zero_regions(const ts_config* cfg, const ts_batch* bt, const SelectWorkspace& w,
                               void* workspace, ZeroSet* zero) {
-  std::vector<VoteLaunch> plan;
+  VotePlan plan;
   int chunks = 0;
   if (plan_vote_launches(cfg, bt, &plan))
-    for (const VoteLaunch& v : plan) chunks = std::max(chunks, v.table_chunks);
+    for (const VoteLaunch& v : plan.parts) chunks = std::max(chunks, v.table_chunks);
   zero->add(stats_zero_region(w, workspace, bt->batch, cfg->num_heads));
   zero->add(sync_zero_region(w, workspace, bt->batch));
   zero->add(partials_zero_region(w, workspace, bt->batch, cfg->num_heads, chunks));
@@ -1384,18 +1410,27 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   return TS_OK;
 }
 
-// Launches of the votes-only form when the host knows upper bounds of the lengths
-// (ts_batch.host_seq_lens): consecutive requests are packed into a launch by what they
-// hold, not by max_seq_len -- as many as fit the device with the most tokens per
-// workgroup that the LDS takes, then the fewest tokens per workgroup with which they
-// still fit.  The grid of such a launch is one-dimensional and has no more workgroups
-// than the device keeps resident, every one of them with candidates by the host's
-// count: a grid [chunks of the longest, requests] with the short requests' surplus
-// workgroups leaving at once would hold no more members, but the workgroups of a grid go
-// to the XCDs (and further down) in turn by their number, and members with gaps between
-// them do not spread evenly: such launches were seen to wait for room that never came.
-static bool plan_packed_launches(const ts_config* cfg, const ts_batch* bt, std::vector<VoteLaunch>* plan) {
-  plan->clear();
+// The votes-only form when the host knows upper bounds of the lengths
+// (ts_batch.host_seq_lens): consecutive requests are packed into phases by what they
+// hold, not by max_seq_len -- as many as fit half the device (all of it, when a request
+// needs more) with the most tokens per workgroup that the LDS takes.  One launch holds the workgroups of
+// many phases, one after the other in a one-dimensional grid.  The device starts the
+// workgroups of a grid in the order of their numbers as room becomes free (of those that
+// go to one XCD, every eighth): with phases of half the device two of them are resident
+// side by side, and when the workgroups of the earlier one leave, those of the next but
+// one take their places.  A phase ends with the memory idle (the statistics on their
+// way, scores turned into votes); the other phase streams meanwhile.  Two phases that
+// start together would also wait together, so the second phase is given about half the
+// candidates of a full one.  Nothing can wait forever: the workgroups of the earliest
+// unfinished phase wait for each other only, and all of them have been started, since
+// every workgroup started before them has left and fewer than fit are left to start.
+// (A grid [chunks of the longest, requests] whose surplus workgroups leave at once is
+// not an alternative: its members have gaps between them and do not spread evenly over
+// the XCDs; such launches were seen to wait for room that never came.)
+static bool plan_packed_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan) {
+  plan->parts.clear();
+  plan->packed = true;
+  plan->phases_per_launch = kMaxPhases;
   if (!bt->host_seq_lens || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256) return false;
   const int capacity = fused_capacity(cfg, /*packed=*/true);
   if (capacity <= 0) return false;
@@ -1404,43 +1439,50 @@ static bool plan_packed_launches(const ts_config* cfg, const ts_batch* bt, std::
   if (fused_lds_bytes(tpb_max, cfg->num_heads) > kFusedStageBytes) return false;
   const int fixed = cfg->n_init + cfg->n_local;
   auto candidates = [&](int b) { return std::max(std::min(bt->host_seq_lens[b], bt->max_seq_len) - fixed, 0); };
+  // Phases of half the device when every request fits that.
+  bool halves = bt->batch >= 2;
+  for (int b = 0; b < bt->batch && halves; ++b)
+    if (ceil_div(candidates(b), tpb_max) > capacity / 2) halves = false;
+  const int room_full = halves ? capacity / 2 : capacity;
   for (int first = 0; first < bt->batch;) {
+    // (the second phase: half a phase, see above)
+    const bool shorter = halves && plan->parts.size() == 1;
     int64_t wgs = 0;
     int last = first, longest = 0;
-    for (; last < bt->batch && last - first < kMaxPacked; ++last) {
-      const int64_t more = ceil_div(candidates(last), tpb_max);
-      if (wgs + more > capacity) break;
-      wgs += more;
-      longest = std::max(longest, std::min(bt->host_seq_lens[last], bt->max_seq_len));
+    for (int pass = shorter ? 0 : 1; pass < 2 && last == first; ++pass) {
+      const int64_t room = pass == 0 ? room_full / 2 : room_full;
+      for (; last < bt->batch && last - first < kMaxPacked; ++last) {
+        const int64_t more = ceil_div(candidates(last), tpb_max);
+        if (wgs + more > room) break;
+        wgs += more;
+        longest = std::max(longest, std::min(bt->host_seq_lens[last], bt->max_seq_len));
+      }
     }
     if (last == first) return false;  // a single request does not fit the device
-    // the statistics' table of a request holds at most kSelMaxChunks chunks
-    int tpb = (int)std::max<int64_t>(64, ceil_div(ceil_div(longest, kSelMaxChunks), 64) * 64);
-    if (tpb > tpb_max) return false;
-    for (; tpb <= tpb_max; tpb += 64) {
-      wgs = 0;
-      for (int b = first; b < last; ++b) wgs += ceil_div(candidates(b), tpb);
-      if (wgs <= capacity) break;
-    }
-    if (tpb > tpb_max) return false;
-    if (wgs > 0)  // (nothing to launch for requests that are all sink and local window)
-      plan->push_back(VoteLaunch{first, last - first, tpb, (int)wgs, (int)ceil_div(longest, tpb), true});
+    // Every workgroup takes as many tokens as the LDS holds (the statistics' table of a
+    // request has room for kSelMaxChunks chunks): the fewer workgroups a phase has, the
+    // sooner those of the next one find room, and the less each token carries of what a
+    // workgroup does once (queries, statistics, the wait for them).
+    const int tpb = tpb_max;
+    if (ceil_div(longest, tpb) > kSelMaxChunks) return false;
+    if (wgs > 0)  // (nothing to do for requests that are all sink and local window)
+      plan->parts.push_back(VoteLaunch{first, last - first, tpb, (int)wgs, (int)ceil_div(longest, tpb)});
     first = last;
   }
   return true;
 }
 
 bool score_votes_packed(const ts_config* cfg, const ts_batch* bt) {
-  std::vector<VoteLaunch> plan;
+  VotePlan plan;
   return plan_packed_launches(cfg, bt, &plan);
 }
 
-// The launches of the votes-only form for a batch: packed by the host's lengths where
-// it has them, else groups of as many requests of max_seq_len as fit the device, each
-// launch a grid [chunks of max_seq_len, requests].  False: not even one request fits.
-bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<VoteLaunch>* plan) {
+// The parts of the votes-only form for a batch: packed by the host's lengths where it
+// has them, else groups of as many requests of max_seq_len as fit the device, each a
+// launch with a grid [chunks of max_seq_len, requests].  False: not even one request fits.
+bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan) {
   if (plan_packed_launches(cfg, bt, plan)) return true;
-  plan->clear();
+  *plan = VotePlan{};
   const int group = score_votes_group(cfg, bt->batch, bt->max_seq_len);
   if (group <= 0) return false;
   for (int first = 0; first < bt->batch; first += group) {
@@ -1448,7 +1490,7 @@ bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<Vo
     const SelectWorkspace w = select_workspace(cfg, requests, bt->max_seq_len, true);
     if (w.tokens_per_block <= 0) return false;
     if (w.blocks_per_req > 0)
-      plan->push_back(VoteLaunch{first, requests, w.tokens_per_block, w.blocks_per_req, w.blocks_per_req, false});
+      plan->parts.push_back(VoteLaunch{first, requests, w.tokens_per_block, w.blocks_per_req, w.blocks_per_req});
   }
   return true;
 }
@@ -1456,19 +1498,20 @@ bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, std::vector<Vo
 int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
                        int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
                        uint32_t* hist_ws, size_t hist_ws_stride, void* workspace, hipStream_t stream) {
-  std::vector<VoteLaunch> plan;
+  VotePlan plan;
   TS_REQUIRE(plan_vote_launches(cfg, bt, &plan), TS_ESHAPE,
              "fused scoring + vote: not even one request of %d tokens fits", bt->max_seq_len);
   // Offsets of the pieces: those of the whole batch's workspace, whatever the launches.
   const SelectWorkspace all = select_workspace(cfg, bt->batch, bt->max_seq_len, true);
   char* ws = (char*)workspace;
-  int launch = 0;
-  for (const VoteLaunch& v : plan) {
-    const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, v.packed);
+  const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, plan.packed);
+  const int per_launch = plan.packed ? plan.phases_per_launch : 1;
+  for (size_t at = 0; at < plan.parts.size(); at += per_launch) {
+    const VoteLaunch& v = plan.parts[at];
     ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, skip, (float*)(ws + all.partials),
                                  v.tokens_per_block);
     a.nchunks = kSelMaxChunks;
-    a.sync = (uint32_t*)(ws + all.sync) + (size_t)launch++ * kSyncWords;
+    a.sync = (uint32_t*)(ws + all.sync) + at * kSyncWords;  // one rendezvous area per part
     a.fault_word = (uint32_t*)(ws + all.sync);
     a.stats = (float*)(ws + all.stats);
     a.stats_stride = all.stats_stride;
@@ -1485,19 +1528,33 @@ int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf,
     a.hist_ws = hist_ws;
     a.hist_ws_stride = hist_ws_stride;
     dim3 grid((unsigned)v.workgroups, (unsigned)v.requests);
-    if (v.packed) {
-      a.packed = v.requests;
-      a.pack_first[0] = 0;
+    int tpb_lds = v.tokens_per_block;
+    if (plan.packed) {
+      const int phases = (int)std::min<size_t>(per_launch, plan.parts.size() - at);
       const int fixed = cfg->n_init + cfg->n_local;
-      for (int r = 0; r < v.requests; ++r) {
-        const int cand = std::max(std::min(bt->host_seq_lens[v.first + r], bt->max_seq_len) - fixed, 0);
-        a.pack_first[r + 1] = a.pack_first[r] + (int)ceil_div(cand, v.tokens_per_block);
+      a.nphases = phases;
+      int workgroups = 0;
+      for (int p = 0; p < phases; ++p) {
+        const VoteLaunch& part = plan.parts[at + p];
+        VotePhase& ph = a.phases[p];
+        ph.tokens_per_block = part.tokens_per_block;
+        ph.first = part.first;
+        ph.requests = part.requests;
+        ph.first_workgroup = workgroups;
+        ph.pack_first[0] = 0;
+        for (int r = 0; r < part.requests; ++r) {
+          const int cand =
+              std::max(std::min(bt->host_seq_lens[part.first + r], bt->max_seq_len) - fixed, 0);
+          ph.pack_first[r + 1] = ph.pack_first[r] + (int)ceil_div(cand, part.tokens_per_block);
+        }
+        workgroups += part.workgroups;
+        tpb_lds = std::max(tpb_lds, part.tokens_per_block);
       }
-      grid = dim3((unsigned)v.workgroups, 1u);
+      grid = dim3((unsigned)workgroups, 1u);
     }
     void* params[] = {(void*)&a};
     const hipError_t e = hipLaunchKernel(fn, grid, dim3(256), params,
-                                         fused_lds_bytes(v.tokens_per_block, cfg->num_heads), stream);
+                                         fused_lds_bytes(tpb_lds, cfg->num_heads), stream);
     if (e != hipSuccess) {
       (void)hipGetLastError();
       return fail(TS_EHIP, "fused scoring + vote launch: %s", hipGetErrorString(e));

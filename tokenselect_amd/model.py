@@ -131,6 +131,9 @@ class Decoder:
             raise RuntimeError("the KV cache has no slot left for another token")
         loc = self.free[self.decoded]
         max_len = max(self.contexts) + self.decoded + 1
+        # The lengths after this step's store, on the host too (a serving stack has them
+        # there): the layer then packs its scoring launches by what the requests hold.
+        host_lens = torch.tensor([c + self.decoded + 1 for c in self.contexts], dtype=torch.int32)
         hd, kvd = mc.num_heads * mc.head_dim, mc.num_kv_heads * mc.head_dim
         x = self.embed[tokens]
         for l in range(mc.layers):
@@ -145,7 +148,7 @@ class Decoder:
                 ops.kv_store(cfg, k, v, loc, self.k_pools[l], self.v_pools[l], self.table,
                              self.num_tokens[l])
             attn, sel, _, sel_len = self.attention(
-                q, self.k_pools[l], self.v_pools[l], Batch(self.num_tokens[l], self.table, max_len),
+                q, self.k_pools[l], self.v_pools[l], Batch(self.num_tokens[l], self.table, max_len, host_seq_lens=host_lens),
                 self.caches[l])
             if trace is not None:
                 if k is None:   # the rows as they landed in the pools
