@@ -147,15 +147,17 @@ def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
             sys.exit("bench.py: a grid-wide wait of the selection kernel gave up")
         dom_kernel = "ts::score_kernel<Hkv,G,false,2> (ts_select: score + vote + top-k in one launch)"
     elif ops.layer_selection_form(c, bt) == 1:
-        # Scores and votes request by request, the scores never in memory: B launches of
-        # the fused kernel in its votes-only form (+ one small clearing kernel); the
-        # figure is the bytes of all of them over the time of all of them.
+        # Scores and votes request by request, the scores never in memory: the fused kernel
+        # in its votes-only form (+ one small clearing kernel), one launch whose phases are
+        # packed by the host's lengths, or one launch per request without them; the figure
+        # is the bytes of all requests over the time of all launches.
         space = ops.select_workspace(c, bt, dev)
         dom_us, dom_min = event_time_us(
             lambda i: ops.score_vote(c, bt, qf, k_pools[i % n_pools], workspace=space), steps, warmup,
             burst=4)
-        dom_kernel = ("ts::score_kernel<Hkv,G,false,2> votes-only form, launches packed by the host's "
-                      "lengths (ts_score_vote: score + statistics + vote)" if bt.host_seq_lens is not None
+        dom_kernel = ("ts::score_kernel<Hkv,G,false,3> votes-only form, one launch whose phases are packed "
+                      "by the host's lengths (ts_score_vote: score + statistics + vote)"
+                      if bt.host_seq_lens is not None
                       else f"ts::score_kernel<Hkv,G,false,2> votes-only form x {B} launches "
                            "(ts_score_vote: score + statistics + vote, one request per launch)")
     else:
@@ -183,8 +185,9 @@ def bench_layer(args, ops, workloads, dev, which=None):
     make = {"c1": workloads.config1, "c2": workloads.config2, "c3": workloads.config3,
             "c5": workloads.config5_layer}[which or args.workload]
     wl = make(dev)
-    # A ragged batch: the lengths are handed over on the host as well (a serving framework
-    # holds them there), so that the launches are packed by what the requests hold.
+    # Batches too large for one ts_select launch: the lengths are handed over on the host as
+    # well (a serving framework holds them there), so that the scoring is one launch whose
+    # phases are packed by what the requests hold.
     wl.host_lengths = (which or args.workload) in ("c3", "c5") and not args.device_lengths_only
     c, bt, B = wl.cfg, wl.batch, len(wl.seq_lens)
     layer = ops.DecodeLayer(c, B, bt.max_seq_len, dev)
@@ -433,7 +436,8 @@ def bench_model(args, ops, dev):
     m.decode_step(tokens, trace)
     torch.cuda.synchronize()
     Lnow = L + args.warmup + args.steps + 1
-    bt = ops.Batch(m.num_tokens[0], m.table, Lnow)
+    bt = ops.Batch(m.num_tokens[0], m.table, Lnow,
+                   host_seq_lens=torch.full((B,), Lnow, dtype=torch.int32))  # as the model's layers pass them
     row = c.num_kv_heads * c.head_dim * 2
     score_bytes = B * ((Lnow - c.n_init - c.n_local) * row + Lnow * 4 + c.num_heads * c.head_dim * 2)
     cos, sin = ops.scoring_cos_sin(c.head_dim, c.rope_theta, c.rope_scale, c.n_local, dev)
@@ -448,15 +452,16 @@ def bench_model(args, ops, dev):
                   "frac": round(score_bytes / score_us / 1e3 / HBM_PEAK_GBS, 4),
                   "us_per_launch": round(score_us, 2), "us_min": round(score_min, 2)}
     dom_kernel = "ts::score_kernel<Hkv,G,false,1> (ts_score, one launch per layer)"
-    if ops.layer_selection_form(c, B, bt.max_seq_len) == 1:
-        # What the layers of this model run: scores and votes request by request, the
-        # scores never in memory (B launches; the figure is all their bytes over all their time).
+    if ops.layer_selection_form(c, bt) == 1:
+        # What the layers of this model run: scores and votes request by request, the scores
+        # never in memory (the requests as phases of one launch; the figure is all their
+        # bytes over all its time).
         space = ops.select_workspace(c, bt, dev)
         score_us, score_min = event_time_us(
             lambda i: ops.score_vote(c, bt, qf, m.k_pools[i % mc.layers], workspace=space),
             2 * mc.layers, mc.layers, burst=4)
-        dom_kernel = (f"ts::score_kernel<Hkv,G,false,2> votes-only form x {B} launches per layer "
-                      "(ts_score_vote: score + statistics + vote, one request per launch)")
+        dom_kernel = (f"ts::score_kernel<Hkv,G,false,3> votes-only form, {B} requests as phases of one "
+                      "launch per layer (ts_score_vote: score + statistics + vote)")
         del space
     gbs = score_bytes / score_us / 1e3
     weights = sum(w.numel() * 2 for ws in (m.wqkv, m.wo, m.w_gate_up, m.w_down) for w in ws) \
@@ -579,7 +584,7 @@ def main():
     ap.add_argument("--cpu-requests", type=int, default=2,
                     help="requests of a large batch the CPU oracle is run on")
     ap.add_argument("--device-lengths-only", action="store_true",
-                    help="c3: do not hand the lengths to the library on the host")
+                    help="c3, c5: do not hand the lengths to the library on the host")
     ap.add_argument("--no-extra", action="store_true",
                     help="default run: only the headline workload, not the compact lines of the others")
     ap.add_argument("--prefill-context", type=int, default=131072,
