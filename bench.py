@@ -149,17 +149,15 @@ def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
     elif ops.layer_selection_form(c, bt) == 1:
         # Scores and votes request by request, the scores never in memory: the fused kernel
         # in its votes-only form (+ one small clearing kernel), one launch whose phases are
-        # packed by the host's lengths, or one launch per request without them; the figure
-        # is the bytes of all requests over the time of all launches.
+        # packed by the host's lengths, or by max_seq_len without them; the figure is the
+        # bytes of all requests over the launch's time.
         space = ops.select_workspace(c, bt, dev)
         dom_us, dom_min = event_time_us(
             lambda i: ops.score_vote(c, bt, qf, k_pools[i % n_pools], workspace=space), steps, warmup,
             burst=4)
         dom_kernel = ("ts::score_kernel<Hkv,G,false,3> votes-only form, one launch whose phases are packed "
-                      "by the host's lengths (ts_score_vote: score + statistics + vote)"
-                      if bt.host_seq_lens is not None
-                      else f"ts::score_kernel<Hkv,G,false,2> votes-only form x {B} launches "
-                           "(ts_score_vote: score + statistics + vote, one request per launch)")
+                      + ("by the host's lengths" if bt.host_seq_lens is not None else "by max_seq_len")
+                      + " (ts_score_vote: score + statistics + vote)")
     else:
         dom_us, dom_min, dom_kernel = score_us, score_min, score_only["kernel"]
     gbs = score_bytes / dom_us / 1e3

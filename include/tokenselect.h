@@ -88,14 +88,17 @@ typedef struct ts_batch {
   const int32_t* host_seq_lens; /* NULL, or [B] in host memory: upper bounds of
                                seq_lens[] that the host knows (a serving
                                framework's CPU copy of the lengths), each <=
-                               max_seq_len.  Only sizes launches: a ragged batch
-                               that is too large for one ts_select launch is then
-                               scored and voted on in launches packed by what
-                               the requests hold (as by ts_score_vote) instead of
-                               by max_seq_len.  The device's seq_lens[] still
-                               rule; a bound below the device's value is an
-                               error the library cannot see (workgroups of the
-                               request would be missing)                        */
+                               max_seq_len.  Only sizes launches: a batch that
+                               is too large for one ts_select launch is scored
+                               and voted on in phases (as by ts_score_vote)
+                               packed by these bounds instead of by
+                               max_seq_len, which saves the workgroups that
+                               would find no candidates (16 requests of
+                               4K..128K: 447 instead of 461 us per layer).
+                               The device's seq_lens[] still rule; a bound
+                               below the device's value is an error the
+                               library cannot see (workgroups of the request
+                               would be missing)                               */
 } ts_batch;
 
 /* Optional selection-cache state for one layer (tr.py:301-322, 394-421).
@@ -176,14 +179,14 @@ int ts_vote(const ts_config* cfg, const ts_batch* bt, const float* scores,
             float* votes, float* pooled, int64_t vote_stride, ts_stream_t stream);
 
 /* ts_score + ts_vote without the [H, n] scores in memory (tr.py:350-361): the
- * requests are served in groups whose fp32 scores fit the LDS of the device, one
- * launch per group in which the workgroups poll for each other's softmax
+ * requests are served in groups ("phases") whose fp32 scores fit the LDS of the
+ * device, in which the workgroups poll for each other's softmax
  * statistics (and meet once with cfg->pool_kernel > 0) and then write the votes; a batch of
  * any size is served as long as one request fits (some 260K candidates for 32
- * heads) and pool_kernel is at most 256 (ts_score_vote_supported).  The groups are
- * sized by max_seq_len, or, with ts_batch.host_seq_lens, packed by what the requests
- * hold: phases of up to 8 consecutive requests that fit half the device (all of it
- * for a request that needs more), the workgroups of up to 24 phases in one launch,
+ * heads) and pool_kernel is at most 256 (ts_score_vote_supported).  The requests are
+ * packed by what they can hold (ts_batch.host_seq_lens where given, max_seq_len
+ * else) into phases of up to 8 consecutive requests that fit half the device (all of
+ * it for a request that needs more), the workgroups of up to 24 phases in one launch,
  * which the device works through in order, so that one phase streams keys while
  * another waits for its statistics.  votes
  * [B, vote_stride] fp32 receives what ts_vote's votes (pooled with pool_kernel > 0)
@@ -411,21 +414,20 @@ int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, in
  * cache may be NULL (QUERY_CACHE=False as released, tr.py:918).
  *
  * When ts_select_supported() holds, the selection runs as the single ts_select
- * kernel; a batch of contexts so long that each request needs the device to itself
- * is scored and voted on request by request as by ts_score_vote and then ranked by
- * the kernels of ts_topk_ragged (so is a ragged batch whose lengths the host passes
- * in ts_batch.host_seq_lens, the whole batch in one launch as a rule); otherwise ts_score, ts_vote and
- * ts_topk_ragged run
- * as they do on their own.  All forms give the same selection.
+ * kernel; a batch too large for that (many requests, or contexts so long that each
+ * request needs the device to itself) is scored and voted on as by ts_score_vote, in
+ * one launch as a rule, and then ranked by the kernels of ts_topk_ragged; where
+ * neither serves (pool_kernel above 256, a request that does not fit the device)
+ * ts_score, ts_vote and ts_topk_ragged run as they do on their own.  All forms give
+ * the same selection.
  * ts_set_fused_select(0) forces the separate kernels for the calling process
  * (1 restores the default); it returns the previous setting and has no
  * counterpart in the reference. */
 int ts_set_fused_select(int enable);
 /* Which form ts_decode_layer takes for a shape: 2 = ts_select, 1 = ts_score_vote's
- * launches (one request each) + top-k kernels, 0 = ts_score + ts_vote + top-k
- * kernels; -1 for an unsupported configuration.  The second form answers for a batch
- * descriptor: with host_seq_lens, a ragged batch too large for one ts_select launch
- * takes form 1 with its requests packed into one launch by those lengths. */
+ * launch + top-k kernels, 0 = ts_score + ts_vote + top-k kernels; -1 for an
+ * unsupported configuration.  The second form answers for a batch descriptor (the
+ * same answer: host_seq_lens changes how the phases are packed, not the form). */
 int ts_decode_layer_selection(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
 int ts_decode_layer_selection_of(const ts_config* cfg, const ts_batch* bt);
 size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);

@@ -147,19 +147,25 @@ def test_scores_at_full_size_against_a_dense_product(dev):
     assert (got - ref).abs().max().item() <= 1e-3 * scale
 
 
-@pytest.mark.parametrize("host_lengths", [False, True], ids=["device-lengths", "host-lengths"])
-def test_ragged_batch_config(dev, host_lengths):
-    """With the lengths known on the host as well, the batch is scored and voted on in a few
-    launches packed by those lengths (form 1); without, by the separate kernels (form 0)."""
-    wl = workloads.config3(dev)
-    wl.host_lengths = host_lengths
-    say(f"full size {wl.name} lens={wl.seq_lens} host_lengths={host_lengths}")
-    assert ops.layer_selection_form(wl.cfg, wl.batch) == (1 if host_lengths else 0)
-    result = _run(wl, dev)
-    votes, _ = _votes_on_device(wl)
-    _check_properties(wl, result, votes, wl.name)
-    order = sorted(range(len(wl.seq_lens)), key=lambda b: wl.seq_lens[b])
-    _check_against_oracle(wl, result, [order[0], order[len(order) // 2], order[-1]], wl.name)
+@pytest.mark.parametrize("host_lengths,fused", [(False, True), (True, True), (False, False)],
+                         ids=["device-lengths", "host-lengths", "separate-kernels"])
+def test_ragged_batch_config(dev, host_lengths, fused):
+    """The batch is too large for one co-resident launch: it is scored and voted on as phases
+    of one launch (form 1), packed by the host's lengths where the batch carries them and by
+    max_seq_len where not; with the fused kernels switched off, by the separate kernels."""
+    previous = ops.set_fused_select(fused)
+    try:
+        wl = workloads.config3(dev)
+        wl.host_lengths = host_lengths
+        say(f"full size {wl.name} lens={wl.seq_lens} host_lengths={host_lengths} fused={fused}")
+        assert ops.layer_selection_form(wl.cfg, wl.batch) == (1 if fused else 0)
+        result = _run(wl, dev)
+        votes, _ = _votes_on_device(wl)
+        _check_properties(wl, result, votes, wl.name)
+        order = sorted(range(len(wl.seq_lens)), key=lambda b: wl.seq_lens[b])
+        _check_against_oracle(wl, result, [order[0], order[len(order) // 2], order[-1]], wl.name)
+    finally:
+        ops.set_fused_select(previous)
 
 
 def test_large_context_layer_config(dev):

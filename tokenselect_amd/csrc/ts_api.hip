@@ -168,27 +168,21 @@ size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int3
 }
 
 // How ts_decode_layer selects for a shape: 2 = the single ts_select kernel, 1 = scores and
-// votes per request as by ts_score_vote, then the top-k kernels, 0 = ts_score, ts_vote
-// and the top-k kernels.
+// votes as by ts_score_vote (a batch too large for one co-resident launch: its requests as
+// phases of one launch), then the top-k kernels, 0 = ts_score, ts_vote and the top-k
+// kernels (fused kernels switched off, a max-pool window above 256, a request that does
+// not fit the device).
 static int layer_selection_form(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (select_workspace(cfg, batch, max_seq_len).tokens_per_block > 0) return 2;
   const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
-  // A request of max_seq_len needs the device to itself (4 x 256K: 463 us per layer
-  // against 481 us with the separate kernels).  The grids are sized by max_seq_len, so
-  // with several requests per launch a ragged batch (16 x 4K..128K: 617 against 534 us)
-  // leaves most workgroups of a launch without tokens: those take the separate kernels.
-  if (max_n > 0 && cfg->pool_kernel <= 256 && score_votes_group(cfg, batch, max_seq_len) == 1) return 1;
+  if (max_n > 0 && cfg->pool_kernel <= 256 && score_votes_group(cfg, 1, max_seq_len) > 0) return 1;
   return 0;
 }
 
-// The same for a batch whose descriptor may carry the host's lengths: a ragged batch too
-// large for one launch then takes form 1 with its launches packed by those lengths (16 x
-// 4K..128K: five launches instead of the fp32 scores written and read back).
+// The same for a batch descriptor (the host's lengths, where it carries them, change how
+// the phases are packed, not the form).
 static int layer_selection_form(const ts_config* cfg, const ts_batch* bt) {
-  const int form = layer_selection_form(cfg, bt->batch, bt->max_seq_len);
-  if (form != 0 || !bt->host_seq_lens) return form;
-  const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
-  return (max_n > 0 && cfg->pool_kernel <= 256 && score_votes_packed(cfg, bt)) ? 1 : 0;
+  return layer_selection_form(cfg, bt->batch, bt->max_seq_len);
 }
 
 // Decode (chunk_rows == 0: one query row per request, q_cos / q_sin are the [D] rows

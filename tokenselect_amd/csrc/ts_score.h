@@ -55,17 +55,14 @@ struct ScoreArgs {
   uint32_t* clear;        // words to clear for the next kernel of the stream, or NULL
   int clear_per_req;
   uint64_t spin_ticks;    // bound of a grid-wide wait, in 100 MHz ticks
-  // Votes-only form of the fused kernel (groups of requests of a large batch, one
-  // launch each): request index of the launch's first request; the launch ends with
-  // the votes in memory and their first-level histogram added to the top-k workspace.
-  int batch_offset;
-  int votes_only;
-  // Votes-only launches packed by the host's lengths (a kernel instantiation of their
-  // own): a one-dimensional grid that holds the workgroups of `nphases` phases one after
+  int batch_offset;       // request index of the launch's first request
+  // Votes-only form of the fused kernel (a kernel instantiation of its own): the launch
+  // ends with the votes in memory and their first-level histogram added to the top-k
+  // workspace.  A one-dimensional grid holds the workgroups of `nphases` phases one after
   // the other, each phase a group of requests that fits half the device (or all of it).
-  // A workgroup serves one phase; one without candidates (the host's length was an upper
-  // bound) leaves at once and is not on the phase's team.  Phase p's rendezvous area is
-  // sync + p * kSyncWords.
+  // A workgroup serves one phase; one without candidates (the length was below the bound
+  // the phase was sized by) leaves at once and is not on the phase's team.  Phase p's
+  // rendezvous area is sync + p * kSyncWords.
   int nphases;
   VotePhase phases[kMaxPhases];
   uint32_t* hist_ws;      // per-request top-k workspace (ts_topk.h) whose hist0 is counted into, or NULL
@@ -131,17 +128,14 @@ int launch_select_zero(const ZeroSet& zero, hipStream_t stream);
 constexpr uint64_t kSelectWaitTicks = 200000000ull;
 
 // Scores and votes of a batch of any size without the [H, n] scores in memory: the
-// requests are served in groups whose scores fit the LDS of the device, one launch of
-// the fused kernel in its votes-only form per group (score, statistics rendezvous,
-// votes, [max-pool]); each launch also counts the first histogram level of the top-k
-// into hist_ws.  score_votes_group() is the number of requests per launch, 0 when not
-// even one request fits (or the fused kernels are switched off): then the separate
-// kernels serve.  The workspace is that of ts_select for the whole batch; the
-// statistics (per workgroup and merged) and the rendezvous areas (score_votes_zero_regions)
-// are zero.
-// Whether the batch is served by votes-only launches packed by the host's lengths
-// (ts_batch.host_seq_lens given, every request fits the device).
-bool score_votes_packed(const ts_config* cfg, const ts_batch* bt);
+// requests are served in phases whose scores fit the LDS of half the device (of all of it
+// for a request that needs more), the workgroups of all phases in one launch of the fused
+// kernel's votes-only form (score, statistics, votes, [max-pool]); the launch also counts
+// the first histogram level of the top-k into hist_ws.  score_votes_group() is positive
+// when a request of max_seq_len fits the device and the fused kernels are switched on:
+// else the separate kernels serve.  The workspace is that of ts_select for the whole
+// batch; the statistics (per workgroup and merged) and the rendezvous areas
+// (score_votes_zero_regions) are zero.
 int score_votes_group(const ts_config* cfg, int batch, int max_seq_len);
 void score_votes_zero_regions(const ts_config* cfg, const ts_batch* bt, const SelectWorkspace& w,
                               void* workspace, ZeroSet* zero);

@@ -83,8 +83,8 @@ constexpr int kQuadSwap2 = 0x4E;  // quad_perm [2,3,0,1]
 //     where its selected positions, in ascending order, belong (tr.py:371-373,
 //     433-449); masses of exact ties go through all three levels and a count round.
 constexpr int kScoreDirect = 0, kScoreTiled = 1, kScoreFused = 2;
-// The fused kernel's votes-only form for launches packed by the host's lengths: a kernel
-// of its own, so that the single-launch selection does not carry the bookkeeping.
+// The fused kernel's votes-only form (phases of requests in one launch): a kernel of its
+// own, so that the single-launch selection does not carry the bookkeeping.
 constexpr int kScorePacked = 3;
 constexpr int kMaxHeads = 128;
 
@@ -379,7 +379,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   if constexpr (FUSED) {
     __shared__ uint32_t team_lds[8];
     TS_MARK(0);
-    if (!a.votes_only) fixed_segments(a, b);
+    if (!PACKED) fixed_segments(a, b);
     if (n <= 0) return;  // dense or served by the cache: nothing to select, not on the team
     if (PACKED && block_lo >= n) return;  // no candidates here, and the team is made without it
     team = selecting_team<PACKED>(a, lp, team_lds, req, chunk);
@@ -387,7 +387,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   if (block_lo >= n) {
     if constexpr (FUSED) {  // no tokens here: only help with the statistics
       merge_request_stats<PACKED>(a, lp, team, threadIdx.x & 63, threadIdx.x >> 6);
-      const uint32_t rounds = (a.votes_only ? 0u : kSelectRounds) + (a.pool_kernel > 0 ? 1u : 0u);
+      const uint32_t rounds = kSelectRounds + (a.pool_kernel > 0 ? 1u : 0u);  // (not PACKED here)
       for (uint32_t round = 1; round <= rounds; ++round)
         grid_arrive(lp.sync, round, false, a.spin_ticks, team.size, team.index);
     }
@@ -716,7 +716,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       for (int i = tid; i < count + halo; i += 256) lh[i] = 0u;
       __syncthreads();
     }
-    if (PACKED || a.votes_only) {
+    if (PACKED) {
       // The launch ends here: the votes are in memory, and their first histogram level
       // goes to the top-k workspace, where the kernels after this one pick it up.
       if (a.hist_ws) {
@@ -1246,18 +1246,14 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
   return w;
 }
 
-// One part of the votes-only form (a launch, or a phase of a packed launch): requests
-// [first, first + requests), `workgroups` along x (packed: all of the part's; else per
-// request), `table_chunks` an upper bound of the chunks of any of its requests.
+// One phase of the votes-only form: requests [first, first + requests), `workgroups` in
+// all, `table_chunks` an upper bound of the chunks of any of its requests.
 struct VoteLaunch {
   int first, requests, tokens_per_block, workgroups, table_chunks;
 };
-// The parts of a batch.  packed: phases, up to phases_per_launch of them to a launch;
-// else one launch each.
+// The phases of a batch, up to kMaxPhases of them to a launch.
 struct VotePlan {
   std::vector<VoteLaunch> parts;
-  bool packed = false;
-  int phases_per_launch = 1;
 };
 bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan);
 
@@ -1410,35 +1406,37 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   return TS_OK;
 }
 
-// The votes-only form when the host knows upper bounds of the lengths
-// (ts_batch.host_seq_lens): consecutive requests are packed into phases by what they
-// hold, not by max_seq_len -- as many as fit half the device (all of it, when a request
-// needs more) with the most tokens per workgroup that the LDS takes.  One launch holds the workgroups of
-// many phases, one after the other in a one-dimensional grid.  The device starts the
-// workgroups of a grid in the order of their numbers as room becomes free (of those that
-// go to one XCD, every eighth): with phases of half the device two of them are resident
-// side by side, and when the workgroups of the earlier one leave, those of the next but
-// one take their places.  A phase ends with the memory idle (the statistics on their
-// way, scores turned into votes); the other phase streams meanwhile.  Two phases that
-// start together would also wait together, so the second phase is given about half the
-// candidates of a full one.  Nothing can wait forever: the workgroups of the earliest
-// unfinished phase wait for each other only, and all of them have been started, since
-// every workgroup started before them has left and fewer than fit are left to start.
-// (A grid [chunks of the longest, requests] whose surplus workgroups leave at once is
-// not an alternative: its members have gaps between them and do not spread evenly over
-// the XCDs; such launches were seen to wait for room that never came.)
-static bool plan_packed_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan) {
+// The votes-only form: consecutive requests are packed into phases by what they can
+// hold -- the host's upper bounds of the lengths (ts_batch.host_seq_lens) where it has
+// them, max_seq_len else -- as many as fit half the device (all of it, when a request
+// needs more) with the most tokens per workgroup that the LDS takes.  One launch holds
+// the workgroups of many phases, one after the other in a one-dimensional grid.  The
+// device starts the workgroups of a grid in the order of their numbers as room becomes
+// free (of those that go to one XCD, every eighth): with phases of half the device two
+// of them are resident side by side, and when the workgroups of the earlier one leave,
+// those of the next but one take their places.  A phase ends with the memory idle (the
+// statistics on their way, scores turned into votes); the other phase streams
+// meanwhile.  Two phases that start together would also wait together, so the second
+// phase is given about half the candidates of a full one.  A workgroup without
+// candidates (the bound was above the length) leaves at once and is not on the phase's
+// team.  Nothing can wait forever: the workgroups of the earliest unfinished phase wait
+// for each other only, and all of them have been started, since every workgroup started
+// before them has left and fewer than fit are left to start.
+// (A grid [chunks of the longest, requests] of a group of requests that must all be
+// resident at once is not an alternative: its members have gaps between them and do not
+// spread evenly over the XCDs; such launches were seen to wait for room that never came.)
+bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan) {
   plan->parts.clear();
-  plan->packed = true;
-  plan->phases_per_launch = kMaxPhases;
-  if (!bt->host_seq_lens || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256) return false;
+  if (!g_fused_select.load()) return false;
+  if (cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256) return false;
   const int capacity = fused_capacity(cfg, /*packed=*/true);
   if (capacity <= 0) return false;
   int tpb_max = 64;
   while (fused_lds_bytes(tpb_max + 64, cfg->num_heads) <= kFusedStageBytes) tpb_max += 64;
   if (fused_lds_bytes(tpb_max, cfg->num_heads) > kFusedStageBytes) return false;
   const int fixed = cfg->n_init + cfg->n_local;
-  auto candidates = [&](int b) { return std::max(std::min(bt->host_seq_lens[b], bt->max_seq_len) - fixed, 0); };
+  auto bound = [&](int b) { return bt->host_seq_lens ? std::min(bt->host_seq_lens[b], bt->max_seq_len) : bt->max_seq_len; };
+  auto candidates = [&](int b) { return std::max(bound(b) - fixed, 0); };
   // Phases of half the device when every request fits that.
   bool halves = bt->batch >= 2;
   for (int b = 0; b < bt->batch && halves; ++b)
@@ -1455,7 +1453,7 @@ static bool plan_packed_launches(const ts_config* cfg, const ts_batch* bt, VoteP
         const int64_t more = ceil_div(candidates(last), tpb_max);
         if (wgs + more > room) break;
         wgs += more;
-        longest = std::max(longest, std::min(bt->host_seq_lens[last], bt->max_seq_len));
+        longest = std::max(longest, bound(last));
       }
     }
     if (last == first) return false;  // a single request does not fit the device
@@ -1472,29 +1470,6 @@ static bool plan_packed_launches(const ts_config* cfg, const ts_batch* bt, VoteP
   return true;
 }
 
-bool score_votes_packed(const ts_config* cfg, const ts_batch* bt) {
-  VotePlan plan;
-  return plan_packed_launches(cfg, bt, &plan);
-}
-
-// The parts of the votes-only form for a batch: packed by the host's lengths where it
-// has them, else groups of as many requests of max_seq_len as fit the device, each a
-// launch with a grid [chunks of max_seq_len, requests].  False: not even one request fits.
-bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan) {
-  if (plan_packed_launches(cfg, bt, plan)) return true;
-  *plan = VotePlan{};
-  const int group = score_votes_group(cfg, bt->batch, bt->max_seq_len);
-  if (group <= 0) return false;
-  for (int first = 0; first < bt->batch; first += group) {
-    const int requests = std::min(group, bt->batch - first);
-    const SelectWorkspace w = select_workspace(cfg, requests, bt->max_seq_len, true);
-    if (w.tokens_per_block <= 0) return false;
-    if (w.blocks_per_req > 0)
-      plan->parts.push_back(VoteLaunch{first, requests, w.tokens_per_block, w.blocks_per_req, w.blocks_per_req});
-  }
-  return true;
-}
-
 int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
                        int64_t pool_rows, const int32_t* skip, float* votes, int64_t vote_stride,
                        uint32_t* hist_ws, size_t hist_ws_stride, void* workspace, hipStream_t stream) {
@@ -1504,8 +1479,8 @@ int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf,
   // Offsets of the pieces: those of the whole batch's workspace, whatever the launches.
   const SelectWorkspace all = select_workspace(cfg, bt->batch, bt->max_seq_len, true);
   char* ws = (char*)workspace;
-  const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, plan.packed);
-  const int per_launch = plan.packed ? plan.phases_per_launch : 1;
+  const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, true);
+  const int per_launch = kMaxPhases;
   for (size_t at = 0; at < plan.parts.size(); at += per_launch) {
     const VoteLaunch& v = plan.parts[at];
     ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, skip, (float*)(ws + all.partials),
@@ -1524,12 +1499,11 @@ int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf,
     a.pool_votes = (float*)(ws + all.pool_votes);
     a.pool_stride = all.pool_stride;
     a.batch_offset = v.first;
-    a.votes_only = 1;
     a.hist_ws = hist_ws;
     a.hist_ws_stride = hist_ws_stride;
-    dim3 grid((unsigned)v.workgroups, (unsigned)v.requests);
     int tpb_lds = v.tokens_per_block;
-    if (plan.packed) {
+    dim3 grid;
+    {
       const int phases = (int)std::min<size_t>(per_launch, plan.parts.size() - at);
       const int fixed = cfg->n_init + cfg->n_local;
       a.nphases = phases;
@@ -1543,8 +1517,9 @@ int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf,
         ph.first_workgroup = workgroups;
         ph.pack_first[0] = 0;
         for (int r = 0; r < part.requests; ++r) {
-          const int cand =
-              std::max(std::min(bt->host_seq_lens[part.first + r], bt->max_seq_len) - fixed, 0);
+          const int len = bt->host_seq_lens ? std::min(bt->host_seq_lens[part.first + r], bt->max_seq_len)
+                                            : bt->max_seq_len;
+          const int cand = std::max(len - fixed, 0);
           ph.pack_first[r + 1] = ph.pack_first[r] + (int)ceil_div(cand, part.tokens_per_block);
         }
         workgroups += part.workgroups;

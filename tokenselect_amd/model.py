@@ -132,7 +132,7 @@ class Decoder:
         loc = self.free[self.decoded]
         max_len = max(self.contexts) + self.decoded + 1
         # The lengths after this step's store, on the host too (a serving stack has them
-        # there): the layer then packs its scoring launches by what the requests hold.
+        # there): the layer then packs its scoring phases by what the requests hold.
         host_lens = torch.tensor([c + self.decoded + 1 for c in self.contexts], dtype=torch.int32)
         hd, kvd = mc.num_heads * mc.head_dim, mc.num_kv_heads * mc.head_dim
         x = self.embed[tokens]

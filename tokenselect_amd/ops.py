@@ -66,8 +66,8 @@ class Batch:
     # selection sets to 1 when one of its grid-wide waits gave up, or None.
     fault: Optional[torch.Tensor] = None
     # Upper bounds of seq_lens that the host knows ([B] int32 on the CPU, e.g. a serving
-    # framework's CPU copy of the lengths), or None: a ragged batch too large for one
-    # selection launch is then served in launches packed by what the requests hold.
+    # framework's CPU copy of the lengths), or None: a batch too large for one selection
+    # launch is then scored in phases packed by these bounds instead of by max_seq_len.
     host_seq_lens: Optional[torch.Tensor] = None
 
     @property
@@ -402,8 +402,8 @@ def vote(cfg: LayerConfig, bt: Batch, scores: torch.Tensor, partials: torch.Tens
 
 def layer_selection_form(cfg: LayerConfig, batch, max_seq_len: Optional[int] = None) -> int:
     """How :class:`DecodeLayer` selects for a shape ``(batch, max_seq_len)`` or for a
-    :class:`Batch` (whose ``host_seq_lens`` count): 2 = one ``ts_select`` launch, 1 =
-    ``ts_score_vote``'s launches + the top-k kernels, 0 = the separate kernels."""
+    :class:`Batch`: 2 = one ``ts_select`` launch, 1 = ``ts_score_vote``'s launch + the top-k
+    kernels, 0 = the separate kernels."""
     if isinstance(batch, Batch):
         cb = _c_batch(cfg, batch)
         return int(_lib.load().ts_decode_layer_selection_of(ctypes.byref(cfg.to_c()), ctypes.byref(cb)))

@@ -227,8 +227,8 @@ class BatchTokenRetriever:
         if runner is None:
             runner = ops.DecodeLayer(cfg, self.batch, self.max_num_tokens, self.device)
             self._layers[key] = runner
-        # The lengths go along on the host too: a ragged batch that is too large for one
-        # selection launch is then served in launches packed by what the requests hold.
+        # The lengths go along on the host too: a batch that is too large for one selection
+        # launch is then scored in phases packed by what the requests hold.
         bt = ops.Batch(self._num_tokens_dev[layer_id], self.token_indices[layer_id],
                        max(self.num_tokens[layer_id]),
                        host_seq_lens=torch.tensor(self.num_tokens[layer_id], dtype=torch.int32))
