@@ -96,9 +96,10 @@ typedef struct ts_batch {
                                would find no candidates (16 requests of
                                4K..128K: 447 instead of 461 us per layer).
                                The device's seq_lens[] still rule; a bound
-                               below the device's value is an error the
-                               library cannot see (workgroups of the request
-                               would be missing)                               */
+                               below the device's value is the caller's error:
+                               the tokens beyond it are not scored, and the
+                               launch reports it like a wait that gave up
+                               (fault, sel_len = -1)                           */
 } ts_batch;
 
 /* Optional selection-cache state for one layer (tr.py:301-322, 394-421).

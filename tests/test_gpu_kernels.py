@@ -749,6 +749,41 @@ def test_score_vote_phases_of_one_launch(dev, case, pool_kernel):
                 f"b={b} L={L} attempt={attempt}"
 
 
+def test_score_vote_reports_a_length_above_its_bound(dev):
+    """host_seq_lens are upper bounds; a request that is longer on the device than the host
+    said has no workgroups for its last tokens.  The launch says so at once (the caller's
+    fault word, without waiting for statistics that cannot come), and the same call with
+    honest bounds on the same workspace is correct."""
+    import time
+    lens = [3000, 2000, 2500]
+    say(f"score_vote with a bound below the length, lens={lens}")
+    wl = small(dev, SHAPES[0], seed=53, lens=lens, ks=[64] * 3, page=16, top_k=64)
+    c = wl.cfg
+    qf = fingerprint(wl, dev)
+    word = ops.fault_word()
+    space = ops.select_workspace(c, wl.batch, dev)
+    low = ops.Batch(wl.batch.seq_lens, wl.batch.table, max(lens), wl.batch.k_per_req, word,
+                    host_seq_lens=torch.tensor([1400, 2000, 2500], dtype=torch.int32))
+    torch.cuda.synchronize()
+    t0 = time.time()
+    ops.score_vote(c, low, qf, wl.k_pool, workspace=space)
+    torch.cuda.synchronize()
+    assert time.time() - t0 < 1.0, "reported without running into the bound of a wait"
+    with pytest.raises(ops.SelectionGaveUp):
+        ops.raise_if_gave_up(word)
+    word.zero_()
+    good = ops.Batch(wl.batch.seq_lens, wl.batch.table, max(lens), wl.batch.k_per_req, word,
+                     host_seq_lens=torch.tensor(lens, dtype=torch.int32))
+    votes = ops.score_vote(c, good, qf, wl.k_pool, workspace=space)
+    votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool))
+    torch.cuda.synchronize()
+    ops.raise_if_gave_up(word)
+    for b, L in enumerate(lens):
+        n = L - c.n_init - c.n_local
+        want = votes_sep[b, :n]
+        assert (votes[b, :n] - want).abs().max().item() <= 1e-5 * want.abs().max().item(), f"b={b}"
+
+
 @pytest.mark.parametrize("pool_kernel", [-1, 5])
 @pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
 def test_layer_split_at_the_vote(dev, fused_select, pool_kernel):

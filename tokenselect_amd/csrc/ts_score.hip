@@ -107,6 +107,14 @@ struct LaunchPart {
   uint32_t* sync;         // rendezvous area
 };
 
+// Chunks of request r of a phase that hold candidates: those of its n candidates, but no
+// more than the phase has workgroups for it (a length above the bound the phase was sized
+// by is the caller's error: the tokens beyond are not scored, and the launch reports it).
+__device__ __forceinline__ int packed_chunks(const LaunchPart& lp, int r, int n) {
+  const int chunks = (n + lp.tokens_per_block - 1) / lp.tokens_per_block;
+  return min(chunks, lp.pack_first[r + 1] - lp.pack_first[r]);
+}
+
 template <bool PACKED>
 __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const LaunchPart& lp,
                                                     const GridTeam& team, int lane, int wave) {
@@ -120,7 +128,8 @@ __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const La
     const ReqGeom geo =
         request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
     if (geo.n <= 0) continue;
-    const int chunks = (geo.n + lp.tokens_per_block - 1) / lp.tokens_per_block;
+    const int chunks = PACKED ? packed_chunks(lp, item / H, geo.n)
+                              : (geo.n + lp.tokens_per_block - 1) / lp.tokens_per_block;
     const float2* part = (const float2*)a.partials + ((size_t)b * H + h) * a.nchunks;
     float m = kNegBig, l = 0.f;
     const uint64_t t0 = wall_clock64();
@@ -195,8 +204,7 @@ __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, const Lau
       if (a.skip && a.skip[b]) continue;
       const int n = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
                                      a.max_seq_len).n;
-      const uint32_t members =
-          n > 0 ? (uint32_t)((n + lp.tokens_per_block - 1) / lp.tokens_per_block) : 0u;
+      const uint32_t members = n > 0 ? (uint32_t)packed_chunks(lp, r, n) : 0u;
       total += members;
       if (r < req) before += members;
     }
@@ -382,6 +390,9 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     if (!PACKED) fixed_segments(a, b);
     if (n <= 0) return;  // dense or served by the cache: nothing to select, not on the team
     if (PACKED && block_lo >= n) return;  // no candidates here, and the team is made without it
+    if (PACKED && chunk == 0 && threadIdx.x == 0 &&
+        (n + lp.tokens_per_block - 1) / lp.tokens_per_block > lp.pack_first[req + 1] - lp.pack_first[req])
+      __hip_atomic_store(&lp.sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // length above its bound
     team = selecting_team<PACKED>(a, lp, team_lds, req, chunk);
   }
   if (block_lo >= n) {

@@ -78,7 +78,8 @@ class Batch:
 class SelectionGaveUp(RuntimeError):
     """A grid-wide wait of the single-launch selection ran into its bound: the launch
     did not have the device to itself (its workgroups were not all resident together)
-    and what it selected, and what was attended over, is not valid."""
+    and what it selected, and what was attended over, is not valid.  Also raised when a
+    request was longer on the device than ``Batch.host_seq_lens`` said."""
 
 
 def fault_word() -> torch.Tensor:
@@ -93,8 +94,9 @@ def raise_if_gave_up(word: Optional[torch.Tensor]) -> None:
     if word is not None and int(word[0]) != 0:
         raise SelectionGaveUp(
             "ts_select gave up waiting for its workgroups (is another stream or process using the "
-            "GPU?); results since the last check are not valid.  Serialise the GPU work, or call "
-            "ops.set_fused_select(False) to use the separate kernels, clear the word and rerun")
+            "GPU?), or a request was longer than its entry of host_seq_lens; results since the last "
+            "check are not valid.  Serialise the GPU work, or call ops.set_fused_select(False) to "
+            "use the separate kernels, clear the word and rerun")
 
 
 @dataclass
