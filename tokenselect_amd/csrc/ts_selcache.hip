@@ -19,6 +19,8 @@ struct SelCacheArgs {
   int32_t* hit;
 };
 
+constexpr int kSelCacheMaxVec = 4;  // 16-byte pieces per thread: 64 heads x 128 / 8 / 256
+
 __global__ __launch_bounds__(256) void selcache_kernel(SelCacheArgs a) {
   const int b = blockIdx.x;
   const ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
@@ -30,13 +32,28 @@ __global__ __launch_bounds__(256) void selcache_kernel(SelCacheArgs a) {
   uint16_t* qc = a.q_cache + (size_t)b * a.dim;
   const bool have = a.cache_len[b] > 0;  // is_first_query is false
 
+  // dim = H * 128 elements, at most kMaxVec 16-byte pieces per thread, all requested at
+  // once (one piece per thread and pass: a loop of dependent 2-byte loads took 8 us).
+  constexpr int kMaxVec = kSelCacheMaxVec;
+  const int pieces = a.dim >> 3;
+  uint4 qv[kMaxVec], cv[kMaxVec];
+#pragma unroll
+  for (int j = 0; j < kMaxVec; ++j) {
+    const int i = threadIdx.x + 256 * j;
+    qv[j] = i < pieces ? ((const uint4*)q)[i] : make_uint4(0u, 0u, 0u, 0u);
+    cv[j] = (have && i < pieces) ? ((const uint4*)qc)[i] : make_uint4(0u, 0u, 0u, 0u);
+  }
   float dot = 0.f, nq = 0.f, nc = 0.f;
-  if (have) {
-    for (int i = threadIdx.x; i < a.dim; i += 256) {
-      const float x = bf16_to_f32(q[i]), y = bf16_to_f32(qc[i]);
-      dot += x * y;
-      nq += x * x;
-      nc += y * y;
+#pragma unroll
+  for (int j = 0; j < kMaxVec; ++j) {
+    const uint32_t xs[4] = {qv[j].x, qv[j].y, qv[j].z, qv[j].w};
+    const uint32_t ys[4] = {cv[j].x, cv[j].y, cv[j].z, cv[j].w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float x0 = bf16_lo(xs[e]), x1 = bf16_hi(xs[e]), y0 = bf16_lo(ys[e]), y1 = bf16_hi(ys[e]);
+      dot += x0 * y0 + x1 * y1;
+      nq += x0 * x0 + x1 * x1;
+      nc += y0 * y0 + y1 * y1;
     }
   }
   __shared__ float red[3][4];
@@ -56,8 +73,13 @@ __global__ __launch_bounds__(256) void selcache_kernel(SelCacheArgs a) {
   nc = red[2][0] + red[2][1] + red[2][2] + red[2][3];
   const float cosine = dot / fmaxf(sqrtf(nq) * sqrtf(nc), 1e-8f);
   const bool is_hit = have && !(cosine < a.threshold);  // tr.py:395-401
-  if (!is_hit)
-    for (int i = threadIdx.x; i < a.dim; i += 256) qc[i] = q[i];  // tr.py:416
+  if (!is_hit) {  // tr.py:416
+#pragma unroll
+    for (int j = 0; j < kMaxVec; ++j) {
+      const int i = threadIdx.x + 256 * j;
+      if (i < pieces) ((uint4*)qc)[i] = qv[j];
+    }
+  }
   if (threadIdx.x == 0) {
     a.hit[b] = is_hit ? 1 : 0;
     if (is_hit) a.counters[2 * b] += 1;  // skip_count, tr.py:420
@@ -89,6 +111,8 @@ extern "C" int ts_selcache_step(const ts_config* cfg, const ts_batch* bt, const 
   a.top_k = cfg->top_k;
   a.max_seq_len = bt->max_seq_len;
   a.dim = cfg->num_heads * cfg->head_dim;
+  TS_REQUIRE(a.dim % 8 == 0 && a.dim <= kSelCacheMaxVec * 256 * 8, TS_ESHAPE,
+             "ts_selcache_step: %d query elements per request (at most %d)", a.dim, kSelCacheMaxVec * 256 * 8);
   a.hit = hit;
   hipLaunchKernelGGL(selcache_kernel, dim3((unsigned)bt->batch), dim3(256), 0, (hipStream_t)stream, a);
   return check_launch("selcache_kernel");
