@@ -675,7 +675,7 @@ def test_kv_store(dev):
 
 @pytest.mark.parametrize("pool_kernel", [-1, 6])
 def test_score_vote_in_groups_of_requests(dev, pool_kernel):
-    """ts_score_vote (scores never in memory, the batch served in groups of requests)
+    """ts_score_vote (scores never in memory, the batch served in phases of requests)
     against the oracle's votes and against ts_score + ts_vote; ragged, with a dense
     request and a skipped one."""
     lens, ks = [3000, 777, 40, 1531, 2048, 900], [64] * 6

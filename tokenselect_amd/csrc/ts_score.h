@@ -7,10 +7,10 @@
 
 namespace ts {
 
-constexpr int kMaxPacked = 8;   // requests per phase of a packed launch of the votes-only form
-constexpr int kMaxPhases = 24;  // phases per packed launch
+constexpr int kMaxPacked = 8;   // requests per phase of a launch of the votes-only form
+constexpr int kMaxPhases = 24;  // phases per launch
 
-// One phase of a packed launch: `requests` requests from `first` on share the workgroups
+// One phase of a votes-only launch: `requests` requests from `first` on share the workgroups
 // [first_workgroup, next phase's first_workgroup) of the grid, request r owning those from
 // pack_first[r] on (relative to the phase).
 struct VotePhase {

@@ -88,16 +88,8 @@ constexpr int kScoreDirect = 0, kScoreTiled = 1, kScoreFused = 2;
 constexpr int kScorePacked = 3;
 constexpr int kMaxHeads = 128;
 
-// The softmax statistics of the fused kernel, without a rendezvous: every workgroup
-// publishes its per-head (max, sum exp) into a table that was zero at launch; the
-// (request, head) pairs are dealt out over all wavefronts of the team; a wavefront polls
-// the entries of its pair, a lane per chunk, until none is zero any more (a sum of
-// exponentials never is: the data is its own flag), merges them in a fixed order and
-// writes the result into 64 replicas, lane r into replica r.  The workgroups poll the
-// words of the replica of their index in the same way.  The wait is bounded like those
-// of the rendezvous: on giving up it sets the fault word and merges what is there.
 // What a workgroup of the fused kernel serves: the whole launch, or one phase of a
-// packed launch.
+// launch of the votes-only form.
 struct LaunchPart {
   int tokens_per_block;
   int batch_offset;       // first request
@@ -115,6 +107,14 @@ __device__ __forceinline__ int packed_chunks(const LaunchPart& lp, int r, int n)
   return min(chunks, lp.pack_first[r + 1] - lp.pack_first[r]);
 }
 
+// The softmax statistics of the fused kernel, without a rendezvous: every workgroup
+// publishes its per-head (max, sum exp) into a table that was zero at launch; the
+// (request, head) pairs are dealt out over all wavefronts of the team; a wavefront polls
+// the entries of its pair, a lane per chunk, until none is zero any more (a sum of
+// exponentials never is: the data is its own flag), merges them in a fixed order and
+// writes the result into 64 replicas, lane r into replica r.  The workgroups poll the
+// words of the replica of their index in the same way.  The wait is bounded like those
+// of the rendezvous: on giving up it sets the fault word and merges what is there.
 template <bool PACKED>
 __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const LaunchPart& lp,
                                                     const GridTeam& team, int lane, int wave) {
@@ -196,7 +196,7 @@ __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, const Lau
                                                    uint32_t* lds, int req, int chunk) {
   GridTeam team;
   if (PACKED) {
-    // A packed launch holds a handful of requests and its members are the workgroups
+    // A phase holds a handful of requests and its members are the workgroups
     // that hold candidates: every thread adds them up for itself.
     uint32_t before = 0, total = 0;
     for (int r = 0; r < lp.packed; ++r) {

@@ -422,7 +422,7 @@ def score_vote_supported(cfg: LayerConfig, batch: int, max_seq_len: int) -> bool
 def score_vote(cfg: LayerConfig, bt: Batch, qf: torch.Tensor, k_pool: torch.Tensor,
                skip: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):
     """:func:`score` + :func:`vote` without the scores in memory (``ts_score_vote``), a
-    batch of any size in groups of requests that fit the LDS of the device.  Returns
+    batch of any size, its requests in phases that fit the LDS of the device.  Returns
     ``votes [B, stride]`` fp32 (pooled when ``cfg.pool_kernel > 0``)."""
     c, cb = cfg.to_c(), _c_batch(cfg, bt)
     _need(qf, "qf", torch.bfloat16)
