@@ -749,6 +749,29 @@ def test_score_vote_phases_of_one_launch(dev, case, pool_kernel):
                 f"b={b} L={L} attempt={attempt}"
 
 
+@pytest.mark.parametrize("shape", SHAPES[1:], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+def test_score_vote_phases_head_shapes(dev, shape):
+    """The phased votes-only launch for the other head shapes (seven and eight query heads per
+    KV head run one workgroup per CU, one KV head streams 256-byte rows): 40 requests, five
+    phases, against ts_score + ts_vote."""
+    rnd = random.Random(9)
+    lens = [rnd.randrange(700, 6000) for _ in range(40)]
+    say(f"score_vote in phases: H={shape['num_heads']} kv={shape['num_kv_heads']}")
+    wl = small(dev, shape, seed=49, lens=lens, ks=[64] * 40, page=16, top_k=64)
+    c = wl.cfg
+    qf = fingerprint(wl, dev)
+    votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool))
+    for host in (None, torch.tensor(lens, dtype=torch.int32)):
+        bt = ops.Batch(wl.batch.seq_lens, wl.batch.table, max(lens), wl.batch.k_per_req, host_seq_lens=host)
+        votes = ops.score_vote(c, bt, qf, wl.k_pool)
+        torch.cuda.synchronize()
+        for b, L in enumerate(lens):
+            n = L - c.n_init - c.n_local
+            want = votes_sep[b, :n]
+            assert (votes[b, :n] - want).abs().max().item() <= 1e-5 * want.abs().max().item(), \
+                f"b={b} L={L} host lengths: {host is not None}"
+
+
 def test_score_vote_reports_a_length_above_its_bound(dev):
     """host_seq_lens are upper bounds; a request that is longer on the device than the host
     said has no workgroups for its last tokens.  The launch says so at once (the caller's
