@@ -67,26 +67,62 @@ __device__ __forceinline__ uint32_t key_bin2(uint32_t key) { return key & 1023u;
 // count(bins > t) < need <= count(bins >= t).  `hist` has NB entries (global or
 // LDS) per copy, NB a multiple of blockDim.x; COPIES consecutive copies are added
 // up.  Returns t and count(bins > t) to every thread.  `scratch` is LDS of
-// blockDim.x/64 + 2 words.
-template <int NB, int COPIES = 1>
-__device__ __forceinline__ void find_threshold_bin(const uint32_t* hist, uint32_t need,
-                                                   uint32_t* scratch, uint32_t& t_out,
-                                                   uint32_t& above_out) {
-  const int tid = threadIdx.x, nthreads = blockDim.x;
+// blockDim.x/64 + 2 words.  VECTOR: the number of threads of the workgroup, given at
+// compile time when `hist` is 16-byte aligned global memory (vector loads).
+// The search comes in two halves, so that a caller can request the bins of several
+// histograms (and whatever else it needs from memory) before it searches the first: the
+// searches end in barriers that later loads would wait behind.
+template <int NB, int COPIES = 1, int VECTOR = 0>
+__device__ __forceinline__ void load_threshold_bins(const uint32_t* hist, uint32_t (&local)[8]) {
+  const int tid = threadIdx.x, nthreads = VECTOR ? VECTOR : (int)blockDim.x;
   const int per = NB / nthreads;  // bins per thread, thread 0 owns the highest bins
+  const int hi_bin = NB - 1 - tid * per;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) local[i] = 0;
+  if (VECTOR && (per == 8 || per == 4 || per == 2)) {
+    // The thread's bins as one or two aligned vector loads (ascending addresses, taken in
+    // descending order below): eight separate loads per thread, each wave instruction
+    // strided over 2 KB, made this search 5 us of the top-k mark kernel.
+#pragma unroll
+    for (int c = 0; c < COPIES; ++c) {
+      const uint32_t* base = hist + c * NB + (NB - (tid + 1) * per);
+      uint32_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (per == 8) {
+        const uint4 a = ((const uint4*)base)[0], b = ((const uint4*)base)[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+      } else if (per == 4) {
+        const uint4 a = ((const uint4*)base)[0];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+      } else {
+        const uint2 a = ((const uint2*)base)[0];
+        v[0] = a.x; v[1] = a.y;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (i < per) local[i] += v[per - 1 - i];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (i < per) {
+#pragma unroll
+        for (int c = 0; c < COPIES; ++c) local[i] += hist[c * NB + hi_bin - i];
+      }
+  }
+}
+
+template <int NB, int VECTOR = 0>
+__device__ __forceinline__ void search_threshold_bins(const uint32_t (&local)[8], uint32_t need,
+                                                      uint32_t* scratch, uint32_t& t_out,
+                                                      uint32_t& above_out) {
+  const int tid = threadIdx.x, nthreads = VECTOR ? VECTOR : (int)blockDim.x;
+  const int per = NB / nthreads;
   const int lane = tid & 63, wave = tid >> 6, nwaves = nthreads >> 6;
   const int hi_bin = NB - 1 - tid * per;
-  uint32_t local[8];
   uint32_t mine = 0;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    local[i] = 0;
-    if (i < per) {
-#pragma unroll
-      for (int c = 0; c < COPIES; ++c) local[i] += hist[c * NB + hi_bin - i];
-      mine += local[i];
-    }
-  }
+  for (int i = 0; i < 8; ++i)
+    if (i < per) mine += local[i];
   // exclusive prefix of `mine` over threads (descending bins)
   uint32_t incl = mine;
 #pragma unroll
@@ -119,6 +155,15 @@ __device__ __forceinline__ void find_threshold_bin(const uint32_t* hist, uint32_
   t_out = scratch[nwaves];
   above_out = scratch[nwaves + 1];
   __syncthreads();
+}
+
+template <int NB, int COPIES = 1, int VECTOR = 0>
+__device__ __forceinline__ void find_threshold_bin(const uint32_t* hist, uint32_t need,
+                                                   uint32_t* scratch, uint32_t& t_out,
+                                                   uint32_t& above_out) {
+  uint32_t local[8];
+  load_threshold_bins<NB, COPIES, VECTOR>(hist, local);
+  search_threshold_bins<NB, VECTOR>(local, need, scratch, t_out, above_out);
 }
 
 size_t topk_ws_stride_words(int max_n);

@@ -69,22 +69,38 @@ __global__ __launch_bounds__(256) void topk_mark_kernel(TopkArgs a) {
   __shared__ uint32_t scratch[8];
   __shared__ uint32_t lh[kTopkBins];
   uint32_t* ws = topk_ws(a.ws, a.ws_stride, b);
+  // The votes of the slice are requested together with the histogram: they arrive while
+  // the threshold bin is searched for.
+  const float* votes = a.votes + (int64_t)b * a.vote_stride;
+  const int lane = threadIdx.x & 63;
+  const int first = lo + (threadIdx.x & ~63);
+  const int end = min(lo + a.slice, n);
+  constexpr int kAhead = 4096 / 256;  // passes of the largest slice
+  uint32_t bins0[8];
+  load_threshold_bins<kTopkBins, 1, 256>(ws + kTopkHist0, bins0);
+  float ahead[kAhead];
+#pragma unroll
+  for (int it = 0; it < kAhead; ++it) {
+    const int i = first + 256 * it + lane;
+    ahead[it] = (first + 256 * it < end && i < n) ? votes[i] : 0.f;
+  }
   uint32_t t0, above0;
-  find_threshold_bin<kTopkBins>(ws + kTopkHist0, (uint32_t)geo.k, scratch, t0, above0);
+  search_threshold_bins<kTopkBins, 256>(bins0, (uint32_t)geo.k, scratch, t0, above0);
   for (int i = threadIdx.x; i < kTopkBins; i += 256) lh[i] = 0u;
   __syncthreads();
 
-  const float* votes = a.votes + (int64_t)b * a.vote_stride;
   uint64_t* bitmap = (uint64_t*)(ws + kTopkCounterWords);
   uint2* cand = (uint2*)(ws + kTopkCounterWords + a.bitmap_words);
-  const int lane = threadIdx.x & 63;
   // Whole 64-position groups per wave iteration so that a bitmap word has one writer.
-  for (int base = lo + (threadIdx.x & ~63); base < min(lo + a.slice, n); base += 256) {
+#pragma unroll
+  for (int it = 0; it < kAhead; ++it) {
+    const int base = first + 256 * it;
+    if (base >= end) break;
     const int i = base + lane;
     uint32_t key = 0;
     bool gt = false, eq = false;
     if (i < n) {
-      key = vote_key(votes[i]);
+      key = vote_key(ahead[it]);
       const uint32_t bin = key_bin0(key);
       gt = bin > t0;
       eq = bin == t0;
@@ -165,6 +181,15 @@ __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs 
   __shared__ uint32_t scratch[kTopkFinalThreads / 64 + 2];
   __shared__ uint32_t lh[1024];
   __shared__ uint32_t lbits[kTopkPartWords];
+  // Both histograms are requested before anything else is waited for: the searches
+  // below end in barriers that their loads would otherwise queue behind.
+  uint32_t bins0[8], bins1[8];
+  load_threshold_bins<kTopkBins, 1, kTopkFinalThreads>(ws + kTopkHist0, bins0);
+  load_threshold_bins<kTopkBins, 1, kTopkFinalThreads>(ws + kTopkHist1, bins1);
+  // ... and this thread's first entry of the short list (the list rarely has more entries
+  // than the workgroup has threads; one past its end is never used).
+  const uint2 cand_first = (uint32_t)tid < a.cand_cap ? cand[tid] : make_uint2(0u, 0u);
+  auto cand_at = [&](int i) { return i == tid ? cand_first : cand[i]; };
   uint32_t before = 0;  // selected positions before the slice, this thread's share
   for (int w = tid; w < w_lo; w += kTopkFinalThreads) before += __popc(bitmap32[w]);
   for (int w = w_lo + tid; w < w_hi; w += kTopkFinalThreads) {
@@ -182,15 +207,15 @@ __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs 
   };
 
   uint32_t t0, above0, t1, above1, t2, above2;
-  find_threshold_bin<kTopkBins>(ws + kTopkHist0, (uint32_t)k, scratch, t0, above0);
+  search_threshold_bins<kTopkBins, kTopkFinalThreads>(bins0, (uint32_t)k, scratch, t0, above0);
   const uint32_t need1 = (uint32_t)k - above0;  // still to take inside bin t0
-  find_threshold_bin<kTopkBins>(ws + kTopkHist1, need1, scratch, t1, above1);
+  search_threshold_bins<kTopkBins, kTopkFinalThreads>(bins1, need1, scratch, t1, above1);
   const uint32_t need2 = need1 - above1;  // still to take inside (t0, t1)
 
   for (int i = tid; i < 1024; i += kTopkFinalThreads) lh[i] = 0u;
   __syncthreads();
   for (int i = tid; i < ncand; i += kTopkFinalThreads) {
-    const uint2 c = cand[i];
+    const uint2 c = cand_at(i);
     const uint32_t b1 = key_bin1(c.x);
     if (b1 > t1)
       mark(c.y);
@@ -205,7 +230,7 @@ __global__ __launch_bounds__(kTopkFinalThreads) void topk_final_kernel(TopkArgs 
 
   if (count_eq == need_eq) {  // the usual case: every tie is selected
     for (int i = tid; i < ncand; i += kTopkFinalThreads) {
-      const uint2 c = cand[i];
+      const uint2 c = cand_at(i);
       if (key_bin1(c.x) == t1 && key_bin2(c.x) >= t2) mark(c.y);
     }
   } else {
