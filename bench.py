@@ -223,7 +223,9 @@ def bench_layer(args, ops, workloads, dev, which=None):
         "config": {"workload": wl.name, "batch": B, "seq_lens_max": max(wl.seq_lens),
                    "page_size": c.page_size, "top_k": c.top_k, "n_init": c.n_init,
                    "n_local": c.n_local, "kv_pool_copies": n_pools,
-                   "lengths_on_host_too": bool(wl.host_lengths)},
+                   "lengths_on_host_too": bool(wl.host_lengths),
+                   "selection": {2: "ts_select", 1: "ts_score_vote + top-k kernels",
+                                 0: "ts_score + ts_vote + top-k kernels"}[ops.layer_selection_form(c, bt)]},
         "tokens_per_s": round(B / (us_per_layer * 1e-6 * args.layers), 1),
         "tokens_per_s_note": f"selection+attention only, {args.layers} layers per token",
         "roofline": roofline, "score_only": score_only, "gather_attention": attn,
@@ -590,6 +592,8 @@ def main():
     ap.add_argument("--prefill-rows", type=int, default=512, help="rows of the prefill chunk")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run five 256 MiB device copies (reference for counter runs)")
+    ap.add_argument("--separate-kernels", action="store_true",
+                    help="ts_set_fused_select(0): the selection as ts_score + ts_vote + the top-k kernels")
     args = ap.parse_args()
     if args.steps is None:
         args.steps = 128 if args.workload == "model" else 200
@@ -604,6 +608,8 @@ def main():
     from tokenselect_amd import ops, workloads
 
     dev = torch.device("cuda:0")
+    if args.separate_kernels:
+        ops.set_fused_select(False)
     if args.workload == "c4":
         result = bench_trace(args, ops, workloads, dev)
     elif args.workload == "prefill":
