@@ -94,7 +94,7 @@ typedef struct ts_batch {
                                packed by these bounds instead of by
                                max_seq_len, which saves the workgroups that
                                would find no candidates (16 requests of
-                               4K..128K: 447 instead of 461 us per layer).
+                               4K..128K: 439 instead of 453 us per layer).
                                The device's seq_lens[] still rule; a bound
                                below the device's value is the caller's error:
                                the tokens beyond it are not scored, and the
