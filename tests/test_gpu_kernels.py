@@ -772,6 +772,41 @@ def test_score_vote_phases_head_shapes(dev, shape):
                 f"b={b} L={L} host lengths: {host is not None}"
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_score_vote_randomised(dev, seed):
+    """Random batches through the phased votes-only launch against ts_score + ts_vote: 1 to 40
+    requests of 30 to 30 000 tokens (some dense), random slack in the host's bounds or no
+    bounds at all, random skip flags, with or without max-pooling, one of the head shapes."""
+    rnd = random.Random(7000 + seed)
+    shape = SHAPES[rnd.randrange(len(SHAPES))]
+    B = rnd.randrange(1, 41)
+    lens = [rnd.choice([rnd.randrange(30, 300), rnd.randrange(300, 4000), rnd.randrange(4000, 30000)])
+            for _ in range(B)]
+    pool_kernel = rnd.choice([-1, -1, 3, 6])
+    say(f"score_vote randomised seed={seed} H={shape['num_heads']} kv={shape['num_kv_heads']} B={B} "
+        f"pool={pool_kernel}")
+    wl = small(dev, shape, seed=7100 + seed, lens=lens, ks=[32] * B, page=rnd.choice([1, 16]), top_k=32,
+               pool_kernel=pool_kernel)
+    c = wl.cfg
+    qf = fingerprint(wl, dev)
+    skip = torch.tensor([1 if rnd.random() < 0.15 else 0 for _ in range(B)], dtype=torch.int32, device=dev)
+    host = None
+    if rnd.random() < 0.7:
+        host = torch.tensor([min(L + rnd.choice([0, 0, 5, 900]), max(lens)) for L in lens], dtype=torch.int32)
+    bt = ops.Batch(wl.batch.seq_lens, wl.batch.table, max(lens), wl.batch.k_per_req, host_seq_lens=host)
+    votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool, skip=skip), skip=skip)
+    votes = ops.score_vote(c, bt, qf, wl.k_pool, skip=skip)
+    torch.cuda.synchronize()
+    for b, L in enumerate(lens):
+        n = L - c.n_init - c.n_local
+        if pool_kernel > 0 and pool_kernel % 2 == 0:
+            n -= 1
+        if L <= c.n_init + 32 + c.n_local or skip[b] or n <= 0:   # dense or skipped: no votes are taken
+            continue
+        want = votes_sep[b, :n]
+        assert (votes[b, :n] - want).abs().max().item() <= 1e-5 * want.abs().max().item(), f"b={b} L={L}"
+
+
 def test_score_vote_reports_a_length_above_its_bound(dev):
     """host_seq_lens are upper bounds; a request that is longer on the device than the host
     said has no workgroups for its last tokens.  The launch says so at once (the caller's

@@ -1209,6 +1209,13 @@ static int fused_capacity(const ts_config* cfg, bool packed = false) {
   return capacity;
 }
 
+// With max-pooling a workgroup gathers its votes and kernel - 1 neighbours into the LDS
+// array of the histogram (kTopkBins words): the most tokens a workgroup may take then.
+static int pooling_tokens_cap(const ts_config* cfg) {
+  if (cfg->pool_kernel <= 0) return 1 << 30;
+  return (kTopkBins - (cfg->pool_kernel - 1)) / 64 * 64;
+}
+
 int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch) {
   // Max-pool windows beyond 256 would not fit the LDS the neighbours are gathered into.
   if ((!ignore_switch && !g_fused_select.load()) || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256)
@@ -1220,7 +1227,7 @@ int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, boo
 
   int tpb = score_tokens_per_block((int64_t)batch * max_seq_len, cfg->num_heads);
   while ((int64_t)ceil_div(max_n, tpb) * batch > capacity) tpb += 64;
-  if (fused_lds_bytes(tpb, cfg->num_heads) > kFusedStageBytes)
+  if (fused_lds_bytes(tpb, cfg->num_heads) > kFusedStageBytes || tpb > pooling_tokens_cap(cfg))
     return 0;
   if (ceil_div(max_seq_len, tpb) > kSelMaxChunks) return 0;  // what the workspace is laid out for
   return tpb;
@@ -1443,7 +1450,9 @@ bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan
   const int capacity = fused_capacity(cfg, /*packed=*/true);
   if (capacity <= 0) return false;
   int tpb_max = 64;
-  while (fused_lds_bytes(tpb_max + 64, cfg->num_heads) <= kFusedStageBytes) tpb_max += 64;
+  while (fused_lds_bytes(tpb_max + 64, cfg->num_heads) <= kFusedStageBytes &&
+         tpb_max + 64 <= pooling_tokens_cap(cfg))
+    tpb_max += 64;
   if (fused_lds_bytes(tpb_max, cfg->num_heads) > kFusedStageBytes) return false;
   const int fixed = cfg->n_init + cfg->n_local;
   auto bound = [&](int b) { return bt->host_seq_lens ? std::min(bt->host_seq_lens[b], bt->max_seq_len) : bt->max_seq_len; };
