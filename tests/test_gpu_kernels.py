@@ -580,6 +580,34 @@ def test_decode_layer(dev, shape, page, fused_select):
     check_layer(wl, dev, "decode_layer")
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_decode_layer_randomised(dev, seed):
+    """Random batches through ts_decode_layer against the oracle, whatever form the layer
+    takes for them (one selection launch, the phased votes-only launch + top-k kernels, the
+    separate kernels): 1 to 14 requests of 40 to 40 000 tokens, ragged k, any head shape,
+    pages of 1 or 16, lengths on the host too or not, with or without max-pooling."""
+    rnd = random.Random(9000 + seed)
+    shape = SHAPES[rnd.randrange(len(SHAPES))]
+    B = rnd.randrange(1, 15)
+    lens = [rnd.choice([rnd.randrange(40, 400), rnd.randrange(400, 6000), rnd.randrange(6000, 40000)])
+            for _ in range(B)]
+    top_k = rnd.choice([16, 64, 256])
+    ks = [rnd.randrange(1, top_k + 1) for _ in range(B)]
+    pool_kernel = rnd.choice([-1, -1, 5, 8])
+    fused = rnd.random() < 0.8
+    wl = small(dev, shape, seed=9100 + seed, lens=lens, ks=ks, page=rnd.choice([1, 16]), top_k=top_k,
+               n_init=rnd.choice([4, 16]), n_local=rnd.choice([8, 32]), pool_kernel=pool_kernel)
+    wl.host_lengths = rnd.random() < 0.5
+    previous = ops.set_fused_select(fused)
+    try:
+        form = ops.layer_selection_form(wl.cfg, wl.batch)
+        say(f"decode_layer randomised seed={seed} H={shape['num_heads']} kv={shape['num_kv_heads']} B={B} "
+            f"tokens={sum(lens)} pool={pool_kernel} host_lengths={wl.host_lengths} form={form}")
+        check_layer(wl, dev, f"randomised layer seed={seed}")
+    finally:
+        ops.set_fused_select(previous)
+
+
 @pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
 def test_decode_layer_object_serves_smaller_batches(dev, fused_select):
     """A layer object sized for the largest batch and context is called with batches of
