@@ -64,6 +64,41 @@ def test_sparse_prefill_attention(dev, shape, rope_mode):
     assert err <= 2e-2, err
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_sparse_prefill_attention_randomised(dev, seed):
+    """Random chunk sizes, selection lengths and head shapes through the causal attention
+    (its key tiles are streamed by four groups of wavefronts that hand buffers to each
+    other through counters: every length is another pattern of full, partial and missing
+    rounds), with or without the rotation and the soft cap, scaled queries so that the
+    running maximum moves.  Within 2e-2 plus two bf16 units of the reference value: the
+    rotated keys and the softmax weights enter the matrix products as bf16, which shows
+    in outputs above one when doubled queries make the softmax peaked."""
+    import random
+    rnd = random.Random(4000 + seed)
+    shape = SHAPES[rnd.randrange(len(SHAPES))]
+    m = rnd.choice([rnd.randrange(1, 17), rnd.randrange(17, 200), rnd.randrange(200, 513)])
+    S = m + rnd.choice([0, rnd.randrange(0, 40), rnd.randrange(40, 700), rnd.randrange(700, 2800)])
+    rope_mode = rnd.choice(["ROPE_LLAMA", "ROPE_LLAMA", "NONE"])
+    cap = rnd.choice([0.0, 0.0, 30.0])
+    say(f"prefill attention randomised seed={seed} H={shape['num_heads']} kv={shape['num_kv_heads']} "
+        f"m={m} S={S} {rope_mode} cap={cap}")
+    wl = workloads.build("pf", shape, [S + 50], [64], 1, dev, seed=4100 + seed, n_init=8, n_local=m)
+    c = wl.cfg
+    c.rope_mode, c.logit_cap = rope_mode, cap
+    g = torch.Generator(device=dev).manual_seed(4200 + seed)
+    q = (torch.randn((m, c.num_heads * 128), generator=g, device=dev) * rnd.choice([0.3, 1.0, 2.0])).bfloat16()
+    sel = wl.table[0, torch.randperm(S + 50, generator=g, device=dev)[:S].long()].contiguous()
+    sel_len = torch.tensor([S], dtype=torch.int32, device=dev)
+    out = ops.sparse_prefill_attention(c, q, wl.k_pool, wl.v_pool, sel, sel_len)
+    torch.cuda.synchronize()
+    ref = oracle.prefill.sparse_prefill_attention(q.cpu().view(m, c.num_heads, 128), wl.k_pool.cpu(),
+                                                  wl.v_pool.cpu(), sel.cpu(), _sm(c), c.rope_theta,
+                                                  c.rope_scale, c.logit_cap, rope_mode)
+    ref = ref.reshape(m, -1).float()
+    excess = ((out.cpu().float() - ref).abs() - (2e-2 + 2.0 ** -6 * ref.abs())).max().item()
+    assert excess <= 0.0, excess
+
+
 def test_sparse_prefill_attention_full_chunk_and_soft_cap(dev):
     """A whole 512-row chunk over the selected-list length of the served configs, the
     chunk starting exactly at S - m; and the soft cap."""
