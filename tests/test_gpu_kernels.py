@@ -527,6 +527,46 @@ def test_sparse_attention(dev, shape, rope_mode):
         assert err <= 2e-2, f"attention b={b}: max abs err {err}"
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_sparse_attention_randomised(dev, seed):
+    """Random batches and ragged list lengths through the decode attention: one pass or
+    several per workgroup, one round of workgroups, requests with empty and with one-entry
+    lists, any head shape, with or without the rotation and the soft cap; every replay of
+    the same call bit-identical (the splits are merged in a fixed order)."""
+    rnd = random.Random(6000 + seed)
+    shape = SHAPES[rnd.randrange(len(SHAPES))]
+    B = rnd.choice([1, 2, rnd.randrange(3, 9), rnd.randrange(9, 25)])
+    max_sel = rnd.choice([rnd.randrange(1, 130), rnd.randrange(130, 1500), rnd.randrange(1500, 5000)])
+    lens = [rnd.choice([max_sel, rnd.randrange(0, max_sel + 1), rnd.randrange(0, max_sel + 1), 1]) for _ in range(B)]
+    lens[rnd.randrange(B)] = max_sel
+    rope_mode = rnd.choice(["ROPE_LLAMA", "ROPE_LLAMA", "NONE"])
+    cap = rnd.choice([0.0, 0.0, 20.0])
+    say(f"attention randomised seed={seed} H={shape['num_heads']} kv={shape['num_kv_heads']} B={B} "
+        f"max_sel={max_sel} {rope_mode} cap={cap}")
+    wl = small(dev, shape, seed=6100 + seed, lens=[3000] * B, ks=[64] * B)
+    c = wl.cfg
+    c.rope_mode, c.logit_cap = rope_mode, cap
+    g = torch.Generator().manual_seed(6200 + seed)
+    sel = torch.zeros((B, max_sel), dtype=torch.int32)
+    for b, S in enumerate(lens):
+        sel[b, :S] = torch.randint(0, wl.k_pool.shape[0], (S,), generator=g).int()
+    sel_len = torch.tensor(lens, dtype=torch.int32)
+    out = ops.sparse_decode_attention(c, wl.q, wl.k_pool, wl.v_pool, sel.to(dev), sel_len.to(dev)).clone()
+    again = ops.sparse_decode_attention(c, wl.q, wl.k_pool, wl.v_pool, sel.to(dev), sel_len.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), again.view(torch.int16))
+    kc, vc, qc = wl.k_pool.cpu(), wl.v_pool.cpu(), wl.q.cpu()
+    for b, S in enumerate(lens):
+        if S == 0:      # an empty list attends to nothing: the output is defined as zero
+            assert not bool(out[b].any()), f"b={b}: empty list"
+            continue
+        ref = oracle.attend.sparse_decode_attention(
+            qc[b].view(c.num_heads, 128), kc, vc, sel[b, :S], 128 ** -0.5, c.rope_theta, 1.0, cap,
+            rope_mode)
+        err = (out[b].cpu().float() - ref.reshape(-1).float()).abs().max().item()
+        assert err <= 2e-2, f"attention b={b} S={S}: max abs err {err}"
+
+
 def test_attention_soft_cap(dev):
     say("attention logit_cap=30")
     wl = small(dev, SHAPES[0], seed=12, lens=[500], ks=[64])
