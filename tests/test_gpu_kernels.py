@@ -527,6 +527,47 @@ def test_sparse_attention(dev, shape, rope_mode):
         assert err <= 2e-2, f"attention b={b}: max abs err {err}"
 
 
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+def test_selection_cache_decisions(dev, shape):
+    """ts_selcache_step on its own, every head shape (4 to 32 heads: one to four 16-byte
+    pieces of the query per thread): queries at chosen cosines to the cached one on both sides
+    of the threshold, decisions, cached queries and counters against the oracle's state
+    machine over twelve steps."""
+    say(f"selection cache decisions H={shape['num_heads']}")
+    B = 6
+    wl = small(dev, shape, seed=57, lens=[3000] * B, ks=[64] * B)
+    c = wl.cfg
+    dim = c.num_heads * c.head_dim
+    cache = ops.SelectionCache.allocate(c, B, dev)
+    refs = [oracle.selcache.SelectionCache() for _ in range(B)]
+    g = torch.Generator().manual_seed(58)
+    base = torch.randn(B, dim, generator=g)
+    for step in range(12):
+        # a mix of the anchor direction and a fresh one: cosines from -0.2 to 1.0, several near 0.9
+        mix = torch.tensor([1.0, 0.95, 0.9, 0.88, 0.5, -0.2])[torch.randperm(B, generator=g)]
+        fresh = torch.randn(B, dim, generator=g)
+        fresh -= (fresh * base).sum(1, keepdim=True) / (base * base).sum(1, keepdim=True) * base
+        fresh *= base.norm(dim=1, keepdim=True) / fresh.norm(dim=1, keepdim=True)
+        qf = (mix[:, None] * base + (1 - mix[:, None] ** 2).clamp_min(0).sqrt() * fresh).bfloat16()
+        hit = ops.selcache_step(c, wl.batch, qf.to(dev), cache)
+        # (a miss stores the query; the selection that would fill cache_len is stood in for)
+        cache.cache_len.copy_(torch.full((B,), 64, dtype=torch.int32))
+        torch.cuda.synchronize()
+        for b in range(B):
+            before = refs[b].q_cached
+            cos = None if before is None else oracle.selcache.cosine(before.float(), qf[b].float())
+            _, ref_hit = refs[b].step(qf[b], lambda: torch.zeros(1))
+            if cos is not None and abs(cos - refs[b].threshold) < 1e-4:
+                refs[b].q_cached = cache.q_cache[b].cpu().clone()   # too close to call: follow the device
+                refs[b].skip_count = int(cache.counters[b, 0])
+            else:
+                assert bool(hit[b]) == ref_hit, f"step {step} b={b} cosine {cos}"
+                assert torch.equal(cache.q_cache[b].cpu(), refs[b].q_cached), f"step {step} b={b}: cached query"
+                assert int(cache.counters[b, 0]) == refs[b].skip_count
+            base[b] = cache.q_cache[b].cpu().float()    # the anchor: the query of the last miss
+        assert cache.counters[:, 1].tolist() == [step + 1] * B
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_sparse_attention_randomised(dev, seed):
     """Random batches and ragged list lengths through the decode attention: one pass or
