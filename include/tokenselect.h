@@ -5,7 +5,9 @@
  * Every entry point takes plain pointers and sizes.  All data pointers are
  * device pointers unless a parameter says "host".  bf16 tensors are passed as
  * `const void*` (16-bit brain floats, row-major, innermost dimension
- * contiguous).  Launches are asynchronous on the given HIP stream; the library
+ * contiguous).  Tensors and KV pools must be aligned to 16 bytes, workspaces to
+ * 256 (what hipMalloc and the framework allocators give; a view at an odd
+ * offset is refused with TS_EINVAL).  Launches are asynchronous on the given HIP stream; the library
  * never synchronises and never allocates device memory.  Its only mutable
  * process-wide state is the ts_set_fused_select() switch (and the built-in
  * scratch buffer of ts_sparse_decode_attn_static); everything else lives in the

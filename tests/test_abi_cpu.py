@@ -126,6 +126,26 @@ def test_null_and_range_errors_need_no_gpu(lib):
     assert "workspace" in err(lib)
 
 
+def test_misaligned_buffers_are_refused_on_the_host(lib):
+    """Tensors are read with 16-byte vector loads and workspaces hold 8-byte atomics: a view at
+    an odd offset fails the call instead of faulting the device."""
+    c = cfg()
+    one, odd = ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1004)
+    bt = _lib.TsBatch(1, 4096, one, one, 4096, None)
+    big = 1 << 30
+    assert lib.ts_score_vote(ctypes.byref(c), ctypes.byref(bt), one, odd, 10, None, one, 4096, one, big,
+                             None) == _lib.TS_EINVAL
+    assert "k_pool must be aligned" in err(lib)
+    assert lib.ts_score_vote(ctypes.byref(c), ctypes.byref(bt), one, one, 10, None, one, 4096,
+                             ctypes.c_void_p(0x1010), big, None) == _lib.TS_EINVAL
+    assert "workspace must be aligned to 256" in err(lib)
+    assert lib.ts_topk_ragged(ctypes.byref(c), ctypes.byref(bt), one, 4096, None, None, one, one, 4096,
+                              one, ctypes.c_void_p(0x1008), big, None) == _lib.TS_EINVAL
+    assert lib.ts_sparse_decode_attn(ctypes.byref(c), odd, one, one, 10, one, 4096, one, 1, 2688,
+                                     one, one, big, None) == _lib.TS_EINVAL
+    assert "q must be aligned" in err(lib)
+
+
 def test_static_scratch_entry_point_rejects_what_does_not_fit(lib):
     assert lib.ts_attn_static_scratch_bytes() == 4 << 20
     one = ctypes.c_void_p(0x1000)  # never dereferenced: the size check fails first

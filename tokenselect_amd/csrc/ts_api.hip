@@ -201,6 +201,11 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);
+  TS_REQUIRE_ALIGNED(workspace, 256, "workspace");
+  TS_REQUIRE_ALIGNED(q, 16, "q");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
+  TS_REQUIRE_ALIGNED(out, 16, "out");
   // The tie-break of the ragged top-k orders positions by two 10-bit digits.
   TS_REQUIRE(bt->max_seq_len - cfg->n_init - cfg->n_local <= (1 << 20), TS_ESHAPE,
              "layer: at most 2^20 candidates per request (max_seq_len %d)", bt->max_seq_len);
@@ -302,6 +307,9 @@ int ts_decode_layer_votes(const ts_config* cfg, const ts_batch* bt, const void* 
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
   TS_REQUIRE(q && q_cos && q_sin && k_pool && votes, TS_EINVAL, "layer votes: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(workspace, 256, "workspace");
+  TS_REQUIRE_ALIGNED(q, 16, "q");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   const LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);
@@ -345,6 +353,11 @@ int ts_decode_layer_attend(const ts_config* cfg, const ts_batch* bt, const void*
   TS_TRY(validate_batch(cfg, bt));
   TS_REQUIRE(q && votes && k_pool && v_pool && out && sel && sel_pos && sel_len, TS_EINVAL,
              "layer attend: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(workspace, 256, "workspace");
+  TS_REQUIRE_ALIGNED(q, 16, "q");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
+  TS_REQUIRE_ALIGNED(out, 16, "out");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   const LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);

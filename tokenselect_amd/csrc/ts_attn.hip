@@ -558,6 +558,11 @@ int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_poo
   const size_t need = ts_attn_workspace_bytes(cfg, batch, max_sel_len);
   TS_REQUIRE(workspace != nullptr && workspace_bytes >= need, TS_EWORKSPACE,
              "ts_sparse_decode_attn: workspace %zu bytes < required %zu", workspace_bytes, need);
+  TS_REQUIRE_ALIGNED(workspace, 256, "workspace");
+  TS_REQUIRE_ALIGNED(q, 16, "q");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
+  TS_REQUIRE_ALIGNED(out, 16, "out");
   return launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, batch, max_sel_len,
                      out, workspace, /*tickets_clear=*/false, (hipStream_t)stream);
 }

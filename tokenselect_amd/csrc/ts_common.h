@@ -26,6 +26,13 @@ bool group_supported(int num_kv_heads, int group);
     if (_rc != TS_OK) return _rc; \
   } while (0)
 
+// Device buffers are read and written with 16-byte vector accesses and 8-byte atomics:
+// what hipMalloc and the framework allocators return is aligned far beyond that, a view
+// at an odd offset is not, and would fault the device instead of failing a call.
+#define TS_REQUIRE_ALIGNED(ptr, bytes, what)                                                   \
+  TS_REQUIRE((reinterpret_cast<uintptr_t>(ptr) & ((bytes)-1)) == 0, TS_EINVAL,                  \
+             "%s must be aligned to %d bytes", what, (int)(bytes))
+
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

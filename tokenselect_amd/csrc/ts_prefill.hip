@@ -792,6 +792,11 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
   const size_t need = ts_prefill_attn_workspace_bytes(cfg, max_sel_len);
   TS_REQUIRE(workspace != nullptr && workspace_bytes >= need, TS_EWORKSPACE,
              "ts_sparse_prefill_attn: workspace %zu bytes < required %zu", workspace_bytes, need);
+  TS_REQUIRE_ALIGNED(workspace, 256, "workspace");
+  TS_REQUIRE_ALIGNED(q, 16, "q");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
+  TS_REQUIRE_ALIGNED(out, 16, "out");
   PrefillArgs a;
   a.q = (const uint16_t*)q;
   a.k_pool = (const uint16_t*)k_pool;

@@ -1583,6 +1583,10 @@ int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const voi
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
   TS_REQUIRE(qf && k_pool && scores && partials, TS_EINVAL, "ts_score: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(qf, 16, "qf");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(scores, 16, "scores");
+  TS_REQUIRE_ALIGNED(partials, 16, "partials");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   const int max_n = bt->max_seq_len - cfg->n_init - cfg->n_local;
@@ -1615,6 +1619,9 @@ int ts_score_vote(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
   TS_REQUIRE(qf && k_pool && votes && workspace, TS_EINVAL, "ts_score_vote: NULL argument");
+  TS_REQUIRE_ALIGNED(workspace, 256, "workspace");
+  TS_REQUIRE_ALIGNED(qf, 16, "qf");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   TS_REQUIRE(ts_score_vote_supported(cfg, bt->batch, bt->max_seq_len), TS_ESHAPE,
@@ -1651,6 +1658,7 @@ static int check_select(const ts_config* cfg, const ts_batch* bt, const void* wo
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
   TS_REQUIRE(workspace != nullptr, TS_EINVAL, "ts_select: NULL workspace");
+  TS_REQUIRE_ALIGNED(workspace, 256, "workspace");
   const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len);
   TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE,
              "ts_select: batch %d x %d tokens does not fit one co-resident grid (or pool_kernel is "
@@ -1683,6 +1691,8 @@ int ts_select_cleared_bounded(const ts_config* cfg, const ts_batch* bt, const vo
              (unsigned long long)wait_ticks, absent_workgroups);
   TS_TRY(check_select(cfg, bt, workspace, workspace_bytes, &w));
   TS_REQUIRE(qf && k_pool && sel && sel_pos && sel_len, TS_EINVAL, "ts_select: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(qf, 16, "qf");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   const int max_sel = cfg->n_init + cfg->top_k + cfg->n_local;
@@ -1725,6 +1735,8 @@ int ts_paged_matmul(const void* query, const void* token, int64_t pool_rows,
                     int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
                     ts_stream_t stream) {
   TS_REQUIRE(query && token && indices && scores, TS_EINVAL, "ts_paged_matmul: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(query, 16, "query");
+  TS_REQUIRE_ALIGNED(token, 16, "token");
   TS_REQUIRE(head_dim == kHeadDim, TS_ESHAPE, "head_dim %d not supported (only 128)", head_dim);
   TS_REQUIRE(num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0, TS_ESHAPE,
              "num_heads %d / num_kv_heads %d invalid", num_heads, num_kv_heads);

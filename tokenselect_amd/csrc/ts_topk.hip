@@ -433,6 +433,7 @@ int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
   const size_t need = ts_topk_workspace_bytes(cfg, bt->batch, bt->max_seq_len);
   TS_REQUIRE(workspace != nullptr && workspace_bytes >= need, TS_EWORKSPACE,
              "ts_topk_ragged: workspace %zu bytes < required %zu", workspace_bytes, need);
+  TS_REQUIRE_ALIGNED(workspace, 256, "workspace");
   const TopkArgs a = make_topk_args(cfg, bt, votes, vote_stride, hit, cache, sel, sel_pos,
                                     sel_stride, sel_len, (uint32_t*)workspace);
   return launch_topk(a, bt->batch, max_n, (hipStream_t)stream);
