@@ -144,6 +144,18 @@ def test_misaligned_buffers_are_refused_on_the_host(lib):
     assert lib.ts_sparse_decode_attn(ctypes.byref(c), odd, one, one, 10, one, 4096, one, 1, 2688,
                                      one, one, big, None) == _lib.TS_EINVAL
     assert "q must be aligned" in err(lib)
+    # the stores and the projection: rows are copied as 16-byte vectors
+    assert lib.ts_kv_store(ctypes.byref(c), one, odd, one, None, one, one, 10, one, 4096, one, 1, 4096,
+                           None) == _lib.TS_EINVAL
+    assert "v must be aligned" in err(lib)
+    assert lib.ts_kv_store_chunk(ctypes.byref(c), one, one, one, None, 4, one, odd, 10, one, one, 4096,
+                                 None) == _lib.TS_EINVAL
+    assert "v_pool must be aligned" in err(lib)
+    assert lib.ts_qkv_store(ctypes.byref(c), one, odd, None, 4096, one, None, one, one, one, 10, one,
+                            4096, one, 1, 4096, None) == _lib.TS_EINVAL
+    assert "w must be aligned" in err(lib)
+    assert lib.ts_fingerprint(ctypes.byref(c), odd, 4, one, one, 4096, one, one) == _lib.TS_EINVAL
+    assert "q must be aligned" in err(lib)
 
 
 def test_static_scratch_entry_point_rejects_what_does_not_fit(lib):

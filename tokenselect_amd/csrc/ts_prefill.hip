@@ -748,6 +748,9 @@ int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const 
                        hipStream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_REQUIRE(q && cos_table && sin_table && qf, TS_EINVAL, "ts_fingerprint: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(q, 16, "q");
+  TS_REQUIRE_ALIGNED(cos_table, 16, "cos_table");
+  TS_REQUIRE_ALIGNED(sin_table, 16, "sin_table");
   TS_REQUIRE(rows >= 1, TS_EINVAL, "ts_fingerprint: rows %d < 1", rows);
   TS_REQUIRE(table_rows >= (int64_t)cfg->n_local + rows, TS_EINVAL,
              "ts_fingerprint: cos/sin tables have %lld rows, need n_local + rows = %lld",

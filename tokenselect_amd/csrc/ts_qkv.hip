@@ -204,6 +204,11 @@ extern "C" int ts_qkv_store(const ts_config* cfg, const void* x, const void* w, 
   TS_TRY(validate_config(cfg));
   TS_REQUIRE(x && w && q_out && k_pool && v_pool && table && seq_lens, TS_EINVAL,
              "ts_qkv_store: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(x, 16, "x");
+  TS_REQUIRE_ALIGNED(w, 16, "w");
+  TS_REQUIRE_ALIGNED(q_out, 16, "q_out");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
   if (pages) {
     TS_REQUIRE(pages->free_pages && pages->free_count && pages->ticket, TS_EINVAL,
                "ts_qkv_store: page pool has a NULL array");

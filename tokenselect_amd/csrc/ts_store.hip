@@ -199,6 +199,10 @@ extern "C" int ts_kv_store(const ts_config* cfg, const void* k, const void* v,
   TS_TRY(validate_config(cfg));
   TS_REQUIRE(k && v && k_pool && v_pool && table && seq_lens, TS_EINVAL,
              "ts_kv_store: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(k, 16, "k");
+  TS_REQUIRE_ALIGNED(v, 16, "v");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
   TS_TRY(check_pool_arg(cfg, out_cache_loc, pages, "ts_kv_store"));
   TS_REQUIRE(batch >= 1 && pool_rows >= 1 && pool_rows <= 0x7fffffffLL && max_tokens >= 1, TS_EINVAL,
              "ts_kv_store: batch=%d pool_rows=%lld max_tokens=%d out of range", batch,
@@ -227,6 +231,10 @@ extern "C" int ts_kv_store_chunk(const ts_config* cfg, const void* k, const void
   TS_TRY(validate_config(cfg));
   TS_REQUIRE(k && v && k_pool && v_pool && table && seq_len, TS_EINVAL,
              "ts_kv_store_chunk: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(k, 16, "k");
+  TS_REQUIRE_ALIGNED(v, 16, "v");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
   TS_TRY(check_pool_arg(cfg, out_cache_loc, pages, "ts_kv_store_chunk"));
   TS_REQUIRE(rows >= 0 && pool_rows >= 1 && pool_rows <= 0x7fffffffLL && max_tokens >= 1, TS_EINVAL,
              "ts_kv_store_chunk: rows=%d pool_rows=%lld max_tokens=%d out of range", rows,
