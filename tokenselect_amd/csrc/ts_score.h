@@ -109,6 +109,7 @@ struct SelectWorkspace {
   int64_t pool_stride;
   int tokens_per_block;  // 0: the shape does not fit the fused kernel
   int blocks_per_req;
+  size_t lds_bytes;      // dynamic LDS of the launch (decides how many workgroups share a CU)
 };
 // ignore_switch: lay out as if ts_set_fused_select were on (for sizing a workspace that
 // must serve both settings).

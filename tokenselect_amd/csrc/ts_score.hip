@@ -1168,9 +1168,17 @@ static size_t fused_lds_bytes(int tokens_per_block, int num_heads) {
   return (size_t)(tokens_per_block / 16) * (16 * num_heads + 16) * sizeof(float);
 }
 
-// Dynamic LDS the fused form may use: with the 10 KB of static arrays, two
-// workgroups fit the 160 KB of a CU.
+// Dynamic LDS the fused form may use.  With the 10 KB of static arrays two workgroups
+// of 68 KB fit the 160 KB of a CU; a workgroup of up to 140 KB has the CU to itself and
+// takes twice the tokens.  Half as many workgroups make every hand-off between them
+// cheaper (arrivals counted, readers of one line, adds to one histogram line), and four
+// wavefronts per CU still keep enough loads in flight for the stream; but a request
+// that is skipped or short leaves its CUs idle, and there are half as many to share.
+// So the large workgroups serve where one request takes more than half of the device.
 constexpr size_t kFusedStageBytes = 68 * 1024;
+constexpr size_t kFusedLargeStageBytes = 140 * 1024;
+constexpr size_t kFusedLargeFloorBytes = 76 * 1024;  // more than half a CU's LDS: one workgroup per CU
+static size_t fused_stage_bytes(bool large) { return large ? kFusedLargeStageBytes : kFusedStageBytes; }
 
 // The one process-wide switch of the library (ts_set_fused_select).
 static std::atomic<int> g_fused_select{1};
@@ -1179,24 +1187,25 @@ int set_fused_select(int enable) { return g_fused_select.exchange(enable ? 1 : 0
 
 // Workgroups of the fused kernel that the current device keeps resident at once (0: the
 // shape has no fused kernel, or the runtime refused); depends on the kernel only.
-static int fused_capacity(const ts_config* cfg, bool packed = false) {
+static int fused_capacity(const ts_config* cfg, bool packed, bool large) {
   const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads, packed);
   if (!fn) return 0;
-  struct Entry { const void* fn; int device; int capacity; };
-  static thread_local Entry memo[8] = {};
+  struct Entry { const void* fn; int device; bool large; int capacity; };
+  static thread_local Entry memo[16] = {};
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return 0;
   int capacity = 0;
   for (const Entry& e : memo)
-    if (e.fn == fn && e.device == device) capacity = e.capacity;
+    if (e.fn == fn && e.device == device && e.large == large) capacity = e.capacity;
   if (capacity == 0) {
     int per_cu = 0, cus = 0;
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedStageBytes) !=
-        hipSuccess) {
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)kFusedLargeStageBytes) != hipSuccess) {
       (void)hipGetLastError();
       return 0;
     }
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, kFusedStageBytes) != hipSuccess ||
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, fused_stage_bytes(large)) !=
+            hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) {
       (void)hipGetLastError();
       return 0;
@@ -1204,7 +1213,7 @@ static int fused_capacity(const ts_config* cfg, bool packed = false) {
     capacity = per_cu * cus;
     if (capacity <= 0) return 0;
     static thread_local int next = 0;
-    memo[next++ % 8] = Entry{fn, device, capacity};
+    memo[next++ % 16] = Entry{fn, device, large, capacity};
   }
   return capacity;
 }
@@ -1216,20 +1225,36 @@ static int pooling_tokens_cap(const ts_config* cfg) {
   return (kTopkBins - (cfg->pool_kernel - 1)) / 64 * 64;
 }
 
-int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch) {
+// Tokens per workgroup of ts_select for a batch, 0 when the shape is not served; *large:
+// whether the workgroups are the large ones.
+int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch,
+                           bool* large_out) {
+  if (large_out) *large_out = false;
   // Max-pool windows beyond 256 would not fit the LDS the neighbours are gathered into.
   if ((!ignore_switch && !g_fused_select.load()) || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256)
     return 0;
   const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
   if (max_n <= 0) return 0;
-  const int capacity = fused_capacity(cfg);
-  if (capacity <= 0) return 0;
-
-  int tpb = score_tokens_per_block((int64_t)batch * max_seq_len, cfg->num_heads);
-  while ((int64_t)ceil_div(max_n, tpb) * batch > capacity) tpb += 64;
-  if (fused_lds_bytes(tpb, cfg->num_heads) > kFusedStageBytes || tpb > pooling_tokens_cap(cfg))
-    return 0;
-  if (ceil_div(max_seq_len, tpb) > kSelMaxChunks) return 0;  // what the workspace is laid out for
+  auto plan = [&](bool large, int* capacity_out) {
+    const int capacity = fused_capacity(cfg, false, large);
+    *capacity_out = capacity;
+    if (capacity <= 0) return 0;
+    int tpb = score_tokens_per_block((int64_t)batch * max_seq_len, cfg->num_heads);
+    while ((int64_t)ceil_div(max_n, tpb) * batch > capacity) tpb += 64;
+    if (fused_lds_bytes(tpb, cfg->num_heads) > fused_stage_bytes(large) || tpb > pooling_tokens_cap(cfg))
+      return 0;
+    if (ceil_div(max_seq_len, tpb) > kSelMaxChunks) return 0;  // what the workspace is laid out for
+    return tpb;
+  };
+  int capacity = 0, capacity_large = 0;
+  const int tpb = plan(false, &capacity);
+  if (tpb == 0 || (int64_t)ceil_div(max_n, tpb) * 2 > capacity) {
+    const int tpb_large = plan(true, &capacity_large);
+    if (tpb_large > 0) {
+      if (large_out) *large_out = true;
+      return tpb_large;
+    }
+  }
   return tpb;
 }
 
@@ -1239,7 +1264,12 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
   // length, not on how the candidates are dealt out, and is the same whether or not
   // this shape is served: a workspace sized for the longest context serves every
   // shorter one.
-  w.tokens_per_block = fused_tokens_per_block(cfg, batch, max_seq_len, ignore_switch);
+  bool large = false;
+  w.tokens_per_block = fused_tokens_per_block(cfg, batch, max_seq_len, ignore_switch, &large);
+  w.lds_bytes = w.tokens_per_block > 0
+                    ? std::max(fused_lds_bytes(w.tokens_per_block, cfg->num_heads),
+                               large ? kFusedLargeFloorBytes : (size_t)0)
+                    : 0;
   const int max_n = std::max(max_seq_len - cfg->n_init - cfg->n_local, 0);
   w.blocks_per_req = w.tokens_per_block > 0 ? (int)ceil_div(max_n, w.tokens_per_block) : 0;
   const size_t B = (size_t)batch, H = (size_t)cfg->num_heads;
@@ -1330,7 +1360,7 @@ void score_votes_zero_regions(const ts_config* cfg, const ts_batch* bt, const Se
 
 int score_votes_group(const ts_config* cfg, int batch, int max_seq_len) {
   for (int g = batch; g >= 1; --g)
-    if (fused_tokens_per_block(cfg, g, max_seq_len, false) > 0) return g;
+    if (fused_tokens_per_block(cfg, g, max_seq_len, false, nullptr) > 0) return g;
   return 0;
 }
 
@@ -1415,8 +1445,7 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   // as long as the device runs nothing else beside this stream.  (The cooperative
   // launch API would guarantee it, at some 25 us of extra launch latency.)
   const hipError_t e =
-      hipLaunchKernel(fn, grid, dim3(256), params,
-                      fused_lds_bytes(w.tokens_per_block, cfg->num_heads), stream);
+      hipLaunchKernel(fn, grid, dim3(256), params, w.lds_bytes, stream);
   if (e != hipSuccess) {
     (void)hipGetLastError();
     return fail(TS_EHIP, "fused selection launch: %s", hipGetErrorString(e));
@@ -1447,16 +1476,32 @@ bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan
   plan->parts.clear();
   if (!g_fused_select.load()) return false;
   if (cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256) return false;
-  const int capacity = fused_capacity(cfg, /*packed=*/true);
-  if (capacity <= 0) return false;
-  int tpb_max = 64;
-  while (fused_lds_bytes(tpb_max + 64, cfg->num_heads) <= kFusedStageBytes &&
-         tpb_max + 64 <= pooling_tokens_cap(cfg))
-    tpb_max += 64;
-  if (fused_lds_bytes(tpb_max, cfg->num_heads) > kFusedStageBytes) return false;
   const int fixed = cfg->n_init + cfg->n_local;
   auto bound = [&](int b) { return bt->host_seq_lens ? std::min(bt->host_seq_lens[b], bt->max_seq_len) : bt->max_seq_len; };
   auto candidates = [&](int b) { return std::max(bound(b) - fixed, 0); };
+  int longest_n = 0;
+  for (int b = 0; b < bt->batch; ++b) longest_n = std::max(longest_n, candidates(b));
+  // The most tokens a workgroup of either size takes, and what is resident of them.
+  auto size_up = [&](bool large, int* capacity_out) {
+    *capacity_out = fused_capacity(cfg, /*packed=*/true, large);
+    int most = 64;
+    while (fused_lds_bytes(most + 64, cfg->num_heads) <= fused_stage_bytes(large) &&
+           most + 64 <= pooling_tokens_cap(cfg))
+      most += 64;
+    return (*capacity_out > 0 && fused_lds_bytes(most, cfg->num_heads) <= fused_stage_bytes(large)) ? most : 0;
+  };
+  int capacity = 0;
+  int tpb_max = size_up(false, &capacity);
+  // The large workgroups when the longest request takes more than half of the device.
+  if (tpb_max == 0 || ceil_div(longest_n, tpb_max) > capacity / 2) {
+    int capacity_large = 0;
+    const int most = size_up(true, &capacity_large);
+    if (most > tpb_max) {
+      tpb_max = most;
+      capacity = capacity_large;
+    }
+  }
+  if (tpb_max == 0) return false;
   // Phases of half the device when every request fits that.
   bool halves = bt->batch >= 2;
   for (int b = 0; b < bt->batch && halves; ++b)
@@ -1644,7 +1689,7 @@ int ts_score_vote(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
 
 int ts_select_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
-  return fused_tokens_per_block(cfg, batch, max_seq_len, false) > 0 ? 1 : 0;
+  return fused_tokens_per_block(cfg, batch, max_seq_len, false, nullptr) > 0 ? 1 : 0;
 }
 
 size_t ts_select_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
