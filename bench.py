@@ -43,7 +43,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # figures are recorded under profiles/.  Workloads not measured that way give null.
 # Each figure carries the commit of the kernels it was measured on: a later change to the
 # kernel makes it stale until the two counter runs are repeated.
-MEASURED_TRAFFIC = {"C2": (271611207, "63c56af")}  # profiles/decode_layer_c2_hbm_traffic.txt
+MEASURED_TRAFFIC = {"C2": (269711053, "6c0d379")}  # profiles/decode_layer_c2_hbm_traffic.txt
 
 
 def event_time_us(fn, launches: int, warmup: int, before=None, burst: int = 1):
