@@ -64,6 +64,7 @@ struct ScoreArgs {
   // the phase was sized by) leaves at once and is not on the phase's team.  Phase p's
   // rendezvous area is sync + p * kSyncWords.
   int nphases;
+  int resident;           // workgroups of the launch that the device holds at once
   VotePhase phases[kMaxPhases];
   uint32_t* hist_ws;      // per-request top-k workspace (ts_topk.h) whose hist0 is counted into, or NULL
   size_t hist_ws_stride;

@@ -344,6 +344,57 @@ __device__ __forceinline__ int block_threshold_scan(uint32_t mine, uint32_t need
   return who == 0xffffffffu ? -1 : (int)who;
 }
 
+// Votes-only launches: a phase ends with the memory idle while its statistics are on
+// their way, and when a request takes the whole device no other phase streams meanwhile.
+// The wavefronts that do not poll for the statistics touch the first keys of the
+// workgroup that is going to take this one's place: `resident` workgroups further on in
+// the grid, hence on the same XCD, whose L2 then holds what each of that workgroup's
+// wavefronts asks for first.  One 4-byte load per 128-byte line; the values are only
+// kept so that the loads are (the caller hands them to an empty asm at its end).
+// Eight tokens per wavefront of the successor (64 KB per workgroup at eight KV heads, 2 MB
+// per XCD): C5 layer 425 -> 420 us, C3 442 -> 438 us; 16 tokens bring less, 24 are slower
+// than none (the L2 of an XCD holds 4 MB).
+constexpr int kAheadTokens = 8;
+constexpr int kAheadLoads = (4 * kAheadTokens * 16 + 191) / 192;  // per lane, at 16 lines per row
+template <int HKV>
+__device__ __forceinline__ void touch_successor_keys(const ScoreArgs& a, int wave, int lane,
+                                                     uint32_t (&got)[kAheadLoads]) {
+  constexpr uint32_t ROW_BYTES = HKV * kHeadDim * 2;
+  constexpr int kLines = (int)ROW_BYTES / 128;
+  constexpr int kItems = 4 * kAheadTokens * kLines;
+  static_assert(kItems <= kAheadLoads * 192, "three wavefronts cover the lines");
+#pragma unroll
+  for (int i = 0; i < kAheadLoads; ++i) got[i] = 0u;
+  const int g = (int)blockIdx.x + a.resident;
+  if (a.resident <= 0 || g >= (int)gridDim.x) return;
+  int phase = 0;
+  while (phase + 1 < a.nphases && g >= a.phases[phase + 1].first_workgroup) ++phase;
+  const VotePhase& ph = a.phases[phase];
+  const int x = g - ph.first_workgroup;
+  int req = 0;
+  while (req + 1 < ph.requests && x >= ph.pack_first[req + 1]) ++req;
+  const int b = ph.first + req;
+  if (a.skip && a.skip[b]) return;
+  const ReqGeom geo =
+      request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  const int block_lo = (x - ph.pack_first[req]) * ph.tokens_per_block;
+  if (block_lo >= geo.n) return;
+  const int per_wave = ph.tokens_per_block >> 2;
+  const int32_t* tab = a.table + (int64_t)b * a.table_stride;
+#pragma unroll
+  for (int i = 0; i < kAheadLoads; ++i) {
+    const int item = (wave - 1) * 64 + lane + 192 * i;
+    if (item < kItems) {
+      const int t = item / kLines, line = item % kLines;
+      const int tok = min(block_lo + (t / kAheadTokens) * per_wave + t % kAheadTokens, geo.n - 1);
+      const int pos = a.n_init + tok;
+      uint32_t slot = ((uint32_t)tab[pos >> a.page_shift] << a.page_shift) + (uint32_t)(pos & (a.page_size - 1));
+      slot = slot < a.pool_rows ? slot : a.pool_rows - 1;
+      got[i] = *(const uint32_t*)((const char*)a.k_pool + (size_t)slot * ROW_BYTES + line * 128);
+    }
+  }
+}
+
 template <int HKV, int G, bool OUT_BF16, int MODE>
 __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a) {
   extern __shared__ float stage[];  // tiled / fused: [tiles of the workgroup][tile_stride]
@@ -638,6 +689,12 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     TS_MARK(2);
     merge_request_stats<PACKED>(a, lp, team, lane, wave);
     TS_MARK(3);
+    uint32_t ahead[kAheadLoads];
+#pragma unroll
+    for (int i = 0; i < kAheadLoads; ++i) ahead[i] = 0u;
+    if constexpr (PACKED) {
+      if (wave != 0) touch_successor_keys<HKV>(a, wave, lane, ahead);  // (wavefront 0 polls)
+    }
     // While the merged statistics are on their way: the exponentials, relative to this
     // workgroup's own maxima; exp(s - max) / sum = exp(s - own max) * exp(own max - max) / sum.
     const ReqGeom geo =
@@ -742,6 +799,8 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         if (a.fault_out)
           __hip_atomic_store(a.fault_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       }
+#pragma unroll
+      for (int i = 0; i < kAheadLoads; ++i) asm volatile("" ::"v"(ahead[i]));
       return;
     }
     // Local histogram: one LDS atomic per candidate (lanes that hit the same bin are
@@ -1302,6 +1361,7 @@ struct VoteLaunch {
 // The phases of a batch, up to kMaxPhases of them to a launch.
 struct VotePlan {
   std::vector<VoteLaunch> parts;
+  int resident = 0;  // workgroups of the kernel that the device holds at once
 };
 bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan);
 
@@ -1502,6 +1562,7 @@ bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan
     }
   }
   if (tpb_max == 0) return false;
+  plan->resident = capacity;
   // Phases of half the device when every request fits that.
   bool halves = bt->batch >= 2;
   for (int b = 0; b < bt->batch && halves; ++b)
@@ -1566,6 +1627,7 @@ int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf,
     a.batch_offset = v.first;
     a.hist_ws = hist_ws;
     a.hist_ws_stride = hist_ws_stride;
+    a.resident = plan.resident;
     int tpb_lds = v.tokens_per_block;
     dim3 grid;
     {
