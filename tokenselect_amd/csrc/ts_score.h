@@ -100,7 +100,7 @@ constexpr int kSelListCount = kSelMaxBin + kSelHistCopies * 32;
 constexpr int kSelCounterWords = kSelListCount + kSelListParts * 32;
 
 // Workgroups of one request the workspace of ts_select is laid out for (the device keeps
-// some 510 resident at once).
+// at most 512 resident at once).
 constexpr int kSelMaxChunks = 1024;
 
 // Workspace of ts_select, carved in this order (256-byte aligned pieces).
