@@ -110,12 +110,15 @@ struct SelectWorkspace {
   int64_t pool_stride;
   int tokens_per_block;  // 0: the shape does not fit the fused kernel
   int blocks_per_req;
+  int clear_chunks;      // per-workgroup statistics of a (request, head) row to clear before a launch
   size_t lds_bytes;      // dynamic LDS of the launch (decides how many workgroups share a CU)
 };
 // ignore_switch: lay out as if ts_set_fused_select were on (for sizing a workspace that
 // must serve both settings).
+// may_skip: requests of the launch may be skipped on the device (selection cache), which
+// decides between one and two workgroups per CU; the layout does not depend on it.
 SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len,
-                                 bool ignore_switch = false);
+                                 bool ignore_switch = false, bool may_skip = false);
 
 // Regions the kernel before ts_select on the stream has to clear (counters, replicas
 // of the merged statistics, rendezvous words, the per-workgroup statistics), in the form

@@ -1228,12 +1228,9 @@ static size_t fused_lds_bytes(int tokens_per_block, int num_heads) {
 }
 
 // Dynamic LDS the fused form may use.  With the 10 KB of static arrays two workgroups
-// of 68 KB fit the 160 KB of a CU; a workgroup of up to 140 KB has the CU to itself and
-// takes twice the tokens.  Half as many workgroups make every hand-off between them
-// cheaper (arrivals counted, readers of one line, adds to one histogram line), and four
-// wavefronts per CU still keep enough loads in flight for the stream; but a request
-// that is skipped or short leaves its CUs idle, and there are half as many to share.
-// So the large workgroups serve where one request takes more than half of the device.
+// of 68 KB fit the 160 KB of a CU; a workgroup that asks for more than half of a CU's LDS
+// (up to 140 KB) has the CU to itself.  Which of the two a launch gets is decided by its
+// planner (fused_tokens_per_block, plan_vote_launches).
 constexpr size_t kFusedStageBytes = 68 * 1024;
 constexpr size_t kFusedLargeStageBytes = 140 * 1024;
 constexpr size_t kFusedLargeFloorBytes = 76 * 1024;  // more than half a CU's LDS: one workgroup per CU
@@ -1285,18 +1282,28 @@ static int pooling_tokens_cap(const ts_config* cfg) {
 }
 
 // Tokens per workgroup of ts_select for a batch, 0 when the shape is not served; *large:
-// whether the workgroups are the large ones.
+// whether the workgroups have a CU to themselves; *most_blocks: the most workgroups per
+// request of any plan this shape may get (what has to be cleared for it).
+// One workgroup per CU wherever the batch fits that way with no more LDS than a small
+// workgroup has (C2 64.2 -> 61.9 us; 1.7-2.9 us at every length from 8K on for one request,
+// 1-2 us for 2 x 64K and 4 x 32K): below 256 workgroups the dispatcher otherwise doubles
+// them up on some CUs while others idle, above that half as many workgroups stream as
+// fast and hand over less.  Batches that need more LDS per CU than that run as well or
+// better on two workgroups per CU (2 x 128K the same, 4 x 64K and 8 x 32K 1-2 us better),
+// and so do batches in which requests may be skipped (selection cache): what a skipped
+// request leaves idle are whole CUs then, and the others' keys stream through half as many
+// (C4 93 -> 104 us per step).
 int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch,
-                           bool* large_out) {
+                           bool* large_out, bool may_skip, int* most_blocks_out) {
   if (large_out) *large_out = false;
+  if (most_blocks_out) *most_blocks_out = 0;
   // Max-pool windows beyond 256 would not fit the LDS the neighbours are gathered into.
   if ((!ignore_switch && !g_fused_select.load()) || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256)
     return 0;
   const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
   if (max_n <= 0) return 0;
-  auto plan = [&](bool large, int* capacity_out) {
+  auto plan = [&](bool large) {
     const int capacity = fused_capacity(cfg, false, large);
-    *capacity_out = capacity;
     if (capacity <= 0) return 0;
     int tpb = score_tokens_per_block((int64_t)batch * max_seq_len, cfg->num_heads);
     while ((int64_t)ceil_div(max_n, tpb) * batch > capacity) tpb += 64;
@@ -1305,26 +1312,28 @@ int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, boo
     if (ceil_div(max_seq_len, tpb) > kSelMaxChunks) return 0;  // what the workspace is laid out for
     return tpb;
   };
-  int capacity = 0, capacity_large = 0;
-  const int tpb = plan(false, &capacity);
-  if (tpb == 0 || (int64_t)ceil_div(max_n, tpb) * 2 > capacity) {
-    const int tpb_large = plan(true, &capacity_large);
-    if (tpb_large > 0) {
-      if (large_out) *large_out = true;
-      return tpb_large;
-    }
+  const int tpb_small = plan(false), tpb_large = plan(true);
+  if (most_blocks_out)
+    *most_blocks_out = std::max(tpb_small > 0 ? (int)ceil_div(max_n, tpb_small) : 0,
+                                tpb_large > 0 ? (int)ceil_div(max_n, tpb_large) : 0);
+  const bool roomy = tpb_large > 0 && fused_lds_bytes(tpb_large, cfg->num_heads) <= kFusedStageBytes;
+  if ((roomy && !(may_skip && batch >= 2)) || tpb_small == 0) {
+    if (large_out) *large_out = tpb_large > 0;
+    return tpb_large;
   }
-  return tpb;
+  return tpb_small;
 }
 
-SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch) {
+SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch,
+                                 bool may_skip) {
   SelectWorkspace w{};
   // The layout depends on the batch, the head count and (for the pooled votes) the
   // length, not on how the candidates are dealt out, and is the same whether or not
   // this shape is served: a workspace sized for the longest context serves every
   // shorter one.
   bool large = false;
-  w.tokens_per_block = fused_tokens_per_block(cfg, batch, max_seq_len, ignore_switch, &large);
+  w.tokens_per_block =
+      fused_tokens_per_block(cfg, batch, max_seq_len, ignore_switch, &large, may_skip, &w.clear_chunks);
   w.lds_bytes = w.tokens_per_block > 0
                     ? std::max(fused_lds_bytes(w.tokens_per_block, cfg->num_heads),
                                large ? kFusedLargeFloorBytes : (size_t)0)
@@ -1404,7 +1413,7 @@ void select_zero_regions(const ts_config* cfg, const SelectWorkspace& w, void* w
   zero->add(counters);
   zero->add(stats_zero_region(w, workspace, batch, cfg->num_heads));
   zero->add(sync_zero_region(w, workspace, 1));
-  zero->add(partials_zero_region(w, workspace, batch, cfg->num_heads, w.blocks_per_req));
+  zero->add(partials_zero_region(w, workspace, batch, cfg->num_heads, w.clear_chunks));
 }
 
 void score_votes_zero_regions(const ts_config* cfg, const ts_batch* bt, const SelectWorkspace& w,
@@ -1420,7 +1429,7 @@ void score_votes_zero_regions(const ts_config* cfg, const ts_batch* bt, const Se
 
 int score_votes_group(const ts_config* cfg, int batch, int max_seq_len) {
   for (int g = batch; g >= 1; --g)
-    if (fused_tokens_per_block(cfg, g, max_seq_len, false, nullptr) > 0) return g;
+    if (fused_tokens_per_block(cfg, g, max_seq_len, false, nullptr, false, nullptr) > 0) return g;
   return 0;
 }
 
@@ -1470,7 +1479,8 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
                   int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
                   int64_t vote_stride, void* workspace, uint32_t* clear, int clear_per_req,
                   hipStream_t stream, uint64_t wait_ticks, uint32_t absent) {
-  const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len);
+  // (requests may be skipped when the caller brings hit flags: the selection cache)
+  const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len, false, hit != nullptr);
   TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE, "fused selection: unsupported shape");
   char* ws = (char*)workspace;
   ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, hit, (float*)(ws + w.partials),
@@ -1751,7 +1761,7 @@ int ts_score_vote(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
 
 int ts_select_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
-  return fused_tokens_per_block(cfg, batch, max_seq_len, false, nullptr) > 0 ? 1 : 0;
+  return fused_tokens_per_block(cfg, batch, max_seq_len, false, nullptr, false, nullptr) > 0 ? 1 : 0;
 }
 
 size_t ts_select_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
