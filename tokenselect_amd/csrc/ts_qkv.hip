@@ -7,17 +7,16 @@
 // and the separate store launch disappear.
 //
 // With a handful of rows in x the product is a stream over W (bound: HBM).  A
-// wavefront owns two whole rows of W: a lane reads up to eight 16-byte pieces of
-// each (all requested before the first is used, before x is staged), multiplies
+// wavefront owns two or three whole rows of W: a lane reads up to eight 16-byte pieces
+// of each (all requested before the first is used, before x is staged), multiplies
 // them with the matching pieces of x from LDS (bf16, staged once per workgroup of
-// eight wavefronts) and the wavefront reduces its 2 x B sums on its own: no
+// eight wavefronts) and the wavefront reduces its sums (rows x B) on its own: no
 // exchange between wavefronts.
 #include "ts_pages.h"
 
 namespace ts {
 
 constexpr int kQkvMaxBatch = 8;      // rows of x
-constexpr int kQkvRows = 2;          // rows of W per wavefront
 constexpr int kQkvWaves = 8;         // wavefronts per workgroup
 constexpr int kQkvPieces = 8;        // 16-byte pieces of a row per lane
 constexpr int kQkvMaxHidden = 4096;  // 64 lanes x kQkvPieces x 8 elements
@@ -58,7 +57,9 @@ __device__ __forceinline__ uint4 load_streaming(const uint4* p) {
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 
-template <int B>
+// kQkvRows: rows of W per wavefront (two or three, whichever spreads the rows more evenly
+// over the CUs).
+template <int B, int kQkvRows>
 __global__ __launch_bounds__(64 * kQkvWaves) void qkv_store_kernel(QkvArgs a) {
   extern __shared__ uint4 lds_x[];  // [B][hidden / 8]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -185,9 +186,23 @@ __global__ __launch_bounds__(64 * kQkvWaves) void qkv_store_kernel(QkvArgs a) {
 template <int B>
 static int launch_qkv(const QkvArgs& a, hipStream_t stream) {
   const size_t lds = (size_t)B * a.hidden * 2;  // at most 64 KB
-  hipLaunchKernelGGL(qkv_store_kernel<B>,
-                     dim3((unsigned)ceil_div(a.n_out, kQkvRows * kQkvWaves)), dim3(64 * kQkvWaves),
-                     lds, stream, a);
+  // The kernel is one burst of loads per wavefront, and the slowest CU decides: 6144 rows
+  // (Llama-3-8B) in 16-row workgroups are 384 workgroups, one and a half per CU, 16.3 us;
+  // in 24-row workgroups 256, one per CU, 14.5 us; in 32-row workgroups 192: 16.8 us.
+  int cus = 0, device = 0;
+  if (hipGetDevice(&device) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) {
+    (void)hipGetLastError();
+    cus = 256;
+  }
+  auto rounds = [&](int rows) { return ceil_div(ceil_div(a.n_out, rows * kQkvWaves), cus) * rows; };
+  if (rounds(3) < rounds(2)) {
+    hipLaunchKernelGGL((qkv_store_kernel<B, 3>), dim3((unsigned)ceil_div(a.n_out, 3 * kQkvWaves)),
+                       dim3(64 * kQkvWaves), lds, stream, a);
+  } else {
+    hipLaunchKernelGGL((qkv_store_kernel<B, 2>), dim3((unsigned)ceil_div(a.n_out, 2 * kQkvWaves)),
+                       dim3(64 * kQkvWaves), lds, stream, a);
+  }
   return check_launch("qkv_store_kernel");
 }
 
