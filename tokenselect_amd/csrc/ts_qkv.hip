@@ -189,9 +189,15 @@ static int launch_qkv(const QkvArgs& a, hipStream_t stream) {
   // The kernel is one burst of loads per wavefront, and the slowest CU decides: 6144 rows
   // (Llama-3-8B) in 16-row workgroups are 384 workgroups, one and a half per CU, 16.3 us;
   // in 24-row workgroups 256, one per CU, 14.5 us; in 32-row workgroups 192: 16.8 us.
-  int cus = 0, device = 0;
-  if (hipGetDevice(&device) != hipSuccess ||
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) {
+  static thread_local int cus_of[64] = {};  // by device, asked once per thread
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    device = 0;
+  }
+  int& cus = cus_of[device & 63];
+  if (cus <= 0 &&
+      (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)) {
     (void)hipGetLastError();
     cus = 256;
   }
