@@ -1687,8 +1687,9 @@ size_t ts_score_partials_bytes(const ts_config* cfg, int32_t batch, int32_t max_
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
   // A bound that never shrinks when max_seq_len grows, unlike the number of workgroups
   // itself (the candidates per workgroup move in steps of 64), so that a buffer sized
-  // for the longest context serves every shorter one: 512 workgroups are aimed at, more
-  // only once a workgroup holds as many candidates as its LDS takes.
+  // for the longest context serves every shorter one: 256 workgroups are aimed at (the
+  // bound leaves room for twice that), more only once a workgroup holds as many candidates
+  // as its LDS takes.
   const int64_t cap = std::max<int64_t>((16384 / cfg->num_heads) / 64 * 64, 64);
   const size_t nchunks = (size_t)std::max<int64_t>(520, ceil_div(max_seq_len, cap) + 8);
   return align_up((size_t)batch * cfg->num_heads * nchunks * 2 * sizeof(float), 256);
