@@ -152,6 +152,48 @@ def test_fused_select(dev, shape, page):
             assert torch.equal(sel[b, :S].cpu(), tabs[b][pos.long()])
 
 
+@pytest.mark.parametrize("lens", [[5000, 3000, 9000], [40000, 20000]], ids=["3x<=9K", "2x<=40K"])
+def test_fused_select_same_with_either_workgroup_size(dev, lens):
+    """A batch whose scores fit one workgroup per CU is served that way, unless requests
+    may be skipped (hit flags given), which puts it on two smaller workgroups per CU: the
+    same inputs through both, alternating on one workspace, must give the same votes up
+    to the rounding of the merged statistics (the chunks they are merged from differ:
+    2e-6 relative) and the same selection; the votes are also held against the oracle's."""
+    say(f"fused select, one and two workgroups per CU, lens={lens}")
+    ks = [256] * len(lens)
+    wl = small(dev, SHAPES[0], seed=len(lens), lens=lens, ks=ks, page=16, top_k=256)
+    c = wl.cfg
+    qf = fingerprint(wl, dev)
+    details = []
+    oracle_layer(wl, details)
+    nobody = torch.zeros(len(lens), dtype=torch.int32, device=dev)  # hit flags: every request misses
+    cache = ops.SelectionCache.allocate(c, len(lens), dev)
+    space = None
+    results = []
+    for attempt in range(4):
+        skipping = dict(hit=nobody, cache=cache) if attempt % 2 else {}
+        sel, sel_pos, sel_len, votes, space = ops.select(c, wl.batch, qf, wl.k_pool, want_votes=True,
+                                                         workspace=space, **skipping)
+        torch.cuda.synchronize()
+        assert not ops.select_fault(c, wl.batch, space)
+        results.append((sel.clone(), sel_pos.clone(), sel_len.clone(), votes.clone()))
+    first = results[0]
+    for attempt, got in enumerate(results[1:], 1):
+        assert torch.equal(got[2], first[2]), f"attempt {attempt}: lengths"
+        for b, (L, k) in enumerate(zip(lens, ks)):
+            S, n = int(first[2][b]), L - c.n_init - c.n_local
+            assert torch.allclose(got[3][b, :n], first[3][b, :n], rtol=2e-6, atol=0), f"attempt {attempt} b={b}: votes"
+            mid = got[1][b, c.n_init:c.n_init + k].cpu()
+            assert_index_sets_match(mid, first[1][b, c.n_init:c.n_init + k].cpu(), first[3][b, :n].cpu(),
+                                    c.n_init, f"attempt {attempt} b={b}")
+            assert torch.equal(got[0][b, :S].cpu(), cpu_tabs(wl)[b][got[1][b, :S].cpu().long()])
+    for b, L in enumerate(lens):
+        n = L - c.n_init - c.n_local
+        assert torch.allclose(first[3][b, :n].cpu(), details[b]["votes"], rtol=2e-4, atol=1e-9), f"votes b={b}"
+        assert_index_sets_match(first[1][b, c.n_init:c.n_init + ks[b]].cpu(), details[b]["top_pos"],
+                                details[b]["votes"], c.n_init, f"oracle b={b}")
+
+
 def test_select_clear_then_cleared_equals_select(dev):
     """ts_select is ts_select_clear + ts_select_cleared: the two calls made by hand,
     twice in a row on one workspace, give what the single call gives."""
