@@ -102,7 +102,28 @@ typedef struct ts_batch {
                                the tokens beyond it are not scored, and the
                                launch reports it like a wait that gave up
                                (fault, sel_len = -1)                           */
+  /* Per-call options; all zero = the defaults. */
+  int32_t separate_kernels; /* 1: this call selects with ts_score + ts_vote +
+                               ts_topk_ragged's kernels, whose workgroups never wait
+                               for each other, whatever ts_set_fused_select says:
+                               the way out for a caller whose ts_select gave up  */
+  int32_t rerun;            /* 1: this call repeats the caller's previous call of
+                               the same step after that one gave up (sel_len[b] =
+                               -1 marks the requests concerned, and sel_len must be
+                               the array of that call): the selection cache takes a
+                               request that gave up as a miss whatever it cached
+                               meanwhile, and its counters do not advance again  */
+  uint32_t wait_us;         /* bound of a grid-wide wait of the fused kernels in
+                               microseconds; 0 = TS_DEFAULT_WAIT_US              */
+  int32_t absent_workgroups; /* tests of the give-up path only (0 in production):
+                               workgroups counted as members of every rendezvous
+                               that never arrive, so that every wait gives up
+                               after wait_us while all kernels still exit        */
 } ts_batch;
+
+/* Default bound of a grid-wide wait: a selection that has the device to itself
+ * meets within tens of microseconds, so 10 ms means something else holds the GPU. */
+#define TS_DEFAULT_WAIT_US 10000u
 
 /* Optional selection-cache state for one layer (tr.py:301-322, 394-421).
  * All arrays are device memory owned by the caller and persist across steps. */
@@ -238,14 +259,15 @@ int ts_topk_ragged(const ts_config* cfg, const ts_batch* bt, const float* votes,
  * ts_score + ts_vote + ts_topk_ragged.  The launch is an ordinary one sized so
  * that all its workgroups are resident together; that holds while nothing else
  * runs on the device beside the caller's stream (a cooperative launch would
- * enforce it, at about 25 us per call).  Every grid-wide wait is bounded (2 s);
+ * enforce it, at about 25 us per call).  Every grid-wide wait is bounded (bt->wait_us,
+ * 10 ms unless the caller says otherwise);
  * once one has given up the others return at once, the kernel drains, and the
  * launch reports it without any host synchronisation: sel_len[b] = -1 for
  * every request that was selecting (the other outputs of those requests are
  * not valid; ts_sparse_decode_attn treats a negative length as an empty list),
  * *bt->fault = 1 when bt->fault is given, and the first 32-bit word of the
  * last batch * 65 * 4096 bytes of the workspace is 1 until the next clearing.  A
- * caller that sees it reruns the step with the separate kernels.
+ * caller that sees it reruns the step with the separate kernels (bt->separate_kernels).
  * No counterpart in the reference, which materialises every intermediate. */
 int ts_select_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
 size_t ts_select_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_seq_len);
@@ -269,7 +291,8 @@ int ts_select_cleared(const ts_config* cfg, const ts_batch* bt, const void* qf, 
                       ts_stream_t stream);
 
 /* ts_select_cleared with an explicit bound for the grid-wide waits, in ticks of
- * the device's 100 MHz clock (ts_select uses 200 000 000 = 2 s), and a number of
+ * the device's 100 MHz clock (ts_select uses bt->wait_us x 100, by default 1 000 000 = 10 ms;
+ * these arguments take the place of bt->wait_us and bt->absent_workgroups), and a number of
  * workgroups that are counted as members of the rendezvous but never arrive
  * (0 in production): with absent_workgroups > 0 every wait gives up after
  * wait_ticks, which is how the give-up path is tested without hanging a GPU.
@@ -313,7 +336,9 @@ int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_poo
  * of 520 bytes; with 32 query / 8 KV heads: every batch up to 251).  All calls on one GPU share the buffer:
  * calls that overlap on one GPU (two streams, two threads) race and must be
  * serialised by the caller; calls on one stream are ordered by the stream.
- * No counterpart in the reference. */
+ * ts_attn_static_scratch_bytes() also looks up the buffer of the current device (as
+ * the first call on a device would): make it once per device at set-up, before any
+ * capture begins.  No counterpart in the reference. */
 size_t ts_attn_static_scratch_bytes(void);
 int ts_sparse_decode_attn_static(const ts_config* cfg, const void* q, const void* k_pool,
                                  const void* v_pool, int64_t pool_rows, const int32_t* sel,

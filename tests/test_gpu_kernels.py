@@ -311,14 +311,112 @@ def test_fused_select_reports_a_wait_that_gave_up(dev):
     for b in range(3):
         S = int(sel_len[b])
         assert torch.equal(sel[b, :S], sel_sep[b, :S]) and torch.equal(sel_pos[b, :S], pos_sep[b, :S])
-    # the layer object refuses to go on once its word is set
-    layer = ops.DecodeLayer(c, 3, max(lens), dev)
-    layer(wl.q, wl.k_pool, wl.v_pool, wl.batch)
+
+
+def layer_matches_oracle(wl, out, sel, sel_pos, sel_len, tag):
+    details = []
+    ref_sel, ref_out = oracle_layer(wl, details)
+    c = wl.cfg
+    for b in range(len(wl.seq_lens)):
+        S = int(sel_len[b])
+        assert S == ref_sel[b].shape[0], f"{tag} b={b}: {S} slots, oracle {ref_sel[b].shape[0]}"
+        if details[b]:
+            assert_index_sets_match(sel_pos[b, c.n_init:S - c.n_local].cpu(), details[b]["top_pos"],
+                                    details[b]["votes"], c.n_init, f"{tag} top-k b={b}")
+        assert_attention_close(wl, b, out[b], sel[b, :S], ref_sel[b], ref_out[b], f"{tag} b={b}")
+
+
+def test_layer_object_recovers_a_step_that_gave_up(dev):
+    """A decode layer whose selection gives up (forced from the host: one team member that
+    never arrives, a 20 us bound; every kernel exits normally) reports it in its pinned word;
+    recover() at the caller's synchronisation point repeats the step's selection and
+    attention with the separate kernels and returns the oracle's output, and the object
+    stays on the separate kernels.  A give-up that nobody recovered makes the next call
+    switch over and raise, after which the object works."""
+    import dataclasses
+    lens, ks = [3000, 40, 1531], [64, 64, 100]
+    say(f"decode layer, forced give-up and recovery lens={lens}")
+    wl = small(dev, SHAPES[0], seed=78, lens=lens, ks=ks, page=16, top_k=100)
+    forced = dataclasses.replace(wl.batch, wait_us=20, absent_workgroups=1)
+    layer = ops.DecodeLayer(wl.cfg, 3, max(lens), dev)
+    assert ops.layer_selection_form(wl.cfg, wl.batch) == 2
+    out, sel, sel_pos, sel_len = layer(wl.q, wl.k_pool, wl.v_pool, forced)
     torch.cuda.synchronize()
-    layer.check()
-    layer.fault[0] = 1
+    assert layer.gave_up() and sel_len.tolist() == [-1, 40, -1]
+    got = layer.recover(wl.q, wl.k_pool, wl.v_pool, forced)
+    assert got is not None and layer.separate and not layer.gave_up()
+    torch.cuda.synchronize()
+    layer_matches_oracle(wl, *got, "recovered step")
+    # nothing to recover now, and the object no longer launches kernels that could give up
+    assert layer.recover(wl.q, wl.k_pool, wl.v_pool, forced) is None
+    again = layer(wl.q, wl.k_pool, wl.v_pool, forced)
+    torch.cuda.synchronize()
+    assert not layer.gave_up()
+    layer_matches_oracle(wl, *again, "after the switch")
+    # a give-up that nobody recovered: the next call switches over and raises, then works
+    other = ops.DecodeLayer(wl.cfg, 3, max(lens), dev)
+    other(wl.q, wl.k_pool, wl.v_pool, forced)
+    torch.cuda.synchronize()
     with pytest.raises(ops.SelectionGaveUp):
-        layer(wl.q, wl.k_pool, wl.v_pool, wl.batch)
+        other(wl.q, wl.k_pool, wl.v_pool, wl.batch)
+    assert other.separate and not other.gave_up()
+    retried = other(wl.q, wl.k_pool, wl.v_pool, wl.batch)
+    torch.cuda.synchronize()
+    layer_matches_oracle(wl, *retried, "retried step")
+    # one call on the separate kernels without touching the process-wide switch
+    third = ops.DecodeLayer(wl.cfg, 3, max(lens), dev)
+    once = third(wl.q, wl.k_pool, wl.v_pool, dataclasses.replace(forced, separate_kernels=True))
+    torch.cuda.synchronize()
+    assert not third.gave_up() and not third.separate
+    layer_matches_oracle(wl, *once, "separate kernels for one call")
+
+
+def test_recovery_keeps_the_selection_cache_consistent(dev):
+    """Selection-cache trace in which one step gives up (forced) and is recovered: the requests
+    that were selecting select afresh, those that hit keep their cached positions, the counters
+    advance once per step, and every later decision equals that of an undisturbed run."""
+    import dataclasses
+    B, steps, bad = 3, 8, 4
+    lens = [2500, 3000, 2800]
+    say(f"selection cache trace with a recovered give-up at step {bad}")
+    wl = small(dev, SHAPES[0], seed=91, lens=lens, ks=[64] * B, page=1, top_k=64)
+    c = wl.cfg
+    g = torch.Generator().manual_seed(92)
+    qs = [wl.q.cpu().float()]
+    for t in range(1, steps):   # request 0 drifts slowly (hits), 1 jumps (misses), 2 alternates
+        fresh = torch.randn(qs[0].shape, generator=g)
+        mix = torch.tensor([0.99, 0.0, 0.99 if t % 2 else 0.0])[:, None]
+        qs.append(mix * qs[-1] + (1 - mix ** 2).sqrt() * fresh)
+    qs = [q.bfloat16().to(dev) for q in qs]
+
+    def run(disturb):
+        cache = ops.SelectionCache.allocate(c, B, dev)
+        layer = ops.DecodeLayer(c, B, max(lens), dev)
+        trace = []
+        for t in range(steps):
+            bt = wl.batch
+            if disturb and t == bad:
+                bt = dataclasses.replace(bt, wait_us=20, absent_workgroups=1)
+            res = layer(qs[t], wl.k_pool, wl.v_pool, bt, cache)
+            if disturb:
+                got = layer.recover(qs[t], wl.k_pool, wl.v_pool, bt, cache)
+                assert (got is not None) == (t == bad)
+                res = got or res
+            torch.cuda.synchronize()
+            trace.append([x.clone() for x in res] + [cache.counters.clone(), cache.cache_len.clone(),
+                                                       cache.topk_cache.clone()])
+        return trace
+
+    plain, disturbed = run(False), run(True)
+    for t in range(steps):
+        for name, x, y in zip(("out", "sel", "sel_pos", "sel_len", "counters", "cache_len", "topk_cache"),
+                              plain[t], disturbed[t]):
+            if name == "out":
+                assert (x.float() - y.float()).abs().max().item() <= 2e-2, f"step {t}"
+            else:
+                assert torch.equal(x, y), f"step {t}: {name} differs after the recovery"
+    hits = plain[-1][4][:, 0].tolist()
+    assert hits[0] >= steps - 2 and hits[1] == 0, f"the trace should mix hits and misses: {hits}"
 
 
 def test_fused_select_rejects_unsupported(dev):
@@ -1047,3 +1145,30 @@ def test_layer_split_at_the_vote(dev, fused_select, pool_kernel):
             else:
                 want = out.view(B, H, D)[b, r * H // 2:(r + 1) * H // 2].reshape(-1).float()
                 assert (out_r[b].float() - want).abs().max().item() <= 2e-2
+
+
+def test_selection_form_agrees_with_what_the_launchers_serve(dev):
+    """ts_decode_layer picks its selection form from the very plans its launchers follow: over
+    a sweep of head shapes, batches, lengths and pooling windows the form is 2 exactly where
+    ts_select serves, 1 exactly where only ts_score_vote does, and a per-call switch to the
+    separate kernels gives 0 without touching the process-wide setting."""
+    import dataclasses
+    say("selection form sweep")
+    seen = set()
+    for shape in SHAPES:
+        for pool_kernel in (-1, 5, 300):
+            for B in (1, 2, 4, 16, 64):
+                for L in (700, 5000, 65536, 131072, 262144, 1048000):
+                    c = ops.LayerConfig(page_size=16, n_init=128, n_local=512, top_k=2048,
+                                        pool_kernel=pool_kernel, **shape)
+                    form = ops.layer_selection_form(c, B, L)
+                    sel_ok = ops.select_supported(c, B, L)
+                    vote_ok = ops.score_vote_supported(c, B, L)
+                    want = 2 if sel_ok else (1 if vote_ok else 0)
+                    assert form == want, (shape, pool_kernel, B, L, form, sel_ok, vote_ok)
+                    seen.add(form)
+    assert seen == {0, 1, 2}
+    wl = small(dev, SHAPES[0], seed=5, lens=[3000], ks=[64])
+    assert ops.layer_selection_form(wl.cfg, wl.batch) == 2
+    assert ops.layer_selection_form(wl.cfg, dataclasses.replace(wl.batch, separate_kernels=True)) == 0
+    assert ops.layer_selection_form(wl.cfg, wl.batch) == 2

@@ -118,3 +118,34 @@ def test_generate_is_deterministic_and_bounded(dev):
     assert torch.equal(runs[0], runs[1])
     with pytest.raises(RuntimeError, match="no slot left"):
         m.decode_step(torch.tensor([1, 2], device=dev))
+
+
+def test_a_step_that_gave_up_is_redone_where_the_tokens_are_read_back(dev):
+    """A fused selection that gives up in the middle of a decode step (forced from the host:
+    an absent team member and a 20 us bound, every kernel still exits) is noticed where the
+    step's tokens reach the host; the step is undone and repeated with the separate kernels,
+    and the tokens, logits, tables and lengths equal those of an undisturbed model."""
+    say("toy decoder, a decode step that gave up and is redone")
+    mc = ModelConfig(**TOY)
+    contexts, steps, bad = [300, 260], 4, 1
+    runs = []
+    for disturb in (False, True):
+        m = Decoder(mc, contexts, steps, dev, seed=33)
+        tokens = torch.tensor([7, 123], device=dev)
+        out = []
+        for t in range(steps):
+            if disturb and t == bad:
+                m.layer_options = dict(wait_us=20, absent_workgroups=1)
+            logits, tokens, host = m.decode_step_checked(tokens)
+            out.append((logits.float().cpu(), host.clone()))
+        torch.cuda.synchronize()
+        assert m.steps_redone == (1 if disturb else 0)
+        assert m.attention.separate == disturb
+        runs.append((out, m.table.cpu(), m.num_tokens.cpu()))
+    (plain, tab0, n0), (redone, tab1, n1) = runs
+    assert torch.equal(tab0, tab1) and torch.equal(n0, n1)
+    assert n0.tolist() == [[c + steps for c in contexts]] * mc.layers
+    for t in range(steps):
+        scale = plain[t][0].pow(2).mean().sqrt().item()
+        assert (plain[t][0] - redone[t][0]).abs().max().item() <= 0.02 * scale, t
+        assert torch.equal(plain[t][1], redone[t][1]), f"step {t}: tokens differ"

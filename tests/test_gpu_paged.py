@@ -64,6 +64,60 @@ def test_kv_store_paged(dev):
     assert ref_free == []
 
 
+def test_kv_store_paged_across_wavefront_rounds(dev):
+    """A batch of 150: the plan walks the requests 64 at a time and carries the rank of the
+    requests that need a page from one round to the next.  Requests on page boundaries sit in
+    all three rounds, the list runs dry inside the third, and one entry of the list is a page
+    beyond the pool (dropped with its request left untouched, the stack staying contiguous).
+    Table, lengths, free list and pool rows against the oracle, three steps in a row."""
+    B, ps, pages_per_req = 150, 16, 6
+    say(f"paged kv_store: B={B} across rounds of 64")
+    c = ops.LayerConfig(num_heads=8, num_kv_heads=2, page_size=ps, n_init=2, n_local=4, top_k=8,
+                        rope_theta=1e4)
+    g = torch.Generator().manual_seed(11)
+    lens = torch.randint(1, 70, (B,), generator=g)
+    lens[torch.randperm(B, generator=g)[:60]] //= ps
+    lens = (lens.clamp_min(0) * 1).tolist()
+    lens = [L * ps if i % 5 == 0 else L for i, L in enumerate(lens)]     # many on a boundary
+    lens = [min(L, pages_per_req * ps - 2) for L in lens]
+    total_pages = B * pages_per_req + 40
+    perm = torch.randperm(total_pages, generator=g).int()
+    table = torch.full((B, pages_per_req), -1, dtype=torch.int32)
+    at = 0
+    for b, L in enumerate(lens):
+        used = -(-L // ps)
+        table[b, :used] = perm[at:at + used]
+        at += used
+    need_now = sum(1 for L in lens if L % ps == 0)
+    free = perm[at:at + need_now - 7].clone()            # seven requests too few
+    free[len(free) // 2] = total_pages + 5               # a page beyond the pool
+    pool_rows = total_pages * ps
+    k_pool = torch.zeros((pool_rows, 2, 128), dtype=torch.bfloat16, device=dev)
+    v_pool = torch.zeros_like(k_pool)
+    table_d, seq = table.to(dev), torch.tensor(lens, dtype=torch.int32, device=dev)
+    pool = ops.PagePool.of(free.to(dev))
+    ref_table, ref_lens, ref_free = table.clone(), list(lens), free.tolist()
+    kc, vc = k_pool.cpu().clone(), v_pool.cpu().clone()
+    gd = torch.Generator(device=dev).manual_seed(12)
+    refused = 0
+    for step in range(3):
+        k = torch.randn((B, 2, 128), generator=gd, device=dev).bfloat16()
+        v = torch.randn((B, 2, 128), generator=gd, device=dev).bfloat16()
+        ops.kv_store(c, k, v, None, k_pool, v_pool, table_d, seq, pages=pool)
+        torch.cuda.synchronize()
+        slots = oracle.store.append_token_paged(ref_table, ref_lens, ref_free, ps, pages_per_req * ps,
+                                                pool_rows)
+        for b, s_ in enumerate(slots):
+            if s_ is not None:
+                kc[s_], vc[s_] = k[b].cpu(), v[b].cpu()
+        refused += sum(1 for s_ in slots if s_ is None)
+        assert seq.cpu().tolist() == ref_lens, f"step {step}"
+        assert torch.equal(table_d.cpu(), ref_table), f"step {step}"
+        assert _pool_state(pool) == ref_free and int(pool.ticket) == 0, f"step {step}"
+    assert refused >= 8 and ref_free == []
+    assert torch.equal(k_pool.cpu(), kc) and torch.equal(v_pool.cpu(), vc)
+
+
 def test_qkv_store_paged_equals_the_unfused_store(dev):
     say("paged qkv_store against F.linear + paged kv_store")
     ps, lens = 16, [16, 5, 48, 33]

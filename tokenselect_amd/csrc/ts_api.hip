@@ -173,17 +173,19 @@ size_t ts_decode_layer_workspace_bytes(const ts_config* cfg, int32_t batch, int3
 // phases of one launch), then the top-k kernels, 0 = ts_score, ts_vote and the top-k
 // kernels (fused kernels switched off, a max-pool window above 256, a request that does
 // not fit the device).
-static int layer_selection_form(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
-  if (select_workspace(cfg, batch, max_seq_len).tokens_per_block > 0) return 2;
-  const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
-  if (max_n > 0 && cfg->pool_kernel <= 256 && score_votes_group(cfg, 1, max_seq_len) > 0) return 1;
-  return 0;
+// The second form is decided by the plan its launcher is going to follow, so that the
+// driver, the regions cleared for it and the launch cannot disagree.
+static int layer_selection_form(const ts_config* cfg, const ts_batch* bt) {
+  SeparateKernelsScope separate(bt->separate_kernels != 0);
+  if (select_workspace(cfg, bt->batch, bt->max_seq_len).tokens_per_block > 0) return 2;
+  return vote_launches_planned(cfg, bt) ? 1 : 0;
 }
 
-// The same for a batch descriptor (the host's lengths, where it carries them, change how
-// the phases are packed, not the form).
-static int layer_selection_form(const ts_config* cfg, const ts_batch* bt) {
-  return layer_selection_form(cfg, bt->batch, bt->max_seq_len);
+static int layer_selection_form(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
+  ts_batch bt{};
+  bt.batch = batch;
+  bt.max_seq_len = max_seq_len;
+  return layer_selection_form(cfg, &bt);
 }
 
 // Decode (chunk_rows == 0: one query row per request, q_cos / q_sin are the [D] rows
@@ -197,6 +199,7 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
                      ts_stream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
+  SeparateKernelsScope separate(bt->separate_kernels != 0);
   TS_REQUIRE(q && q_cos && q_sin && k_pool && v_pool && out && sel && sel_pos && sel_len, TS_EINVAL,
              "layer: NULL tensor argument");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
@@ -256,11 +259,13 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
     TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
                        zero, (hipStream_t)stream));
   }
-  if (cache) TS_TRY(ts_selcache_step(cfg, bt, qf, cache, hit, stream));
+  if (cache)
+    TS_TRY(launch_selcache(cfg, bt, qf, cache, hit, bt->rerun ? sel_len : nullptr, (hipStream_t)stream));
   if (one_launch) {
     TS_TRY(launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,
                          nullptr, 0, ws + w.select_ws, tickets, attn_tickets_per_request(cfg),
-                         (hipStream_t)stream));
+                         (hipStream_t)stream, select_wait_ticks(bt),
+                         (uint32_t)(bt->absent_workgroups > 0 ? bt->absent_workgroups : 0)));
   } else if (vote_group > 0) {
     // With max-pooling the kernel writes the pooled votes (there is no un-pooled copy).
     TS_TRY(launch_score_votes(cfg, bt, qf, k_pool, pool_rows, hit, votes, w.score_stride, topk.ws,
@@ -307,6 +312,7 @@ int ts_decode_layer_votes(const ts_config* cfg, const ts_batch* bt, const void* 
                           void* workspace, size_t workspace_bytes, ts_stream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
+  SeparateKernelsScope separate(bt->separate_kernels != 0);
   TS_REQUIRE(q && q_cos && q_sin && k_pool && votes, TS_EINVAL, "layer votes: NULL tensor argument");
   TS_REQUIRE_ALIGNED(workspace, 256, "workspace");
   TS_REQUIRE_ALIGNED(q, 16, "q");
@@ -328,7 +334,7 @@ int ts_decode_layer_votes(const ts_config* cfg, const ts_batch* bt, const void* 
   void* qf = ws + w.qf;
   int32_t* hit = cache ? (int32_t*)(ws + w.hit) : nullptr;
   const SelectWorkspace fused = select_workspace(&plain, bt->batch, bt->max_seq_len);
-  const int group = max_n > 0 ? score_votes_group(&plain, bt->batch, bt->max_seq_len) : 0;
+  const int group = vote_launches_planned(&plain, bt) ? 1 : 0;
   ZeroSet zero;
   if (group > 0) score_votes_zero_regions(&plain, bt, fused, ws + w.select_ws, &zero);
   TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
@@ -352,6 +358,7 @@ int ts_decode_layer_attend(const ts_config* cfg, const ts_batch* bt, const void*
                            size_t workspace_bytes, ts_stream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
+  SeparateKernelsScope separate(bt->separate_kernels != 0);
   TS_REQUIRE(q && votes && k_pool && v_pool && out && sel && sel_pos && sel_len, TS_EINVAL,
              "layer attend: NULL tensor argument");
   TS_REQUIRE_ALIGNED(workspace, 256, "workspace");
@@ -388,7 +395,7 @@ int ts_decode_layer_attend(const ts_config* cfg, const ts_batch* bt, const void*
   topk.clear_per_req = attn_tickets_per_request(cfg);
   ts_config plain = *cfg;
   plain.pool_kernel = -1;
-  if (max_n > 0 && score_votes_group(&plain, bt->batch, bt->max_seq_len) > 0)
+  if (vote_launches_planned(&plain, bt))
     topk.fault = score_votes_fault_word(&plain, bt->batch, bt->max_seq_len, ws + w.select_ws);
   TS_TRY(launch_topk(topk, bt->batch, max_n, (hipStream_t)stream));
   return launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, bt->batch, w.max_sel,

@@ -567,7 +567,15 @@ int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_poo
                      out, workspace, /*tickets_clear=*/false, (hipStream_t)stream);
 }
 
-size_t ts_attn_static_scratch_bytes(void) { return kStaticScratchBytes; }
+size_t ts_attn_static_scratch_bytes(void) {
+  // The query a caller makes at set-up also looks up the buffer's address on the current
+  // device, so that a first call under graph capture makes no runtime query of its own.
+  // (Without a device there is nothing to look up, and the size is still the answer.)
+  int devices = 0;
+  if (hipGetDeviceCount(&devices) == hipSuccess && devices > 0) (void)static_scratch();
+  (void)hipGetLastError();
+  return kStaticScratchBytes;
+}
 
 int ts_sparse_decode_attn_static(const ts_config* cfg, const void* q, const void* k_pool,
                                  const void* v_pool, int64_t pool_rows, const int32_t* sel,
@@ -587,6 +595,10 @@ int ts_sparse_decode_attn_static(const ts_config* cfg, const void* q, const void
              "ts_sparse_decode_attn_static: batch %d x %d heads x %d selected needs %zu bytes of "
              "scratch, the built-in buffer holds %zu; use ts_sparse_decode_attn with a workspace",
              batch, cfg->num_heads, max_sel_len, need, kStaticScratchBytes);
+  TS_REQUIRE_ALIGNED(q, 16, "q");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
+  TS_REQUIRE_ALIGNED(out, 16, "out");
   void* ptr = static_scratch();
   if (ptr == nullptr) return TS_EHIP;
   // The tickets are cleared by a fill kernel on the caller's stream (the previous call

@@ -53,8 +53,13 @@ constexpr int kZeroRegions = 4;
 struct ZeroSet {
   ZeroRegion r[kZeroRegions];
   int used = 0;
+  bool overflow = false;  // a region did not fit: the launchers refuse such a set
   void add(const ZeroRegion& region) {
-    if (region.count > 0 && region.words > 0 && used < kZeroRegions) r[used++] = region;
+    if (region.count <= 0 || region.words <= 0) return;
+    if (used < kZeroRegions)
+      r[used++] = region;
+    else
+      overflow = true;
   }
   int64_t total() const {
     int64_t t = 0;
@@ -80,6 +85,11 @@ int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const 
 int launch_rope(const void* x, void* out, const float* cos_table, const float* sin_table,
                 const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
                 const ZeroSet& zero, hipStream_t stream);
+
+// Selection-cache decision (ts_selcache.hip); gave_up_len: see ts_batch.rerun (NULL: an
+// ordinary step).
+int launch_selcache(const ts_config* cfg, const ts_batch* bt, const void* qf, const ts_selcache* cache,
+                    int32_t* hit, const int32_t* gave_up_len, hipStream_t stream);
 
 // Sparse decode attention (ts_attn.hip).  The kernel counts its workgroups in per
 // (request, KV head) tickets inside the workspace, which must be zero at launch:

@@ -61,8 +61,13 @@ __device__ __forceinline__ AppendPlan make_append_plan(const int32_t* table_row,
   return p;
 }
 
-// One whole wavefront walks the requests in order; f(b, plan) sees every request's
-// plan.  Returns the number of pages the launch takes from the list.
+// One whole wavefront walks the requests in order (64 per round, the rank of the requests
+// that need a page carried from round to round); f(b, plan) sees every request's plan.
+// Returns the number of pages the launch takes from the list: one per request that needed
+// one while the list lasted, the top `taken` entries, so that the stack stays contiguous.
+// An entry that is no page of the pool (negative, or beyond pool_rows) is taken like the
+// others and dropped: its request is left untouched this step and finds the next entry at
+// the next one, instead of meeting the same entry for ever.
 template <typename F>
 __device__ __forceinline__ int for_each_append(const int32_t* seq_lens, const int32_t* table,
                                                int64_t table_stride, int batch, const PagePool& pool,

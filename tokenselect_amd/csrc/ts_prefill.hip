@@ -747,6 +747,7 @@ int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const 
                        const float* sin_table, int64_t table_rows, void* qf, const ZeroSet& zero,
                        hipStream_t stream) {
   TS_TRY(validate_config(cfg));
+  TS_REQUIRE(!zero.overflow, TS_EINVAL, "internal: more than %d regions to clear in one launch", kZeroRegions);
   TS_REQUIRE(q && cos_table && sin_table && qf, TS_EINVAL, "ts_fingerprint: NULL tensor argument");
   TS_REQUIRE_ALIGNED(q, 16, "q");
   TS_REQUIRE_ALIGNED(cos_table, 16, "cos_table");

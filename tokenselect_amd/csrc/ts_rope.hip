@@ -43,6 +43,7 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(const uint16_t* __restr
 int launch_rope(const void* x, void* out, const float* cos_table, const float* sin_table,
                 const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
                 const ZeroSet& zero, hipStream_t stream) {
+  TS_REQUIRE(!zero.overflow, TS_EINVAL, "internal: more than %d regions to clear in one launch", kZeroRegions);
   const int64_t pairs = rows * heads * (dim / 2);
   // Enough workgroups for the clearing on the side as well: four words per thread.
   const int64_t to_clear = zero.total();

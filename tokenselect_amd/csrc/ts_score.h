@@ -129,19 +129,34 @@ void select_zero_regions(const ts_config* cfg, const SelectWorkspace& w, void* w
 // Clears the regions (the stand-alone form of what the rotation kernel does on the side).
 int launch_select_zero(const ZeroSet& zero, hipStream_t stream);
 
-// Bound of a grid-wide wait of the fused selection: 2 s of the 100 MHz clock.
-constexpr uint64_t kSelectWaitTicks = 200000000ull;
+// Bound of a grid-wide wait of the fused kernels in ticks of the 100 MHz clock: the
+// caller's ts_batch.wait_us, by default TS_DEFAULT_WAIT_US (10 ms).
+static inline uint64_t select_wait_ticks(const ts_batch* bt) {
+  return (uint64_t)(bt->wait_us ? bt->wait_us : TS_DEFAULT_WAIT_US) * 100ull;
+}
+
+// Whether the fused kernels (ts_select, the votes-only form) may serve on this thread
+// right now: the process-wide switch, unless a call is running that asked for the
+// separate kernels (ts_batch.separate_kernels).  SeparateKernelsScope is that call's guard.
+bool fused_kernels_enabled();
+struct SeparateKernelsScope {
+  explicit SeparateKernelsScope(bool on);
+  ~SeparateKernelsScope();
+  bool was;
+};
 
 // Scores and votes of a batch of any size without the [H, n] scores in memory: the
 // requests are served in phases whose scores fit the LDS of half the device (of all of it
 // for a request that needs more), the workgroups of all phases in one launch of the fused
 // kernel's votes-only form (score, statistics, votes, [max-pool]); the launch also counts
-// the first histogram level of the top-k into hist_ws.  score_votes_group() is positive
-// when a request of max_seq_len fits the device and the fused kernels are switched on:
-// else the separate kernels serve.  The workspace is that of ts_select for the whole
+// the first histogram level of the top-k into hist_ws.  vote_launches_planned() tells
+// whether the launcher's own plan serves the batch (every request fits the device, the
+// fused kernels are switched on, the max-pool window fits): else the separate kernels
+// serve.  The driver, the zero regions and the launch all go by that one plan.  The workspace is that of ts_select for the whole
 // batch; the statistics (per workgroup and merged) and the rendezvous areas
 // (score_votes_zero_regions) are zero.
-int score_votes_group(const ts_config* cfg, int batch, int max_seq_len);
+bool vote_launches_planned(const ts_config* cfg, const ts_batch* bt);
+bool vote_launches_planned(const ts_config* cfg, int batch, int max_seq_len);
 void score_votes_zero_regions(const ts_config* cfg, const ts_batch* bt, const SelectWorkspace& w,
                               void* workspace, ZeroSet* zero);
 int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
@@ -156,6 +171,6 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
                   int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
                   int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
                   int64_t vote_stride, void* workspace, uint32_t* clear, int clear_per_req,
-                  hipStream_t stream, uint64_t wait_ticks = kSelectWaitTicks, uint32_t absent = 0);
+                  hipStream_t stream, uint64_t wait_ticks, uint32_t absent);
 
 }  // namespace ts

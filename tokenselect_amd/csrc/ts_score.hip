@@ -171,15 +171,8 @@ __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const La
 constexpr int kStatsPollSleep = 12;     // x 64 clocks between a workgroup's polls for the merged statistics
 constexpr uint32_t kSelectRounds = 4;  // rendezvous of the fused kernel at most (without the max-pool's)
 
-#ifdef TS_TRACE  // development builds: per-workgroup phase timestamps of the fused kernel
-__device__ uint64_t g_trace[4096 * 24];
-extern "C" int ts_debug_trace(void* out, size_t bytes) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), bytes);
-}
-#define TS_MARK(i)                                                                              \
-  do {                                                                                          \
-    if (threadIdx.x == 0) g_trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 24 + (i)] = wall_clock64(); \
-  } while (0)
+#ifdef TS_TRACE  // development builds only: per-workgroup phase timestamps of the fused kernel
+#include "ts_trace.h"
 #else
 #define TS_MARK(i) \
   do {             \
@@ -1241,6 +1234,13 @@ static std::atomic<int> g_fused_select{1};
 
 int set_fused_select(int enable) { return g_fused_select.exchange(enable ? 1 : 0); }
 
+static thread_local bool g_separate_call = false;
+bool fused_kernels_enabled() { return g_fused_select.load() != 0 && !g_separate_call; }
+SeparateKernelsScope::SeparateKernelsScope(bool on) : was(g_separate_call) {
+  if (on) g_separate_call = true;
+}
+SeparateKernelsScope::~SeparateKernelsScope() { g_separate_call = was; }
+
 // Workgroups of the fused kernel that the current device keeps resident at once (0: the
 // shape has no fused kernel, or the runtime refused); depends on the kernel only.
 static int fused_capacity(const ts_config* cfg, bool packed, bool large) {
@@ -1298,7 +1298,7 @@ int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, boo
   if (large_out) *large_out = false;
   if (most_blocks_out) *most_blocks_out = 0;
   // Max-pool windows beyond 256 would not fit the LDS the neighbours are gathered into.
-  if ((!ignore_switch && !g_fused_select.load()) || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256)
+  if ((!ignore_switch && !fused_kernels_enabled()) || cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256)
     return 0;
   const int max_n = max_seq_len - cfg->n_init - cfg->n_local;
   if (max_n <= 0) return 0;
@@ -1427,10 +1427,16 @@ void score_votes_zero_regions(const ts_config* cfg, const ts_batch* bt, const Se
   zero->add(partials_zero_region(w, workspace, bt->batch, cfg->num_heads, chunks));
 }
 
-int score_votes_group(const ts_config* cfg, int batch, int max_seq_len) {
-  for (int g = batch; g >= 1; --g)
-    if (fused_tokens_per_block(cfg, g, max_seq_len, false, nullptr, false, nullptr) > 0) return g;
-  return 0;
+bool vote_launches_planned(const ts_config* cfg, const ts_batch* bt) {
+  if (bt->max_seq_len - cfg->n_init - cfg->n_local <= 0) return false;
+  VotePlan plan;
+  return plan_vote_launches(cfg, bt, &plan);
+}
+bool vote_launches_planned(const ts_config* cfg, int batch, int max_seq_len) {
+  ts_batch bt{};
+  bt.batch = batch;
+  bt.max_seq_len = max_seq_len;
+  return vote_launches_planned(cfg, &bt);
 }
 
 const uint32_t* score_votes_fault_word(const ts_config* cfg, int batch, int max_seq_len,
@@ -1442,6 +1448,7 @@ __global__ __launch_bounds__(256) void select_zero_kernel(ZeroSet zero) {
   clear_regions(zero, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
 }
 int launch_select_zero(const ZeroSet& zero, hipStream_t stream) {
+  TS_REQUIRE(!zero.overflow, TS_EINVAL, "internal: more than %d regions to clear in one launch", kZeroRegions);
   const int64_t blocks = std::max<int64_t>(1, std::min<int64_t>(1024, ceil_div(zero.total(), 1024)));
   hipLaunchKernelGGL(select_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, zero);
   return check_launch("select_zero_kernel");
@@ -1544,7 +1551,7 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
 // spread evenly over the XCDs; such launches were seen to wait for room that never came.)
 bool plan_vote_launches(const ts_config* cfg, const ts_batch* bt, VotePlan* plan) {
   plan->parts.clear();
-  if (!g_fused_select.load()) return false;
+  if (!fused_kernels_enabled()) return false;
   if (cfg->num_heads > kMaxHeads || cfg->pool_kernel > 256) return false;
   const int fixed = cfg->n_init + cfg->n_local;
   auto bound = [&](int b) { return bt->host_seq_lens ? std::min(bt->host_seq_lens[b], bt->max_seq_len) : bt->max_seq_len; };
@@ -1629,7 +1636,8 @@ int launch_score_votes(const ts_config* cfg, const ts_batch* bt, const void* qf,
     a.votes = votes;
     a.vote_stride = vote_stride;
     a.counters = (uint32_t*)(ws + all.counters);
-    a.spin_ticks = kSelectWaitTicks;
+    a.spin_ticks = select_wait_ticks(bt);
+    a.absent = (uint32_t)std::max(bt->absent_workgroups, 0);
     a.fault_out = bt->fault;
     a.pool_kernel = cfg->pool_kernel;
     a.pool_votes = (float*)(ws + all.pool_votes);
@@ -1728,7 +1736,7 @@ int ts_score(const ts_config* cfg, const ts_batch* bt, const void* qf, const voi
 
 int ts_score_vote_supported(const ts_config* cfg, int32_t batch, int32_t max_seq_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_seq_len < 1) return 0;
-  return (cfg->pool_kernel <= 256 && score_votes_group(cfg, batch, max_seq_len) > 0) ? 1 : 0;
+  return vote_launches_planned(cfg, batch, max_seq_len) ? 1 : 0;
 }
 
 int ts_score_vote(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
@@ -1836,7 +1844,8 @@ int ts_select_cleared(const ts_config* cfg, const ts_batch* bt, const void* qf, 
                       ts_stream_t stream) {
   return ts_select_cleared_bounded(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride,
                                    sel_len, votes, vote_stride, workspace, workspace_bytes,
-                                   kSelectWaitTicks, 0, stream);
+                                   bt ? select_wait_ticks(bt) : 1, bt ? std::max(bt->absent_workgroups, 0) : 0,
+                                   stream);
 }
 
 int ts_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,

@@ -17,6 +17,10 @@ struct SelCacheArgs {
   int n_init, n_local, top_k, max_seq_len;
   int dim;  // H*D
   int32_t* hit;
+  // A call that repeats the step's previous one after a give-up: requests whose entry of
+  // gave_up_len is negative were selecting when it happened and their cache entry is not
+  // valid (a miss whatever the cache holds); the counters have advanced already.
+  const int32_t* gave_up_len;  // or NULL
 };
 
 constexpr int kSelCacheMaxVec = 4;  // 16-byte pieces per thread: 64 heads x 128 / 8 / 256
@@ -30,7 +34,8 @@ __global__ __launch_bounds__(256) void selcache_kernel(SelCacheArgs a) {
   }
   const uint16_t* q = a.qf + (size_t)b * a.dim;
   uint16_t* qc = a.q_cache + (size_t)b * a.dim;
-  const bool have = a.cache_len[b] > 0;  // is_first_query is false
+  const bool have = a.cache_len[b] > 0 &&  // is_first_query is false
+                    !(a.gave_up_len && a.gave_up_len[b] < 0);
 
   // dim = H * 128 elements, at most kMaxVec 16-byte pieces per thread, all requested at
   // once (one piece per thread and pass: a loop of dependent 2-byte loads took 8 us).
@@ -82,17 +87,15 @@ __global__ __launch_bounds__(256) void selcache_kernel(SelCacheArgs a) {
   }
   if (threadIdx.x == 0) {
     a.hit[b] = is_hit ? 1 : 0;
-    if (is_hit) a.counters[2 * b] += 1;  // skip_count, tr.py:420
-    a.counters[2 * b + 1] += 1;          // retrieval_count, tr.py:421
+    if (a.gave_up_len == nullptr) {
+      if (is_hit) a.counters[2 * b] += 1;  // skip_count, tr.py:420
+      a.counters[2 * b + 1] += 1;          // retrieval_count, tr.py:421
+    }
   }
 }
 
-}  // namespace ts
-
-using namespace ts;
-
-extern "C" int ts_selcache_step(const ts_config* cfg, const ts_batch* bt, const void* qf,
-                                const ts_selcache* cache, int32_t* hit, ts_stream_t stream) {
+int launch_selcache(const ts_config* cfg, const ts_batch* bt, const void* qf, const ts_selcache* cache,
+                    int32_t* hit, const int32_t* gave_up_len, hipStream_t stream) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
   TS_REQUIRE(qf && cache && hit, TS_EINVAL, "ts_selcache_step: NULL argument");
@@ -114,6 +117,16 @@ extern "C" int ts_selcache_step(const ts_config* cfg, const ts_batch* bt, const 
   TS_REQUIRE(a.dim % 8 == 0 && a.dim <= kSelCacheMaxVec * 256 * 8, TS_ESHAPE,
              "ts_selcache_step: %d query elements per request (at most %d)", a.dim, kSelCacheMaxVec * 256 * 8);
   a.hit = hit;
-  hipLaunchKernelGGL(selcache_kernel, dim3((unsigned)bt->batch), dim3(256), 0, (hipStream_t)stream, a);
+  a.gave_up_len = gave_up_len;
+  hipLaunchKernelGGL(selcache_kernel, dim3((unsigned)bt->batch), dim3(256), 0, stream, a);
   return check_launch("selcache_kernel");
+}
+
+}  // namespace ts
+
+using namespace ts;
+
+extern "C" int ts_selcache_step(const ts_config* cfg, const ts_batch* bt, const void* qf,
+                                const ts_selcache* cache, int32_t* hit, ts_stream_t stream) {
+  return launch_selcache(cfg, bt, qf, cache, hit, nullptr, (hipStream_t)stream);
 }

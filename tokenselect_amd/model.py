@@ -116,6 +116,9 @@ class Decoder:
         self.caches: List[Optional[SelectionCache]] = [
             SelectionCache.allocate(self.cfg, B, device) if query_cache else None
             for _ in range(mc.layers)]
+        # Per-call options handed to the layer (tests force a give-up through them).
+        self.layer_options = {}
+        self.steps_redone = 0
 
     def _norm(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         return F.rms_norm(x, (self.mc.hidden,), w, self.mc.rms_eps)
@@ -148,7 +151,8 @@ class Decoder:
                 ops.kv_store(cfg, k, v, loc, self.k_pools[l], self.v_pools[l], self.table,
                              self.num_tokens[l])
             attn, sel, _, sel_len = self.attention(
-                q, self.k_pools[l], self.v_pools[l], Batch(self.num_tokens[l], self.table, max_len, host_seq_lens=host_lens),
+                q, self.k_pools[l], self.v_pools[l],
+                Batch(self.num_tokens[l], self.table, max_len, host_seq_lens=host_lens, **self.layer_options),
                 self.caches[l])
             if trace is not None:
                 if k is None:   # the rows as they landed in the pools
@@ -162,10 +166,54 @@ class Decoder:
         return F.linear(self._norm(x, self.final_norm), self.lm_head)
 
     @torch.no_grad()
-    def generate(self, tokens: torch.Tensor, steps: int) -> torch.Tensor:
-        """Greedy decoding: ``[steps, B]`` token ids, no host synchronisation inside."""
+    def decode_step_checked(self, tokens: torch.Tensor):
+        """:meth:`decode_step` the way a serving loop runs it: the next tokens are read
+        back to the host, and at that synchronisation point a fused selection kernel that
+        gave up anywhere in the step is noticed.  The step is then undone (the token
+        counts go back by one; the slots, and so the stored K/V, are the same when it
+        runs again; selection-cache entries, which the failed launch may have half
+        written, are dropped, so the requests select afresh) and repeated with the
+        separate kernels, which the model keeps from then on.  Returns ``(logits, next
+        tokens on the device, next tokens on the host)``."""
+        before = self.decoded
+        try:
+            logits = self.decode_step(tokens)
+            nxt = logits.argmax(dim=-1)
+            host = nxt.cpu()
+            failed = self.attention.gave_up()
+        except ops.SelectionGaveUp:  # a later layer's call saw the word before the step ended
+            torch.cuda.current_stream().synchronize()
+            failed = True
+        if failed:
+            self.attention._latch()
+            self.decoded = before
+            lens = torch.tensor([c + before for c in self.contexts], dtype=torch.int32)
+            self.num_tokens.copy_(lens.repeat(self.mc.layers, 1))
+            for cache in self.caches:
+                if cache is not None:
+                    cache.cache_len.zero_()
+            self.layer_options = {k: v for k, v in self.layer_options.items()
+                                  if k not in ("absent_workgroups", "wait_us")}
+            self.steps_redone += 1
+            logits = self.decode_step(tokens)
+            nxt = logits.argmax(dim=-1)
+            host = nxt.cpu()
+        return logits, nxt, host
+
+    @torch.no_grad()
+    def generate(self, tokens: torch.Tensor, steps: int, read_back: bool = False) -> torch.Tensor:
+        """Greedy decoding: ``[steps, B]`` token ids.  Without ``read_back`` there is no
+        host synchronisation inside, and a selection that gave up is reported when the
+        loop ends (SelectionGaveUp: the tokens are not valid); with it every step's tokens
+        go to the host as a server's would, and a step that gave up is redone there."""
         out = torch.empty((steps, self.batch), dtype=torch.int64, device=self.device)
         for t in range(steps):
-            tokens = self.decode_step(tokens).argmax(dim=-1)
+            if read_back:
+                tokens = self.decode_step_checked(tokens)[1]
+            else:
+                tokens = self.decode_step(tokens).argmax(dim=-1)
             out[t] = tokens
+        if not read_back:
+            torch.cuda.current_stream().synchronize()
+            self.attention.check()
         return out

@@ -69,6 +69,14 @@ class Batch:
     # framework's CPU copy of the lengths), or None: a batch too large for one selection
     # launch is then scored in phases packed by these bounds instead of by max_seq_len.
     host_seq_lens: Optional[torch.Tensor] = None
+    # Per-call options (``ts_batch``): take the separate kernels for this call; the call
+    # repeats the step's previous one after a give-up; bound of a grid-wide wait in
+    # microseconds (0: the library's 10 ms); workgroups that never arrive (tests of the
+    # give-up path only).
+    separate_kernels: bool = False
+    rerun: bool = False
+    wait_us: int = 0
+    absent_workgroups: int = 0
 
     @property
     def batch(self) -> int:
@@ -76,10 +84,12 @@ class Batch:
 
 
 class SelectionGaveUp(RuntimeError):
-    """A grid-wide wait of the single-launch selection ran into its bound: the launch
-    did not have the device to itself (its workgroups were not all resident together)
-    and what it selected, and what was attended over, is not valid.  Also raised when a
-    request was longer on the device than ``Batch.host_seq_lens`` said."""
+    """A grid-wide wait of a fused selection kernel ran into its bound: the launch did
+    not have the device to itself (its workgroups were not all resident together) and
+    what it selected, and what was attended over, is not valid.  Also raised when a
+    request was longer on the device than ``Batch.host_seq_lens`` said.  Raised only for
+    a give-up that nobody recovered at a synchronisation point (``recover()``); the object
+    that raises has switched itself to the separate kernels, so retrying works."""
 
 
 def fault_word() -> torch.Tensor:
@@ -88,15 +98,61 @@ def fault_word() -> torch.Tensor:
     return torch.zeros((1,), dtype=torch.int32).pin_memory()
 
 
+def gave_up(word: Optional[torch.Tensor]) -> bool:
+    """Whether ``word`` has been set by an earlier launch.  A plain host read: a set word
+    is seen at the latest after the next synchronisation."""
+    return word is not None and int(word[0]) != 0
+
+
+_GAVE_UP_MESSAGE = (
+    "a fused selection kernel gave up waiting for its workgroups (is another stream or process "
+    "using the GPU?), or a request was longer than its entry of host_seq_lens; results since the "
+    "last check are not valid.  Rerun the step with the separate kernels (Batch.separate_kernels, "
+    "or recover() of the layer object)")
+
+
 def raise_if_gave_up(word: Optional[torch.Tensor]) -> None:
-    """Raises SelectionGaveUp when ``word`` has been set by an earlier launch.  A plain
-    host read: a set word is seen at the latest after the next synchronisation."""
-    if word is not None and int(word[0]) != 0:
-        raise SelectionGaveUp(
-            "ts_select gave up waiting for its workgroups (is another stream or process using the "
-            "GPU?), or a request was longer than its entry of host_seq_lens; results since the last "
-            "check are not valid.  Serialise the GPU work, or call ops.set_fused_select(False) to "
-            "use the separate kernels, clear the word and rerun")
+    """Raises SelectionGaveUp when ``word`` has been set by an earlier launch."""
+    if gave_up(word):
+        raise SelectionGaveUp(_GAVE_UP_MESSAGE)
+
+
+class _GiveUpLatch:
+    """What DecodeLayer and PrefillChunk share: the pinned fault word, the switch to the
+    separate kernels that a give-up latches for the object, and the options of a call."""
+
+    def _init_latch(self):
+        self.fault = fault_word()
+        self.separate = False  # latched by a give-up: the separate kernels from then on
+
+    def gave_up(self) -> bool:
+        """Whether a selection of this object gave up since the last check (a host memory
+        read; meaningful once the stream has been synchronised)."""
+        return gave_up(self.fault)
+
+    def _latch(self) -> None:
+        self.separate = True
+        self.fault.zero_()
+
+    def check(self) -> None:
+        """For callers that did not recover a give-up where they synchronised: switches the
+        object to the separate kernels, clears the word and raises SelectionGaveUp (the
+        outputs since the last check are not valid; a retry now succeeds).  Runs at the
+        start of every call."""
+        if self.gave_up():
+            self._latch()
+            raise SelectionGaveUp(_GAVE_UP_MESSAGE + "; this object now uses the separate kernels")
+
+    def _options(self, bt: "Batch", rerun: bool = False) -> "Batch":
+        kw = {}
+        if bt.fault is None:
+            kw["fault"] = self.fault
+        if self.separate and not bt.separate_kernels:
+            kw["separate_kernels"] = True
+        if rerun:
+            kw["rerun"] = True
+            kw["absent_workgroups"] = 0
+        return dataclasses.replace(bt, **kw) if kw else bt
 
 
 @dataclass
@@ -170,7 +226,9 @@ def _c_batch(cfg: LayerConfig, bt: Batch) -> TsBatch:
         raise ValueError("host_seq_lens must be a contiguous [B] int32 tensor on the CPU")
     host = bt.host_seq_lens.data_ptr() if bt.host_seq_lens is not None else None
     return TsBatch(bt.batch, int(bt.max_seq_len), _p(bt.seq_lens), _p(bt.table),
-                   int(bt.table.stride(0)), _p(bt.k_per_req), _p(bt.fault), host)
+                   int(bt.table.stride(0)), _p(bt.k_per_req), _p(bt.fault), host,
+                   1 if bt.separate_kernels else 0, 1 if bt.rerun else 0, int(bt.wait_us),
+                   int(bt.absent_workgroups))
 
 
 def _c_cache(cache: Optional[SelectionCache], cfg: LayerConfig, batch: int):
@@ -627,9 +685,15 @@ def scoring_cos_sin(head_dim: int, rope_base: float, rope_scale, n_local: int, d
     return emb.cos().to(device).contiguous(), emb.sin().to(device).contiguous()
 
 
-class DecodeLayer:
+class DecodeLayer(_GiveUpLatch):
     """One layer of the patched decode forward after the KV store
-    (tr.py:791-825) as a single library call; buffers are allocated once."""
+    (tr.py:791-825) as a single library call; buffers are allocated once.
+
+    A fused selection kernel that gave up (``SelectionGaveUp``) has left ``sel_len[b] = -1``
+    and an output attended over nothing.  A caller that synchronises before the output is
+    consumed calls :meth:`recover` there with the arguments of the call: it repeats the
+    step's selection and attention with the separate kernels (the KV store before the
+    layer is not repeated) and keeps the object on them."""
 
     def __init__(self, cfg: LayerConfig, batch: int, max_seq_len: int, device):
         self.cfg, self.batch, self.max_seq_len = cfg, batch, max_seq_len
@@ -645,20 +709,29 @@ class DecodeLayer:
         self.sel = torch.empty((batch, cfg.max_sel), dtype=torch.int32, device=device)
         self.sel_pos = torch.empty_like(self.sel)
         self.sel_len = torch.empty((batch,), dtype=torch.int32, device=device)
-        self.fault = fault_word()
+        self._init_latch()
 
-    def check(self) -> None:
-        """Raises SelectionGaveUp if a selection of this layer gave up since the last
-        check.  Costs a host memory read; call it wherever the stream has been
-        synchronised anyway (it also runs at the start of every call)."""
-        raise_if_gave_up(self.fault)
+    def recover(self, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch,
+                cache: Optional[SelectionCache] = None, out: Optional[torch.Tensor] = None):
+        """Synchronises the stream; when the last call gave up, repeats it (same
+        arguments) with the separate kernels, which stay switched on for this object, and
+        returns what the call returns; ``None`` when there was nothing to recover.  With
+        the selection cache the requests that gave up select afresh, the others hit
+        again, and the counters do not advance twice."""
+        torch.cuda.current_stream().synchronize()
+        if not self.gave_up():
+            return None
+        self._latch()
+        return self._run(q, k_pool, v_pool, bt, cache, out, rerun=True)
 
     def __call__(self, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch,
                  cache: Optional[SelectionCache] = None, out: Optional[torch.Tensor] = None):
-        cfg = self.cfg
         self.check()
-        if bt.fault is None:
-            bt = dataclasses.replace(bt, fault=self.fault)
+        return self._run(q, k_pool, v_pool, bt, cache, out)
+
+    def _run(self, q, k_pool, v_pool, bt, cache, out, rerun: bool = False):
+        cfg = self.cfg
+        bt = self._options(bt, rerun)
         cb = _c_batch(cfg, bt)
         if bt.batch > self.batch or bt.max_seq_len > self.max_seq_len:
             raise ValueError("batch / max_seq_len exceed what this DecodeLayer was sized for")
@@ -690,8 +763,7 @@ class DecodeLayer:
               cache: Optional[SelectionCache] = None) -> torch.Tensor:
         cfg = self.cfg
         self.check()
-        if bt.fault is None:
-            bt = dataclasses.replace(bt, fault=self.fault)
+        bt = self._options(bt)
         cb = _c_batch(cfg, bt)
         if bt.batch > self.batch or bt.max_seq_len > self.max_seq_len:
             raise ValueError("batch / max_seq_len exceed what this DecodeLayer was sized for")
@@ -712,8 +784,7 @@ class DecodeLayer:
     def attend(self, q: torch.Tensor, votes: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                bt: Batch, cache: Optional[SelectionCache] = None, out: Optional[torch.Tensor] = None):
         cfg = self.cfg
-        if bt.fault is None:
-            bt = dataclasses.replace(bt, fault=self.fault)
+        bt = self._options(bt)
         cb = _c_batch(cfg, bt)
         _need(q, "q", torch.bfloat16)
         _need(votes, "votes", torch.float32, 2)
@@ -813,9 +884,10 @@ def sparse_prefill_attention(cfg: LayerConfig, q: torch.Tensor, k_pool: torch.Te
     return out
 
 
-class PrefillChunk:
+class PrefillChunk(_GiveUpLatch):
     """One chunk of the patched extend forward after its KV store (tr.py:735-773) as a
-    single library call, for one request; buffers are allocated once."""
+    single library call, for one request; buffers are allocated once.  :meth:`recover`
+    as for :class:`DecodeLayer`."""
 
     def __init__(self, cfg: LayerConfig, max_seq_len: int, device, max_rows: int = 512):
         self.cfg, self.max_seq_len, self.max_rows = cfg, max_seq_len, max_rows
@@ -829,18 +901,26 @@ class PrefillChunk:
         self.sel = torch.empty((1, cfg.max_sel), dtype=torch.int32, device=device)
         self.sel_pos = torch.empty_like(self.sel)
         self.sel_len = torch.empty((1,), dtype=torch.int32, device=device)
-        self.fault = fault_word()
+        self._init_latch()
 
-    def check(self) -> None:
-        """As DecodeLayer.check()."""
-        raise_if_gave_up(self.fault)
+    def recover(self, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch,
+                out: Optional[torch.Tensor] = None):
+        """As :meth:`DecodeLayer.recover`: after a synchronisation, repeats a chunk whose
+        selection gave up with the separate kernels; ``None`` when nothing gave up."""
+        torch.cuda.current_stream().synchronize()
+        if not self.gave_up():
+            return None
+        self._latch()
+        return self._run(q, k_pool, v_pool, bt, out, rerun=True)
 
     def __call__(self, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch,
                  out: Optional[torch.Tensor] = None):
-        cfg = self.cfg
         self.check()
-        if bt.fault is None:
-            bt = dataclasses.replace(bt, fault=self.fault)
+        return self._run(q, k_pool, v_pool, bt, out)
+
+    def _run(self, q, k_pool, v_pool, bt, out, rerun: bool = False):
+        cfg = self.cfg
+        bt = self._options(bt, rerun)
         cb = _c_batch(cfg, bt)
         _need(q, "q", torch.bfloat16, 2)
         rows = q.shape[0]

@@ -390,24 +390,34 @@ class TokenRetriever:
         bt = ops.Batch(self._num_tokens_dev[layer_id:layer_id + 1],
                        self.token_indices[layer_id:layer_id + 1], current_num_tokens)
         cache = self._cache(layer_id)
-        hit = ops.selcache_step(cfg, bt, qf, cache) if cache is not None else None
         k_buffer = self.token_fingerprints[layer_id]
         # The large buffers are kept between calls, sized for the longest table.
         key = ("select", n_init, n_local, topk, KERNEL_SIZE)
         sized = ops.Batch(bt.seq_lens, bt.table, self.max_num_tokens)
-        if ops.select_supported(cfg, 1, self.max_num_tokens):
+        one_launch = not getattr(self, "_separate", False) and \
+            ops.select_supported(cfg, 1, self.max_num_tokens)
+        held = self._layers.get(key)
+        if one_launch and held is not None and ops.gave_up(held[1]):
+            # An earlier launch gave up and nobody noticed at a synchronisation point: what it
+            # selected was not valid.  From now on the separate kernels, whose workgroups never
+            # wait for each other; the caller retries the request.
+            self._separate = True
+            del self._layers[key]
+            raise ops.SelectionGaveUp(
+                "the single-launch selection gave up waiting for its workgroups (another stream "
+                "or process on the GPU?): the selection of an earlier call was not valid; this "
+                "retriever now uses the separate kernels, retry the request")
+        hit = ops.selcache_step(cfg, bt, qf, cache) if cache is not None else None
+        if one_launch:
             # the whole selection in one launch
-            held = self._layers.get(key)
             if held is None:
                 held = (ops.select_workspace(cfg, sized, self.device), ops.fault_word())
                 self._layers[key] = held
             workspace, fault = held
-            ops.raise_if_gave_up(fault)
             bt.fault = fault
             sel, _, _, _, _ = ops.select(cfg, bt, qf, k_buffer, hit=hit, cache=cache,
                                          workspace=workspace)
         else:
-            held = self._layers.get(key)
             if held is None:
                 held = ops.score_buffers(cfg, sized, self.device)
                 self._layers[key] = held
