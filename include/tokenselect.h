@@ -153,7 +153,7 @@ int ts_version(void);
 const char* ts_last_error(void);
 
 /* TS_OK when the library supports this configuration (head_dim 128; Hkv in
- * {1,2,4,8}; H/Hkv in {1,2,4,7,8}; power-of-two page size), else the error. */
+ * {1,2,4,8}; H/Hkv from 1 to 8; power-of-two page size), else the error. */
 int ts_check_config(const ts_config* cfg);
 
 /* RotaryEmbedding.apply_rotary_pos_emb (tr.py:98-107):
@@ -411,8 +411,10 @@ int ts_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const floa
 
 /* FlashInfer paged prefill over the selected slots with causal=True
  * (tr.py:759-771), page size 1, one request: query row i of q [rows, H, D] sits
- * at position S - rows + i (S = *sel_len <= max_sel_len, S >= rows), is rotated
- * to it, and attends to the keys sel[j], rotated to j, for j <= S - rows + i;
+ * at position S - rows + i (S = *sel_len <= max_sel_len), is rotated
+ * to it, and attends to the keys sel[j], rotated to j, for j <= S - rows + i
+ * (FlashInfer's alignment of the last query row with the last key; with fewer keys
+ * than rows the first rows - S rows see no key and their output is zero);
  * GQA head h reads KV head h / (H/Hkv); sm_scale, logit_cap as in
  * ts_sparse_decode_attn.  out: [rows, H, D] bf16.  The workspace receives the
  * selected keys, rotated, and the selected values, transposed, once per call
@@ -425,8 +427,11 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
 
 /* One chunk of the extend forward after its KV store (tr.py:735-773):
  * fingerprint -> selection -> causal sparse attention, for the single request
- * of bt (batch 1; seq_lens[0] already counts the chunk).  rows <= n_local, so
- * that the chunk's own tokens are the tail of the selected list.  Workspace as
+ * of bt (batch 1; seq_lens[0] already counts the chunk).  While rows <= n_local the
+ * chunk's own tokens are the tail of the selected list; a longer chunk is served as
+ * the reference serves it (tr.py:716-738 with any N_Local): the list ends with the
+ * last n_local tokens, the chunk's earlier rows are candidates like any other token,
+ * and row i still sees the list's entries j <= S - rows + i.  Workspace as
  * for ts_decode_layer (ts_decode_layer_workspace_bytes(cfg, 1, max_seq_len)).
  * q, out: [rows, H*D] bf16. */
 int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, int32_t rows,

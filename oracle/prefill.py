@@ -14,8 +14,14 @@ and sees key ``j`` iff ``j <= S - m + i``; with ``pos_encoding_mode="ROPE_LLAMA"
 the query is rotated to that position and key ``j`` to ``j``; GQA head ``h``
 reads KV head ``h // (H / Hkv)``; ``logit = sm_scale * q' . k'``, optional soft
 cap, fp32 softmax, output in the query dtype.  The chunk's own tokens are the
-last ``m`` entries of the selected list (they lie inside the local window as
-long as ``n_local >= m``), which is what makes the causal mask meaningful.
+last ``m`` entries of the selected list as long as ``n_local >= m`` (they lie inside
+the local window), which is what makes the causal mask meaningful; the reference
+runs any ``N_Local`` (its ``patch()`` default is 16 with 512-row chunks,
+tr.py:885-894), and the alignment above then applies to whatever the list holds.
+With fewer keys than rows (``S < m``) the first ``m - S`` rows see no key; FlashInfer
+normalises such a row with a zero reciprocal, so its output is zero.  **Parity
+unpinned** for that corner (FlashInfer is not in the tree): pinned only by the
+mathematics of the mask (``tests/test_oracle.py``).
 """
 
 from typing import List, Optional
@@ -33,14 +39,13 @@ def sparse_prefill_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torc
                              rope_scale: float = 1.0, logit_cap: float = 0.0,
                              rope_mode: str = "ROPE_LLAMA", causal: bool = True) -> torch.Tensor:
     """``q`` [m, H, D] bf16 un-rotated, pools [P, Hkv, D] bf16, ``slots`` [S]
-    physical KV slots in attention order (S >= m).  Returns [m, H, D] in q's dtype."""
+    physical KV slots in attention order.  Returns [m, H, D] in q's dtype; rows that see
+    no key (position ``S - m + i`` negative) are zero."""
     m, num_heads, _ = q.shape
     num_kv = k_pool.shape[1]
     group = num_heads // num_kv
     idx = slots.to(torch.int64)
     s_len = idx.shape[0]
-    if s_len < m:
-        raise ValueError("fewer keys than query rows")
     k = k_pool[idx].float()                                # [S, Hkv, D]
     v = v_pool[idx].float()
     qf = q.float()
@@ -58,7 +63,11 @@ def sparse_prefill_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torc
     if causal:
         visible = torch.arange(s_len).unsqueeze(0) <= q_pos.unsqueeze(1)   # [m, S]
         logits = logits.masked_fill(~visible.unsqueeze(0), float("-inf"))
+        blind = ~visible.any(dim=1)                                        # [m]
+        logits[:, blind] = 0.0                                             # (softmax of -inf rows is NaN)
     p = torch.softmax(logits, dim=-1)
+    if causal:
+        p[:, blind] = 0.0
     out = torch.einsum("hms,shd->mhd", p, v[:, kv_of_head])
     return out.to(q.dtype)
 

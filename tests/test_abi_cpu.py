@@ -60,12 +60,13 @@ def test_config_validation(lib):
     assert lib.ts_check_config(ctypes.byref(cfg(head_dim=64))) == _lib.TS_ESHAPE
     assert "head_dim 64" in err(lib)
     assert lib.ts_check_config(ctypes.byref(cfg(num_heads=30))) == _lib.TS_ESHAPE
-    assert lib.ts_check_config(ctypes.byref(cfg(num_heads=24, num_kv_heads=8))) == _lib.TS_ESHAPE
+    assert lib.ts_check_config(ctypes.byref(cfg(num_heads=72, num_kv_heads=8))) == _lib.TS_ESHAPE
+    assert lib.ts_check_config(ctypes.byref(cfg(num_heads=24, num_kv_heads=3))) == _lib.TS_ESHAPE
     assert lib.ts_check_config(ctypes.byref(cfg(page_size=12))) == _lib.TS_EINVAL
     assert lib.ts_check_config(ctypes.byref(cfg(top_k=0))) == _lib.TS_EINVAL
     assert lib.ts_check_config(ctypes.byref(cfg(rope_mode=7))) == _lib.TS_EINVAL
     assert lib.ts_check_config(ctypes.byref(cfg(rope_theta=0.0))) == _lib.TS_EINVAL
-    for hkv, g in [(1, 8), (2, 2), (4, 7), (8, 4), (8, 8), (4, 1)]:
+    for hkv, g in [(1, 8), (2, 2), (4, 7), (8, 4), (8, 8), (4, 1), (8, 3), (2, 6), (4, 5)]:
         assert lib.ts_check_config(ctypes.byref(cfg(num_heads=hkv * g, num_kv_heads=hkv))) == 0
 
 

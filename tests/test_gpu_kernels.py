@@ -22,6 +22,9 @@ SHAPES = [
     dict(num_heads=4, num_kv_heads=2, rope_theta=1e4),
     dict(num_heads=8, num_kv_heads=8, rope_theta=1e4),    # MHA
     dict(num_heads=16, num_kv_heads=4, rope_theta=1e4),
+    dict(num_heads=24, num_kv_heads=8, rope_theta=5e5),   # Llama-3.2-3B: three query heads per KV head
+    dict(num_heads=12, num_kv_heads=2, rope_theta=1e6),   # Qwen2-1.5B: six
+    dict(num_heads=20, num_kv_heads=4, rope_theta=1e4),   # five
 ]
 
 

@@ -181,15 +181,23 @@ def test_selection_cache_trace(dev, anchor_jump):
     assert 0 < total_hits < B * steps, "the trace must exercise both hits and misses"
 
 
-def test_patched_extend_forward(dev):
+@pytest.mark.parametrize("defaults", [False, True], ids=["chunk 32 in a window of 32", "patch() defaults"])
+def test_patched_extend_forward(dev, defaults):
     """Chunked prefill through the patched RadixAttention.forward in EXTEND mode: a
     prompt of three chunks (the last one ragged) on an empty cache, then one more
-    extend on top; every chunk against the oracle's extend loop on the same pools."""
-    say("patched extend forward: 2 layers, H8/kv2, chunk 32, top_k 24")
+    extend on top; every chunk against the oracle's extend loop on the same pools.
+    Second case: the reference's own patch() defaults (top_k 16, n_init 1, n_local 16,
+    tr.py:885-894) with its 512-row chunks, which are far longer than the local window."""
     H, Hkv, D, layers = 8, 2, 128, 2
-    n_init, n_local, top_k, chunk = 4, 32, 24, 32
-    tr.patch(rope_base=1e4, rope_scale=1, rope_model="ROPE_LLAMA", max_n_tokens=512, top_k=top_k,
-             n_init=n_init, n_local=n_local)
+    if defaults:
+        n_init, n_local, top_k, chunk, rope_base, prompts = 1, 16, 16, 512, 1e6, (600, 45)
+        say("patched extend forward: 2 layers, H8/kv2, patch() defaults, chunk 512")
+        tr.patch()
+    else:
+        n_init, n_local, top_k, chunk, rope_base, prompts = 4, 32, 24, 32, 1e4, (80, 45)
+        say("patched extend forward: 2 layers, H8/kv2, chunk 32, top_k 24")
+        tr.patch(rope_base=1e4, rope_scale=1, rope_model="ROPE_LLAMA", max_n_tokens=512, top_k=top_k,
+                 n_init=n_init, n_local=n_local)
     tr.PREFILL_CHUNK_SIZE = chunk
     try:
         g = torch.Generator(device=dev).manual_seed(17)
@@ -201,9 +209,9 @@ def test_patched_extend_forward(dev):
         attns = [sg.RadixAttention(H, D, D ** -0.5, Hkv, layer_id=l) for l in range(layers)]
         ref_k = [pool.k_buffer[l].cpu().clone() for l in range(layers)]
         ref_v = [pool.v_buffer[l].cpu().clone() for l in range(layers)]
-        ref_tab = [torch.zeros(512, dtype=torch.int32) for _ in range(layers)]
+        ref_tab = [torch.zeros(1024, dtype=torch.int32) for _ in range(layers)]
         L = 0
-        for T in (80, 45):
+        for T in prompts:
             loc = slots[L:L + T].contiguous()
             meta = sg.InputMetadata(sg.ForwardMode.EXTEND, retriever, pool, loc)
             for l, attn in enumerate(attns):
@@ -222,7 +230,7 @@ def test_patched_extend_forward(dev):
                 details = []
                 ref = oracle.prefill.prefill(q.cpu(), k.cpu().view(T, Hkv, D), v.cpu().view(T, Hkv, D),
                                              ref_k[l], ref_v[l], ref_tab[l], L, loc.cpu(), H, D, n_init,
-                                             n_local, top_k, 1e4, 1, D ** -0.5, chunk=chunk,
+                                             n_local, top_k, rope_base, 1, D ** -0.5, chunk=chunk,
                                              details=details, qf_overrides=qfs)
                 assert torch.equal(pool.k_buffer[l].cpu(), ref_k[l])
                 err = (got.cpu().float() - ref.float()).abs().max().item()

@@ -18,6 +18,9 @@ SHAPES = [
     dict(num_heads=8, num_kv_heads=1, rope_theta=1e4),
     dict(num_heads=4, num_kv_heads=2, rope_theta=1e4),
     dict(num_heads=8, num_kv_heads=8, rope_theta=1e4),
+    dict(num_heads=24, num_kv_heads=8, rope_theta=5e5),   # Llama-3.2-3B: three query heads per KV head
+    dict(num_heads=12, num_kv_heads=2, rope_theta=1e6),   # Qwen2-1.5B: six
+    dict(num_heads=20, num_kv_heads=4, rope_theta=1e4),   # five
 ]
 IDS = [f"H{s['num_heads']}kv{s['num_kv_heads']}" for s in SHAPES]
 
@@ -178,19 +181,31 @@ def test_sparse_prefill_attention_moving_maximum(dev, direction):
 
 
 def test_sparse_prefill_attention_fewer_keys_than_rows(dev):
-    """A selection that reports fewer keys than the chunk has rows (a selection that gave
-    up reports -1) leaves a defined output: zeros."""
+    """A selection that reports no keys (one that gave up reports -1) leaves a defined output:
+    zeros.  With fewer keys than rows (a chunk longer than the selected list) the first
+    rows - S rows sit at negative positions, see nothing and are zero; the others attend to
+    their key prefix as the oracle's do."""
     m = 40
     say("prefill attention with fewer keys than rows")
     wl = workloads.build("pf", SHAPES[1], [100], [8], 1, dev, seed=25, n_init=1, n_local=m)
     c = wl.cfg
-    q = torch.ones((m, c.num_heads * 128), dtype=torch.bfloat16, device=dev)
+    g = torch.Generator(device=dev).manual_seed(26)
+    q = torch.randn((m, c.num_heads * 128), generator=g, device=dev).bfloat16()
     sel = wl.table[0, :100].contiguous()
-    for reported in (-1, 0, m - 1):
+    for reported in (-1, 0):
         sel_len = torch.tensor([reported], dtype=torch.int32, device=dev)
         out = ops.sparse_prefill_attention(c, q, wl.k_pool, wl.v_pool, sel, sel_len)
         torch.cuda.synchronize()
         assert torch.count_nonzero(out).item() == 0, reported
+    for S, width in ((m - 1, 100), (7, 100), (17, 17), (33, 33)):
+        sel_len = torch.tensor([S], dtype=torch.int32, device=dev)
+        out = ops.sparse_prefill_attention(c, q, wl.k_pool, wl.v_pool, sel[:width].contiguous(), sel_len)
+        torch.cuda.synchronize()
+        ref = oracle.prefill.sparse_prefill_attention(q.cpu().view(m, c.num_heads, 128), wl.k_pool.cpu(),
+                                                      wl.v_pool.cpu(), sel[:S].cpu(), _sm(c), c.rope_theta)
+        assert torch.count_nonzero(out[:m - S]).item() == 0, S
+        assert torch.count_nonzero(out[m - S]).item() > 0, S
+        assert (out.cpu().float() - ref.reshape(m, -1).float()).abs().max().item() <= 2e-2, S
 
 
 @pytest.mark.parametrize("rows", [1, 7, 8, 9, 513, 8184, 8200])
@@ -323,9 +338,41 @@ def test_prefill_short_context_attends_densely(dev):
     assert (out.cpu().float() - ref.reshape(m, -1).float()).abs().max().item() <= 2e-2
 
 
-def test_prefill_chunk_rejects_rows_beyond_the_local_window(dev):
-    wl = workloads.build("pf", SHAPES[3], [500], [16], 1, dev, seed=15, n_init=4, n_local=16)
-    layer = ops.PrefillChunk(wl.cfg, 500, dev, max_rows=64)
-    q = torch.zeros((32, wl.cfg.num_heads * 128), dtype=torch.bfloat16, device=dev)
-    with pytest.raises(RuntimeError, match="local window"):
-        layer(q, wl.k_pool, wl.v_pool, wl.batch)
+@pytest.mark.parametrize("case", ["rows 64, window 16", "the reference's defaults"])
+def test_prefill_chunk_longer_than_the_local_window(dev, case):
+    """The reference runs any N_Local with its 512-row chunks (its patch() defaults are
+    n_init 1, top_k 16, n_local 16): the selected list then ends with the last n_local
+    tokens only, the chunk's earlier rows are candidates like any other token, and row i
+    sees the entries j <= S - rows + i of the list; with the defaults the list (33 entries)
+    is shorter than the chunk, and the rows before the last 33 see nothing."""
+    if case == "rows 64, window 16":
+        L, m, kw = 500, 64, dict(n_init=4, n_local=16, top_k=96)
+    else:
+        L, m, kw = 700, 100, dict(n_init=1, n_local=16, top_k=16)
+    say(f"prefill chunk beyond the local window: {case}")
+    wl = workloads.build("pf", SHAPES[3], [L], [kw["top_k"]], 1, dev, seed=15, **kw)
+    c = wl.cfg
+    g = torch.Generator(device=dev).manual_seed(16)
+    q = torch.randn((m, c.num_heads * 128), generator=g, device=dev).bfloat16()
+    layer = ops.PrefillChunk(c, L, dev, max_rows=m)
+    out, sel, sel_pos, sel_len = layer(q, wl.k_pool, wl.v_pool, wl.batch)
+    torch.cuda.synchronize()
+    S = int(sel_len[0])
+    assert S == c.n_init + c.top_k + c.n_local
+    qf = ops.fingerprint(c, q.view(m, c.num_heads, 128).contiguous(), layer.cos, layer.sin).cpu()
+    d = {}
+    tab = cpu_tabs(wl)[0]
+    ref_slots, ref_out = oracle.prefill.prefill_chunk(
+        q.cpu(), wl.k_pool.cpu(), wl.v_pool.cpu(), tab, L, c.num_heads, 128, c.n_init, c.n_local,
+        c.top_k, c.rope_theta, c.rope_scale, _sm(c), detail=d, qf_override=qf)
+    pos = sel_pos[0, :S].cpu()
+    assert_index_sets_match(pos[c.n_init:c.n_init + c.top_k], d["top_pos"], d["votes"], c.n_init, case)
+    assert pos[-c.n_local:].tolist() == list(range(L - c.n_local, L))
+    assert torch.equal(sel[0, :S].cpu(), tab[pos.long()])
+    if not torch.equal(sel[0, :S].cpu(), ref_slots):   # a tie went the other way
+        ref_out = oracle.prefill.sparse_prefill_attention(
+            q.cpu().view(m, c.num_heads, 128), wl.k_pool.cpu(), wl.v_pool.cpu(), sel[0, :S].cpu(),
+            _sm(c), c.rope_theta, c.rope_scale).reshape(m, -1)
+    if S < m:
+        assert torch.count_nonzero(out[:m - S]).item() == 0
+    assert (out.cpu().float() - ref_out.float()).abs().max().item() <= 2e-2

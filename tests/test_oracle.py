@@ -379,6 +379,20 @@ def test_prefill_rows_are_decode_steps_over_key_prefixes():
     assert (full[0].float() - got[0].float()).abs().max().item() > 1e-3
 
 
+def test_prefill_with_fewer_keys_than_rows():
+    """S < m (a chunk longer than the selected list, as with the reference's own defaults):
+    the first m - S rows sit at negative positions and see no key, so their output is zero;
+    every later row is still the decode attention over its key prefix."""
+    q, kp, vp, slots = _prefill_case(seed=2, m=40, S=25)
+    m, S = q.shape[0], slots.shape[0]
+    got = oracle.prefill.sparse_prefill_attention(q, kp, vp, slots, 0.09, 5e5)
+    assert torch.count_nonzero(got[:m - S]) == 0
+    assert not torch.isnan(got.float()).any()
+    for i in (m - S, m - S + 3, m - 1):
+        ref = oracle.attend.sparse_decode_attention(q[i], kp, vp, slots[:S - m + i + 1], 0.09, 5e5)
+        assert (got[i].float() - ref.float()).abs().max().item() <= 1e-2
+
+
 def test_prefill_one_row_chunk_is_the_decode_layer():
     g = torch.Generator().manual_seed(5)
     H, Hkv, L = 4, 2, 300

@@ -27,7 +27,7 @@ int check_launch(const char* what) {
 
 bool group_supported(int num_kv_heads, int group) {
   bool kv_ok = num_kv_heads == 1 || num_kv_heads == 2 || num_kv_heads == 4 || num_kv_heads == 8;
-  bool g_ok = group == 1 || group == 2 || group == 4 || group == 7 || group == 8;
+  bool g_ok = group >= 1 && group <= 8;
   return kv_ok && g_ok;
 }
 
@@ -40,7 +40,7 @@ int validate_config(const ts_config* cfg) {
   TS_REQUIRE(cfg->num_heads % cfg->num_kv_heads == 0, TS_ESHAPE,
              "num_heads %d not a multiple of num_kv_heads %d", cfg->num_heads, cfg->num_kv_heads);
   TS_REQUIRE(group_supported(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads), TS_ESHAPE,
-             "unsupported head shape: num_kv_heads=%d (1,2,4,8) group=%d (1,2,4,7,8)",
+             "unsupported head shape: num_kv_heads=%d (1,2,4,8) group=%d (1 to 8)",
              cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
   TS_REQUIRE(page_shift_of(cfg->page_size) >= 0, TS_EINVAL, "page_size %d is not a power of two",
              cfg->page_size);
@@ -410,10 +410,6 @@ int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, in
   TS_REQUIRE(bt != nullptr && bt->batch == 1, TS_EINVAL,
              "ts_prefill_chunk serves one request at a time (batch must be 1)");
   TS_REQUIRE(rows >= 1, TS_EINVAL, "ts_prefill_chunk: rows %d < 1", rows);
-  TS_REQUIRE(cfg != nullptr && cfg->n_local >= rows, TS_EINVAL,
-             "ts_prefill_chunk: the chunk (%d rows) must lie inside the local window (n_local %d), "
-             "otherwise its own tokens are not all attended to",
-             rows, cfg ? cfg->n_local : 0);
   return run_layer(cfg, bt, q, rows, cos_table, sin_table, table_rows, k_pool, v_pool, pool_rows,
                    nullptr, out, sel, sel_pos, sel_stride, sel_len, workspace, workspace_bytes,
                    stream);

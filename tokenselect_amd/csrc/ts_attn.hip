@@ -80,8 +80,8 @@ template <int G, bool ROPE, bool CAP>
 __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   const int split = blockIdx.x, b = blockIdx.z;
   const int kvh = blockIdx.y / a.parts, part = blockIdx.y % a.parts;
-  // Head g of this workgroup: the last part of a group of seven has one head too many,
-  // which is computed (on the last real head's query) and not stored.
+  // Head g of this workgroup: the last part of a group of five or seven has one head too
+  // many, which is computed (on the last real head's query) and not stored.
   auto head_of_slot = [&](int g) { return kvh * a.group + min(part * G + g, a.group - 1); };
   auto slot_active = [&](int g) { return part * G + g < a.group; };
   // The ranges are cut from the longest list the launch was sized for, not from this
@@ -404,8 +404,9 @@ __global__ __launch_bounds__(256) void attn_zero_kernel(uint32_t* tickets, int c
 }
 
 // Workgroups per KV head and heads per workgroup for a group of `group` query heads.
-static int attn_parts(int group) { return group > 4 ? (group + 3) / 4 : 1; }
-static int attn_heads_per_part(int group) { return group > 4 ? 4 : group; }
+// (five or six heads: two workgroups of three; seven or eight: two of four)
+static int attn_parts(int group) { return (group + 3) / 4; }
+static int attn_heads_per_part(int group) { return (group + attn_parts(group) - 1) / attn_parts(group); }
 int attn_tickets_per_request(const ts_config* cfg) {
   return cfg->num_kv_heads * attn_parts(cfg->num_heads / cfg->num_kv_heads);
 }
@@ -490,6 +491,7 @@ int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const v
   switch (group) {
     TS_ATTN_CASE(1)
     TS_ATTN_CASE(2)
+    TS_ATTN_CASE(3)
     TS_ATTN_CASE(4)
     default: return fail(TS_ESHAPE, "unsupported head group %d", a.group);
   }

@@ -405,9 +405,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int shift = S - m;  // query row i sits at position shift + i and sees keys <= that
   const bool rope = a.rope_mode == TS_ROPE_LLAMA;
   const bool wave_active = head_active[0];
-  if (S < m || S <= 0) {
-    // Fewer keys than rows (not a prefill chunk, or a selection that reported a
-    // fault): the rows attend to nothing and the output is defined as zero.
+  if (S <= 0) {
+    // No keys (a selection that reported a fault): the rows attend to nothing and the
+    // output is defined as zero.  (With fewer keys than rows, 0 < S < m, the rows whose
+    // position S - m + i is negative see no key either: every tile is masked for them,
+    // their sums stay zero and so does their output; the others attend as usual.)
 #pragma unroll
     for (int rb = 0; rb < HEADS; ++rb)
       if (head_active[rb])
@@ -789,8 +791,6 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
   TS_REQUIRE(q && k_pool && v_pool && sel && sel_len && out, TS_EINVAL,
              "ts_sparse_prefill_attn: NULL tensor argument");
   TS_REQUIRE(rows >= 1 && rows <= 65535 * 16, TS_EINVAL, "rows %d out of range", rows);
-  TS_REQUIRE(max_sel_len >= rows, TS_EINVAL,
-             "max_sel_len %d < rows %d: a chunk attends at least to itself", max_sel_len, rows);
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   const size_t need = ts_prefill_attn_workspace_bytes(cfg, max_sel_len);
@@ -845,7 +845,10 @@ int ts_sparse_prefill_attn(const ts_config* cfg, const void* q, int32_t rows, co
   switch (group) {
     TS_PF_CASE(1)
     TS_PF_CASE(2)
+    TS_PF_CASE(3)
     TS_PF_CASE(4)
+    TS_PF_CASE(5)
+    TS_PF_CASE(6)
     TS_PF_CASE(7)
     TS_PF_CASE(8)
     default: return fail(TS_ESHAPE, "unsupported head group %d", group);

@@ -1189,7 +1189,8 @@ static int launch_score(int hkv, int group, const ScoreArgs& a, dim3 grid, hipSt
     return check_launch("score_kernel");                                                         \
   }
 #define TS_SCORE_ROW(HKV_) \
-  TS_SCORE_CASE(HKV_, 1) TS_SCORE_CASE(HKV_, 2) TS_SCORE_CASE(HKV_, 4) TS_SCORE_CASE(HKV_, 7) TS_SCORE_CASE(HKV_, 8)
+  TS_SCORE_CASE(HKV_, 1) TS_SCORE_CASE(HKV_, 2) TS_SCORE_CASE(HKV_, 3) TS_SCORE_CASE(HKV_, 4) \
+      TS_SCORE_CASE(HKV_, 5) TS_SCORE_CASE(HKV_, 6) TS_SCORE_CASE(HKV_, 7) TS_SCORE_CASE(HKV_, 8)
   TS_SCORE_ROW(1)
   TS_SCORE_ROW(2)
   TS_SCORE_ROW(4)
@@ -1206,7 +1207,8 @@ static const void* fused_kernel_of(int hkv, int group, bool packed = false) {
     return packed ? (const void*)&score_kernel<HKV_, G_, false, kScorePacked>          \
                   : (const void*)&score_kernel<HKV_, G_, false, kScoreFused>;
 #define TS_SCORE_ROW(HKV_) \
-  TS_SCORE_CASE(HKV_, 1) TS_SCORE_CASE(HKV_, 2) TS_SCORE_CASE(HKV_, 4) TS_SCORE_CASE(HKV_, 7) TS_SCORE_CASE(HKV_, 8)
+  TS_SCORE_CASE(HKV_, 1) TS_SCORE_CASE(HKV_, 2) TS_SCORE_CASE(HKV_, 3) TS_SCORE_CASE(HKV_, 4) \
+      TS_SCORE_CASE(HKV_, 5) TS_SCORE_CASE(HKV_, 6) TS_SCORE_CASE(HKV_, 7) TS_SCORE_CASE(HKV_, 8)
   TS_SCORE_ROW(1)
   TS_SCORE_ROW(2)
   TS_SCORE_ROW(4)
