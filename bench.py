@@ -43,7 +43,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # figures are recorded under profiles/.  Workloads not measured that way give null.
 # Each figure carries the commit of the kernels it was measured on: a later change to the
 # kernel makes it stale until the two counter runs are repeated.
-MEASURED_TRAFFIC = {"C2": (269711053, "6c0d379")}  # profiles/decode_layer_c2_hbm_traffic.txt
+MEASURED_TRAFFIC = {  # workload -> (bytes per launch of its dominant kernel, commit)
+    "C2": (269711053, "6c0d379"),  # profiles/decode_layer_c2_hbm_traffic.txt
+}
 
 
 def event_time_us(fn, launches: int, warmup: int, before=None, burst: int = 1):
@@ -306,8 +308,21 @@ def bench_trace(args, ops, workloads, dev):
         "hit_rate": round(hits / max(lookups, 1), 4), "hits": hits, "lookups": lookups,
         "tokens_per_s": round(B / (us_per_step * 1e-6 * args.layers), 1),
         "tokens_per_s_note": f"selection+attention only, {args.layers} layers per token",
-        "roofline": None, "cpu_baseline": None,
+        "cpu_baseline": None,
     }
+    # What a step needs from HBM: the keys of the requests that missed (a hit scores nothing)
+    # and the gathered K/V rows of every request, over the whole step's time (the store, the
+    # cache comparison, the selection and the attention): a figure for the trace as a whole,
+    # not for one kernel.
+    row = c.num_kv_heads * c.head_dim * 2
+    miss_bytes = (lookups - hits) * ((L0 + steps // 2 - c.n_init - c.n_local) * row)
+    gather_bytes = lookups * c.max_sel * 2 * row
+    step_bytes = (miss_bytes + gather_bytes) / steps
+    gbs = step_bytes / us_per_step / 1e3
+    result["roofline"] = {"bound": "hbm", "kernel": "whole step (ts_kv_store + ts_decode_layer with the cache)",
+                          "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                          "bytes_per_step": int(step_bytes), "us_per_step": round(us_per_step, 2)}
     return result
 
 
@@ -544,7 +559,7 @@ def extra_workloads(args, ops, workloads, dev):
             "workload": r["config"]["workload"], "us_per_layer": r["value"],
             "dominant_kernel": roof["kernel"].split(" ")[0], "us_per_launch": roof["us_per_launch"],
             "bytes_per_launch": roof["bytes_per_launch"], "frac": roof["frac"],
-            "score_only_frac": r["score_only"]["frac"],
+            "traffic": roof["traffic"], "score_only_frac": r["score_only"]["frac"],
             "attn_us": r["gather_attention"]["us_per_launch"], "parity": r.get("parity"),
             "wall_s": round(time.perf_counter() - t0, 1)})
         torch.cuda.empty_cache()
@@ -552,12 +567,39 @@ def extra_workloads(args, ops, workloads, dev):
     small.steps, small.warmup = 64, 64
     r = bench_trace(small, ops, workloads, dev)
     lines.append({"workload": r["config"]["workload"], "us_per_step": r["value"],
-                  "hit_rate": r["hit_rate"], "wall_s": round(time.perf_counter() - t0, 1)})
+                  "hit_rate": r["hit_rate"], "bytes_per_step": r["roofline"]["bytes_per_step"],
+                  "frac": r["roofline"]["frac"], "wall_s": round(time.perf_counter() - t0, 1)})
     small.page_size = 16
     t0 = time.perf_counter()
     r = bench_trace(small, ops, workloads, dev)
     lines.append({"workload": r["config"]["workload"], "us_per_step": r["value"],
-                  "hit_rate": r["hit_rate"], "wall_s": round(time.perf_counter() - t0, 1)})
+                  "hit_rate": r["hit_rate"], "bytes_per_step": r["roofline"]["bytes_per_step"],
+                  "frac": r["roofline"]["frac"], "wall_s": round(time.perf_counter() - t0, 1)})
+    torch.cuda.empty_cache()
+    # One 512-row chunk of the extend forward on a 128K context.
+    t0 = time.perf_counter()
+    small.steps, small.warmup, small.page_size = 50, 10, 1
+    r = bench_prefill(small, ops, workloads, dev)
+    lines.append({"workload": r["config"]["workload"], "us_per_chunk": r["value"],
+                  "dominant_kernel": "ts::prefill_attn_kernel<G>", "bound": "mfma",
+                  "us_per_launch": r["roofline"]["us_per_launch"],
+                  "flops_per_launch": r["roofline"]["flops_per_launch"],
+                  "tflops": r["roofline"]["achieved"], "frac": r["roofline"]["frac"],
+                  "parity": r.get("parity"), "wall_s": round(time.perf_counter() - t0, 1)})
+    torch.cuda.empty_cache()
+    # The whole 32-layer decoder (BASELINE.json configs[4]) over 32 greedy steps.
+    t0 = time.perf_counter()
+    small.steps, small.warmup = 32, 2
+    r = bench_model(small, ops, dev)
+    lines.append({"workload": r["config"]["workload"], "tokens_per_s": r["value"],
+                  "greedy_steps": r["steps"], "ms_per_decode_step": r["ms_per_step"],
+                  "us_per_layer": r["us_per_layer"], "hbm_frac_whole_step": r["hbm_frac_whole_step"],
+                  "dominant_kernel": r["roofline"]["kernel"].split(" ")[0],
+                  "us_per_launch": r["roofline"]["us_per_launch"], "frac": r["roofline"]["frac"],
+                  "traffic": r["roofline"]["traffic"],
+                  "cpu_tokens_per_s": (r.get("cpu_baseline") or {}).get("value"),
+                  "parity": r.get("parity"), "wall_s": round(time.perf_counter() - t0, 1)})
+    torch.cuda.empty_cache()
     return lines
 
 
