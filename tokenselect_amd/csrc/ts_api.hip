@@ -255,11 +255,14 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
     // Chunk fingerprint: row i rotated to n_local + i, mean over the rows (tr.py:380-392).
     TS_TRY(launch_fingerprint(cfg, q, chunk_rows, q_cos, q_sin, table_rows, qf, zero,
                               (hipStream_t)stream));
+  } else if (cache) {  // rotation and cache decision in one launch
+    TS_TRY(launch_rope_selcache(cfg, bt, q, qf, q_cos, q_sin, cache, hit, bt->rerun ? sel_len : nullptr,
+                                zero, (hipStream_t)stream));
   } else {
     TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
                        zero, (hipStream_t)stream));
   }
-  if (cache)
+  if (cache && chunk_rows > 0)
     TS_TRY(launch_selcache(cfg, bt, qf, cache, hit, bt->rerun ? sel_len : nullptr, (hipStream_t)stream));
   if (one_launch) {
     TS_TRY(launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,

@@ -91,6 +91,13 @@ int launch_rope(const void* x, void* out, const float* cos_table, const float* s
 int launch_selcache(const ts_config* cfg, const ts_batch* bt, const void* qf, const ts_selcache* cache,
                     int32_t* hit, const int32_t* gave_up_len, hipStream_t stream);
 
+// The fingerprint rotation of a decode step (one query row per request, q_cos / q_sin the
+// [D] table rows of its position) and the cache decision in one launch, which also clears
+// the regions of `zero`.
+int launch_rope_selcache(const ts_config* cfg, const ts_batch* bt, const void* q, void* qf,
+                         const float* q_cos, const float* q_sin, const ts_selcache* cache, int32_t* hit,
+                         const int32_t* gave_up_len, const ZeroSet& zero, hipStream_t stream);
+
 // Sparse decode attention (ts_attn.hip).  The kernel counts its workgroups in per
 // (request, KV head) tickets inside the workspace, which must be zero at launch:
 // tickets_clear = false makes the launcher clear them first, true says an earlier

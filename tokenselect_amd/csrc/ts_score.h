@@ -56,6 +56,8 @@ struct ScoreArgs {
   int clear_per_req;
   uint64_t spin_ticks;    // bound of a grid-wide wait, in 100 MHz ticks
   int batch_offset;       // request index of the launch's first request
+  int batch;              // requests of the launch (the single-launch selection deals its
+                          // one-dimensional grid over those of them that select)
   // Votes-only form of the fused kernel (a kernel instantiation of its own): the launch
   // ends with the votes in memory and their first-level histogram added to the top-k
   // workspace.  A one-dimensional grid holds the workgroups of `nphases` phases one after

@@ -119,7 +119,7 @@ template <bool PACKED>
 __device__ __forceinline__ void merge_request_stats(const ScoreArgs& a, const LaunchPart& lp,
                                                     const GridTeam& team, int lane, int wave) {
   const int H = a.num_heads;
-  const int items = (PACKED ? lp.packed : (int)gridDim.y) * H;
+  const int items = (PACKED ? lp.packed : a.batch) * H;
   const int first = (int)team.index * 4 + wave;
   const int step = (int)team.size * 4;
   for (int item = first; item < items; item += step) {
@@ -187,7 +187,7 @@ constexpr uint32_t kSelectRounds = 4;  // rendezvous of the fused kernel at most
 template <bool PACKED>
 __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, const LaunchPart& lp,
                                                    uint32_t* lds, int req, int chunk) {
-  GridTeam team;
+  GridTeam team{0u, 0u};
   if (PACKED) {
     // A phase holds a handful of requests and its members are the workgroups
     // that hold candidates: every thread adds them up for itself.
@@ -205,34 +205,124 @@ __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, const Lau
     team.index = before + (uint32_t)chunk;
     return team;
   }
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int B = gridDim.y, mine = req;
-  uint32_t before = 0, total = 0;  // selecting requests below this one / in all
-  for (int base = 0; base < B; base += 256) {
-    const int b = lp.batch_offset + base + tid;  // requests of this launch
-    bool selects = false;
-    if (base + tid < B && !(a.skip && a.skip[b]))
-      selects = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k,
-                                 a.max_seq_len).n > 0;
-    const uint64_t mask = __ballot(selects);
-    if (lane == 0) {
-      lds[wave] = (uint32_t)__popcll(mask);
-      // requests of this chunk below `mine` that lie in this wavefront's 64
-      const int lo = base + 64 * wave;
-      const int upto = mine - lo;  // bits [0, upto) count
-      lds[4 + wave] = upto <= 0 ? 0u
-                                : (uint32_t)__popcll(upto >= 64 ? mask : mask & ((1ull << upto) - 1ull));
+  (void)lds;
+  return team;  // (the single launch deals its workgroups itself: deal_workgroups)
+}
+
+// The single-launch selection deals its workgroups on the device, from the lengths and the
+// hit flags as they are at launch: only the requests that select (neither dense nor served
+// by the selection cache) get workgroups, all of them the same number of tokens, the
+// smallest multiple of 64 with which the requests' chunks fit the grid; consecutive
+// workgroups serve consecutive chunks, request after request.  A step in which one request
+// of four misses the cache thus streams that request's keys through the whole device
+// instead of through the quarter a fixed [chunks, requests] grid would give it, and a
+// ragged batch is spread by what the requests hold, not by the longest.  Workgroups past
+// the last chunk have nothing to do.  The workgroups with tokens are the team of the
+// rendezvous, in grid order.
+struct Deal {
+  int tokens_per_block;  // of every selecting request of this launch
+  int req;               // this workgroup's request (within the launch), -1: none
+  int chunk, chunks;     // its chunk of that request, and the request's chunks
+  uint32_t team_size, team_index;
+};
+constexpr int kDealPerLane = 8;  // requests per lane of the dealing wavefront: batches of up to 512
+
+__device__ __forceinline__ int wave_sum(int x) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off);
+  return x;
+}
+
+__device__ __forceinline__ Deal deal_workgroups(const ScoreArgs& a, int* lds) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int B = a.batch, T = (int)gridDim.x, w = (int)blockIdx.x;
+  if (B == 1) {  // one request: every thread works it out for itself, no exchange
+    Deal d{a.tokens_per_block, -1, 0, 0, a.absent, (uint32_t)w};
+    int n = 0;
+    if (!(a.skip && a.skip[a.batch_offset]))
+      n = request_geometry(a.seq_lens, a.k_per_req, a.batch_offset, a.n_init, a.n_local, a.top_k,
+                           a.max_seq_len).n;
+    if (n <= 0) return d;
+    int tpb = max((n + T * 64 - 1) / (T * 64) * 64, 64);
+    while ((n + tpb - 1) / tpb > T && tpb < a.tokens_per_block) tpb += 64;
+    d.tokens_per_block = tpb;
+    d.chunks = (n + tpb - 1) / tpb;
+    d.team_size = (uint32_t)d.chunks + a.absent;
+    if (w < d.chunks) {
+      d.req = 0;
+      d.chunk = w;
     }
-    __syncthreads();
-    for (int w = 0; w < 4; ++w) {
-      total += lds[w];
-      before += lds[4 + w];
-    }
-    __syncthreads();
+    return d;
   }
-  team.size = total * gridDim.x + a.absent;
-  team.index = before * gridDim.x + (uint32_t)chunk;
-  return team;
+  if (tid < 64) {
+    // Request lane + 64 j: its candidates if it selects, else 0.
+    int n[kDealPerLane];
+    int all = 0;  // (what one launch holds fits the LDS of the device: far below 2^31)
+#pragma unroll
+    for (int j = 0; j < kDealPerLane; ++j) {
+      const int b = lane + 64 * j;
+      n[j] = 0;
+      if (64 * j < B && b < B && !(a.skip && a.skip[a.batch_offset + b]))
+        n[j] = request_geometry(a.seq_lens, a.k_per_req, a.batch_offset + b, a.n_init, a.n_local, a.top_k,
+                                a.max_seq_len).n;
+      all += n[j];
+    }
+    const long long total_n = wave_sum(all);
+    // Fewest tokens per workgroup that could do, then upwards until the chunks fit (a step
+    // or two: the rounding of every request's last chunk).  The launch's own figure always
+    // fits: the host sized the grid for every request at the longest length.
+    int tpb = (int)((total_n + (long long)T * 64 - 1) / ((long long)T * 64)) * 64;
+    tpb = max(tpb, 64);
+    int chunks[kDealPerLane];
+    for (;; tpb += 64) {
+      int mine = 0;
+#pragma unroll
+      for (int j = 0; j < kDealPerLane; ++j) {
+        chunks[j] = 64 * j < B ? (n[j] + tpb - 1) / tpb : 0;
+        mine += chunks[j];
+      }
+      if (wave_sum(mine) <= T || tpb >= a.tokens_per_block) break;
+    }
+    // First workgroup of every request, in request order (lane + 64 j: j by j).
+    int base = 0, req = -1, chunk = 0, req_chunks = 0;
+#pragma unroll
+    for (int j = 0; j < kDealPerLane; ++j) {
+      if (64 * j >= B) break;
+      int incl = chunks[j];
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+      }
+      const int first = base + incl - chunks[j];
+      const bool here = w >= first && w < first + chunks[j];
+      const uint64_t who = __ballot(here);
+      if (who) {
+        const int src = __ffsll((unsigned long long)who) - 1;
+        req = 64 * j + src;
+        chunk = w - __shfl(first, src);
+        req_chunks = __shfl(chunks[j], src);
+      }
+      base += __shfl(incl, 63);
+    }
+    if (lane == 0) {
+      lds[0] = tpb;
+      lds[1] = req;
+      lds[2] = chunk;
+      lds[3] = req_chunks;
+      lds[4] = base;  // workgroups with tokens: the team
+    }
+  }
+  __syncthreads();
+  Deal d;
+  d.tokens_per_block = lds[0];
+  d.req = lds[1];
+  d.chunk = lds[2];
+  d.chunks = lds[3];
+  d.team_size = (uint32_t)lds[4] + a.absent;
+  d.team_index = (uint32_t)w;
+  __syncthreads();
+  return d;
 }
 
 // The parts of the output that need no votes, written while the keys stream: a
@@ -240,19 +330,20 @@ __device__ __forceinline__ GridTeam selecting_team(const ScoreArgs& a, const Lau
 // (both spread over the request's workgroups); workgroup 0 of a request writes the
 // length, the sink and the local window, and clears the words the next kernel of
 // the stream wants cleared.
-__device__ __forceinline__ void fixed_segments(const ScoreArgs& a, int b) {
+// (x of nx: this workgroup among those that write the request's fixed parts.)
+__device__ __forceinline__ void fixed_segments(const ScoreArgs& a, int b, int x, int nx) {
   const ReqGeom geo =
       request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
   const int32_t* tab = a.table + (int64_t)b * a.table_stride;
   int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
   int32_t* sel_pos = a.sel_pos + (int64_t)b * a.sel_stride;
   const int L = geo.seq_len;
-  const int first = blockIdx.x * 256 + threadIdx.x, step = gridDim.x * 256;
+  const int first = x * 256 + threadIdx.x, step = nx * 256;
   auto emit = [&](int out_idx, int pos) {
     sel_pos[out_idx] = pos;
     sel[out_idx] = (int32_t)lookup_slot(tab, pos, a.page_size, a.page_shift, a.pool_rows);
   };
-  if (blockIdx.x == 0 && a.clear)
+  if (x == 0 && a.clear)
     for (int i = threadIdx.x; i < a.clear_per_req; i += 256)
       a.clear[(size_t)b * a.clear_per_req + i] = 0u;
   if (geo.dense) {  // tr.py:377-378, 741-744: attend over every token
@@ -266,9 +357,11 @@ __device__ __forceinline__ void fixed_segments(const ScoreArgs& a, int b) {
     const int32_t* cached = a.topk_cache + (int64_t)b * a.top_k;
     for (int i = first; i < k; i += step) emit(a.n_init + i, cached[i]);
   }
-  if (blockIdx.x != 0) return;
+  if (x != 0) return;
   if (threadIdx.x == 0) {
-    a.sel_len[b] = a.n_init + k + a.n_local;
+    // (The length of a request that selects is written when its selection is through, by
+    // the workgroup that also reports a wait that gave up: one writer, one order.)
+    if (is_hit) a.sel_len[b] = a.n_init + k + a.n_local;
     if (!is_hit && a.cache_len) a.cache_len[b] = k;
   }
   for (int i = threadIdx.x; i < a.n_init; i += 256) emit(i, i);
@@ -404,6 +497,8 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   // This workgroup's request within the launch, and its chunk of that request.
   LaunchPart lp{a.tokens_per_block, a.batch_offset, 0, nullptr, (int)blockIdx.x, a.sync};
   int req = blockIdx.y, chunk = blockIdx.x;
+  int req_chunks = (int)gridDim.x;  // chunks of this workgroup's request (the single launch: dealt)
+  GridTeam team{0u, 0u};
   if (PACKED) {
     // This workgroup's phase, and its request and chunk within the phase.
     int phase = 0;
@@ -414,6 +509,22 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     req = 0;
     while (req + 1 < lp.packed && lp.x >= lp.pack_first[req + 1]) ++req;
     chunk = lp.x - lp.pack_first[req];
+  }
+  if constexpr (FUSED && !PACKED) {
+    __shared__ int deal_lds[8];
+    TS_MARK(0);
+    // The parts of the output that need no votes: request w % B by workgroup w / B of its share.
+    {
+      const int B = a.batch, w = (int)blockIdx.x, T = (int)gridDim.x;
+      fixed_segments(a, a.batch_offset + w % B, w / B, (T - w % B + B - 1) / B);
+    }
+    const Deal deal = deal_workgroups(a, deal_lds);
+    if (deal.req < 0) return;  // no chunk left for this workgroup
+    lp.tokens_per_block = deal.tokens_per_block;
+    req = deal.req;
+    chunk = deal.chunk;
+    req_chunks = deal.chunks;
+    team = GridTeam{deal.team_size, deal.team_index};
   }
   const int b = req + lp.batch_offset;
   int n, first_pos;
@@ -427,27 +538,16 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     first_pos = a.n_init;
   }
   const int block_lo = chunk * lp.tokens_per_block;
-  GridTeam team{0u, 0u};
-  if constexpr (FUSED) {
+  if constexpr (PACKED) {
     __shared__ uint32_t team_lds[8];
-    TS_MARK(0);
-    if (!PACKED) fixed_segments(a, b);
     if (n <= 0) return;  // dense or served by the cache: nothing to select, not on the team
-    if (PACKED && block_lo >= n) return;  // no candidates here, and the team is made without it
-    if (PACKED && chunk == 0 && threadIdx.x == 0 &&
+    if (block_lo >= n) return;  // no candidates here, and the team is made without it
+    if (chunk == 0 && threadIdx.x == 0 &&
         (n + lp.tokens_per_block - 1) / lp.tokens_per_block > lp.pack_first[req + 1] - lp.pack_first[req])
       __hip_atomic_store(&lp.sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // length above its bound
     team = selecting_team<PACKED>(a, lp, team_lds, req, chunk);
   }
-  if (block_lo >= n) {
-    if constexpr (FUSED) {  // no tokens here: only help with the statistics
-      merge_request_stats<PACKED>(a, lp, team, threadIdx.x & 63, threadIdx.x >> 6);
-      const uint32_t rounds = kSelectRounds + (a.pool_kernel > 0 ? 1u : 0u);  // (not PACKED here)
-      for (uint32_t round = 1; round <= rounds; ++round)
-        grid_arrive(lp.sync, round, false, a.spin_ticks, team.size, team.index);
-    }
-    return;
-  }
+  if (block_lo >= n) return;  // (a dealt workgroup always has tokens)
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -814,7 +914,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     // of the copies and note the highest occupied bin; afterwards each searches
     // downwards from that bin, 256 bins at a time (one is enough unless the votes
     // span more than 64 binades).
-    uint32_t* hist0 = ctr + kSelHist0 + (blockIdx.x % kSelHistCopies) * kTopkBins;
+    uint32_t* hist0 = ctr + kSelHist0 + (chunk % kSelHistCopies) * kTopkBins;
     {
       // Two adjacent bins per 64-bit add (their counts cannot carry into each other):
       // half as many read-modify-writes on the few hot lines.
@@ -828,7 +928,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
                                          __HIP_MEMORY_SCOPE_AGENT);
       }
       if (tid == 0)
-        done += fetch_max_coherent(&ctr[kSelMaxBin + (blockIdx.x % kSelHistCopies) * 32], scratch[8]);
+        done += fetch_max_coherent(&ctr[kSelMaxBin + (chunk % kSelHistCopies) * 32], scratch[8]);
       await(done);
     }
     TS_MARK(7);
@@ -894,7 +994,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       uint32_t done = 0;
       for (int base = 0; base < count; base += 256) {
         const uint32_t key = base + tid < count ? key_of(base + tid) : 0u;
-        done += wave_histogram_add(ctr + kSelHist1 + (blockIdx.x % kSelHist1Copies) * kTopkBins,
+        done += wave_histogram_add(ctr + kSelHist1 + (chunk % kSelHist1Copies) * kTopkBins,
                                    base + tid < count && key_bin0(key) == t0, key_bin1(key), lane);
       }
       await(done);
@@ -924,7 +1024,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       __syncthreads();
     }
 
-    uint2* counts = a.block_counts + (size_t)b * gridDim.x;
+    uint2* counts = a.block_counts + (size_t)b * kSelMaxChunks;
     const bool listed = in_bin <= (uint32_t)kSelListCap;
     uint32_t kth, need_eq = 0, pos_thr = 0;
     if (tid < 8) scratch[8 + tid] = 0u;
@@ -935,7 +1035,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       // its entries with one add), and every workgroup publishes how many of its
       // tokens lie above the bin.
       uint2* list = a.short_list + (size_t)b * kSelListParts * kSelListCap;
-      const int part = blockIdx.x % kSelListParts;
+      const int part = chunk % kSelListParts;
       const uint64_t below_mask = (1ull << lane) - 1ull;
       uint32_t above = 0;
       for (int base = 0; base < count; base += 256) {
@@ -959,7 +1059,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       for (int off = 32; off >= 1; off >>= 1) above += __shfl_xor(above, off);
       if (lane == 0) atomicAdd(&scratch[8], above);
       __syncthreads();
-      if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], 0u);
+      if (tid == 0) store_coherent(&counts[chunk], scratch[8], 0u);
       TS_MARK(10);
       grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
       TS_MARK(11);
@@ -975,7 +1075,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       uint2 e = load_coherent(&list[(tid % kSelListParts) * kSelListCap + tid / kSelListParts]);
       {
         uint32_t sure = 0;
-        for (int j = tid; j < (int)blockIdx.x; j += 256) sure += load_coherent(&counts[j]).x;
+        for (int j = tid; j < chunk; j += 256) sure += load_coherent(&counts[j]).x;
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) sure += __shfl_xor(sure, off);
         if (lane == 0) atomicAdd(&scratch[10], sure);
@@ -1087,12 +1187,12 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         atomicAdd(&scratch[9], tie);
       }
       __syncthreads();
-      if (tid == 0) store_coherent(&counts[blockIdx.x], scratch[8], scratch[9]);
+      if (tid == 0) store_coherent(&counts[chunk], scratch[8], scratch[9]);
       grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
     }
     // The requests of a batch may need different numbers of rounds, and the rendezvous
     // spans them all: whoever is through counts itself in for the rounds it skipped.
-    if (team.size != gridDim.x) {
+    if (team.size != (uint32_t)req_chunks) {  // other requests select in this launch as well
       const uint32_t rounds = kSelectRounds + (a.pool_kernel > 0 ? 1u : 0u);
       while (round < rounds)
         grid_arrive(lp.sync, ++round, false, a.spin_ticks, team.size, team.index);
@@ -1100,7 +1200,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     if (!listed) {
       // Counts of the workgroups before this one.
       uint32_t sure = 0, tie = 0;
-      for (int j = tid; j < (int)blockIdx.x; j += 256) {
+      for (int j = tid; j < chunk; j += 256) {
         const uint2 v = load_coherent(&counts[j]);
         sure += v.x;
         tie += v.y;
@@ -1171,9 +1271,10 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     // A grid-wide wait of this launch gave up (the workgroups were not all resident
     // within the bound): what was selected is not valid.  The first workgroup of every
     // selecting request says so in place of the length, and in the caller's word.
-    if (blockIdx.x == 0 && tid == 0 && load_coherent(&lp.sync[0]) != 0u) {
-      a.sel_len[b] = -1;
-      if (a.fault_out)
+    if (chunk == 0 && tid == 0) {
+      const bool gave_up = load_coherent(&lp.sync[0]) != 0u;
+      a.sel_len[b] = gave_up ? -1 : a.n_init + (int)k + a.n_local;
+      if (gave_up && a.fault_out)
         __hip_atomic_store(a.fault_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
@@ -1292,9 +1393,9 @@ static int pooling_tokens_cap(const ts_config* cfg) {
 // them up on some CUs while others idle, above that half as many workgroups stream as
 // fast and hand over less.  Batches that need more LDS per CU than that run as well or
 // better on two workgroups per CU (2 x 128K the same, 4 x 64K and 8 x 32K 1-2 us better),
-// and so do batches in which requests may be skipped (selection cache): what a skipped
-// request leaves idle are whole CUs then, and the others' keys stream through half as many
-// (C4 93 -> 104 us per step).
+// unless requests may be skipped (selection cache): the workgroups are dealt over the
+// requests that select, a step rarely has all of them, and the large workgroups then
+// hold fewer tokens than they could (C4: 89.0 -> 87.4 us per step).
 int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, bool ignore_switch,
                            bool* large_out, bool may_skip, int* most_blocks_out) {
   if (large_out) *large_out = false;
@@ -1315,11 +1416,14 @@ int fused_tokens_per_block(const ts_config* cfg, int batch, int max_seq_len, boo
     return tpb;
   };
   const int tpb_small = plan(false), tpb_large = plan(true);
+  // (the workgroups of a launch are dealt over the requests that select: one request may
+  // get them all)
   if (most_blocks_out)
-    *most_blocks_out = std::max(tpb_small > 0 ? (int)ceil_div(max_n, tpb_small) : 0,
-                                tpb_large > 0 ? (int)ceil_div(max_n, tpb_large) : 0);
+    *most_blocks_out = std::min<int>(
+        kSelMaxChunks, batch * std::max(tpb_small > 0 ? (int)ceil_div(max_n, tpb_small) : 0,
+                                        tpb_large > 0 ? (int)ceil_div(max_n, tpb_large) : 0));
   const bool roomy = tpb_large > 0 && fused_lds_bytes(tpb_large, cfg->num_heads) <= kFusedStageBytes;
-  if ((roomy && !(may_skip && batch >= 2)) || tpb_small == 0) {
+  if (roomy || tpb_small == 0 || (may_skip && batch >= 2 && tpb_large > 0)) {
     if (large_out) *large_out = tpb_large > 0;
     return tpb_large;
   }
@@ -1518,7 +1622,9 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   a.pool_votes = (float*)(ws + w.pool_votes);
   a.pool_stride = w.pool_stride;
   const void* fn = fused_kernel_of(cfg->num_kv_heads, cfg->num_heads / cfg->num_kv_heads);
-  const dim3 grid((unsigned)w.blocks_per_req, (unsigned)bt->batch);
+  // One-dimensional: the kernel deals these workgroups over the requests that select.
+  a.batch = bt->batch;
+  const dim3 grid((unsigned)(w.blocks_per_req * bt->batch), 1u);
   void* params[] = {(void*)&a};
   // An ordinary launch: the grid was sized to be resident all at once, which holds
   // as long as the device runs nothing else beside this stream.  (The cooperative
