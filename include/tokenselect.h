@@ -102,6 +102,16 @@ typedef struct ts_batch {
                                the tokens beyond it are not scored, and the
                                launch reports it like a wait that gave up
                                (fault, sel_len = -1)                           */
+  int32_t* threshold_hint;  /* NULL, or [B] in device memory, owned by the caller and
+                               kept per (request, layer) across decode steps; zero
+                               before a request's first step.  ts_select leaves a
+                               coarse code of where the k-th vote lay there and uses
+                               the previous step's as a guess: while the votes of a
+                               layer drift slowly from step to step, as the queries
+                               do, the selection is then through after one meeting of
+                               its workgroups instead of two (C2: 4 us of 62).  Only
+                               ever a guess: a wrong or stale value costs the saving,
+                               never the result, which is exact either way          */
   /* Per-call options; all zero = the defaults. */
   int32_t separate_kernels; /* 1: this call selects with ts_score + ts_vote +
                                ts_topk_ragged's kernels, whose workgroups never wait

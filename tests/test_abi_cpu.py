@@ -46,9 +46,10 @@ def test_header_symbols_are_exported_and_bound(lib):
 
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.TsConfig) == 14 * 4
-    assert ctypes.sizeof(_lib.TsBatch) == 8 + 8 + 8 + 8 + 8 + 8 + 8 + 4 * 4
-    assert _lib.TsBatch.separate_kernels.offset == 56 and _lib.TsBatch.rerun.offset == 60
-    assert _lib.TsBatch.wait_us.offset == 64 and _lib.TsBatch.absent_workgroups.offset == 68
+    assert ctypes.sizeof(_lib.TsBatch) == 8 + 8 + 8 + 8 + 8 + 8 + 8 + 8 + 4 * 4
+    assert _lib.TsBatch.threshold_hint.offset == 56
+    assert _lib.TsBatch.separate_kernels.offset == 64 and _lib.TsBatch.rerun.offset == 68
+    assert _lib.TsBatch.wait_us.offset == 72 and _lib.TsBatch.absent_workgroups.offset == 76
     assert _lib.TsBatch.fault.offset == 40 and _lib.TsBatch.host_seq_lens.offset == 48
     assert _lib.TsBatch.seq_lens.offset == 8 and _lib.TsBatch.table_stride.offset == 24
     assert ctypes.sizeof(_lib.TsSelCache) == 4 * 8 + 8

@@ -1175,3 +1175,95 @@ def test_selection_form_agrees_with_what_the_launchers_serve(dev):
     assert ops.layer_selection_form(wl.cfg, wl.batch) == 2
     assert ops.layer_selection_form(wl.cfg, dataclasses.replace(wl.batch, separate_kernels=True)) == 0
     assert ops.layer_selection_form(wl.cfg, wl.batch) == 2
+
+
+@pytest.mark.parametrize("shape", [SHAPES[0], SHAPES[1], SHAPES[6]],
+                         ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+def test_fused_select_with_a_threshold_hint(dev, shape):
+    """ts_batch.threshold_hint: the selection notes the bin of the k-th vote and, given it
+    back, publishes what its last round needs before the first rendezvous, so that one
+    rendezvous is enough.  The result is that of a launch without a hint, bit for bit: with
+    the right hint (one round met for), with hints off by a few bins inside the band, with
+    hints outside it and with nonsense (two rounds again), and for another query whose
+    threshold has moved."""
+    import dataclasses
+    L, k = 40000, 512
+    say(f"fused select with a threshold hint H={shape['num_heads']} L={L}")
+    wl = small(dev, shape, seed=101, lens=[L], ks=[k], page=16, top_k=k, n_init=128, n_local=512)
+    c = wl.cfg
+    qf = fingerprint(wl, dev)
+    space = ops.select_workspace(c, wl.batch, dev)
+    want = ops.select(c, wl.batch, qf, wl.k_pool, workspace=space)[:3]
+    torch.cuda.synchronize()
+    assert ops.select_rounds(c, wl.batch, space)[:2][1] > 0, "without a hint: a second round"
+    hint = torch.zeros(1, dtype=torch.int32, device=dev)
+    hinted = dataclasses.replace(wl.batch, hint=hint)
+
+    def run(q=qf, expect=want):
+        got = ops.select(c, hinted, q, wl.k_pool, workspace=space)[:3]
+        torch.cuda.synchronize()
+        assert not ops.select_fault(c, hinted, space)
+        for name, x, y in zip(("sel", "sel_pos", "sel_len"), got, expect):
+            assert torch.equal(x, y), name
+        return ops.select_rounds(c, hinted, space)
+
+    assert run()[1] > 0                 # no hint yet: the usual two rounds, and the hint is left
+    code = int(hint[0])
+    assert 1 <= code <= 2048
+    assert run()[1] == 0                # the right hint: one round
+    for off in (-3, -1, 1, 4):          # the band [hint - 4, hint + 3] still holds the bin
+        hint.fill_(code + off)
+        assert run()[1] == 0, off
+        assert int(hint[0]) == code
+    for off in (-4, 5, 300, -code):     # it does not, or there is no hint at all: the list round is back
+        hint.fill_(code + off)
+        assert run()[1] > 0, off
+        assert int(hint[0]) == code
+    hint.fill_(5000)                    # nonsense
+    assert run()[1] > 0
+    # another query: its own selection, whatever the old hint says
+    g = torch.Generator(device=dev).manual_seed(102)
+    q2 = (qf.float() + 0.3 * torch.randn(qf.shape, generator=g, device=dev)).bfloat16()
+    want2 = ops.select(c, wl.batch, q2, wl.k_pool, workspace=space)[:3]
+    run(q2, want2)
+    run(q2, want2)
+
+
+def test_fused_select_hint_with_ties_and_a_batch(dev):
+    """The band path where it is hardest: exact ties at the k-th vote inside and across
+    workgroups (duplicated key rows), and a batch whose requests differ in length, one of them
+    dense; the second launch (hints set by the first) equals the first."""
+    import dataclasses
+    lens, ks = [9000, 40, 5200, 7000], [256, 64, 100, 256]
+    say(f"fused select with hints, ties, lens={lens}")
+    wl = small(dev, SHAPES[0], seed=103, lens=lens, ks=ks, page=16, top_k=256)
+    c = wl.cfg
+    # duplicate rows: every candidate of request 0 shares its key row with two others
+    tabs = cpu_tabs(wl)
+    rows = tabs[0][c.n_init:lens[0] - c.n_local].long().to(dev)
+    src = rows[torch.arange(rows.shape[0], device=dev) // 3 * 3]
+    wl.k_pool[rows] = wl.k_pool[src]
+    qf = fingerprint(wl, dev)
+    space = ops.select_workspace(c, wl.batch, dev)
+    want = ops.select(c, wl.batch, qf, wl.k_pool, workspace=space)[:3]
+    hint = torch.zeros(len(lens), dtype=torch.int32, device=dev)
+    hinted = dataclasses.replace(wl.batch, hint=hint)
+    for launch in range(3):
+        got = ops.select(c, hinted, qf, wl.k_pool, workspace=space)[:3]
+        torch.cuda.synchronize()
+        assert not ops.select_fault(c, hinted, space)
+        assert torch.equal(got[2], want[2])
+        for b in range(len(lens)):
+            S = int(want[2][b])
+            assert torch.equal(got[0][b, :S], want[0][b, :S]), (launch, b)
+            assert torch.equal(got[1][b, :S], want[1][b, :S]), (launch, b)
+    assert int(hint[1]) == 0 and all(int(hint[b]) > 0 for b in (0, 2, 3))
+    # and against the oracle
+    votes = ops.select(c, wl.batch, qf, wl.k_pool, want_votes=True, workspace=space)[3]
+    torch.cuda.synchronize()
+    for b in (0, 2, 3):
+        n = lens[b] - c.n_init - c.n_local
+        v = votes[b, :n].cpu()
+        order = sorted(range(n), key=lambda t: (-v[t].item(), t))[:ks[b]]
+        S = int(got[2][b])
+        assert sorted(order) == (got[1][b, c.n_init:S - c.n_local] - c.n_init).tolist(), b

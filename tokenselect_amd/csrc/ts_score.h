@@ -73,6 +73,9 @@ struct ScoreArgs {
   uint32_t* fault_word;   // votes-only: the word the kernels after this one consult
   uint32_t absent;        // team members that never arrive (tests of the give-up path)
   uint32_t* fault_out;    // caller's word, set to 1 when a wait gave up, or NULL
+  int32_t* hint;          // [B] threshold bin + 1 of the last selection (0: none), or NULL
+  uint32_t* band_above;   // [B][kBandBins][kSelMaxChunks]: tokens of a workgroup above a band bin << 16 | in it
+  uint4* band_slots;      // [B][kBandBins][kSelMaxChunks]: kBandSlots packed candidates
   int pool_kernel;        // max-pool window over the votes (tr.py:366-369), <= 0: off
   float* pool_votes;      // [B,pool_stride] un-pooled votes exchanged between workgroups
   int64_t pool_stride;
@@ -99,7 +102,28 @@ constexpr int kSelMaxBin = kSelHist2 + 1024;
 constexpr int kSelListCap = 256;
 constexpr int kSelListParts = 8;
 constexpr int kSelListCount = kSelMaxBin + kSelHistCopies * 32;
-constexpr int kSelCounterWords = kSelListCount + kSelListParts * 32;
+// With a hint of where the threshold bin is going to be (ts_batch.threshold_hint: the bin of
+// the request's previous selection on the same layer), every workgroup publishes, together
+// with its histogram and before the first rendezvous, what the last round would otherwise
+// need a rendezvous of its own for, for each of the kBandBins bins around the hint: one word
+// with the number of its tokens above that bin and of its candidates in it; those
+// candidates (up to kBandSlots, packed into 32 bits each: the low 21 key bits and the
+// token's index in the workgroup, which is why the band needs workgroups of at most 1024
+// tokens; into a 16-byte piece of its own, no counter to reserve from, and only the entries
+// the word counts are ever read, so nothing is cleared); and its counts of the band's bins
+// added to a small histogram of the band (kBandHistCopies copies a line apart, slot
+// kBandBins of each: the tokens above the band).  After the rendezvous the small histogram
+// says whether the threshold bin lies in the band, and if no workgroup had more candidates
+// in it than slots, the selection is through: one rendezvous, and a fraction of the
+// histogram to read.  Every memory-side atomic counts here (a few thousand of them in a
+// microsecond are what the device serves): a narrow band, and nothing written that is empty.
+constexpr int kBandBins = 8;
+constexpr int kBandBelow = 4;   // the band is [hint - kBandBelow, hint - kBandBelow + kBandBins)
+constexpr int kBandSlots = 4;   // candidates a workgroup can publish per bin (one 16-byte piece)
+constexpr int kBandMaxTokens = 1024;  // tokens per workgroup the packed index can address
+constexpr int kBandHistCopies = 32;   // one 128-byte line each: adds to one line are served one by one
+constexpr int kSelBandHist = kSelListCount + kSelListParts * 32;  // copies x 32 words (kBandBins + 1 live)
+constexpr int kSelCounterWords = kSelBandHist + kBandHistCopies * 32;
 
 // Workgroups of one request the workspace of ts_select is laid out for (the device keeps
 // at most 512 resident at once).
@@ -107,7 +131,8 @@ constexpr int kSelMaxChunks = 1024;
 
 // Workspace of ts_select, carved in this order (256-byte aligned pieces).
 struct SelectWorkspace {
-  size_t partials, counters, stats, block_counts, short_list, pool_votes, sync, total;  // sync stays last
+  size_t partials, counters, stats, block_counts, short_list, band_above, band_slots, pool_votes, sync,
+      total;  // sync stays last
   int64_t stats_stride;
   int64_t pool_stride;
   int tokens_per_block;  // 0: the shape does not fit the fused kernel

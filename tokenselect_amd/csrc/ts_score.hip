@@ -538,6 +538,8 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     first_pos = a.n_init;
   }
   const int block_lo = chunk * lp.tokens_per_block;
+  // (asked for here, long before it is used: the bin of the request's last selection)
+  const int hint_word = (FUSED && !PACKED && a.hint) ? a.hint[b] : 0;
   if constexpr (PACKED) {
     __shared__ uint32_t team_lds[8];
     if (n <= 0) return;  // dense or served by the cache: nothing to select, not on the team
@@ -775,8 +777,13 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     __shared__ uint32_t lh[kTopkBins];
     __shared__ uint32_t scratch[16];
     const int tid = threadIdx.x;
+    static_assert(kBandSlots == 4, "a workgroup's candidates of a bin are one 16-byte piece");
+    __shared__ uint32_t band_lds[kBandBins][kBandSlots];
+    __shared__ uint32_t band_count[kBandBins + 1];  // per bin; [kBandBins]: tokens above the band
     for (int i = tid; i < kTopkBins; i += 256) lh[i] = 0u;
     if (tid < 16) scratch[tid] = 0u;
+    if (tid < kBandBins * kBandSlots) band_lds[tid / kBandSlots][tid % kBandSlots] = 0u;
+    if (tid <= kBandBins) band_count[tid] = 0u;
     TS_MARK(1);
     __syncthreads();  // scores, own maxima and the cleared histogram are in LDS for all
     TS_MARK(2);
@@ -898,14 +905,36 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     }
     // Local histogram: one LDS atomic per candidate (lanes that hit the same bin are
     // performed one after the other, which for 256 candidates is a few hundred cycles).
+    // With a hint, also what the band around it needs: the candidates of each band bin go
+    // to slots in LDS (published below), and the tokens above the band are counted.
+    const int hint_bin = hint_word - 1;
+    const bool banded = hint_bin >= 0 && hint_bin < kTopkBins && lp.tokens_per_block <= kBandMaxTokens &&
+                        req_chunks <= kSelMaxChunks / 2;
+    const int band_lo = hint_bin - kBandBelow;  // (bins outside [0, kTopkBins) hold nothing)
+    uint32_t over_band = 0;  // this thread's tokens above the band
     for (int base = 0; base < count; base += 256) {
       const bool have = base + tid < count;
-      const uint32_t bin = have ? key_bin0(key_of(base + tid)) : 0u;
+      const uint32_t key = have ? key_of(base + tid) : 0u;
+      const uint32_t bin = have ? key_bin0(key) : 0u;
       if (have) atomicAdd(&lh[bin], 1u);
       uint32_t top = bin;
 #pragma unroll
       for (int off = 32; off >= 1; off >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, off));
       if (lane == 0) atomicMax(&scratch[8], top);
+      if (banded) {
+        const int d = (int)bin - band_lo;
+        if (have && d >= 0 && d < kBandBins) {
+          const uint32_t at = atomicAdd(&band_count[d], 1u);
+          if (at < (uint32_t)kBandSlots)
+            band_lds[d][at] = 0x80000000u | ((key & 0x1fffffu) << 10) | (uint32_t)(base + tid);
+        }
+        over_band += (have && d >= kBandBins) ? 1u : 0u;
+      }
+    }
+    if (banded) {
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) over_band += __shfl_xor(over_band, off);
+      if (lane == 0 && over_band) atomicAdd(&band_count[kBandBins], over_band);
     }
     __syncthreads();
 
@@ -929,12 +958,116 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       }
       if (tid == 0)
         done += fetch_max_coherent(&ctr[kSelMaxBin + (chunk % kSelHistCopies) * 32], scratch[8]);
+      if (banded && wave == 1) {
+        // The band.  Lane l holds the count of band bin l (lane kBandBins: of the bins above
+        // the band); the tokens above bin l are the sum over the lanes after it.
+        uint4* slots = a.band_slots + (size_t)b * kBandBins * kSelMaxChunks;
+        uint32_t* above = a.band_above + (size_t)b * kBandBins * kSelMaxChunks;
+        const uint32_t here = lane <= kBandBins ? band_count[lane] : 0u;
+        uint32_t run = here;  // becomes the sum over lanes l .. l + 15
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) {
+          const uint32_t up = (uint32_t)__shfl_down((int)run, off);
+          run += lane + off < 64 ? up : 0u;
+        }
+        static_assert(kBandBins + 1 <= 16, "the sum spans the band");
+        if (lane < kBandBins) {
+          done += __hip_atomic_exchange(&above[(size_t)lane * kSelMaxChunks + chunk], ((run - here) << 16) | here,
+                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          // (the candidates: the first 8-byte half of the piece, the second only if used)
+          uint64_t* piece = (uint64_t*)&slots[(size_t)lane * kSelMaxChunks + chunk];
+          if (here >= 1)
+            done += __hip_atomic_exchange(piece, (uint64_t)band_lds[lane][0] | ((uint64_t)band_lds[lane][1] << 32),
+                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (here >= 3)
+            done += __hip_atomic_exchange(piece + 1, (uint64_t)band_lds[lane][2] | ((uint64_t)band_lds[lane][3] << 32),
+                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (lane <= kBandBins && here)
+          done += fetch_add_coherent(&ctr[kSelBandHist + (chunk % kBandHistCopies) * 32 + lane], here);
+      }
       await(done);
     }
     TS_MARK(7);
     grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
     TS_MARK(8);
     uint32_t t0 = 0, above0 = 0, in_bin0 = 0;
+    // With a hint: the band's small histogram, the flags, the counts of the workgroups before
+    // this one and every workgroup's slots for the bin the hint names are requested
+    // together (the bin is a guess: the threshold bin is known after the search, and
+    // another bin of the band costs one more round of loads).
+    constexpr int kBandLoads = kSelMaxChunks / 2 / 256;  // (512 chunks at most)
+    uint32_t band_word[kBandLoads];
+    uint4 band_piece[kBandLoads];
+    auto load_band = [&](int d) {
+      const uint32_t* above = a.band_above + ((size_t)b * kBandBins + d) * kSelMaxChunks;
+      const uint4* slots = a.band_slots + ((size_t)b * kBandBins + d) * kSelMaxChunks;
+#pragma unroll
+      for (int r = 0; r < kBandLoads; ++r) {
+        const int at = tid + 256 * r;
+        band_word[r] = 0u;
+        band_piece[r] = make_uint4(0u, 0u, 0u, 0u);
+        if (at < req_chunks) {
+          band_word[r] = load_coherent(&above[at]);
+          const uint64_t lo = __hip_atomic_load((const uint64_t*)&slots[at], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint64_t hi = __hip_atomic_load((const uint64_t*)&slots[at] + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          band_piece[r] = make_uint4((uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32));
+        }
+      }
+    };
+    bool found = false;     // the threshold bin is known
+    bool from_band = false; // and the band's slots hold its candidates
+    if (banded) {
+      uint32_t* band_hist = lh + 1960;   // [kBandBins + 1] (the histogram array is free again)
+      if (tid <= kBandBins) band_hist[tid] = 0u;
+      if (tid == 32) lh[2000] = 0u;      // a workgroup with more candidates in the bin than slots
+      __syncthreads();
+      constexpr int kWords = kBandHistCopies * (kBandBins + 1);
+      constexpr int kPerThread = (kWords + 255) / 256;
+      uint32_t part[kPerThread];
+#pragma unroll
+      for (int r = 0; r < kPerThread; ++r) {
+        const int word = tid + 256 * r;
+        part[r] = word < kWords
+                      ? load_coherent(&ctr[kSelBandHist + (word / (kBandBins + 1)) * 32 + word % (kBandBins + 1)])
+                      : 0u;
+      }
+      load_band(kBandBelow);
+#pragma unroll
+      for (int r = 0; r < kPerThread; ++r)
+        if (part[r]) atomicAdd(&band_hist[(tid + 256 * r) % (kBandBins + 1)], part[r]);
+      __syncthreads();
+      // Downwards from the bins above the band: the bin in which the count reaches k.
+      uint32_t run = band_hist[kBandBins];
+      int d0 = -1;
+      if (run < k) {
+        for (int d = kBandBins - 1; d >= 0; --d) {
+          const uint32_t here = band_hist[d];
+          if (run + here >= k) {
+            d0 = d;
+            in_bin0 = here;
+            break;
+          }
+          run += here;
+        }
+      }
+      if (d0 >= 0 && band_lo + d0 >= 0) {
+        found = true;
+        t0 = (uint32_t)(band_lo + d0);
+        above0 = run;
+        if (in_bin0 <= (uint32_t)kSelListCap) {
+          if (d0 != kBandBelow) load_band(d0);
+          bool fits = true;
+#pragma unroll
+          for (int r = 0; r < kBandLoads; ++r) fits = fits && (band_word[r] & 0xffffu) <= (uint32_t)kBandSlots;
+          if (!fits) lh[2000] = 1u;
+          __syncthreads();
+          from_band = lh[2000] == 0u;
+        }
+      }
+      __syncthreads();
+    }
+    if (!found) {
     // The search starts at the highest occupied bin of the request.  Together with the
     // words that hold it, the 128 bins below a guess (a little above this workgroup's
     // own highest bin) are fetched; the guess serves if no bin above it is occupied.
@@ -980,6 +1113,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       top -= kWindow;
       if (top < 0) break;
       mine = bins_below(top);
+    }
     }
 
     TS_MARK(9);
@@ -1029,7 +1163,40 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     uint32_t kth, need_eq = 0, pos_thr = 0;
     if (tid < 8) scratch[8 + tid] = 0u;
     __syncthreads();
-    if (listed) {
+    // With a hint whose band holds the threshold bin, everything the ranking needs was
+    // published before the first rendezvous: no list round.  The test was the same for every
+    // workgroup of the request (the band's histogram, the flags), so all take the same way.
+    bool has = false;
+    uint2 e = make_uint2(0u, 0u);
+    if (from_band) {
+      uint2* entries_lds = (uint2*)(lh + 1024);  // [kSelListCap]
+      uint32_t band_sure = 0;  // tokens above the bin in the workgroups before this one
+#pragma unroll
+      for (int r = 0; r < kBandLoads; ++r) {
+        const uint32_t packed[4] = {band_piece[r].x, band_piece[r].y, band_piece[r].z, band_piece[r].w};
+        const uint32_t from = (uint32_t)(tid + 256 * r) * (uint32_t)lp.tokens_per_block;  // that workgroup's first token
+        const uint32_t have = band_word[r] & 0xffffu;  // (zero where the load was skipped)
+        if (tid + 256 * r < chunk) band_sure += band_word[r] >> 16;
+#pragma unroll
+        for (int h2 = 0; h2 < 4; ++h2)
+          if ((uint32_t)h2 < have) {
+            const uint32_t at = atomicAdd(&scratch[15], 1u);
+            if (at < (uint32_t)kSelListCap)
+              entries_lds[at] = make_uint2((t0 << 21) | ((packed[h2] >> 10) & 0x1fffffu), from + (packed[h2] & 1023u));
+          }
+      }
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) band_sure += __shfl_xor(band_sure, off);
+      if (lane == 0) atomicAdd(&scratch[10], band_sure);
+      __syncthreads();
+      // (every candidate of the bin is in a slot: the count is that of the histogram)
+      if (scratch[15] != in_bin && tid == 0)
+        __hip_atomic_store(&lp.sync[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      has = (uint32_t)tid < min(scratch[15], (uint32_t)kSelListCap);
+      if (has) e = entries_lds[tid];
+      __syncthreads();
+      TS_MARK(10);
+    } else if (listed) {
       // Last round, short form: the candidates of the threshold bin are appended to
       // the list (in kSelListParts parts with a counter each, a wavefront reserving
       // its entries with one add), and every workgroup publishes how many of its
@@ -1072,7 +1239,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       constexpr uint32_t kPerPart = kSelListCap / kSelListParts;
       const uint32_t fill =
           tid < kSelListParts ? load_coherent(&ctr[kSelListCount + tid * 32]) : 0u;
-      uint2 e = load_coherent(&list[(tid % kSelListParts) * kSelListCap + tid / kSelListParts]);
+      e = load_coherent(&list[(tid % kSelListParts) * kSelListCap + tid / kSelListParts]);
       {
         uint32_t sure = 0;
         for (int j = tid; j < chunk; j += 256) sure += load_coherent(&counts[j]).x;
@@ -1088,7 +1255,6 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         entries += scratch[p];
         longest = max(longest, scratch[p]);
       }
-      bool has;
       if (longest <= kPerPart) {
         has = (uint32_t)tid / kSelListParts < scratch[tid % kSelListParts];
       } else {  // uneven parts: entry t of the concatenation
@@ -1106,6 +1272,8 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         has = has && (uint32_t)tid < min(entries, (uint32_t)kSelListCap);
         if (has) e = load_coherent(&list[from * kSelListCap + at]);
       }
+    }
+    if (listed) {
       const uint64_t mine = has ? ((uint64_t)e.x << 32) | (uint64_t)(0xffffffffu - e.y) : 0ull;
       const uint32_t my_pos = e.y;
       // The need-th largest entry: one more histogram level, over the next 8 key bits
@@ -1274,6 +1442,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     if (chunk == 0 && tid == 0) {
       const bool gave_up = load_coherent(&lp.sync[0]) != 0u;
       a.sel_len[b] = gave_up ? -1 : a.n_init + (int)k + a.n_local;
+      if (a.hint && !gave_up) a.hint[b] = (int)t0 + 1;  // where the next step's band is going to lie
       if (gave_up && a.fault_out)
         __hip_atomic_store(a.fault_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
@@ -1461,6 +1630,8 @@ SelectWorkspace select_workspace(const ts_config* cfg, int batch, int max_seq_le
   w.stats = take((size_t)kSyncSlots * w.stats_stride * sizeof(float));
   w.block_counts = take(B * (size_t)kSelMaxChunks * sizeof(uint2));
   w.short_list = take(B * kSelListParts * kSelListCap * sizeof(uint2));
+  w.band_above = take(B * kBandBins * (size_t)kSelMaxChunks * sizeof(uint32_t));
+  w.band_slots = take(B * kBandBins * (size_t)kSelMaxChunks * sizeof(uint4));
   w.pool_stride = (int64_t)align_up((size_t)std::max(max_n, 1), 64);
   w.pool_votes = take(cfg->pool_kernel > 0 ? B * (size_t)w.pool_stride * sizeof(float) : 0);
   w.sync = take(B * kSyncWords * 4);  // one rendezvous area per launch of a batch served in groups
@@ -1607,6 +1778,9 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   a.counters = (uint32_t*)(ws + w.counters);
   a.block_counts = (uint2*)(ws + w.block_counts);
   a.short_list = (uint2*)(ws + w.short_list);
+  a.hint = bt->threshold_hint;
+  a.band_above = (uint32_t*)(ws + w.band_above);
+  a.band_slots = (uint4*)(ws + w.band_slots);
   a.sel = sel;
   a.sel_pos = sel_pos;
   a.sel_stride = sel_stride;

@@ -69,6 +69,10 @@ class Batch:
     # framework's CPU copy of the lengths), or None: a batch too large for one selection
     # launch is then scored in phases packed by these bounds instead of by max_seq_len.
     host_seq_lens: Optional[torch.Tensor] = None
+    # [B] int32 on the device, zero before a request's first step and kept per (request,
+    # layer) across decode steps, or None: where the single-launch selection notes where the
+    # k-th vote lay, as a guess for the next step (ts_batch.threshold_hint).
+    hint: Optional[torch.Tensor] = None
     # Per-call options (``ts_batch``): take the separate kernels for this call; the call
     # repeats the step's previous one after a give-up; bound of a grid-wide wait in
     # microseconds (0: the library's 10 ms); workgroups that never arrive (tests of the
@@ -225,8 +229,12 @@ def _c_batch(cfg: LayerConfig, bt: Batch) -> TsBatch:
             not bt.host_seq_lens.is_contiguous()):
         raise ValueError("host_seq_lens must be a contiguous [B] int32 tensor on the CPU")
     host = bt.host_seq_lens.data_ptr() if bt.host_seq_lens is not None else None
+    if bt.hint is not None:
+        _need(bt.hint, "hint", torch.int32, 1)
+        if bt.hint.shape[0] != bt.batch:
+            raise ValueError("hint must have one entry per request")
     return TsBatch(bt.batch, int(bt.max_seq_len), _p(bt.seq_lens), _p(bt.table),
-                   int(bt.table.stride(0)), _p(bt.k_per_req), _p(bt.fault), host,
+                   int(bt.table.stride(0)), _p(bt.k_per_req), _p(bt.fault), host, _p(bt.hint),
                    1 if bt.separate_kernels else 0, 1 if bt.rerun else 0, int(bt.wait_us),
                    int(bt.absent_workgroups))
 
@@ -423,6 +431,15 @@ def select_fault(cfg: LayerConfig, bt: Batch, workspace: torch.Tensor) -> bool:
     # the rendezvous areas (one of 65 x 4096 bytes per request) end the workspace; the
     # fault word is the first word of the first
     return bool(workspace.view(torch.int32)[nbytes // 4 - bt.batch * 65 * 1024].item())
+
+
+def select_rounds(cfg: LayerConfig, bt: Batch, workspace: torch.Tensor, rounds: int = 4):
+    """How many groups of workgroups completed each grid-wide round of the last
+    :func:`select` on ``workspace`` (synchronises): a round nobody met for shows zero."""
+    nbytes = _lib.load().ts_select_workspace_bytes(ctypes.byref(cfg.to_c()), bt.batch,
+                                                   bt.max_seq_len)
+    first = nbytes // 4 - bt.batch * 65 * 1024
+    return workspace.view(torch.int32)[first + 2:first + 2 + rounds].tolist()
 
 
 def scores_head_major(cfg: LayerConfig, scores: torch.Tensor) -> torch.Tensor:

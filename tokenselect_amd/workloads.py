@@ -35,12 +35,13 @@ class Workload:
     planted: List[torch.Tensor] = field(default_factory=list)  # per request: logical positions
     free_pages: Optional[torch.Tensor] = None   # [extra_pages] int32: pages no request holds
     host_lengths: bool = False                  # hand the lengths to the library on the host too
+    hint: Optional[torch.Tensor] = None         # [B] int32: Batch.hint, kept across the steps of a run
 
     @property
     def batch(self) -> Batch:
         host = torch.tensor(self.seq_lens, dtype=torch.int32) if self.host_lengths else None
         return Batch(self.seq_lens_dev, self.table, max(self.seq_lens), self.k_per_req,
-                     host_seq_lens=host)
+                     host_seq_lens=host, hint=self.hint)
 
     def score_bytes(self) -> int:
         """Algorithmic bytes of the scoring pass: every candidate K row once,
