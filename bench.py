@@ -284,13 +284,14 @@ def bench_trace(args, ops, workloads, dev):
     def run_trace():
         table, seq = table0.clone(), wl.seq_lens_dev.clone()
         cache = ops.SelectionCache.allocate(c, B, dev)
+        hint = None if args.no_hint else torch.zeros(B, dtype=torch.int32, device=dev)
         pages = ops.PagePool.of(wl.free_pages) if ps > 1 else None
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for t in range(steps):
             ops.kv_store(c, k_new[t], v_new[t], None if pages else free[t], wl.k_pool, wl.v_pool, table,
                          seq, pages=pages)
-            layer(qs[t], wl.k_pool, wl.v_pool, ops.Batch(seq, table, L0 + t + 1), cache)
+            layer(qs[t], wl.k_pool, wl.v_pool, ops.Batch(seq, table, L0 + t + 1, hint=hint), cache)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps * 1e6, cache
 

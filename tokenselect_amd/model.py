@@ -116,6 +116,9 @@ class Decoder:
         self.caches: List[Optional[SelectionCache]] = [
             SelectionCache.allocate(self.cfg, B, device) if query_cache else None
             for _ in range(mc.layers)]
+        # Per (layer, request): where the k-th vote of the last selection lay, the single-launch
+        # selection's guess for the next step.
+        self.hints = torch.zeros((mc.layers, B), dtype=torch.int32, device=device)
         # Per-call options handed to the layer (tests force a give-up through them).
         self.layer_options = {}
         self.steps_redone = 0
@@ -152,7 +155,8 @@ class Decoder:
                              self.num_tokens[l])
             attn, sel, _, sel_len = self.attention(
                 q, self.k_pools[l], self.v_pools[l],
-                Batch(self.num_tokens[l], self.table, max_len, host_seq_lens=host_lens, **self.layer_options),
+                Batch(self.num_tokens[l], self.table, max_len, host_seq_lens=host_lens, hint=self.hints[l],
+                      **self.layer_options),
                 self.caches[l])
             if trace is not None:
                 if k is None:   # the rows as they landed in the pools

@@ -187,6 +187,7 @@ class BatchTokenRetriever:
         self.token_indices = torch.stack([r.token_indices for r in retrievers], dim=1).contiguous()
         self.num_tokens = [[r.num_tokens[l] for r in retrievers] for l in range(self.num_layers)]
         self._num_tokens_dev = torch.stack([r._num_tokens_dev for r in retrievers], dim=1).contiguous()
+        self._threshold_hints = torch.stack([r._threshold_hints for r in retrievers], dim=1).contiguous()
         self._layers = {}
         self._caches = None
         if QUERY_CACHE:
@@ -231,7 +232,8 @@ class BatchTokenRetriever:
         # launch is then scored in phases packed by what the requests hold.
         bt = ops.Batch(self._num_tokens_dev[layer_id], self.token_indices[layer_id],
                        max(self.num_tokens[layer_id]),
-                       host_seq_lens=torch.tensor(self.num_tokens[layer_id], dtype=torch.int32))
+                       host_seq_lens=torch.tensor(self.num_tokens[layer_id], dtype=torch.int32),
+                       hint=self._threshold_hints[layer_id])
         out = torch.empty((self.batch, self.num_heads * self.head_dim), dtype=q.dtype, device=q.device)
         runner(q, k_buffer, v_buffer, bt, self._caches[layer_id] if self._caches else None, out=out)
         return out
@@ -280,6 +282,9 @@ class TokenRetriever:
         self._num_tokens_dev = torch.zeros((num_layers,), device=device, dtype=torch.int32)
         self._cache_len_dev = torch.zeros((num_layers,), device=device, dtype=torch.int32)
         self._counters_dev = torch.zeros((num_layers, 2), device=device, dtype=torch.int64)
+        # Where the k-th vote of a layer's last selection lay: the single-launch selection's
+        # guess for the next step (ts_batch.threshold_hint), one word per layer.
+        self._threshold_hints = torch.zeros((num_layers,), device=device, dtype=torch.int32)
         self._layers = {}
         self.clear()
 
@@ -291,6 +296,7 @@ class TokenRetriever:
         self._num_tokens_dev.zero_()
         self._cache_len_dev.zero_()
         self._counters_dev.zero_()
+        self._threshold_hints.zero_()
 
     def get_all_tokens(self, layer_id):
         return self.token_indices[layer_id, : self.num_tokens[layer_id]]
@@ -388,7 +394,8 @@ class TokenRetriever:
         cfg = self._config(n_init, n_local, topk)
         qf = self._fingerprint(query)
         bt = ops.Batch(self._num_tokens_dev[layer_id:layer_id + 1],
-                       self.token_indices[layer_id:layer_id + 1], current_num_tokens)
+                       self.token_indices[layer_id:layer_id + 1], current_num_tokens,
+                       hint=self._threshold_hints[layer_id:layer_id + 1] if query.shape[0] == 1 else None)
         cache = self._cache(layer_id)
         k_buffer = self.token_fingerprints[layer_id]
         # The large buffers are kept between calls, sized for the longest table.
@@ -440,7 +447,8 @@ class TokenRetriever:
             runner = ops.DecodeLayer(cfg, 1, self.max_num_tokens, self.device)
             self._layers[key] = runner
         bt = ops.Batch(self._num_tokens_dev[layer_id:layer_id + 1],
-                       self.token_indices[layer_id:layer_id + 1], self.num_tokens[layer_id])
+                       self.token_indices[layer_id:layer_id + 1], self.num_tokens[layer_id],
+                       hint=self._threshold_hints[layer_id:layer_id + 1])
         out = torch.empty((1, self.num_heads * self.head_dim), dtype=q.dtype, device=q.device)
         cache = self._cache(layer_id)
         runner(q, k_buffer, v_buffer, bt, cache, out=out)
