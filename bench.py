@@ -43,9 +43,13 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # figures are recorded under profiles/.  Workloads not measured that way give null.
 # Each figure carries the commit of the kernels it was measured on: a later change to the
 # kernel makes it stale until the two counter runs are repeated.
-MEASURED_TRAFFIC = {  # workload -> (bytes per launch of its dominant kernel, commit)
-    "C2": (269711053, "6c0d379"),  # profiles/decode_layer_c2_hbm_traffic.txt
+MEASURED_TRAFFIC = {  # workload -> (bytes per launch of its dominant kernel, commit); profiles/decode_layer_hbm_traffic.txt
+    "C2": (269663584, "385f8a7"),        # ts_select, score_kernel<8,4,false,2>
+    "C3": (2229693645, "385f8a7"),       # the votes-only launch, score_kernel<8,4,false,3>
+    "C5-layer": (2154547035, "385f8a7"),  # likewise
+    "MODEL": (2159012843, "385f8a7"),     # likewise, inside the 32-layer decoder (page 1)
 }
+MEASURED_ATTN_TRAFFIC = {"C2": 12175815, "C3": 198546049, "C5-layer": 102095478}  # attn_kernel<4>, same runs
 
 
 def event_time_us(fn, launches: int, warmup: int, before=None, burst: int = 1):
@@ -177,6 +181,7 @@ def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
     attn = {"kernel": "ts::attn_kernel<G> (+ a 1 us ticket-clearing kernel when called on its own)",
             "achieved": round(attn_bytes / attn_us / 1e3, 1), "unit": "GB/s",
             "frac": round(attn_bytes / attn_us / 1e3 / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_ATTN_TRAFFIC.get(wl.name.split()[0]),
             "bytes_per_launch": attn_bytes, "us_per_launch": round(attn_us, 2)}
     return roofline, score_only, attn
 
@@ -508,7 +513,9 @@ def bench_model(args, ops, dev):
         "hbm_frac_whole_step": round(step_bytes / step_s / 1e9 / HBM_PEAK_GBS, 4),
         "roofline": {"bound": "hbm", "kernel": dom_kernel,
                      "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC["MODEL"][0] if (B, L, c.top_k) == (4, 262144, 4096) else None,
+                     "traffic_measured_at": MEASURED_TRAFFIC["MODEL"][1],
                      "bytes_per_launch": score_bytes, "us_per_launch": round(score_us, 2),
                      "us_min": round(score_min, 2)},
         "score_only": score_only,
