@@ -591,6 +591,23 @@ def test_select_randomised(dev):
         assert not ops.select_fault(c, wl.batch, space)
         votes_sep, _ = ops.vote(c, wl.batch, *ops.score(c, wl.batch, qf, wl.k_pool))
         separate = ops.topk_ragged(c, wl.batch, votes_sep)
+        # The same launch with threshold hints: none yet, its own from the launch before, then
+        # hints moved by a few bins or set to nonsense, request by request.  Bit for bit the same.
+        import dataclasses
+        hint = torch.zeros(B, dtype=torch.int32, device=dev)
+        hinted = dataclasses.replace(wl.batch, hint=hint)
+        for launch in range(4):
+            if launch >= 2:
+                moved = [rnd.choice([-5, -3, -1, 0, 1, 2, 4, 6, 900, -10000]) for _ in range(B)]
+                hint.add_(torch.tensor(moved, dtype=torch.int32, device=dev))
+            got = ops.select(c, hinted, qf, wl.k_pool, workspace=space)
+            torch.cuda.synchronize()
+            assert not ops.select_fault(c, hinted, space), f"seed={seed} launch {launch}"
+            assert torch.equal(got[2], sel_len), f"seed={seed} launch {launch}: lengths"
+            for b in range(B):
+                S = int(sel_len[b])
+                assert torch.equal(got[0][b, :S], sel[b, :S]) and torch.equal(got[1][b, :S], sel_pos[b, :S]), \
+                    f"seed={seed} launch {launch} b={b}: the selection with a hint differs"
         for path, (sel, sel_pos, sel_len), votes in (("fused", (sel, sel_pos, sel_len), votes),
                                                      ("separate", separate, votes_sep)):
             for b, (L, k) in enumerate(zip(lens, ks)):
