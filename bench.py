@@ -178,7 +178,9 @@ def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
     attn_us, _ = event_time_us(
         lambda i: ops.sparse_decode_attention(c, wl.q, k_pools[i % n_pools], v_pools[i % n_pools],
                                               sel, sel_len), steps, warmup, burst=8)
-    attn = {"kernel": "ts::attn_kernel<G> (+ a 1 us ticket-clearing kernel when called on its own)",
+    mfma = ops.attention_kernel_form(c, sel.shape[0], sel.shape[1]) == 1
+    attn = {"kernel": ("ts::attn_mfma_kernel<G> (matrix cores)" if mfma else "ts::attn_kernel<G> (vector units)")
+                      + " + a 1 us ticket-clearing kernel when called on its own",
             "achieved": round(attn_bytes / attn_us / 1e3, 1), "unit": "GB/s",
             "frac": round(attn_bytes / attn_us / 1e3 / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_ATTN_TRAFFIC.get(wl.name.split()[0]),

@@ -328,8 +328,16 @@ int ts_selcache_step(const ts_config* cfg, const ts_batch* bt, const void* qf,
  * q, out: [B,H,D] bf16; k_pool, v_pool: [pool_rows,Hkv,D] bf16;
  * sel [B, sel_stride] int32 with sel_len[b] valid entries (<= max_sel_len); every
  * row holds at least max_sel_len entries, those past sel_len[b] are read (the
- * slots are requested together with the length) but not used. */
+ * slots are requested together with the length) but not used.
+ * Two kernels serve it.  Launches in which a workgroup reads one batch of rows (a few
+ * requests: up to 512 workgroups of 128 list entries cover the lists) compute in fp32 on
+ * the vector units.  Launches with longer ranges per workgroup (many requests) run on the
+ * matrix cores: rotated keys and softmax weights are rounded to bf16 for
+ * v_mfma_f32_16x16x32_bf16 with fp32 accumulation, as the tensor-core path of the
+ * reference's attention library does; the outputs of the two differ by about one unit of
+ * bf16 rounding.  ts_attn_kernel_form tells which one a shape gets (0 vector, 1 matrix). */
 size_t ts_attn_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_sel_len);
+int ts_attn_kernel_form(const ts_config* cfg, int32_t batch, int32_t max_sel_len);
 int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_pool,
                           const void* v_pool, int64_t pool_rows, const int32_t* sel,
                           int64_t sel_stride, const int32_t* sel_len, int32_t batch,

@@ -688,6 +688,44 @@ def test_sparse_attention(dev, shape, rope_mode):
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("rope_mode,cap", [("ROPE_LLAMA", 0.0), ("NONE", 0.0), ("ROPE_LLAMA", 25.0)])
+def test_sparse_attention_on_the_matrix_cores(dev, shape, rope_mode, cap):
+    """Many requests with long lists: a workgroup walks several tiles and the launch takes the
+    matrix-core kernel (asserted), every head shape, with and without the rotation and the soft
+    cap; ragged lengths that end inside a tile, inside a wavefront's range, at one entry and at
+    none; the one-request launch of the same lists (vector kernel) agrees within the rounding
+    of the matrix operands."""
+    say(f"attention on the matrix cores H={shape['num_heads']} Hkv={shape['num_kv_heads']} {rope_mode} cap={cap}")
+    lens = [2600, 2599, 2541, 1025, 700, 333, 65, 64, 33, 17, 1, 0, 2600, 1800]
+    B, width = len(lens), 2600
+    wl = small(dev, shape, seed=41, lens=[3000] * B, ks=[64] * B)
+    c = wl.cfg
+    c.rope_mode, c.logit_cap = rope_mode, cap
+    assert ops.attention_kernel_form(c, B, width) == 1
+    assert ops.attention_kernel_form(c, 1, width) == 0
+    g = torch.Generator().manual_seed(42)
+    sel = torch.zeros((B, width), dtype=torch.int32)
+    for b, S in enumerate(lens):
+        sel[b, :S] = torch.randint(0, wl.k_pool.shape[0], (S,), generator=g).int()
+        sel[b, S:] = 0x7fffffff     # entries past the length are never used
+    sel_len = torch.tensor(lens, dtype=torch.int32)
+    out = ops.sparse_decode_attention(c, wl.q, wl.k_pool, wl.v_pool, sel.to(dev), sel_len.to(dev))
+    torch.cuda.synchronize()
+    kc, vc, qc = wl.k_pool.cpu(), wl.v_pool.cpu(), wl.q.cpu()
+    for b, S in enumerate(lens):
+        if S == 0:
+            assert not bool(out[b].any()), f"b={b}: empty list"
+            continue
+        ref = oracle.attend.sparse_decode_attention(
+            qc[b].view(c.num_heads, 128), kc, vc, sel[b, :S], 128 ** -0.5, c.rope_theta, 1.0, cap, rope_mode)
+        err = (out[b].cpu().float() - ref.reshape(-1).float()).abs().max().item()
+        assert err <= 2e-2, f"attention b={b} S={S}: max abs err {err}"
+        alone = ops.sparse_decode_attention(c, wl.q[b:b + 1], wl.k_pool, wl.v_pool, sel[b:b + 1].to(dev),
+                                            sel_len[b:b + 1].to(dev))
+        assert (alone[0].float() - out[b].float()).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
 def test_selection_cache_decisions(dev, shape):
     """ts_selcache_step on its own, every head shape (4 to 32 heads: one to four 16-byte
     pieces of the query per thread): queries at chosen cosines to the cached one on both sides

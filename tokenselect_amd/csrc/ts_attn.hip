@@ -2,8 +2,11 @@
 // reference calls at tr.py:815-823 (page size 1, in-kernel Llama RoPE).
 //
 // Split-K in one launch: grid (splits, Hkv, B).  A workgroup owns a contiguous
-// range of the request's selected list for one KV head and keeps the G = H/Hkv
-// query heads that read it in registers.  Sixteen lanes gather one K row and one
+// range of the request's selected list for one KV head and the G = H/Hkv query heads
+// that read it.  Two kernels: attn_kernel (vector units, fp32 throughout) where a
+// workgroup reads one batch of rows, attn_mfma_kernel (matrix cores) where it walks
+// several; they share the end of the workgroup (attn_finish).  In attn_kernel the
+// query heads stay in registers and sixteen lanes gather one K row and one
 // V row (256 bytes each, as two 128-byte halves); the sixteen lane groups of a
 // workgroup walk the range with stride 16, eight tokens per lane group in flight
 // (the slots, then all keys, then all values are requested before the first is
@@ -15,6 +18,7 @@
 #include <math.h>
 
 #include <mutex>
+#include <type_traits>
 
 #include "ts_common.h"
 
@@ -60,6 +64,103 @@ __device__ __forceinline__ void store_coherent2(float* p, float x, float y) {
   __hip_atomic_store((uint64_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The end of an attention workgroup: its four wavefronts' partial (max, sum, acc) triples
+// of G head slots lie in LDS; they are merged, written with device-coherent stores, and the
+// workgroup that draws the last ticket of its (request, KV head, part) merges the splits and
+// writes the bf16 output.
+template <int G>
+__device__ __forceinline__ void attn_finish(const AttnArgs& a, int b, int kvh, int part, int split,
+                                            float (*sm_acc)[G][kHeadDim], float (*sm_m)[G],
+                                            float (*sm_l)[G], uint32_t* s_last_ptr) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int H = a.num_heads;
+  auto head_of_slot = [&](int g) { return kvh * a.group + min(part * G + g, a.group - 1); };
+  auto slot_active = [&](int g) { return part * G + g < a.group; };
+  uint32_t& s_last = *s_last_ptr;
+  __syncthreads();
+  // A thread owns two adjacent dims of one head: one 64-bit coherent store.
+  for (int idx = tid; idx < G * (kHeadDim / 2); idx += 256) {
+    const int g = idx / (kHeadDim / 2), d = (idx % (kHeadDim / 2)) * 2;
+    float mm = kNegBig;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mm = fmaxf(mm, sm_m[w][g]);
+    float o0 = 0.f, o1 = 0.f, ll = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float sc = __expf(sm_m[w][g] - mm);
+      o0 += sm_acc[w][g][d] * sc;
+      o1 += sm_acc[w][g][d + 1] * sc;
+      ll += sm_l[w][g] * sc;
+    }
+    if (!slot_active(g)) continue;
+    const size_t ph = ((size_t)b * H + head_of_slot(g)) * a.nsplit + split;
+    store_coherent2(a.part_acc + ph * kHeadDim + d, o0, o1);
+    if (d == 0) store_coherent2(a.part_ml + ph * 2, mm, ll);
+  }
+
+  // Ticket: the stores above are acknowledged before the workgroup is counted.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  uint32_t* ticket = a.tickets + ((size_t)b * a.num_kv_heads + kvh) * a.parts + part;
+  if (tid == 0) {
+    const uint32_t before =
+        __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = before + 1 == (uint32_t)a.nsplit ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!s_last) return;
+
+  // out[b,h,:] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s, rounded to bf16.
+  // A wavefront per head slot (a thread owns two adjacent dims, and a head has 64 such
+  // pairs): lane s fetches the (max, sum) of split s, the wave takes the maximum and
+  // lane s the weight of its split, so that the accumulators, all requested at once, are
+  // added up with weights that are ready (read lane by lane): no chain of dependent
+  // exponentials, and one statistics load per wave instead of one per split and thread.
+  static_assert(kHeadDim / 2 == 64, "one wavefront per head slot");
+  for (int idx = tid; idx < G * (kHeadDim / 2); idx += 256) {
+    const int g = idx / (kHeadDim / 2), d = (idx % (kHeadDim / 2)) * 2;
+    if (!slot_active(g)) continue;  // (uniform over the wave)
+    const size_t ph = ((size_t)b * H + head_of_slot(g)) * a.nsplit;
+    float mm = kNegBig, ll = 0.f, o0 = 0.f, o1 = 0.f;
+    for (int s0 = 0; s0 < a.nsplit; s0 += 32) {
+      // 32 splits at a time, branch-free: loads past the last split repeat it and get
+      // the weight zero.
+      float2 ac[32];
+#pragma unroll
+      for (int i = 0; i < 32; ++i)
+        ac[i] = load_coherent2(a.part_acc + (ph + min(s0 + i, a.nsplit - 1)) * kHeadDim + d);
+      const float2 ml = (lane < 32 && s0 + lane < a.nsplit)
+                            ? load_coherent2(a.part_ml + (ph + s0 + lane) * 2)
+                            : make_float2(kNegBig, 0.f);
+      float mx = ml.x;
+      mx = fmaxf(mx, dpp_move<kRowRor8>(mx));
+      mx = fmaxf(mx, dpp_move<kRowRor4>(mx));
+      mx = fmaxf(mx, dpp_move<kRowRor2>(mx));
+      mx = fmaxf(mx, dpp_move<kRowRor1>(mx));
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      const float mn = fmaxf(mm, __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(mx))));
+      const float keep = __expf(mm - mn);  // what earlier batches hold
+      const float w = (lane < 32 && s0 + lane < a.nsplit) ? __expf(ml.x - mn) : 0.f;
+      const float wl = ml.y * w;
+      o0 *= keep;
+      o1 *= keep;
+      ll *= keep;
+      mm = mn;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        const float wi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), i));
+        ll += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wl), i));
+        o0 += ac[i].x * wi;
+        o1 += ac[i].y * wi;
+      }
+    }
+    const uint32_t packed = (uint32_t)f32_to_bf16(ll > 0.f ? o0 / ll : 0.f) |
+                            ((uint32_t)f32_to_bf16(ll > 0.f ? o1 / ll : 0.f) << 16);
+    *(uint32_t*)(a.out + ((size_t)b * H + head_of_slot(g)) * kHeadDim + d) = packed;
+  }
+  if (tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 constexpr int kAttnInFlight = 8;  // tokens per lane group requested together
 
 // ROPE and CAP are compile-time so that the token loop carries no branches other
@@ -83,7 +184,6 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
   // Head g of this workgroup: the last part of a group of five or seven has one head too
   // many, which is computed (on the last real head's query) and not stored.
   auto head_of_slot = [&](int g) { return kvh * a.group + min(part * G + g, a.group - 1); };
-  auto slot_active = [&](int g) { return part * G + g < a.group; };
   // The ranges are cut from the longest list the launch was sized for, not from this
   // request's own length: the first slots can then be requested together with the
   // length instead of after it (a shorter request leaves its last workgroups idle).
@@ -315,88 +415,340 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
       }
     }
   }
-  __syncthreads();
-  // A thread owns two adjacent dims of one head: one 64-bit coherent store.
-  for (int idx = tid; idx < G * (kHeadDim / 2); idx += 256) {
-    const int g = idx / (kHeadDim / 2), d = (idx % (kHeadDim / 2)) * 2;
-    float mm = kNegBig;
+  attn_finish<G>(a, b, kvh, part, split, sm_acc, sm_m, sm_l, &s_last);
+}
+
+// ---------------------------------------------------------------------------------------
+// The same attention on the matrix cores, for launches in which a workgroup walks several
+// hundred tokens (many requests at once): there the loop above is bound by its vector
+// instructions (some 40 per token and wavefront: dot products, reductions over 16 lanes, a
+// softmax every lane of a token's group repeats), here a token costs about 16.
+//
+// A wavefront walks a contiguous quarter of the workgroup's range in tiles of 32 tokens.
+// v_mfma_f32_16x16x32_bf16 three times over:
+//   logits   S[token][head] = K' Q'^T : A = 16 rotated keys x 32 dims (lane (token l%16,
+//            l/16) loads 16 bytes of its token's row per 32 dims, rotates them in fp32 - the
+//            partner dims d and d + 64 are in the same lane - and rounds to bf16, as the
+//            tensor-core path of the reference's attention library does), B = the query
+//            heads as columns (G of 16 used), rotated to S - 1 and rounded once.
+//   V^T      a value row arrives like a key row (a lane holds 8 consecutive dims of one
+//            token); the matrix product with a 0/1 matrix that selects 16 of 32 dims leaves
+//            lane (dim l%16, l/16) with that dim of four consecutive tokens, exactly (bf16
+//            values summed with zeros in fp32): the transposition, without LDS.
+//   output   O^T[dim][head] += V^T P : A = 16 dims x 32 tokens from the step above, B = the
+//            weights of the tile, which the logits' product left in the lanes that need them
+//            (lane (head l%16, l/16): tokens 4 (l/16) + r of both 16-token halves).
+// Everything of a head lives in the four lanes of its column: the running maximum moves once
+// per tile (two exchanges between the lane groups), the sums stay per lane until the end.
+// The loads of the next tile's keys are issued when this tile's have been rotated, those of
+// its values after this tile's have been consumed: some 8 KB per wavefront are in flight at
+// any time.
+typedef __attribute__((ext_vector_type(8))) __bf16 at_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float at_f32x4;
+constexpr float kAttnLog2e = 1.4426950408889634f, kAttnLn2 = 0.6931471805599453f;
+constexpr int kAttnTile = 32;        // tokens per step of a wavefront
+constexpr int kAttnChunkUnit = 64;   // a workgroup's range is a multiple of this (16 per wavefront)
+
+__device__ __forceinline__ at_bf16x8 pack8(const float* x) {
+  const uint4 w = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]),
+                             pack_bf16(x[6], x[7]));
+  return __builtin_bit_cast(at_bf16x8, w);
+}
+__device__ __forceinline__ void unpack8(const uint4& w, float* f) {
+  f[0] = bf16_lo(w.x);
+  f[1] = bf16_hi(w.x);
+  f[2] = bf16_lo(w.y);
+  f[3] = bf16_hi(w.y);
+  f[4] = bf16_lo(w.z);
+  f[5] = bf16_hi(w.z);
+  f[6] = bf16_lo(w.w);
+  f[7] = bf16_hi(w.w);
+}
+
+// Tokens per workgroup of the matrix-core kernel for a launch of nsplit splits.
+__host__ __device__ __forceinline__ int attn_mfma_chunk(int max_sel_len, int nsplit) {
+  const int even = (max_sel_len + nsplit - 1) / nsplit;
+  return (even + kAttnChunkUnit - 1) / kAttnChunkUnit * kAttnChunkUnit;
+}
+
+// An index offset of zero that the compiler cannot see through, produced after `after` is:
+// LDS reads addressed with it stay where they are written (inside the loop, next to their
+// use) instead of being gathered at the top, where they would hold dozens of registers.
+__device__ __forceinline__ int opaque_zero(uint32_t after) {
+  int z = 0;
+  asm volatile("" : "+v"(z) : "v"(after));
+  return z;
+}
+
+template <int G, bool ROPE, bool CAP>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_kernel(
+    AttnArgs a) {
+  const int split = blockIdx.x, b = blockIdx.z;
+  const int kvh = blockIdx.y / a.parts, part = blockIdx.y % a.parts;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, qd = lane >> 4;
+  const int H = a.num_heads;
+  const int chunk = attn_mfma_chunk(a.max_sel_len, a.nsplit);
+  const int wlen = chunk / 4;
+  const int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
+  const size_t row_elems = (size_t)a.num_kv_heads * kHeadDim;
+
+  // What every wavefront reads again and again lives in LDS, not in registers (the loop
+  // below needs them all): the query operand, the 0/1 matrices, the rotation of one step.
+  __shared__ __attribute__((aligned(16))) uint4 sm_q[4][64];     // B operand per 32 dims, per lane
+  __shared__ __attribute__((aligned(16))) uint4 sm_pick[2][64];  // B operand per half, per lane
+  __shared__ __attribute__((aligned(16))) float2 sm_step[kHeadDim / 2];  // (cos, sin) of 16 tokens
+  __shared__ float sm_acc[4][G][kHeadDim];
+  __shared__ float sm_m[4][G], sm_l[4][G];
+  __shared__ uint32_t s_last;
+
+  // Column n of the logits: head slot n of this workgroup (zeros beyond its heads).  Wavefront
+  // kb2 < 2 prepares the dims [32 kb2, +32) and their partners 64 further on.
+  const bool real = n < G && part * G + n < a.group;
+  const int head = kvh * a.group + min(part * G + min(n, G - 1), a.group - 1);
+  // (No load of the start-up sits behind a branch: where a branch joins, the compiler waits
+  // for every load that either side may have issued.)
+  uint4 q_raw[2];
+  {
+    const uint16_t* qrow = a.q + ((size_t)b * H + head) * kHeadDim + 32 * (wave & 1) + 8 * qd;
+    q_raw[0] = *(const uint4*)qrow;
+    q_raw[1] = *(const uint4*)(qrow + 64);
+  }
+  // The first tile's slots are asked for together with the list's length, not after it.
+  // An entry past the wavefront's range (its token gets the weight zero) is replaced by the
+  // slot of the range's first token: its row must still be one that holds numbers.
+  const int wlo = split * chunk + wave * wlen;
+  auto raw_slot = [&](int j) { return (uint32_t)sel[min(j, a.max_sel_len - 1)]; };
+  uint32_t slot_cur[2] = {raw_slot(wlo + n), raw_slot(wlo + 16 + n)};
+  uint32_t slot_next[2] = {raw_slot(wlo + kAttnTile + n), raw_slot(wlo + kAttnTile + 16 + n)};
+  const int S = min(max(a.sel_len[b], 0), a.max_sel_len);
+  const int whi = min(S, wlo + wlen);
+  const uint32_t first_slot =
+      min((uint32_t)__builtin_amdgcn_readfirstlane((int)slot_cur[0]), a.pool_rows - 1);
+  auto checked = [&](uint32_t slot, int j) { return j < whi && slot < a.pool_rows ? slot : first_slot; };
+  slot_cur[0] = checked(slot_cur[0], wlo + n);
+  slot_cur[1] = checked(slot_cur[1], wlo + 16 + n);
+  slot_next[0] = checked(slot_next[0], wlo + kAttnTile + n);
+  slot_next[1] = checked(slot_next[1], wlo + kAttnTile + 16 + n);
+  // ... and the first tile's rows before the set-up below, which then runs while they travel.
+  uint4 kr[2][4], vr[2][4];
+  auto request = [&](const uint16_t* pool, const uint32_t* slots, uint4 (&dst)[2][4]) {
 #pragma unroll
-    for (int w = 0; w < 4; ++w) mm = fmaxf(mm, sm_m[w][g]);
-    float o0 = 0.f, o1 = 0.f, ll = 0.f;
+    for (int t = 0; t < 2; ++t) {
+      const uint16_t* row = pool + (size_t)slots[t] * row_elems + (size_t)kvh * kHeadDim + 8 * qd;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float sc = __expf(sm_m[w][g] - mm);
-      o0 += sm_acc[w][g][d] * sc;
-      o1 += sm_acc[w][g][d + 1] * sc;
-      ll += sm_l[w][g] * sc;
+      for (int kb = 0; kb < 4; ++kb) dst[t][kb] = *(const uint4*)(row + 32 * kb);
     }
-    if (!slot_active(g)) continue;
-    const size_t ph = ((size_t)b * H + head_of_slot(g)) * a.nsplit + split;
-    store_coherent2(a.part_acc + ph * kHeadDim + d, o0, o1);
-    if (d == 0) store_coherent2(a.part_ml + ph * 2, mm, ll);
-  }
+  };
+  // (a wavefront without tokens asks too: rows of some entry of the list, never used)
+  request(a.k_pool, slot_cur, kr);
+  request(a.v_pool, slot_cur, vr);
 
-  // Ticket: the stores above are acknowledged before the workgroup is counted.
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  uint32_t* ticket = a.tickets + (size_t)b * gridDim.y + blockIdx.y;
-  if (tid == 0) {
-    const uint32_t before =
-        __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_last = before + 1 == (uint32_t)a.nsplit ? 1u : 0u;
+  if (tid < kHeadDim / 2) {
+    float sn = 0.f, cs = 1.f;
+    if (ROPE) {
+      const float freq =
+          a.rope_rcp_scale * __builtin_amdgcn_exp2f(-(float)tid * (2.0f / kHeadDim) * a.log2_theta);
+      sincos_reduced(16.0f * freq, sn, cs);
+    }
+    sm_step[tid] = make_float2(cs, sn);
+    // 0/1 matrices that pick the dims [16 h, 16 h + 16) of a 32-dim block: B operand, lane
+    // (column n, qd) holds rows 8 qd .. 8 qd + 7, of which row 16 h + n is the one.
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint32_t w[4] = {0u, 0u, 0u, 0u};
+      if (qd == 2 * h + (n >> 3)) w[(n & 7) >> 1] = (n & 1) ? 0x3f800000u : 0x00003f80u;
+      sm_pick[h][lane] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
   }
-  __syncthreads();
-  if (!s_last) return;
-
-  // out[b,h,:] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s, rounded to bf16.
-  // A wavefront per head slot (a thread owns two adjacent dims, and a head has 64 such
-  // pairs): lane s fetches the (max, sum) of split s, the wave takes the maximum and
-  // lane s the weight of its split, so that the accumulators, all requested at once, are
-  // added up with weights that are ready (read lane by lane): no chain of dependent
-  // exponentials, and one statistics load per wave instead of one per split and thread.
-  static_assert(kHeadDim / 2 == 64, "one wavefront per head slot");
-  for (int idx = tid; idx < G * (kHeadDim / 2); idx += 256) {
-    const int g = idx / (kHeadDim / 2), d = (idx % (kHeadDim / 2)) * 2;
-    if (!slot_active(g)) continue;  // (uniform over the wave)
-    const size_t ph = ((size_t)b * H + head_of_slot(g)) * a.nsplit;
-    float mm = kNegBig, ll = 0.f, o0 = 0.f, o1 = 0.f;
-    for (int s0 = 0; s0 < a.nsplit; s0 += 32) {
-      // 32 splits at a time, branch-free: loads past the last split repeat it and get
-      // the weight zero.
-      float2 ac[32];
+  if (wave < 2) {  // the query rotated to position S - 1, rounded once
+    float x[8], y[8];
+    unpack8(real ? q_raw[0] : make_uint4(0u, 0u, 0u, 0u), x);
+    unpack8(real ? q_raw[1] : make_uint4(0u, 0u, 0u, 0u), y);
+    if (ROPE) {
 #pragma unroll
-      for (int i = 0; i < 32; ++i)
-        ac[i] = load_coherent2(a.part_acc + (ph + min(s0 + i, a.nsplit - 1)) * kHeadDim + d);
-      const float2 ml = (lane < 32 && s0 + lane < a.nsplit)
-                            ? load_coherent2(a.part_ml + (ph + s0 + lane) * 2)
-                            : make_float2(kNegBig, 0.f);
-      float mx = ml.x;
-      mx = fmaxf(mx, dpp_move<kRowRor8>(mx));
-      mx = fmaxf(mx, dpp_move<kRowRor4>(mx));
-      mx = fmaxf(mx, dpp_move<kRowRor2>(mx));
-      mx = fmaxf(mx, dpp_move<kRowRor1>(mx));
-      mx = fmaxf(mx, __shfl_xor(mx, 16));
-      const float mn = fmaxf(mm, __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(mx))));
-      const float keep = __expf(mm - mn);  // what earlier batches hold
-      const float w = (lane < 32 && s0 + lane < a.nsplit) ? __expf(ml.x - mn) : 0.f;
-      const float wl = ml.y * w;
-      o0 *= keep;
-      o1 *= keep;
-      ll *= keep;
-      mm = mn;
-#pragma unroll
-      for (int i = 0; i < 32; ++i) {
-        const float wi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), i));
-        ll += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wl), i));
-        o0 += ac[i].x * wi;
-        o1 += ac[i].y * wi;
+      for (int e = 0; e < 8; ++e) {
+        const int pair = 32 * wave + 8 * qd + e;
+        const float freq =
+            a.rope_rcp_scale * __builtin_amdgcn_exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
+        float sn, cs;
+        sincos_reduced((float)(S - 1) * freq, sn, cs);
+        const float xr = x[e] * cs - y[e] * sn;
+        y[e] = y[e] * cs + x[e] * sn;
+        x[e] = xr;
       }
     }
-    const uint32_t packed = (uint32_t)f32_to_bf16(ll > 0.f ? o0 / ll : 0.f) |
-                            ((uint32_t)f32_to_bf16(ll > 0.f ? o1 / ll : 0.f) << 16);
-    *(uint32_t*)(a.out + ((size_t)b * H + head_of_slot(g)) * kHeadDim + d) = packed;
+    sm_q[wave][lane] = __builtin_bit_cast(uint4, pack8(x));
+    sm_q[wave + 2][lane] = __builtin_bit_cast(uint4, pack8(y));
   }
-  if (tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // This lane's 16 rotation pairs: dims 32 kb2 + 8 qd + e (kb2 < 2, e < 8) and their partners
+  // 64 further on; key state at token wlo + n, 16 tokens per step.
+  float kc[16], ks[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    kc[i] = 1.f;
+    ks[i] = 0.f;
+    if (ROPE) {
+      const int pair = 32 * (i >> 3) + 8 * qd + (i & 7);
+      const float freq =
+          a.rope_rcp_scale * __builtin_amdgcn_exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
+      sincos_reduced((float)(wlo + n) * freq, ks[i], kc[i]);
+    }
+  }
+  __syncthreads();  // sm_q, sm_pick, sm_step
+
+  float m = kNegBig, l = 0.f;  // base-2 running maximum, this lane's share of the sum
+  at_f32x4 acc[8];             // O^T: dims 16 dt + 4 qd + r of head n
+#pragma unroll
+  for (int dt = 0; dt < 8; ++dt) acc[dt] = at_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (wlo < whi) {
+    const float scale2 = a.sm_scale * kAttnLog2e;
+
+    // One tile; `more` (a compile-time flag: the last tile is a copy of the loop's body
+    // without the requests) says that another tile follows.  Its loads are unconditional:
+    // behind a branch the compiler would wait for all loads where the branch joins, the ones
+    // just issued included.
+    auto tile = [&](const int j0, auto more_flag) __attribute__((always_inline)) {
+      constexpr bool more = decltype(more_flag)::value;
+      // The slots of the tile after the next are asked for before the next tile's rows, so
+      // that waiting for them does not mean waiting for those rows (loads return in order).
+      uint32_t slot_after[2] = {0u, 0u};
+      if (more) {
+        slot_after[0] = raw_slot(j0 + 2 * kAttnTile + n);
+        slot_after[1] = raw_slot(j0 + 2 * kAttnTile + 16 + n);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- keys, 16 tokens at a time: rotate, round, multiply, step the rotation
+      at_f32x4 s[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        at_bf16x8 ka[4];
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; ++kb2) {
+          float x[8], y[8];
+          unpack8(kr[t][kb2], x);
+          unpack8(kr[t][kb2 + 2], y);
+          if (ROPE) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float c = kc[8 * kb2 + e], sn = ks[8 * kb2 + e];
+              const float xr = x[e] * c - y[e] * sn;
+              y[e] = y[e] * c + x[e] * sn;
+              x[e] = xr;
+            }
+          }
+          ka[kb2] = pack8(x);
+          ka[kb2 + 2] = pack8(y);
+        }
+        const int zq = opaque_zero(__builtin_bit_cast(uint4, ka[3]).w);
+        s[t] = at_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+          s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              ka[kb], __builtin_bit_cast(at_bf16x8, sm_q[kb][lane + zq]), s[t], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ROPE) {  // the same rows of the next 16 tokens
+#pragma unroll
+          for (int kb2 = 0; kb2 < 2; ++kb2) {
+            const int zs = opaque_zero(__float_as_uint(kc[8 * kb2]));
+            const float4* step = (const float4*)&sm_step[32 * kb2 + 8 * qd + zs];
+#pragma unroll
+            for (int e2 = 0; e2 < 4; ++e2) {
+              const float4 d = step[e2];
+              const float dcs[2] = {d.x, d.z}, dsn[2] = {d.y, d.w};
+#pragma unroll
+              for (int o = 0; o < 2; ++o) {
+                const int i = 8 * kb2 + 2 * e2 + o;
+                const float c2 = kc[i] * dcs[o] - ks[i] * dsn[o];
+                ks[i] = ks[i] * dcs[o] + kc[i] * dsn[o];
+                kc[i] = c2;
+              }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      }
+      // the next tile's keys, into the registers just read
+      if (more) request(a.k_pool, slot_next, kr);
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- weights of 32 tokens x 16 head columns
+      float p[8];
+      float mx = kNegBig;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v;
+          if (CAP)
+            v = a.logit_cap * tanhf(s[t][r] * a.sm_scale / a.logit_cap) * kAttnLog2e;
+          else
+            v = s[t][r] * scale2;
+          v = j0 + 16 * t + 4 * qd + r < whi ? v : -INFINITY;
+          p[4 * t + r] = v;
+          mx = fmaxf(mx, v);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float mn = fmaxf(m, mx);
+      const float alpha = __builtin_amdgcn_exp2f(m - mn);
+      m = mn;
+      float sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        p[i] = __builtin_amdgcn_exp2f(p[i] - mn);
+        sum += p[i];
+      }
+      l = l * alpha + sum;
+#pragma unroll
+      for (int dt = 0; dt < 8; ++dt) acc[dt] *= alpha;
+      const at_bf16x8 pb = pack8(p);
+      // ---- values: transpose 16 dims at a time, accumulate
+      const int zp = opaque_zero(__builtin_bit_cast(uint4, pb).x);
+      at_bf16x8 pick[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) pick[h] = __builtin_bit_cast(at_bf16x8, sm_pick[h][lane + zp]);
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const at_f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+          const at_f32x4 d0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(at_bf16x8, vr[0][c]), pick[h], zero, 0, 0, 0);
+          const at_f32x4 d1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(at_bf16x8, vr[1][c]), pick[h], zero, 0, 0, 0);
+          const float vt[8] = {d0[0], d0[1], d0[2], d0[3], d1[0], d1[1], d1[2], d1[3]};
+          acc[2 * c + h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pack8(vt), pb, acc[2 * c + h], 0, 0, 0);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+      if (more) {
+        request(a.v_pool, slot_next, vr);
+        slot_next[0] = checked(slot_after[0], j0 + 2 * kAttnTile + n);
+        slot_next[1] = checked(slot_after[1], j0 + 2 * kAttnTile + 16 + n);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // (Lowering a wavefront's priority as it advances, which evens out the two workgroups of
+    // a CU in the kernel above, evens them out here too and gains nothing: the rows arrive
+    // as fast as the memory system delivers them either way.)
+    int j0 = wlo;
+    for (; j0 + kAttnTile < whi; j0 += kAttnTile) tile(j0, std::true_type{});
+    tile(j0, std::false_type{});
+  }
+
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+  if (n < G) {
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt)
+      *(float4*)&sm_acc[wave][n][16 * dt + 4 * qd] = make_float4(acc[dt][0], acc[dt][1], acc[dt][2], acc[dt][3]);
+    if (qd == 0) {
+      sm_m[wave][n] = m * kAttnLn2;  // natural-log units, as the merge expects
+      sm_l[wave][n] = l;
+    }
+  }
+  attn_finish<G>(a, b, kvh, part, split, sm_acc, sm_m, sm_l, &s_last);
 }
 
 __global__ __launch_bounds__(256) void attn_zero_kernel(uint32_t* tickets, int count) {
@@ -411,7 +763,11 @@ int attn_tickets_per_request(const ts_config* cfg) {
   return cfg->num_kv_heads * attn_parts(cfg->num_heads / cfg->num_kv_heads);
 }
 
-static int attn_splits(int batch, int num_kv_heads, int max_sel_len) {
+struct AttnPlan {
+  int nsplit;  // workgroups per (request, KV head, part)
+  bool mfma;   // the matrix-core kernel: a workgroup walks more than one batch of loads
+};
+static AttnPlan attn_plan(int batch, int num_kv_heads, int max_sel_len) {
   // One batch of loads per lane group (16 groups x 8 tokens = 128 tokens per
   // workgroup) as long as the grid stays within the 512 workgroups that are
   // resident at once (two per CU): a second round of workgroups pays the start-up
@@ -420,7 +776,16 @@ static int attn_splits(int batch, int num_kv_heads, int max_sel_len) {
   const int64_t cap = ceil_div(512, (int64_t)batch * num_kv_heads);
   if (want > cap) want = cap;
   if (want < 1) want = 1;
-  return (int)want;
+  AttnPlan plan;
+  plan.nsplit = (int)want;
+  plan.mfma = ceil_div(max_sel_len, want) > 16 * kAttnInFlight;
+  // (ranges of the matrix-core kernel are whole multiples of 64 tokens: the last splits
+  // may have nothing left)
+  if (plan.mfma) plan.nsplit = (int)ceil_div(max_sel_len, attn_mfma_chunk(max_sel_len, plan.nsplit));
+  return plan;
+}
+static int attn_splits(int batch, int num_kv_heads, int max_sel_len) {
+  return attn_plan(batch, num_kv_heads, max_sel_len).nsplit;
 }
 
 struct AttnWorkspace {
@@ -463,7 +828,8 @@ int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const v
   a.rope_rcp_scale = cfg->rope_mode == TS_ROPE_LLAMA ? 1.0f / cfg->rope_scale : 1.0f;
   a.sm_scale = cfg->sm_scale;
   a.logit_cap = cfg->logit_cap;
-  a.nsplit = attn_splits(batch, attn_tickets_per_request(cfg), max_sel_len);
+  const AttnPlan plan = attn_plan(batch, attn_tickets_per_request(cfg), max_sel_len);
+  a.nsplit = plan.nsplit;
   a.max_sel_len = max_sel_len;
   a.part_acc = (float*)((char*)workspace + w.acc);
   a.part_ml = (float*)((char*)workspace + w.ml);
@@ -479,8 +845,13 @@ int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const v
   const dim3 grid((unsigned)a.nsplit, (unsigned)attn_tickets_per_request(cfg), (unsigned)batch);
   const int group = attn_heads_per_part(a.group);
   const bool rope = cfg->rope_mode == TS_ROPE_LLAMA, cap = cfg->logit_cap > 0.f;
-#define TS_ATTN_LAUNCH(G_, R_, C_) \
-  hipLaunchKernelGGL((attn_kernel<G_, R_, C_>), grid, dim3(256), 0, st, a)
+#define TS_ATTN_LAUNCH(G_, R_, C_)                                                      \
+  do {                                                                                 \
+    if (plan.mfma)                                                                     \
+      hipLaunchKernelGGL((attn_mfma_kernel<G_, R_, C_>), grid, dim3(256), 0, st, a);   \
+    else                                                                               \
+      hipLaunchKernelGGL((attn_kernel<G_, R_, C_>), grid, dim3(256), 0, st, a);        \
+  } while (0)
 #define TS_ATTN_CASE(G_)                           \
   case G_:                                         \
     if (rope && cap) TS_ATTN_LAUNCH(G_, true, true);        \
@@ -541,6 +912,11 @@ extern "C" {
 size_t ts_attn_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_sel_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_sel_len < 1) return 0;
   return attn_workspace(cfg, batch, max_sel_len).total;
+}
+
+int ts_attn_kernel_form(const ts_config* cfg, int32_t batch, int32_t max_sel_len) {
+  if (validate_config(cfg) != TS_OK || batch < 1 || max_sel_len < 1) return -1;
+  return attn_plan(batch, attn_tickets_per_request(cfg), max_sel_len).mfma ? 1 : 0;
 }
 
 int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_pool,

@@ -126,6 +126,14 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
   return (uint16_t)(u >> 16);
 }
 
+// Two floats to packed bf16, round to nearest even, in one v_cvt_pk_bf16_f32.
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float x) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));

@@ -195,14 +195,6 @@ constexpr float kPfRaise = 8.0f;       // a row's maximum is raised when a logit
 // and the next one wants those 8 as one 16-byte operand, in the order 4 kb + r.
 __device__ __forceinline__ int kv_pos(int kk) { return 8 * ((kk >> 2) & 3) + 4 * (kk >> 4) + (kk & 3); }
 
-// Two floats to packed bf16, round to nearest even, in one v_cvt_pk_bf16_f32.
-typedef __attribute__((ext_vector_type(2))) __bf16 pf_bf16x2;
-typedef __attribute__((ext_vector_type(2))) float pf_f32x2;
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  const pf_f32x2 v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, pf_bf16x2));
-}
-
 // Grid (32-key tiles, KV heads).  Thread (key kk, chunk c) moves dims [8c, 8c+8) and
 // [64+8c, +8) of key j = tile + kk.  Keys past S are written as zeros.
 __global__ __launch_bounds__(256) void prefill_gather_kernel(PrefillArgs a) {
