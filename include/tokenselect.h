@@ -129,6 +129,18 @@ typedef struct ts_batch {
                                workgroups counted as members of every rendezvous
                                that never arrive, so that every wait gives up
                                after wait_us while all kernels still exit        */
+  int32_t workspace_clean;  /* ts_decode_layer only.  1: the caller states that this
+                               workspace was last used by a ts_decode_layer call with
+                               the same cfg, batch, max_seq_len and cache == NULL that
+                               completed without a give-up, and by nothing since (every
+                               such call leaves the selection's counters zero again:
+                               its attention kernel clears them on the side).  The
+                               layer then starts with the selection kernel, which
+                               rotates the query itself (bit-identical to ts_rope_apply);
+                               the launch that rotates and clears is not needed.  Honoured
+                               where the selection is the single ts_select launch and no
+                               selection cache is used; ignored otherwise.  A wrong
+                               statement gives wrong selections or waits that give up */
 } ts_batch;
 
 /* Default bound of a grid-wide wait: a selection that has the device to itself

@@ -46,7 +46,8 @@ def test_header_symbols_are_exported_and_bound(lib):
 
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.TsConfig) == 14 * 4
-    assert ctypes.sizeof(_lib.TsBatch) == 8 + 8 + 8 + 8 + 8 + 8 + 8 + 8 + 4 * 4
+    assert ctypes.sizeof(_lib.TsBatch) == 8 + 8 + 8 + 8 + 8 + 8 + 8 + 8 + 4 * 4 + 8  # 5 ints, padded
+    assert _lib.TsBatch.workspace_clean.offset == 80
     assert _lib.TsBatch.threshold_hint.offset == 56
     assert _lib.TsBatch.separate_kernels.offset == 64 and _lib.TsBatch.rerun.offset == 68
     assert _lib.TsBatch.wait_us.offset == 72 and _lib.TsBatch.absent_workgroups.offset == 76

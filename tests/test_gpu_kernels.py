@@ -830,6 +830,50 @@ def fused_select(request):
     ops.set_fused_select(previous)
 
 
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("lens", [[3000], [2500, 700, 3000]], ids=["B1", "B3"])
+def test_layer_starts_with_the_selection_on_a_clean_workspace(dev, shape, lens):
+    """From its second call of a shape on, a layer object without a selection cache tells the
+    library that its workspace is clean (the attention kernel of the call before cleared the
+    selection's counters) and the call starts with the selection kernel, which rotates the
+    query itself: selections and outputs bit-identical to those of a fresh object, whose first
+    call runs the rotation kernel, step after step with new queries; a call of another shape,
+    with a selection cache or split at the vote in between makes the next call a full one."""
+    say(f"layer on a clean workspace H={shape['num_heads']} kv={shape['num_kv_heads']} B={len(lens)}")
+    wl = small(dev, shape, seed=71, lens=lens, ks=[64] * len(lens))
+    c, B = wl.cfg, len(lens)
+    layer = ops.DecodeLayer(c, B, max(lens), dev)
+    layer.workspace.fill_(0xa5)          # whatever an allocation holds
+    gen = torch.Generator(device=dev).manual_seed(72)
+    cache = ops.SelectionCache.allocate(c, B, dev)
+    for step in range(6):
+        q = torch.randn(wl.q.shape, device=dev, generator=gen).to(wl.q.dtype)
+        was_clean = layer._clean_for
+        if step == 3:      # a call with the selection cache: the call after it is a full one
+            layer(q, wl.k_pool, wl.v_pool, wl.batch, cache=cache)
+            assert layer._clean_for is None
+            continue
+        if step == 5:      # another shape (one request fewer tokens than the object was sized for)
+            import dataclasses
+            bt = dataclasses.replace(wl.batch, max_seq_len=max(lens) - 1)
+            layer(q, wl.k_pool, wl.v_pool, bt)
+            assert layer._clean_for == (B, max(lens) - 1)
+            continue
+        got = [t.clone() for t in layer(q, wl.k_pool, wl.v_pool, wl.batch)]
+        assert layer._clean_for == (B, max(lens))
+        assert (was_clean == (B, max(lens))) == (step in (1, 2)), f"step {step}: {was_clean}"
+        fresh = ops.DecodeLayer(c, B, max(lens), dev)
+        want = fresh(q, wl.k_pool, wl.v_pool, wl.batch)
+        torch.cuda.synchronize()
+        assert not layer.gave_up() and not fresh.gave_up()
+        assert torch.equal(got[3], want[3]), f"step {step}: lengths"
+        for b in range(B):
+            S = int(want[3][b])
+            assert torch.equal(got[1][b, :S], want[1][b, :S]) and torch.equal(got[2][b, :S], want[2][b, :S]), \
+                f"step {step} b={b}: selection"
+        assert torch.equal(got[0].view(torch.int16), want[0].view(torch.int16)), f"step {step}: output"
+
+
 def check_layer(wl, dev, tag):
     lens = wl.seq_lens
     layer = ops.DecodeLayer(wl.cfg, len(lens), max(lens), dev)

@@ -37,7 +37,7 @@ class TsBatch(ctypes.Structure):
         ("batch", _i32), ("max_seq_len", _i32), ("seq_lens", _ptr), ("table", _ptr),
         ("table_stride", _i64), ("k_per_req", _ptr), ("fault", _ptr), ("host_seq_lens", _ptr),
         ("threshold_hint", _ptr), ("separate_kernels", _i32), ("rerun", _i32), ("wait_us", ctypes.c_uint32),
-        ("absent_workgroups", _i32),
+        ("absent_workgroups", _i32), ("workspace_clean", _i32),
     ]
 
 

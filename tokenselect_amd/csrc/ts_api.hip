@@ -251,7 +251,14 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
     zero.add(topk_zero_region(topk, bt->batch));
     if (vote_group > 0) score_votes_zero_regions(cfg, bt, fused, ws + w.select_ws, &zero);
   }
-  if (chunk_rows > 0) {
+  // A decode step without a selection cache whose single-launch selection finds its
+  // counters zero (the caller says so: the attention kernel of its previous call, of the
+  // same shape, cleared them on the side) starts with the selection kernel, which rotates
+  // the query itself; this call's attention kernel clears the counters again.
+  const bool plain_decode = one_launch && chunk_rows == 0 && !cache;
+  const bool starts_with_selection = plain_decode && bt->workspace_clean != 0;
+  if (starts_with_selection) {
+  } else if (chunk_rows > 0) {
     // Chunk fingerprint: row i rotated to n_local + i, mean over the rows (tr.py:380-392).
     TS_TRY(launch_fingerprint(cfg, q, chunk_rows, q_cos, q_sin, table_rows, qf, zero,
                               (hipStream_t)stream));
@@ -264,11 +271,13 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
   }
   if (cache && chunk_rows > 0)
     TS_TRY(launch_selcache(cfg, bt, qf, cache, hit, bt->rerun ? sel_len : nullptr, (hipStream_t)stream));
+  const UnrotatedQuery unrotated{q, q_cos, q_sin};
   if (one_launch) {
     TS_TRY(launch_select(cfg, bt, qf, k_pool, pool_rows, hit, cache, sel, sel_pos, sel_stride, sel_len,
                          nullptr, 0, ws + w.select_ws, tickets, attn_tickets_per_request(cfg),
                          (hipStream_t)stream, select_wait_ticks(bt),
-                         (uint32_t)(bt->absent_workgroups > 0 ? bt->absent_workgroups : 0)));
+                         (uint32_t)(bt->absent_workgroups > 0 ? bt->absent_workgroups : 0),
+                         starts_with_selection ? &unrotated : nullptr));
   } else if (vote_group > 0) {
     // With max-pooling the kernel writes the pooled votes (there is no un-pooled copy).
     TS_TRY(launch_score_votes(cfg, bt, qf, k_pool, pool_rows, hit, votes, w.score_stride, topk.ws,
@@ -293,7 +302,8 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
     return ts_sparse_prefill_attn(cfg, q, chunk_rows, k_pool, v_pool, pool_rows, sel, sel_len,
                                   w.max_sel, out, ws + w.attn_ws, w.total - w.attn_ws, stream);
   return launch_attn(cfg, q, k_pool, v_pool, pool_rows, sel, sel_stride, sel_len, bt->batch,
-                     w.max_sel, out, ws + w.attn_ws, /*tickets_clear=*/true, (hipStream_t)stream);
+                     w.max_sel, out, ws + w.attn_ws, /*tickets_clear=*/true, (hipStream_t)stream,
+                     plain_decode ? &zero : nullptr);
 }
 
 int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, const float* q_cos,

@@ -42,7 +42,15 @@ struct AttnArgs {
   float* part_ml;     // [B,H,nsplit,2]
   uint32_t* tickets;  // [B,Hkv*parts], zero at launch and again when the kernel ends
   uint16_t* out;      // [B,H,128] bf16
+  ZeroSet zero;       // cleared on the side (counters of the stream's next selection)
 };
+
+// A workgroup's share of the regions to clear, at the start of an attention kernel.
+__device__ __forceinline__ void attn_clear_on_the_side(const AttnArgs& a) {
+  if (a.zero.used == 0) return;
+  const int64_t wg = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+  clear_regions(a.zero, wg * 256 + threadIdx.x, (int64_t)gridDim.x * gridDim.y * gridDim.z * 256);
+}
 
 __device__ __forceinline__ void unpack4(const uint2& w, float* f) {
   f[0] = bf16_lo(w.x);
@@ -179,6 +187,7 @@ constexpr int kAttnInFlight = 8;  // tokens per lane group requested together
 // KV heads, 32K context: 20.6 us against the 14 us of 32 heads on 8).
 template <int G, bool ROPE, bool CAP>
 __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
+  attn_clear_on_the_side(a);
   const int split = blockIdx.x, b = blockIdx.z;
   const int kvh = blockIdx.y / a.parts, part = blockIdx.y % a.parts;
   // Head g of this workgroup: the last part of a group of five or seven has one head too
@@ -483,6 +492,7 @@ __device__ __forceinline__ int opaque_zero(uint32_t after) {
 template <int G, bool ROPE, bool CAP>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_kernel(
     AttnArgs a) {
+  attn_clear_on_the_side(a);
   const int split = blockIdx.x, b = blockIdx.z;
   const int kvh = blockIdx.y / a.parts, part = blockIdx.y % a.parts;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -809,9 +819,14 @@ uint32_t* attn_tickets(const ts_config* cfg, int batch, int max_sel_len, void* w
 int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const void* v_pool,
                 int64_t pool_rows, const int32_t* sel, int64_t sel_stride, const int32_t* sel_len,
                 int batch, int max_sel_len, void* out, void* workspace, bool tickets_clear,
-                hipStream_t st) {
+                hipStream_t st, const ZeroSet* clear_after) {
   const AttnWorkspace w = attn_workspace(cfg, batch, max_sel_len);
   AttnArgs a;
+  if (clear_after) {
+    TS_REQUIRE(!clear_after->overflow, TS_EINVAL, "internal: more than %d regions to clear in one launch",
+               kZeroRegions);
+    a.zero = *clear_after;
+  }
   a.q = (const uint16_t*)q;
   a.k_pool = (const uint16_t*)k_pool;
   a.v_pool = (const uint16_t*)v_pool;

@@ -105,10 +105,12 @@ int launch_rope_selcache(const ts_config* cfg, const ts_batch* bt, const void* q
 uint32_t* attn_tickets(const ts_config* cfg, int batch, int max_sel_len, void* workspace);
 // Tickets per request (the words to clear): one per workgroup row of the attention's grid.
 int attn_tickets_per_request(const ts_config* cfg);
+// clear_after: regions that the kernel clears on the side (the counters of the stream's
+// next selection), or NULL.
 int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const void* v_pool,
                 int64_t pool_rows, const int32_t* sel, int64_t sel_stride, const int32_t* sel_len,
                 int batch, int max_sel_len, void* out, void* workspace, bool tickets_clear,
-                hipStream_t stream);
+                hipStream_t stream, const ZeroSet* clear_after = nullptr);
 
 constexpr int kHeadDim = 128;
 constexpr float kNegBig = -3.0e38f;  // finite stand-in for -inf in running maxima
@@ -158,6 +160,17 @@ __device__ __forceinline__ void sincos_reduced(float x, float& sn, float& cs) {
   r = fmaf(-k, -1.7484555e-07f, r);
   sn = __sinf(r);
   cs = __cosf(r);
+}
+
+// One element of the scoring query's rotation (RotaryEmbedding.apply_rotary_pos_emb,
+// tr.py:98-107): own * cos + (+-other) * sin, where `other` is the element 64 dims away and
+// enters negated for the lower half.  Products and the sum are rounded one by one (no FMA
+// contraction), which is what the reference's elementwise torch expression does.
+__device__ __forceinline__ float rotate_element(float own, float other, float cs, float sn, bool lower) {
+#pragma clang fp contract(off)
+  const float a = own * cs;
+  const float b = (lower ? -other : other) * sn;
+  return a + b;
 }
 
 // Merge two (max, sum-of-exp) softmax partials.

@@ -34,8 +34,8 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(const uint16_t* __restr
   const int64_t base = rh * dim;
   const float x1 = bf16_to_f32(x[base + i]);
   const float x2 = bf16_to_f32(x[base + i + half]);
-  const float lo = x1 * c[i] + (-x2) * s[i];
-  const float hi = x2 * c[i + half] + x1 * s[i + half];
+  const float lo = rotate_element(x1, x2, c[i], s[i], true);
+  const float hi = rotate_element(x2, x1, c[i + half], s[i + half], false);
   out[base + i] = f32_to_bf16(lo);
   out[base + i + half] = f32_to_bf16(hi);
 }

@@ -20,6 +20,12 @@ struct VotePhase {
 
 struct ScoreArgs {
   const uint16_t* qf;      // [B,H,128] bf16 rotated fingerprints
+  // Single-launch selection only: when q_raw is set, qf is not read; the kernel rotates
+  // q_raw [B,H,128] (un-rotated bf16) itself with the [128] rows q_cos / q_sin, bit-identical
+  // to what the rotation kernel would have written to qf.
+  const uint16_t* q_raw;
+  const float* q_cos;
+  const float* q_sin;
   const uint16_t* k_pool;  // [pool_rows,Hkv,128] bf16
   uint32_t pool_rows;
   const int32_t* seq_lens;
@@ -194,10 +200,17 @@ const uint32_t* score_votes_fault_word(const ts_config* cfg, int batch, int max_
                                        const void* workspace);
 
 // Launch without the clearing pass: the regions above are known to be zero.
+// A query that the selection kernel rotates itself (see ScoreArgs::q_raw).
+struct UnrotatedQuery {
+  const void* q;
+  const float* cos;
+  const float* sin;
+};
 int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, const void* k_pool,
                   int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
                   int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
                   int64_t vote_stride, void* workspace, uint32_t* clear, int clear_per_req,
-                  hipStream_t stream, uint64_t wait_ticks, uint32_t absent);
+                  hipStream_t stream, uint64_t wait_ticks, uint32_t absent,
+                  const UnrotatedQuery* unrotated = nullptr);
 
 }  // namespace ts

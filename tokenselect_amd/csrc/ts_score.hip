@@ -571,7 +571,32 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     for (int na = 0; na < NA; ++na) {
       const int g = 4 * na + t4;
       const int h = head_of<HKV, G>(kvh, g < G ? g : 0, a.head_map);
-      uint4 v = *(const uint4*)((const char*)(a.qf + ((size_t)b * H + h) * kHeadDim) + lane_off);
+      uint4 v;
+      if (FUSED && !PACKED && a.q_raw != nullptr) {
+        // The caller's un-rotated query: this lane's 8 dims and the 8 dims 64 further on (or
+        // back), rotated as the rotation kernel does it.
+        const bool lower = rg < 2;
+        const uint32_t other_off = lower ? lane_off + 128u : lane_off - 128u;
+        const char* qrow = (const char*)(a.q_raw + ((size_t)b * H + h) * kHeadDim);
+        const uint4 own = *(const uint4*)(qrow + lane_off), other = *(const uint4*)(qrow + other_off);
+        const float4 c0 = *(const float4*)((const char*)a.q_cos + 2 * lane_off);
+        const float4 c1 = *(const float4*)((const char*)a.q_cos + 2 * lane_off + 16);
+        const float4 s0 = *(const float4*)((const char*)a.q_sin + 2 * lane_off);
+        const float4 s1 = *(const float4*)((const char*)a.q_sin + 2 * lane_off + 16);
+        const uint32_t ow[4] = {own.x, own.y, own.z, own.w}, th[4] = {other.x, other.y, other.z, other.w};
+        const float cs[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+        const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        uint32_t r[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float lo = rotate_element(bf16_lo(ow[e]), bf16_lo(th[e]), cs[2 * e], sn[2 * e], lower);
+          const float hi = rotate_element(bf16_hi(ow[e]), bf16_hi(th[e]), cs[2 * e + 1], sn[2 * e + 1], lower);
+          r[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+        }
+        v = make_uint4(r[0], r[1], r[2], r[3]);
+      } else {
+        v = *(const uint4*)((const char*)(a.qf + ((size_t)b * H + h) * kHeadDim) + lane_off);
+      }
       if (g >= G) v = make_uint4(0u, 0u, 0u, 0u);
       qa[kvh][na] = __builtin_bit_cast(bf16x8_t, v);
     }
@@ -1762,7 +1787,8 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
                   int64_t pool_rows, const int32_t* hit, const ts_selcache* cache, int32_t* sel,
                   int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, float* votes,
                   int64_t vote_stride, void* workspace, uint32_t* clear, int clear_per_req,
-                  hipStream_t stream, uint64_t wait_ticks, uint32_t absent) {
+                  hipStream_t stream, uint64_t wait_ticks, uint32_t absent,
+                  const UnrotatedQuery* unrotated) {
   // (requests may be skipped when the caller brings hit flags: the selection cache)
   const SelectWorkspace w = select_workspace(cfg, bt->batch, bt->max_seq_len, false, hit != nullptr);
   TS_REQUIRE(w.tokens_per_block > 0, TS_ESHAPE, "fused selection: unsupported shape");
@@ -1770,6 +1796,11 @@ int launch_select(const ts_config* cfg, const ts_batch* bt, const void* qf, cons
   ScoreArgs a = selection_args(cfg, bt, qf, k_pool, pool_rows, hit, (float*)(ws + w.partials),
                                w.tokens_per_block);
   a.nchunks = kSelMaxChunks;  // the row of a (request, head) pair in the statistics' table
+  if (unrotated) {
+    a.q_raw = (const uint16_t*)unrotated->q;
+    a.q_cos = unrotated->cos;
+    a.q_sin = unrotated->sin;
+  }
   a.sync = (uint32_t*)(ws + w.sync);
   a.stats = (float*)(ws + w.stats);
   a.stats_stride = w.stats_stride;

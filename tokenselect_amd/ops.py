@@ -81,6 +81,9 @@ class Batch:
     rerun: bool = False
     wait_us: int = 0
     absent_workgroups: int = 0
+    # ``ts_batch.workspace_clean``: the workspace was left by a completed call of the same
+    # shape without a selection cache (set by :class:`DecodeLayer`, which knows).
+    workspace_clean: bool = False
 
     @property
     def batch(self) -> int:
@@ -236,7 +239,7 @@ def _c_batch(cfg: LayerConfig, bt: Batch) -> TsBatch:
     return TsBatch(bt.batch, int(bt.max_seq_len), _p(bt.seq_lens), _p(bt.table),
                    int(bt.table.stride(0)), _p(bt.k_per_req), _p(bt.fault), host, _p(bt.hint),
                    1 if bt.separate_kernels else 0, 1 if bt.rerun else 0, int(bt.wait_us),
-                   int(bt.absent_workgroups))
+                   int(bt.absent_workgroups), 1 if bt.workspace_clean else 0)
 
 
 def _c_cache(cache: Optional[SelectionCache], cfg: LayerConfig, batch: int):
@@ -734,6 +737,11 @@ class DecodeLayer(_GiveUpLatch):
         self.sel_pos = torch.empty_like(self.sel)
         self.sel_len = torch.empty((batch,), dtype=torch.int32, device=device)
         self._init_latch()
+        # (batch, max_seq_len) of the last call when it was a plain layer call without a
+        # selection cache that raised nothing: that call's attention kernel has left the
+        # selection's counters zero, and the next call of the same shape says so
+        # (``ts_batch.workspace_clean``) and starts with the selection kernel.
+        self._clean_for = None
 
     def recover(self, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch,
                 cache: Optional[SelectionCache] = None, out: Optional[torch.Tensor] = None):
@@ -756,6 +764,11 @@ class DecodeLayer(_GiveUpLatch):
     def _run(self, q, k_pool, v_pool, bt, cache, out, rerun: bool = False):
         cfg = self.cfg
         bt = self._options(bt, rerun)
+        shape = (bt.batch, int(bt.max_seq_len))
+        plain = cache is None and not bt.separate_kernels and not rerun
+        if plain and self._clean_for == shape and not bt.workspace_clean:
+            bt = dataclasses.replace(bt, workspace_clean=True)
+        self._clean_for = None
         cb = _c_batch(cfg, bt)
         if bt.batch > self.batch or bt.max_seq_len > self.max_seq_len:
             raise ValueError("batch / max_seq_len exceed what this DecodeLayer was sized for")
@@ -778,6 +791,8 @@ class DecodeLayer(_GiveUpLatch):
             _p(k_pool), _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, B), _p(out),
             _p(self.sel), _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
             self.workspace.numel(), _stream()))
+        if plain:
+            self._clean_for = shape
         return out, self.sel[:B], self.sel_pos[:B], self.sel_len[:B]
 
     # The layer split at the vote (tensor parallelism, tr.py:361-364): votes() leaves this
@@ -787,6 +802,7 @@ class DecodeLayer(_GiveUpLatch):
               cache: Optional[SelectionCache] = None) -> torch.Tensor:
         cfg = self.cfg
         self.check()
+        self._clean_for = None  # (other kernels use the workspace from here on)
         bt = self._options(bt)
         cb = _c_batch(cfg, bt)
         if bt.batch > self.batch or bt.max_seq_len > self.max_seq_len:
@@ -808,6 +824,7 @@ class DecodeLayer(_GiveUpLatch):
     def attend(self, q: torch.Tensor, votes: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                bt: Batch, cache: Optional[SelectionCache] = None, out: Optional[torch.Tensor] = None):
         cfg = self.cfg
+        self._clean_for = None
         bt = self._options(bt)
         cb = _c_batch(cfg, bt)
         _need(q, "q", torch.bfloat16)
