@@ -687,6 +687,44 @@ def test_sparse_attention(dev, shape, rope_mode):
         assert err <= 2e-2, f"attention b={b}: max abs err {err}"
 
 
+@pytest.mark.parametrize("B", [1, 14], ids=["vector", "matrix"])
+def test_attention_never_reads_a_row_it_was_not_given(dev, B):
+    """A KV pool as a server holds it: only the rows in use hold numbers.  Every row that no
+    list names is filled with NaN, and the entries of `sel` past the lengths point at such rows
+    (or outside the pool): a token past a range has the weight zero, but 0 x NaN is NaN, so the
+    kernels must not fetch those rows at all.  Both kernels (one request: vector; 14: matrix)."""
+    lens = [2541] if B == 1 else [2600, 2599, 2541, 1025, 700, 333, 65, 64, 33, 17, 1, 0, 2600, 1800]
+    width = 2600
+    say(f"attention over a pool with NaN in every unused row B={B}")
+    wl = small(dev, SHAPES[0], seed=43, lens=[3000] * B, ks=[64] * B)
+    c = wl.cfg
+    assert ops.attention_kernel_form(c, B, width) == (0 if B == 1 else 1)
+    P = wl.k_pool.shape[0]
+    g = torch.Generator().manual_seed(44)
+    used = torch.zeros(P, dtype=torch.bool)
+    sel = torch.zeros((B, width), dtype=torch.int32)
+    for b, S in enumerate(lens):
+        rows = torch.randint(0, P - 1, (S,), generator=g)     # (the pool's last row stays unused)
+        used[rows] = True
+        sel[b, :S] = rows.int()
+        sel[b, S:] = torch.where(torch.arange(width - S) % 2 == 0, 0x7fffffff, P - 1).int()
+    k_pool, v_pool = wl.k_pool.clone(), wl.v_pool.clone()
+    k_pool[~used.to(dev)] = float("nan")
+    v_pool[~used.to(dev)] = float("nan")
+    sel_len = torch.tensor(lens, dtype=torch.int32)
+    out = ops.sparse_decode_attention(c, wl.q, k_pool, v_pool, sel.to(dev), sel_len.to(dev))
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out.float()).all()), "NaN from a row that no list names"
+    kc, vc, qc = wl.k_pool.cpu(), wl.v_pool.cpu(), wl.q.cpu()
+    for b, S in enumerate(lens):
+        if S == 0:
+            assert not bool(out[b].any())
+            continue
+        ref = oracle.attend.sparse_decode_attention(
+            qc[b].view(c.num_heads, 128), kc, vc, sel[b, :S], 128 ** -0.5, c.rope_theta, 1.0, 0.0, c.rope_mode)
+        assert (out[b].cpu().float() - ref.reshape(-1).float()).abs().max().item() <= 2e-2
+
+
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
 @pytest.mark.parametrize("rope_mode,cap", [("ROPE_LLAMA", 0.0), ("NONE", 0.0), ("ROPE_LLAMA", 25.0)])
 def test_sparse_attention_on_the_matrix_cores(dev, shape, rope_mode, cap):

@@ -219,8 +219,12 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
       slot[u] = (uint32_t)sel[min(j0 + 16 * u, a.max_sel_len - 1)];
   };
   load_slots(lo + lg);
+  // The slot of the range's first entry stands in for entries past the range: their tokens
+  // get the weight zero, and 0 x whatever an unused or stale entry points at need not be 0.
+  uint32_t first_slot = (uint32_t)sel[min(lo, a.max_sel_len - 1)];
   const int S = min(max(a.sel_len[b], 0), a.max_sel_len);
   const int hi = min(S, lo + chunk);
+  first_slot = first_slot < a.pool_rows ? first_slot : a.pool_rows - 1;
 
   // Frequencies of this lane's 4 rotation pairs: theta^(-2 pair / 128) / scale.
   float freq[4];
@@ -301,8 +305,8 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
     uint2 klo[kAttnInFlight], khi[kAttnInFlight], vlo[kAttnInFlight], vhi[kAttnInFlight];
 #pragma unroll
     for (int u = 0; u < kAttnInFlight; ++u) {
-      const uint32_t sl = slot[u] < a.pool_rows ? slot[u] : a.pool_rows - 1;
-      const size_t at = (size_t)sl * row_elems + (size_t)kvh * kHeadDim + l16 * 4;
+      slot[u] = (j0 + 16 * u < hi && slot[u] < a.pool_rows) ? slot[u] : first_slot;
+      const size_t at = (size_t)slot[u] * row_elems + (size_t)kvh * kHeadDim + l16 * 4;
       klo[u] = *(const uint2*)(a.k_pool + at);
       khi[u] = *(const uint2*)(a.k_pool + at + 64);
     }
@@ -310,8 +314,7 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
     // the values arrive while they are being computed.
 #pragma unroll
     for (int u = 0; u < kAttnInFlight; ++u) {
-      const uint32_t sl = slot[u] < a.pool_rows ? slot[u] : a.pool_rows - 1;
-      const size_t at = (size_t)sl * row_elems + (size_t)kvh * kHeadDim + l16 * 4;
+      const size_t at = (size_t)slot[u] * row_elems + (size_t)kvh * kHeadDim + l16 * 4;
       vlo[u] = *(const uint2*)(a.v_pool + at);
       vhi[u] = *(const uint2*)(a.v_pool + at + 64);
     }
