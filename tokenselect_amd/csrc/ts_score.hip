@@ -500,6 +500,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
   int req_chunks = (int)gridDim.x;  // chunks of this workgroup's request (the single launch: dealt)
   GridTeam team{0u, 0u};
   if (PACKED) {
+    TS_MARK(0);
     // This workgroup's phase, and its request and chunk within the phase.
     int phase = 0;
     while (phase + 1 < a.nphases && (int)blockIdx.x >= a.phases[phase + 1].first_workgroup) ++phase;
