@@ -214,3 +214,29 @@ def test_workspace_sizes_never_shrink_with_the_context_or_the_batch(lib):
             assert sizes == sorted(sizes), fn.__name__
         by_batch = [lib.ts_decode_layer_workspace_bytes(ctypes.byref(c), B, 65536) for B in range(1, 33)]
         assert by_batch == sorted(by_batch)
+
+
+def test_header_is_plain_c_and_agrees_with_the_ctypes_mirror(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 (no C++ in it), and a C program
+    sees the struct sizes and field offsets that the ctypes mirror and the library use."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "layout.c"
+    src.write_text(
+        '#include <stddef.h>\n#include <stdio.h>\n#include "tokenselect.h"\n'
+        'int main(void) {\n'
+        '  printf("%zu %zu %zu %zu %zu %zu %zu\\n", sizeof(ts_config), sizeof(ts_batch), sizeof(ts_selcache),\n'
+        '         offsetof(ts_batch, threshold_hint), offsetof(ts_batch, wait_us),\n'
+        '         offsetof(ts_batch, workspace_clean), offsetof(ts_batch, host_seq_lens));\n'
+        '  return 0;\n}\n')
+    exe = tmp_path / "layout"
+    include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", include, str(src),
+                    "-o", str(exe)], check=True)
+    got = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
+    assert got == [ctypes.sizeof(_lib.TsConfig), ctypes.sizeof(_lib.TsBatch), ctypes.sizeof(_lib.TsSelCache),
+                   _lib.TsBatch.threshold_hint.offset, _lib.TsBatch.wait_us.offset,
+                   _lib.TsBatch.workspace_clean.offset, _lib.TsBatch.host_seq_lens.offset]
