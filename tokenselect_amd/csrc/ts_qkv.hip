@@ -39,15 +39,10 @@ struct QkvArgs {
   int page_shift;
 };
 
-__device__ __forceinline__ void unpack8(const uint4& w, float (&f)[8]) {
-  f[0] = bf16_lo(w.x);
-  f[1] = bf16_hi(w.x);
-  f[2] = bf16_lo(w.y);
-  f[3] = bf16_hi(w.y);
-  f[4] = bf16_lo(w.z);
-  f[5] = bf16_hi(w.z);
-  f[6] = bf16_lo(w.w);
-  f[7] = bf16_hi(w.w);
+// a.lo * b.lo + a.hi * b.hi + c on packed bf16 pairs.
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c,
+                                         false);
 }
 
 // W is read once: a non-temporal load keeps it from displacing the rest of the cache.
@@ -85,20 +80,21 @@ __global__ __launch_bounds__(64 * kQkvWaves) void qkv_store_kernel(QkvArgs a) {
   for (int r = 0; r < kQkvRows; ++r)
 #pragma unroll
     for (int b = 0; b < B; ++b) acc[r][b] = 0.f;
+  // Two bf16 products per instruction, accumulated in fp32 (v_dot2c_f32_bf16): the operands
+  // stay packed as they were loaded, nothing is unpacked.
 #pragma unroll
   for (int j = 0; j < kQkvPieces; ++j) {
     const int v = min(lane + 64 * j, kvec - 1);  // past the row: W piece is zero
-    float wf[kQkvRows][8];
-#pragma unroll
-    for (int r = 0; r < kQkvRows; ++r) unpack8(wv[r][j], wf[r]);
 #pragma unroll
     for (int b = 0; b < B; ++b) {
-      float xf[8];
-      unpack8(lds_x[b * kvec + v], xf);
+      const uint4 xv = lds_x[b * kvec + v];
 #pragma unroll
-      for (int r = 0; r < kQkvRows; ++r)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[r][b] += wf[r][e] * xf[e];
+      for (int r = 0; r < kQkvRows; ++r) {
+        acc[r][b] = dot2_bf16(wv[r][j].x, xv.x, acc[r][b]);
+        acc[r][b] = dot2_bf16(wv[r][j].y, xv.y, acc[r][b]);
+        acc[r][b] = dot2_bf16(wv[r][j].z, xv.z, acc[r][b]);
+        acc[r][b] = dot2_bf16(wv[r][j].w, xv.w, acc[r][b]);
+      }
     }
   }
 
@@ -106,8 +102,10 @@ __global__ __launch_bounds__(64 * kQkvWaves) void qkv_store_kernel(QkvArgs a) {
   for (int r = 0; r < kQkvRows; ++r)
 #pragma unroll
     for (int b = 0; b < B; ++b) {
-#pragma unroll
-      for (int off = 32; off >= 1; off >>= 1) acc[r][b] += __shfl_xor(acc[r][b], off);
+      // (within a row of 16 lanes by DPP, the four rows through the LDS crossbar)
+      acc[r][b] = row16_sum(acc[r][b]);
+      acc[r][b] += __shfl_xor(acc[r][b], 16);
+      acc[r][b] += __shfl_xor(acc[r][b], 32);
     }
   // Lane r * B + b writes y[b][n0 + r] (every lane holds every sum).
   float y = 0.f;
