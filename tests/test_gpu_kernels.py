@@ -687,6 +687,29 @@ def test_sparse_attention(dev, shape, rope_mode):
         assert err <= 2e-2, f"attention b={b}: max abs err {err}"
 
 
+@pytest.mark.parametrize("B,S", [(1, 40000), (3, 23456)])
+def test_attention_over_a_long_dense_list(dev, B, S):
+    """A dense request attends over every token (tr.py:377-378, 741-744): lists of tens of
+    thousands of entries, 64 workgroups of hundreds of tokens per KV head on the matrix cores,
+    a wavefront's rotation advanced over dozens of steps; against the oracle in fp32."""
+    say(f"attention over dense lists B={B} S={S}")
+    wl = small(dev, SHAPES[0], seed=45, lens=[S] * B, ks=[64] * B)
+    c = wl.cfg
+    assert ops.attention_kernel_form(c, B, S) == 1
+    g = torch.Generator().manual_seed(46)
+    lens = [S - 777 * b for b in range(B)]
+    sel = torch.stack([torch.randperm(wl.k_pool.shape[0], generator=g)[:S] for _ in range(B)]).int()
+    sel_len = torch.tensor(lens, dtype=torch.int32)
+    out = ops.sparse_decode_attention(c, wl.q, wl.k_pool, wl.v_pool, sel.to(dev), sel_len.to(dev))
+    torch.cuda.synchronize()
+    kc, vc, qc = wl.k_pool.cpu(), wl.v_pool.cpu(), wl.q.cpu()
+    for b in range(B):
+        ref = oracle.attend.sparse_decode_attention(
+            qc[b].view(c.num_heads, 128), kc, vc, sel[b, :lens[b]], 128 ** -0.5, c.rope_theta, 1.0, 0.0, c.rope_mode)
+        err = (out[b].cpu().float() - ref.reshape(-1).float()).abs().max().item()
+        assert err <= 2e-2, f"b={b}: max abs err {err}"
+
+
 @pytest.mark.parametrize("B", [1, 14], ids=["vector", "matrix"])
 def test_attention_never_reads_a_row_it_was_not_given(dev, B):
     """A KV pool as a server holds it: only the rows in use hold numbers.  Every row that no
