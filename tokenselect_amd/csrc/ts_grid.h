@@ -79,9 +79,10 @@ __device__ __forceinline__ void grid_poll(uint32_t* sync, uint32_t round, uint64
         break;
       }
     }
-    // About 0.5 us between polls: polling faster costs more (the early workgroups' polls
-    // compete with the key stream of the late ones) than seeing the flag sooner brings.
-    __builtin_amdgcn_s_sleep(20);
+    // About 0.16 us between polls.  (Every rendezvous of the fused kernels comes after the
+    // statistics exchange, when no workgroup of the request streams keys any more: the polls
+    // compete with nothing.  The statistics are polled for more sparsely, see there.)
+    __builtin_amdgcn_s_sleep(6);
   }
 }
 

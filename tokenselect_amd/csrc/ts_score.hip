@@ -938,15 +938,13 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
                         req_chunks <= kSelMaxChunks / 2;
     const int band_lo = hint_bin - kBandBelow;  // (bins outside [0, kTopkBins) hold nothing)
     uint32_t over_band = 0;  // this thread's tokens above the band
+    uint32_t top = 0;        // this thread's highest bin
     for (int base = 0; base < count; base += 256) {
       const bool have = base + tid < count;
       const uint32_t key = have ? key_of(base + tid) : 0u;
       const uint32_t bin = have ? key_bin0(key) : 0u;
       if (have) atomicAdd(&lh[bin], 1u);
-      uint32_t top = bin;
-#pragma unroll
-      for (int off = 32; off >= 1; off >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, off));
-      if (lane == 0) atomicMax(&scratch[8], top);
+      top = max(top, bin);
       if (banded) {
         const int d = (int)bin - band_lo;
         if (have && d >= 0 && d < kBandBins) {
@@ -957,6 +955,9 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         over_band += (have && d >= kBandBins) ? 1u : 0u;
       }
     }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, off));
+    if (lane == 0) atomicMax(&scratch[8], top);
     if (banded) {
 #pragma unroll
       for (int off = 32; off >= 1; off >>= 1) over_band += __shfl_xor(over_band, off);
