@@ -929,6 +929,16 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       for (int i = 0; i < kAheadLoads; ++i) asm volatile("" ::"v"(ahead[i]));
       return;
     }
+    // The physical slots of this thread's tokens, for the emission at the very end: the
+    // table entries are asked for here, several rendezvous ahead, instead of in the
+    // kernel's last microsecond with the stores waiting behind them.
+    constexpr int kEmitAhead = 5;  // x 256 tokens: the largest workgroup (1056 tokens)
+    uint32_t slot_ahead[kEmitAhead];
+#pragma unroll
+    for (int it = 0; it < kEmitAhead; ++it) {
+      const int i = min(it * 256 + tid, count - 1);
+      slot_ahead[it] = lookup_slot(tab, a.n_init + block_lo + i, a.page_size, a.page_shift, a.pool_rows);
+    }
     // Local histogram: one LDS atomic per candidate (lanes that hit the same bin are
     // performed one after the other, which for 256 candidates is a few hundred cycles).
     // With a hint, also what the band around it needs: the candidates of each band bin go
@@ -1423,44 +1433,53 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     int32_t* sel_pos = a.sel_pos + (int64_t)b * a.sel_stride;
     int32_t* cache_out = a.topk_cache ? a.topk_cache + (int64_t)b * a.top_k : nullptr;
     const uint64_t below = (1ull << lane) - 1ull;
-    for (int base = 0; base < count; base += 256) {
+#pragma unroll 1
+    for (int base = 0, it = 0; base < count; base += 256, ++it) {
       const int i = base + tid;
       const uint32_t key = i < count ? key_of(i) : 0u;
       const bool tie = i < count && key == kth;
-      const uint64_t tie_mask = __ballot(tie);
-      if (lane == 0) scratch[wave] = (uint32_t)__popcll(tie_mask);
-      __syncthreads();
-      uint32_t tie_rank = tie_run + (uint32_t)__popcll(tie_mask & below);
-      uint32_t tie_total = 0;
+      // The per-wavefront counts of an iteration go to one of two sets of words in turn: a
+      // set is written again two iterations later, after a barrier that every wavefront
+      // reaches only once it has read the set, so no barrier closes an iteration.
+      uint32_t* counts_lds = scratch + (it & 1) * 8;
+      uint32_t tie_rank = 0, tie_total = 0;
+      if (!listed) {  // (with the short list a tie is taken by its position: no ranks needed)
+        const uint64_t tie_mask = __ballot(tie);
+        if (lane == 0) counts_lds[wave] = (uint32_t)__popcll(tie_mask);
+        __syncthreads();
+        tie_rank = tie_run + (uint32_t)__popcll(tie_mask & below);
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        if (w < wave) tie_rank += scratch[w];
-        tie_total += scratch[w];
+        for (int w = 0; w < 4; ++w) {
+          if (w < wave) tie_rank += counts_lds[w];
+          tie_total += counts_lds[w];
+        }
       }
       // A tie is taken if it is among the first need_eq in position order; with the
       // short list that is: not beyond the position of the k-th entry.
       const bool tie_taken = listed ? (uint32_t)(block_lo + i) <= pos_thr : tie_rank < need_eq;
       const bool chosen = i < count && (key > kth || (tie && tie_taken));
       const uint64_t chosen_mask = __ballot(chosen);
-      if (lane == 0) scratch[4 + wave] = (uint32_t)__popcll(chosen_mask);
+      if (lane == 0) counts_lds[4 + wave] = (uint32_t)__popcll(chosen_mask);
       __syncthreads();
       uint32_t rank = out_run + (uint32_t)__popcll(chosen_mask & below);
       uint32_t chosen_total = 0;
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
-        if (w < wave) rank += scratch[4 + w];
-        chosen_total += scratch[4 + w];
+        if (w < wave) rank += counts_lds[4 + w];
+        chosen_total += counts_lds[4 + w];
       }
       if (chosen && rank < k) {
         const int pos = a.n_init + block_lo + i;
         sel_pos[a.n_init + rank] = pos;
-        sel[a.n_init + rank] =
-            (int32_t)lookup_slot(tab_b, pos, a.page_size, a.page_shift, a.pool_rows);
+        uint32_t slot = slot_ahead[0];
+#pragma unroll
+        for (int x = 1; x < kEmitAhead; ++x) slot = it == x ? slot_ahead[x] : slot;
+        if (it >= kEmitAhead) slot = lookup_slot(tab_b, pos, a.page_size, a.page_shift, a.pool_rows);
+        sel[a.n_init + rank] = (int32_t)slot;
         if (cache_out) cache_out[rank] = pos;
       }
       tie_run += tie_total;
       out_run += chosen_total;
-      __syncthreads();
     }
     TS_MARK(14);
     // A grid-wide wait of this launch gave up (the workgroups were not all resident
