@@ -49,7 +49,7 @@ MEASURED_TRAFFIC = {  # workload -> (bytes per launch of its dominant kernel, co
     "C5-layer": (2154387218, "e500026"),  # likewise
     "MODEL": (2158869023, "e500026"),     # likewise, inside the 32-layer decoder (page 1)
 }
-# attn_kernel<4> (C2) / attn_mfma_kernel<4> (C3, C5), same runs
+# attn_kernel<4>, same runs
 MEASURED_ATTN_TRAFFIC = {"C2": 12333004, "C3": 180835444, "C5-layer": 82174810}
 
 
@@ -179,9 +179,7 @@ def kernel_rooflines(ops, wl, k_pools, v_pools, layer, steps, warmup):
     attn_us, _ = event_time_us(
         lambda i: ops.sparse_decode_attention(c, wl.q, k_pools[i % n_pools], v_pools[i % n_pools],
                                               sel, sel_len), steps, warmup, burst=8)
-    mfma = ops.attention_kernel_form(c, sel.shape[0], sel.shape[1]) == 1
-    attn = {"kernel": ("ts::attn_mfma_kernel<G> (matrix cores)" if mfma else "ts::attn_kernel<G> (vector units)")
-                      + " + a 1 us ticket-clearing kernel when called on its own",
+    attn = {"kernel": "ts::attn_kernel<G> (+ a 1 us ticket-clearing kernel when called on its own)",
             "achieved": round(attn_bytes / attn_us / 1e3, 1), "unit": "GB/s",
             "frac": round(attn_bytes / attn_us / 1e3 / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_ATTN_TRAFFIC.get(wl.name.split()[0]),

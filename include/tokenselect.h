@@ -341,15 +341,10 @@ int ts_selcache_step(const ts_config* cfg, const ts_batch* bt, const void* qf,
  * sel [B, sel_stride] int32 with sel_len[b] valid entries (<= max_sel_len); every
  * row holds at least max_sel_len entries, those past sel_len[b] are read (the
  * slots are requested together with the length) but not used.
- * Two kernels serve it.  Launches in which a workgroup reads one batch of rows (a few
- * requests: up to 512 workgroups of 128 list entries cover the lists) compute in fp32 on
- * the vector units.  Launches with longer ranges per workgroup (many requests) run on the
- * matrix cores: rotated keys and softmax weights are rounded to bf16 for
- * v_mfma_f32_16x16x32_bf16 with fp32 accumulation, as the tensor-core path of the
- * reference's attention library does; the outputs of the two differ by about one unit of
- * bf16 rounding.  ts_attn_kernel_form tells which one a shape gets (0 vector, 1 matrix). */
+ * The products run on the matrix cores (v_mfma_f32_16x16x32_bf16, fp32 accumulation) with
+ * every fp32 operand - rotated key, rotated query, softmax weight - split into two bf16
+ * halves, so that the result equals an fp32 evaluation to the rounding of the bf16 output. */
 size_t ts_attn_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_sel_len);
-int ts_attn_kernel_form(const ts_config* cfg, int32_t batch, int32_t max_sel_len);
 int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_pool,
                           const void* v_pool, int64_t pool_rows, const int32_t* sel,
                           int64_t sel_stride, const int32_t* sel_len, int32_t batch,

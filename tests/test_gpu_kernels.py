@@ -690,12 +690,11 @@ def test_sparse_attention(dev, shape, rope_mode):
 @pytest.mark.parametrize("B,S", [(1, 40000), (3, 23456)])
 def test_attention_over_a_long_dense_list(dev, B, S):
     """A dense request attends over every token (tr.py:377-378, 741-744): lists of tens of
-    thousands of entries, 64 workgroups of hundreds of tokens per KV head on the matrix cores,
-    a wavefront's rotation advanced over dozens of steps; against the oracle in fp32."""
+    thousands of entries, 64 workgroups of hundreds of tokens per KV head, a wavefront's
+    rotation advanced over dozens of steps; against the oracle in fp32."""
     say(f"attention over dense lists B={B} S={S}")
     wl = small(dev, SHAPES[0], seed=45, lens=[S] * B, ks=[64] * B)
     c = wl.cfg
-    assert ops.attention_kernel_form(c, B, S) == 1
     g = torch.Generator().manual_seed(46)
     lens = [S - 777 * b for b in range(B)]
     sel = torch.stack([torch.randperm(wl.k_pool.shape[0], generator=g)[:S] for _ in range(B)]).int()
@@ -710,18 +709,17 @@ def test_attention_over_a_long_dense_list(dev, B, S):
         assert err <= 2e-2, f"b={b}: max abs err {err}"
 
 
-@pytest.mark.parametrize("B", [1, 14], ids=["vector", "matrix"])
+@pytest.mark.parametrize("B", [1, 14])
 def test_attention_never_reads_a_row_it_was_not_given(dev, B):
     """A KV pool as a server holds it: only the rows in use hold numbers.  Every row that no
     list names is filled with NaN, and the entries of `sel` past the lengths point at such rows
     (or outside the pool): a token past a range has the weight zero, but 0 x NaN is NaN, so the
-    kernels must not fetch those rows at all.  Both kernels (one request: vector; 14: matrix)."""
+    kernel must not fetch those rows at all.  One request (one tile per wavefront) and 14."""
     lens = [2541] if B == 1 else [2600, 2599, 2541, 1025, 700, 333, 65, 64, 33, 17, 1, 0, 2600, 1800]
     width = 2600
     say(f"attention over a pool with NaN in every unused row B={B}")
     wl = small(dev, SHAPES[0], seed=43, lens=[3000] * B, ks=[64] * B)
     c = wl.cfg
-    assert ops.attention_kernel_form(c, B, width) == (0 if B == 1 else 1)
     P = wl.k_pool.shape[0]
     g = torch.Generator().manual_seed(44)
     used = torch.zeros(P, dtype=torch.bool)
@@ -750,20 +748,17 @@ def test_attention_never_reads_a_row_it_was_not_given(dev, B):
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
 @pytest.mark.parametrize("rope_mode,cap", [("ROPE_LLAMA", 0.0), ("NONE", 0.0), ("ROPE_LLAMA", 25.0)])
-def test_sparse_attention_on_the_matrix_cores(dev, shape, rope_mode, cap):
-    """Many requests with long lists: a workgroup walks several tiles and the launch takes the
-    matrix-core kernel (asserted), every head shape, with and without the rotation and the soft
-    cap; ragged lengths that end inside a tile, inside a wavefront's range, at one entry and at
-    none; the one-request launch of the same lists (vector kernel) agrees within the rounding
-    of the matrix operands."""
-    say(f"attention on the matrix cores H={shape['num_heads']} Hkv={shape['num_kv_heads']} {rope_mode} cap={cap}")
+def test_sparse_attention_of_many_requests(dev, shape, rope_mode, cap):
+    """Many requests with long lists: a workgroup walks several tiles, every head shape, with
+    and without the rotation and the soft cap; ragged lengths that end inside a tile, inside a
+    wavefront's range, at one entry and at none; the one-request launch of the same lists (one
+    tile per wavefront, other ranges) agrees to the rounding of the output."""
+    say(f"attention of many requests H={shape['num_heads']} Hkv={shape['num_kv_heads']} {rope_mode} cap={cap}")
     lens = [2600, 2599, 2541, 1025, 700, 333, 65, 64, 33, 17, 1, 0, 2600, 1800]
     B, width = len(lens), 2600
     wl = small(dev, shape, seed=41, lens=[3000] * B, ks=[64] * B)
     c = wl.cfg
     c.rope_mode, c.logit_cap = rope_mode, cap
-    assert ops.attention_kernel_form(c, B, width) == 1
-    assert ops.attention_kernel_form(c, 1, width) == 0
     g = torch.Generator().manual_seed(42)
     sel = torch.zeros((B, width), dtype=torch.int32)
     for b, S in enumerate(lens):
@@ -783,7 +778,8 @@ def test_sparse_attention_on_the_matrix_cores(dev, shape, rope_mode, cap):
         assert err <= 2e-2, f"attention b={b} S={S}: max abs err {err}"
         alone = ops.sparse_decode_attention(c, wl.q[b:b + 1], wl.k_pool, wl.v_pool, sel[b:b + 1].to(dev),
                                             sel_len[b:b + 1].to(dev))
-        assert (alone[0].float() - out[b].float()).abs().max().item() <= 2e-2
+        # (the same fp32-equivalent arithmetic over other ranges: a unit of the output's rounding)
+        assert (alone[0].float() - out[b].float()).abs().max().item() <= 2 ** -6 * max(1.0, out[b].float().abs().max().item())
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")

@@ -82,7 +82,6 @@ SIGNATURES = {
     "ts_select_clear": (_i32, [_CFG, _BT, _ptr, _size, _ptr]),
     "ts_selcache_step": (_i32, [_CFG, _BT, _ptr, _SC, _ptr, _ptr]),
     "ts_attn_workspace_bytes": (_size, [_CFG, _i32, _i32]),
-    "ts_attn_kernel_form": (_i32, [_CFG, _i32, _i32]),
     "ts_sparse_decode_attn": (_i32, [_CFG, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32,
                                      _ptr, _ptr, _size, _ptr]),
     "ts_attn_static_scratch_bytes": (_size, []),

@@ -1,20 +1,13 @@
 // Decode attention over the selected KV slots: the FlashInfer paged decode the
 // reference calls at tr.py:815-823 (page size 1, in-kernel Llama RoPE).
 //
-// Split-K in one launch: grid (splits, Hkv, B).  A workgroup owns a contiguous
-// range of the request's selected list for one KV head and the G = H/Hkv query heads
-// that read it.  Two kernels: attn_kernel (vector units, fp32 throughout) where a
-// workgroup reads one batch of rows, attn_mfma_kernel (matrix cores) where it walks
-// several; they share the end of the workgroup (attn_finish).  In attn_kernel the
-// query heads stay in registers and sixteen lanes gather one K row and one
-// V row (256 bytes each, as two 128-byte halves); the sixteen lane groups of a
-// workgroup walk the range with stride 16, eight tokens per lane group in flight
-// (the slots, then all keys, then all values are requested before the first is
-// used: the pass is bound by memory latency, not bandwidth).  Keys are rotated to their index in
-// the selected list, the query to S-1; softmax is online in fp32.  Partial
-// (max, sum, acc) triples are merged across the lane groups and waves, written
-// with device-coherent stores, and the workgroup that draws the last ticket of
-// its (request, KV head) merges the splits and writes the bf16 output.
+// Split-K in one launch: grid (splits, Hkv, B).  A workgroup owns a contiguous range of
+// the request's selected list for one KV head and all G = H/Hkv query heads that read it;
+// its four wavefronts walk a quarter of the range each, in tiles of 32 tokens, on the
+// matrix cores (see attn_kernel).  Keys are rotated to their index in the selected list,
+// the query to S-1; softmax is online in fp32.  Partial (max, sum, acc) triples are merged
+// across the wavefronts, written with device-coherent stores, and the workgroup that draws
+// the last ticket of its (request, KV head) merges the splits and writes the bf16 output.
 #include <math.h>
 
 #include <mutex>
@@ -34,13 +27,12 @@ struct AttnArgs {
   const int32_t* sel_len;
   int num_heads, num_kv_heads;
   int group;          // query heads per KV head
-  int parts;          // workgroups that share the heads of a KV head (grid.y = Hkv * parts)
   int rope_mode;
   float log2_theta, rope_rcp_scale, sm_scale, logit_cap;
   int nsplit, max_sel_len;
   float* part_acc;    // [B,H,nsplit,128]
   float* part_ml;     // [B,H,nsplit,2]
-  uint32_t* tickets;  // [B,Hkv*parts], zero at launch and again when the kernel ends
+  uint32_t* tickets;  // [B,Hkv], zero at launch and again when the kernel ends
   uint16_t* out;      // [B,H,128] bf16
   ZeroSet zero;       // cleared on the side (counters of the stream's next selection)
 };
@@ -50,13 +42,6 @@ __device__ __forceinline__ void attn_clear_on_the_side(const AttnArgs& a) {
   if (a.zero.used == 0) return;
   const int64_t wg = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
   clear_regions(a.zero, wg * 256 + threadIdx.x, (int64_t)gridDim.x * gridDim.y * gridDim.z * 256);
-}
-
-__device__ __forceinline__ void unpack4(const uint2& w, float* f) {
-  f[0] = bf16_lo(w.x);
-  f[1] = bf16_hi(w.x);
-  f[2] = bf16_lo(w.y);
-  f[3] = bf16_hi(w.y);
 }
 
 __device__ __forceinline__ float2 load_coherent2(const float* p) {
@@ -74,16 +59,15 @@ __device__ __forceinline__ void store_coherent2(float* p, float x, float y) {
 
 // The end of an attention workgroup: its four wavefronts' partial (max, sum, acc) triples
 // of G head slots lie in LDS; they are merged, written with device-coherent stores, and the
-// workgroup that draws the last ticket of its (request, KV head, part) merges the splits and
+// workgroup that draws the last ticket of its (request, KV head) merges the splits and
 // writes the bf16 output.
 template <int G>
-__device__ __forceinline__ void attn_finish(const AttnArgs& a, int b, int kvh, int part, int split,
+__device__ __forceinline__ void attn_finish(const AttnArgs& a, int b, int kvh, int split,
                                             float (*sm_acc)[G][kHeadDim], float (*sm_m)[G],
                                             float (*sm_l)[G], uint32_t* s_last_ptr) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int H = a.num_heads;
-  auto head_of_slot = [&](int g) { return kvh * a.group + min(part * G + g, a.group - 1); };
-  auto slot_active = [&](int g) { return part * G + g < a.group; };
+  auto head_of_slot = [&](int g) { return kvh * G + g; };
   uint32_t& s_last = *s_last_ptr;
   __syncthreads();
   // A thread owns two adjacent dims of one head: one 64-bit coherent store.
@@ -100,7 +84,6 @@ __device__ __forceinline__ void attn_finish(const AttnArgs& a, int b, int kvh, i
       o1 += sm_acc[w][g][d + 1] * sc;
       ll += sm_l[w][g] * sc;
     }
-    if (!slot_active(g)) continue;
     const size_t ph = ((size_t)b * H + head_of_slot(g)) * a.nsplit + split;
     store_coherent2(a.part_acc + ph * kHeadDim + d, o0, o1);
     if (d == 0) store_coherent2(a.part_ml + ph * 2, mm, ll);
@@ -109,7 +92,7 @@ __device__ __forceinline__ void attn_finish(const AttnArgs& a, int b, int kvh, i
   // Ticket: the stores above are acknowledged before the workgroup is counted.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  uint32_t* ticket = a.tickets + ((size_t)b * a.num_kv_heads + kvh) * a.parts + part;
+  uint32_t* ticket = a.tickets + (size_t)b * a.num_kv_heads + kvh;
   if (tid == 0) {
     const uint32_t before =
         __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -127,7 +110,6 @@ __device__ __forceinline__ void attn_finish(const AttnArgs& a, int b, int kvh, i
   static_assert(kHeadDim / 2 == 64, "one wavefront per head slot");
   for (int idx = tid; idx < G * (kHeadDim / 2); idx += 256) {
     const int g = idx / (kHeadDim / 2), d = (idx % (kHeadDim / 2)) * 2;
-    if (!slot_active(g)) continue;  // (uniform over the wave)
     const size_t ph = ((size_t)b * H + head_of_slot(g)) * a.nsplit;
     float mm = kNegBig, ll = 0.f, o0 = 0.f, o1 = 0.f;
     for (int s0 = 0; s0 < a.nsplit; s0 += 32) {
@@ -169,280 +151,14 @@ __device__ __forceinline__ void attn_finish(const AttnArgs& a, int b, int kvh, i
   if (tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-constexpr int kAttnInFlight = 8;  // tokens per lane group requested together
-
-// ROPE and CAP are compile-time so that the token loop carries no branches other
-// than the wave-uniform ones that skip tokens past the range.
-//
-// A lane owns four rotation pairs of the head dimension: dims 4*l16 .. 4*l16+3 and
-// their partners 64 dims further on, so a key row arrives as two 8-byte pieces per
-// lane (the sixteen lanes of a group still read two full 128-byte lines) and the
-// rotation needs no exchange between lanes.  The softmax runs on batches of tokens:
-// the logits of a batch are collected first, the running maximum moves once per
-// batch and every token costs one exponential per head.
-// G = query heads per workgroup.  A KV head with more than four query heads is served by
-// several workgroups (parts) of four heads each, which fetch the same rows: with seven or
-// eight heads in one workgroup the registers allowed softmax batches of two or four tokens
-// only, and half as many workgroups shared the same number of rows (Qwen2-7B, 28 heads on 4
-// KV heads, 32K context: 20.6 us against the 14 us of 32 heads on 8).
-template <int G, bool ROPE, bool CAP>
-__global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
-  attn_clear_on_the_side(a);
-  const int split = blockIdx.x, b = blockIdx.z;
-  const int kvh = blockIdx.y / a.parts, part = blockIdx.y % a.parts;
-  // Head g of this workgroup: the last part of a group of five or seven has one head too
-  // many, which is computed (on the last real head's query) and not stored.
-  auto head_of_slot = [&](int g) { return kvh * a.group + min(part * G + g, a.group - 1); };
-  // The ranges are cut from the longest list the launch was sized for, not from this
-  // request's own length: the first slots can then be requested together with the
-  // length instead of after it (a shorter request leaves its last workgroups idle).
-  const int chunk = (a.max_sel_len + a.nsplit - 1) / a.nsplit;
-  const int lo = split * chunk;
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int lg = tid >> 4;   // lane group 0..15 inside the workgroup
-  const int l16 = tid & 15;  // owns dims [4*l16, 4*l16+4) and [64+4*l16, 64+4*l16+4)
-  const int H = a.num_heads;
-  constexpr bool rope = ROPE;
-  // Tokens per softmax batch: as many as the registers allow at two waves per SIMD.
-  static_assert(G <= 4, "at most four heads per workgroup");
-  constexpr int kBatch = kAttnInFlight;
-  const int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
-  const size_t row_elems = (size_t)a.num_kv_heads * kHeadDim;
-
-  // First batch of slots: requested before the rotation set-up below.  Entries past
-  // the request's length are read (they lie inside its row of `sel`) and never used.
-  uint32_t slot[kAttnInFlight];
-  auto load_slots = [&](int j0) {
-#pragma unroll
-    for (int u = 0; u < kAttnInFlight; ++u)
-      slot[u] = (uint32_t)sel[min(j0 + 16 * u, a.max_sel_len - 1)];
-  };
-  load_slots(lo + lg);
-  // The slot of the range's first entry stands in for entries past the range: their tokens
-  // get the weight zero, and 0 x whatever an unused or stale entry points at need not be 0.
-  uint32_t first_slot = (uint32_t)sel[min(lo, a.max_sel_len - 1)];
-  const int S = min(max(a.sel_len[b], 0), a.max_sel_len);
-  const int hi = min(S, lo + chunk);
-  first_slot = first_slot < a.pool_rows ? first_slot : a.pool_rows - 1;
-
-  // Frequencies of this lane's 4 rotation pairs: theta^(-2 pair / 128) / scale.
-  float freq[4];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const int pair = l16 * 4 + e;
-    freq[e] = a.rope_rcp_scale * __builtin_amdgcn_exp2f(-(float)pair * (2.0f / kHeadDim) * a.log2_theta);
-  }
-
-  // Query rows of the G heads, rotated to position S-1: [0..3] low dims, [4..7] partners.
-  float qv[G][8];
-  {
-    float qc[4], qs[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      qc[e] = 1.f;
-      qs[e] = 0.f;
-      if (rope) sincos_reduced((float)(S - 1) * freq[e], qs[e], qc[e]);
-    }
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const uint16_t* qrow = a.q + ((size_t)b * H + head_of_slot(g)) * kHeadDim;
-      float x[4], y[4];
-      unpack4(*(const uint2*)(qrow + l16 * 4), x);
-      unpack4(*(const uint2*)(qrow + 64 + l16 * 4), y);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        qv[g][e] = x[e] * qc[e] - y[e] * qs[e];
-        qv[g][4 + e] = y[e] * qc[e] + x[e] * qs[e];
-      }
-    }
-  }
-
-  // Key rotation state: angle of token j is j*freq; advance by 16 tokens per step.
-  float kc[4], ks[4], dc[4], ds[4];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    kc[e] = 1.f;
-    ks[e] = 0.f;
-    dc[e] = 1.f;
-    ds[e] = 0.f;
-    if (rope) {
-      sincos_reduced((float)(lo + lg) * freq[e], ks[e], kc[e]);
-      sincos_reduced(16.0f * freq[e], ds[e], dc[e]);
-    }
-  }
-
-  float m[G], l[G], acc[G][8];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    m[g] = kNegBig;
-    l[g] = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
-  }
-
-  // Two workgroups share a CU and the older one is served first: left alone it finishes
-  // well ahead and the other one then runs by itself, its memory waits uncovered.  A
-  // wavefront therefore lowers its priority as it advances through its range, so that
-  // whichever workgroup is behind is the one served first.
-  const int passes = (chunk + 16 * kAttnInFlight - 1) / (16 * kAttnInFlight);
-  int pass = 0;
-  for (int j0 = lo + lg; j0 < hi + (lg & 3); j0 += 16 * kAttnInFlight, ++pass) {
-    if (passes > 1) {
-      const int level = __builtin_amdgcn_readfirstlane(3 - (4 * pass) / passes);
-      if (level >= 3)
-        __builtin_amdgcn_s_setprio(3);
-      else if (level == 2)
-        __builtin_amdgcn_s_setprio(2);
-      else if (level == 1)
-        __builtin_amdgcn_s_setprio(1);
-      else
-        __builtin_amdgcn_s_setprio(0);
-    }
-    // The first token of the wavefront's four lane groups in this pass: a token
-    // step whose first token lies past the range is skipped by the whole wavefront.
-    const int wave_j0 = __builtin_amdgcn_readfirstlane(j0 - (lg & 3));
-    uint2 klo[kAttnInFlight], khi[kAttnInFlight], vlo[kAttnInFlight], vhi[kAttnInFlight];
-#pragma unroll
-    for (int u = 0; u < kAttnInFlight; ++u) {
-      slot[u] = (j0 + 16 * u < hi && slot[u] < a.pool_rows) ? slot[u] : first_slot;
-      const size_t at = (size_t)slot[u] * row_elems + (size_t)kvh * kHeadDim + l16 * 4;
-      klo[u] = *(const uint2*)(a.k_pool + at);
-      khi[u] = *(const uint2*)(a.k_pool + at + 64);
-    }
-    // The values after all the keys: the logits of the batch need every key, and
-    // the values arrive while they are being computed.
-#pragma unroll
-    for (int u = 0; u < kAttnInFlight; ++u) {
-      const size_t at = (size_t)slot[u] * row_elems + (size_t)kvh * kHeadDim + l16 * 4;
-      vlo[u] = *(const uint2*)(a.v_pool + at);
-      vhi[u] = *(const uint2*)(a.v_pool + at + 64);
-    }
-    if (wave_j0 + 16 * kAttnInFlight < hi) load_slots(j0 + 16 * kAttnInFlight);
-#pragma unroll
-    for (int u0 = 0; u0 < kAttnInFlight; u0 += kBatch) {
-      if (wave_j0 + 16 * u0 >= hi) break;
-      // Logits of the batch; a token past the range gets -inf: weight 0, maximum
-      // unchanged (the running maximum starts at a finite value, so nothing becomes NaN).
-      float p[G][kBatch];
-#pragma unroll
-      for (int ub = 0; ub < kBatch; ++ub) {
-        const int u = u0 + ub;
-#pragma unroll
-        for (int g = 0; g < G; ++g) p[g][ub] = -INFINITY;
-        if (wave_j0 + 16 * u < hi) {
-          const bool valid = j0 + 16 * u < hi;  // uniform over the 16 lanes of a group
-          float kx[4], ky[4];
-          unpack4(klo[u], kx);
-          unpack4(khi[u], ky);
-          if (rope) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const float x = kx[e] * kc[e] - ky[e] * ks[e];
-              ky[e] = ky[e] * kc[e] + kx[e] * ks[e];
-              kx[e] = x;
-            }
-          }
-#pragma unroll
-          for (int g = 0; g < G; ++g) {
-            float d = 0.f;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) d += qv[g][e] * kx[e] + qv[g][4 + e] * ky[e];
-            d = row16_sum(d) * a.sm_scale;
-            if (CAP) d = a.logit_cap * tanhf(d / a.logit_cap);
-            p[g][ub] = valid ? d : -INFINITY;
-          }
-        }
-        if (rope) {  // next token of this lane group: 16 positions further
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float c2 = kc[e] * dc[e] - ks[e] * ds[e];
-            ks[e] = ks[e] * dc[e] + kc[e] * ds[e];
-            kc[e] = c2;
-          }
-        }
-      }
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        float mn = m[g];
-#pragma unroll
-        for (int ub = 0; ub < kBatch; ++ub) mn = fmaxf(mn, p[g][ub]);
-        const float alpha = __expf(m[g] - mn);
-        float sum = 0.f;
-#pragma unroll
-        for (int ub = 0; ub < kBatch; ++ub) {
-          p[g][ub] = __expf(p[g][ub] - mn);
-          sum += p[g][ub];
-        }
-        l[g] = l[g] * alpha + sum;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] *= alpha;
-        m[g] = mn;
-      }
-#pragma unroll
-      for (int ub = 0; ub < kBatch; ++ub) {
-        const int u = u0 + ub;
-        if (wave_j0 + 16 * u < hi) {
-          float vx[4], vy[4];
-          unpack4(vlo[u], vx);
-          unpack4(vhi[u], vy);
-#pragma unroll
-          for (int g = 0; g < G; ++g)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              acc[g][e] += p[g][ub] * vx[e];
-              acc[g][4 + e] += p[g][ub] * vy[e];
-            }
-        }
-      }
-    }
-  }
-
-  __builtin_amdgcn_s_setprio(0);
-  // Merge the four lane groups of a wave (rows of 16 lanes), then the four waves.
-  __shared__ float sm_acc[4][G][kHeadDim];
-  __shared__ float sm_m[4][G], sm_l[4][G];
-  __shared__ uint32_t s_last;
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-#pragma unroll
-    for (int off = 16; off <= 32; off <<= 1) {
-      const float m2 = __shfl_xor(m[g], off), l2 = __shfl_xor(l[g], off);
-      const float mn = fmaxf(m[g], m2);
-      const float a1 = __expf(m[g] - mn), a2 = __expf(m2 - mn);
-      l[g] = l[g] * a1 + l2 * a2;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * a1 + __shfl_xor(acc[g][e], off) * a2;
-      m[g] = mn;
-    }
-    if (lane < 16) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        sm_acc[wave][g][l16 * 4 + e] = acc[g][e];
-        sm_acc[wave][g][64 + l16 * 4 + e] = acc[g][4 + e];
-      }
-      if (lane == 0) {
-        sm_m[wave][g] = m[g];
-        sm_l[wave][g] = l[g];
-      }
-    }
-  }
-  attn_finish<G>(a, b, kvh, part, split, sm_acc, sm_m, sm_l, &s_last);
-}
-
 // ---------------------------------------------------------------------------------------
-// The same attention on the matrix cores, for launches in which a workgroup walks several
-// hundred tokens (many requests at once): there the loop above is bound by its vector
-// instructions (some 40 per token and wavefront: dot products, reductions over 16 lanes, a
-// softmax every lane of a token's group repeats), here a token costs about 16.
-//
-// A wavefront walks a contiguous quarter of the workgroup's range in tiles of 32 tokens.
-// v_mfma_f32_16x16x32_bf16 three times over:
+// attn_kernel<G, ROPE, CAP>: G = H / Hkv query heads per workgroup (1 to 8), on the matrix
+// cores.  A wavefront walks a contiguous quarter of the workgroup's range in tiles of 32
+// tokens.  v_mfma_f32_16x16x32_bf16 three times over:
 //   logits   S[token][head] = K' Q'^T : A = 16 rotated keys x 32 dims (lane (token l%16,
-//            l/16) loads 16 bytes of its token's row per 32 dims, rotates them in fp32 - the
-//            partner dims d and d + 64 are in the same lane - and rounds to bf16, as the
-//            tensor-core path of the reference's attention library does), B = the query
-//            heads as columns (G of 16 used), rotated to S - 1 and rounded once.
+//            l/16) loads 16 bytes of its token's row per 32 dims and rotates them in fp32 -
+//            the partner dims d and d + 64 are in the same lane), B = the query heads as
+//            columns (G of 16 used), rotated to S - 1 once.
 //   V^T      a value row arrives like a key row (a lane holds 8 consecutive dims of one
 //            token); the matrix product with a 0/1 matrix that selects 16 of 32 dims leaves
 //            lane (dim l%16, l/16) with that dim of four consecutive tokens, exactly (bf16
@@ -450,6 +166,13 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnArgs a) {
 //   output   O^T[dim][head] += V^T P : A = 16 dims x 32 tokens from the step above, B = the
 //            weights of the tile, which the logits' product left in the lanes that need them
 //            (lane (head l%16, l/16): tokens 4 (l/16) + r of both 16-token halves).
+// The matrix instructions take bf16, the reference's attention works in fp32 on rotated keys:
+// every fp32 operand (rotated key, rotated query, softmax weight) is therefore split into a
+// bf16 value and the bf16 of what the rounding left, x = hi + lo to 2^-18 of x, and the
+// products are taken as hi hi + lo hi + hi lo (fp32 accumulation; the values are bf16 as
+// stored).  The results match an fp32 evaluation to the rounding of the bf16 output; with
+// single bf16 operands the mean error was a hundred times larger and the largest one
+// exceeded 2e-2 for outputs of magnitude 2 under a peaked softmax.
 // Everything of a head lives in the four lanes of its column: the running maximum moves once
 // per tile (two exchanges between the lane groups), the sums stay per lane until the end.
 // The loads of the next tile's keys are issued when this tile's have been rotated, those of
@@ -477,8 +200,19 @@ __device__ __forceinline__ void unpack8(const uint4& w, float* f) {
   f[7] = bf16_hi(w.w);
 }
 
+// x = hi + lo with both halves in bf16: hi = x rounded, lo = the remainder rounded (the
+// subtraction is exact); what is lost is 2^-18 of x.
+__device__ __forceinline__ void split8(const float* x, at_bf16x8& hi, at_bf16x8& lo) {
+  const uint4 h = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]),
+                             pack_bf16(x[6], x[7]));
+  const float r[8] = {x[0] - bf16_lo(h.x), x[1] - bf16_hi(h.x), x[2] - bf16_lo(h.y), x[3] - bf16_hi(h.y),
+                      x[4] - bf16_lo(h.z), x[5] - bf16_hi(h.z), x[6] - bf16_lo(h.w), x[7] - bf16_hi(h.w)};
+  hi = __builtin_bit_cast(at_bf16x8, h);
+  lo = pack8(r);
+}
+
 // Tokens per workgroup of the matrix-core kernel for a launch of nsplit splits.
-__host__ __device__ __forceinline__ int attn_mfma_chunk(int max_sel_len, int nsplit) {
+__host__ __device__ __forceinline__ int attn_chunk(int max_sel_len, int nsplit) {
   const int even = (max_sel_len + nsplit - 1) / nsplit;
   return (even + kAttnChunkUnit - 1) / kAttnChunkUnit * kAttnChunkUnit;
 }
@@ -493,16 +227,16 @@ __device__ __forceinline__ int opaque_zero(uint32_t after) {
 }
 
 template <int G, bool ROPE, bool CAP>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_kernel(
-    AttnArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_kernel(AttnArgs a) {
+  constexpr bool SPLIT = true;  // (false: single bf16 operands, for measurements)
+  static_assert(G >= 1 && G <= 8, "the query heads of a KV head are columns of one tile");
   attn_clear_on_the_side(a);
-  const int split = blockIdx.x, b = blockIdx.z;
-  const int kvh = blockIdx.y / a.parts, part = blockIdx.y % a.parts;
+  const int split = blockIdx.x, b = blockIdx.z, kvh = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, qd = lane >> 4;
   const int H = a.num_heads;
-  const int chunk = attn_mfma_chunk(a.max_sel_len, a.nsplit);
+  const int chunk = attn_chunk(a.max_sel_len, a.nsplit);
   const int wlen = chunk / 4;
   const int32_t* sel = a.sel + (int64_t)b * a.sel_stride;
   const size_t row_elems = (size_t)a.num_kv_heads * kHeadDim;
@@ -510,16 +244,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // What every wavefront reads again and again lives in LDS, not in registers (the loop
   // below needs them all): the query operand, the 0/1 matrices, the rotation of one step.
   __shared__ __attribute__((aligned(16))) uint4 sm_q[4][64];     // B operand per 32 dims, per lane
+  __shared__ __attribute__((aligned(16))) uint4 sm_q_lo[SPLIT ? 4 : 1][64];  // its low halves
   __shared__ __attribute__((aligned(16))) uint4 sm_pick[2][64];  // B operand per half, per lane
   __shared__ __attribute__((aligned(16))) float2 sm_step[kHeadDim / 2];  // (cos, sin) of 16 tokens
   __shared__ float sm_acc[4][G][kHeadDim];
   __shared__ float sm_m[4][G], sm_l[4][G];
   __shared__ uint32_t s_last;
 
-  // Column n of the logits: head slot n of this workgroup (zeros beyond its heads).  Wavefront
+  // Column n of the logits: query head n of the KV head (zeros beyond its heads).  Wavefront
   // kb2 < 2 prepares the dims [32 kb2, +32) and their partners 64 further on.
-  const bool real = n < G && part * G + n < a.group;
-  const int head = kvh * a.group + min(part * G + min(n, G - 1), a.group - 1);
+  const bool real = n < G;
+  const int head = kvh * G + min(n, G - 1);
   // (No load of the start-up sits behind a branch: where a branch joins, the compiler waits
   // for every load that either side may have issued.)
   uint4 q_raw[2];
@@ -592,8 +327,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         x[e] = xr;
       }
     }
-    sm_q[wave][lane] = __builtin_bit_cast(uint4, pack8(x));
-    sm_q[wave + 2][lane] = __builtin_bit_cast(uint4, pack8(y));
+    if (SPLIT) {
+      at_bf16x8 hi, lo;
+      split8(x, hi, lo);
+      sm_q[wave][lane] = __builtin_bit_cast(uint4, hi);
+      sm_q_lo[wave][lane] = __builtin_bit_cast(uint4, lo);
+      split8(y, hi, lo);
+      sm_q[wave + 2][lane] = __builtin_bit_cast(uint4, hi);
+      sm_q_lo[SPLIT ? wave + 2 : 0][lane] = __builtin_bit_cast(uint4, lo);
+    } else {
+      sm_q[wave][lane] = __builtin_bit_cast(uint4, pack8(x));
+      sm_q[wave + 2][lane] = __builtin_bit_cast(uint4, pack8(y));
+    }
   }
   // This lane's 16 rotation pairs: dims 32 kb2 + 8 qd + e (kb2 < 2, e < 8) and their partners
   // 64 further on; key state at token wlo + n, 16 tokens per step.
@@ -637,7 +382,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       at_f32x4 s[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        at_bf16x8 ka[4];
+        at_bf16x8 ka[4], ka_lo[4];
 #pragma unroll
         for (int kb2 = 0; kb2 < 2; ++kb2) {
           float x[8], y[8];
@@ -652,15 +397,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
               x[e] = xr;
             }
           }
-          ka[kb2] = pack8(x);
-          ka[kb2 + 2] = pack8(y);
+          if (SPLIT) {
+            split8(x, ka[kb2], ka_lo[kb2]);
+            split8(y, ka[kb2 + 2], ka_lo[kb2 + 2]);
+          } else {
+            ka[kb2] = pack8(x);
+            ka[kb2 + 2] = pack8(y);
+          }
         }
         const int zq = opaque_zero(__builtin_bit_cast(uint4, ka[3]).w);
         s[t] = at_f32x4{0.f, 0.f, 0.f, 0.f};
+        if (SPLIT) {
+          // (k_hi + k_lo) (q_hi + q_lo) without the product of the two low halves: three
+          // chains that do not wait for each other, added up at the end.
+          at_f32x4 s_lh = {0.f, 0.f, 0.f, 0.f}, s_hl = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
-          s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              ka[kb], __builtin_bit_cast(at_bf16x8, sm_q[kb][lane + zq]), s[t], 0, 0, 0);
+          for (int kb = 0; kb < 4; ++kb) {
+            const at_bf16x8 q_hi = __builtin_bit_cast(at_bf16x8, sm_q[kb][lane + zq]);
+            const at_bf16x8 q_lo = __builtin_bit_cast(at_bf16x8, sm_q_lo[SPLIT ? kb : 0][lane + zq]);
+            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kb], q_hi, s[t], 0, 0, 0);
+            s_lh = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka_lo[kb], q_hi, s_lh, 0, 0, 0);
+            s_hl = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kb], q_lo, s_hl, 0, 0, 0);
+          }
+          s[t] += s_lh + s_hl;
+        } else {
+#pragma unroll
+          for (int kb = 0; kb < 4; ++kb)
+            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                ka[kb], __builtin_bit_cast(at_bf16x8, sm_q[kb][lane + zq]), s[t], 0, 0, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
         if (ROPE) {  // the same rows of the next 16 tokens
 #pragma unroll
@@ -716,7 +481,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       l = l * alpha + sum;
 #pragma unroll
       for (int dt = 0; dt < 8; ++dt) acc[dt] *= alpha;
-      const at_bf16x8 pb = pack8(p);
+      at_bf16x8 pb, pb_lo;
+      if (SPLIT)
+        split8(p, pb, pb_lo);
+      else
+        pb = pb_lo = pack8(p);
       // ---- values: transpose 16 dims at a time, accumulate
       const int zp = opaque_zero(__builtin_bit_cast(uint4, pb).x);
       at_bf16x8 pick[2];
@@ -732,7 +501,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           const at_f32x4 d1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
               __builtin_bit_cast(at_bf16x8, vr[1][c]), pick[h], zero, 0, 0, 0);
           const float vt[8] = {d0[0], d0[1], d0[2], d0[3], d1[0], d1[1], d1[2], d1[3]};
-          acc[2 * c + h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pack8(vt), pb, acc[2 * c + h], 0, 0, 0);
+          const at_bf16x8 vta = pack8(vt);
+          acc[2 * c + h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vta, pb, acc[2 * c + h], 0, 0, 0);
+          if (SPLIT) acc[2 * c + h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vta, pb_lo, acc[2 * c + h], 0, 0, 0);
         }
       __builtin_amdgcn_sched_barrier(0);
       if (more) {
@@ -761,44 +532,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       sm_l[wave][n] = l;
     }
   }
-  attn_finish<G>(a, b, kvh, part, split, sm_acc, sm_m, sm_l, &s_last);
+  attn_finish<G>(a, b, kvh, split, sm_acc, sm_m, sm_l, &s_last);
 }
 
 __global__ __launch_bounds__(256) void attn_zero_kernel(uint32_t* tickets, int count) {
   for (int i = blockIdx.x * 256 + threadIdx.x; i < count; i += gridDim.x * 256) tickets[i] = 0u;
 }
 
-// Workgroups per KV head and heads per workgroup for a group of `group` query heads.
-// (five or six heads: two workgroups of three; seven or eight: two of four)
-static int attn_parts(int group) { return (group + 3) / 4; }
-static int attn_heads_per_part(int group) { return (group + attn_parts(group) - 1) / attn_parts(group); }
-int attn_tickets_per_request(const ts_config* cfg) {
-  return cfg->num_kv_heads * attn_parts(cfg->num_heads / cfg->num_kv_heads);
-}
+// Tickets per request (the words to clear): one per KV head.
+int attn_tickets_per_request(const ts_config* cfg) { return cfg->num_kv_heads; }
 
-struct AttnPlan {
-  int nsplit;  // workgroups per (request, KV head, part)
-  bool mfma;   // the matrix-core kernel: a workgroup walks more than one batch of loads
-};
-static AttnPlan attn_plan(int batch, int num_kv_heads, int max_sel_len) {
-  // One batch of loads per lane group (16 groups x 8 tokens = 128 tokens per
-  // workgroup) as long as the grid stays within the 512 workgroups that are
-  // resident at once (two per CU): a second round of workgroups pays the start-up
-  // and merge latencies again, which costs more than longer ranges do.
-  int64_t want = ceil_div(max_sel_len, 16 * kAttnInFlight);
+constexpr int kAttnRange = 128;  // list entries per workgroup as long as the device has room
+static int attn_splits(int batch, int num_kv_heads, int max_sel_len) {
+  // One tile per wavefront (128 entries per workgroup) as long as the grid stays within the
+  // 512 workgroups that are resident at once (two per CU): a second round of workgroups pays
+  // the start-up and merge latencies again, which costs more than longer ranges do.
+  int64_t want = ceil_div(max_sel_len, kAttnRange);
   const int64_t cap = ceil_div(512, (int64_t)batch * num_kv_heads);
   if (want > cap) want = cap;
   if (want < 1) want = 1;
-  AttnPlan plan;
-  plan.nsplit = (int)want;
-  plan.mfma = ceil_div(max_sel_len, want) > 16 * kAttnInFlight;
-  // (ranges of the matrix-core kernel are whole multiples of 64 tokens: the last splits
-  // may have nothing left)
-  if (plan.mfma) plan.nsplit = (int)ceil_div(max_sel_len, attn_mfma_chunk(max_sel_len, plan.nsplit));
-  return plan;
-}
-static int attn_splits(int batch, int num_kv_heads, int max_sel_len) {
-  return attn_plan(batch, num_kv_heads, max_sel_len).nsplit;
+  // (ranges are whole multiples of 64 entries: the last splits may have nothing left)
+  return (int)ceil_div(max_sel_len, attn_chunk(max_sel_len, (int)want));
 }
 
 struct AttnWorkspace {
@@ -840,14 +594,12 @@ int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const v
   a.num_heads = cfg->num_heads;
   a.num_kv_heads = cfg->num_kv_heads;
   a.group = cfg->num_heads / cfg->num_kv_heads;
-  a.parts = attn_parts(a.group);
   a.rope_mode = cfg->rope_mode;
   a.log2_theta = cfg->rope_mode == TS_ROPE_LLAMA ? (float)log2((double)cfg->rope_theta) : 0.f;
   a.rope_rcp_scale = cfg->rope_mode == TS_ROPE_LLAMA ? 1.0f / cfg->rope_scale : 1.0f;
   a.sm_scale = cfg->sm_scale;
   a.logit_cap = cfg->logit_cap;
-  const AttnPlan plan = attn_plan(batch, attn_tickets_per_request(cfg), max_sel_len);
-  a.nsplit = plan.nsplit;
+  a.nsplit = attn_splits(batch, attn_tickets_per_request(cfg), max_sel_len);
   a.max_sel_len = max_sel_len;
   a.part_acc = (float*)((char*)workspace + w.acc);
   a.part_ml = (float*)((char*)workspace + w.ml);
@@ -861,27 +613,24 @@ int launch_attn(const ts_config* cfg, const void* q, const void* k_pool, const v
     TS_TRY(check_launch("attn_zero_kernel"));
   }
   const dim3 grid((unsigned)a.nsplit, (unsigned)attn_tickets_per_request(cfg), (unsigned)batch);
-  const int group = attn_heads_per_part(a.group);
   const bool rope = cfg->rope_mode == TS_ROPE_LLAMA, cap = cfg->logit_cap > 0.f;
-#define TS_ATTN_LAUNCH(G_, R_, C_)                                                      \
-  do {                                                                                 \
-    if (plan.mfma)                                                                     \
-      hipLaunchKernelGGL((attn_mfma_kernel<G_, R_, C_>), grid, dim3(256), 0, st, a);   \
-    else                                                                               \
-      hipLaunchKernelGGL((attn_kernel<G_, R_, C_>), grid, dim3(256), 0, st, a);        \
-  } while (0)
-#define TS_ATTN_CASE(G_)                           \
-  case G_:                                         \
-    if (rope && cap) TS_ATTN_LAUNCH(G_, true, true);        \
-    else if (rope) TS_ATTN_LAUNCH(G_, true, false);         \
-    else if (cap) TS_ATTN_LAUNCH(G_, false, true);          \
-    else TS_ATTN_LAUNCH(G_, false, false);                  \
+#define TS_ATTN_LAUNCH(G_, R_, C_) hipLaunchKernelGGL((attn_kernel<G_, R_, C_>), grid, dim3(256), 0, st, a)
+#define TS_ATTN_CASE(G_)                              \
+  case G_:                                            \
+    if (rope && cap) TS_ATTN_LAUNCH(G_, true, true);  \
+    else if (rope) TS_ATTN_LAUNCH(G_, true, false);   \
+    else if (cap) TS_ATTN_LAUNCH(G_, false, true);    \
+    else TS_ATTN_LAUNCH(G_, false, false);            \
     break;
-  switch (group) {
+  switch (a.group) {
     TS_ATTN_CASE(1)
     TS_ATTN_CASE(2)
     TS_ATTN_CASE(3)
     TS_ATTN_CASE(4)
+    TS_ATTN_CASE(5)
+    TS_ATTN_CASE(6)
+    TS_ATTN_CASE(7)
+    TS_ATTN_CASE(8)
     default: return fail(TS_ESHAPE, "unsupported head group %d", a.group);
   }
 #undef TS_ATTN_CASE
@@ -930,11 +679,6 @@ extern "C" {
 size_t ts_attn_workspace_bytes(const ts_config* cfg, int32_t batch, int32_t max_sel_len) {
   if (validate_config(cfg) != TS_OK || batch < 1 || max_sel_len < 1) return 0;
   return attn_workspace(cfg, batch, max_sel_len).total;
-}
-
-int ts_attn_kernel_form(const ts_config* cfg, int32_t batch, int32_t max_sel_len) {
-  if (validate_config(cfg) != TS_OK || batch < 1 || max_sel_len < 1) return -1;
-  return attn_plan(batch, attn_tickets_per_request(cfg), max_sel_len).mfma ? 1 : 0;
 }
 
 int ts_sparse_decode_attn(const ts_config* cfg, const void* q, const void* k_pool,

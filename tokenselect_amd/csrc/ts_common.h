@@ -103,7 +103,7 @@ int launch_rope_selcache(const ts_config* cfg, const ts_batch* bt, const void* q
 // tickets_clear = false makes the launcher clear them first, true says an earlier
 // kernel of the stream already did (attn_tickets() tells it where they are).
 uint32_t* attn_tickets(const ts_config* cfg, int batch, int max_sel_len, void* workspace);
-// Tickets per request (the words to clear): one per workgroup row of the attention's grid.
+// Tickets per request (the words to clear): one per KV head.
 int attn_tickets_per_request(const ts_config* cfg);
 // clear_after: regions that the kernel clears on the side (the counters of the stream's
 // next selection), or NULL.

@@ -585,13 +585,6 @@ def sparse_decode_attention(cfg: LayerConfig, q: torch.Tensor, k_pool: torch.Ten
     return out
 
 
-def attention_kernel_form(cfg: LayerConfig, batch: int, max_sel_len: int) -> int:
-    """Which kernel :func:`sparse_decode_attention` launches for a shape
-    (``ts_attn_kernel_form``): 0 = the fp32 vector kernel (a workgroup reads one batch of
-    rows), 1 = the matrix-core kernel (longer ranges per workgroup)."""
-    return int(_lib.load().ts_attn_kernel_form(ctypes.byref(cfg.to_c()), int(batch), int(max_sel_len)))
-
-
 @dataclass
 class PagePool:
     """Free pages of a paged KV pool (``ts_page_pool``): a stack of physical page
