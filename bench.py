@@ -560,12 +560,12 @@ def bench_model(args, ops, dev):
 
 def extra_workloads(args, ops, workloads, dev):
     """Compact lines for the other configurations, appended to the default run so that one
-    driver-run command measures them all: fewer steps, two pool copies, the oracle on one
+    driver-run command measures them all: fewer steps, the oracle on one
     request (parity only)."""
     import copy
     lines = []
     small = copy.copy(args)
-    small.steps, small.warmup, small.pools = 50, 10, 2
+    small.steps, small.warmup, small.pools = 50, 10, 4
     small.cpu_reps, small.cpu_requests = 1, 1
     for which in ("c1", "c3", "c5"):
         t0 = time.perf_counter()

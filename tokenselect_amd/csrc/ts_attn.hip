@@ -368,8 +368,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // without the requests) says that another tile follows.  Its loads are unconditional:
     // behind a branch the compiler would wait for all loads where the branch joins, the ones
     // just issued included.
-    auto tile = [&](const int j0, auto more_flag) __attribute__((always_inline)) {
+    // `half` (compile-time as well, last tile only): the range ends within the tile's first 16
+    // tokens, and nothing is computed for the other 16.
+    auto tile = [&](const int j0, auto more_flag, auto half_flag) __attribute__((always_inline)) {
       constexpr bool more = decltype(more_flag)::value;
+      constexpr bool half = decltype(half_flag)::value;
+      static_assert(!(more && half), "only a last tile ends early");
       // The slots of the tile after the next are asked for before the next tile's rows, so
       // that waiting for them does not mean waiting for those rows (loads return in order).
       uint32_t slot_after[2] = {0u, 0u};
@@ -379,9 +383,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
       __builtin_amdgcn_sched_barrier(0);
       // ---- keys, 16 tokens at a time: rotate, round, multiply, step the rotation
-      at_f32x4 s[2];
+      at_f32x4 s[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+      for (int t = 0; t < (half ? 1 : 2); ++t) {
         at_bf16x8 ka[4], ka_lo[4];
 #pragma unroll
         for (int kb2 = 0; kb2 < 2; ++kb2) {
@@ -427,7 +431,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 ka[kb], __builtin_bit_cast(at_bf16x8, sm_q[kb][lane + zq]), s[t], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (ROPE) {  // the same rows of the next 16 tokens
+        if (ROPE && (more || (t == 0 && !half))) {  // the same rows of the next 16 tokens
 #pragma unroll
           for (int kb2 = 0; kb2 < 2; ++kb2) {
             const int zs = opaque_zero(__float_as_uint(kc[8 * kb2]));
@@ -458,6 +462,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
+          if (half && t == 1) {
+            p[4 + r] = -INFINITY;
+            continue;
+          }
           float v;
           if (CAP)
             v = a.logit_cap * tanhf(s[t][r] * a.sm_scale / a.logit_cap) * kAttnLog2e;
@@ -475,7 +483,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       float sum = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        p[i] = __builtin_amdgcn_exp2f(p[i] - mn);
+        p[i] = half && i >= 4 ? 0.f : __builtin_amdgcn_exp2f(p[i] - mn);
         sum += p[i];
       }
       l = l * alpha + sum;
@@ -498,8 +506,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           const at_f32x4 zero = {0.f, 0.f, 0.f, 0.f};
           const at_f32x4 d0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
               __builtin_bit_cast(at_bf16x8, vr[0][c]), pick[h], zero, 0, 0, 0);
-          const at_f32x4 d1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              __builtin_bit_cast(at_bf16x8, vr[1][c]), pick[h], zero, 0, 0, 0);
+          const at_f32x4 d1 = half ? zero
+                                   : __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                         __builtin_bit_cast(at_bf16x8, vr[1][c]), pick[h], zero, 0, 0, 0);
           const float vt[8] = {d0[0], d0[1], d0[2], d0[3], d1[0], d1[1], d1[2], d1[3]};
           const at_bf16x8 vta = pack8(vt);
           acc[2 * c + h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vta, pb, acc[2 * c + h], 0, 0, 0);
@@ -517,8 +526,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // a CU in the kernel above, evens them out here too and gains nothing: the rows arrive
     // as fast as the memory system delivers them either way.)
     int j0 = wlo;
-    for (; j0 + kAttnTile < whi; j0 += kAttnTile) tile(j0, std::true_type{});
-    tile(j0, std::false_type{});
+    for (; j0 + kAttnTile < whi; j0 += kAttnTile) tile(j0, std::true_type{}, std::false_type{});
+    if (whi - j0 <= kAttnTile / 2)
+      tile(j0, std::false_type{}, std::true_type{});
+    else
+      tile(j0, std::false_type{}, std::false_type{});
   }
 
   l += __shfl_xor(l, 16);
