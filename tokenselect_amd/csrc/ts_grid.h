@@ -128,6 +128,41 @@ __device__ __forceinline__ void grid_arrive(uint32_t* sync, uint32_t round, bool
   __syncthreads();
 }
 
+// Arrival at the rounds first..last (at most 64 of them) at once, waiting for none: for a
+// workgroup that is through with its rendezvous while others of the launch still need
+// rounds.  Lane r counts the workgroup in for round first + r, so the rounds cost one chain of
+// two dependent read-modify-writes instead of one chain each.  A later round may complete
+// before an earlier one does (the counts of different rounds interleave); that is
+// harmless, since whoever arrives at a later round has published all it ever will, and a
+// waiter of round r may proceed as soon as any round >= r is complete.
+__device__ __forceinline__ void grid_arrive_rest(uint32_t* sync, uint32_t first, uint32_t last,
+                                                 uint32_t workgroups, uint32_t index) {
+  if (first > last) return;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    const uint32_t round = first + threadIdx.x;
+    uint32_t completes = 0;
+    if (round <= last) {
+      uint32_t groups = 1;
+      while (groups * groups < workgroups && groups < (uint32_t)kSyncSlots) ++groups;
+      const uint32_t group = index % groups;
+      const uint32_t members = workgroups / groups + (group < workgroups % groups ? 1u : 0u);
+      if (__hip_atomic_fetch_add(&sync[(size_t)(group + 1) * kSyncSlotWords + 1 + round], 1u,
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == members)
+        completes = __hip_atomic_fetch_add(&sync[1 + round], 1u, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT) + 1 == groups ? 1u : 0u;
+    }
+    const uint64_t which = __ballot(completes != 0u);
+    if (which) {  // the highest round this workgroup completed, raised in every replica
+      static_assert(kSyncSlots == 64, "one replica per lane");
+      const uint32_t highest = first + 63u - (uint32_t)__builtin_clzll(which);
+      __hip_atomic_fetch_max(&sync[(size_t)(threadIdx.x + 1) * kSyncSlotWords], highest,
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
 // One lane waits until the 64-bit word at `p` is no longer zero and returns it; 0 when
 // the wait ran into its bound (the fault word is then set) or another one did.  SLEEP
 // spaces the polls (in units of 64 clocks): a wait that begins while other workgroups

@@ -1399,8 +1399,8 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     // spans them all: whoever is through counts itself in for the rounds it skipped.
     if (team.size != (uint32_t)req_chunks) {  // other requests select in this launch as well
       const uint32_t rounds = kSelectRounds + (a.pool_kernel > 0 ? 1u : 0u);
-      while (round < rounds)
-        grid_arrive(lp.sync, ++round, false, a.spin_ticks, team.size, team.index);
+      grid_arrive_rest(lp.sync, round + 1, rounds, team.size, team.index);
+      round = rounds;
     }
     if (!listed) {
       // Counts of the workgroups before this one.
