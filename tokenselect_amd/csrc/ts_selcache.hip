@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void selcache_kernel(SelCacheArgs a) {
   for (int j = 0; j < kMaxVec; ++j) {
     const int i = threadIdx.x + 256 * j;
     qv[j] = i < pieces ? ((const uint4*)q)[i] : make_uint4(0u, 0u, 0u, 0u);
-    cv[j] = (have && i < pieces) ? ((const uint4*)qc)[i] : make_uint4(0u, 0u, 0u, 0u);
+    cv[j] = i < pieces ? ((const uint4*)qc)[i] : make_uint4(0u, 0u, 0u, 0u);  // (valid or not: see `have`)
   }
   float dot = 0.f, nq = 0.f, nc = 0.f;
 #pragma unroll
@@ -132,8 +132,10 @@ __global__ __launch_bounds__(256) void rope_selcache_kernel(const uint16_t* __re
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
     lo_raw[j] = live ? *(const uint4*)(q + at) : zero4;
     hi_raw[j] = live ? *(const uint4*)(q + at + 64) : zero4;
-    clo[j] = (live && have) ? *(const uint4*)(qc + at) : zero4;
-    chi[j] = (live && have) ? *(const uint4*)(qc + at + 64) : zero4;
+    // (the cached query is asked for whether or not the entry is valid: waiting for the
+    // request's length and the cache's state first would be a round trip of its own)
+    clo[j] = live ? *(const uint4*)(qc + at) : zero4;
+    chi[j] = live ? *(const uint4*)(qc + at + 64) : zero4;
 #pragma unroll
     for (int v = 0; v < 2; ++v) {
       c_lo[j][v] = *(const float4*)(cos_row + d0 + 4 * v);

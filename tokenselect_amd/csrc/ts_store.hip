@@ -18,10 +18,22 @@ __global__ __launch_bounds__(256) void kv_store_kernel(const uint4* __restrict__
                                                        int32_t* __restrict__ seq_lens,
                                                        int row_vec, int max_tokens) {
   const int b = blockIdx.x;
+  // The new rows are asked for together with the slot and the length, not after them: the
+  // kernel is two memory round trips long instead of three.
+  const int first = threadIdx.x;
+  uint4 k0 = make_uint4(0u, 0u, 0u, 0u), v0 = k0;
+  if (first < row_vec) {
+    k0 = k[(size_t)b * row_vec + first];
+    v0 = v[(size_t)b * row_vec + first];
+  }
   const int slot = loc[b];
   const int len = seq_lens[b];
   if (slot < 0 || slot >= pool_rows || len >= max_tokens) return;
-  for (int i = threadIdx.x; i < row_vec; i += blockDim.x) {
+  if (first < row_vec) {
+    k_pool[(size_t)slot * row_vec + first] = k0;
+    v_pool[(size_t)slot * row_vec + first] = v0;
+  }
+  for (int i = first + blockDim.x; i < row_vec; i += blockDim.x) {
     k_pool[(size_t)slot * row_vec + i] = k[(size_t)b * row_vec + i];
     v_pool[(size_t)slot * row_vec + i] = v[(size_t)b * row_vec + i];
   }
@@ -96,6 +108,13 @@ __global__ __launch_bounds__(256) void kv_store_paged_kernel(
     int32_t* seq_lens, int batch, int row_vec, int max_tokens, int page_shift, PagePool pool) {
   __shared__ uint32_t plan_slot, plan_ok;
   const int b = blockIdx.x, lane = threadIdx.x & 63;
+  // (the new rows are asked for before the plan is made, not after)
+  const int first = threadIdx.x;
+  uint4 k0 = make_uint4(0u, 0u, 0u, 0u), v0 = k0;
+  if (first < row_vec) {
+    k0 = k[(size_t)b * row_vec + first];
+    v0 = v[(size_t)b * row_vec + first];
+  }
   if (threadIdx.x < 64)
     for_each_append(seq_lens, table, table_stride, batch, pool, page_shift, max_tokens, pool_rows,
                     lane, [&](int req, const AppendPlan& p) {
@@ -107,7 +126,11 @@ __global__ __launch_bounds__(256) void kv_store_paged_kernel(
   __syncthreads();
   if (plan_ok) {
     const size_t slot = plan_slot;
-    for (int i = threadIdx.x; i < row_vec; i += blockDim.x) {
+    if (first < row_vec) {
+      k_pool[slot * row_vec + first] = k0;
+      v_pool[slot * row_vec + first] = v0;
+    }
+    for (int i = first + blockDim.x; i < row_vec; i += blockDim.x) {
       k_pool[slot * row_vec + i] = k[(size_t)b * row_vec + i];
       v_pool[slot * row_vec + i] = v[(size_t)b * row_vec + i];
     }
