@@ -228,7 +228,6 @@ __device__ __forceinline__ int opaque_zero(uint32_t after) {
 
 template <int G, bool ROPE, bool CAP>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_kernel(AttnArgs a) {
-  constexpr bool SPLIT = true;  // (false: single bf16 operands, for measurements)
   static_assert(G >= 1 && G <= 8, "the query heads of a KV head are columns of one tile");
   attn_clear_on_the_side(a);
   const int split = blockIdx.x, b = blockIdx.z, kvh = blockIdx.y;
@@ -244,7 +243,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // What every wavefront reads again and again lives in LDS, not in registers (the loop
   // below needs them all): the query operand, the 0/1 matrices, the rotation of one step.
   __shared__ __attribute__((aligned(16))) uint4 sm_q[4][64];     // B operand per 32 dims, per lane
-  __shared__ __attribute__((aligned(16))) uint4 sm_q_lo[SPLIT ? 4 : 1][64];  // its low halves
+  __shared__ __attribute__((aligned(16))) uint4 sm_q_lo[4][64];  // its low halves
   __shared__ __attribute__((aligned(16))) uint4 sm_pick[2][64];  // B operand per half, per lane
   __shared__ __attribute__((aligned(16))) float2 sm_step[kHeadDim / 2];  // (cos, sin) of 16 tokens
   __shared__ float sm_acc[4][G][kHeadDim];
@@ -327,18 +326,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         x[e] = xr;
       }
     }
-    if (SPLIT) {
-      at_bf16x8 hi, lo;
-      split8(x, hi, lo);
-      sm_q[wave][lane] = __builtin_bit_cast(uint4, hi);
-      sm_q_lo[wave][lane] = __builtin_bit_cast(uint4, lo);
-      split8(y, hi, lo);
-      sm_q[wave + 2][lane] = __builtin_bit_cast(uint4, hi);
-      sm_q_lo[SPLIT ? wave + 2 : 0][lane] = __builtin_bit_cast(uint4, lo);
-    } else {
-      sm_q[wave][lane] = __builtin_bit_cast(uint4, pack8(x));
-      sm_q[wave + 2][lane] = __builtin_bit_cast(uint4, pack8(y));
-    }
+    at_bf16x8 hi, lo;
+    split8(x, hi, lo);
+    sm_q[wave][lane] = __builtin_bit_cast(uint4, hi);
+    sm_q_lo[wave][lane] = __builtin_bit_cast(uint4, lo);
+    split8(y, hi, lo);
+    sm_q[wave + 2][lane] = __builtin_bit_cast(uint4, hi);
+    sm_q_lo[wave + 2][lane] = __builtin_bit_cast(uint4, lo);
   }
   // This lane's 16 rotation pairs: dims 32 kb2 + 8 qd + e (kb2 < 2, e < 8) and their partners
   // 64 further on; key state at token wlo + n, 16 tokens per step.
@@ -401,35 +395,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
               x[e] = xr;
             }
           }
-          if (SPLIT) {
-            split8(x, ka[kb2], ka_lo[kb2]);
-            split8(y, ka[kb2 + 2], ka_lo[kb2 + 2]);
-          } else {
-            ka[kb2] = pack8(x);
-            ka[kb2 + 2] = pack8(y);
-          }
+          split8(x, ka[kb2], ka_lo[kb2]);
+          split8(y, ka[kb2 + 2], ka_lo[kb2 + 2]);
         }
         const int zq = opaque_zero(__builtin_bit_cast(uint4, ka[3]).w);
         s[t] = at_f32x4{0.f, 0.f, 0.f, 0.f};
-        if (SPLIT) {
-          // (k_hi + k_lo) (q_hi + q_lo) without the product of the two low halves: three
-          // chains that do not wait for each other, added up at the end.
-          at_f32x4 s_lh = {0.f, 0.f, 0.f, 0.f}, s_hl = {0.f, 0.f, 0.f, 0.f};
+        // (k_hi + k_lo) (q_hi + q_lo) without the product of the two low halves: three
+        // chains that do not wait for each other, added up at the end.
+        at_f32x4 s_lh = {0.f, 0.f, 0.f, 0.f}, s_hl = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int kb = 0; kb < 4; ++kb) {
-            const at_bf16x8 q_hi = __builtin_bit_cast(at_bf16x8, sm_q[kb][lane + zq]);
-            const at_bf16x8 q_lo = __builtin_bit_cast(at_bf16x8, sm_q_lo[SPLIT ? kb : 0][lane + zq]);
-            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kb], q_hi, s[t], 0, 0, 0);
-            s_lh = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka_lo[kb], q_hi, s_lh, 0, 0, 0);
-            s_hl = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kb], q_lo, s_hl, 0, 0, 0);
-          }
-          s[t] += s_lh + s_hl;
-        } else {
-#pragma unroll
-          for (int kb = 0; kb < 4; ++kb)
-            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                ka[kb], __builtin_bit_cast(at_bf16x8, sm_q[kb][lane + zq]), s[t], 0, 0, 0);
+        for (int kb = 0; kb < 4; ++kb) {
+          const at_bf16x8 q_hi = __builtin_bit_cast(at_bf16x8, sm_q[kb][lane + zq]);
+          const at_bf16x8 q_lo = __builtin_bit_cast(at_bf16x8, sm_q_lo[kb][lane + zq]);
+          s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kb], q_hi, s[t], 0, 0, 0);
+          s_lh = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka_lo[kb], q_hi, s_lh, 0, 0, 0);
+          s_hl = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kb], q_lo, s_hl, 0, 0, 0);
         }
+        s[t] += s_lh + s_hl;
         __builtin_amdgcn_sched_barrier(0);
         if (ROPE && (more || (t == 0 && !half))) {  // the same rows of the next 16 tokens
 #pragma unroll
@@ -490,10 +472,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int dt = 0; dt < 8; ++dt) acc[dt] *= alpha;
       at_bf16x8 pb, pb_lo;
-      if (SPLIT)
-        split8(p, pb, pb_lo);
-      else
-        pb = pb_lo = pack8(p);
+      split8(p, pb, pb_lo);
       // ---- values: transpose 16 dims at a time, accumulate
       const int zp = opaque_zero(__builtin_bit_cast(uint4, pb).x);
       at_bf16x8 pick[2];
@@ -512,7 +491,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           const float vt[8] = {d0[0], d0[1], d0[2], d0[3], d1[0], d1[1], d1[2], d1[3]};
           const at_bf16x8 vta = pack8(vt);
           acc[2 * c + h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vta, pb, acc[2 * c + h], 0, 0, 0);
-          if (SPLIT) acc[2 * c + h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vta, pb_lo, acc[2 * c + h], 0, 0, 0);
+          acc[2 * c + h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vta, pb_lo, acc[2 * c + h], 0, 0, 0);
         }
       __builtin_amdgcn_sched_barrier(0);
       if (more) {

@@ -86,8 +86,8 @@ __device__ __forceinline__ void grid_poll(uint32_t* sync, uint32_t round, uint64
   }
 }
 
-// Every participating workgroup arrives exactly once per round; those that need the others' data
-// of that round wait for it to complete.  Each thread first waits for its
+// Every participating workgroup arrives exactly once per round and waits for the round to
+// complete (a workgroup that needs no more rounds arrives at the rest with grid_arrive_rest).  Each thread first waits for its
 // outstanding memory operations (what it published has been performed by then);
 // thread 0 then counts the workgroup in.  Arrivals are counted in two levels,
 // about sqrt(workgroups) groups of as many members: read-modify-writes of one
@@ -100,8 +100,8 @@ __device__ __forceinline__ void grid_poll(uint32_t* sync, uint32_t round, uint64
 // round does not complete within `ticks` of the 100 MHz clock the fault word is
 // set and the workgroup carries on, so the kernel always drains.
 // `workgroups` of the grid take part, this one as number `index` among them.
-__device__ __forceinline__ void grid_arrive(uint32_t* sync, uint32_t round, bool wait,
-                                            uint64_t ticks, uint32_t workgroups, uint32_t index) {
+__device__ __forceinline__ void grid_arrive(uint32_t* sync, uint32_t round, uint64_t ticks,
+                                            uint32_t workgroups, uint32_t index) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (threadIdx.x < 64) {  // the first wavefront; lane 0 counts, all lanes raise the flags
@@ -121,7 +121,7 @@ __device__ __forceinline__ void grid_arrive(uint32_t* sync, uint32_t round, bool
       static_assert(kSyncSlots == 64, "one replica per lane");
       __hip_atomic_fetch_max(&sync[(size_t)(threadIdx.x + 1) * kSyncSlotWords], round,
                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    } else if (wait && threadIdx.x == 0) {
+    } else if (threadIdx.x == 0) {
       grid_poll(sync, round, ticks, index);
     }
   }

@@ -889,7 +889,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
                            __HIP_MEMORY_SCOPE_AGENT);
         window[pad + i] = c;
       }
-      grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      grid_arrive(lp.sync, ++round, a.spin_ticks, team.size, team.index);
       for (int hx = tid; hx < halo; hx += 256) {
         const int t = hx < pad ? block_lo - pad + hx : block_lo + count + (hx - pad);
         const int at = hx < pad ? hx : count + hx;
@@ -1026,7 +1026,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       await(done);
     }
     TS_MARK(7);
-    grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
+    grid_arrive(lp.sync, ++round, a.spin_ticks, team.size, team.index);
     TS_MARK(8);
     uint32_t t0 = 0, above0 = 0, in_bin0 = 0;
     // With a hint: the band's small histogram, the flags, the counts of the workgroups before
@@ -1169,7 +1169,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
                                    base + tid < count && key_bin0(key) == t0, key_bin1(key), lane);
       }
       await(done);
-      grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      grid_arrive(lp.sync, ++round, a.spin_ticks, team.size, team.index);
       {
         uint32_t h[kTopkBins / 256];
 #pragma unroll
@@ -1265,7 +1265,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       __syncthreads();
       if (tid == 0) store_coherent(&counts[chunk], scratch[8], 0u);
       TS_MARK(10);
-      grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      grid_arrive(lp.sync, ++round, a.spin_ticks, team.size, team.index);
       TS_MARK(11);
 
       // Every workgroup ranks the list on its own, one entry per thread, in the order
@@ -1358,7 +1358,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
         }
         await(done);
       }
-      grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      grid_arrive(lp.sync, ++round, a.spin_ticks, team.size, team.index);
       {
         uint32_t h[4];
 #pragma unroll
@@ -1393,7 +1393,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       }
       __syncthreads();
       if (tid == 0) store_coherent(&counts[chunk], scratch[8], scratch[9]);
-      grid_arrive(lp.sync, ++round, true, a.spin_ticks, team.size, team.index);
+      grid_arrive(lp.sync, ++round, a.spin_ticks, team.size, team.index);
     }
     // The requests of a batch may need different numbers of rounds, and the rendezvous
     // spans them all: whoever is through counts itself in for the rounds it skipped.
