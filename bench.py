@@ -603,7 +603,7 @@ def extra_workloads(args, ops, workloads, dev):
                   "tflops": r["roofline"]["achieved"], "frac": r["roofline"]["frac"],
                   "parity": r.get("parity"), "wall_s": round(time.perf_counter() - t0, 1)})
     torch.cuda.empty_cache()
-    # The whole 32-layer decoder (BASELINE.json configs[4]) over 32 greedy steps.
+    # The whole 32-layer decoder (the reference's full-model configuration) over 32 greedy steps.
     t0 = time.perf_counter()
     small.steps, small.warmup = 32, 2
     r = bench_model(small, ops, dev)

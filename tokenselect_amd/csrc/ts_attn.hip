@@ -107,46 +107,65 @@ __device__ __forceinline__ void attn_finish(const AttnArgs& a, int b, int kvh, i
   // lane s the weight of its split, so that the accumulators, all requested at once, are
   // added up with weights that are ready (read lane by lane): no chain of dependent
   // exponentials, and one statistics load per wave instead of one per split and thread.
+  // With more than four head slots a wavefront has two of them, and works on both at once:
+  // one after the other they would be two chains of loads.
   static_assert(kHeadDim / 2 == 64, "one wavefront per head slot");
-  for (int idx = tid; idx < G * (kHeadDim / 2); idx += 256) {
-    const int g = idx / (kHeadDim / 2), d = (idx % (kHeadDim / 2)) * 2;
-    const size_t ph = ((size_t)b * H + head_of_slot(g)) * a.nsplit;
-    float mm = kNegBig, ll = 0.f, o0 = 0.f, o1 = 0.f;
-    for (int s0 = 0; s0 < a.nsplit; s0 += 32) {
-      // 32 splits at a time, branch-free: loads past the last split repeat it and get
-      // the weight zero.
-      float2 ac[32];
+  constexpr int SLOTS = (G + 3) / 4;  // head slots per wavefront: wave, wave + 4
+  const int wave_id = tid >> 6, d = lane * 2;
+  size_t ph[SLOTS];
+  float mm[SLOTS], ll[SLOTS], o0[SLOTS], o1[SLOTS];
+#pragma unroll
+  for (int it = 0; it < SLOTS; ++it) {
+    // (a slot past the last head repeats the last one and is not written)
+    ph[it] = ((size_t)b * H + head_of_slot(min(wave_id + 4 * it, G - 1))) * a.nsplit;
+    mm[it] = kNegBig;
+    ll[it] = o0[it] = o1[it] = 0.f;
+  }
+  for (int s0 = 0; s0 < a.nsplit; s0 += 32) {
+    // 32 splits at a time, branch-free: loads past the last split repeat it and get
+    // the weight zero.
+    float2 ac[SLOTS][32], ml[SLOTS];
+#pragma unroll
+    for (int it = 0; it < SLOTS; ++it) {
 #pragma unroll
       for (int i = 0; i < 32; ++i)
-        ac[i] = load_coherent2(a.part_acc + (ph + min(s0 + i, a.nsplit - 1)) * kHeadDim + d);
-      const float2 ml = (lane < 32 && s0 + lane < a.nsplit)
-                            ? load_coherent2(a.part_ml + (ph + s0 + lane) * 2)
-                            : make_float2(kNegBig, 0.f);
-      float mx = ml.x;
+        ac[it][i] = load_coherent2(a.part_acc + (ph[it] + min(s0 + i, a.nsplit - 1)) * kHeadDim + d);
+      ml[it] = (lane < 32 && s0 + lane < a.nsplit) ? load_coherent2(a.part_ml + (ph[it] + s0 + lane) * 2)
+                                                   : make_float2(kNegBig, 0.f);
+    }
+#pragma unroll
+    for (int it = 0; it < SLOTS; ++it) {
+      float mx = ml[it].x;
       mx = fmaxf(mx, dpp_move<kRowRor8>(mx));
       mx = fmaxf(mx, dpp_move<kRowRor4>(mx));
       mx = fmaxf(mx, dpp_move<kRowRor2>(mx));
       mx = fmaxf(mx, dpp_move<kRowRor1>(mx));
       mx = fmaxf(mx, __shfl_xor(mx, 16));
-      const float mn = fmaxf(mm, __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(mx))));
-      const float keep = __expf(mm - mn);  // what earlier batches hold
-      const float w = (lane < 32 && s0 + lane < a.nsplit) ? __expf(ml.x - mn) : 0.f;
-      const float wl = ml.y * w;
-      o0 *= keep;
-      o1 *= keep;
-      ll *= keep;
-      mm = mn;
+      const float mn = fmaxf(mm[it], __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(mx))));
+      const float keep = __expf(mm[it] - mn);  // what earlier batches hold
+      const float w = (lane < 32 && s0 + lane < a.nsplit) ? __expf(ml[it].x - mn) : 0.f;
+      const float wl = ml[it].y * w;
+      o0[it] *= keep;
+      o1[it] *= keep;
+      ll[it] *= keep;
+      mm[it] = mn;
 #pragma unroll
       for (int i = 0; i < 32; ++i) {
         const float wi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), i));
-        ll += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wl), i));
-        o0 += ac[i].x * wi;
-        o1 += ac[i].y * wi;
+        ll[it] += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wl), i));
+        o0[it] += ac[it][i].x * wi;
+        o1[it] += ac[it][i].y * wi;
       }
     }
-    const uint32_t packed = (uint32_t)f32_to_bf16(ll > 0.f ? o0 / ll : 0.f) |
-                            ((uint32_t)f32_to_bf16(ll > 0.f ? o1 / ll : 0.f) << 16);
-    *(uint32_t*)(a.out + ((size_t)b * H + head_of_slot(g)) * kHeadDim + d) = packed;
+  }
+#pragma unroll
+  for (int it = 0; it < SLOTS; ++it) {
+    const int g = wave_id + 4 * it;
+    if (g < G) {
+      const uint32_t packed = (uint32_t)f32_to_bf16(ll[it] > 0.f ? o0[it] / ll[it] : 0.f) |
+                              ((uint32_t)f32_to_bf16(ll[it] > 0.f ? o1[it] / ll[it] : 0.f) << 16);
+      *(uint32_t*)(a.out + ((size_t)b * H + head_of_slot(g)) * kHeadDim + d) = packed;
+    }
   }
   if (tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }

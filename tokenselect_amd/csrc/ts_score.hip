@@ -976,7 +976,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     __syncthreads();
 
     TS_MARK(6);
-    // Round 3: top 11 key bits.  The workgroups add their local histograms to one
+    // First level: top 11 key bits.  The workgroups add their local histograms to one
     // of the copies and note the highest occupied bin; afterwards each searches
     // downwards from that bin, 256 bins at a time (one is enough unless the votes
     // span more than 64 binades).
@@ -1161,7 +1161,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
     uint32_t need = k - above0, in_bin = in_bin0, prefix = t0;
     int shift = 21;
     if (in_bin > (uint32_t)kSelListCap) {
-      // Round 4: next 11 bits of the candidates inside bin t0.
+      // Second level: next 11 bits of the candidates inside bin t0.
       uint32_t done = 0;
       for (int base = 0; base < count; base += 256) {
         const uint32_t key = base + tid < count ? key_of(base + tid) : 0u;
@@ -1346,7 +1346,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       pos_thr = scratch[12];
       TS_MARK(12);
     } else {
-      // Round 5: last 10 bits of the candidates inside (t0, t1).
+      // Third level: last 10 bits of the candidates inside (t0, t1).
       const uint32_t t1 = prefix & 2047u;
       {
         uint32_t done = 0;
@@ -1372,7 +1372,7 @@ __global__ __launch_bounds__(256, (G > 4 ? 1 : 2)) void score_kernel(ScoreArgs a
       need_eq = need - above2;  // ties at the k-th key still to take
       kth = (t0 << 21) | (t1 << 10) | t2;
 
-      // Round 6: every workgroup publishes how many of its tokens lie above the k-th
+      // Count step: every workgroup publishes how many of its tokens lie above the k-th
       // key and how many tie with it; ties are taken lowest position first, so the
       // counts of the workgroups before this one fix where its output starts and
       // how many of its ties still fit.
