@@ -44,13 +44,13 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # Each figure carries the commit of the kernels it was measured on: a later change to the
 # kernel makes it stale until the two counter runs are repeated.
 MEASURED_TRAFFIC = {  # workload -> (bytes per launch of its dominant kernel, commit); profiles/decode_layer_hbm_traffic.txt
-    "C2": (269827098, "2e6a801"),        # ts_select, score_kernel<8,4,false,2>
-    "C3": (2230278193, "2e6a801"),       # the votes-only launch, score_kernel<8,4,false,3>
-    "C5-layer": (2154603199, "2e6a801"),  # likewise
-    "MODEL": (2159035248, "2e6a801"),     # likewise, inside the 32-layer decoder (page 1)
+    "C2": (269809597, "4450ee1"),        # ts_select, score_kernel<8,4,false,2>
+    "C3": (2229968665, "4450ee1"),       # the votes-only launch, score_kernel<8,4,false,3>
+    "C5-layer": (2154816489, "4450ee1"),  # likewise
+    "MODEL": (2158891701, "4450ee1"),     # likewise, inside the 32-layer decoder (page 1)
 }
 # attn_kernel<4>, same runs
-MEASURED_ATTN_TRAFFIC = {"C2": 12249277, "C3": 180841370, "C5-layer": 82184748}
+MEASURED_ATTN_TRAFFIC = {"C2": 12260317, "C3": 180834543, "C5-layer": 82181000}
 
 
 def event_time_us(fn, launches: int, warmup: int, before=None, burst: int = 1):
