@@ -563,7 +563,10 @@ def extra_workloads(args, ops, workloads, dev):
     driver-run command measures them all: fewer steps, the oracle on one
     request (parity only)."""
     import copy
+    import gc
     lines = []
+    gc.collect()
+    torch.cuda.empty_cache()  # the main workload's pools go back to the device first
     small = copy.copy(args)
     small.steps, small.warmup, small.pools = 50, 10, 4
     small.cpu_reps, small.cpu_requests = 1, 1
