@@ -295,9 +295,9 @@ def bench_trace(args, ops, workloads, dev):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for t in range(steps):
-            ops.kv_store(c, k_new[t], v_new[t], None if pages else free[t], wl.k_pool, wl.v_pool, table,
-                         seq, pages=pages)
-            layer(qs[t], wl.k_pool, wl.v_pool, ops.Batch(seq, table, L0 + t + 1, hint=hint), cache)
+            # store + layer in one call, as the reference's decode forward does both
+            layer.step(qs[t], k_new[t], v_new[t], None if pages else free[t], wl.k_pool, wl.v_pool,
+                       ops.Batch(seq, table, L0 + t + 1, hint=hint), cache, pages=pages)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps * 1e6, cache
 

@@ -387,6 +387,30 @@ int ts_kv_store(const ts_config* cfg, const void* k, const void* v, const int32_
                 int32_t* table, int64_t table_stride, int32_t* seq_lens, int32_t batch,
                 int32_t max_tokens, ts_stream_t stream);
 
+/* The reference's decode forward of a layer in one call
+ * (patched_radix_attention_decode_forward_flashinfer, tr.py:777-825): the new token's
+ * K/V stored and appended as ts_kv_store does it (kv: its k, v, out_cache_loc, pages
+ * and max_tokens; the table and the lengths are bt's, which the call therefore
+ * writes), then ts_decode_layer on the lengths after the append (bt->max_seq_len and
+ * host_seq_lens bound those).  Results are those of the two calls.  With a selection
+ * cache and slots chosen by the caller (pages == NULL, page_size 1) the store rides
+ * in the layer's first launch, the rotation and cache decision, and a step is four
+ * kernels instead of five; otherwise the two calls follow each other.  With
+ * bt->rerun the step's token has been appended by the call that gave up, and only
+ * the layer runs. */
+typedef struct ts_new_kv {
+  const void* k;                 /* [batch, Hkv, D] bf16 */
+  const void* v;
+  const int32_t* out_cache_loc;  /* [batch] slots, or NULL with pages */
+  const ts_page_pool* pages;     /* or NULL */
+  int32_t max_tokens;            /* as for ts_kv_store */
+} ts_new_kv;
+int ts_decode_step(const ts_config* cfg, const ts_batch* bt, const ts_new_kv* kv, const void* q,
+                   const float* q_cos, const float* q_sin, void* k_pool, void* v_pool,
+                   int64_t pool_rows, const ts_selcache* cache, void* out, int32_t* sel,
+                   int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
+                   size_t workspace_bytes, ts_stream_t stream);
+
 /* The QKV projection of a decode step with the KV store as its epilogue: what the
  * serving stack does in two places, qkv = x W^T (+ bias) in the model's attention
  * module and then patched_radix_attention_store_kv_cache (tr.py:844-854) +

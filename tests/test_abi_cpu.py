@@ -54,6 +54,7 @@ def test_struct_layouts_match_the_header():
     assert _lib.TsBatch.fault.offset == 40 and _lib.TsBatch.host_seq_lens.offset == 48
     assert _lib.TsBatch.seq_lens.offset == 8 and _lib.TsBatch.table_stride.offset == 24
     assert ctypes.sizeof(_lib.TsSelCache) == 4 * 8 + 8
+    assert ctypes.sizeof(_lib.TsNewKv) == 4 * 8 + 8 and _lib.TsNewKv.max_tokens.offset == 32
 
 
 def test_config_validation(lib):
@@ -223,9 +224,10 @@ def test_header_is_plain_c_and_agrees_with_the_ctypes_mirror(tmp_path):
     src.write_text(
         '#include <stddef.h>\n#include <stdio.h>\n#include "tokenselect.h"\n'
         'int main(void) {\n'
-        '  printf("%zu %zu %zu %zu %zu %zu %zu\\n", sizeof(ts_config), sizeof(ts_batch), sizeof(ts_selcache),\n'
+        '  printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu\\n", sizeof(ts_config), sizeof(ts_batch), sizeof(ts_selcache),\n'
         '         offsetof(ts_batch, threshold_hint), offsetof(ts_batch, wait_us),\n'
-        '         offsetof(ts_batch, workspace_clean), offsetof(ts_batch, host_seq_lens));\n'
+        '         offsetof(ts_batch, workspace_clean), offsetof(ts_batch, host_seq_lens),\n'
+        '         sizeof(ts_new_kv), offsetof(ts_new_kv, max_tokens));\n'
         '  return 0;\n}\n')
     exe = tmp_path / "layout"
     include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
@@ -234,4 +236,5 @@ def test_header_is_plain_c_and_agrees_with_the_ctypes_mirror(tmp_path):
     got = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
     assert got == [ctypes.sizeof(_lib.TsConfig), ctypes.sizeof(_lib.TsBatch), ctypes.sizeof(_lib.TsSelCache),
                    _lib.TsBatch.threshold_hint.offset, _lib.TsBatch.wait_us.offset,
-                   _lib.TsBatch.workspace_clean.offset, _lib.TsBatch.host_seq_lens.offset]
+                   _lib.TsBatch.workspace_clean.offset, _lib.TsBatch.host_seq_lens.offset,
+                   ctypes.sizeof(_lib.TsNewKv), _lib.TsNewKv.max_tokens.offset]

@@ -931,6 +931,69 @@ def test_layer_starts_with_the_selection_on_a_clean_workspace(dev, shape, lens):
         assert torch.equal(got[0].view(torch.int16), want[0].view(torch.int16)), f"step {step}: output"
 
 
+@pytest.mark.parametrize("shape", SHAPES[:3], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("mode", ["cache", "plain", "paged"])
+def test_decode_step_is_store_then_layer(dev, shape, mode):
+    """ts_decode_step (the reference's decode forward in one call, tr.py:777-825) against
+    ts_kv_store followed by ts_decode_layer over a few steps of AR(1) queries: pools,
+    tables, lengths, selections, outputs and the cache's counters bit-identical.  With the
+    selection cache and caller-chosen slots the store rides in the layer's first launch;
+    without the cache, or with a page pool, the call is the two calls in a row.  A request
+    whose table is full is left untouched by both."""
+    import dataclasses
+    page = 16 if mode == "paged" else 1
+    lens, steps = [3000, 700, 2047], 5
+    say(f"decode_step H={shape['num_heads']} kv={shape['num_kv_heads']} mode={mode}")
+    wl = small(dev, shape, seed=81, lens=lens, ks=[64] * len(lens), page=page, extra_pages=len(lens) * (steps + 2))
+    c, B = wl.cfg, len(lens)
+    gen = torch.Generator(device=dev).manual_seed(82)
+    qs = workloads.ar1_queries(B, c.num_heads * c.head_dim, steps, dev)
+    row = c.num_kv_heads * c.head_dim
+    cols = -(-(max(lens) + steps) // page)
+    cols = max(cols, wl.table.shape[1])
+    results = []
+    for fused in (True, False):
+        k_pool, v_pool = wl.k_pool.clone(), wl.v_pool.clone()
+        table = torch.zeros((B, cols), dtype=torch.int32, device=dev)
+        table[:, :wl.table.shape[1]] = wl.table
+        if mode != "paged":
+            table = table[:, :max(lens) + 3].contiguous()   # the longest request's table fills up at step 3
+        seq = wl.seq_lens_dev.clone()
+        cache = ops.SelectionCache.allocate(c, B, dev) if mode == "cache" else None
+        pages = ops.PagePool.of(wl.free_pages.clone()) if mode == "paged" else None
+        free = wl.free_pages[:B * steps].view(steps, B) if mode != "paged" else None
+        layer = ops.DecodeLayer(c, B, max(lens) + steps, dev)
+        g2 = torch.Generator(device=dev).manual_seed(83)
+        trace = []
+        for t in range(steps):
+            k_new = torch.randn((B, row), generator=g2, device=dev).bfloat16()
+            v_new = torch.randn((B, row), generator=g2, device=dev).bfloat16()
+            bt = ops.Batch(seq, table, min(max(lens) + t + 1, table.shape[1] * page))
+            loc = None if pages else free[t].contiguous()
+            if fused:
+                got = layer.step(qs[t], k_new, v_new, loc, k_pool, v_pool, bt, cache, pages=pages)
+            else:
+                ops.kv_store(c, k_new, v_new, loc, k_pool, v_pool, table, seq, pages=pages)
+                got = layer(qs[t], k_pool, v_pool, bt, cache)
+            torch.cuda.synchronize()
+            assert not layer.gave_up()
+            trace.append([x.clone() for x in got] + [seq.clone(), table.clone()])
+        results.append((trace, k_pool, v_pool, None if cache is None else cache.counters.clone()))
+    (ta, ka, va, ca), (tb, kb, vb, cb) = results
+    assert torch.equal(ka, kb) and torch.equal(va, vb)
+    if ca is not None:
+        assert torch.equal(ca, cb)
+    for t, (x, y) in enumerate(zip(ta, tb)):
+        assert torch.equal(x[4], y[4]) and torch.equal(x[5], y[5]), f"step {t}: lengths / table"
+        assert torch.equal(x[3], y[3]), f"step {t}: selection lengths"
+        for b in range(B):
+            S = int(x[3][b])
+            assert torch.equal(x[1][b, :S], y[1][b, :S]) and torch.equal(x[2][b, :S], y[2][b, :S]), f"step {t} b={b}"
+        assert torch.equal(x[0].view(torch.int16), y[0].view(torch.int16)), f"step {t}: output"
+    if mode != "paged":   # the first request's table was full from step 3 on: its length stayed
+        assert int(ta[-1][4][0]) == max(lens) + 3
+
+
 def check_layer(wl, dev, tag):
     lens = wl.seq_lens
     layer = ops.DecodeLayer(wl.cfg, len(lens), max(lens), dev)

@@ -52,8 +52,14 @@ class TsPagePool(ctypes.Structure):
     _fields_ = [("free_pages", _ptr), ("free_count", _ptr), ("ticket", _ptr)]
 
 
+class TsNewKv(ctypes.Structure):
+    _fields_ = [("k", _ptr), ("v", _ptr), ("out_cache_loc", _ptr), ("pages", ctypes.POINTER(TsPagePool)),
+                ("max_tokens", _i32)]
+
+
 _CFG, _BT, _SC = ctypes.POINTER(TsConfig), ctypes.POINTER(TsBatch), ctypes.POINTER(TsSelCache)
 _PP = ctypes.POINTER(TsPagePool)
+_KV = ctypes.POINTER(TsNewKv)
 
 # name -> (restype, argtypes); mirrors include/tokenselect.h one to one.
 SIGNATURES = {
@@ -109,6 +115,8 @@ SIGNATURES = {
                                       _ptr, _i64, _ptr, _ptr, _size, _ptr]),
     "ts_decode_layer": (_i32, [_CFG, _BT, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _SC, _ptr, _ptr,
                                _ptr, _i64, _ptr, _ptr, _size, _ptr]),
+    "ts_decode_step": (_i32, [_CFG, _BT, _KV, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _SC, _ptr, _ptr,
+                              _ptr, _i64, _ptr, _ptr, _size, _ptr]),
 }
 
 _lib = None

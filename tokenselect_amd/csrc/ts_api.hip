@@ -196,12 +196,14 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
                      const void* k_pool, const void* v_pool, int64_t pool_rows,
                      const ts_selcache* cache, void* out, int32_t* sel, int32_t* sel_pos,
                      int64_t sel_stride, int32_t* sel_len, void* workspace, size_t workspace_bytes,
-                     ts_stream_t stream) {
+                     ts_stream_t stream, const StepStore* store = nullptr) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
   SeparateKernelsScope separate(bt->separate_kernels != 0);
   TS_REQUIRE(q && q_cos && q_sin && k_pool && v_pool && out && sel && sel_pos && sel_len, TS_EINVAL,
              "layer: NULL tensor argument");
+  TS_REQUIRE(store == nullptr || (cache != nullptr && chunk_rows == 0), TS_EINVAL,
+             "internal: a store rides in the rotation + cache decision launch only");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);
@@ -264,7 +266,7 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
                               (hipStream_t)stream));
   } else if (cache) {  // rotation and cache decision in one launch
     TS_TRY(launch_rope_selcache(cfg, bt, q, qf, q_cos, q_sin, cache, hit, bt->rerun ? sel_len : nullptr,
-                                zero, (hipStream_t)stream));
+                                zero, (hipStream_t)stream, store));
   } else {
     TS_TRY(launch_rope(q, qf, q_cos, q_sin, nullptr, 1, bt->batch, cfg->num_heads, cfg->head_dim,
                        zero, (hipStream_t)stream));
@@ -313,6 +315,59 @@ int ts_decode_layer(const ts_config* cfg, const ts_batch* bt, const void* q, con
                     size_t workspace_bytes, ts_stream_t stream) {
   return run_layer(cfg, bt, q, 0, q_cos, q_sin, 1, k_pool, v_pool, pool_rows, cache, out, sel,
                    sel_pos, sel_stride, sel_len, workspace, workspace_bytes, stream);
+}
+
+// The reference's decode forward in one call (tr.py:777-825): store_kv_cache + add_k_cache,
+// then selection and attention.  With a selection cache and slots chosen by the caller the
+// store rides in the layer's first launch (the rotation and the cache decision, whose
+// workgroup of a request stores that request's rows first); otherwise the two calls follow
+// each other.
+int ts_decode_step(const ts_config* cfg, const ts_batch* bt, const ts_new_kv* kv, const void* q,
+                   const float* q_cos, const float* q_sin, void* k_pool, void* v_pool,
+                   int64_t pool_rows, const ts_selcache* cache, void* out, int32_t* sel,
+                   int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
+                   size_t workspace_bytes, ts_stream_t stream) {
+  TS_REQUIRE(bt != nullptr && kv != nullptr, TS_EINVAL, "ts_decode_step: NULL batch / new K,V");
+  TS_REQUIRE(bt->table != nullptr && bt->seq_lens != nullptr, TS_EINVAL, "ts_decode_step: NULL table / seq_lens");
+  int32_t* table = const_cast<int32_t*>(bt->table);
+  int32_t* seq_lens = const_cast<int32_t*>(bt->seq_lens);
+  // (a call that repeats a step after a give-up does not append again: it is the layer alone)
+  const bool rides = cache != nullptr && kv->pages == nullptr && bt->rerun == 0;
+  if (!rides) {
+    if (bt->rerun == 0)
+      TS_TRY(ts_kv_store(cfg, kv->k, kv->v, kv->out_cache_loc, kv->pages, k_pool, v_pool, pool_rows, table,
+                         bt->table_stride, seq_lens, bt->batch, kv->max_tokens, stream));
+    return run_layer(cfg, bt, q, 0, q_cos, q_sin, 1, k_pool, v_pool, pool_rows, cache, out, sel, sel_pos,
+                     sel_stride, sel_len, workspace, workspace_bytes, stream);
+  }
+  // The checks ts_kv_store makes.
+  TS_TRY(validate_config(cfg));
+  TS_REQUIRE(kv->k && kv->v && kv->out_cache_loc && k_pool && v_pool, TS_EINVAL,
+             "ts_decode_step: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(kv->k, 16, "k");
+  TS_REQUIRE_ALIGNED(kv->v, 16, "v");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
+  TS_REQUIRE(cfg->page_size == 1, TS_EINVAL, "ts_decode_step: pages of %d tokens need a page pool", cfg->page_size);
+  TS_REQUIRE(bt->batch >= 1 && pool_rows >= 1 && pool_rows <= 0x7fffffffLL && kv->max_tokens >= 1, TS_EINVAL,
+             "ts_decode_step: batch=%d pool_rows=%lld max_tokens=%d out of range", bt->batch,
+             (long long)pool_rows, kv->max_tokens);
+  TS_REQUIRE(bt->batch == 1 || bt->table_stride >= kv->max_tokens, TS_EINVAL,
+             "ts_decode_step: table_stride %lld < max_tokens %d", (long long)bt->table_stride, kv->max_tokens);
+  StepStore st;
+  st.k = (const uint4*)kv->k;
+  st.v = (const uint4*)kv->v;
+  st.loc = kv->out_cache_loc;
+  st.k_pool = (uint4*)k_pool;
+  st.v_pool = (uint4*)v_pool;
+  st.pool_rows = pool_rows;
+  st.table = table;
+  st.table_stride = bt->table_stride;
+  st.seq_lens = seq_lens;
+  st.row_vec = cfg->num_kv_heads * cfg->head_dim * 2 / 16;
+  st.max_tokens = kv->max_tokens;
+  return run_layer(cfg, bt, q, 0, q_cos, q_sin, 1, k_pool, v_pool, pool_rows, cache, out, sel, sel_pos,
+                   sel_stride, sel_len, workspace, workspace_bytes, stream, &st);
 }
 
 // The layer split at the vote, for tensor parallelism (tr.py:361-364): every rank scores

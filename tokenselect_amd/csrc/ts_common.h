@@ -94,9 +94,25 @@ int launch_selcache(const ts_config* cfg, const ts_batch* bt, const void* qf, co
 // The fingerprint rotation of a decode step (one query row per request, q_cos / q_sin the
 // [D] table rows of its position) and the cache decision in one launch, which also clears
 // the regions of `zero`.
+// The new token's K/V rows of a decode step, stored by the first launch of the layer (as
+// kv_store_kernel stores them): slots chosen by the caller, one per request.
+struct StepStore {
+  const uint4* k;  // [B, Hkv*D] bf16 as 16-byte pieces
+  const uint4* v;
+  const int32_t* loc;
+  uint4* k_pool;
+  uint4* v_pool;
+  int64_t pool_rows;
+  int32_t* table;
+  int64_t table_stride;
+  int32_t* seq_lens;
+  int row_vec;     // 16-byte pieces per row
+  int max_tokens;
+};
 int launch_rope_selcache(const ts_config* cfg, const ts_batch* bt, const void* q, void* qf,
                          const float* q_cos, const float* q_sin, const ts_selcache* cache, int32_t* hit,
-                         const int32_t* gave_up_len, const ZeroSet& zero, hipStream_t stream);
+                         const int32_t* gave_up_len, const ZeroSet& zero, hipStream_t stream,
+                         const StepStore* store = nullptr);
 
 // Sparse decode attention (ts_attn.hip).  The kernel counts its workgroups in per
 // (request, KV head) tickets inside the workspace, which must be zero at launch:

@@ -107,7 +107,8 @@ __global__ __launch_bounds__(256) void rope_selcache_kernel(const uint16_t* __re
                                                            uint16_t* __restrict__ qf_out,
                                                            const float* __restrict__ cos_row,
                                                            const float* __restrict__ sin_row,
-                                                           SelCacheArgs a, int batch, ZeroSet zero) {
+                                                           SelCacheArgs a, int batch, ZeroSet zero,
+                                                           StepStore st) {
 #pragma clang fp contract(off)
   const int b = blockIdx.x;
   if (b >= batch) {  // the clearing is the other workgroups' job: the decision is a chain of its own
@@ -116,7 +117,53 @@ __global__ __launch_bounds__(256) void rope_selcache_kernel(const uint16_t* __re
   }
   constexpr int kMaxUnits = kSelCacheMaxVec / 2;
   const int units = a.dim >> 4;  // (heads x 8)
-  const ReqGeom geo = request_geometry(a.seq_lens, a.k_per_req, b, a.n_init, a.n_local, a.top_k, a.max_seq_len);
+  // With a token to store (st.k): this workgroup stores request b's rows and appends the slot
+  // exactly as kv_store_kernel does, and decides with the length after the append, which it
+  // knows without reading it back.
+  // (One thread reads the length and hands it round: the append below rewrites the word.)
+  __shared__ int len_before;
+  if (threadIdx.x == 0) len_before = a.seq_lens[b];
+  __syncthreads();
+  int len_now = len_before;
+  // The rows are asked for here and written at the kernel's end: a store waits for its data,
+  // and every instruction behind it (the query's loads among them) would wait with it.
+  const int first = threadIdx.x;
+  uint4 k0 = make_uint4(0u, 0u, 0u, 0u), v0 = k0;
+  int store_slot = -1;
+  if (st.k != nullptr) {
+    if (first < st.row_vec) {
+      k0 = st.k[(size_t)b * st.row_vec + first];
+      v0 = st.v[(size_t)b * st.row_vec + first];
+    }
+    const int slot = st.loc[b];
+    if (slot >= 0 && slot < st.pool_rows && len_now < st.max_tokens) {
+      store_slot = slot;
+      if (threadIdx.x == 0) {
+        st.table[(int64_t)b * st.table_stride + len_now] = slot;
+        st.seq_lens[b] = len_now + 1;
+      }
+      len_now += 1;
+    }
+  }
+  auto store_rows = [&]() {
+    if (store_slot < 0) return;
+    if (first < st.row_vec) {
+      st.k_pool[(size_t)store_slot * st.row_vec + first] = k0;
+      st.v_pool[(size_t)store_slot * st.row_vec + first] = v0;
+    }
+    for (int i = first + 256; i < st.row_vec; i += 256) {
+      st.k_pool[(size_t)store_slot * st.row_vec + i] = st.k[(size_t)b * st.row_vec + i];
+      st.v_pool[(size_t)store_slot * st.row_vec + i] = st.v[(size_t)b * st.row_vec + i];
+    }
+  };
+  ReqGeom geo;
+  {
+    geo.seq_len = min(max(len_now, 0), a.max_seq_len);
+    const int kk = a.k_per_req ? a.k_per_req[b] : a.top_k;
+    geo.k = kk < 0 ? 0 : (kk > a.top_k ? a.top_k : kk);
+    geo.dense = (a.n_init + geo.k + a.n_local >= geo.seq_len);
+    geo.n = geo.dense ? 0 : geo.seq_len - a.n_init - a.n_local;
+  }
   const uint16_t* q = x + (size_t)b * a.dim;
   uint16_t* qo = qf_out + (size_t)b * a.dim;
   uint16_t* qc = a.q_cache + (size_t)b * a.dim;
@@ -193,6 +240,7 @@ __global__ __launch_bounds__(256) void rope_selcache_kernel(const uint16_t* __re
   }
   if (geo.dense) {  // tr.py:377-378 returns before the cache is consulted
     if (threadIdx.x == 0) a.hit[b] = 0;
+    store_rows();
     return;
   }
   __shared__ float red[3][4];
@@ -230,6 +278,7 @@ __global__ __launch_bounds__(256) void rope_selcache_kernel(const uint16_t* __re
       a.counters[2 * b + 1] += 1;          // retrieval_count, tr.py:421
     }
   }
+  store_rows();
 }
 
 static int fill_selcache_args(const ts_config* cfg, const ts_batch* bt, const void* qf,
@@ -271,15 +320,18 @@ int launch_selcache(const ts_config* cfg, const ts_batch* bt, const void* qf, co
 
 int launch_rope_selcache(const ts_config* cfg, const ts_batch* bt, const void* q, void* qf,
                          const float* q_cos, const float* q_sin, const ts_selcache* cache, int32_t* hit,
-                         const int32_t* gave_up_len, const ZeroSet& zero, hipStream_t stream) {
+                         const int32_t* gave_up_len, const ZeroSet& zero, hipStream_t stream,
+                         const StepStore* store) {
   SelCacheArgs a;
   TS_TRY(fill_selcache_args(cfg, bt, qf, cache, hit, gave_up_len, &a));
+  StepStore st{};
+  if (store) st = *store;
   TS_REQUIRE(!zero.overflow, TS_EINVAL, "internal: more than %d regions to clear in one launch", kZeroRegions);
   TS_REQUIRE_ALIGNED(q_cos, 16, "q_cos");
   TS_REQUIRE_ALIGNED(q_sin, 16, "q_sin");
   const int64_t blocks = bt->batch + std::max<int64_t>(1, ceil_div(zero.total(), 1024));
   hipLaunchKernelGGL(rope_selcache_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
-                     (const uint16_t*)q, (uint16_t*)qf, q_cos, q_sin, a, bt->batch, zero);
+                     (const uint16_t*)q, (uint16_t*)qf, q_cos, q_sin, a, bt->batch, zero, st);
   return check_launch("rope_selcache_kernel");
 }
 

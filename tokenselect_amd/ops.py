@@ -754,7 +754,32 @@ class DecodeLayer(_GiveUpLatch):
         self.check()
         return self._run(q, k_pool, v_pool, bt, cache, out)
 
-    def _run(self, q, k_pool, v_pool, bt, cache, out, rerun: bool = False):
+    def step(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out_cache_loc: Optional[torch.Tensor],
+             k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch, cache: Optional[SelectionCache] = None,
+             out: Optional[torch.Tensor] = None, pages: Optional["PagePool"] = None):
+        """The reference's decode forward of a layer in one call (tr.py:777-825,
+        ``ts_decode_step``): :func:`kv_store` of the new token's ``k`` / ``v`` into the pools
+        and ``bt.table`` / ``bt.seq_lens`` (both written), then the layer on the lengths after
+        the append, which ``bt.max_seq_len`` and ``bt.host_seq_lens`` must bound.  Same
+        results as the two calls; with a selection cache and caller-chosen slots the store
+        rides in the layer's first launch."""
+        self.check()
+        cfg = self.cfg
+        _need(k, "k", torch.bfloat16)
+        _need(v, "v", torch.bfloat16)
+        loc, pool, _keep = _c_pages(cfg, out_cache_loc, pages)
+        _need(bt.table, "table", torch.int32, 2)
+        B = bt.batch
+        row = cfg.num_kv_heads * cfg.head_dim
+        if k.numel() != B * row or v.numel() != B * row or bt.table.shape[0] != B or \
+                (pages is None and out_cache_loc.shape[0] != B):
+            raise ValueError("k / v / out_cache_loc / table do not match the batch")
+        kv = _lib.TsNewKv(_p(k), _p(v), loc, ctypes.pointer(_keep) if pages is not None else None,
+                          bt.table.shape[1] * cfg.page_size)
+        kv._pool = _keep  # (the struct the pointer refers to lives as long as kv)
+        return self._run(q, k_pool, v_pool, bt, cache, out, new_kv=kv)
+
+    def _run(self, q, k_pool, v_pool, bt, cache, out, rerun: bool = False, new_kv=None):
         cfg = self.cfg
         bt = self._options(bt, rerun)
         shape = (bt.batch, int(bt.max_seq_len))
@@ -779,11 +804,18 @@ class DecodeLayer(_GiveUpLatch):
             _need(out, "out", torch.bfloat16)
             if out.numel() != q.numel():
                 raise ValueError("out must hold B*H*D elements")
-        _lib.check(_lib.load().ts_decode_layer(
-            ctypes.byref(self._c), ctypes.byref(cb), _p(q), _p(self.q_cos), _p(self.q_sin),
-            _p(k_pool), _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, B), _p(out),
-            _p(self.sel), _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
-            self.workspace.numel(), _stream()))
+        if new_kv is not None:
+            _lib.check(_lib.load().ts_decode_step(
+                ctypes.byref(self._c), ctypes.byref(cb), ctypes.byref(new_kv), _p(q), _p(self.q_cos),
+                _p(self.q_sin), _p(k_pool), _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, B), _p(out),
+                _p(self.sel), _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
+                self.workspace.numel(), _stream()))
+        else:
+            _lib.check(_lib.load().ts_decode_layer(
+                ctypes.byref(self._c), ctypes.byref(cb), _p(q), _p(self.q_cos), _p(self.q_sin),
+                _p(k_pool), _p(v_pool), k_pool.shape[0], _c_cache(cache, cfg, B), _p(out),
+                _p(self.sel), _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
+                self.workspace.numel(), _stream()))
         if plain:
             self._clean_for = shape
         return out, self.sel[:B], self.sel_pos[:B], self.sel_len[:B]
