@@ -64,8 +64,8 @@ def _cpu_forward(m: Decoder, tokens, kc, vc, tab, lens, loc, device_sels):
     return norm(x, m.final_norm) @ m.lm_head.cpu().float().T
 
 
-@pytest.mark.parametrize("query_cache,fused_qkv", [(False, True), (False, False), (True, True)],
-                         ids=["plain", "plain-gemm-then-store", "query_cache"])
+@pytest.mark.parametrize("query_cache,fused_qkv", [(False, True), (False, False), (True, True), (True, False)],
+                         ids=["plain", "plain-gemm-then-store", "query_cache", "query_cache-gemm-then-store"])
 def test_decoder_steps_match_the_oracle(dev, query_cache, fused_qkv):
     say(f"toy decoder, query_cache={query_cache} fused_qkv={fused_qkv}")
     mc = ModelConfig(**TOY)

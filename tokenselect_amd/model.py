@@ -151,13 +151,13 @@ class Decoder:
             else:
                 q, k, v = F.linear(h, self.wqkv[l]).split((hd, kvd, kvd), dim=-1)
                 q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-                ops.kv_store(cfg, k, v, loc, self.k_pools[l], self.v_pools[l], self.table,
-                             self.num_tokens[l])
-            attn, sel, _, sel_len = self.attention(
-                q, self.k_pools[l], self.v_pools[l],
-                Batch(self.num_tokens[l], self.table, max_len, host_seq_lens=host_lens, hint=self.hints[l],
-                      **self.layer_options),
-                self.caches[l])
+            bt = Batch(self.num_tokens[l], self.table, max_len, host_seq_lens=host_lens, hint=self.hints[l],
+                       **self.layer_options)
+            if k is None:
+                attn, sel, _, sel_len = self.attention(q, self.k_pools[l], self.v_pools[l], bt, self.caches[l])
+            else:  # the store and the layer in one call, as the reference's decode forward has them
+                attn, sel, _, sel_len = self.attention.step(q, k, v, loc, self.k_pools[l], self.v_pools[l], bt,
+                                                            self.caches[l])
             if trace is not None:
                 if k is None:   # the rows as they landed in the pools
                     k = self.k_pools[l][loc.long()].reshape(self.batch, kvd)
