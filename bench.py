@@ -368,8 +368,8 @@ def bench_prefill(args, ops, workloads, dev):
     def step(i):
         p = i % n_pools
         seqs[p].fill_(L0)          # the chunk is appended afresh every time
-        ops.kv_store_chunk(c, k_new, v_new, loc, k_pools[p], v_pools[p], tables[p][0], seqs[p])
-        return layer(q, k_pools[p], v_pools[p], ops.Batch(seqs[p], tables[p], L0 + m))
+        # store + chunk in one call, as the reference's extend forward has them per chunk
+        return layer.step(q, k_new, v_new, loc, k_pools[p], v_pools[p], ops.Batch(seqs[p], tables[p], L0 + m))
 
     for i in range(args.warmup):
         step(i)

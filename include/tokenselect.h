@@ -489,6 +489,20 @@ int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, in
                      int32_t* sel, int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len,
                      void* workspace, size_t workspace_bytes, ts_stream_t stream);
 
+/* One chunk of the extend forward in one call (tr.py:725-773): ts_kv_store_chunk of the
+ * chunk's K/V (kv: k, v [rows, Hkv, D], out_cache_loc [rows], pages, max_tokens; the
+ * table row and the length word are bt's, which the call therefore writes), then
+ * ts_prefill_chunk on the length after the append (which bt->max_seq_len bounds).
+ * Results are those of the two calls.  With slots chosen by the caller (pages == NULL,
+ * page_size 1) the store rides in the chunk's first launch, the fingerprint, as spare
+ * workgroups; otherwise the two calls follow each other.  With bt->rerun the chunk has been
+ * appended by the call that gave up, and only ts_prefill_chunk runs. */
+int ts_prefill_step(const ts_config* cfg, const ts_batch* bt, const ts_new_kv* kv, const void* q,
+                    int32_t rows, const float* cos_table, const float* sin_table, int64_t table_rows,
+                    void* k_pool, void* v_pool, int64_t pool_rows, void* out, int32_t* sel,
+                    int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
+                    size_t workspace_bytes, ts_stream_t stream);
+
 /* One layer of patched_radix_attention_decode_forward_flashinfer after the KV
  * store (tr.py:791-825): fingerprint (q rotated with q_cos/q_sin, the [D] table
  * rows of position n_local, tr.py:380-388) -> [selection cache] -> score ->

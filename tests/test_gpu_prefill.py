@@ -318,6 +318,57 @@ def test_prefill_chunks(dev, shape, fused):
         ops.set_fused_select(previous)
 
 
+@pytest.mark.parametrize("shape", SHAPES[:3], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("chunk", [64, 500])
+def test_prefill_step_is_store_then_chunk(dev, shape, chunk):
+    """ts_prefill_step (one chunk of the extend forward in one call, tr.py:725-773) against
+    ts_kv_store_chunk followed by ts_prefill_chunk, chunk by chunk (the last one ragged, and
+    the table full before the end, so that rows are dropped): pools, table, length,
+    selections and outputs bit-identical.  The store rides in the fingerprint launch."""
+    L0, T, top_k = 3000, 3 * chunk - 17, 96
+    say(f"prefill step H={shape['num_heads']} L0={L0} T={T} chunk={chunk}")
+    wl = workloads.build("pf", shape, [L0], [top_k], 1, dev, seed=15, n_init=8, n_local=chunk,
+                         top_k=top_k, extra_pages=T)
+    c = wl.cfg
+    g = torch.Generator(device=dev).manual_seed(16)
+    q = torch.randn((T, c.num_heads * 128), generator=g, device=dev).bfloat16()
+    k_new = torch.randn((T, c.num_kv_heads, 128), generator=g, device=dev).bfloat16()
+    v_new = torch.randn((T, c.num_kv_heads, 128), generator=g, device=dev).bfloat16()
+    new_slots = (L0 + torch.randperm(T, generator=g, device=dev)).int()
+    cols = L0 + T - 5                          # the table is full five rows before the end
+    results = []
+    for one_call in (True, False):
+        k_pool, v_pool = wl.k_pool.clone(), wl.v_pool.clone()
+        table = torch.zeros((1, cols), dtype=torch.int32, device=dev)
+        table[0, :L0] = wl.table[0, :L0]
+        seq = wl.seq_lens_dev.clone()
+        layer = ops.PrefillChunk(c, cols, dev, max_rows=chunk)
+        trace, L = [], L0
+        for start in range(0, T, chunk):
+            end = min(start + chunk, T)
+            L = min(L + end - start, cols)
+            bt = ops.Batch(seq, table, L)
+            args = (k_new[start:end].contiguous(), v_new[start:end].contiguous(), new_slots[start:end].contiguous())
+            if one_call:
+                got = layer.step(q[start:end].contiguous(), *args, k_pool, v_pool, bt)
+            else:
+                ops.kv_store_chunk(c, *args, k_pool, v_pool, table[0], seq)
+                got = layer(q[start:end].contiguous(), k_pool, v_pool, bt)
+            torch.cuda.synchronize()
+            assert not layer.gave_up()
+            trace.append([x.clone() for x in got] + [seq.clone(), table.clone()])
+        results.append((trace, k_pool, v_pool))
+    (ta, ka, va), (tb, kb, vb) = results
+    assert torch.equal(ka, kb) and torch.equal(va, vb)
+    assert int(ta[-1][4][0]) == cols
+    for t, (x, y) in enumerate(zip(ta, tb)):
+        assert torch.equal(x[4], y[4]) and torch.equal(x[5], y[5]), f"chunk {t}: length / table"
+        assert torch.equal(x[3], y[3]), f"chunk {t}: selection length"
+        S = int(x[3][0])
+        assert torch.equal(x[1][0, :S], y[1][0, :S]) and torch.equal(x[2][0, :S], y[2][0, :S]), f"chunk {t}"
+        assert torch.equal(x[0].view(torch.int16), y[0].view(torch.int16)), f"chunk {t}: output"
+
+
 def test_prefill_short_context_attends_densely(dev):
     """n_init + k + n_local >= L: the chunk attends over every token so far (tr.py:741-744)."""
     say("prefill chunk, dense context")

@@ -105,6 +105,8 @@ SIGNATURES = {
                                       _size, _ptr]),
     "ts_prefill_chunk": (_i32, [_CFG, _BT, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i64, _ptr, _ptr,
                                 _ptr, _i64, _ptr, _ptr, _size, _ptr]),
+    "ts_prefill_step": (_i32, [_CFG, _BT, _KV, _ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _i64, _ptr, _ptr,
+                               _ptr, _i64, _ptr, _ptr, _size, _ptr]),
     "ts_set_fused_select": (_i32, [_i32]),
     "ts_decode_layer_selection": (_i32, [_CFG, _i32, _i32]),
     "ts_decode_layer_selection_of": (_i32, [_CFG, _BT]),

@@ -196,7 +196,8 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
                      const void* k_pool, const void* v_pool, int64_t pool_rows,
                      const ts_selcache* cache, void* out, int32_t* sel, int32_t* sel_pos,
                      int64_t sel_stride, int32_t* sel_len, void* workspace, size_t workspace_bytes,
-                     ts_stream_t stream, const StepStore* store = nullptr) {
+                     ts_stream_t stream, const StepStore* store = nullptr,
+                     const ChunkStore* chunk_store = nullptr) {
   TS_TRY(validate_config(cfg));
   TS_TRY(validate_batch(cfg, bt));
   SeparateKernelsScope separate(bt->separate_kernels != 0);
@@ -204,6 +205,8 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
              "layer: NULL tensor argument");
   TS_REQUIRE(store == nullptr || (cache != nullptr && chunk_rows == 0), TS_EINVAL,
              "internal: a store rides in the rotation + cache decision launch only");
+  TS_REQUIRE(chunk_store == nullptr || chunk_rows > 0, TS_EINVAL,
+             "internal: a chunk's store rides in the fingerprint launch only");
   TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL, TS_EINVAL, "pool_rows %lld out of range",
              (long long)pool_rows);
   LayerWorkspace w = layer_workspace(cfg, bt->batch, bt->max_seq_len);
@@ -263,7 +266,7 @@ static int run_layer(const ts_config* cfg, const ts_batch* bt, const void* q, in
   } else if (chunk_rows > 0) {
     // Chunk fingerprint: row i rotated to n_local + i, mean over the rows (tr.py:380-392).
     TS_TRY(launch_fingerprint(cfg, q, chunk_rows, q_cos, q_sin, table_rows, qf, zero,
-                              (hipStream_t)stream));
+                              (hipStream_t)stream, chunk_store));
   } else if (cache) {  // rotation and cache decision in one launch
     TS_TRY(launch_rope_selcache(cfg, bt, q, qf, q_cos, q_sin, cache, hit, bt->rerun ? sel_len : nullptr,
                                 zero, (hipStream_t)stream, store));
@@ -481,6 +484,56 @@ int ts_prefill_chunk(const ts_config* cfg, const ts_batch* bt, const void* q, in
   return run_layer(cfg, bt, q, rows, cos_table, sin_table, table_rows, k_pool, v_pool, pool_rows,
                    nullptr, out, sel, sel_pos, sel_stride, sel_len, workspace, workspace_bytes,
                    stream);
+}
+
+// One chunk of the reference's extend forward in one call (tr.py:725-773): the chunk's K/V
+// stored and appended (ts_kv_store_chunk), then ts_prefill_chunk.  With slots chosen by the
+// caller the store rides in the chunk's first launch, the fingerprint, as spare workgroups.
+int ts_prefill_step(const ts_config* cfg, const ts_batch* bt, const ts_new_kv* kv, const void* q,
+                    int32_t rows, const float* cos_table, const float* sin_table, int64_t table_rows,
+                    void* k_pool, void* v_pool, int64_t pool_rows, void* out, int32_t* sel,
+                    int32_t* sel_pos, int64_t sel_stride, int32_t* sel_len, void* workspace,
+                    size_t workspace_bytes, ts_stream_t stream) {
+  TS_REQUIRE(bt != nullptr && bt->batch == 1 && kv != nullptr, TS_EINVAL,
+             "ts_prefill_step serves one request at a time (batch must be 1) and needs the chunk's K/V");
+  TS_REQUIRE(rows >= 1, TS_EINVAL, "ts_prefill_step: rows %d < 1", rows);
+  TS_REQUIRE(bt->table != nullptr && bt->seq_lens != nullptr, TS_EINVAL, "ts_prefill_step: NULL table / seq_lens");
+  int32_t* table = const_cast<int32_t*>(bt->table);
+  int32_t* seq_len = const_cast<int32_t*>(bt->seq_lens);
+  const bool rides = kv->pages == nullptr && bt->rerun == 0 && kv->max_tokens <= 0x1fffff &&
+                     rows <= 1023 * 32;
+  if (!rides) {
+    if (bt->rerun == 0)  // (a call that repeats a chunk after a give-up does not append again)
+      TS_TRY(ts_kv_store_chunk(cfg, kv->k, kv->v, kv->out_cache_loc, kv->pages, rows, k_pool, v_pool, pool_rows,
+                               table, seq_len, kv->max_tokens, stream));
+    return run_layer(cfg, bt, q, rows, cos_table, sin_table, table_rows, k_pool, v_pool, pool_rows, nullptr,
+                     out, sel, sel_pos, sel_stride, sel_len, workspace, workspace_bytes, stream);
+  }
+  // The checks ts_kv_store_chunk makes.
+  TS_TRY(validate_config(cfg));
+  TS_REQUIRE(kv->k && kv->v && kv->out_cache_loc && k_pool && v_pool, TS_EINVAL,
+             "ts_prefill_step: NULL tensor argument");
+  TS_REQUIRE_ALIGNED(kv->k, 16, "k");
+  TS_REQUIRE_ALIGNED(kv->v, 16, "v");
+  TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
+  TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
+  TS_REQUIRE(cfg->page_size == 1, TS_EINVAL, "ts_prefill_step: pages of %d tokens need a page pool", cfg->page_size);
+  TS_REQUIRE(pool_rows >= 1 && pool_rows <= 0x7fffffffLL && kv->max_tokens >= 1, TS_EINVAL,
+             "ts_prefill_step: pool_rows=%lld max_tokens=%d out of range", (long long)pool_rows, kv->max_tokens);
+  ChunkStore cs{};
+  cs.k = (const uint4*)kv->k;
+  cs.v = (const uint4*)kv->v;
+  cs.loc = kv->out_cache_loc;
+  cs.k_pool = (uint4*)k_pool;
+  cs.v_pool = (uint4*)v_pool;
+  cs.pool_rows = pool_rows;
+  cs.table = table;
+  cs.seq_len = seq_len;
+  cs.rows = rows;
+  cs.row_vec = cfg->num_kv_heads * cfg->head_dim * 2 / 16;
+  cs.max_tokens = kv->max_tokens;
+  return run_layer(cfg, bt, q, rows, cos_table, sin_table, table_rows, k_pool, v_pool, pool_rows, nullptr,
+                   out, sel, sel_pos, sel_stride, sel_len, workspace, workspace_bytes, stream, nullptr, &cs);
 }
 
 }  // extern "C"

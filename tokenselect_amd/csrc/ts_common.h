@@ -79,9 +79,23 @@ __device__ __forceinline__ void clear_regions(const ZeroSet& zero, int64_t gid, 
 }
 // Chunk fingerprint (ts_prefill.hip) with the same side job as launch_rope: the
 // regions are cleared by the same launch.
+// The K/V rows of a prefill chunk, stored by the fingerprint launch on the side (as
+// kv_store_chunk_kernel stores them): slots chosen by the caller, one per row.
+struct ChunkStore {
+  const uint4* k;  // [rows, Hkv*D] bf16 as 16-byte pieces
+  const uint4* v;
+  const int32_t* loc;
+  uint4* k_pool;
+  uint4* v_pool;
+  int64_t pool_rows;
+  int32_t* table;    // the request's row
+  int32_t* seq_len;  // the request's length word
+  int rows, row_vec, max_tokens;
+  int workgroups;    // of the launch that store (set by the launcher)
+};
 int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
                        const float* sin_table, int64_t table_rows, void* qf, const ZeroSet& zero,
-                       hipStream_t stream);
+                       hipStream_t stream, const ChunkStore* store = nullptr);
 int launch_rope(const void* x, void* out, const float* cos_table, const float* sin_table,
                 const int64_t* position_ids, int64_t table_rows, int64_t rows, int heads, int dim,
                 const ZeroSet& zero, hipStream_t stream);

@@ -7,6 +7,7 @@
 #include <type_traits>
 
 #include "ts_common.h"
+#include "ts_store.h"
 
 namespace ts {
 
@@ -26,7 +27,7 @@ constexpr int kFpSplit = 2;     // workgroups per head
 __global__ __launch_bounds__(1024) void fingerprint_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ qf, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int64_t table_rows, int first_pos, int rows, int heads,
-    ZeroSet zero) {
+    ZeroSet zero, ChunkStore cs) {
 #pragma clang fp contract(off)
   constexpr int half = kHeadDim / 2;
   constexpr int kPairs = half / kFpSplit;   // rotation pairs of this workgroup
@@ -40,6 +41,14 @@ __global__ __launch_bounds__(1024) void fingerprint_kernel(
     const int64_t gid = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 1024 + threadIdx.x;
     const int64_t step = (int64_t)gridDim.x * gridDim.y * 1024;
     clear_regions(zero, gid, step);
+  }
+  // Also on the side: the workgroups past the fingerprint's own store the chunk's K/V
+  // rows (the caller's store of the chunk, which the selection after this launch must find
+  // done, riding here instead of in a launch of its own).
+  if ((int)blockIdx.y >= kFpSplit) {
+    const int wg = ((int)blockIdx.y - kFpSplit) * (int)gridDim.x + (int)blockIdx.x;
+    if (cs.k != nullptr && wg < cs.workgroups) store_chunk_rows<true>(cs, wg, 1024);
+    return;
   }
   float lo_sum[kFpVec] = {0.f, 0.f, 0.f, 0.f}, hi_sum[kFpVec] = {0.f, 0.f, 0.f, 0.f};
   // Four rows per step: their loads are independent and go out together; the sums
@@ -739,7 +748,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const float* cos_table,
                        const float* sin_table, int64_t table_rows, void* qf, const ZeroSet& zero,
-                       hipStream_t stream) {
+                       hipStream_t stream, const ChunkStore* store) {
   TS_TRY(validate_config(cfg));
   TS_REQUIRE(!zero.overflow, TS_EINVAL, "internal: more than %d regions to clear in one launch", kZeroRegions);
   TS_REQUIRE(q && cos_table && sin_table && qf, TS_EINVAL, "ts_fingerprint: NULL tensor argument");
@@ -750,9 +759,18 @@ int launch_fingerprint(const ts_config* cfg, const void* q, int32_t rows, const 
   TS_REQUIRE(table_rows >= (int64_t)cfg->n_local + rows, TS_EINVAL,
              "ts_fingerprint: cos/sin tables have %lld rows, need n_local + rows = %lld",
              (long long)table_rows, (long long)cfg->n_local + rows);
-  hipLaunchKernelGGL(fingerprint_kernel, dim3((unsigned)cfg->num_heads, kFpSplit), dim3(1024), 0, stream,
+  ChunkStore cs{};
+  unsigned grid_y = kFpSplit;
+  if (store) {  // rows of 32 threads: 32 rows per workgroup of 1024
+    cs = *store;
+    cs.workgroups = (int)ceil_div(cs.rows, 1024 / kChunkThreadsPerRow);
+    TS_REQUIRE(cs.workgroups <= kChunkCountedWgs && cs.max_tokens <= kLenMask, TS_EINVAL,
+               "internal: a chunk store of %d rows does not ride in the fingerprint launch", cs.rows);
+    grid_y += (unsigned)ceil_div(cs.workgroups, cfg->num_heads);
+  }
+  hipLaunchKernelGGL(fingerprint_kernel, dim3((unsigned)cfg->num_heads, grid_y), dim3(1024), 0, stream,
                      (const uint16_t*)q, (uint16_t*)qf, cos_table, sin_table, table_rows,
-                     cfg->n_local, rows, cfg->num_heads, zero);
+                     cfg->n_local, rows, cfg->num_heads, zero, cs);
   return check_launch("fingerprint_kernel");
 }
 

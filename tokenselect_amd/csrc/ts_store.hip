@@ -1,6 +1,7 @@
 // KV store and token-table append for a decode step
 // (patched_radix_attention_store_kv_cache tr.py:844-854, add_k_cache tr.py:332-336).
 #include "ts_pages.h"
+#include "ts_store.h"
 
 namespace ts {
 
@@ -44,52 +45,17 @@ __global__ __launch_bounds__(256) void kv_store_kernel(const uint4* __restrict__
   }
 }
 
-// Chunked prefill (tr.py:725-733): a workgroup copies kChunkRowsPerWg rows of the chunk
-// (row r to pool slot loc[r]) and writes table[len + r] for them.  Every workgroup must read the same old
-// length, and the new one must be there when the launch ends: the workgroups count
-// themselves in the upper bits of the length word itself (a length stays below 2^21,
-// the count below 2^10), everybody masks those bits off, and the workgroup that
-// completes the count writes the new length.  No second launch, no other memory.
-// Rows that would not fit the table are dropped; slots are clamped to the pool.
-constexpr int kLenBits = 21;
-constexpr int kLenMask = (1 << kLenBits) - 1;
-constexpr int kChunkRowsPerWg = 8;        // 32 threads per row: few workgroups, few counts on one word
-constexpr int kChunkCountedWgs = 1023;    // more workgroups take the two-launch form below
+// Chunked prefill (tr.py:725-733): ts_store.h has the counted form's body, which the
+// fingerprint launch of a chunk can also run on the side.
+constexpr int kChunkRowsPerWg = 256 / kChunkThreadsPerRow;  // few workgroups, few counts on one word
 
 template <bool COUNTED>
 __global__ __launch_bounds__(256) void kv_store_chunk_kernel(
     const uint4* __restrict__ k, const uint4* __restrict__ v, const int32_t* __restrict__ loc,
     uint4* __restrict__ k_pool, uint4* __restrict__ v_pool, int64_t pool_rows,
     int32_t* __restrict__ table, int32_t* seq_len, int rows, int row_vec, int max_tokens) {
-  // Counted: the upper bits may already hold other workgroups' counts.
-  const int len = COUNTED ? (__hip_atomic_load(seq_len, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kLenMask)
-                          : *seq_len;
-  constexpr int kThreadsPerRow = 256 / kChunkRowsPerWg;
-  const int r = blockIdx.x * kChunkRowsPerWg + threadIdx.x / kThreadsPerRow;
-  const int t = threadIdx.x % kThreadsPerRow;
-  const int at = len + r;
-  if (r < rows && at >= 0 && at < max_tokens) {
-    int64_t slot = loc[r];
-    slot = slot < 0 ? 0 : (slot >= pool_rows ? pool_rows - 1 : slot);
-    for (int i = t; i < row_vec; i += kThreadsPerRow) {
-      k_pool[(size_t)slot * row_vec + i] = k[(size_t)r * row_vec + i];
-      v_pool[(size_t)slot * row_vec + i] = v[(size_t)r * row_vec + i];
-    }
-    if (t == 0) table[at] = (int32_t)slot;
-  }
-  if (COUNTED) {
-    // A workgroup counts itself in when all its wavefronts have read the length, at its
-    // end, where nobody waits for the answer; whoever completes the count knows that
-    // every workgroup has read the old length, and writes the new one.
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      const int before = __hip_atomic_fetch_add(seq_len, 1 << kLenBits, __ATOMIC_RELAXED,
-                                                __HIP_MEMORY_SCOPE_AGENT);
-      if ((before >> kLenBits) + 1 == (int)gridDim.x)
-        __hip_atomic_store(seq_len, min(len + rows, max_tokens), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
+  ChunkStore cs{k, v, loc, k_pool, v_pool, pool_rows, table, seq_len, rows, row_vec, max_tokens, (int)gridDim.x};
+  store_chunk_rows<COUNTED>(cs, (int)blockIdx.x, 256);
 }
 
 __global__ void seq_len_add_kernel(int32_t* seq_len, int rows, int max_tokens) {

@@ -984,7 +984,31 @@ class PrefillChunk(_GiveUpLatch):
         self.check()
         return self._run(q, k_pool, v_pool, bt, out)
 
-    def _run(self, q, k_pool, v_pool, bt, out, rerun: bool = False):
+    def step(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out_cache_loc: Optional[torch.Tensor],
+             k_pool: torch.Tensor, v_pool: torch.Tensor, bt: Batch, out: Optional[torch.Tensor] = None,
+             pages: Optional["PagePool"] = None):
+        """One chunk of the extend forward in one call (tr.py:725-773, ``ts_prefill_step``):
+        :func:`kv_store_chunk` of the chunk's ``k`` / ``v`` into the pools and ``bt.table`` /
+        ``bt.seq_lens`` (both written), then the chunk on the length after the append, which
+        ``bt.max_seq_len`` must bound.  Same results as the two calls; with caller-chosen
+        slots the store rides in the chunk's first launch."""
+        self.check()
+        cfg = self.cfg
+        _need(k, "k", torch.bfloat16)
+        _need(v, "v", torch.bfloat16)
+        loc, pool, _keep = _c_pages(cfg, out_cache_loc, pages)
+        _need(bt.table, "table", torch.int32, 2)
+        row = cfg.num_kv_heads * cfg.head_dim
+        rows = q.shape[0]
+        if k.numel() != rows * row or v.numel() != rows * row or bt.table.shape[0] != 1 or \
+                (pages is None and out_cache_loc.shape[0] != rows):
+            raise ValueError("k / v / out_cache_loc / table do not match the chunk")
+        kv = _lib.TsNewKv(_p(k), _p(v), loc, ctypes.pointer(_keep) if pages is not None else None,
+                          bt.table.shape[1] * cfg.page_size)
+        kv._pool = _keep
+        return self._run(q, k_pool, v_pool, bt, out, new_kv=kv)
+
+    def _run(self, q, k_pool, v_pool, bt, out, rerun: bool = False, new_kv=None):
         cfg = self.cfg
         bt = self._options(bt, rerun)
         cb = _c_batch(cfg, bt)
@@ -1002,11 +1026,18 @@ class PrefillChunk(_GiveUpLatch):
             _need(out, "out", torch.bfloat16)
             if out.numel() != q.numel():
                 raise ValueError("out must hold rows*H*D elements")
-        _lib.check(_lib.load().ts_prefill_chunk(
-            ctypes.byref(self._c), ctypes.byref(cb), _p(q), rows, _p(self.cos), _p(self.sin),
-            self.cos.shape[0], _p(k_pool), _p(v_pool), k_pool.shape[0], _p(out), _p(self.sel),
-            _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
-            self.workspace.numel(), _stream()))
+        if new_kv is not None:
+            _lib.check(_lib.load().ts_prefill_step(
+                ctypes.byref(self._c), ctypes.byref(cb), ctypes.byref(new_kv), _p(q), rows, _p(self.cos),
+                _p(self.sin), self.cos.shape[0], _p(k_pool), _p(v_pool), k_pool.shape[0], _p(out),
+                _p(self.sel), _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
+                self.workspace.numel(), _stream()))
+        else:
+            _lib.check(_lib.load().ts_prefill_chunk(
+                ctypes.byref(self._c), ctypes.byref(cb), _p(q), rows, _p(self.cos), _p(self.sin),
+                self.cos.shape[0], _p(k_pool), _p(v_pool), k_pool.shape[0], _p(out), _p(self.sel),
+                _p(self.sel_pos), cfg.max_sel, _p(self.sel_len), _p(self.workspace),
+                self.workspace.numel(), _stream()))
         return out, self.sel, self.sel_pos, self.sel_len
 
 
