@@ -933,7 +933,8 @@ def test_layer_starts_with_the_selection_on_a_clean_workspace(dev, shape, lens):
 
 @pytest.mark.parametrize("shape", SHAPES[:3], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
 @pytest.mark.parametrize("mode", ["cache", "plain", "paged"])
-def test_decode_step_is_store_then_layer(dev, shape, mode):
+@pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
+def test_decode_step_is_store_then_layer(dev, shape, mode, fused_select):
     """ts_decode_step (the reference's decode forward in one call, tr.py:777-825) against
     ts_kv_store followed by ts_decode_layer over a few steps of AR(1) queries: pools,
     tables, lengths, selections, outputs and the cache's counters bit-identical.  With the
