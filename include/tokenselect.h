@@ -393,9 +393,9 @@ int ts_kv_store(const ts_config* cfg, const void* k, const void* v, const int32_
  * and max_tokens; the table and the lengths are bt's, which the call therefore
  * writes), then ts_decode_layer on the lengths after the append (bt->max_seq_len and
  * host_seq_lens bound those).  Results are those of the two calls.  With a selection
- * cache and slots chosen by the caller (pages == NULL, page_size 1) the store rides
- * in the layer's first launch, the rotation and cache decision, and a step is four
- * kernels instead of five; otherwise the two calls follow each other.  With
+ * cache the store rides in the layer's first launch, the rotation and cache decision
+ * (slots chosen by the caller or taken from a page pool alike), and a step is three
+ * kernels instead of four; otherwise the two calls follow each other.  With
  * bt->rerun the step's token has been appended by the call that gave up, and only
  * the layer runs. */
 typedef struct ts_new_kv {

@@ -932,17 +932,20 @@ def test_layer_starts_with_the_selection_on_a_clean_workspace(dev, shape, lens):
 
 
 @pytest.mark.parametrize("shape", SHAPES[:3], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
-@pytest.mark.parametrize("mode", ["cache", "plain", "paged"])
+@pytest.mark.parametrize("mode", ["cache", "plain", "paged", "paged-cache"])
 @pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
 def test_decode_step_is_store_then_layer(dev, shape, mode, fused_select):
     """ts_decode_step (the reference's decode forward in one call, tr.py:777-825) against
     ts_kv_store followed by ts_decode_layer over a few steps of AR(1) queries: pools,
     tables, lengths, selections, outputs and the cache's counters bit-identical.  With the
     selection cache and caller-chosen slots the store rides in the layer's first launch;
-    without the cache, or with a page pool, the call is the two calls in a row.  A request
-    whose table is full is left untouched by both."""
+    with a page pool the slots come from the table and the pool as the paged store takes them
+    (2047 and 3000 tokens: one request on a page boundary at the third step, one at the first);
+    without the cache the call is the two calls in a row.  A request whose table is full is left
+    untouched by both."""
     import dataclasses
-    page = 16 if mode == "paged" else 1
+    paged = mode.startswith("paged")
+    page = 16 if paged else 1
     lens, steps = [3000, 700, 2047], 5
     say(f"decode_step H={shape['num_heads']} kv={shape['num_kv_heads']} mode={mode}")
     wl = small(dev, shape, seed=81, lens=lens, ks=[64] * len(lens), page=page, extra_pages=len(lens) * (steps + 2))
@@ -957,12 +960,12 @@ def test_decode_step_is_store_then_layer(dev, shape, mode, fused_select):
         k_pool, v_pool = wl.k_pool.clone(), wl.v_pool.clone()
         table = torch.zeros((B, cols), dtype=torch.int32, device=dev)
         table[:, :wl.table.shape[1]] = wl.table
-        if mode != "paged":
+        if not paged:
             table = table[:, :max(lens) + 3].contiguous()   # the longest request's table fills up at step 3
         seq = wl.seq_lens_dev.clone()
-        cache = ops.SelectionCache.allocate(c, B, dev) if mode == "cache" else None
-        pages = ops.PagePool.of(wl.free_pages.clone()) if mode == "paged" else None
-        free = wl.free_pages[:B * steps].view(steps, B) if mode != "paged" else None
+        cache = ops.SelectionCache.allocate(c, B, dev) if mode.endswith("cache") else None
+        pages = ops.PagePool.of(wl.free_pages.clone()) if paged else None
+        free = wl.free_pages[:B * steps].view(steps, B) if not paged else None
         layer = ops.DecodeLayer(c, B, max(lens) + steps, dev)
         g2 = torch.Generator(device=dev).manual_seed(83)
         trace = []
@@ -979,8 +982,10 @@ def test_decode_step_is_store_then_layer(dev, shape, mode, fused_select):
             torch.cuda.synchronize()
             assert not layer.gave_up()
             trace.append([x.clone() for x in got] + [seq.clone(), table.clone()])
-        results.append((trace, k_pool, v_pool, None if cache is None else cache.counters.clone()))
-    (ta, ka, va, ca), (tb, kb, vb, cb) = results
+        results.append((trace, k_pool, v_pool, None if cache is None else cache.counters.clone(),
+                        None if pages is None else (int(pages.free_count), int(pages.ticket))))
+    (ta, ka, va, ca, pa), (tb, kb, vb, cb, pb) = results
+    assert pa == pb and (pa is None or pa[1] == 0)
     assert torch.equal(ka, kb) and torch.equal(va, vb)
     if ca is not None:
         assert torch.equal(ca, cb)
@@ -991,7 +996,7 @@ def test_decode_step_is_store_then_layer(dev, shape, mode, fused_select):
             S = int(x[3][b])
             assert torch.equal(x[1][b, :S], y[1][b, :S]) and torch.equal(x[2][b, :S], y[2][b, :S]), f"step {t} b={b}"
         assert torch.equal(x[0].view(torch.int16), y[0].view(torch.int16)), f"step {t}: output"
-    if mode != "paged":   # the first request's table was full from step 3 on: its length stayed
+    if not paged:   # the first request's table was full from step 3 on: its length stayed
         assert int(ta[-1][4][0]) == max(lens) + 3
 
 

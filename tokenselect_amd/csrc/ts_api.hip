@@ -335,7 +335,7 @@ int ts_decode_step(const ts_config* cfg, const ts_batch* bt, const ts_new_kv* kv
   int32_t* table = const_cast<int32_t*>(bt->table);
   int32_t* seq_lens = const_cast<int32_t*>(bt->seq_lens);
   // (a call that repeats a step after a give-up does not append again: it is the layer alone)
-  const bool rides = cache != nullptr && kv->pages == nullptr && bt->rerun == 0;
+  const bool rides = cache != nullptr && bt->rerun == 0;
   if (!rides) {
     if (bt->rerun == 0)
       TS_TRY(ts_kv_store(cfg, kv->k, kv->v, kv->out_cache_loc, kv->pages, k_pool, v_pool, pool_rows, table,
@@ -345,19 +345,26 @@ int ts_decode_step(const ts_config* cfg, const ts_batch* bt, const ts_new_kv* kv
   }
   // The checks ts_kv_store makes.
   TS_TRY(validate_config(cfg));
-  TS_REQUIRE(kv->k && kv->v && kv->out_cache_loc && k_pool && v_pool, TS_EINVAL,
-             "ts_decode_step: NULL tensor argument");
+  TS_REQUIRE(kv->k && kv->v && k_pool && v_pool, TS_EINVAL, "ts_decode_step: NULL tensor argument");
   TS_REQUIRE_ALIGNED(kv->k, 16, "k");
   TS_REQUIRE_ALIGNED(kv->v, 16, "v");
   TS_REQUIRE_ALIGNED(k_pool, 16, "k_pool");
   TS_REQUIRE_ALIGNED(v_pool, 16, "v_pool");
-  TS_REQUIRE(cfg->page_size == 1, TS_EINVAL, "ts_decode_step: pages of %d tokens need a page pool", cfg->page_size);
+  if (kv->pages) {
+    TS_REQUIRE(kv->pages->free_pages && kv->pages->free_count && kv->pages->ticket, TS_EINVAL,
+               "ts_decode_step: page pool has a NULL array");
+  } else {
+    TS_REQUIRE(cfg->page_size == 1, TS_EINVAL, "ts_decode_step: pages of %d tokens need a page pool",
+               cfg->page_size);
+    TS_REQUIRE(kv->out_cache_loc != nullptr, TS_EINVAL, "ts_decode_step: NULL out_cache_loc and no page pool");
+  }
   TS_REQUIRE(bt->batch >= 1 && pool_rows >= 1 && pool_rows <= 0x7fffffffLL && kv->max_tokens >= 1, TS_EINVAL,
              "ts_decode_step: batch=%d pool_rows=%lld max_tokens=%d out of range", bt->batch,
              (long long)pool_rows, kv->max_tokens);
-  TS_REQUIRE(bt->batch == 1 || bt->table_stride >= kv->max_tokens, TS_EINVAL,
-             "ts_decode_step: table_stride %lld < max_tokens %d", (long long)bt->table_stride, kv->max_tokens);
-  StepStore st;
+  TS_REQUIRE(bt->batch == 1 || bt->table_stride * (int64_t)cfg->page_size >= kv->max_tokens, TS_EINVAL,
+             "ts_decode_step: table_stride %lld x page_size %d < max_tokens %d", (long long)bt->table_stride,
+             cfg->page_size, kv->max_tokens);
+  StepStore st{};
   st.k = (const uint4*)kv->k;
   st.v = (const uint4*)kv->v;
   st.loc = kv->out_cache_loc;
@@ -369,6 +376,12 @@ int ts_decode_step(const ts_config* cfg, const ts_batch* bt, const ts_new_kv* kv
   st.seq_lens = seq_lens;
   st.row_vec = cfg->num_kv_heads * cfg->head_dim * 2 / 16;
   st.max_tokens = kv->max_tokens;
+  if (kv->pages) {
+    st.free_pages = kv->pages->free_pages;
+    st.free_count = kv->pages->free_count;
+    st.ticket = kv->pages->ticket;
+    st.page_shift = page_shift_of(cfg->page_size);
+  }
   return run_layer(cfg, bt, q, 0, q_cos, q_sin, 1, k_pool, v_pool, pool_rows, cache, out, sel, sel_pos,
                    sel_stride, sel_len, workspace, workspace_bytes, stream, &st);
 }

@@ -122,6 +122,12 @@ struct StepStore {
   int32_t* seq_lens;
   int row_vec;     // 16-byte pieces per row
   int max_tokens;
+  // With a page pool (free_pages != NULL; loc is not read): the slots come from the table and
+  // the pool as kv_store_paged_kernel takes them.
+  const int32_t* free_pages;
+  int32_t* free_count;
+  uint32_t* ticket;
+  int page_shift;
 };
 int launch_rope_selcache(const ts_config* cfg, const ts_batch* bt, const void* q, void* qf,
                          const float* q_cos, const float* q_sin, const ts_selcache* cache, int32_t* hit,

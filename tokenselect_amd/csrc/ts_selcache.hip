@@ -5,6 +5,7 @@
 #include <algorithm>
 
 #include "ts_common.h"
+#include "ts_pages.h"
 
 namespace ts {
 
@@ -130,31 +131,54 @@ __global__ __launch_bounds__(256) void rope_selcache_kernel(const uint16_t* __re
   const int first = threadIdx.x;
   uint4 k0 = make_uint4(0u, 0u, 0u, 0u), v0 = k0;
   int store_slot = -1;
+  const bool paged = st.k != nullptr && st.free_pages != nullptr;
+  const PagePool pool{st.free_pages, st.free_count, st.ticket};
   if (st.k != nullptr) {
     if (first < st.row_vec) {
       k0 = st.k[(size_t)b * st.row_vec + first];
       v0 = st.v[(size_t)b * st.row_vec + first];
     }
-    const int slot = st.loc[b];
-    if (slot >= 0 && slot < st.pool_rows && len_now < st.max_tokens) {
-      store_slot = slot;
-      if (threadIdx.x == 0) {
-        st.table[(int64_t)b * st.table_stride + len_now] = slot;
-        st.seq_lens[b] = len_now + 1;
+    if (paged) {
+      // The plan of the whole batch from the snapshot that no workgroup modifies before the
+      // launch's last one commits it (at the end of this kernel); this request's part of it.
+      __shared__ int plan_slot;
+      if (threadIdx.x == 0) plan_slot = -1;
+      __syncthreads();
+      if (threadIdx.x < 64)
+        for_each_append(st.seq_lens, st.table, st.table_stride, batch, pool, st.page_shift, st.max_tokens,
+                        (uint32_t)st.pool_rows, (int)threadIdx.x, [&](int req, const AppendPlan& p) {
+                          if (req == b && p.ok) plan_slot = (int)p.slot;
+                        });
+      __syncthreads();
+      store_slot = plan_slot;
+      if (store_slot >= 0) len_now += 1;
+    } else {
+      const int slot = st.loc[b];
+      if (slot >= 0 && slot < st.pool_rows && len_now < st.max_tokens) {
+        store_slot = slot;
+        if (threadIdx.x == 0) {
+          st.table[(int64_t)b * st.table_stride + len_now] = slot;
+          st.seq_lens[b] = len_now + 1;
+        }
+        len_now += 1;
       }
-      len_now += 1;
     }
   }
   auto store_rows = [&]() {
-    if (store_slot < 0) return;
-    if (first < st.row_vec) {
-      st.k_pool[(size_t)store_slot * st.row_vec + first] = k0;
-      st.v_pool[(size_t)store_slot * st.row_vec + first] = v0;
+    if (store_slot >= 0) {
+      if (first < st.row_vec) {
+        st.k_pool[(size_t)store_slot * st.row_vec + first] = k0;
+        st.v_pool[(size_t)store_slot * st.row_vec + first] = v0;
+      }
+      for (int i = first + 256; i < st.row_vec; i += 256) {
+        st.k_pool[(size_t)store_slot * st.row_vec + i] = st.k[(size_t)b * st.row_vec + i];
+        st.v_pool[(size_t)store_slot * st.row_vec + i] = st.v[(size_t)b * st.row_vec + i];
+      }
     }
-    for (int i = first + 256; i < st.row_vec; i += 256) {
-      st.k_pool[(size_t)store_slot * st.row_vec + i] = st.k[(size_t)b * st.row_vec + i];
-      st.v_pool[(size_t)store_slot * st.row_vec + i] = st.v[(size_t)b * st.row_vec + i];
-    }
+    // (the workgroups of the requests are the launch that stores: the last of them commits)
+    if (paged && threadIdx.x < 64)
+      commit_appends(st.seq_lens, st.table, st.table_stride, batch, pool, st.page_shift, st.max_tokens,
+                     (uint32_t)st.pool_rows, (int)threadIdx.x, (uint32_t)batch);
   };
   ReqGeom geo;
   {

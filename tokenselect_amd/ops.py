@@ -761,8 +761,8 @@ class DecodeLayer(_GiveUpLatch):
         ``ts_decode_step``): :func:`kv_store` of the new token's ``k`` / ``v`` into the pools
         and ``bt.table`` / ``bt.seq_lens`` (both written), then the layer on the lengths after
         the append, which ``bt.max_seq_len`` and ``bt.host_seq_lens`` must bound.  Same
-        results as the two calls; with a selection cache and caller-chosen slots the store
-        rides in the layer's first launch."""
+        results as the two calls; with a selection cache the store rides in the layer's
+        first launch."""
         self.check()
         cfg = self.cfg
         _need(k, "k", torch.bfloat16)
