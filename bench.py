@@ -44,13 +44,13 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # Each figure carries the commit of the kernels it was measured on: a later change to the
 # kernel makes it stale until the two counter runs are repeated.
 MEASURED_TRAFFIC = {  # workload -> (bytes per launch of its dominant kernel, commit); profiles/decode_layer_hbm_traffic.txt
-    "C2": (269791301, "0932e2f"),        # ts_select, score_kernel<8,4,false,2>
-    "C3": (2230243937, "0932e2f"),       # the votes-only launch, score_kernel<8,4,false,3>
-    "C5-layer": (2154586623, "0932e2f"),  # likewise
-    "MODEL": (2159009107, "0932e2f"),     # likewise, inside the 32-layer decoder (page 1)
+    "C2": (269799462, "e5a4a17"),        # ts_select, score_kernel<8,4,false,2>
+    "C3": (2229654966, "e5a4a17"),       # the votes-only launch, score_kernel<8,4,false,3>
+    "C5-layer": (2154403375, "e5a4a17"),  # likewise
+    "MODEL": (2158824315, "e5a4a17"),     # likewise, inside the 32-layer decoder (page 1)
 }
 # attn_kernel<4>, same runs
-MEASURED_ATTN_TRAFFIC = {"C2": 12259748, "C3": 180843808, "C5-layer": 82196263}
+MEASURED_ATTN_TRAFFIC = {"C2": 12261315, "C3": 180831151, "C5-layer": 82185305}
 
 
 def event_time_us(fn, launches: int, warmup: int, before=None, burst: int = 1):
