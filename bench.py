@@ -21,7 +21,9 @@ Prints one JSON line: the per-layer latency, the roofline figures of the
 dominant kernel (algorithmic bytes / HIP-event time of the call that streams the
 keys: ``ts_select``, the whole selection in one kernel, when the batch fits it,
 else ``ts_score``), the same for the stand-alone scoring kernel and the gather
-attention, and the CPU oracle timed on the host cores.
+attention, and the CPU oracle timed on the host cores.  The default run appends a
+compact line for each of the other workloads, every one measured by a child process
+of this script (``--no-extra`` leaves them out).
 """
 
 import argparse
@@ -558,10 +560,24 @@ def bench_model(args, ops, dev):
     return result
 
 
+def _own_process(argv, timeout_s=600):
+    """One workload measured by a child process of this script (the parent exits with its own
+    result afterwards; nothing is replaced): a process of its own gives every workload the device
+    memory as a freshly started server finds it, whatever the workloads before it allocated and
+    freed.  Returns the child's JSON line."""
+    import subprocess
+    res = subprocess.run([sys.executable, os.path.abspath(__file__)] + argv, capture_output=True,
+                         text=True, timeout=timeout_s)
+    if res.returncode != 0:
+        raise RuntimeError(f"bench.py {' '.join(argv)} exited with {res.returncode}: {res.stderr[-400:]}")
+    return json.loads(res.stdout.strip().splitlines()[-1])
+
+
 def extra_workloads(args, ops, workloads, dev):
     """Compact lines for the other configurations, appended to the default run so that one
-    driver-run command measures them all: fewer steps, the oracle on one
-    request (parity only)."""
+    driver-run command measures them all: fewer steps, the oracle on one request (parity
+    only).  Each is measured in a process of its own (see _own_process), or in this one if
+    that process cannot be had."""
     import copy
     import gc
     lines = []
@@ -570,9 +586,21 @@ def extra_workloads(args, ops, workloads, dev):
     small = copy.copy(args)
     small.steps, small.warmup, small.pools = 50, 10, 4
     small.cpu_reps, small.cpu_requests = 1, 1
+    common = ["--pools", "4", "--cpu-reps", "1", "--cpu-requests", "1", "--no-extra"]
+
+    def measured(argv, here):
+        try:
+            return _own_process(argv + common)
+        except Exception as e:  # (no child process to be had: measure here)
+            print(f"bench.py: {e}; measuring in this process", file=sys.stderr, flush=True)
+            r = here()
+            torch.cuda.empty_cache()
+            return r
+
     for which in ("c1", "c3", "c5"):
         t0 = time.perf_counter()
-        r = bench_layer(small, ops, workloads, dev, which)
+        r = measured(["--workload", which, "--steps", "50", "--warmup", "10"],
+                     lambda: bench_layer(small, ops, workloads, dev, which))
         roof = r["roofline"]
         lines.append({
             "workload": r["config"]["workload"], "us_per_layer": r["value"],
@@ -581,35 +609,33 @@ def extra_workloads(args, ops, workloads, dev):
             "traffic": roof["traffic"], "score_only_frac": r["score_only"]["frac"],
             "attn_us": r["gather_attention"]["us_per_launch"], "parity": r.get("parity"),
             "wall_s": round(time.perf_counter() - t0, 1)})
-        torch.cuda.empty_cache()
-    t0 = time.perf_counter()
-    small.steps, small.warmup = 64, 64
-    r = bench_trace(small, ops, workloads, dev)
-    lines.append({"workload": r["config"]["workload"], "us_per_step": r["value"],
-                  "hit_rate": r["hit_rate"], "bytes_per_step": r["roofline"]["bytes_per_step"],
-                  "frac": r["roofline"]["frac"], "wall_s": round(time.perf_counter() - t0, 1)})
-    small.page_size = 16
-    t0 = time.perf_counter()
-    r = bench_trace(small, ops, workloads, dev)
-    lines.append({"workload": r["config"]["workload"], "us_per_step": r["value"],
-                  "hit_rate": r["hit_rate"], "bytes_per_step": r["roofline"]["bytes_per_step"],
-                  "frac": r["roofline"]["frac"], "wall_s": round(time.perf_counter() - t0, 1)})
-    torch.cuda.empty_cache()
+    trace = copy.copy(small)
+    trace.steps, trace.warmup = 64, 64
+    for page in (1, 16):
+        t0 = time.perf_counter()
+        paged = copy.copy(trace)
+        paged.page_size = page
+        r = measured(["--workload", "c4", "--steps", "64", "--warmup", "64", "--page-size", str(page)],
+                     lambda: bench_trace(paged, ops, workloads, dev))
+        lines.append({"workload": r["config"]["workload"], "us_per_step": r["value"],
+                      "hit_rate": r["hit_rate"], "bytes_per_step": r["roofline"]["bytes_per_step"],
+                      "frac": r["roofline"]["frac"], "wall_s": round(time.perf_counter() - t0, 1)})
     # One 512-row chunk of the extend forward on a 128K context.
     t0 = time.perf_counter()
-    small.steps, small.warmup, small.page_size = 50, 10, 1
-    r = bench_prefill(small, ops, workloads, dev)
+    r = measured(["--workload", "prefill", "--steps", "50", "--warmup", "10"],
+                 lambda: bench_prefill(small, ops, workloads, dev))
     lines.append({"workload": r["config"]["workload"], "us_per_chunk": r["value"],
                   "dominant_kernel": "ts::prefill_attn_kernel<G>", "bound": "mfma",
                   "us_per_launch": r["roofline"]["us_per_launch"],
                   "flops_per_launch": r["roofline"]["flops_per_launch"],
                   "tflops": r["roofline"]["achieved"], "frac": r["roofline"]["frac"],
                   "parity": r.get("parity"), "wall_s": round(time.perf_counter() - t0, 1)})
-    torch.cuda.empty_cache()
     # The whole 32-layer decoder (the reference's full-model configuration) over 32 greedy steps.
     t0 = time.perf_counter()
-    small.steps, small.warmup = 32, 2
-    r = bench_model(small, ops, dev)
+    model = copy.copy(small)
+    model.steps, model.warmup = 32, 2
+    r = measured(["--workload", "model", "--steps", "32", "--warmup", "2"],
+                 lambda: bench_model(model, ops, dev))
     lines.append({"workload": r["config"]["workload"], "tokens_per_s": r["value"],
                   "greedy_steps": r["steps"], "ms_per_decode_step": r["ms_per_step"],
                   "us_per_layer": r["us_per_layer"], "hbm_frac_whole_step": r["hbm_frac_whole_step"],
@@ -618,7 +644,6 @@ def extra_workloads(args, ops, workloads, dev):
                   "traffic": r["roofline"]["traffic"],
                   "cpu_tokens_per_s": (r.get("cpu_baseline") or {}).get("value"),
                   "parity": r.get("parity"), "wall_s": round(time.perf_counter() - t0, 1)})
-    torch.cuda.empty_cache()
     return lines
 
 
