@@ -23,7 +23,8 @@ keys: ``ts_select``, the whole selection in one kernel, when the batch fits it,
 else ``ts_score``), the same for the stand-alone scoring kernel and the gather
 attention, and the CPU oracle timed on the host cores.  The default run appends a
 compact line for each of the other workloads, every one measured by a child process
-of this script (``--no-extra`` leaves them out).
+of this script, started before this process touches the GPU (``--no-extra`` leaves
+them out, ``--extra-in-process`` measures them here).
 """
 
 import argparse
@@ -560,90 +561,109 @@ def bench_model(args, ops, dev):
     return result
 
 
-def _own_process(argv, timeout_s=600):
-    """One workload measured by a child process of this script (the parent exits with its own
-    result afterwards; nothing is replaced): a process of its own gives every workload the device
-    memory as a freshly started server finds it, whatever the workloads before it allocated and
-    freed.  Returns the child's JSON line."""
-    import subprocess
-    res = subprocess.run([sys.executable, os.path.abspath(__file__)] + argv, capture_output=True,
-                         text=True, timeout=timeout_s)
-    if res.returncode != 0:
-        raise RuntimeError(f"bench.py {' '.join(argv)} exited with {res.returncode}: {res.stderr[-400:]}")
-    return json.loads(res.stdout.strip().splitlines()[-1])
-
-
-def extra_workloads(args, ops, workloads, dev):
-    """Compact lines for the other configurations, appended to the default run so that one
-    driver-run command measures them all: fewer steps, the oracle on one request (parity
-    only).  Each is measured in a process of its own (see _own_process), or in this one if
-    that process cannot be had."""
-    import copy
-    import gc
-    lines = []
-    gc.collect()
-    torch.cuda.empty_cache()  # the main workload's pools go back to the device first
-    small = copy.copy(args)
-    small.steps, small.warmup, small.pools = 50, 10, 4
-    small.cpu_reps, small.cpu_requests = 1, 1
-    common = ["--pools", "4", "--cpu-reps", "1", "--cpu-requests", "1", "--no-extra"]
-
-    def measured(argv, here):
-        try:
-            return _own_process(argv + common)
-        except Exception as e:  # (no child process to be had: measure here)
-            print(f"bench.py: {e}; measuring in this process", file=sys.stderr, flush=True)
-            r = here()
-            torch.cuda.empty_cache()
-            return r
-
-    for which in ("c1", "c3", "c5"):
-        t0 = time.perf_counter()
-        r = measured(["--workload", which, "--steps", "50", "--warmup", "10"],
-                     lambda: bench_layer(small, ops, workloads, dev, which))
-        roof = r["roofline"]
-        lines.append({
-            "workload": r["config"]["workload"], "us_per_layer": r["value"],
+def _layer_line(r):
+    roof = r["roofline"]
+    return {"workload": r["config"]["workload"], "us_per_layer": r["value"],
             "dominant_kernel": roof["kernel"].split(" ")[0], "us_per_launch": roof["us_per_launch"],
             "bytes_per_launch": roof["bytes_per_launch"], "frac": roof["frac"],
             "traffic": roof["traffic"], "score_only_frac": r["score_only"]["frac"],
-            "attn_us": r["gather_attention"]["us_per_launch"], "parity": r.get("parity"),
-            "wall_s": round(time.perf_counter() - t0, 1)})
-    trace = copy.copy(small)
-    trace.steps, trace.warmup = 64, 64
-    for page in (1, 16):
+            "attn_us": r["gather_attention"]["us_per_launch"], "parity": r.get("parity")}
+
+
+def _trace_line(r):
+    return {"workload": r["config"]["workload"], "us_per_step": r["value"],
+            "hit_rate": r["hit_rate"], "bytes_per_step": r["roofline"]["bytes_per_step"],
+            "frac": r["roofline"]["frac"]}
+
+
+def _prefill_line(r):
+    return {"workload": r["config"]["workload"], "us_per_chunk": r["value"],
+            "dominant_kernel": "ts::prefill_attn_kernel<G>", "bound": "mfma",
+            "us_per_launch": r["roofline"]["us_per_launch"],
+            "flops_per_launch": r["roofline"]["flops_per_launch"],
+            "tflops": r["roofline"]["achieved"], "frac": r["roofline"]["frac"],
+            "parity": r.get("parity")}
+
+
+def _model_line(r):
+    return {"workload": r["config"]["workload"], "tokens_per_s": r["value"],
+            "greedy_steps": r["steps"], "ms_per_decode_step": r["ms_per_step"],
+            "us_per_layer": r["us_per_layer"], "hbm_frac_whole_step": r["hbm_frac_whole_step"],
+            "dominant_kernel": r["roofline"]["kernel"].split(" ")[0],
+            "us_per_launch": r["roofline"]["us_per_launch"], "frac": r["roofline"]["frac"],
+            "traffic": r["roofline"]["traffic"],
+            "cpu_tokens_per_s": (r.get("cpu_baseline") or {}).get("value"),
+            "parity": r.get("parity")}
+
+
+# The other configurations of the default run: fewer steps, the oracle on one request (parity
+# only).  (name, arguments of this script, what makes the compact line of the result)
+EXTRA = [
+    ("c1", ["--workload", "c1", "--steps", "50", "--warmup", "10"], _layer_line),
+    ("c3", ["--workload", "c3", "--steps", "50", "--warmup", "10"], _layer_line),
+    ("c5", ["--workload", "c5", "--steps", "50", "--warmup", "10"], _layer_line),
+    ("c4", ["--workload", "c4", "--steps", "64", "--warmup", "64", "--page-size", "1"], _trace_line),
+    ("c4-pages", ["--workload", "c4", "--steps", "64", "--warmup", "64", "--page-size", "16"], _trace_line),
+    # one 512-row chunk of the extend forward on a 128K context
+    ("prefill", ["--workload", "prefill", "--steps", "50", "--warmup", "10"], _prefill_line),
+    # the whole 32-layer decoder (the reference's full-model configuration) over 32 greedy steps
+    ("model", ["--workload", "model", "--steps", "32", "--warmup", "2"], _model_line),
+]
+EXTRA_COMMON = ["--pools", "4", "--cpu-reps", "1", "--cpu-requests", "1", "--no-extra"]
+
+
+def extra_in_own_processes():
+    """Every other workload measured by a child process of this script, one after the other,
+    before this process touches the GPU: a process of its own gives a workload the device
+    memory as a freshly started server finds it, whatever other workloads allocated and
+    freed (in one process C3 and C5 came out up to 3 % slower by that).  Returns the compact
+    lines, None where a child could not be had."""
+    import subprocess
+    lines = []
+    for name, argv, line_of in EXTRA:
         t0 = time.perf_counter()
-        paged = copy.copy(trace)
-        paged.page_size = page
-        r = measured(["--workload", "c4", "--steps", "64", "--warmup", "64", "--page-size", str(page)],
-                     lambda: bench_trace(paged, ops, workloads, dev))
-        lines.append({"workload": r["config"]["workload"], "us_per_step": r["value"],
-                      "hit_rate": r["hit_rate"], "bytes_per_step": r["roofline"]["bytes_per_step"],
-                      "frac": r["roofline"]["frac"], "wall_s": round(time.perf_counter() - t0, 1)})
-    # One 512-row chunk of the extend forward on a 128K context.
-    t0 = time.perf_counter()
-    r = measured(["--workload", "prefill", "--steps", "50", "--warmup", "10"],
-                 lambda: bench_prefill(small, ops, workloads, dev))
-    lines.append({"workload": r["config"]["workload"], "us_per_chunk": r["value"],
-                  "dominant_kernel": "ts::prefill_attn_kernel<G>", "bound": "mfma",
-                  "us_per_launch": r["roofline"]["us_per_launch"],
-                  "flops_per_launch": r["roofline"]["flops_per_launch"],
-                  "tflops": r["roofline"]["achieved"], "frac": r["roofline"]["frac"],
-                  "parity": r.get("parity"), "wall_s": round(time.perf_counter() - t0, 1)})
-    # The whole 32-layer decoder (the reference's full-model configuration) over 32 greedy steps.
-    t0 = time.perf_counter()
-    model = copy.copy(small)
-    model.steps, model.warmup = 32, 2
-    r = measured(["--workload", "model", "--steps", "32", "--warmup", "2"],
-                 lambda: bench_model(model, ops, dev))
-    lines.append({"workload": r["config"]["workload"], "tokens_per_s": r["value"],
-                  "greedy_steps": r["steps"], "ms_per_decode_step": r["ms_per_step"],
-                  "us_per_layer": r["us_per_layer"], "hbm_frac_whole_step": r["hbm_frac_whole_step"],
-                  "dominant_kernel": r["roofline"]["kernel"].split(" ")[0],
-                  "us_per_launch": r["roofline"]["us_per_launch"], "frac": r["roofline"]["frac"],
-                  "traffic": r["roofline"]["traffic"],
-                  "cpu_tokens_per_s": (r.get("cpu_baseline") or {}).get("value"),
-                  "parity": r.get("parity"), "wall_s": round(time.perf_counter() - t0, 1)})
+        try:
+            res = subprocess.run([sys.executable, os.path.abspath(__file__)] + argv + EXTRA_COMMON,
+                                 capture_output=True, text=True, timeout=600)
+            if res.returncode != 0:
+                raise RuntimeError(f"exit code {res.returncode}: {res.stderr[-400:]}")
+            line = line_of(json.loads(res.stdout.strip().splitlines()[-1]))
+            line["wall_s"] = round(time.perf_counter() - t0, 1)
+            lines.append(line)
+        except Exception as e:
+            print(f"bench.py: workload {name} in a process of its own: {e}", file=sys.stderr, flush=True)
+            lines.append(None)
+    return lines
+
+
+def extra_here(lines, args, ops, workloads, dev):
+    """The workloads no child process could be had for, measured in this process."""
+    import copy
+    import gc
+    parser_defaults = copy.copy(args)
+    for i, (name, argv, line_of) in enumerate(EXTRA):
+        if lines[i] is not None:
+            continue
+        gc.collect()
+        torch.cuda.empty_cache()
+        t0 = time.perf_counter()
+        small = copy.copy(parser_defaults)
+        small.pools, small.cpu_reps, small.cpu_requests = 4, 1, 1
+        opts = dict(zip(argv[0::2], argv[1::2]))
+        small.steps, small.warmup = int(opts["--steps"]), int(opts["--warmup"])
+        small.page_size = int(opts.get("--page-size", 1))
+        which = opts["--workload"]
+        if which == "c4":
+            r = bench_trace(small, ops, workloads, dev)
+        elif which == "prefill":
+            r = bench_prefill(small, ops, workloads, dev)
+        elif which == "model":
+            r = bench_model(small, ops, dev)
+        else:
+            r = bench_layer(small, ops, workloads, dev, which)
+        lines[i] = line_of(r)
+        lines[i]["wall_s"] = round(time.perf_counter() - t0, 1)
+    torch.cuda.empty_cache()
     return lines
 
 
@@ -671,6 +691,8 @@ def main():
                     help="requests of a large batch the CPU oracle is run on")
     ap.add_argument("--device-lengths-only", action="store_true",
                     help="c3, c5: do not hand the lengths to the library on the host")
+    ap.add_argument("--extra-in-process", action="store_true",
+                    help="measure the default run's other workloads in this process, not in child processes")
     ap.add_argument("--no-extra", action="store_true",
                     help="default run: only the headline workload, not the compact lines of the others")
     ap.add_argument("--prefill-context", type=int, default=131072,
@@ -690,6 +712,10 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the one-GPU hot path only; run with --gpus 1 "
                  "(no multi-GPU figure exists for it).")
+    extra = None
+    if args.workload == "c2" and not args.no_extra and torch.cuda.device_count() > 0:
+        # (before this process initialises the GPU)
+        extra = [None] * len(EXTRA) if args.extra_in_process else extra_in_own_processes()
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback.")
 
@@ -706,8 +732,8 @@ def main():
         result = bench_model(args, ops, dev)
     else:
         result = bench_layer(args, ops, workloads, dev)
-        if args.workload == "c2" and not args.no_extra:
-            result["extra_workloads"] = extra_workloads(args, ops, workloads, dev)
+        if extra is not None:
+            result["extra_workloads"] = extra_here(extra, args, ops, workloads, dev)
     print(json.dumps(result), flush=True)
 
 
