@@ -931,7 +931,7 @@ def test_layer_starts_with_the_selection_on_a_clean_workspace(dev, shape, lens):
         assert torch.equal(got[0].view(torch.int16), want[0].view(torch.int16)), f"step {step}: output"
 
 
-@pytest.mark.parametrize("shape", SHAPES[:3], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
 @pytest.mark.parametrize("mode", ["cache", "plain", "paged", "paged-cache"])
 @pytest.mark.parametrize("fused_select", [True, False], indirect=True, ids=["fused", "separate"])
 def test_decode_step_is_store_then_layer(dev, shape, mode, fused_select):

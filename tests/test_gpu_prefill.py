@@ -318,7 +318,7 @@ def test_prefill_chunks(dev, shape, fused):
         ops.set_fused_select(previous)
 
 
-@pytest.mark.parametrize("shape", SHAPES[:3], ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"H{s['num_heads']}kv{s['num_kv_heads']}")
 @pytest.mark.parametrize("chunk", [64, 500])
 def test_prefill_step_is_store_then_chunk(dev, shape, chunk):
     """ts_prefill_step (one chunk of the extend forward in one call, tr.py:725-773) against
